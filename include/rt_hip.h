@@ -1,0 +1,170 @@
+/*
+ * rt_hip.h -- C ABI of the MI355X (gfx950) backend for rtensors.
+ *
+ * This is the boundary a Rust `impl Backend for Hip` binds (one entry point per required method family of
+ * `trait Backend`, libs/rtensors/src/backend/mod.rs:216-472, in the de-genericised form the reference already
+ * uses for its remote protocol, backend/remote/protocol.rs:246-291).  Plain pointers and sizes only.
+ *
+ * Conventions
+ *   - Every function returns an rt_status (0 = ok).  Nothing aborts; a bad descriptor is an error code, never a
+ *     device fault (checks follow backend/remote/server.rs:241-380).  rt_last_error() gives the message of the
+ *     last failure on the calling thread.
+ *   - `dtype` uses the reference's DType codes (core/value.rs:567-581), binary ops its BinaryOpType codes
+ *     (ops/base.rs:7-12), reductions its ReductionOpTypes codes (ops/reduction/mod.rs:161-175), unary and scalar
+ *     ops the declaration order of UnaryOp / ScalarOp (backend/remote/protocol.rs:213-232).
+ *   - Buffers are device pointers returned by rt_alloc*; every call that touches a buffer also takes its length
+ *     in elements so that extents can be validated.  Offsets, strides and lengths are in elements.
+ *   - Work is enqueued on the context's stream and returns immediately; rt_read / rt_dump / rt_equal /
+ *     rt_sync wait for it (as the reference's Cuda backend does, backend/cuda.rs:164-185, 719-836).
+ *   - A context may be used from several host threads; calls are serialised internally.
+ */
+#ifndef RT_HIP_H
+#define RT_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct rt_ctx rt_ctx;
+
+typedef enum rt_status {
+    RT_OK = 0,
+    RT_E_INVALID = 1,      /* malformed argument (null pointer, unknown code, shape/stride mismatch) */
+    RT_E_DTYPE = 2,        /* dtype/op combination the trait bounds of the reference do not admit, or not built */
+    RT_E_OUT_OF_BOUNDS = 3,/* a descriptor addresses elements outside its buffer (TensorError::IdxOutOfBounds) */
+    RT_E_HIP = 4,          /* HIP runtime failure; see rt_last_error() */
+    RT_E_OOM = 5,          /* device allocation failed */
+    RT_E_RANK = 6,         /* more than RT_MAX_RANK dims remain after collapsing */
+    RT_E_ARITH = 7,        /* integer division by a zero scalar / mean over an empty integer axis (reference panics) */
+    RT_E_WRONG_DIMS = 8,   /* TensorError::WrongDims: reduction source is not contiguous (backend/mod.rs:386-390) */
+    RT_E_SIZE_MISMATCH = 9 /* TensorError::SizeMismatch (backend/cpu.rs:151-161) */
+} rt_status;
+
+/* core/value.rs:567-581 */
+typedef enum rt_dtype {
+    RT_U8 = 0, RT_I8 = 1, RT_U16 = 2, RT_I16 = 3, RT_U32 = 4, RT_U128 = 5, RT_I32 = 6, RT_U64 = 7, RT_I64 = 8,
+    RT_I128 = 9, RT_F32 = 10, RT_F64 = 11, RT_BOOL = 12
+} rt_dtype;
+
+/* ops/base.rs:7-12 */
+typedef enum rt_binary_op { RT_ADD = 0, RT_SUB = 1, RT_MUL = 2, RT_DIV = 3 } rt_binary_op;
+
+/* backend/remote/protocol.rs:226-232 */
+typedef enum rt_scalar_op {
+    RT_S_ADD = 0, RT_S_SUB = 1, RT_S_MUL = 2, RT_S_DIV = 3, RT_S_LOG = 4, RT_S_LOG1P = 5, RT_S_LEAKY_RELU = 6, RT_S_ELU = 7
+} rt_scalar_op;
+
+/* backend/remote/protocol.rs:213-224 */
+typedef enum rt_unary_op {
+    RT_U_NEG = 0, RT_U_RELU, RT_U_SIGMOID, RT_U_SILU, RT_U_TANH, RT_U_ABS, RT_U_SQRT, RT_U_LN, RT_U_EXPM1, RT_U_LN1P,
+    RT_U_FLOOR, RT_U_CEIL, RT_U_ROUND, RT_U_TRUNC, RT_U_SIN, RT_U_COS, RT_U_TAN, RT_U_ASIN, RT_U_ACOS, RT_U_ATAN,
+    RT_U_SINH, RT_U_COSH, RT_U_ASINH, RT_U_ACOSH, RT_U_ATANH, RT_U_RSQRT, RT_U_RECIPROCAL, RT_U_SQUARE, RT_U_CUBE,
+    RT_U_EXP, RT_U_SIGN, RT_U_COUNT
+} rt_unary_op;
+
+/* ops/reduction/mod.rs:161-175 (codes 6-10 -- variance, logsumexp, norm, argmax, argmin -- are outside this path) */
+typedef enum rt_reduce_op { RT_R_SUM = 1, RT_R_PROD = 2, RT_R_MAX = 3, RT_R_MIN = 4, RT_R_MEAN = 5 } rt_reduce_op;
+
+#define RT_MAX_RANK 8        /* dims a kernel descriptor holds after size-1 removal and merging of adjacent dims */
+#define RT_MAX_INPUT_RANK 128 /* the reference's own cap on rank (core/primitives.rs:377-383) */
+
+/* ---- context ------------------------------------------------------------------------------------------------
+ * Replaces the lazily built per-device singleton + default stream of backend/cuda.rs:38-51, 143-185. */
+int32_t rt_ctx_create(int32_t device, rt_ctx** out);
+int32_t rt_ctx_destroy(rt_ctx* ctx);
+int32_t rt_sync(rt_ctx* ctx);                       /* Cuda::sync, backend/cuda.rs:164-185 */
+const char* rt_last_error(void);                    /* message of the last failing call on this thread */
+const char* rt_status_name(int32_t status);
+int32_t rt_dtype_size(int32_t dtype);               /* bytes per element, 0 for an unknown code */
+int32_t rt_device_count(int32_t* out);
+
+/* ---- buffers and transfers (Backend::alloc .. dump, backend/mod.rs:225-233; Cpu backend/cpu.rs:147-243) ------- */
+/* Backend::alloc: `len` elements, zero-initialised like the Cpu backend's vec![T::default(); len]. */
+int32_t rt_alloc(rt_ctx* ctx, int32_t dtype, uint64_t len, void** out);
+/* Same without the zero fill, for outputs every element of which is about to be written. */
+int32_t rt_alloc_uninit(rt_ctx* ctx, int32_t dtype, uint64_t len, void** out);
+/* Backend::alloc_from_slice: allocate and upload `len` host elements. */
+int32_t rt_alloc_from_slice(rt_ctx* ctx, int32_t dtype, const void* host_src, uint64_t len, void** out);
+/* Drop of Backend::Buf: returns the block to the context's caching allocator (stream ordered). */
+int32_t rt_free(rt_ctx* ctx, void* buf);
+/* Backend::copy_from_slice: lengths must match (RT_E_SIZE_MISMATCH otherwise). */
+int32_t rt_copy_from_slice(rt_ctx* ctx, int32_t dtype, void* dst, uint64_t dst_len, const void* host_src, uint64_t src_len);
+/* Backend::copy_range_within: device-to-device copy of `len` elements. */
+int32_t rt_copy_range_within(rt_ctx* ctx, int32_t dtype, void* dst, uint64_t dst_len, const void* src, uint64_t src_len,
+                             uint64_t dst_offset, uint64_t src_offset, uint64_t len);
+/* Backend::read / Backend::write: one element; synchronises first. */
+int32_t rt_read(rt_ctx* ctx, int32_t dtype, const void* buf, uint64_t buf_len, uint64_t offset, void* out_value);
+int32_t rt_write(rt_ctx* ctx, int32_t dtype, void* buf, uint64_t buf_len, uint64_t offset, const void* value);
+/* Backend::copy: fresh buffer holding a copy of `src`. */
+int32_t rt_copy(rt_ctx* ctx, int32_t dtype, const void* src, uint64_t len, void** out);
+/* Backend::dump: download the whole buffer into `host_dst` (len elements); synchronises. */
+int32_t rt_dump(rt_ctx* ctx, int32_t dtype, const void* src, uint64_t len, void* host_dst);
+/* PartialEq of Backend::Buf (backend/cuda.rs:59-141): lengths equal and all elements `==` (NaN != NaN). */
+int32_t rt_equal(rt_ctx* ctx, int32_t dtype, const void* a, uint64_t a_len, const void* b, uint64_t b_len, int32_t* out_equal);
+/* Backend::convert: elementwise dtype conversion between equally long buffers (core/value.rs:255-462). */
+int32_t rt_convert(rt_ctx* ctx, int32_t src_dtype, const void* src, uint64_t src_len, int32_t dst_dtype, void* dst, uint64_t dst_len);
+
+/* ---- fill (Backend::fill_contiguous / fill_1d_strided / fill_nd, backend/mod.rs:270-294) ----------------------- */
+int32_t rt_fill_contiguous(rt_ctx* ctx, int32_t dtype, void* buf, uint64_t buf_len, const void* value, uint64_t start, uint64_t len);
+int32_t rt_fill_1d_strided(rt_ctx* ctx, int32_t dtype, void* buf, uint64_t buf_len, const void* value,
+                           uint64_t offset, int64_t stride, uint64_t len);
+int32_t rt_fill_nd(rt_ctx* ctx, int32_t dtype, void* buf, uint64_t buf_len, const void* value,
+                   uint64_t offset, int32_t rank, const uint64_t* shape, const int64_t* strides);
+
+/* ---- in-place unary ops (Backend::apply_<op>_{contiguous,1d_strided,nd}, backend/mod.rs:96-141, 311-355) ------ */
+int32_t rt_unary_contiguous(rt_ctx* ctx, int32_t dtype, int32_t op, void* buf, uint64_t buf_len, uint64_t start, uint64_t len);
+int32_t rt_unary_1d_strided(rt_ctx* ctx, int32_t dtype, int32_t op, void* buf, uint64_t buf_len,
+                            uint64_t offset, int64_t stride, uint64_t len);
+int32_t rt_unary_nd(rt_ctx* ctx, int32_t dtype, int32_t op, void* buf, uint64_t buf_len,
+                    uint64_t offset, int32_t rank, const uint64_t* shape, const int64_t* strides);
+
+/* ---- in-place scalar ops (Backend::scalar_apply_<op>_{...}, backend/mod.rs:143-213, 327-334) ----------------- */
+int32_t rt_scalar_contiguous(rt_ctx* ctx, int32_t dtype, int32_t op, void* buf, uint64_t buf_len, const void* value,
+                             uint64_t start, uint64_t len);
+int32_t rt_scalar_1d_strided(rt_ctx* ctx, int32_t dtype, int32_t op, void* buf, uint64_t buf_len, const void* value,
+                             uint64_t offset, int64_t stride, uint64_t len);
+int32_t rt_scalar_nd(rt_ctx* ctx, int32_t dtype, int32_t op, void* buf, uint64_t buf_len, const void* value,
+                     uint64_t offset, int32_t rank, const uint64_t* shape, const int64_t* strides);
+
+/* ---- N-d broadcast (Backend::broadcast, backend/mod.rs:296-309; Cpu backend/cpu.rs:292-352) --------------------
+ * dst[c] = left[c] (op) right[c] for every coordinate c of `shape`.  The three operands share `shape`
+ * (expansion is expressed as stride 0, ops/broadcast/mod.rs:13-55); strides may be negative.  dst may be the
+ * same buffer as left with the same layout (in-place `a op= b`). */
+int32_t rt_broadcast(rt_ctx* ctx, int32_t dtype, int32_t op, int32_t rank, const uint64_t* shape,
+                     const void* left, uint64_t left_len, uint64_t left_offset, const int64_t* left_strides,
+                     const void* right, uint64_t right_len, uint64_t right_offset, const int64_t* right_strides,
+                     void* dst, uint64_t dst_len, uint64_t dst_offset, const int64_t* dst_strides);
+
+/* ---- reductions (Backend::apply_reduce_contiguous_flat / _nd, backend/mod.rs:357-409; Cpu backend/cpu.rs:397-449)
+ * Flat: dst[0] = fold(src[start .. start+len]).  Nd: `src` described by (offset, shape, strides) must be row-major
+ * contiguous; viewed as (outer, R = shape[dim], inner), dst[o*inner + i] = fold_k src[offset + (o*R + k)*inner + i].
+ * The offset is honoured (as backend/cuda.rs:1934 does; the Cpu backend drops it, backend/cpu.rs:434).
+ * Float sums are tree sums: within 1e-5 (f32) / 1e-12 (f64) of sum|x| of the sequential result; integer results,
+ * max and min are bit-exact.  f32/f64 as in the reference, plus the 8..64-bit integers. */
+int32_t rt_reduce_flat(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, uint64_t src_len,
+                       void* dst, uint64_t dst_len, uint64_t start, uint64_t len);
+int32_t rt_reduce_nd(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, uint64_t src_len,
+                     uint64_t offset, int32_t rank, const uint64_t* shape, const int64_t* strides,
+                     void* dst, uint64_t dst_len, int32_t dim);
+
+/* ---- strided gather (what TensorView::owned / contiguous need, core/tensor.rs:299-325: the reference issues one
+ * copy_range_within per forward-contiguous run; this is the same result in one launch) ------------------------- */
+int32_t rt_gather(rt_ctx* ctx, int32_t dtype, const void* src, uint64_t src_len, uint64_t offset, int32_t rank,
+                  const uint64_t* shape, const int64_t* strides, void* dst, uint64_t dst_len);
+
+/* ---- timing and allocator introspection (no counterpart in the reference; used by the benchmark) -------------- */
+typedef struct rt_event rt_event;
+int32_t rt_event_create(rt_ctx* ctx, rt_event** out);
+int32_t rt_event_record(rt_ctx* ctx, rt_event* ev);              /* on the context's stream */
+int32_t rt_event_elapsed_ms(rt_ctx* ctx, rt_event* start, rt_event* stop, float* out_ms);   /* waits for `stop` */
+int32_t rt_event_destroy(rt_ctx* ctx, rt_event* ev);
+/* bytes currently handed out, bytes cached in free lists, number of hipMalloc calls so far */
+int32_t rt_mem_stats(rt_ctx* ctx, uint64_t* in_use, uint64_t* cached, uint64_t* device_allocs);
+int32_t rt_mem_trim(rt_ctx* ctx);                                /* hipFree everything in the free lists */
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RT_HIP_H */

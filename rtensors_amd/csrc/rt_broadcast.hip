@@ -1,0 +1,504 @@
+// N-d broadcast binary kernel family: dst[c] = left[c] (op) right[c] over a shared shape, operands pre-broadcast
+// (expansion = stride 0), strides signed.  Replaces Backend::broadcast (backend/mod.rs:296-309; Cpu loop
+// backend/cpu.rs:292-352; the reference's CUDA kernel is K/kernels/elementwise/binary/broadcast.cu:3-55).
+//
+// Host side: size-1 dims are dropped, dims are flipped/sorted so that dst is walked in ascending address order, and
+// adjacent dims that are mergeable in all three operands are merged (rt_collapse).  The descriptor travels in the
+// kernel arguments; nothing is uploaded per call.
+//
+// Device side, three shapes of kernel:
+//   contig : all three operands are one unit-stride run -> 16-byte accesses, 2 loads + 1 store per vector
+//   rows   : dst's innermost collapsed dim is unit-stride.  A block owns a column tile of a row and loops over a
+//            chosen outer dim `g`; an operand whose stride along g is 0 (the broadcast one) is loaded once and kept
+//            in registers for the whole loop, so it costs no traffic per output row.  (row, chunk, tile) come from
+//            blockIdx by multiply-high division on the scalar unit; no per-element index arithmetic.
+//   generic: anything else, one element per lane, per-element multiply-high index decomposition.
+// Algorithmic traffic: (|left|_unique + |right|_unique + N) * sizeof(T).
+#include "rt_common.h"
+
+#include <type_traits>
+
+namespace {
+
+struct boolean_t { uint8_t v; };
+template <class T> struct is_flt : std::integral_constant<bool, std::is_same<T, float>::value || std::is_same<T, double>::value> {};
+template <class T> struct is_bool : std::is_same<T, boolean_t> {};
+
+template <class T, class E = void> struct carrier { typedef T type; };
+template <class T> struct carrier<T, typename std::enable_if<std::is_integral<T>::value && sizeof(T) <= 4>::type> { typedef uint32_t type; };
+template <class T> struct carrier<T, typename std::enable_if<std::is_integral<T>::value && sizeof(T) == 8>::type> { typedef uint64_t type; };
+
+// ops/base.rs:27-37 on T; integers wrap (release build), integer division truncates toward zero
+constexpr int kOpCopy = 4;      // internal: dst = left (strided gather); right is ignored
+
+template <int OP, class T> __device__ __forceinline__ T bin_apply(T a, T b) {
+    if constexpr (OP == kOpCopy) {
+        return a;
+    } else if constexpr (is_flt<T>::value) {
+        if constexpr (OP == RT_ADD) return a + b;
+        else if constexpr (OP == RT_SUB) return a - b;
+        else if constexpr (OP == RT_MUL) return a * b;
+        else return a / b;
+    } else if constexpr (is_bool<T>::value) {
+        if constexpr (OP == RT_ADD) return boolean_t{(uint8_t)(a.v | b.v)};            // core/value.rs:708-713 (OR)
+        else if constexpr (OP == RT_SUB) return boolean_t{(uint8_t)(a.v ^ b.v)};       // core/value.rs:715-720 (XOR)
+        else return boolean_t{(uint8_t)(a.v & b.v)};                                   // core/value.rs:722-727 (AND)
+    } else {
+        typedef typename carrier<T>::type W;
+        if constexpr (OP == RT_ADD) return (T)(W)((W)a + (W)b);
+        else if constexpr (OP == RT_SUB) return (T)(W)((W)a - (W)b);
+        else if constexpr (OP == RT_MUL) return (T)(W)((W)a * (W)b);
+        else {
+            // the reference panics on b == 0 and MIN / -1; the device yields 0 and MIN there and raises no error
+            if (b == 0) return (T)0;
+            if constexpr (std::is_signed<T>::value) {
+                if (b == (T)-1) return (T)(W)((W)0 - (W)a);
+            }
+            return (T)(a / b);
+        }
+    }
+}
+
+template <class T> struct alignas(16) Vec16 { T e[16 / sizeof(T)]; };
+
+constexpr int kBlock = 256;
+constexpr int kGU = 4;          // iterations of the loop dim whose loads are issued before the first store
+
+enum Mode : int { M_VEC = 0, M_BCAST = 1, M_ELEM = 2 };
+
+// ---- contig ---------------------------------------------------------------------------------------------------------
+template <class T, int OP>
+__global__ __launch_bounds__(kBlock) void bin_contig_kernel(const Vec16<T>* l, const Vec16<T>* r, Vec16<T>* d, size_t nvec) {
+    constexpr int N = 16 / sizeof(T);
+    constexpr int U = 4;
+    const size_t base = (size_t)blockIdx.x * (kBlock * U) + threadIdx.x;
+    if (base + (size_t)(U - 1) * kBlock < nvec) {
+        Vec16<T> a[U], b[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) { a[u] = l[base + (size_t)u * kBlock]; b[u] = r[base + (size_t)u * kBlock]; }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+            for (int j = 0; j < N; ++j) a[u].e[j] = bin_apply<OP, T>(a[u].e[j], b[u].e[j]);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) d[base + (size_t)u * kBlock] = a[u];
+    } else {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const size_t i = base + (size_t)u * kBlock;
+            if (i < nvec) {
+                Vec16<T> a = l[i], b = r[i];
+#pragma unroll
+                for (int j = 0; j < N; ++j) a.e[j] = bin_apply<OP, T>(a.e[j], b.e[j]);
+                d[i] = a;
+            }
+        }
+    }
+}
+
+// ---- rows -------------------------------------------------------------------------------------------------------------
+struct RowArgs {
+    uint32_t L;                     // inner length (elements)
+    uint32_t G;                     // extent of the loop dim (1 when there is none)
+    uint32_t gchunk;                // loop-dim iterations owned by one block
+    uint32_t nchunks;               // ceil(G / gchunk)
+    uint32_t tiles;                 // column tiles per row
+    uint32_t tpr;                   // lanes per row inside a block (power of two <= kBlock)
+    FastDiv32 tiles_div, nchunks_div;
+    int nouter;                     // remaining outer dims (loop dim and inner dim excluded), outermost first
+    uint32_t oshape[RT_MAX_RANK];
+    FastDiv32 odiv[RT_MAX_RANK];
+    int64_t ostride[3][RT_MAX_RANK];
+    int64_t gstride[3];
+    int64_t istride[2];             // inner strides of left, right (dst: 1)
+};
+
+template <class T, int MODE>
+__device__ __forceinline__ Vec16<T> load_vec(const T* __restrict__ rowp, uint32_t c, int64_t istride) {
+    constexpr int N = 16 / sizeof(T);
+    Vec16<T> v;
+    if constexpr (MODE == M_VEC) {
+        v = *reinterpret_cast<const Vec16<T>*>(rowp + c);
+    } else if constexpr (MODE == M_BCAST) {
+        T x = rowp[0];
+#pragma unroll
+        for (int j = 0; j < N; ++j) v.e[j] = x;
+    } else {
+#pragma unroll
+        for (int j = 0; j < N; ++j) v.e[j] = rowp[(int64_t)(c + j) * istride];
+    }
+    return v;
+}
+
+template <class T, int OP, int LM, int RM>
+__global__ __launch_bounds__(kBlock) void bin_rows_kernel(const T* l, const T* r, T* d, RowArgs a) {
+    constexpr int N = 16 / sizeof(T);
+    // blockIdx -> (outer index, chunk of the loop dim, column tile); all uniform, computed on the scalar unit
+    uint32_t b = blockIdx.x;
+    uint32_t q = fd_div(b, a.tiles_div);
+    const uint32_t tile = b - q * a.tiles;
+    b = q;
+    q = fd_div(b, a.nchunks_div);
+    const uint32_t chunk = b - q * a.nchunks;
+    uint32_t rem = q;
+    int64_t ol = 0, orr = 0, od = 0;
+#pragma unroll
+    for (int k = RT_MAX_RANK - 1; k >= 0; --k) {
+        if (k < a.nouter) {
+            uint32_t qq = fd_div(rem, a.odiv[k]);
+            uint32_t c = rem - qq * a.oshape[k];
+            ol += (int64_t)c * a.ostride[0][k];
+            orr += (int64_t)c * a.ostride[1][k];
+            od += (int64_t)c * a.ostride[2][k];
+            rem = qq;
+        }
+    }
+    const uint32_t tx = threadIdx.x & (a.tpr - 1);
+    const uint32_t ty = threadIdx.x / a.tpr;
+    const uint32_t gy = kBlock / a.tpr;
+    const uint32_t c = (tile * a.tpr + tx) * N;                 // first column of this lane's vector
+    if (c >= a.L) return;
+    const uint32_t g_begin = chunk * a.gchunk;
+    const uint32_t g_end = min(a.G, g_begin + a.gchunk);
+    const bool full = (c + N <= a.L);
+
+    const bool l_fixed = (a.gstride[0] == 0), r_fixed = (a.gstride[1] == 0);
+    Vec16<T> lh, rh;                                            // operands that do not move along the loop dim
+    if (full) {
+        if (l_fixed) lh = load_vec<T, LM>(l + ol, c, a.istride[0]);
+        if (r_fixed) rh = load_vec<T, RM>(r + orr, c, a.istride[1]);
+    }
+    for (uint32_t g0 = g_begin + ty; g0 < g_end; g0 += gy * kGU) {
+        if (full) {
+            Vec16<T> x[kGU], y[kGU];
+#pragma unroll
+            for (int u = 0; u < kGU; ++u) {
+                const uint32_t g = g0 + u * gy;
+                if (g < g_end) {
+                    x[u] = l_fixed ? lh : load_vec<T, LM>(l + ol + (int64_t)g * a.gstride[0], c, a.istride[0]);
+                    y[u] = r_fixed ? rh : load_vec<T, RM>(r + orr + (int64_t)g * a.gstride[1], c, a.istride[1]);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kGU; ++u) {
+                const uint32_t g = g0 + u * gy;
+                if (g < g_end) {
+#pragma unroll
+                    for (int j = 0; j < N; ++j) x[u].e[j] = bin_apply<OP, T>(x[u].e[j], y[u].e[j]);
+                    *reinterpret_cast<Vec16<T>*>(d + od + (int64_t)g * a.gstride[2] + c) = x[u];
+                }
+            }
+        } else {
+            // ragged end of a row: element accesses
+            for (int u = 0; u < kGU; ++u) {
+                const uint32_t g = g0 + u * gy;
+                if (g < g_end) {
+                    const T* lp = l + ol + (int64_t)g * a.gstride[0];
+                    const T* rp = r + orr + (int64_t)g * a.gstride[1];
+                    T* dp = d + od + (int64_t)g * a.gstride[2];
+                    for (uint32_t k = c; k < a.L; ++k)
+                        dp[k] = bin_apply<OP, T>(lp[(int64_t)k * a.istride[0]], rp[(int64_t)k * a.istride[1]]);
+                }
+            }
+        }
+    }
+}
+
+// ---- generic ------------------------------------------------------------------------------------------------------------
+struct GenArgs {
+    int rank;
+    uint32_t shape[RT_MAX_RANK];
+    FastDiv32 div[RT_MAX_RANK];
+    int64_t stride[3][RT_MAX_RANK];
+};
+
+template <class T, int OP>
+__global__ __launch_bounds__(kBlock) void bin_generic_kernel(const T* l, const T* r, T* d, GenArgs a, uint32_t n) {
+    uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+    const uint32_t step = gridDim.x * kBlock;
+    for (; i < n; i += step) {
+        uint32_t rem = i;
+        int64_t ol = 0, orr = 0, od = 0;
+#pragma unroll
+        for (int k = RT_MAX_RANK - 1; k >= 0; --k) {
+            if (k < a.rank) {
+                uint32_t q = fd_div(rem, a.div[k]);
+                uint32_t c = rem - q * a.shape[k];
+                ol += (int64_t)c * a.stride[0][k];
+                orr += (int64_t)c * a.stride[1][k];
+                od += (int64_t)c * a.stride[2][k];
+                rem = q;
+            }
+        }
+        d[od] = bin_apply<OP, T>(l[ol], r[orr]);
+    }
+}
+
+template <class T, int OP>
+__global__ __launch_bounds__(kBlock) void bin_generic64_kernel(const T* l, const T* r, T* d, NdDesc a, uint64_t n) {
+    uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    const uint64_t step = (uint64_t)gridDim.x * kBlock;
+    for (; i < n; i += step) {
+        uint64_t rem = i;
+        int64_t ol = 0, orr = 0, od = 0;
+        for (int k = a.rank - 1; k >= 0; --k) {
+            uint64_t q = rem / (uint64_t)a.shape[k];
+            int64_t c = (int64_t)(rem - q * (uint64_t)a.shape[k]);
+            ol += c * a.stride[0][k];
+            orr += c * a.stride[1][k];
+            od += c * a.stride[2][k];
+            rem = q;
+        }
+        d[od] = bin_apply<OP, T>(l[ol], r[orr]);
+    }
+}
+
+// ---- host: kernel choice ----------------------------------------------------------------------------------------------
+template <class T, int OP, int LM>
+void launch_rows_r(int rm, dim3 grid, hipStream_t s, const T* l, const T* r, T* d, const RowArgs& a) {
+    switch (rm) {
+        case M_VEC: hipLaunchKernelGGL((bin_rows_kernel<T, OP, LM, M_VEC>), grid, dim3(kBlock), 0, s, l, r, d, a); break;
+        case M_BCAST: hipLaunchKernelGGL((bin_rows_kernel<T, OP, LM, M_BCAST>), grid, dim3(kBlock), 0, s, l, r, d, a); break;
+        default: hipLaunchKernelGGL((bin_rows_kernel<T, OP, LM, M_ELEM>), grid, dim3(kBlock), 0, s, l, r, d, a); break;
+    }
+}
+template <class T, int OP>
+void launch_rows(int lm, int rm, dim3 grid, hipStream_t s, const T* l, const T* r, T* d, const RowArgs& a) {
+    switch (lm) {
+        case M_VEC: launch_rows_r<T, OP, M_VEC>(rm, grid, s, l, r, d, a); break;
+        case M_BCAST: launch_rows_r<T, OP, M_BCAST>(rm, grid, s, l, r, d, a); break;
+        default: launch_rows_r<T, OP, M_ELEM>(rm, grid, s, l, r, d, a); break;
+    }
+}
+
+static inline bool mult_of(int64_t v, int64_t n) { return v % n == 0; }
+
+// Can operand `o` be read with aligned 16-byte loads at every (outer, g, column-vector) position?
+template <class T>
+static bool vec_ok(const T* base, const NdDesc& dsc, int o) {
+    constexpr int64_t N = 16 / sizeof(T);
+    if ((reinterpret_cast<uintptr_t>(base + dsc.offset[o]) & 15) != 0) return false;
+    for (int k = 0; k < dsc.rank - 1; ++k)
+        if (!mult_of(dsc.stride[o][k], N)) return false;
+    return true;
+}
+
+template <class T, int OP>
+int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const void* lv, const void* rv, void* dv) {
+    const T* l = (const T*)lv;
+    const T* r = (const T*)rv;
+    T* d = (T*)dv;
+    constexpr int64_t N = 16 / sizeof(T);
+    hipStream_t s = ctx->stream;
+    const int rank = dsc.rank;
+
+    // (1) one unit-stride run in all three operands
+    if (rank <= 1 && (rank == 0 || (dsc.stride[0][0] == 1 && dsc.stride[1][0] == 1 && dsc.stride[2][0] == 1))) {
+        const T* lp = l + dsc.offset[0];
+        const T* rp = r + dsc.offset[1];
+        T* dp = d + dsc.offset[2];
+        uintptr_t al = reinterpret_cast<uintptr_t>(lp) & 15, ar = reinterpret_cast<uintptr_t>(rp) & 15, ad = reinterpret_cast<uintptr_t>(dp) & 15;
+        if (al == ar && ar == ad) {
+            size_t n = (size_t)count;
+            size_t head = ((16 - ad) & 15) / sizeof(T);
+            if (head > n) head = n;
+            size_t nvec = (n - head) / N, tail = n - head - nvec * N;
+            if (nvec) {
+                size_t blocks = (nvec + (size_t)kBlock * 4 - 1) / ((size_t)kBlock * 4);
+                if (blocks > 0x7fffffffull) return rt_fail(RT_E_INVALID, "broadcast: %zu elements is too long for one launch", n);
+                hipLaunchKernelGGL((bin_contig_kernel<T, OP>), dim3((unsigned)blocks), dim3(kBlock), 0, s,
+                                   reinterpret_cast<const Vec16<T>*>(lp + head), reinterpret_cast<const Vec16<T>*>(rp + head),
+                                   reinterpret_cast<Vec16<T>*>(dp + head), nvec);
+            }
+            // the few elements before / after the 16-byte aligned body
+            auto edge = [&](size_t first, size_t len) {
+                NdDesc e;
+                memset(&e, 0, sizeof(e));
+                e.rank = 1;
+                e.shape[0] = (int64_t)len;
+                e.stride[0][0] = e.stride[1][0] = e.stride[2][0] = 1;
+                hipLaunchKernelGGL((bin_generic64_kernel<T, OP>), dim3(1), dim3(kBlock), 0, s, lp + first, rp + first, dp + first, e, (uint64_t)len);
+            };
+            if (head) edge(0, head);
+            if (tail) edge(head + nvec * N, tail);
+            RT_HIP(hipGetLastError());
+            return RT_OK;
+        }
+    }
+
+    // (2) rows: dst inner dim unit-stride, rows 16-byte aligned, everything indexable in 32 bits
+    if (rank >= 1 && count < (1ull << 31) && dsc.stride[2][rank - 1] == 1 && dsc.shape[rank - 1] >= 2 * N && vec_ok<T>(d, dsc, 2)) {
+        RowArgs a;
+        memset(&a, 0, sizeof(a));
+        a.L = (uint32_t)dsc.shape[rank - 1];
+        a.istride[0] = dsc.stride[0][rank - 1];
+        a.istride[1] = dsc.stride[1][rank - 1];
+        // loop dim: the largest outer dim along which one input does not move; else the innermost outer dim
+        int gdim = -1;
+        for (int k = 0; k < rank - 1; ++k)
+            if ((dsc.stride[0][k] == 0 || dsc.stride[1][k] == 0) && (gdim < 0 || dsc.shape[k] > dsc.shape[gdim])) gdim = k;
+        if (gdim < 0 && rank >= 2) gdim = rank - 2;
+        a.G = gdim >= 0 ? (uint32_t)dsc.shape[gdim] : 1;
+        for (int o = 0; o < 3; ++o) a.gstride[o] = gdim >= 0 ? dsc.stride[o][gdim] : 0;
+        a.nouter = 0;
+        uint64_t outer = 1;
+        for (int k = 0; k < rank - 1; ++k) {
+            if (k == gdim) continue;
+            a.oshape[a.nouter] = (uint32_t)dsc.shape[k];
+            a.odiv[a.nouter] = make_fastdiv((uint32_t)dsc.shape[k]);
+            for (int o = 0; o < 3; ++o) a.ostride[o][a.nouter] = dsc.stride[o][k];
+            outer *= (uint64_t)dsc.shape[k];
+            a.nouter++;
+        }
+        for (int k = a.nouter; k < RT_MAX_RANK; ++k) { a.oshape[k] = 1; a.odiv[k] = make_fastdiv(1); }
+        // lanes per row: enough for one vector per lane, at most a block
+        uint32_t vecs = (uint32_t)((a.L + N - 1) / N);
+        uint32_t tpr = 1;
+        while (tpr < vecs && tpr < (uint32_t)kBlock) tpr <<= 1;
+        a.tpr = tpr;
+        a.tiles = (vecs + tpr - 1) / tpr;
+        const uint32_t gy = kBlock / tpr;
+        // loop-dim iterations per block: as long as possible (an operand that does not move along the loop dim is
+        // then fetched once per block), shortened until there are enough blocks to fill the chip
+        uint32_t gchunk = a.G;
+        const uint64_t want_blocks = (uint64_t)ctx->num_cus * 8;
+        while (gchunk > gy * kGU && outer * a.tiles * ((a.G + gchunk - 1) / gchunk) < want_blocks) gchunk = (gchunk + 1) / 2;
+        if (gchunk < 1) gchunk = 1;
+        a.gchunk = gchunk;
+        a.nchunks = (a.G + gchunk - 1) / gchunk;
+        a.tiles_div = make_fastdiv(a.tiles);
+        a.nchunks_div = make_fastdiv(a.nchunks);
+        const uint64_t blocks = outer * a.nchunks * a.tiles;
+        if (blocks < (1ull << 31)) {
+            auto mode = [&](int o, const T* base) -> int {
+                int64_t is = dsc.stride[o][rank - 1];
+                if (is == 0) return (int)M_BCAST;
+                if (is == 1 && vec_ok<T>(base, dsc, o)) return (int)M_VEC;
+                return (int)M_ELEM;
+            };
+            launch_rows<T, OP>(mode(0, l), mode(1, r), dim3((unsigned)blocks), s, l + dsc.offset[0], r + dsc.offset[1], d + dsc.offset[2], a);
+            RT_HIP(hipGetLastError());
+            return RT_OK;
+        }
+    }
+
+    // (3) generic
+    if (count < (1ull << 31)) {
+        GenArgs g;
+        g.rank = rank;
+        for (int k = 0; k < RT_MAX_RANK; ++k) {
+            g.shape[k] = k < rank ? (uint32_t)dsc.shape[k] : 1;
+            g.div[k] = make_fastdiv(g.shape[k]);
+            for (int o = 0; o < 3; ++o) g.stride[o][k] = k < rank ? dsc.stride[o][k] : 0;
+        }
+        size_t blocks = ((size_t)count + kBlock - 1) / kBlock;
+        size_t cap = (size_t)ctx->num_cus * 64;
+        hipLaunchKernelGGL((bin_generic_kernel<T, OP>), dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(kBlock), 0, s,
+                           l + dsc.offset[0], r + dsc.offset[1], d + dsc.offset[2], g, (uint32_t)count);
+    } else {
+        size_t cap = (size_t)ctx->num_cus * 64;
+        hipLaunchKernelGGL((bin_generic64_kernel<T, OP>), dim3((unsigned)cap), dim3(kBlock), 0, s,
+                           l + dsc.offset[0], r + dsc.offset[1], d + dsc.offset[2], dsc, count);
+    }
+    RT_HIP(hipGetLastError());
+    return RT_OK;
+}
+
+template <class T>
+int32_t broadcast_ops(rt_ctx* ctx, int op, const NdDesc& d, uint64_t count, const void* l, const void* r, void* dst) {
+    switch (op) {
+        case RT_ADD: return broadcast_typed<T, RT_ADD>(ctx, d, count, l, r, dst);
+        case RT_SUB: return broadcast_typed<T, RT_SUB>(ctx, d, count, l, r, dst);
+        case RT_MUL: return broadcast_typed<T, RT_MUL>(ctx, d, count, l, r, dst);
+    }
+    return rt_fail(RT_E_INVALID, "broadcast: unknown op code %d", op);
+}
+
+}  // namespace
+
+// Row-major copy of the elements a view addresses (TensorView::owned / contiguous, core/tensor.rs:299-325).
+extern "C" int32_t rt_gather(rt_ctx* ctx, int32_t dtype, const void* src, uint64_t src_len, uint64_t offset, int32_t rank,
+                             const uint64_t* shape, const int64_t* strides, void* dst, uint64_t dst_len) {
+    RT_TRY(rt_ctx_enter(ctx));
+    const int es = rt_elem_size(dtype);
+    if (!es) return rt_fail(RT_E_DTYPE, "gather: unknown dtype code %d", dtype);
+    uint64_t count = 0;
+    RT_TRY(rt_check_extent("gather source", offset, rank, shape, strides, src_len, &count));
+    if (count > dst_len) return rt_fail(RT_E_OUT_OF_BOUNDS, "gather: %llu elements into a buffer of %llu", (unsigned long long)count, (unsigned long long)dst_len);
+    if (count == 0) return RT_OK;
+    if (!src || !dst) return rt_fail(RT_E_INVALID, "gather: null buffer");
+    // 128-bit elements move as pairs of 64-bit words: one more unit-stride dim of size 2
+    const int words = es == 16 ? 2 : 1;
+    uint64_t shp[RT_MAX_INPUT_RANK + 1];
+    int64_t sst[RT_MAX_INPUT_RANK + 1], dstr[RT_MAX_INPUT_RANK + 1];
+    int r2 = rank;
+    for (int i = 0; i < rank; ++i) { shp[i] = shape[i]; sst[i] = strides[i] * words; }
+    if (words == 2) { shp[rank] = 2; sst[rank] = 1; r2 = rank + 1; }
+    int64_t acc = 1;
+    for (int i = r2 - 1; i >= 0; --i) { dstr[i] = acc; acc *= (int64_t)shp[i]; }
+    NdDesc d;
+    const int64_t* sp[3] = {sst, sst, dstr};
+    const uint64_t offs[3] = {offset * words, offset * words, 0};
+    RT_TRY(rt_collapse(3, r2, shp, sp, offs, /*reorder=*/true, /*key=*/2, &d));
+    for (int k = 0; k < RT_MAX_RANK; ++k) d.stride[1][k] = 0;           // right operand: one element, never advanced
+    CtxGuard g(ctx);
+    const uint64_t n = count * words;
+    switch (es) {
+        case 1: return broadcast_typed<uint8_t, kOpCopy>(ctx, d, n, src, src, dst);
+        case 2: return broadcast_typed<uint16_t, kOpCopy>(ctx, d, n, src, src, dst);
+        case 4: return broadcast_typed<uint32_t, kOpCopy>(ctx, d, n, src, src, dst);
+        default: return broadcast_typed<uint64_t, kOpCopy>(ctx, d, n, src, src, dst);
+    }
+}
+
+extern "C" int32_t rt_broadcast(rt_ctx* ctx, int32_t dtype, int32_t op, int32_t rank, const uint64_t* shape,
+                                const void* left, uint64_t left_len, uint64_t left_offset, const int64_t* left_strides,
+                                const void* right, uint64_t right_len, uint64_t right_offset, const int64_t* right_strides,
+                                void* dst, uint64_t dst_len, uint64_t dst_offset, const int64_t* dst_strides) {
+    RT_TRY(rt_ctx_enter(ctx));
+    if (op < RT_ADD || op > RT_DIV) return rt_fail(RT_E_INVALID, "broadcast: unknown op code %d", op);
+    if (!rt_elem_size(dtype)) return rt_fail(RT_E_DTYPE, "broadcast: unknown dtype code %d", dtype);
+    uint64_t count = 0, c2 = 0, c3 = 0;
+    RT_TRY(rt_check_extent("broadcast left", left_offset, rank, shape, left_strides, left_len, &count));
+    RT_TRY(rt_check_extent("broadcast right", right_offset, rank, shape, right_strides, right_len, &c2));
+    RT_TRY(rt_check_extent("broadcast dst", dst_offset, rank, shape, dst_strides, dst_len, &c3));
+    if (count == 0) return RT_OK;
+    if (!left || !right || !dst) return rt_fail(RT_E_INVALID, "broadcast: null buffer");
+    for (int i = 0; i < rank; ++i)
+        if (shape[i] > 1 && dst_strides[i] == 0)
+            return rt_fail(RT_E_INVALID, "broadcast: destination has stride 0 along dim %d of size %llu (it would be written more than once)",
+                           i, (unsigned long long)shape[i]);
+    NdDesc d;
+    const int64_t* sp[3] = {left_strides, right_strides, dst_strides};
+    const uint64_t offs[3] = {left_offset, right_offset, dst_offset};
+    RT_TRY(rt_collapse(3, rank, shape, sp, offs, /*reorder=*/true, /*key=*/2, &d));
+    CtxGuard g(ctx);
+    if (op == RT_DIV) {
+        switch (dtype) {
+            case RT_U8: return broadcast_typed<uint8_t, RT_DIV>(ctx, d, count, left, right, dst);
+            case RT_I8: return broadcast_typed<int8_t, RT_DIV>(ctx, d, count, left, right, dst);
+            case RT_U16: return broadcast_typed<uint16_t, RT_DIV>(ctx, d, count, left, right, dst);
+            case RT_I16: return broadcast_typed<int16_t, RT_DIV>(ctx, d, count, left, right, dst);
+            case RT_U32: return broadcast_typed<uint32_t, RT_DIV>(ctx, d, count, left, right, dst);
+            case RT_I32: return broadcast_typed<int32_t, RT_DIV>(ctx, d, count, left, right, dst);
+            case RT_U64: return broadcast_typed<uint64_t, RT_DIV>(ctx, d, count, left, right, dst);
+            case RT_I64: return broadcast_typed<int64_t, RT_DIV>(ctx, d, count, left, right, dst);
+            case RT_F32: return broadcast_typed<float, RT_DIV>(ctx, d, count, left, right, dst);
+            case RT_F64: return broadcast_typed<double, RT_DIV>(ctx, d, count, left, right, dst);
+            case RT_BOOL: return rt_fail(RT_E_ARITH, "broadcast: division is not implemented for boolean in the reference (todo!())");
+        }
+        return rt_fail(RT_E_DTYPE, "broadcast: 128-bit integers are not built for the device");
+    }
+    // + - * on two's-complement integers do not depend on signedness: one instantiation per width
+    switch (dtype) {
+        case RT_U8: case RT_I8: return broadcast_ops<uint8_t>(ctx, op, d, count, left, right, dst);
+        case RT_U16: case RT_I16: return broadcast_ops<uint16_t>(ctx, op, d, count, left, right, dst);
+        case RT_U32: case RT_I32: return broadcast_ops<uint32_t>(ctx, op, d, count, left, right, dst);
+        case RT_U64: case RT_I64: return broadcast_ops<uint64_t>(ctx, op, d, count, left, right, dst);
+        case RT_F32: return broadcast_ops<float>(ctx, op, d, count, left, right, dst);
+        case RT_F64: return broadcast_ops<double>(ctx, op, d, count, left, right, dst);
+        case RT_BOOL: return broadcast_ops<boolean_t>(ctx, op, d, count, left, right, dst);
+    }
+    return rt_fail(RT_E_DTYPE, "broadcast: 128-bit integers are not built for the device");
+}

@@ -1,0 +1,116 @@
+// Internal definitions shared by the translation units of librt_hip.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <map>
+#include <mutex>
+#include <vector>
+
+#include "../../include/rt_hip.h"
+
+// ---- error plumbing ---------------------------------------------------------------------------------------------
+int32_t rt_fail(int32_t status, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+int32_t rt_hip_fail(hipError_t e, const char* what);
+
+#define RT_HIP(call)                                              \
+    do {                                                          \
+        hipError_t e__ = (call);                                  \
+        if (e__ != hipSuccess) return rt_hip_fail(e__, #call);    \
+    } while (0)
+
+#define RT_TRY(call)                                   \
+    do {                                               \
+        int32_t s__ = (call);                          \
+        if (s__ != RT_OK) return s__;                  \
+    } while (0)
+
+// ---- context ------------------------------------------------------------------------------------------------------
+// One stream per context; every launch and copy is enqueued on it, so a block returned to the free lists by
+// rt_free can be handed out again immediately: its next user runs after its previous user in stream order.
+struct rt_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    std::mutex mu;
+    // caching allocator: exact-size-class free lists
+    std::multimap<size_t, void*> free_blocks;      // capacity -> block
+    std::map<void*, size_t> live;                  // block -> capacity
+    uint64_t bytes_in_use = 0, bytes_cached = 0, device_allocs = 0;
+    // scratch for two-stage reductions (partials), grown on demand, reused across calls
+    void* scratch = nullptr;
+    size_t scratch_bytes = 0;
+    // one pinned 8-byte cell + device flag used by rt_equal / rt_read
+    int32_t* flag_dev = nullptr;
+    int num_cus = 256;
+};
+
+struct CtxGuard {
+    rt_ctx* c;
+    std::unique_lock<std::mutex> lk;
+    explicit CtxGuard(rt_ctx* ctx) : c(ctx), lk(ctx->mu) {}
+};
+
+int32_t rt_ctx_enter(rt_ctx* ctx);                                   // validates ctx and makes its device current
+int32_t rt_alloc_bytes(rt_ctx* ctx, size_t bytes, void** out);       // caller holds ctx->mu
+int32_t rt_free_locked(rt_ctx* ctx, void* p);
+int32_t rt_scratch(rt_ctx* ctx, size_t bytes, void** out);           // caller holds ctx->mu
+
+static inline int rt_elem_size(int dtype) {
+    switch (dtype) {
+        case RT_U8: case RT_I8: case RT_BOOL: return 1;
+        case RT_U16: case RT_I16: return 2;
+        case RT_U32: case RT_I32: case RT_F32: return 4;
+        case RT_U64: case RT_I64: case RT_F64: return 8;
+        case RT_U128: case RT_I128: return 16;
+    }
+    return 0;
+}
+
+// ---- descriptor validation and canonicalisation (host) -----------------------------------------------------------
+// check_extent of the reference's remote server (backend/remote/server.rs:241-270): lowest and highest addressed
+// element must lie inside [0, len).  Returns the element count through *count (0 when any dim is 0).
+int32_t rt_check_extent(const char* what, uint64_t offset, int rank, const uint64_t* shape, const int64_t* strides,
+                        uint64_t len, uint64_t* count);
+
+// A view over up to three operands sharing one shape, after removal of size-1 dims and merging of adjacent dims
+// that are mergeable in every operand.  Dim 0 is outermost.
+struct NdDesc {
+    int rank;
+    int64_t shape[RT_MAX_RANK];
+    int64_t stride[3][RT_MAX_RANK];
+    int64_t offset[3];
+};
+
+// Collapses `nops` operands (1..3).  When `reorder` is set (allowed whenever the visiting order of elements is
+// irrelevant, i.e. for every elementwise op), dims are first flipped so operand `key`'s strides are non-negative
+// and sorted by that operand's stride, largest first, which maximises merging and makes its accesses ascend.
+int32_t rt_collapse(int nops, int rank, const uint64_t* shape, const int64_t* const* strides, const uint64_t* offsets,
+                    bool reorder, int key, NdDesc* out);
+
+// ---- device helpers ------------------------------------------------------------------------------------------------
+#define RT_WAVE 64
+
+// Division of a 32-bit numerator by a runtime-constant divisor via multiply-high (round-up method); exact for
+// every n < 2^31 and 1 <= d < 2^31.
+struct FastDiv32 {
+    uint32_t d, mul, shift;
+};
+static inline FastDiv32 make_fastdiv(uint32_t d) {
+    FastDiv32 f;
+    f.d = d;
+    if (d == 1) { f.mul = 0; f.shift = 0; return f; }
+    uint32_t l = 32 - __builtin_clz(d - 1);                       // ceil(log2 d)
+    uint64_t m = (((uint64_t)1 << 32) * (((uint64_t)1 << l) - d)) / d + 1;
+    f.mul = (uint32_t)m;
+    f.shift = l;
+    return f;
+}
+__device__ __forceinline__ uint32_t fd_div(uint32_t n, const FastDiv32& f) {
+    if (f.d == 1) return n;
+    uint32_t t = __umulhi(n, f.mul);
+    return (uint32_t)(((uint64_t)t + n) >> f.shift);
+}

@@ -1,0 +1,574 @@
+// In-place elementwise family: fill, the 31 unary ops and the 8 scalar ops over the three layouts of the
+// reference's Backend trait (contiguous run, 1-D strided, N-d view).
+// Element definitions follow the reference's Cpu backend (backend/cpu.rs:485-724), which is the parity target:
+// e.g. relu is `x > 0 ? x : 0` (NaN -> 0, -0.0 -> +0.0) and sign(0) = 0.
+//
+// Memory behaviour: the contiguous kernel moves 16 bytes per lane per access (global_load/store_dwordx4), a whole
+// wavefront touching 1 KiB of consecutive addresses, UNROLL independent accesses in flight per lane.  Algorithmic
+// traffic is 2*N*sizeof(T) for read-modify-write ops and N*sizeof(T) for fill.
+#include "rt_common.h"
+
+#include <type_traits>
+
+namespace {
+
+// ---- element types ---------------------------------------------------------------------------------------------
+struct boolean_t { uint8_t v; };      // core/value.rs:650-765: + is OR, - is XOR, * is AND
+
+template <class T> struct is_flt : std::integral_constant<bool, std::is_same<T, float>::value || std::is_same<T, double>::value> {};
+template <class T> struct is_bool : std::is_same<T, boolean_t> {};
+template <class T> struct is_sint : std::integral_constant<bool, std::is_integral<T>::value && std::is_signed<T>::value> {};
+template <class T> struct is_uint : std::integral_constant<bool, std::is_integral<T>::value && std::is_unsigned<T>::value> {};
+
+template <class T, class E = void> struct carrier { typedef T type; };
+template <class T> struct carrier<T, typename std::enable_if<std::is_integral<T>::value && sizeof(T) <= 4>::type> { typedef uint32_t type; };
+template <class T> struct carrier<T, typename std::enable_if<std::is_integral<T>::value && sizeof(T) == 8>::type> { typedef uint64_t type; };
+
+// wrapping integer arithmetic (Rust release semantics) through an unsigned carrier; IEEE for floats
+template <class T> __device__ __forceinline__ T w_add(T a, T b) {
+    if constexpr (is_flt<T>::value) return a + b;
+    else if constexpr (is_bool<T>::value) return boolean_t{(uint8_t)(a.v | b.v)};
+    else { typedef typename carrier<T>::type W; return (T)(W)((W)a + (W)b); }
+}
+template <class T> __device__ __forceinline__ T w_sub(T a, T b) {
+    if constexpr (is_flt<T>::value) return a - b;
+    else if constexpr (is_bool<T>::value) return boolean_t{(uint8_t)(a.v ^ b.v)};
+    else { typedef typename carrier<T>::type W; return (T)(W)((W)a - (W)b); }
+}
+template <class T> __device__ __forceinline__ T w_mul(T a, T b) {
+    if constexpr (is_flt<T>::value) return a * b;
+    else if constexpr (is_bool<T>::value) return boolean_t{(uint8_t)(a.v & b.v)};
+    else { typedef typename carrier<T>::type W; return (T)(W)((W)a * (W)b); }
+}
+// Integer division truncates toward zero.  A zero divisor (and MIN / -1) panics in the reference; the host refuses
+// a zero scalar up front, and the device result for the remaining undefined cases is 0 / MIN respectively.
+template <class T> __device__ __forceinline__ T w_div(T a, T b) {
+    if constexpr (is_flt<T>::value) return a / b;
+    else if constexpr (is_bool<T>::value) return boolean_t{0};
+    else if constexpr (is_sint<T>::value) {
+        if (b == 0) return 0;
+        if (b == (T)-1) return w_sub<T>((T)0, a);
+        return (T)(a / b);
+    } else {
+        if (b == 0) return 0;
+        return (T)(a / b);
+    }
+}
+template <class T> __device__ __forceinline__ bool gt0(T x) {
+    if constexpr (is_bool<T>::value) return x.v != 0;
+    else return x > (T)0;
+}
+template <class T> __device__ __forceinline__ T zero_of() {
+    if constexpr (is_bool<T>::value) return boolean_t{0};
+    else return (T)0;
+}
+
+// libm spellings per precision
+__device__ __forceinline__ float m_exp(float x) { return expf(x); }
+__device__ __forceinline__ double m_exp(double x) { return exp(x); }
+__device__ __forceinline__ float m_expm1(float x) { return expm1f(x); }
+__device__ __forceinline__ double m_expm1(double x) { return expm1(x); }
+__device__ __forceinline__ float m_log(float x) { return logf(x); }
+__device__ __forceinline__ double m_log(double x) { return log(x); }
+__device__ __forceinline__ float m_log1p(float x) { return log1pf(x); }
+__device__ __forceinline__ double m_log1p(double x) { return log1p(x); }
+__device__ __forceinline__ float m_sqrt(float x) { return sqrtf(x); }
+__device__ __forceinline__ double m_sqrt(double x) { return sqrt(x); }
+__device__ __forceinline__ float m_sin(float x) { return sinf(x); }
+__device__ __forceinline__ double m_sin(double x) { return sin(x); }
+__device__ __forceinline__ float m_cos(float x) { return cosf(x); }
+__device__ __forceinline__ double m_cos(double x) { return cos(x); }
+__device__ __forceinline__ float m_tan(float x) { return tanf(x); }
+__device__ __forceinline__ double m_tan(double x) { return tan(x); }
+__device__ __forceinline__ float m_asin(float x) { return asinf(x); }
+__device__ __forceinline__ double m_asin(double x) { return asin(x); }
+__device__ __forceinline__ float m_acos(float x) { return acosf(x); }
+__device__ __forceinline__ double m_acos(double x) { return acos(x); }
+__device__ __forceinline__ float m_atan(float x) { return atanf(x); }
+__device__ __forceinline__ double m_atan(double x) { return atan(x); }
+__device__ __forceinline__ float m_floor(float x) { return floorf(x); }
+__device__ __forceinline__ double m_floor(double x) { return floor(x); }
+__device__ __forceinline__ float m_ceil(float x) { return ceilf(x); }
+__device__ __forceinline__ double m_ceil(double x) { return ceil(x); }
+__device__ __forceinline__ float m_round(float x) { return roundf(x); }     // half away from zero, like Rust's round()
+__device__ __forceinline__ double m_round(double x) { return round(x); }
+__device__ __forceinline__ float m_trunc(float x) { return truncf(x); }
+__device__ __forceinline__ double m_trunc(double x) { return trunc(x); }
+__device__ __forceinline__ float m_abs(float x) { return fabsf(x); }
+__device__ __forceinline__ double m_abs(double x) { return fabs(x); }
+
+// ---- functors ---------------------------------------------------------------------------------------------------
+template <int OP, class T> struct UnaryF {
+    static constexpr bool kReads = true;
+    __device__ __forceinline__ T operator()(T x) const {
+        if constexpr (OP == RT_U_RELU) {                                  // cpu.rs:650-657
+            return gt0(x) ? x : zero_of<T>();
+        } else if constexpr (OP == RT_U_ABS) {                            // core/value.rs:515-557
+            if constexpr (is_flt<T>::value) return m_abs(x);
+            else if constexpr (is_sint<T>::value) return x < 0 ? w_sub<T>((T)0, x) : x;
+            else return x;
+        } else if constexpr (OP == RT_U_NEG) {                            // cpu.rs:644-647
+            if constexpr (is_flt<T>::value) return -x;
+            else return w_sub<T>(zero_of<T>(), x);
+        } else {
+            const T one = (T)1;
+            if constexpr (OP == RT_U_SIGMOID) return one / (one + m_exp(-x));                     // cpu.rs:661-667
+            else if constexpr (OP == RT_U_SILU) return x * (one / (one + m_exp(-x)));             // cpu.rs:669-675
+            else if constexpr (OP == RT_U_TANH) { T a = m_exp(x), b = m_exp(-x); return (a - b) / (a + b); }   // cpu.rs:624-629
+            else if constexpr (OP == RT_U_SQRT) return m_sqrt(x);
+            else if constexpr (OP == RT_U_LN) return m_log(x);
+            else if constexpr (OP == RT_U_EXPM1) return m_expm1(x);
+            else if constexpr (OP == RT_U_LN1P) return m_log1p(x);
+            else if constexpr (OP == RT_U_FLOOR) return m_floor(x);
+            else if constexpr (OP == RT_U_CEIL) return m_ceil(x);
+            else if constexpr (OP == RT_U_ROUND) return m_round(x);
+            else if constexpr (OP == RT_U_TRUNC) return m_trunc(x);
+            else if constexpr (OP == RT_U_SIN) return m_sin(x);
+            else if constexpr (OP == RT_U_COS) return m_cos(x);
+            else if constexpr (OP == RT_U_TAN) return m_tan(x);
+            else if constexpr (OP == RT_U_ASIN) return m_asin(x);
+            else if constexpr (OP == RT_U_ACOS) return m_acos(x);
+            else if constexpr (OP == RT_U_ATAN) return m_atan(x);
+            else if constexpr (OP == RT_U_SINH) { T a = m_exp(x), b = m_exp(-x); return (a - b) / (one + one); }   // cpu.rs:485-490
+            else if constexpr (OP == RT_U_COSH) { T a = m_exp(x), b = m_exp(-x); return (a + b) / (one + one); }   // cpu.rs:492-497
+            else if constexpr (OP == RT_U_ASINH) { T sq = x * x; return m_log(x + m_sqrt(sq + one)); }              // cpu.rs:499-505
+            else if constexpr (OP == RT_U_ACOSH) { T sq = x * x; return m_log(x + m_sqrt(sq - one)); }              // cpu.rs:507-513
+            else if constexpr (OP == RT_U_ATANH) { T two = one + one; return m_log((one + x) / (one - x)) / two; }  // cpu.rs:515-521
+            else if constexpr (OP == RT_U_RSQRT) return one / m_sqrt(x);                          // cpu.rs:523-526
+            else if constexpr (OP == RT_U_RECIPROCAL) return one / x;                             // cpu.rs:528-531
+            else if constexpr (OP == RT_U_SQUARE) return x * x;                                   // cpu.rs:533-536
+            else if constexpr (OP == RT_U_CUBE) return x * x * x;                                 // cpu.rs:538-541
+            else if constexpr (OP == RT_U_EXP) return m_exp(x);
+            else if constexpr (OP == RT_U_SIGN) return x < (T)0 ? -one : (x > (T)0 ? one : (T)0);  // cpu.rs:548-557
+            else return x;
+        }
+    }
+};
+
+template <int OP, class T> struct ScalarF {
+    static constexpr bool kReads = true;
+    T v;
+    __device__ __forceinline__ T operator()(T x) const {
+        if constexpr (OP == RT_S_ADD) return w_add<T>(x, v);                                      // cpu.rs:678-696
+        else if constexpr (OP == RT_S_SUB) return w_sub<T>(x, v);
+        else if constexpr (OP == RT_S_MUL) return w_mul<T>(x, v);
+        else if constexpr (OP == RT_S_DIV) return w_div<T>(x, v);
+        else if constexpr (OP == RT_S_LEAKY_RELU) return gt0(x) ? x : w_mul<T>(x, v);             // cpu.rs:708-715
+        else if constexpr (OP == RT_S_LOG) return m_log(x) / m_log(v);                            // f32::log(base)
+        else if constexpr (OP == RT_S_LOG1P) return m_log1p(x) / m_log(v);                        // core/value.rs vlog1p
+        else if constexpr (OP == RT_S_ELU) return x >= (T)0 ? x : v * m_expm1(x);                 // cpu.rs:717-724
+        else return x;
+    }
+};
+
+template <class T> struct FillF {
+    static constexpr bool kReads = false;
+    T v;
+    __device__ __forceinline__ T operator()(T) const { return v; }
+};
+
+// ---- kernels ------------------------------------------------------------------------------------------------------
+template <class T> struct alignas(16) Vec16 { T e[16 / sizeof(T)]; };
+
+constexpr int kBlock = 256;
+constexpr int kUnroll = 4;      // 16-byte accesses in flight per lane
+
+// Body: `nvec` 16-byte vectors starting at the 16-byte aligned address `p`.
+template <class T, class F>
+__global__ __launch_bounds__(kBlock) void ew_contig_kernel(Vec16<T>* __restrict__ p, size_t nvec, F f) {
+    constexpr int N = 16 / sizeof(T);
+    const size_t base = (size_t)blockIdx.x * (kBlock * kUnroll) + threadIdx.x;
+    Vec16<T> v[kUnroll];
+    if (base + (size_t)(kUnroll - 1) * kBlock < nvec) {       // whole tile inside: no per-access predicate
+        if constexpr (F::kReads) {
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) v[u] = p[base + (size_t)u * kBlock];
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+#pragma unroll
+            for (int j = 0; j < N; ++j) v[u].e[j] = f(v[u].e[j]);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) p[base + (size_t)u * kBlock] = v[u];
+    } else {
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const size_t i = base + (size_t)u * kBlock;
+            if (i < nvec) {
+                Vec16<T> w;
+                if constexpr (F::kReads) w = p[i];
+#pragma unroll
+                for (int j = 0; j < N; ++j) w.e[j] = f(w.e[j]);
+                p[i] = w;
+            }
+        }
+    }
+}
+
+// Edges of a contiguous run that do not fill a 16-byte vector, and 1-D strided views: one element per lane.
+template <class T, class F>
+__global__ __launch_bounds__(kBlock) void ew_strided_kernel(T* __restrict__ p, int64_t stride, size_t n, F f) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * kBlock;
+    for (; i < n; i += step) {
+        T* q = p + (int64_t)i * stride;
+        T x = zero_of<T>();
+        if constexpr (F::kReads) x = *q;
+        *q = f(x);
+    }
+}
+
+struct NdArgs {
+    int rank;                        // >= 2
+    uint32_t shape[RT_MAX_RANK];
+    int64_t stride[RT_MAX_RANK];
+    FastDiv32 div[RT_MAX_RANK];
+};
+
+// N-d view, fewer than 2^31 elements: lane i handles the i-th element in row-major order of the collapsed dims.
+template <class T, class F>
+__global__ __launch_bounds__(kBlock) void ew_nd_kernel(T* __restrict__ p, NdArgs a, uint32_t n, F f) {
+    uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+    const uint32_t step = gridDim.x * kBlock;
+    for (; i < n; i += step) {
+        uint32_t rem = i;
+        int64_t off = 0;
+#pragma unroll
+        for (int d = RT_MAX_RANK - 1; d >= 0; --d) {
+            if (d < a.rank) {
+                uint32_t q = fd_div(rem, a.div[d]);
+                uint32_t c = rem - q * a.shape[d];
+                off += (int64_t)c * a.stride[d];
+                rem = q;
+            }
+        }
+        T* q = p + off;
+        T x = zero_of<T>();
+        if constexpr (F::kReads) x = *q;
+        *q = f(x);
+    }
+}
+
+// N-d view whose innermost collapsed dim is unit-stride: a block walks one row segment with 16-byte accesses when
+// the segment start is 16-byte aligned, element accesses otherwise.  grid.x enumerates (row, column tile).
+template <class T, class F>
+__global__ __launch_bounds__(kBlock) void ew_rows_kernel(T* __restrict__ p, NdArgs a, uint32_t tiles_per_row, FastDiv32 tdiv, F f) {
+    constexpr int N = 16 / sizeof(T);
+    const uint32_t row = fd_div(blockIdx.x, tdiv);
+    const uint32_t tile = blockIdx.x - row * tiles_per_row;
+    uint32_t rem = row;
+    int64_t off = 0;
+#pragma unroll
+    for (int d = RT_MAX_RANK - 2; d >= 0; --d) {
+        if (d < a.rank - 1) {
+            uint32_t q = fd_div(rem, a.div[d]);
+            uint32_t c = rem - q * a.shape[d];
+            off += (int64_t)c * a.stride[d];
+            rem = q;
+        }
+    }
+    const uint32_t L = a.shape[a.rank - 1];
+    T* rowp = p + off;
+    const uint32_t col0 = tile * (kBlock * N * kUnroll);
+    const bool aligned = ((reinterpret_cast<uintptr_t>(rowp) & 15) == 0);
+    if (aligned) {
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const uint32_t c = col0 + (u * kBlock + threadIdx.x) * N;
+            if (c + N <= L) {
+                Vec16<T>* q = reinterpret_cast<Vec16<T>*>(rowp + c);
+                Vec16<T> w;
+                if constexpr (F::kReads) w = *q;
+#pragma unroll
+                for (int j = 0; j < N; ++j) w.e[j] = f(w.e[j]);
+                *q = w;
+            } else {
+                for (uint32_t k = c; k < L && k < c + N; ++k) {
+                    T x = zero_of<T>();
+                    if constexpr (F::kReads) x = rowp[k];
+                    rowp[k] = f(x);
+                }
+            }
+        }
+    } else {
+        const uint32_t end = min(L, col0 + kBlock * N * kUnroll);
+        for (uint32_t k = col0 + threadIdx.x; k < end; k += kBlock) {
+            T x = zero_of<T>();
+            if constexpr (F::kReads) x = rowp[k];
+            rowp[k] = f(x);
+        }
+    }
+}
+
+// 64-bit fallback for views with 2^31 or more elements that are not a single contiguous run.
+template <class T, class F>
+__global__ __launch_bounds__(kBlock) void ew_nd64_kernel(T* __restrict__ p, NdDesc d, uint64_t n, F f) {
+    uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    const uint64_t step = (uint64_t)gridDim.x * kBlock;
+    for (; i < n; i += step) {
+        uint64_t rem = i;
+        int64_t off = 0;
+        for (int k = d.rank - 1; k >= 0; --k) {
+            uint64_t q = rem / (uint64_t)d.shape[k];
+            off += (int64_t)(rem - q * (uint64_t)d.shape[k]) * d.stride[0][k];
+            rem = q;
+        }
+        T* q = p + off;
+        T x = zero_of<T>();
+        if constexpr (F::kReads) x = *q;
+        *q = f(x);
+    }
+}
+
+// ---- launch logic ---------------------------------------------------------------------------------------------------
+static inline unsigned capped_grid(size_t blocks, size_t cap) { return (unsigned)(blocks < 1 ? 1 : (blocks > cap ? cap : blocks)); }
+
+template <class T, class F>
+int32_t launch_contig(rt_ctx* ctx, T* p, size_t n, F f) {
+    if (n == 0) return RT_OK;
+    constexpr size_t N = 16 / sizeof(T);
+    uintptr_t addr = reinterpret_cast<uintptr_t>(p);
+    size_t head = ((16 - (addr & 15)) & 15) / sizeof(T);
+    if (head > n) head = n;
+    size_t nvec = (n - head) / N;
+    size_t tail = n - head - nvec * N;
+    if (nvec) {
+        size_t blocks = (nvec + (size_t)kBlock * kUnroll - 1) / ((size_t)kBlock * kUnroll);
+        if (blocks > 0x7fffffffull) return rt_fail(RT_E_INVALID, "contiguous run of %zu elements is too long for one launch", n);
+        hipLaunchKernelGGL((ew_contig_kernel<T, F>), dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream,
+                           reinterpret_cast<Vec16<T>*>(p + head), nvec, f);
+    }
+    if (head) hipLaunchKernelGGL((ew_strided_kernel<T, F>), dim3(1), dim3(kBlock), 0, ctx->stream, p, (int64_t)1, head, f);
+    if (tail) hipLaunchKernelGGL((ew_strided_kernel<T, F>), dim3(1), dim3(kBlock), 0, ctx->stream, p + head + nvec * N, (int64_t)1, tail, f);
+    RT_HIP(hipGetLastError());
+    return RT_OK;
+}
+
+// `d` is the collapsed single-operand view (operand 0), any element order allowed.
+template <class T, class F>
+int32_t launch_view(rt_ctx* ctx, T* base, const NdDesc& d, uint64_t count, F f) {
+    if (count == 0) return RT_OK;
+    T* p = base + d.offset[0];
+    if (d.rank == 0) return launch_contig<T, F>(ctx, p, 1, f);
+    if (d.rank == 1) {
+        if (d.stride[0][0] == 1) return launch_contig<T, F>(ctx, p, (size_t)d.shape[0], f);
+        size_t blocks = ((size_t)d.shape[0] + kBlock - 1) / kBlock;
+        hipLaunchKernelGGL((ew_strided_kernel<T, F>), dim3(capped_grid(blocks, (size_t)ctx->num_cus * 32)), dim3(kBlock), 0, ctx->stream,
+                           p, d.stride[0][0], (size_t)d.shape[0], f);
+        RT_HIP(hipGetLastError());
+        return RT_OK;
+    }
+    if (count >= (1ull << 31)) {
+        size_t blocks = (size_t)((count + kBlock - 1) / kBlock);
+        hipLaunchKernelGGL((ew_nd64_kernel<T, F>), dim3(capped_grid(blocks, (size_t)ctx->num_cus * 64)), dim3(kBlock), 0, ctx->stream,
+                           p, d, count, f);
+        RT_HIP(hipGetLastError());
+        return RT_OK;
+    }
+    NdArgs a;
+    a.rank = d.rank;
+    for (int i = 0; i < RT_MAX_RANK; ++i) {
+        a.shape[i] = i < d.rank ? (uint32_t)d.shape[i] : 1;
+        a.stride[i] = i < d.rank ? d.stride[0][i] : 0;
+        a.div[i] = make_fastdiv(a.shape[i]);
+    }
+    constexpr uint32_t N = 16 / sizeof(T);
+    const uint32_t L = a.shape[d.rank - 1];
+    if (d.stride[0][d.rank - 1] == 1 && L >= 4 * N) {
+        const uint32_t per_tile = kBlock * N * kUnroll;
+        const uint32_t tiles = (L + per_tile - 1) / per_tile;
+        const uint64_t rows = count / L;
+        if (rows * tiles < (1ull << 31)) {
+            hipLaunchKernelGGL((ew_rows_kernel<T, F>), dim3((unsigned)(rows * tiles)), dim3(kBlock), 0, ctx->stream,
+                               p, a, tiles, make_fastdiv(tiles), f);
+            RT_HIP(hipGetLastError());
+            return RT_OK;
+        }
+    }
+    size_t blocks = ((size_t)count + kBlock - 1) / kBlock;
+    hipLaunchKernelGGL((ew_nd_kernel<T, F>), dim3(capped_grid(blocks, (size_t)ctx->num_cus * 64)), dim3(kBlock), 0, ctx->stream,
+                       p, a, (uint32_t)count, f);
+    RT_HIP(hipGetLastError());
+    return RT_OK;
+}
+
+// validate + collapse one in-place view, then run F over it
+template <class T, class F>
+int32_t run_inplace(rt_ctx* ctx, const char* what, void* buf, uint64_t buf_len, uint64_t offset, int rank,
+                    const uint64_t* shape, const int64_t* strides, F f) {
+    uint64_t count = 0;
+    RT_TRY(rt_check_extent(what, offset, rank, shape, strides, buf_len, &count));
+    if (count == 0) return RT_OK;
+    if (!buf) return rt_fail(RT_E_INVALID, "%s: null buffer", what);
+    for (int i = 0; i < rank; ++i)
+        if (shape[i] > 1 && strides[i] == 0)
+            return rt_fail(RT_E_INVALID, "%s: an in-place op over a zero-stride dim would write one element %llu times", what,
+                           (unsigned long long)shape[i]);
+    NdDesc d;
+    const int64_t* sp[1] = {strides};
+    RT_TRY(rt_collapse(1, rank, shape, sp, &offset, /*reorder=*/true, 0, &d));
+    CtxGuard g(ctx);
+    return launch_view<T, F>(ctx, (T*)buf, d, count, f);
+}
+
+template <class T> T load_scalar(const void* v) { T x; memcpy(&x, v, sizeof(T)); return x; }
+
+// ---- dtype / op dispatch ----------------------------------------------------------------------------------------------
+#define RT_FOR_DTYPE(dtype, BODY)                                           \
+    switch (dtype) {                                                        \
+        case RT_U8: { typedef uint8_t T; BODY; } break;                     \
+        case RT_I8: { typedef int8_t T; BODY; } break;                      \
+        case RT_U16: { typedef uint16_t T; BODY; } break;                   \
+        case RT_I16: { typedef int16_t T; BODY; } break;                    \
+        case RT_U32: { typedef uint32_t T; BODY; } break;                   \
+        case RT_I32: { typedef int32_t T; BODY; } break;                    \
+        case RT_U64: { typedef uint64_t T; BODY; } break;                   \
+        case RT_I64: { typedef int64_t T; BODY; } break;                    \
+        case RT_F32: { typedef float T; BODY; } break;                      \
+        case RT_F64: { typedef double T; BODY; } break;                     \
+        case RT_BOOL: { typedef boolean_t T; BODY; } break;                 \
+        default: break;                                                     \
+    }
+
+int32_t no_dtype(const char* what, int dtype) {
+    if (dtype == RT_U128 || dtype == RT_I128) return rt_fail(RT_E_DTYPE, "%s: 128-bit integers are not built for the device", what);
+    return rt_fail(RT_E_DTYPE, "%s: unknown dtype code %d", what, dtype);
+}
+
+int32_t fill_any(rt_ctx* ctx, int32_t dtype, void* buf, uint64_t buf_len, const void* value, uint64_t offset, int rank,
+                 const uint64_t* shape, const int64_t* strides) {
+    RT_TRY(rt_ctx_enter(ctx));
+    if (!value) return rt_fail(RT_E_INVALID, "fill: null value");
+    RT_FOR_DTYPE(dtype, return (run_inplace<T, FillF<T>>(ctx, "fill", buf, buf_len, offset, rank, shape, strides, FillF<T>{load_scalar<T>(value)})));
+    return no_dtype("fill", dtype);
+}
+
+template <class T, int OP>
+int32_t unary_go(rt_ctx* ctx, void* buf, uint64_t buf_len, uint64_t offset, int rank, const uint64_t* shape, const int64_t* strides) {
+    return run_inplace<T, UnaryF<OP, T>>(ctx, "unary", buf, buf_len, offset, rank, shape, strides, UnaryF<OP, T>{});
+}
+
+template <class T>
+int32_t unary_float(rt_ctx* ctx, int op, void* buf, uint64_t buf_len, uint64_t offset, int rank, const uint64_t* shape, const int64_t* strides) {
+#define RT_UCASE(OP) case OP: return unary_go<T, OP>(ctx, buf, buf_len, offset, rank, shape, strides)
+    switch (op) {
+        RT_UCASE(RT_U_NEG); RT_UCASE(RT_U_RELU); RT_UCASE(RT_U_SIGMOID); RT_UCASE(RT_U_SILU); RT_UCASE(RT_U_TANH); RT_UCASE(RT_U_ABS);
+        RT_UCASE(RT_U_SQRT); RT_UCASE(RT_U_LN); RT_UCASE(RT_U_EXPM1); RT_UCASE(RT_U_LN1P); RT_UCASE(RT_U_FLOOR); RT_UCASE(RT_U_CEIL);
+        RT_UCASE(RT_U_ROUND); RT_UCASE(RT_U_TRUNC); RT_UCASE(RT_U_SIN); RT_UCASE(RT_U_COS); RT_UCASE(RT_U_TAN); RT_UCASE(RT_U_ASIN);
+        RT_UCASE(RT_U_ACOS); RT_UCASE(RT_U_ATAN); RT_UCASE(RT_U_SINH); RT_UCASE(RT_U_COSH); RT_UCASE(RT_U_ASINH); RT_UCASE(RT_U_ACOSH);
+        RT_UCASE(RT_U_ATANH); RT_UCASE(RT_U_RSQRT); RT_UCASE(RT_U_RECIPROCAL); RT_UCASE(RT_U_SQUARE); RT_UCASE(RT_U_CUBE);
+        RT_UCASE(RT_U_EXP); RT_UCASE(RT_U_SIGN);
+    }
+#undef RT_UCASE
+    return rt_fail(RT_E_INVALID, "unary: unknown op code %d", op);
+}
+
+// Non-float dtypes: relu and abs for every dtype, neg for the signed ones (trait bounds, backend/mod.rs:311-355).
+template <class T>
+int32_t unary_other(rt_ctx* ctx, int op, void* buf, uint64_t buf_len, uint64_t offset, int rank, const uint64_t* shape, const int64_t* strides) {
+    if (op < 0 || op >= RT_U_COUNT) return rt_fail(RT_E_INVALID, "unary: unknown op code %d", op);
+    if (op == RT_U_RELU) return unary_go<T, RT_U_RELU>(ctx, buf, buf_len, offset, rank, shape, strides);
+    if (op == RT_U_ABS) return unary_go<T, RT_U_ABS>(ctx, buf, buf_len, offset, rank, shape, strides);
+    if constexpr (is_sint<T>::value) {
+        if (op == RT_U_NEG) return unary_go<T, RT_U_NEG>(ctx, buf, buf_len, offset, rank, shape, strides);
+    }
+    return rt_fail(RT_E_DTYPE, "unary op %d is not defined for this dtype (the reference bounds it on f32/f64)", op);
+}
+
+int32_t unary_any(rt_ctx* ctx, int32_t dtype, int32_t op, void* buf, uint64_t buf_len, uint64_t offset, int rank,
+                  const uint64_t* shape, const int64_t* strides) {
+    RT_TRY(rt_ctx_enter(ctx));
+    if (dtype == RT_F32) return unary_float<float>(ctx, op, buf, buf_len, offset, rank, shape, strides);
+    if (dtype == RT_F64) return unary_float<double>(ctx, op, buf, buf_len, offset, rank, shape, strides);
+    RT_FOR_DTYPE(dtype, return unary_other<T>(ctx, op, buf, buf_len, offset, rank, shape, strides));
+    return no_dtype("unary", dtype);
+}
+
+template <class T, int OP>
+int32_t scalar_go(rt_ctx* ctx, void* buf, uint64_t buf_len, const void* value, uint64_t offset, int rank, const uint64_t* shape,
+                  const int64_t* strides) {
+    return run_inplace<T, ScalarF<OP, T>>(ctx, "scalar", buf, buf_len, offset, rank, shape, strides, ScalarF<OP, T>{load_scalar<T>(value)});
+}
+
+template <class T>
+int32_t scalar_typed(rt_ctx* ctx, int op, void* buf, uint64_t buf_len, const void* value, uint64_t offset, int rank,
+                     const uint64_t* shape, const int64_t* strides) {
+    switch (op) {
+        case RT_S_ADD: return scalar_go<T, RT_S_ADD>(ctx, buf, buf_len, value, offset, rank, shape, strides);
+        case RT_S_SUB: return scalar_go<T, RT_S_SUB>(ctx, buf, buf_len, value, offset, rank, shape, strides);
+        case RT_S_MUL: return scalar_go<T, RT_S_MUL>(ctx, buf, buf_len, value, offset, rank, shape, strides);
+        case RT_S_LEAKY_RELU: return scalar_go<T, RT_S_LEAKY_RELU>(ctx, buf, buf_len, value, offset, rank, shape, strides);
+        case RT_S_DIV:
+            if constexpr (is_bool<T>::value) {
+                return rt_fail(RT_E_ARITH, "scalar div: division is not implemented for boolean in the reference (todo!())");
+            } else {
+                if constexpr (!is_flt<T>::value) {
+                    if (load_scalar<T>(value) == (T)0) return rt_fail(RT_E_ARITH, "scalar div: integer division by zero (the reference panics)");
+                }
+                return scalar_go<T, RT_S_DIV>(ctx, buf, buf_len, value, offset, rank, shape, strides);
+            }
+        case RT_S_LOG: case RT_S_LOG1P: case RT_S_ELU:
+            if constexpr (is_flt<T>::value) {
+                if (op == RT_S_LOG) return scalar_go<T, RT_S_LOG>(ctx, buf, buf_len, value, offset, rank, shape, strides);
+                if (op == RT_S_LOG1P) return scalar_go<T, RT_S_LOG1P>(ctx, buf, buf_len, value, offset, rank, shape, strides);
+                return scalar_go<T, RT_S_ELU>(ctx, buf, buf_len, value, offset, rank, shape, strides);
+            } else {
+                return rt_fail(RT_E_DTYPE, "scalar op %d is only defined for f32/f64", op);
+            }
+    }
+    return rt_fail(RT_E_INVALID, "scalar: unknown op code %d", op);
+}
+
+int32_t scalar_any(rt_ctx* ctx, int32_t dtype, int32_t op, void* buf, uint64_t buf_len, const void* value, uint64_t offset, int rank,
+                   const uint64_t* shape, const int64_t* strides) {
+    RT_TRY(rt_ctx_enter(ctx));
+    if (!value) return rt_fail(RT_E_INVALID, "scalar: null value");
+    RT_FOR_DTYPE(dtype, return scalar_typed<T>(ctx, op, buf, buf_len, value, offset, rank, shape, strides));
+    return no_dtype("scalar", dtype);
+}
+
+}  // namespace
+
+// ---- C ABI ------------------------------------------------------------------------------------------------------------
+// The `_contiguous` and `_1d_strided` forms are the N-d form with one dim; all three canonicalise the layout on the
+// host (signed strides: a reversed view is walked backwards, it is never mistaken for a forward run).
+extern "C" int32_t rt_fill_contiguous(rt_ctx* ctx, int32_t dtype, void* buf, uint64_t buf_len, const void* value, uint64_t start, uint64_t len) {
+    const int64_t one = 1;
+    return fill_any(ctx, dtype, buf, buf_len, value, start, 1, &len, &one);
+}
+extern "C" int32_t rt_fill_1d_strided(rt_ctx* ctx, int32_t dtype, void* buf, uint64_t buf_len, const void* value, uint64_t offset,
+                                      int64_t stride, uint64_t len) {
+    return fill_any(ctx, dtype, buf, buf_len, value, offset, 1, &len, &stride);
+}
+extern "C" int32_t rt_fill_nd(rt_ctx* ctx, int32_t dtype, void* buf, uint64_t buf_len, const void* value, uint64_t offset, int32_t rank,
+                              const uint64_t* shape, const int64_t* strides) {
+    return fill_any(ctx, dtype, buf, buf_len, value, offset, rank, shape, strides);
+}
+
+extern "C" int32_t rt_unary_contiguous(rt_ctx* ctx, int32_t dtype, int32_t op, void* buf, uint64_t buf_len, uint64_t start, uint64_t len) {
+    const int64_t one = 1;
+    return unary_any(ctx, dtype, op, buf, buf_len, start, 1, &len, &one);
+}
+extern "C" int32_t rt_unary_1d_strided(rt_ctx* ctx, int32_t dtype, int32_t op, void* buf, uint64_t buf_len, uint64_t offset, int64_t stride,
+                                       uint64_t len) {
+    return unary_any(ctx, dtype, op, buf, buf_len, offset, 1, &len, &stride);
+}
+extern "C" int32_t rt_unary_nd(rt_ctx* ctx, int32_t dtype, int32_t op, void* buf, uint64_t buf_len, uint64_t offset, int32_t rank,
+                               const uint64_t* shape, const int64_t* strides) {
+    return unary_any(ctx, dtype, op, buf, buf_len, offset, rank, shape, strides);
+}
+
+extern "C" int32_t rt_scalar_contiguous(rt_ctx* ctx, int32_t dtype, int32_t op, void* buf, uint64_t buf_len, const void* value,
+                                        uint64_t start, uint64_t len) {
+    const int64_t one = 1;
+    return scalar_any(ctx, dtype, op, buf, buf_len, value, start, 1, &len, &one);
+}
+extern "C" int32_t rt_scalar_1d_strided(rt_ctx* ctx, int32_t dtype, int32_t op, void* buf, uint64_t buf_len, const void* value,
+                                        uint64_t offset, int64_t stride, uint64_t len) {
+    return scalar_any(ctx, dtype, op, buf, buf_len, value, offset, 1, &len, &stride);
+}
+extern "C" int32_t rt_scalar_nd(rt_ctx* ctx, int32_t dtype, int32_t op, void* buf, uint64_t buf_len, const void* value, uint64_t offset,
+                                int32_t rank, const uint64_t* shape, const int64_t* strides) {
+    return scalar_any(ctx, dtype, op, buf, buf_len, value, offset, rank, shape, strides);
+}

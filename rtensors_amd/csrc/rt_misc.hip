@@ -1,0 +1,153 @@
+// Buffer equality (PartialEq of Backend::Buf) and dtype conversion (Backend::convert).
+#include "rt_common.h"
+
+#include <type_traits>
+#include <limits>
+
+namespace {
+
+constexpr int kBlock = 256;
+
+__global__ void set_flag_kernel(int32_t* flag, int32_t v) { *flag = v; }
+
+// `==` per element: NaN != NaN, -0.0 == 0.0 (what Box<[T]> == Box<[T]> gives; the reference's device version is
+// K/kernels/utils/buffer_equal.cu:7-39).  All lanes that see a mismatch store the same value.
+template <class T>
+__global__ __launch_bounds__(kBlock) void equal_kernel(const T* __restrict__ a, const T* __restrict__ b, size_t n, int32_t* flag) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * kBlock;
+    bool bad = false;
+    for (; i < n; i += step) bad = bad || !(a[i] == b[i]);
+    if (bad) *flag = 0;
+}
+
+template <class T>
+int32_t equal_typed(rt_ctx* ctx, const void* a, const void* b, size_t n) {
+    size_t blocks = (n + kBlock - 1) / kBlock;
+    size_t cap = (size_t)ctx->num_cus * 32;
+    hipLaunchKernelGGL((equal_kernel<T>), dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(kBlock), 0, ctx->stream,
+                       (const T*)a, (const T*)b, n, ctx->flag_dev);
+    RT_HIP(hipGetLastError());
+    return RT_OK;
+}
+
+// ---- convert: `T::convert::<N>` (core/value.rs:255-462) ---------------------------------------------------------------
+// float -> int : round half away from zero, then Rust's saturating `as` (NaN -> 0)
+// int   -> int : Rust `as` (truncate / sign-extend)
+// any   -> bool: x != 0;   bool -> any: 0 / 1
+struct boolean_t { uint8_t v; };
+template <class T> struct is_flt : std::integral_constant<bool, std::is_same<T, float>::value || std::is_same<T, double>::value> {};
+template <class T> struct is_bool : std::is_same<T, boolean_t> {};
+
+template <class D, class S> __device__ __forceinline__ D convert_one(S x) {
+    if constexpr (is_bool<D>::value) {
+        if constexpr (is_bool<S>::value) return x;
+        else return boolean_t{(uint8_t)(x != (S)0)};
+    } else if constexpr (is_bool<S>::value) {
+        return (D)(x.v ? 1 : 0);
+    } else if constexpr (is_flt<S>::value && !is_flt<D>::value) {
+        S r = std::is_same<S, float>::value ? (S)roundf((float)x) : (S)round((double)x);
+        if (r != r) return (D)0;
+        // bounds as doubles/floats: lowest is exact; max+1 is a power of two and exact
+        const S lo = (S)std::numeric_limits<D>::lowest();
+        const S hi_p1 = (S)2 * (S)((std::numeric_limits<D>::max() >> 1) + 1);
+        if (r <= lo) return std::numeric_limits<D>::lowest();
+        if (r >= hi_p1) return std::numeric_limits<D>::max();
+        return (D)r;
+    } else {
+        return (D)x;
+    }
+}
+
+template <class S, class D>
+__global__ __launch_bounds__(kBlock) void convert_kernel(const S* __restrict__ s, D* __restrict__ d, size_t n) {
+    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * kBlock;
+    for (; i < n; i += step) d[i] = convert_one<D, S>(s[i]);
+}
+
+template <class S, class D>
+int32_t convert_go(rt_ctx* ctx, const void* s, void* d, size_t n) {
+    size_t blocks = (n + kBlock - 1) / kBlock;
+    size_t cap = (size_t)ctx->num_cus * 32;
+    hipLaunchKernelGGL((convert_kernel<S, D>), dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(kBlock), 0, ctx->stream,
+                       (const S*)s, (D*)d, n);
+    RT_HIP(hipGetLastError());
+    return RT_OK;
+}
+
+#define RT_DST_CASES(S)                                                            \
+    switch (dd) {                                                                  \
+        case RT_U8: return convert_go<S, uint8_t>(ctx, s, d, n);                   \
+        case RT_I8: return convert_go<S, int8_t>(ctx, s, d, n);                    \
+        case RT_U16: return convert_go<S, uint16_t>(ctx, s, d, n);                 \
+        case RT_I16: return convert_go<S, int16_t>(ctx, s, d, n);                  \
+        case RT_U32: return convert_go<S, uint32_t>(ctx, s, d, n);                 \
+        case RT_I32: return convert_go<S, int32_t>(ctx, s, d, n);                  \
+        case RT_U64: return convert_go<S, uint64_t>(ctx, s, d, n);                 \
+        case RT_I64: return convert_go<S, int64_t>(ctx, s, d, n);                  \
+        case RT_F32: return convert_go<S, float>(ctx, s, d, n);                    \
+        case RT_F64: return convert_go<S, double>(ctx, s, d, n);                   \
+        case RT_BOOL: return convert_go<S, boolean_t>(ctx, s, d, n);               \
+    }                                                                              \
+    break;
+
+int32_t convert_any(rt_ctx* ctx, int sd, const void* s, int dd, void* d, size_t n) {
+    switch (sd) {
+        case RT_U8: RT_DST_CASES(uint8_t)
+        case RT_I8: RT_DST_CASES(int8_t)
+        case RT_U16: RT_DST_CASES(uint16_t)
+        case RT_I16: RT_DST_CASES(int16_t)
+        case RT_U32: RT_DST_CASES(uint32_t)
+        case RT_I32: RT_DST_CASES(int32_t)
+        case RT_U64: RT_DST_CASES(uint64_t)
+        case RT_I64: RT_DST_CASES(int64_t)
+        case RT_F32: RT_DST_CASES(float)
+        case RT_F64: RT_DST_CASES(double)
+        case RT_BOOL: RT_DST_CASES(boolean_t)
+    }
+    return rt_fail(RT_E_DTYPE, "convert: dtype pair (%d -> %d) is not built for the device", sd, dd);
+}
+
+}  // namespace
+
+extern "C" int32_t rt_equal(rt_ctx* ctx, int32_t dtype, const void* a, uint64_t a_len, const void* b, uint64_t b_len, int32_t* out_equal) {
+    RT_TRY(rt_ctx_enter(ctx));
+    if (!out_equal) return rt_fail(RT_E_INVALID, "rt_equal: null out");
+    int es = rt_elem_size(dtype);
+    if (!es) return rt_fail(RT_E_DTYPE, "rt_equal: unknown dtype code %d", dtype);
+    if (a_len != b_len) { *out_equal = 0; return RT_OK; }
+    if (a_len == 0) { *out_equal = 1; return RT_OK; }
+    if (!a || !b) return rt_fail(RT_E_INVALID, "rt_equal: null buffer");
+    CtxGuard g(ctx);
+    hipLaunchKernelGGL(set_flag_kernel, dim3(1), dim3(1), 0, ctx->stream, ctx->flag_dev, 1);
+    int32_t rc;
+    switch (dtype) {
+        // integers and bool: bitwise equality of the element is `==`
+        case RT_U8: case RT_I8: case RT_BOOL: rc = equal_typed<uint8_t>(ctx, a, b, a_len); break;
+        case RT_U16: case RT_I16: rc = equal_typed<uint16_t>(ctx, a, b, a_len); break;
+        case RT_U32: case RT_I32: rc = equal_typed<uint32_t>(ctx, a, b, a_len); break;
+        case RT_U64: case RT_I64: rc = equal_typed<uint64_t>(ctx, a, b, a_len); break;
+        case RT_U128: case RT_I128: rc = equal_typed<uint64_t>(ctx, a, b, a_len * 2); break;
+        case RT_F32: rc = equal_typed<float>(ctx, a, b, a_len); break;
+        default: rc = equal_typed<double>(ctx, a, b, a_len); break;
+    }
+    if (rc != RT_OK) return rc;
+    int32_t host = 0;
+    RT_HIP(hipMemcpyAsync(&host, ctx->flag_dev, sizeof(host), hipMemcpyDeviceToHost, ctx->stream));
+    RT_HIP(hipStreamSynchronize(ctx->stream));
+    *out_equal = host;
+    return RT_OK;
+}
+
+extern "C" int32_t rt_convert(rt_ctx* ctx, int32_t src_dtype, const void* src, uint64_t src_len, int32_t dst_dtype, void* dst, uint64_t dst_len) {
+    RT_TRY(rt_ctx_enter(ctx));
+    if (!rt_elem_size(src_dtype) || !rt_elem_size(dst_dtype)) return rt_fail(RT_E_DTYPE, "convert: unknown dtype code");
+    if (src_len != dst_len)
+        return rt_fail(RT_E_SIZE_MISMATCH, "Buffer size mismatch in convert: src size %llu, dst size %llu", (unsigned long long)src_len,
+                       (unsigned long long)dst_len);
+    if (src_len == 0) return RT_OK;
+    if (!src || !dst) return rt_fail(RT_E_INVALID, "convert: null buffer");
+    CtxGuard g(ctx);
+    return convert_any(ctx, src_dtype, src, dst_dtype, dst, (size_t)src_len);
+}

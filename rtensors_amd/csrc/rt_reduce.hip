@@ -1,0 +1,479 @@
+// Reductions: sum / prod / max / min / mean, full (flat) and along one axis of a row-major contiguous tensor viewed
+// as (outer, R, inner).  Replaces Backend::apply_reduce_contiguous_flat / _nd (backend/mod.rs:357-409); element
+// rules are the Cpu backend's accumulators (ops/reduction/mod.rs:9-137; loops backend/cpu.rs:397-449).  The
+// reference's CUDA path (K/kernels/reduction/reduce.cu:239-274, 463-513) is CUB two-pass + one block per output.
+//
+// Kernels (all HBM-bound, algorithmic traffic (N_in + N_out) * sizeof(T)):
+//   rows  (inner == 1): a block (or a wave, or a lane, depending on R) folds one contiguous row segment with
+//                       16-byte loads, wave64 shuffle reduction, LDS across the waves of a block.
+//   cols  (inner  > 1): lanes run along `inner` (coalesced, 16 bytes per lane), the four waves of a block take
+//                       interleaved k, combined through LDS.
+//   Both split R over several blocks when there are too few outputs to fill the chip; the partial results go to a
+//   scratch buffer and a second launch of the same kernel folds them (two-stage grid reduction, deterministic:
+//   no atomics, fixed combination order).
+//
+// Exactness: integer sum/prod wrap, so any association gives the sequential result; max/min are order independent
+// except for the sign of a zero result (-0.0 == 0.0, the sequential loop keeps the first), which is kept by
+// carrying the position of the current extremum.  Float sum/prod/mean are tree results.
+#include "rt_common.h"
+
+#include <type_traits>
+#include <limits>
+
+namespace {
+
+template <class T> struct is_flt : std::integral_constant<bool, std::is_same<T, float>::value || std::is_same<T, double>::value> {};
+
+template <class T, class E = void> struct carrier { typedef T type; };
+template <class T> struct carrier<T, typename std::enable_if<std::is_integral<T>::value && sizeof(T) <= 4>::type> { typedef uint32_t type; };
+template <class T> struct carrier<T, typename std::enable_if<std::is_integral<T>::value && sizeof(T) == 8>::type> { typedef uint64_t type; };
+
+template <class T> __device__ __host__ constexpr T lowest_of() { return std::numeric_limits<T>::lowest(); }   // T::MIN
+template <class T> __device__ __host__ constexpr T highest_of() { return std::numeric_limits<T>::max(); }     // T::MAX
+
+constexpr int kBlock = 256;
+constexpr int kWaves = kBlock / RT_WAVE;
+
+// Accumulator state.  `pos` is only carried for float max/min (see the header comment).
+template <int OP, class T> struct Acc {
+    static constexpr bool kTrack = is_flt<T>::value && (OP == RT_R_MAX || OP == RT_R_MIN);
+    T v;
+    uint64_t pos;
+
+    __device__ __forceinline__ void init() {
+        if constexpr (OP == RT_R_SUM || OP == RT_R_MEAN) v = (T)0;
+        else if constexpr (OP == RT_R_PROD) v = (T)1;
+        else if constexpr (OP == RT_R_MAX) v = lowest_of<T>();
+        else v = highest_of<T>();
+        pos = ~0ull;
+    }
+    // fold one element that comes after everything folded so far (ascending position)
+    __device__ __forceinline__ void push(T x, uint64_t p) {
+        if constexpr (OP == RT_R_SUM || OP == RT_R_MEAN) {
+            if constexpr (is_flt<T>::value) v = v + x;
+            else { typedef typename carrier<T>::type W; v = (T)(W)((W)v + (W)x); }
+        } else if constexpr (OP == RT_R_PROD) {
+            if constexpr (is_flt<T>::value) v = v * x;
+            else { typedef typename carrier<T>::type W; v = (T)(W)((W)v * (W)x); }
+        } else if constexpr (OP == RT_R_MAX) {
+            if (x > v) { v = x; if constexpr (kTrack) pos = p; }            // NaN never wins; first of equals stays
+        } else {
+            if (x < v) { v = x; if constexpr (kTrack) pos = p; }
+        }
+    }
+    // merge another partial state (any relative order)
+    __device__ __forceinline__ void merge(const Acc& o) {
+        if constexpr (OP == RT_R_SUM || OP == RT_R_MEAN) {
+            if constexpr (is_flt<T>::value) v = v + o.v;
+            else { typedef typename carrier<T>::type W; v = (T)(W)((W)v + (W)o.v); }
+        } else if constexpr (OP == RT_R_PROD) {
+            if constexpr (is_flt<T>::value) v = v * o.v;
+            else { typedef typename carrier<T>::type W; v = (T)(W)((W)v * (W)o.v); }
+        } else if constexpr (OP == RT_R_MAX) {
+            if constexpr (kTrack) { if (o.v > v || (o.v == v && o.pos < pos)) { v = o.v; pos = o.pos; } }
+            else { if (o.v > v) v = o.v; }
+        } else {
+            if constexpr (kTrack) { if (o.v < v || (o.v == v && o.pos < pos)) { v = o.v; pos = o.pos; } }
+            else { if (o.v < v) v = o.v; }
+        }
+    }
+};
+
+// WeightValue::from_usize goes through f32 (core/value.rs:54-56); integers saturate like Rust's `as`.
+template <class T> __device__ __forceinline__ T from_count(uint64_t n) {
+    float f = (float)n;
+    if constexpr (is_flt<T>::value) return (T)f;
+    else {
+        if (f >= (float)highest_of<T>()) return highest_of<T>();
+        return (T)f;
+    }
+}
+
+template <int OP, class T> __device__ __forceinline__ T finalize(T v, uint64_t count) {
+    if constexpr (OP == RT_R_MEAN) {
+        T c = from_count<T>(count);
+        if constexpr (is_flt<T>::value) return v / c;
+        else {
+            if (c == 0) return (T)0;                          // refused on the host before launch
+            if constexpr (std::is_signed<T>::value) { if (c == (T)-1) return (T)(0 - v); }
+            return (T)(v / c);
+        }
+    } else {
+        return v;
+    }
+}
+
+template <class T> __device__ __forceinline__ T shfl_down_t(T v, int d) { return __shfl_down(v, d, RT_WAVE); }
+template <> __device__ __forceinline__ uint8_t shfl_down_t<uint8_t>(uint8_t v, int d) { return (uint8_t)__shfl_down((int)v, d, RT_WAVE); }
+template <> __device__ __forceinline__ int8_t shfl_down_t<int8_t>(int8_t v, int d) { return (int8_t)__shfl_down((int)v, d, RT_WAVE); }
+template <> __device__ __forceinline__ uint16_t shfl_down_t<uint16_t>(uint16_t v, int d) { return (uint16_t)__shfl_down((int)v, d, RT_WAVE); }
+template <> __device__ __forceinline__ int16_t shfl_down_t<int16_t>(int16_t v, int d) { return (int16_t)__shfl_down((int)v, d, RT_WAVE); }
+template <> __device__ __forceinline__ uint64_t shfl_down_t<uint64_t>(uint64_t v, int d) { return (uint64_t)__shfl_down((unsigned long long)v, d, RT_WAVE); }
+template <> __device__ __forceinline__ int64_t shfl_down_t<int64_t>(int64_t v, int d) { return (int64_t)__shfl_down((long long)v, d, RT_WAVE); }
+
+// wave64 tree: after it lane 0 holds the fold of all 64 lanes
+template <int OP, class T> __device__ __forceinline__ void wave_reduce(Acc<OP, T>& a) {
+#pragma unroll
+    for (int d = RT_WAVE / 2; d >= 1; d >>= 1) {
+        Acc<OP, T> o;
+        o.v = shfl_down_t<T>(a.v, d);
+        if constexpr (Acc<OP, T>::kTrack) o.pos = shfl_down_t<uint64_t>(a.pos, d); else o.pos = 0;
+        a.merge(o);
+    }
+}
+
+// block of kBlock lanes: result valid in thread 0
+template <int OP, class T> __device__ __forceinline__ void block_reduce(Acc<OP, T>& a) {
+    __shared__ T sv[kWaves];
+    __shared__ uint64_t sp[kWaves];
+    wave_reduce<OP, T>(a);
+    const int lane = threadIdx.x & (RT_WAVE - 1), w = threadIdx.x / RT_WAVE;
+    if (lane == 0) { sv[w] = a.v; sp[w] = a.pos; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int k = 1; k < kWaves; ++k) { Acc<OP, T> o; o.v = sv[k]; o.pos = sp[k]; a.merge(o); }
+    }
+}
+
+template <class T> struct alignas(16) Vec16 { T e[16 / sizeof(T)]; };
+
+// fold elements [begin, end) of the contiguous run `p`, lanes `tid` of `nthreads` cooperating; positions are
+// reported relative to `p`
+template <int OP, class T>
+__device__ __forceinline__ void fold_run(Acc<OP, T>& a, const T* __restrict__ p, uint64_t begin, uint64_t end, uint32_t tid, uint32_t nthreads) {
+    constexpr uint32_t N = 16 / sizeof(T);
+    constexpr int U = 4;
+    if (begin >= end) return;
+    // elements before the first 16-byte boundary
+    uint64_t head = ((16 - (reinterpret_cast<uintptr_t>(p + begin) & 15)) & 15) / sizeof(T);
+    if (head > end - begin) head = end - begin;
+    if (tid < head) a.push(p[begin + tid], begin + tid);
+    const uint64_t vb = begin + head;
+    const uint64_t nvec = (end - vb) / N;
+    const Vec16<T>* pv = reinterpret_cast<const Vec16<T>*>(p + vb);
+    uint64_t i = tid;
+    for (; i + (uint64_t)(U - 1) * nthreads < nvec; i += (uint64_t)U * nthreads) {
+        Vec16<T> v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = pv[i + (uint64_t)u * nthreads];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+            for (uint32_t j = 0; j < N; ++j) a.push(v[u].e[j], vb + (i + (uint64_t)u * nthreads) * N + j);
+        }
+    }
+    for (; i < nvec; i += nthreads) {
+        Vec16<T> v = pv[i];
+#pragma unroll
+        for (uint32_t j = 0; j < N; ++j) a.push(v.e[j], vb + i * N + j);
+    }
+    const uint64_t tb = vb + nvec * N;
+    if (tb + tid < end) a.push(p[tb + tid], tb + tid);
+}
+
+// ---- rows -------------------------------------------------------------------------------------------------------------
+// grid.x = rows * splits.  Block b folds segment (b % splits) of row (b / splits); out[b] (stage 1 of 2) or out[row].
+template <int OP, class T>
+__global__ __launch_bounds__(kBlock) void reduce_rows_block_kernel(const T* __restrict__ src, T* __restrict__ out, uint64_t R, uint32_t splits,
+                                                                   uint64_t seglen, uint64_t count, int last) {
+    const uint64_t row = blockIdx.x / splits;
+    const uint32_t seg = blockIdx.x - (uint32_t)(row * splits);
+    const uint64_t begin = (uint64_t)seg * seglen;
+    uint64_t end = begin + seglen;
+    if (end > R) end = R;
+    Acc<OP, T> a;
+    a.init();
+    fold_run<OP, T>(a, src + row * R, begin, end, threadIdx.x, kBlock);
+    block_reduce<OP, T>(a);
+    if (threadIdx.x == 0) out[blockIdx.x] = last ? finalize<OP, T>(a.v, count) : a.v;
+}
+
+// one wave per row (64 <= R < a few thousand): grid.x = ceil(rows / kWaves)
+template <int OP, class T>
+__global__ __launch_bounds__(kBlock) void reduce_rows_wave_kernel(const T* __restrict__ src, T* __restrict__ out, uint64_t rows, uint64_t R,
+                                                                  uint64_t count, int last) {
+    const uint64_t row = (uint64_t)blockIdx.x * kWaves + threadIdx.x / RT_WAVE;
+    if (row >= rows) return;
+    Acc<OP, T> a;
+    a.init();
+    fold_run<OP, T>(a, src + row * R, 0, R, threadIdx.x & (RT_WAVE - 1), RT_WAVE);
+    wave_reduce<OP, T>(a);
+    if ((threadIdx.x & (RT_WAVE - 1)) == 0) out[row] = last ? finalize<OP, T>(a.v, count) : a.v;
+}
+
+// one lane per row (R < 64)
+template <int OP, class T>
+__global__ __launch_bounds__(kBlock) void reduce_rows_lane_kernel(const T* __restrict__ src, T* __restrict__ out, uint64_t rows, uint32_t R,
+                                                                  uint64_t count, int last) {
+    const uint64_t row = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (row >= rows) return;
+    Acc<OP, T> a;
+    a.init();
+    const T* p = src + row * R;
+    for (uint32_t k = 0; k < R; ++k) a.push(p[k], k);
+    out[row] = last ? finalize<OP, T>(a.v, count) : a.v;
+}
+
+// ---- cols -------------------------------------------------------------------------------------------------------------
+// src viewed as (outer, R, inner).  VW = elements per lane along `inner` (16 bytes worth when rows are aligned, else 1).
+// blockIdx.x -> (o, seg, tile); lane tx covers columns (tile*64 + tx)*VW .., wave ty takes k = begin+ty, +kWaves, ...
+// out index: ((seg * outer) + o) * inner + column   (seg = 0, splits = 1 when this is the only stage)
+template <int OP, class T, int VW>
+__global__ __launch_bounds__(kBlock) void reduce_cols_kernel(const T* __restrict__ src, T* __restrict__ out, uint64_t R, uint64_t inner, uint64_t outer,
+                                                             uint32_t tiles, uint32_t splits, uint64_t seglen, uint64_t count, int last) {
+    constexpr int U = 4;
+    struct alignas(sizeof(T) * VW) VecW { T e[VW]; };
+    uint64_t b = blockIdx.x;
+    const uint32_t tile = (uint32_t)(b % tiles);
+    b /= tiles;
+    const uint32_t seg = (uint32_t)(b % splits);
+    const uint64_t o = b / splits;
+    const uint32_t tx = threadIdx.x & (RT_WAVE - 1), ty = threadIdx.x / RT_WAVE;
+    const uint64_t col = ((uint64_t)tile * RT_WAVE + tx) * VW;
+    const bool active = col < inner;                           // inner is a multiple of VW
+    const uint64_t begin = (uint64_t)seg * seglen;
+    uint64_t end = begin + seglen;
+    if (end > R) end = R;
+
+    Acc<OP, T> a[VW];
+#pragma unroll
+    for (int j = 0; j < VW; ++j) a[j].init();
+    if (active) {
+        const T* p = src + o * R * inner + col;
+        uint64_t k = begin + ty;
+        for (; k + (uint64_t)(U - 1) * kWaves < end; k += (uint64_t)U * kWaves) {
+            VecW v[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) v[u] = *reinterpret_cast<const VecW*>(p + (k + (uint64_t)u * kWaves) * inner);
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+#pragma unroll
+                for (int j = 0; j < VW; ++j) a[j].push(v[u].e[j], k + (uint64_t)u * kWaves);
+            }
+        }
+        for (; k < end; k += kWaves) {
+            VecW v = *reinterpret_cast<const VecW*>(p + k * inner);
+#pragma unroll
+            for (int j = 0; j < VW; ++j) a[j].push(v.e[j], k);
+        }
+    }
+    // combine the kWaves interleaved partial folds of each column through LDS
+    __shared__ T sv[kWaves][RT_WAVE][VW];
+    __shared__ uint64_t sp[Acc<OP, T>::kTrack ? kWaves : 1][Acc<OP, T>::kTrack ? RT_WAVE : 1][Acc<OP, T>::kTrack ? VW : 1];
+#pragma unroll
+    for (int j = 0; j < VW; ++j) {
+        sv[ty][tx][j] = a[j].v;
+        if constexpr (Acc<OP, T>::kTrack) sp[ty][tx][j] = a[j].pos;
+    }
+    __syncthreads();
+    if (ty == 0 && active) {
+        T* q = out + ((uint64_t)seg * outer + o) * inner + col;
+#pragma unroll
+        for (int j = 0; j < VW; ++j) {
+#pragma unroll
+            for (int w = 1; w < kWaves; ++w) {
+                Acc<OP, T> x;
+                x.v = sv[w][tx][j];
+                if constexpr (Acc<OP, T>::kTrack) x.pos = sp[w][tx][j]; else x.pos = 0;
+                a[j].merge(x);
+            }
+            q[j] = last ? finalize<OP, T>(a[j].v, count) : a[j].v;
+        }
+    }
+}
+
+// ---- host planning ------------------------------------------------------------------------------------------------------
+template <int OP, class T>
+int32_t rows_stage(rt_ctx* ctx, const T* src, T* out, uint64_t rows, uint64_t R, uint64_t count, bool allow_split) {
+    hipStream_t s = ctx->stream;
+    if (rows == 0) return RT_OK;
+    if (R < 64) {
+        uint64_t blocks = (rows + kBlock - 1) / kBlock;
+        if (blocks >= (1ull << 31)) return rt_fail(RT_E_INVALID, "reduce: too many rows for one launch");
+        hipLaunchKernelGGL((reduce_rows_lane_kernel<OP, T>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, out, rows, (uint32_t)R, count, 1);
+        RT_HIP(hipGetLastError());
+        return RT_OK;
+    }
+    const uint64_t want = (uint64_t)ctx->num_cus * 8;
+    if (R < 4096 && rows >= want / 2) {
+        uint64_t blocks = (rows + kWaves - 1) / kWaves;
+        if (blocks >= (1ull << 31)) return rt_fail(RT_E_INVALID, "reduce: too many rows for one launch");
+        hipLaunchKernelGGL((reduce_rows_wave_kernel<OP, T>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, out, rows, R, count, 1);
+        RT_HIP(hipGetLastError());
+        return RT_OK;
+    }
+    // block per (row, segment); split long rows when there are too few of them
+    uint32_t splits = 1;
+    if (allow_split && rows < want) {
+        const uint64_t min_seg = 16384;                       // elements; below this a split is not worth a second pass
+        uint64_t by_size = R / min_seg;
+        uint64_t by_need = (want + rows - 1) / rows;
+        uint64_t sp = by_need < by_size ? by_need : by_size;
+        if (sp > 4096) sp = 4096;
+        if (sp > 1) splits = (uint32_t)sp;
+    }
+    if (rows * splits >= (1ull << 31)) return rt_fail(RT_E_INVALID, "reduce: too many rows for one launch");
+    if (splits == 1) {
+        hipLaunchKernelGGL((reduce_rows_block_kernel<OP, T>), dim3((unsigned)rows), dim3(kBlock), 0, s, src, out, R, 1u, R, count, 1);
+        RT_HIP(hipGetLastError());
+        return RT_OK;
+    }
+    constexpr uint64_t N = 16 / sizeof(T);
+    uint64_t seglen = (R + splits - 1) / splits;
+    seglen = (seglen + N * kBlock - 1) / (N * kBlock) * (N * kBlock);       // whole 16-byte vectors per lane
+    splits = (uint32_t)((R + seglen - 1) / seglen);
+    void* scratch = nullptr;
+    RT_TRY(rt_scratch(ctx, (size_t)(rows * splits) * sizeof(T), &scratch));
+    T* part = (T*)scratch;
+    hipLaunchKernelGGL((reduce_rows_block_kernel<OP, T>), dim3((unsigned)(rows * splits)), dim3(kBlock), 0, s, src, part, R, splits, seglen, count, 0);
+    RT_HIP(hipGetLastError());
+    // second stage: each row of `splits` partials -> one output (mean divides by the original count)
+    if (splits < 64) {
+        uint64_t blocks = (rows + kBlock - 1) / kBlock;
+        hipLaunchKernelGGL((reduce_rows_lane_kernel<OP, T>), dim3((unsigned)blocks), dim3(kBlock), 0, s, part, out, rows, splits, count, 1);
+    } else {
+        hipLaunchKernelGGL((reduce_rows_block_kernel<OP, T>), dim3((unsigned)rows), dim3(kBlock), 0, s, part, out, (uint64_t)splits, 1u, (uint64_t)splits, count, 1);
+    }
+    RT_HIP(hipGetLastError());
+    return RT_OK;
+}
+
+template <int OP, class T, int VW>
+int32_t cols_launch(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t R, uint64_t inner, uint64_t count, bool allow_split) {
+    hipStream_t s = ctx->stream;
+    const uint64_t per_tile = (uint64_t)RT_WAVE * VW;
+    const uint64_t tiles = (inner + per_tile - 1) / per_tile;
+    const uint64_t want = (uint64_t)ctx->num_cus * 8;
+    uint32_t splits = 1;
+    if (allow_split && outer * tiles < want) {
+        const uint64_t min_seg = 64;                          // k values per block
+        uint64_t by_size = R / min_seg;
+        uint64_t by_need = (want + outer * tiles - 1) / (outer * tiles);
+        uint64_t sp = by_need < by_size ? by_need : by_size;
+        if (sp > 1024) sp = 1024;
+        if (sp > 1) splits = (uint32_t)sp;
+    }
+    uint64_t seglen = (R + splits - 1) / splits;
+    if (splits > 1) {
+        seglen = (seglen + 4 * kWaves - 1) / (4 * kWaves) * (4 * kWaves);
+        splits = (uint32_t)((R + seglen - 1) / seglen);
+    }
+    const uint64_t blocks = outer * splits * tiles;
+    if (blocks >= (1ull << 31) || tiles >= (1ull << 31)) return rt_fail(RT_E_INVALID, "reduce: too many outputs for one launch");
+    if (splits == 1) {
+        hipLaunchKernelGGL((reduce_cols_kernel<OP, T, VW>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, out, R, inner, outer,
+                           (uint32_t)tiles, 1u, seglen, count, 1);
+        RT_HIP(hipGetLastError());
+        return RT_OK;
+    }
+    void* scratch = nullptr;
+    RT_TRY(rt_scratch(ctx, (size_t)(splits * outer * inner) * sizeof(T), &scratch));
+    T* part = (T*)scratch;
+    hipLaunchKernelGGL((reduce_cols_kernel<OP, T, VW>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, part, R, inner, outer,
+                       (uint32_t)tiles, splits, seglen, count, 0);
+    RT_HIP(hipGetLastError());
+    // second stage: partials are (splits, outer*inner): a column reduce with R = splits
+    const uint64_t inner2 = outer * inner;
+    const uint64_t tiles2 = (inner2 + per_tile - 1) / per_tile;
+    if (tiles2 >= (1ull << 31)) return rt_fail(RT_E_INVALID, "reduce: too many outputs for one launch");
+    hipLaunchKernelGGL((reduce_cols_kernel<OP, T, VW>), dim3((unsigned)tiles2), dim3(kBlock), 0, s, part, out, (uint64_t)splits, inner2, (uint64_t)1,
+                       (uint32_t)tiles2, 1u, (uint64_t)splits, count, 1);
+    RT_HIP(hipGetLastError());
+    return RT_OK;
+}
+
+template <int OP, class T>
+int32_t reduce_typed(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t R, uint64_t inner) {
+    if (outer == 0 || inner == 0) return RT_OK;
+    if (OP == RT_R_MEAN && !is_flt<T>::value && R == 0) return rt_fail(RT_E_ARITH, "reduce: integer mean over an empty axis divides by zero");
+    if (inner == 1) return rows_stage<OP, T>(ctx, src, out, outer, R, R, true);
+    constexpr int N = 16 / sizeof(T);
+    const bool vec = (inner % N == 0) && ((reinterpret_cast<uintptr_t>(src) & 15) == 0) && ((reinterpret_cast<uintptr_t>(out) & 15) == 0);
+    if (vec) return cols_launch<OP, T, N>(ctx, src, out, outer, R, inner, R, true);
+    return cols_launch<OP, T, 1>(ctx, src, out, outer, R, inner, R, true);
+}
+
+template <class T>
+int32_t reduce_ops(rt_ctx* ctx, int op, const void* src, void* out, uint64_t outer, uint64_t R, uint64_t inner) {
+    switch (op) {
+        case RT_R_SUM: return reduce_typed<RT_R_SUM, T>(ctx, (const T*)src, (T*)out, outer, R, inner);
+        case RT_R_PROD: return reduce_typed<RT_R_PROD, T>(ctx, (const T*)src, (T*)out, outer, R, inner);
+        case RT_R_MAX: return reduce_typed<RT_R_MAX, T>(ctx, (const T*)src, (T*)out, outer, R, inner);
+        case RT_R_MIN: return reduce_typed<RT_R_MIN, T>(ctx, (const T*)src, (T*)out, outer, R, inner);
+        case RT_R_MEAN: return reduce_typed<RT_R_MEAN, T>(ctx, (const T*)src, (T*)out, outer, R, inner);
+    }
+    return rt_fail(RT_E_INVALID, "reduce: op code %d has no accumulator (the reference panics, ops/reduction/mod.rs:185)", op);
+}
+
+int32_t reduce_any(rt_ctx* ctx, int dtype, int op, const void* src, void* out, uint64_t outer, uint64_t R, uint64_t inner) {
+    switch (dtype) {
+        case RT_U8: return reduce_ops<uint8_t>(ctx, op, src, out, outer, R, inner);
+        case RT_I8: return reduce_ops<int8_t>(ctx, op, src, out, outer, R, inner);
+        case RT_U16: return reduce_ops<uint16_t>(ctx, op, src, out, outer, R, inner);
+        case RT_I16: return reduce_ops<int16_t>(ctx, op, src, out, outer, R, inner);
+        case RT_U32: return reduce_ops<uint32_t>(ctx, op, src, out, outer, R, inner);
+        case RT_I32: return reduce_ops<int32_t>(ctx, op, src, out, outer, R, inner);
+        case RT_U64: return reduce_ops<uint64_t>(ctx, op, src, out, outer, R, inner);
+        case RT_I64: return reduce_ops<int64_t>(ctx, op, src, out, outer, R, inner);
+        case RT_F32: return reduce_ops<float>(ctx, op, src, out, outer, R, inner);
+        case RT_F64: return reduce_ops<double>(ctx, op, src, out, outer, R, inner);
+    }
+    return rt_fail(RT_E_DTYPE, "reduce: dtype code %d is not reducible (f32/f64 in the reference, 8..64-bit integers added here)", dtype);
+}
+
+}  // namespace
+
+extern "C" int32_t rt_reduce_flat(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, uint64_t src_len, void* dst, uint64_t dst_len,
+                                  uint64_t start, uint64_t len) {
+    RT_TRY(rt_ctx_enter(ctx));
+    int es = rt_elem_size(dtype);
+    if (!es) return rt_fail(RT_E_DTYPE, "reduce: unknown dtype code %d", dtype);
+    // check_reduce_flat, backend/remote/server.rs:375-380
+    if (start > src_len || len > src_len - start)
+        return rt_fail(RT_E_OUT_OF_BOUNDS, "reduction source: elements %llu..%llu of a buffer with %llu elements",
+                       (unsigned long long)start, (unsigned long long)(start + len), (unsigned long long)src_len);
+    if (dst_len == 0) return rt_fail(RT_E_OUT_OF_BOUNDS, "reduction output buffer is empty");
+    if (!dst || (!src && len)) return rt_fail(RT_E_INVALID, "reduce: null buffer");
+    CtxGuard g(ctx);
+    return reduce_any(ctx, dtype, op, (const char*)src + start * es, dst, 1, len, 1);
+}
+
+extern "C" int32_t rt_reduce_nd(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, uint64_t src_len, uint64_t offset, int32_t rank,
+                                const uint64_t* shape, const int64_t* strides, void* dst, uint64_t dst_len, int32_t dim) {
+    RT_TRY(rt_ctx_enter(ctx));
+    int es = rt_elem_size(dtype);
+    if (!es) return rt_fail(RT_E_DTYPE, "reduce: unknown dtype code %d", dtype);
+    // check_reduce_nd, backend/remote/server.rs:327-373
+    if (rank < 1 || rank > RT_MAX_INPUT_RANK || !shape || !strides) return rt_fail(RT_E_INVALID, "reduce: bad rank %d or null shape", rank);
+    if (dim < 0 || dim >= rank) return rt_fail(RT_E_INVALID, "reduction dim %d out of range for rank %d", dim, rank);
+    unsigned __int128 size = 1, outer = 1, inner = 1;
+    for (int i = 0; i < rank; ++i) {
+        size *= shape[i];
+        if (i < dim) outer *= shape[i];
+        if (i > dim) inner *= shape[i];
+        if (size > (unsigned __int128)INT64_MAX || outer > (unsigned __int128)INT64_MAX || inner > (unsigned __int128)INT64_MAX) {
+            bool has_zero = false;
+            for (int j = 0; j < rank; ++j) has_zero = has_zero || shape[j] == 0;
+            if (!has_zero) return rt_fail(RT_E_INVALID, "reduction source shape has too many elements");
+            size = outer = inner = 0;
+            break;
+        }
+    }
+    if (outer * inner == 0) return RT_OK;                      // no outputs: the kernel must not run
+    int64_t expected = 1;
+    for (int d = rank - 1; d >= 0; --d) {
+        if (shape[d] > 1 && strides[d] != expected)
+            return rt_fail(RT_E_WRONG_DIMS, "Reduction over non-contiguous tensors is not implemented yet.");
+        expected *= (int64_t)shape[d];
+    }
+    if (offset > src_len || (uint64_t)size > src_len - offset)
+        return rt_fail(RT_E_OUT_OF_BOUNDS, "reduction source of %llu elements at offset %llu exceeds buffer of %llu",
+                       (unsigned long long)size, (unsigned long long)offset, (unsigned long long)src_len);
+    if ((unsigned __int128)dst_len < outer * inner)
+        return rt_fail(RT_E_OUT_OF_BOUNDS, "reduction output needs %llu elements, buffer has %llu", (unsigned long long)(outer * inner),
+                       (unsigned long long)dst_len);
+    if (!dst || !src) return rt_fail(RT_E_INVALID, "reduce: null buffer");
+    CtxGuard g(ctx);
+    return reduce_any(ctx, dtype, op, (const char*)src + offset * es, dst, (uint64_t)outer, shape[dim], (uint64_t)inner);
+}

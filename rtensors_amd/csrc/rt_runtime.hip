@@ -1,0 +1,377 @@
+// Context, stream, caching device allocator, host<->device transfers, events.
+// Stands where backend/cuda.rs:38-185 and 668-836 (cudarc context, CudaSlice alloc/copy, sync-on-read) stand in
+// the reference; written directly against the HIP runtime.
+#include "rt_common.h"
+
+#include <string>
+
+// ---- error plumbing ---------------------------------------------------------------------------------------------
+static thread_local char g_err[512] = "";
+
+int32_t rt_fail(int32_t status, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return status;
+}
+
+int32_t rt_hip_fail(hipError_t e, const char* what) {
+    if (e == hipErrorOutOfMemory) return rt_fail(RT_E_OOM, "%s: %s", what, hipGetErrorString(e));
+    return rt_fail(RT_E_HIP, "%s: %s (%d)", what, hipGetErrorString(e), (int)e);
+}
+
+extern "C" const char* rt_last_error(void) { return g_err; }
+
+extern "C" const char* rt_status_name(int32_t s) {
+    switch (s) {
+        case RT_OK: return "RT_OK";
+        case RT_E_INVALID: return "RT_E_INVALID";
+        case RT_E_DTYPE: return "RT_E_DTYPE";
+        case RT_E_OUT_OF_BOUNDS: return "RT_E_OUT_OF_BOUNDS";
+        case RT_E_HIP: return "RT_E_HIP";
+        case RT_E_OOM: return "RT_E_OOM";
+        case RT_E_RANK: return "RT_E_RANK";
+        case RT_E_ARITH: return "RT_E_ARITH";
+        case RT_E_WRONG_DIMS: return "RT_E_WRONG_DIMS";
+        case RT_E_SIZE_MISMATCH: return "RT_E_SIZE_MISMATCH";
+    }
+    return "RT_E_UNKNOWN";
+}
+
+extern "C" int32_t rt_dtype_size(int32_t dtype) { return rt_elem_size(dtype); }
+
+extern "C" int32_t rt_device_count(int32_t* out) {
+    if (!out) return rt_fail(RT_E_INVALID, "rt_device_count: null out");
+    int n = 0;
+    RT_HIP(hipGetDeviceCount(&n));
+    *out = n;
+    return RT_OK;
+}
+
+// ---- context ------------------------------------------------------------------------------------------------------
+int32_t rt_ctx_enter(rt_ctx* ctx) {
+    if (!ctx) return rt_fail(RT_E_INVALID, "null context");
+    RT_HIP(hipSetDevice(ctx->device));
+    return RT_OK;
+}
+
+extern "C" int32_t rt_ctx_create(int32_t device, rt_ctx** out) {
+    if (!out) return rt_fail(RT_E_INVALID, "rt_ctx_create: null out");
+    *out = nullptr;
+    int n = 0;
+    RT_HIP(hipGetDeviceCount(&n));
+    if (device < 0 || device >= n) return rt_fail(RT_E_INVALID, "rt_ctx_create: device %d of %d", device, n);
+    RT_HIP(hipSetDevice(device));
+    rt_ctx* c = new rt_ctx();
+    c->device = device;
+    hipError_t e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking);   // default priority
+    if (e != hipSuccess) { delete c; return rt_hip_fail(e, "hipStreamCreateWithFlags"); }
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device) == hipSuccess && prop.multiProcessorCount > 0) c->num_cus = prop.multiProcessorCount;
+    e = hipMalloc((void**)&c->flag_dev, 256);
+    if (e != hipSuccess) { (void)hipStreamDestroy(c->stream); delete c; return rt_hip_fail(e, "hipMalloc(flag)"); }
+    *out = c;
+    return RT_OK;
+}
+
+extern "C" int32_t rt_ctx_destroy(rt_ctx* ctx) {
+    RT_TRY(rt_ctx_enter(ctx));
+    {
+        CtxGuard g(ctx);
+        (void)hipStreamSynchronize(ctx->stream);
+        for (auto& kv : ctx->free_blocks) (void)hipFree(kv.second);
+        for (auto& kv : ctx->live) (void)hipFree(kv.first);
+        if (ctx->scratch) (void)hipFree(ctx->scratch);
+        if (ctx->flag_dev) (void)hipFree(ctx->flag_dev);
+        (void)hipStreamDestroy(ctx->stream);
+    }
+    delete ctx;
+    return RT_OK;
+}
+
+extern "C" int32_t rt_sync(rt_ctx* ctx) {
+    RT_TRY(rt_ctx_enter(ctx));
+    RT_HIP(hipStreamSynchronize(ctx->stream));
+    return RT_OK;
+}
+
+// ---- caching allocator ---------------------------------------------------------------------------------------------
+// Size classes: multiples of 512 B below 1 MiB, multiples of 2 MiB above.  A freed block keeps its capacity and is
+// reused for the next request of the same class; nothing is split, so there is no fragmentation to manage, and a
+// training step that allocates the same shapes every iteration reaches a state with no hipMalloc at all.
+static size_t size_class(size_t bytes) {
+    if (bytes == 0) bytes = 1;
+    if (bytes < (1u << 20)) return (bytes + 511) & ~(size_t)511;
+    const size_t g = (size_t)2 << 20;
+    return (bytes + g - 1) / g * g;
+}
+
+int32_t rt_alloc_bytes(rt_ctx* ctx, size_t bytes, void** out) {
+    size_t cap = size_class(bytes);
+    auto it = ctx->free_blocks.find(cap);
+    if (it != ctx->free_blocks.end()) {
+        *out = it->second;
+        ctx->free_blocks.erase(it);
+        ctx->bytes_cached -= cap;
+    } else {
+        void* p = nullptr;
+        hipError_t e = hipMalloc(&p, cap);
+        if (e == hipErrorOutOfMemory && !ctx->free_blocks.empty()) {
+            // give cached blocks back to the driver and retry once
+            (void)hipGetLastError();
+            (void)hipStreamSynchronize(ctx->stream);
+            for (auto& kv : ctx->free_blocks) (void)hipFree(kv.second);
+            ctx->free_blocks.clear();
+            ctx->bytes_cached = 0;
+            e = hipMalloc(&p, cap);
+        }
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            *out = nullptr;
+            return rt_hip_fail(e, "hipMalloc");
+        }
+        ctx->device_allocs += 1;
+        *out = p;
+    }
+    ctx->live[*out] = cap;
+    ctx->bytes_in_use += cap;
+    return RT_OK;
+}
+
+int32_t rt_free_locked(rt_ctx* ctx, void* p) {
+    auto it = ctx->live.find(p);
+    if (it == ctx->live.end()) return rt_fail(RT_E_INVALID, "rt_free: %p was not allocated by this context", p);
+    size_t cap = it->second;
+    ctx->live.erase(it);
+    ctx->bytes_in_use -= cap;
+    ctx->free_blocks.emplace(cap, p);
+    ctx->bytes_cached += cap;
+    return RT_OK;
+}
+
+int32_t rt_scratch(rt_ctx* ctx, size_t bytes, void** out) {
+    if (bytes > ctx->scratch_bytes) {
+        if (ctx->scratch) {
+            RT_HIP(hipStreamSynchronize(ctx->stream));
+            RT_HIP(hipFree(ctx->scratch));
+            ctx->scratch = nullptr;
+            ctx->scratch_bytes = 0;
+        }
+        size_t cap = size_class(bytes < (1u << 20) ? (1u << 20) : bytes);
+        RT_HIP(hipMalloc(&ctx->scratch, cap));
+        ctx->scratch_bytes = cap;
+    }
+    *out = ctx->scratch;
+    return RT_OK;
+}
+
+__global__ void rt_zero_kernel(uint4* p, size_t nvec) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    for (; i < nvec; i += step) p[i] = make_uint4(0, 0, 0, 0);
+}
+
+static int32_t checked_bytes(int32_t dtype, uint64_t len, size_t* bytes) {
+    int es = rt_elem_size(dtype);
+    if (es == 0) return rt_fail(RT_E_DTYPE, "unknown dtype code %d", dtype);
+    if (len > (UINT64_MAX >> 5)) return rt_fail(RT_E_INVALID, "length %llu is too large", (unsigned long long)len);
+    *bytes = (size_t)len * (size_t)es;
+    return RT_OK;
+}
+
+static int32_t alloc_impl(rt_ctx* ctx, int32_t dtype, uint64_t len, void** out, bool zero) {
+    if (!out) return rt_fail(RT_E_INVALID, "rt_alloc: null out");
+    *out = nullptr;
+    RT_TRY(rt_ctx_enter(ctx));
+    size_t bytes = 0;
+    RT_TRY(checked_bytes(dtype, len, &bytes));
+    CtxGuard g(ctx);
+    RT_TRY(rt_alloc_bytes(ctx, bytes, out));
+    if (zero && bytes) {
+        // whole size class is zeroed (capacity is a multiple of 512 B), by a fill kernel rather than a memset node
+        size_t nvec = size_class(bytes) / 16;
+        size_t blocks = (nvec + 255) / 256;
+        if (blocks > (size_t)ctx->num_cus * 16) blocks = (size_t)ctx->num_cus * 16;
+        hipLaunchKernelGGL(rt_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (uint4*)*out, nvec);
+        RT_HIP(hipGetLastError());
+    }
+    return RT_OK;
+}
+
+extern "C" int32_t rt_alloc(rt_ctx* ctx, int32_t dtype, uint64_t len, void** out) { return alloc_impl(ctx, dtype, len, out, true); }
+extern "C" int32_t rt_alloc_uninit(rt_ctx* ctx, int32_t dtype, uint64_t len, void** out) { return alloc_impl(ctx, dtype, len, out, false); }
+
+extern "C" int32_t rt_free(rt_ctx* ctx, void* buf) {
+    if (!buf) return RT_OK;
+    RT_TRY(rt_ctx_enter(ctx));
+    CtxGuard g(ctx);
+    return rt_free_locked(ctx, buf);
+}
+
+extern "C" int32_t rt_alloc_from_slice(rt_ctx* ctx, int32_t dtype, const void* host_src, uint64_t len, void** out) {
+    if (!out) return rt_fail(RT_E_INVALID, "rt_alloc_from_slice: null out");
+    *out = nullptr;
+    if (!host_src && len) return rt_fail(RT_E_INVALID, "rt_alloc_from_slice: null source");
+    RT_TRY(rt_ctx_enter(ctx));
+    size_t bytes = 0;
+    RT_TRY(checked_bytes(dtype, len, &bytes));
+    CtxGuard g(ctx);
+    RT_TRY(rt_alloc_bytes(ctx, bytes, out));
+    if (bytes) {
+        hipError_t e = hipMemcpyAsync(*out, host_src, bytes, hipMemcpyHostToDevice, ctx->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);   // the host slice may be dropped on return
+        if (e != hipSuccess) { (void)rt_free_locked(ctx, *out); *out = nullptr; return rt_hip_fail(e, "upload"); }
+    }
+    return RT_OK;
+}
+
+extern "C" int32_t rt_copy_from_slice(rt_ctx* ctx, int32_t dtype, void* dst, uint64_t dst_len, const void* host_src, uint64_t src_len) {
+    RT_TRY(rt_ctx_enter(ctx));
+    if (dst_len != src_len)
+        return rt_fail(RT_E_SIZE_MISMATCH, "copy_from_slice: dst size %llu, src size %llu", (unsigned long long)dst_len, (unsigned long long)src_len);
+    size_t bytes = 0;
+    RT_TRY(checked_bytes(dtype, src_len, &bytes));
+    if (!bytes) return RT_OK;
+    if (!dst || !host_src) return rt_fail(RT_E_INVALID, "copy_from_slice: null pointer");
+    CtxGuard g(ctx);
+    RT_HIP(hipMemcpyAsync(dst, host_src, bytes, hipMemcpyHostToDevice, ctx->stream));
+    RT_HIP(hipStreamSynchronize(ctx->stream));
+    return RT_OK;
+}
+
+extern "C" int32_t rt_copy_range_within(rt_ctx* ctx, int32_t dtype, void* dst, uint64_t dst_len, const void* src, uint64_t src_len,
+                                        uint64_t dst_offset, uint64_t src_offset, uint64_t len) {
+    RT_TRY(rt_ctx_enter(ctx));
+    int es = rt_elem_size(dtype);
+    if (!es) return rt_fail(RT_E_DTYPE, "unknown dtype code %d", dtype);
+    if (dst_offset > dst_len || len > dst_len - dst_offset || src_offset > src_len || len > src_len - src_offset)
+        return rt_fail(RT_E_OUT_OF_BOUNDS, "copy_range_within: dst size %llu, src size %llu, dst_offset %llu, src_offset %llu, len %llu",
+                       (unsigned long long)dst_len, (unsigned long long)src_len, (unsigned long long)dst_offset,
+                       (unsigned long long)src_offset, (unsigned long long)len);
+    if (!len) return RT_OK;
+    if (!dst || !src) return rt_fail(RT_E_INVALID, "copy_range_within: null pointer");
+    CtxGuard g(ctx);
+    RT_HIP(hipMemcpyAsync((char*)dst + dst_offset * es, (const char*)src + src_offset * es, (size_t)len * es,
+                          hipMemcpyDeviceToDevice, ctx->stream));
+    return RT_OK;
+}
+
+extern "C" int32_t rt_read(rt_ctx* ctx, int32_t dtype, const void* buf, uint64_t buf_len, uint64_t offset, void* out_value) {
+    RT_TRY(rt_ctx_enter(ctx));
+    int es = rt_elem_size(dtype);
+    if (!es) return rt_fail(RT_E_DTYPE, "unknown dtype code %d", dtype);
+    if (offset >= buf_len)
+        return rt_fail(RT_E_OUT_OF_BOUNDS, "Index %llu out of bounds for buffer of length %llu", (unsigned long long)offset, (unsigned long long)buf_len);
+    if (!buf || !out_value) return rt_fail(RT_E_INVALID, "rt_read: null pointer");
+    CtxGuard g(ctx);
+    RT_HIP(hipMemcpyAsync(out_value, (const char*)buf + offset * es, es, hipMemcpyDeviceToHost, ctx->stream));
+    RT_HIP(hipStreamSynchronize(ctx->stream));
+    return RT_OK;
+}
+
+struct Cell16 { uint32_t w[4]; };
+
+__global__ void rt_write_one_kernel(unsigned char* dst, Cell16 v, int bytes) {
+    const unsigned char* s = (const unsigned char*)&v;
+    for (int i = 0; i < bytes; ++i) dst[i] = s[i];
+}
+
+extern "C" int32_t rt_write(rt_ctx* ctx, int32_t dtype, void* buf, uint64_t buf_len, uint64_t offset, const void* value) {
+    RT_TRY(rt_ctx_enter(ctx));
+    int es = rt_elem_size(dtype);
+    if (!es) return rt_fail(RT_E_DTYPE, "unknown dtype code %d", dtype);
+    if (offset >= buf_len)
+        return rt_fail(RT_E_OUT_OF_BOUNDS, "Index %llu out of bounds for buffer of length %llu", (unsigned long long)offset, (unsigned long long)buf_len);
+    if (!buf || !value) return rt_fail(RT_E_INVALID, "rt_write: null pointer");
+    Cell16 v = {{0, 0, 0, 0}};
+    memcpy(&v, value, es);
+    CtxGuard g(ctx);
+    // the value travels as a kernel argument, so no host memory has to outlive this call
+    hipLaunchKernelGGL(rt_write_one_kernel, dim3(1), dim3(1), 0, ctx->stream, (unsigned char*)buf + offset * es, v, es);
+    RT_HIP(hipGetLastError());
+    return RT_OK;
+}
+
+extern "C" int32_t rt_copy(rt_ctx* ctx, int32_t dtype, const void* src, uint64_t len, void** out) {
+    if (!out) return rt_fail(RT_E_INVALID, "rt_copy: null out");
+    *out = nullptr;
+    RT_TRY(rt_ctx_enter(ctx));
+    size_t bytes = 0;
+    RT_TRY(checked_bytes(dtype, len, &bytes));
+    if (!src && bytes) return rt_fail(RT_E_INVALID, "rt_copy: null source");
+    CtxGuard g(ctx);
+    RT_TRY(rt_alloc_bytes(ctx, bytes, out));
+    if (bytes) {
+        hipError_t e = hipMemcpyAsync(*out, src, bytes, hipMemcpyDeviceToDevice, ctx->stream);
+        if (e != hipSuccess) { (void)rt_free_locked(ctx, *out); *out = nullptr; return rt_hip_fail(e, "device copy"); }
+    }
+    return RT_OK;
+}
+
+extern "C" int32_t rt_dump(rt_ctx* ctx, int32_t dtype, const void* src, uint64_t len, void* host_dst) {
+    RT_TRY(rt_ctx_enter(ctx));
+    size_t bytes = 0;
+    RT_TRY(checked_bytes(dtype, len, &bytes));
+    if (!bytes) return RT_OK;
+    if (!src || !host_dst) return rt_fail(RT_E_INVALID, "rt_dump: null pointer");
+    CtxGuard g(ctx);
+    RT_HIP(hipMemcpyAsync(host_dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    RT_HIP(hipStreamSynchronize(ctx->stream));
+    return RT_OK;
+}
+
+// ---- events / stats -----------------------------------------------------------------------------------------------
+struct rt_event { hipEvent_t ev; };
+
+extern "C" int32_t rt_event_create(rt_ctx* ctx, rt_event** out) {
+    if (!out) return rt_fail(RT_E_INVALID, "rt_event_create: null out");
+    RT_TRY(rt_ctx_enter(ctx));
+    rt_event* e = new rt_event();
+    hipError_t r = hipEventCreate(&e->ev);
+    if (r != hipSuccess) { delete e; return rt_hip_fail(r, "hipEventCreate"); }
+    *out = e;
+    return RT_OK;
+}
+
+extern "C" int32_t rt_event_record(rt_ctx* ctx, rt_event* ev) {
+    RT_TRY(rt_ctx_enter(ctx));
+    if (!ev) return rt_fail(RT_E_INVALID, "rt_event_record: null event");
+    RT_HIP(hipEventRecord(ev->ev, ctx->stream));
+    return RT_OK;
+}
+
+extern "C" int32_t rt_event_elapsed_ms(rt_ctx* ctx, rt_event* start, rt_event* stop, float* out_ms) {
+    RT_TRY(rt_ctx_enter(ctx));
+    if (!start || !stop || !out_ms) return rt_fail(RT_E_INVALID, "rt_event_elapsed_ms: null argument");
+    RT_HIP(hipEventSynchronize(stop->ev));
+    RT_HIP(hipEventElapsedTime(out_ms, start->ev, stop->ev));
+    return RT_OK;
+}
+
+extern "C" int32_t rt_event_destroy(rt_ctx* ctx, rt_event* ev) {
+    RT_TRY(rt_ctx_enter(ctx));
+    if (!ev) return RT_OK;
+    (void)hipEventDestroy(ev->ev);
+    delete ev;
+    return RT_OK;
+}
+
+extern "C" int32_t rt_mem_stats(rt_ctx* ctx, uint64_t* in_use, uint64_t* cached, uint64_t* device_allocs) {
+    if (!ctx) return rt_fail(RT_E_INVALID, "null context");
+    CtxGuard g(ctx);
+    if (in_use) *in_use = ctx->bytes_in_use;
+    if (cached) *cached = ctx->bytes_cached;
+    if (device_allocs) *device_allocs = ctx->device_allocs;
+    return RT_OK;
+}
+
+extern "C" int32_t rt_mem_trim(rt_ctx* ctx) {
+    RT_TRY(rt_ctx_enter(ctx));
+    CtxGuard g(ctx);
+    RT_HIP(hipStreamSynchronize(ctx->stream));
+    for (auto& kv : ctx->free_blocks) (void)hipFree(kv.second);
+    ctx->free_blocks.clear();
+    ctx->bytes_cached = 0;
+    return RT_OK;
+}

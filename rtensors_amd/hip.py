@@ -1,0 +1,243 @@
+"""`Hip`: host-side mirror of the reference's `Backend` trait (libs/rtensors/src/backend/mod.rs:216-472) over the
+C ABI.  Method names, argument meaning and error behaviour follow the trait; buffers are `HipBuf` (device pointer +
+length + dtype, the counterpart of `CudaBuf`, backend/cuda.rs:53-57).  Host data crosses as 1-D numpy arrays."""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Sequence, Tuple
+
+import numpy as np
+
+from . import _ffi
+from ._ffi import lib
+
+# dtype codes: core/value.rs:567-581
+U8, I8, U16, I16, U32, U128, I32, U64, I64, I128, F32, F64, BOOL = range(13)
+V16 = np.dtype("V16")
+NP_DTYPE = {
+    U8: np.dtype(np.uint8), I8: np.dtype(np.int8), U16: np.dtype(np.uint16), I16: np.dtype(np.int16),
+    U32: np.dtype(np.uint32), I32: np.dtype(np.int32), U64: np.dtype(np.uint64), I64: np.dtype(np.int64),
+    F32: np.dtype(np.float32), F64: np.dtype(np.float64), BOOL: np.dtype(np.bool_), U128: V16, I128: V16,
+}
+DTYPE_BY_NAME = {"u8": U8, "i8": I8, "u16": U16, "i16": I16, "u32": U32, "u128": U128, "i32": I32, "u64": U64, "i64": I64,
+                 "i128": I128, "f32": F32, "f64": F64, "bool": BOOL}
+
+UNARY = {n: i for i, n in enumerate(
+    "neg relu sigmoid silu tanh abs sqrt ln expm1 ln1p floor ceil round trunc sin cos tan asin acos atan sinh cosh "
+    "asinh acosh atanh rsqrt reciprocal square cube exp sign".split())}
+SCALAR = {n: i for i, n in enumerate("add sub mul div log log1p leaky_relu elu".split())}
+BINARY = {"add": 0, "sub": 1, "mul": 2, "div": 3}
+REDUCE = {"sum": 1, "prod": 2, "max": 3, "min": 4, "mean": 5}
+
+# rt_status -> TensorError variant (core/tensor.rs:11-53; HipError stands where CudaError stands)
+_KIND = {1: "InvalidArgument", 2: "UnsupportedOperation", 3: "IdxOutOfBounds", 4: "HipError", 5: "HipError",
+         6: "UnsupportedOperation", 7: "ArithmeticError", 8: "WrongDims", 9: "SizeMismatch"}
+
+
+class TensorError(Exception):
+    def __init__(self, status: int, msg: str):
+        self.status = status
+        self.kind = _KIND.get(status, "HipError")
+        super().__init__(f"{self.kind}: {msg}")
+
+
+def _check(status: int):
+    if status != 0:
+        raise TensorError(status, lib.rt_last_error().decode(errors="replace"))
+
+
+def _u64s(xs: Sequence[int]):
+    return (C.c_uint64 * max(len(xs), 1))(*xs)
+
+
+def _i64s(xs: Sequence[int]):
+    return (C.c_int64 * max(len(xs), 1))(*xs)
+
+
+def _value(dtype: int, value) -> np.ndarray:
+    if dtype in (U128, I128):
+        return np.frombuffer((int(value) & ((1 << 128) - 1)).to_bytes(16, "little"), dtype=V16).copy()
+    return np.array([value], dtype=NP_DTYPE[dtype])
+
+
+class HipBuf:
+    """Owns `len` elements of `dtype` in device memory; returned to the context's allocator when dropped."""
+
+    def __init__(self, backend: "Hip", ptr: int, length: int, dtype: int):
+        self.backend, self.ptr, self.len, self.dtype = backend, ptr, length, dtype
+
+    def __del__(self):
+        try:
+            if self.ptr and self.backend is not None and self.backend._ctx:
+                lib.rt_free(self.backend._ctx, self.ptr)
+        except Exception:
+            pass
+        self.ptr = None
+
+    def __eq__(self, other):                      # PartialEq of Backend::Buf
+        return isinstance(other, HipBuf) and self.dtype == other.dtype and self.backend.equal(self, other)
+
+    __hash__ = None
+
+
+class Hip:
+    """One context (device + stream + allocator).  `Hip.new()` mirrors `Backend::new`."""
+
+    def __init__(self, device: int = 0):
+        ctx = C.c_void_p()
+        _check(lib.rt_ctx_create(device, C.byref(ctx)))
+        self._ctx = ctx
+        self.device = device
+
+    @staticmethod
+    def new(device: int = 0) -> "Hip":
+        return Hip(device)
+
+    def close(self):
+        if self._ctx:
+            lib.rt_ctx_destroy(self._ctx)
+            self._ctx = None
+
+    def sync(self):
+        _check(lib.rt_sync(self._ctx))
+
+    # ---- buffers (backend/mod.rs:225-235) --------------------------------------------------------------------------
+    def alloc(self, dtype: int, length: int) -> HipBuf:
+        p = C.c_void_p()
+        _check(lib.rt_alloc(self._ctx, dtype, length, C.byref(p)))
+        return HipBuf(self, p.value, length, dtype)
+
+    def alloc_uninit(self, dtype: int, length: int) -> HipBuf:
+        p = C.c_void_p()
+        _check(lib.rt_alloc_uninit(self._ctx, dtype, length, C.byref(p)))
+        return HipBuf(self, p.value, length, dtype)
+
+    def alloc_from_slice(self, dtype: int, src: np.ndarray) -> HipBuf:
+        src = np.ascontiguousarray(src, dtype=NP_DTYPE[dtype]).reshape(-1)
+        p = C.c_void_p()
+        _check(lib.rt_alloc_from_slice(self._ctx, dtype, src.ctypes.data_as(C.c_void_p), src.size, C.byref(p)))
+        return HipBuf(self, p.value, src.size, dtype)
+
+    def copy_from_slice(self, dst: HipBuf, src: np.ndarray):
+        src = np.ascontiguousarray(src, dtype=NP_DTYPE[dst.dtype]).reshape(-1)
+        _check(lib.rt_copy_from_slice(self._ctx, dst.dtype, dst.ptr, dst.len, src.ctypes.data_as(C.c_void_p), src.size))
+
+    def copy_range_within(self, dst: HipBuf, src: HipBuf, dst_offset: int, src_offset: int, length: int):
+        _check(lib.rt_copy_range_within(self._ctx, dst.dtype, dst.ptr, dst.len, src.ptr, src.len, dst_offset, src_offset, length))
+
+    def read(self, buf: HipBuf, offset: int):
+        out = np.zeros(1, dtype=NP_DTYPE[buf.dtype])
+        _check(lib.rt_read(self._ctx, buf.dtype, buf.ptr, buf.len, offset, out.ctypes.data_as(C.c_void_p)))
+        return out[0]
+
+    def write(self, buf: HipBuf, offset: int, value):
+        v = _value(buf.dtype, value)
+        _check(lib.rt_write(self._ctx, buf.dtype, buf.ptr, buf.len, offset, v.ctypes.data_as(C.c_void_p)))
+
+    def len(self, buf: HipBuf) -> int:
+        return buf.len
+
+    def copy(self, src: HipBuf) -> HipBuf:
+        p = C.c_void_p()
+        _check(lib.rt_copy(self._ctx, src.dtype, src.ptr, src.len, C.byref(p)))
+        return HipBuf(self, p.value, src.len, src.dtype)
+
+    def dump(self, src: HipBuf) -> np.ndarray:
+        out = np.zeros(src.len, dtype=NP_DTYPE[src.dtype])
+        _check(lib.rt_dump(self._ctx, src.dtype, src.ptr, src.len, out.ctypes.data_as(C.c_void_p)))
+        return out
+
+    def convert(self, src: HipBuf, dst: HipBuf):
+        _check(lib.rt_convert(self._ctx, src.dtype, src.ptr, src.len, dst.dtype, dst.ptr, dst.len))
+
+    def equal(self, a: HipBuf, b: HipBuf) -> bool:
+        out = C.c_int32(0)
+        _check(lib.rt_equal(self._ctx, a.dtype, a.ptr, a.len, b.ptr, b.len, C.byref(out)))
+        return bool(out.value)
+
+    # ---- fill / unary / scalar: the three layouts of the trait -------------------------------------------------------
+    def fill_contiguous(self, buf, value, start, length):
+        v = _value(buf.dtype, value)
+        _check(lib.rt_fill_contiguous(self._ctx, buf.dtype, buf.ptr, buf.len, v.ctypes.data_as(C.c_void_p), start, length))
+
+    def fill_1d_strided(self, buf, value, offset, stride, length):
+        v = _value(buf.dtype, value)
+        _check(lib.rt_fill_1d_strided(self._ctx, buf.dtype, buf.ptr, buf.len, v.ctypes.data_as(C.c_void_p), offset, stride, length))
+
+    def fill_nd(self, buf, value, offset, shape, strides):
+        v = _value(buf.dtype, value)
+        _check(lib.rt_fill_nd(self._ctx, buf.dtype, buf.ptr, buf.len, v.ctypes.data_as(C.c_void_p), offset, len(shape), _u64s(shape), _i64s(strides)))
+
+    def unary_contiguous(self, op: str, buf, start, length):
+        _check(lib.rt_unary_contiguous(self._ctx, buf.dtype, UNARY[op], buf.ptr, buf.len, start, length))
+
+    def unary_1d_strided(self, op: str, buf, offset, stride, length):
+        _check(lib.rt_unary_1d_strided(self._ctx, buf.dtype, UNARY[op], buf.ptr, buf.len, offset, stride, length))
+
+    def unary_nd(self, op: str, buf, offset, shape, strides):
+        _check(lib.rt_unary_nd(self._ctx, buf.dtype, UNARY[op], buf.ptr, buf.len, offset, len(shape), _u64s(shape), _i64s(strides)))
+
+    def scalar_contiguous(self, op: str, buf, value, start, length):
+        v = _value(buf.dtype, value)
+        _check(lib.rt_scalar_contiguous(self._ctx, buf.dtype, SCALAR[op], buf.ptr, buf.len, v.ctypes.data_as(C.c_void_p), start, length))
+
+    def scalar_1d_strided(self, op: str, buf, value, offset, stride, length):
+        v = _value(buf.dtype, value)
+        _check(lib.rt_scalar_1d_strided(self._ctx, buf.dtype, SCALAR[op], buf.ptr, buf.len, v.ctypes.data_as(C.c_void_p), offset, stride, length))
+
+    def scalar_nd(self, op: str, buf, value, offset, shape, strides):
+        v = _value(buf.dtype, value)
+        _check(lib.rt_scalar_nd(self._ctx, buf.dtype, SCALAR[op], buf.ptr, buf.len, v.ctypes.data_as(C.c_void_p), offset, len(shape),
+                                _u64s(shape), _i64s(strides)))
+
+    # The trait's default methods pick one of the three layouts from |stride| contiguity (backend/mod.rs:15-213), which
+    # sends a fully reversed view to the `_contiguous` loop with the offset of its *last* element.  Here the whole
+    # (offset, shape, strides) goes down and the C side canonicalises it with signed strides.
+    def fill(self, buf, value, meta: Tuple[int, Sequence[int], Sequence[int]]):
+        self.fill_nd(buf, value, *meta)
+
+    def apply_unary(self, op: str, buf, meta):
+        self.unary_nd(op, buf, *meta)
+
+    def scalar_apply(self, op: str, buf, value, meta):
+        self.scalar_nd(op, buf, value, *meta)
+
+    # ---- broadcast (backend/mod.rs:296-309) ----------------------------------------------------------------------------
+    def broadcast(self, left: Tuple[HipBuf, tuple], right: Tuple[HipBuf, tuple], dst: Tuple[HipBuf, tuple], op: str):
+        (lb, (loff, shape, lstr)), (rb, (roff, rshape, rstr)), (db, (doff, dshape, dstr)) = left, right, dst
+        if list(shape) != list(rshape) or list(shape) != list(dshape):
+            raise TensorError(1, f"broadcast operands must be pre-broadcast to the output shape {list(dshape)}")
+        _check(lib.rt_broadcast(self._ctx, db.dtype, BINARY[op], len(shape), _u64s(shape),
+                                lb.ptr, lb.len, loff, _i64s(lstr), rb.ptr, rb.len, roff, _i64s(rstr), db.ptr, db.len, doff, _i64s(dstr)))
+
+    # ---- reductions (backend/mod.rs:357-409) -----------------------------------------------------------------------------
+    def apply_reduce_contiguous_flat(self, src: HipBuf, dst: HipBuf, start: int, length: int, op: str):
+        _check(lib.rt_reduce_flat(self._ctx, src.dtype, REDUCE[op], src.ptr, src.len, dst.ptr, dst.len, start, length))
+
+    def apply_reduce_contiguous_nd(self, src: Tuple[HipBuf, tuple], dst: HipBuf, dim: int, op: str):
+        sb, (off, shape, strides) = src
+        _check(lib.rt_reduce_nd(self._ctx, sb.dtype, REDUCE[op], sb.ptr, sb.len, off, len(shape), _u64s(shape), _i64s(strides),
+                                dst.ptr, dst.len, dim))
+
+    def gather(self, src: HipBuf, meta, dst: HipBuf):
+        off, shape, strides = meta
+        _check(lib.rt_gather(self._ctx, src.dtype, src.ptr, src.len, off, len(shape), _u64s(shape), _i64s(strides), dst.ptr, dst.len))
+
+    # ---- timing -----------------------------------------------------------------------------------------------------------
+    def event(self):
+        e = C.c_void_p()
+        _check(lib.rt_event_create(self._ctx, C.byref(e)))
+        return e
+
+    def record(self, ev):
+        _check(lib.rt_event_record(self._ctx, ev))
+
+    def elapsed_ms(self, start, stop) -> float:
+        out = C.c_float(0)
+        _check(lib.rt_event_elapsed_ms(self._ctx, start, stop, C.byref(out)))
+        return out.value
+
+    def mem_stats(self):
+        a, b, c = C.c_uint64(0), C.c_uint64(0), C.c_uint64(0)
+        _check(lib.rt_mem_stats(self._ctx, C.byref(a), C.byref(b), C.byref(c)))
+        return {"in_use": a.value, "cached": b.value, "device_allocs": c.value}

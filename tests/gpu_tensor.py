@@ -1,0 +1,142 @@
+"""Test helper: the reference's tensor surface (views, operators, reductions) driven through the C ABI of the HIP
+backend.  Layout arithmetic comes from the oracle's metadata restatement, so a test can run the same program on the
+oracle's OTensor and on a GTensor and compare buffers."""
+from __future__ import annotations
+
+import numpy as np
+
+from oracle.meta import (MetaTensor, Slice, TensorError, compute_broadcasted_params, compute_permuted_parameters,
+                         compute_sliced_parameters, compute_squeezed_parameters, compute_unsqueezed_parameters,
+                         logical_to_buffer_idx, reduction_output_meta)
+from rtensors_amd import hip as H
+
+
+def _m(meta: MetaTensor):
+    return (meta.offset, list(meta.shape), list(meta.strides))
+
+
+class GTensor:
+    def __init__(self, backend, buf, meta: MetaTensor, is_view=False):
+        self.backend, self.buf, self.meta, self.is_view = backend, buf, meta, is_view
+        self.dtype = buf.dtype
+
+    @staticmethod
+    def from_buf(backend, dtype, values, shape):
+        if isinstance(dtype, str):
+            dtype = H.DTYPE_BY_NAME[dtype]
+        arr = np.asarray(values).astype(H.NP_DTYPE[dtype]).reshape(-1)
+        meta = MetaTensor.row_major(list(shape))
+        if arr.size != meta.size():
+            raise TensorError("InvalidShape", "size")
+        return GTensor(backend, backend.alloc_from_slice(dtype, arr), meta)
+
+    def _view(self, shape, strides, offset):
+        return GTensor(self.backend, self.buf, MetaTensor(list(shape), list(strides), offset), True)
+
+    def view(self): return self._view(self.meta.shape, self.meta.strides, self.meta.offset)
+
+    def slice(self, dim, sl):
+        if isinstance(sl, int):
+            sl = Slice.index(sl)
+        return self._view(*compute_sliced_parameters(self.meta.shape, self.meta.strides, self.meta.offset, dim, sl))
+
+    def permute(self, dims):
+        shape, strides = compute_permuted_parameters(self.meta.shape, self.meta.strides, list(dims))
+        return self._view(shape, strides, self.meta.offset)
+
+    def transpose(self): return self.permute(list(range(self.meta.rank() - 1, -1, -1)))
+
+    def unsqueeze_at(self, d):
+        shape, strides = compute_unsqueezed_parameters(self.meta.shape, self.meta.strides, d)
+        return self._view(shape, strides, self.meta.offset)
+
+    def squeeze_at(self, d):
+        shape, strides = compute_squeezed_parameters(self.meta.shape, self.meta.strides, d)
+        return self._view(shape, strides, self.meta.offset)
+
+    def squeeze(self):
+        shape, strides = compute_squeezed_parameters(self.meta.shape, self.meta.strides, None)
+        return self._view(shape, strides, self.meta.offset)
+
+    def get(self, idx):
+        return self.backend.read(self.buf, logical_to_buffer_idx(list(idx), self.meta.strides, self.meta.offset))
+
+    def dump(self): return self.backend.dump(self.buf)
+
+    def owned(self):
+        if not self.is_view:
+            return GTensor(self.backend, self.backend.copy(self.buf), MetaTensor(list(self.meta.shape), list(self.meta.strides), self.meta.offset))
+        return self._gathered()
+
+    def contiguous(self):
+        if not self.is_view and self.meta.is_contiguous():
+            return self.owned()
+        return self._gathered()
+
+    def _gathered(self):
+        out = self.backend.alloc_uninit(self.dtype, self.meta.size())
+        self.backend.gather(self.buf, _m(self.meta), out)
+        return GTensor(self.backend, out, MetaTensor.row_major(self.meta.shape))
+
+    def to_numpy(self):
+        return self._gathered().dump().reshape(self.meta.shape)
+
+    def _binary(self, other, op):
+        out_shape, stra, strb = compute_broadcasted_params(self.meta, other.meta)
+        result = GTensor(self.backend, self.backend.alloc(self.dtype, int(np.prod(out_shape, dtype=np.int64)) if out_shape else 1),
+                         MetaTensor.row_major(out_shape))
+        self.backend.broadcast((self.buf, (self.meta.offset, out_shape, stra)), (other.buf, (other.meta.offset, out_shape, strb)),
+                               (result.buf, _m(result.meta)), op)
+        return result
+
+    def _binary_assign(self, other, op):
+        out_shape, stra, strb = compute_broadcasted_params(self.meta, other.meta)
+        if list(self.meta.shape) != list(out_shape):
+            raise TensorError("Panic", "incompatible shapes for in-place op")
+        a = (self.meta.offset, out_shape, stra)
+        self.backend.broadcast((self.buf, a), (other.buf, (other.meta.offset, out_shape, strb)), (self.buf, a), op)
+        return self
+
+    def _scalar_assign(self, v, op):
+        self.backend.scalar_apply(op, self.buf, v, _m(self.meta))
+        return self
+
+    def _d(self, o, op, assign):
+        if isinstance(o, GTensor):
+            return self._binary_assign(o, op) if assign else self._binary(o, op)
+        return self._scalar_assign(o, op) if assign else self.owned()._scalar_assign(o, op)
+
+    def __add__(self, o): return self._d(o, "add", False)
+    def __sub__(self, o): return self._d(o, "sub", False)
+    def __mul__(self, o): return self._d(o, "mul", False)
+    def __truediv__(self, o): return self._d(o, "div", False)
+    def __iadd__(self, o): return self._d(o, "add", True)
+    def __isub__(self, o): return self._d(o, "sub", True)
+    def __imul__(self, o): return self._d(o, "mul", True)
+    def __itruediv__(self, o): return self._d(o, "div", True)
+
+    def unary_inplace(self, op):
+        self.backend.apply_unary(op, self.buf, _m(self.meta))
+        return self
+
+    def unary(self, op): return self.owned().unary_inplace(op)
+
+    def scalar_op_inplace(self, op, v):
+        self.backend.scalar_apply(op, self.buf, v, _m(self.meta))
+        return self
+
+    def fill(self, v): self.backend.fill(self.buf, v, _m(self.meta))
+
+    def reduce(self, op, axis=None):
+        t = self if self.meta.is_contiguous() and all(s >= 0 for s in self.meta.strides) else self.contiguous()
+        if axis is None:
+            out = self.backend.alloc(t.dtype, 1)
+            self.backend.apply_reduce_contiguous_flat(t.buf, out, t.meta.offset, t.meta.size(), op)
+            return GTensor(self.backend, out, MetaTensor([], [], 0))
+        om = reduction_output_meta(t.meta, axis)
+        out = self.backend.alloc(t.dtype, om.size())
+        if t.meta.rank() == 1:
+            self.backend.apply_reduce_contiguous_flat(t.buf, out, t.meta.offset, t.meta.size(), op)
+        else:
+            self.backend.apply_reduce_contiguous_nd((t.buf, _m(t.meta)), out, axis, op)
+        return GTensor(self.backend, out, om)
