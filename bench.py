@@ -1,0 +1,327 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X backend hot path: achieved HBM GB/s (and % of the 8 TB/s peak) per kernel.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--kernel NAME] [--no-cpu] [--no-detail]
+
+One "step" is the headline pair of BASELINE.json's metric at its >= 1 GiB shapes: the strided broadcast add of
+config 3 (x (16,1,512,1024) + y (1,64,1,1024) -> 2 GiB f32) followed by the axis sum of config 4 (sum over the last
+axis of (8192,32768) f32, 1 GiB).  Inputs are generated on the device and resident in HBM before the timed region.
+`value` = algorithmic bytes of one step / time of one step.  Every other kernel of configs 1-5 is timed once more in
+`detail`.  `--kernel NAME` runs a single kernel only (used for the rocprofv3 runs whose summaries live in profiles/).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_HBM = 8.0e12   # bytes/s, MI355X HBM3E
+
+# HBM bytes per launch of the config-3 broadcast-add kernel, from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE, each
+# scaled by what the same counter reads for the 1 GiB copy kernel (x2.000 and x1.000); see
+# profiles/bin_rows_kernel_config3_broadcast_add.txt.  Algorithmic bytes are 2181300224: nothing is re-read.
+MEASURED_TRAFFIC_C3A = 2181208987
+
+
+def row_major(shape):
+    st = [1] * len(shape)
+    for i in range(len(shape) - 2, -1, -1):
+        st[i] = st[i + 1] * shape[i + 1]
+    return st
+
+
+class Workloads:
+    """Builds the device tensors of configs 1-5 lazily and exposes each kernel as a closure `() -> None` plus its
+    algorithmic bytes (unique input elements + output elements, times sizeof)."""
+
+    def __init__(self, hip):
+        from rtensors_amd import datagen, hip as H
+        self.hip, self.H, self.dg = hip, H, datagen
+        self._cache = {}
+
+    def _gen(self, name, dtype, n, dist, seed, stream, p0=1.0, p1=0.0):
+        key = (name,)
+        if key not in self._cache:
+            b = self.hip.alloc_uninit(dtype, n)
+            self.dg.fill_device(b, dist, seed, stream, p0, p1)
+            self._cache[key] = b
+        return self._cache[key]
+
+    def _out(self, name, dtype, n):
+        key = (name, "out")
+        if key not in self._cache:
+            self._cache[key] = self.hip.alloc_uninit(dtype, n)
+        return self._cache[key]
+
+    def drop(self):
+        self._cache.clear()
+
+    # ---- config 3: strided broadcast --------------------------------------------------------------------------------
+    def c3a_add(self):
+        H = self.H
+        x = self._gen("c3x", H.F32, 16 * 512 * 1024, "normal", 2, 0)
+        y = self._gen("c3y", H.F32, 64 * 1024, "uniform", 2, 1)
+        shape = [16, 64, 512, 1024]
+        z = self._out("c3z", H.F32, 16 * 64 * 512 * 1024)
+        left = (x, (0, shape, [524288, 0, 1024, 1]))
+        right = (y, (0, shape, [0, 1024, 0, 1]))
+        dst = (z, (0, shape, row_major(shape)))
+        nbytes = (x.len + y.len + z.len) * 4
+        return (lambda: self.hip.broadcast(left, right, dst, "add")), nbytes, z.len
+
+    def c3b_add(self):
+        # x = contiguous (16,1024,512) .permute([0,2,1]) .slice(1, step -1) .unsqueeze_at(1), broadcast along dim 1:
+        # strides (524288, 0, -1, 512), offset 511
+        H = self.H
+        x = self._gen("c3x", H.F32, 16 * 512 * 1024, "normal", 2, 0)
+        y = self._gen("c3y", H.F32, 64 * 1024, "uniform", 2, 1)
+        shape = [16, 64, 512, 1024]
+        z = self._out("c3z", H.F32, 16 * 64 * 512 * 1024)
+        left = (x, (511, shape, [524288, 0, -1, 512]))
+        right = (y, (0, shape, [0, 1024, 0, 1]))
+        dst = (z, (0, shape, row_major(shape)))
+        nbytes = (x.len + y.len + z.len) * 4
+        return (lambda: self.hip.broadcast(left, right, dst, "add")), nbytes, z.len
+
+    # ---- config 4: reductions ---------------------------------------------------------------------------------------------
+    def _c4(self, dtype_name):
+        H = self.H
+        if dtype_name == "f32":
+            return self._gen("c4t", H.F32, 8192 * 32768, "normal", 3, 0)
+        return self._gen("c4i", H.I32, 8192 * 32768, "int", 3, 1, -1000, 1000)
+
+    def _c4_axis(self, dtype_name, op, dim):
+        H = self.H
+        t = self._c4(dtype_name)
+        shape = [8192, 32768]
+        nout = shape[1 - dim]
+        out = self._out(f"c4o{dim}{dtype_name}", t.dtype, nout)
+        src = (t, (0, shape, [32768, 1]))
+        return (lambda: self.hip.apply_reduce_contiguous_nd(src, out, dim, op)), (t.len + nout) * 4, t.len
+
+    def c4_sum1(self): return self._c4_axis("f32", "sum", 1)
+    def c4_mean1(self): return self._c4_axis("f32", "mean", 1)
+    def c4_max1(self): return self._c4_axis("f32", "max", 1)
+    def c4_sum0(self): return self._c4_axis("f32", "sum", 0)
+    def c4_i32_sum1(self): return self._c4_axis("i32", "sum", 1)
+    def c4_i32_max1(self): return self._c4_axis("i32", "max", 1)
+    def c4_i32_min0(self): return self._c4_axis("i32", "min", 0)
+
+    def c4_sum_all(self):
+        t = self._c4("f32")
+        out = self._out("c4oall", t.dtype, 1)
+        return (lambda: self.hip.apply_reduce_contiguous_flat(t, out, 0, t.len, "sum")), (t.len + 1) * 4, t.len
+
+    # ---- config 2: contiguous elementwise chain ----------------------------------------------------------------------------
+    def _c2(self, which, dtype_name="f32"):
+        H = self.H
+        if dtype_name == "f32":
+            dt, n, es = H.F32, 1 << 28, 4
+            a = self._gen("c2a", dt, n, "normal", 1, 0); b = self._gen("c2b", dt, n, "normal", 1, 1)
+        elif dtype_name == "f64":
+            dt, n, es = H.F64, 1 << 27, 8
+            a = self._gen("c2a64", dt, n, "normal", 1, 0); b = self._gen("c2b64", dt, n, "normal", 1, 1)
+        else:
+            dt, n, es = H.I32, 1 << 28, 4
+            a = self._gen("c2ai", dt, n, "int", 1, 0, -(1 << 20), 1 << 20); b = self._gen("c2bi", dt, n, "int", 1, 1, -(1 << 20), 1 << 20)
+        c = self._out("c2c" + dtype_name, dt, n)
+        m = (0, [n], [1])
+        three = 3 if dtype_name == "i32" else 3.0
+        one = 1 if dtype_name == "i32" else 1.0
+        if which == "mul":
+            return (lambda: self.hip.scalar_contiguous("mul", a, three, 0, n)), 2 * n * es, n
+        if which == "add":
+            return (lambda: self.hip.broadcast((a, m), (b, m), (c, m), "add")), 3 * n * es, n
+        if which == "relu":
+            return (lambda: self.hip.unary_contiguous("relu", c, 0, n)), 2 * n * es, n
+        if which == "sub":
+            return (lambda: self.hip.scalar_contiguous("sub", c, one, 0, n)), 2 * n * es, n
+        if which == "copy":
+            return (lambda: self.hip.gather(a, m, c)), 2 * n * es, n
+        if which == "fill":
+            return (lambda: self.hip.fill_contiguous(c, one, 0, n)), n * es, n
+        raise KeyError(which)
+
+    def c2_mul(self): return self._c2("mul")
+    def c2_add(self): return self._c2("add")
+    def c2_relu(self): return self._c2("relu")
+    def c2_sub(self): return self._c2("sub")
+    def c2_f64_add(self): return self._c2("add", "f64")
+    def c2_f64_mul(self): return self._c2("mul", "f64")
+    def c2_i32_add(self): return self._c2("add", "i32")
+    def c2_i32_mul(self): return self._c2("mul", "i32")
+    def copy(self): return self._c2("copy")
+    def fill(self): return self._c2("fill")
+
+    # ---- config 1 -------------------------------------------------------------------------------------------------------------
+    def c1_add(self):
+        H = self.H
+        a = self._gen("c1a", H.F32, 4096, "uniform", 0, 0); b = self._gen("c1b", H.F32, 4096, "uniform", 0, 1)
+        c = self._out("c1c", H.F32, 4096 * 4096)
+        shape = [4096, 4096]
+        return (lambda: self.hip.broadcast((a, (0, shape, [0, 1])), (b, (0, shape, [1, 0])), (c, (0, shape, [4096, 1])), "add")), \
+            (4096 + 4096 + 4096 * 4096) * 4, 4096 * 4096
+
+    def c1_sum1(self):
+        H = self.H
+        self.c1_add()[0]()
+        c = self._out("c1c", H.F32, 4096 * 4096)
+        s = self._out("c1s", H.F32, 4096)
+        return (lambda: self.hip.apply_reduce_contiguous_nd((c, (0, [4096, 4096], [4096, 1])), s, 1, "sum")), (4096 * 4096 + 4096) * 4, 4096 * 4096
+
+    # ---- config 5: the graded reduction (d(bias) = column sum over the batch dim) and the bias add --------------------------------
+    def c5_bias_add(self):
+        H = self.H
+        x = self._gen("c5x", H.F32, 65536 * 4096, "normal", 4, 0)
+        bias = self._gen("c5b", H.F32, 4096, "normal", 4, 1, 0.1)
+        y = self._out("c5y", H.F32, 65536 * 4096)
+        shape = [65536, 4096]
+        return (lambda: self.hip.broadcast((x, (0, shape, [4096, 1])), (bias, (0, shape, [0, 1])), (y, (0, shape, [4096, 1])), "add")), \
+            (2 * x.len + 4096) * 4, x.len
+
+    def c5_colsum(self):
+        H = self.H
+        x = self._gen("c5x", H.F32, 65536 * 4096, "normal", 4, 0)
+        g = self._out("c5g", H.F32, 4096)
+        return (lambda: self.hip.apply_reduce_contiguous_nd((x, (0, [65536, 4096], [4096, 1])), g, 0, "sum")), (x.len + 4096) * 4, x.len
+
+
+HEADLINE = ["c3a_add", "c4_sum1"]
+DETAIL = ["copy", "fill", "c1_add", "c1_sum1", "c2_mul", "c2_add", "c2_relu", "c2_sub", "c2_f64_mul", "c2_f64_add", "c2_i32_mul", "c2_i32_add",
+          "c3a_add", "c3b_add", "c4_sum1", "c4_mean1", "c4_max1", "c4_sum0", "c4_sum_all", "c4_i32_sum1", "c4_i32_max1", "c4_i32_min0",
+          "c5_bias_add", "c5_colsum"]
+KIND = {"copy": "elementwise", "fill": "elementwise"}
+
+
+def time_kernel(hip, fn, iters, warmup):
+    """Average duration in ms of `fn`'s launch, HIP events on the backend's own stream."""
+    for _ in range(warmup):
+        fn()
+    evs = [hip.event() for _ in range(iters + 1)]
+    hip.record(evs[0])
+    for i in range(iters):
+        fn()
+        hip.record(evs[i + 1])
+    hip.sync()
+    times = [hip.elapsed_ms(evs[i], evs[i + 1]) for i in range(iters)]
+    return float(np.mean(times)), float(np.median(times)), float(np.min(times))
+
+
+def cpu_baseline():
+    """The CPU oracle (C++ restatement of the reference's single-threaded Cpu backend) timed on a bounded sample of the
+    headline step: 4 of the 16 batch slices of the config-3 broadcast add, and the whole config-4 axis sum."""
+    from oracle import cpu
+    from oracle.meta import MetaTensor
+    from rtensors_amd import datagen
+    cpu.build()
+    nb = 4
+    x = datagen.normal(np.float32, nb * 512 * 1024, 2, 0)
+    y = datagen.uniform(np.float32, 64 * 1024, 2, 1)
+    shape = [nb, 64, 512, 1024]
+    z = np.zeros(nb * 64 * 512 * 1024, dtype=np.float32)
+    t0 = time.perf_counter()
+    cpu.broadcast(cpu.F32, "add", x, MetaTensor(shape, [524288, 0, 1024, 1], 0), y, MetaTensor(shape, [0, 1024, 0, 1], 0),
+                  z, MetaTensor(shape, row_major(shape), 0))
+    t_add = time.perf_counter() - t0
+    add_bytes = (x.size + y.size + z.size) * 4
+    del z
+    rows = 8192
+    t = datagen.normal(np.float32, rows * 32768, 3, 0)
+    t0 = time.perf_counter()
+    cpu.reduce_nd(cpu.F32, "sum", t, MetaTensor([rows, 32768], [32768, 1], 0), 1)
+    t_sum = time.perf_counter() - t0
+    sum_bytes = (t.size + rows) * 4
+    return {
+        "value": round((add_bytes + sum_bytes) / (t_add + t_sum) / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+        "sample": f"config-3 add on {nb}/16 batch slices ({add_bytes / 2**20:.0f} MiB, {t_add:.2f} s, {add_bytes / t_add / 1e9:.3f} GB/s) "
+                  f"+ full config-4 sum_at(1) ({sum_bytes / 2**20:.0f} MiB, {t_sum:.2f} s, {sum_bytes / t_sum / 1e9:.3f} GB/s); "
+                  f"host has {os.cpu_count()} logical cpus, the reference Cpu backend uses 1",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--kernel", type=str, default=None, help="run only this kernel (see DETAIL) --steps times")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-detail", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    from rtensors_amd import hip as H      # raises if librt_hip.so is missing: there is no CPU fallback
+    hip = H.Hip.new(0)
+    w = Workloads(hip)
+
+    if args.kernel:
+        fn, nbytes, nelem = getattr(w, args.kernel)()
+        mean, med, mn = time_kernel(hip, fn, args.steps, args.warmup)
+        print(json.dumps({"kernel": args.kernel, "ms_mean": mean, "ms_median": med, "ms_min": mn, "bytes": nbytes,
+                          "GBps": nbytes / (mean * 1e-3) / 1e9, "frac_of_peak": nbytes / (mean * 1e-3) / PEAK_HBM}))
+        return
+
+    # ---- headline step ---------------------------------------------------------------------------------------------------
+    add_fn, add_bytes, add_elems = w.c3a_add()
+    sum_fn, sum_bytes, sum_elems = w.c4_sum1()
+    for _ in range(args.warmup):
+        add_fn(); sum_fn()
+    K = args.steps
+    evs = [hip.event() for _ in range(2 * K + 1)]
+    hip.sync()
+    t0 = time.perf_counter()
+    hip.record(evs[0])
+    for i in range(K):
+        add_fn()
+        hip.record(evs[2 * i + 1])
+        sum_fn()
+        hip.record(evs[2 * i + 2])
+    hip.sync()
+    wall = time.perf_counter() - t0
+    add_ms = float(np.mean([hip.elapsed_ms(evs[2 * i], evs[2 * i + 1]) for i in range(K)]))
+    sum_ms = float(np.mean([hip.elapsed_ms(evs[2 * i + 1], evs[2 * i + 2]) for i in range(K)]))
+    ms_per_step = wall * 1e3 / K
+    step_bytes = add_bytes + sum_bytes
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    detail = {}
+    if not args.no_detail:
+        for name in DETAIL:
+            fn, nbytes, nelem = getattr(w, name)()
+            mean, med, mn = time_kernel(hip, fn, 10, 2)
+            detail[name] = {"ms": round(mean, 4), "GBps": round(nbytes / (mean * 1e-3) / 1e9, 1),
+                            "frac": round(nbytes / (mean * 1e-3) / PEAK_HBM, 4), "Gelem_s": round(nelem / (mean * 1e-3) / 1e9, 2)}
+    w.drop()
+
+    out = {
+        "metric": "achieved HBM GB/s (% of peak) for broadcast-add + axis-sum, f32, 1 MI355X",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "config 3 strided broadcast add x(16,1,512,1024)+y(1,64,1,1024)->(16,64,512,1024) f32 (2 GiB out), "
+                               "then config 4 sum over the last axis of (8192,32768) f32 (1 GiB in)",
+                   "bytes_per_step": step_bytes, "pct_of_peak": round(100 * value * 1e9 / PEAK_HBM, 2)},
+        "roofline": {"bound": "hbm", "kernel": "bin_rows_kernel<float, add> (config 3 broadcast add)",
+                     "achieved": round(add_bytes / (add_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM / 1e9, "unit": "GB/s",
+                     "frac": round(add_bytes / (add_ms * 1e-3) / PEAK_HBM, 4), "traffic": MEASURED_TRAFFIC_C3A,
+                     "kernel_ms": round(add_ms, 4),
+                     "axis_sum": {"kernel": "reduce_rows_block_kernel<sum, float>", "achieved": round(sum_bytes / (sum_ms * 1e-3) / 1e9, 1),
+                                  "frac": round(sum_bytes / (sum_ms * 1e-3) / PEAK_HBM, 4), "kernel_ms": round(sum_ms, 4)}},
+        "detail": detail,
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -61,40 +61,24 @@ template <int OP, class T> __device__ __forceinline__ T bin_apply(T a, T b) {
 
 template <class T> struct alignas(16) Vec16 { T e[16 / sizeof(T)]; };
 
-constexpr int kBlock = 256;
-constexpr int kGU = 4;          // iterations of the loop dim whose loads are issued before the first store
+constexpr int kBlock = 256;     // generic kernels
+constexpr int kRBlock = 128;    // contig / rows kernels: small blocks, one 16-byte vector per lane per step
 
 enum Mode : int { M_VEC = 0, M_BCAST = 1, M_ELEM = 2 };
 
 // ---- contig ---------------------------------------------------------------------------------------------------------
+// One vector per lane, non-temporal loads and stores: every byte is touched exactly once.
 template <class T, int OP>
-__global__ __launch_bounds__(kBlock) void bin_contig_kernel(const Vec16<T>* l, const Vec16<T>* r, Vec16<T>* d, size_t nvec) {
+__global__ __launch_bounds__(kRBlock) void bin_contig_kernel(const Vec16<T>* l, const Vec16<T>* r, Vec16<T>* d, size_t nvec) {
     constexpr int N = 16 / sizeof(T);
-    constexpr int U = 4;
-    const size_t base = (size_t)blockIdx.x * (kBlock * U) + threadIdx.x;
-    if (base + (size_t)(U - 1) * kBlock < nvec) {
-        Vec16<T> a[U], b[U];
+    const size_t i = (size_t)blockIdx.x * kRBlock + threadIdx.x;
+    if (i >= nvec) return;
+    Vec16<T> a = rt_ld16_nt(l + i);
+    Vec16<T> b;
+    if constexpr (OP != kOpCopy) b = rt_ld16_nt(r + i); else b = a;
 #pragma unroll
-        for (int u = 0; u < U; ++u) { a[u] = l[base + (size_t)u * kBlock]; b[u] = r[base + (size_t)u * kBlock]; }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-#pragma unroll
-            for (int j = 0; j < N; ++j) a[u].e[j] = bin_apply<OP, T>(a[u].e[j], b[u].e[j]);
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) d[base + (size_t)u * kBlock] = a[u];
-    } else {
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const size_t i = base + (size_t)u * kBlock;
-            if (i < nvec) {
-                Vec16<T> a = l[i], b = r[i];
-#pragma unroll
-                for (int j = 0; j < N; ++j) a.e[j] = bin_apply<OP, T>(a.e[j], b.e[j]);
-                d[i] = a;
-            }
-        }
-    }
+    for (int j = 0; j < N; ++j) a.e[j] = bin_apply<OP, T>(a.e[j], b.e[j]);
+    rt_st16_nt(d + i, a);
 }
 
 // ---- rows -------------------------------------------------------------------------------------------------------------
@@ -104,7 +88,8 @@ struct RowArgs {
     uint32_t gchunk;                // loop-dim iterations owned by one block
     uint32_t nchunks;               // ceil(G / gchunk)
     uint32_t tiles;                 // column tiles per row
-    uint32_t tpr;                   // lanes per row inside a block (power of two <= kBlock)
+    uint32_t tpr;                   // lanes per row inside a block (power of two <= kRBlock)
+    uint32_t nt_mask;               // bit o set: operand o (0 left, 1 right) is streamed -> non-temporal loads
     FastDiv32 tiles_div, nchunks_div;
     int nouter;                     // remaining outer dims (loop dim and inner dim excluded), outermost first
     uint32_t oshape[RT_MAX_RANK];
@@ -115,11 +100,12 @@ struct RowArgs {
 };
 
 template <class T, int MODE>
-__device__ __forceinline__ Vec16<T> load_vec(const T* __restrict__ rowp, uint32_t c, int64_t istride) {
+__device__ __forceinline__ Vec16<T> load_vec(const T* __restrict__ rowp, uint32_t c, int64_t istride, bool nt) {
     constexpr int N = 16 / sizeof(T);
     Vec16<T> v;
     if constexpr (MODE == M_VEC) {
-        v = *reinterpret_cast<const Vec16<T>*>(rowp + c);
+        const Vec16<T>* q = reinterpret_cast<const Vec16<T>*>(rowp + c);
+        v = nt ? rt_ld16_nt(q) : rt_ld16(q);
     } else if constexpr (MODE == M_BCAST) {
         T x = rowp[0];
 #pragma unroll
@@ -132,7 +118,7 @@ __device__ __forceinline__ Vec16<T> load_vec(const T* __restrict__ rowp, uint32_
 }
 
 template <class T, int OP, int LM, int RM>
-__global__ __launch_bounds__(kBlock) void bin_rows_kernel(const T* l, const T* r, T* d, RowArgs a) {
+__global__ __launch_bounds__(kRBlock) void bin_rows_kernel(const T* l, const T* r, T* d, RowArgs a) {
     constexpr int N = 16 / sizeof(T);
     // blockIdx -> (outer index, chunk of the loop dim, column tile); all uniform, computed on the scalar unit
     uint32_t b = blockIdx.x;
@@ -156,51 +142,35 @@ __global__ __launch_bounds__(kBlock) void bin_rows_kernel(const T* l, const T* r
     }
     const uint32_t tx = threadIdx.x & (a.tpr - 1);
     const uint32_t ty = threadIdx.x / a.tpr;
-    const uint32_t gy = kBlock / a.tpr;
+    const uint32_t gy = kRBlock / a.tpr;
     const uint32_t c = (tile * a.tpr + tx) * N;                 // first column of this lane's vector
     if (c >= a.L) return;
     const uint32_t g_begin = chunk * a.gchunk;
     const uint32_t g_end = min(a.G, g_begin + a.gchunk);
-    const bool full = (c + N <= a.L);
+    const bool ntl = (a.nt_mask & 1u) != 0, ntr = (a.nt_mask & 2u) != 0;
 
-    const bool l_fixed = (a.gstride[0] == 0), r_fixed = (a.gstride[1] == 0);
-    Vec16<T> lh, rh;                                            // operands that do not move along the loop dim
-    if (full) {
-        if (l_fixed) lh = load_vec<T, LM>(l + ol, c, a.istride[0]);
-        if (r_fixed) rh = load_vec<T, RM>(r + orr, c, a.istride[1]);
-    }
-    for (uint32_t g0 = g_begin + ty; g0 < g_end; g0 += gy * kGU) {
-        if (full) {
-            Vec16<T> x[kGU], y[kGU];
+    if (c + N <= a.L) {
+        const bool l_fixed = (a.gstride[0] == 0), r_fixed = (a.gstride[1] == 0);
+        Vec16<T> lh, rh;                                        // operands that do not move along the loop dim
+        if (l_fixed) lh = load_vec<T, LM>(l + ol, c, a.istride[0], false);
+        if (r_fixed) rh = load_vec<T, RM>(r + orr, c, a.istride[1], false);
+        for (uint32_t g = g_begin + ty; g < g_end; g += gy) {
+            Vec16<T> x = l_fixed ? lh : load_vec<T, LM>(l + ol + (int64_t)g * a.gstride[0], c, a.istride[0], ntl);
+            Vec16<T> y;
+            if constexpr (OP == kOpCopy) y = x;
+            else y = r_fixed ? rh : load_vec<T, RM>(r + orr + (int64_t)g * a.gstride[1], c, a.istride[1], ntr);
 #pragma unroll
-            for (int u = 0; u < kGU; ++u) {
-                const uint32_t g = g0 + u * gy;
-                if (g < g_end) {
-                    x[u] = l_fixed ? lh : load_vec<T, LM>(l + ol + (int64_t)g * a.gstride[0], c, a.istride[0]);
-                    y[u] = r_fixed ? rh : load_vec<T, RM>(r + orr + (int64_t)g * a.gstride[1], c, a.istride[1]);
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < kGU; ++u) {
-                const uint32_t g = g0 + u * gy;
-                if (g < g_end) {
-#pragma unroll
-                    for (int j = 0; j < N; ++j) x[u].e[j] = bin_apply<OP, T>(x[u].e[j], y[u].e[j]);
-                    *reinterpret_cast<Vec16<T>*>(d + od + (int64_t)g * a.gstride[2] + c) = x[u];
-                }
-            }
-        } else {
-            // ragged end of a row: element accesses
-            for (int u = 0; u < kGU; ++u) {
-                const uint32_t g = g0 + u * gy;
-                if (g < g_end) {
-                    const T* lp = l + ol + (int64_t)g * a.gstride[0];
-                    const T* rp = r + orr + (int64_t)g * a.gstride[1];
-                    T* dp = d + od + (int64_t)g * a.gstride[2];
-                    for (uint32_t k = c; k < a.L; ++k)
-                        dp[k] = bin_apply<OP, T>(lp[(int64_t)k * a.istride[0]], rp[(int64_t)k * a.istride[1]]);
-                }
-            }
+            for (int j = 0; j < N; ++j) x.e[j] = bin_apply<OP, T>(x.e[j], y.e[j]);
+            rt_st16_nt(reinterpret_cast<Vec16<T>*>(d + od + (int64_t)g * a.gstride[2] + c), x);
+        }
+    } else {
+        // ragged end of a row: element accesses
+        for (uint32_t g = g_begin + ty; g < g_end; g += gy) {
+            const T* lp = l + ol + (int64_t)g * a.gstride[0];
+            const T* rp = r + orr + (int64_t)g * a.gstride[1];
+            T* dp = d + od + (int64_t)g * a.gstride[2];
+            for (uint32_t k = c; k < a.L; ++k)
+                dp[k] = bin_apply<OP, T>(lp[(int64_t)k * a.istride[0]], rp[(int64_t)k * a.istride[1]]);
         }
     }
 }
@@ -258,9 +228,9 @@ __global__ __launch_bounds__(kBlock) void bin_generic64_kernel(const T* l, const
 template <class T, int OP, int LM>
 void launch_rows_r(int rm, dim3 grid, hipStream_t s, const T* l, const T* r, T* d, const RowArgs& a) {
     switch (rm) {
-        case M_VEC: hipLaunchKernelGGL((bin_rows_kernel<T, OP, LM, M_VEC>), grid, dim3(kBlock), 0, s, l, r, d, a); break;
-        case M_BCAST: hipLaunchKernelGGL((bin_rows_kernel<T, OP, LM, M_BCAST>), grid, dim3(kBlock), 0, s, l, r, d, a); break;
-        default: hipLaunchKernelGGL((bin_rows_kernel<T, OP, LM, M_ELEM>), grid, dim3(kBlock), 0, s, l, r, d, a); break;
+        case M_VEC: hipLaunchKernelGGL((bin_rows_kernel<T, OP, LM, M_VEC>), grid, dim3(kRBlock), 0, s, l, r, d, a); break;
+        case M_BCAST: hipLaunchKernelGGL((bin_rows_kernel<T, OP, LM, M_BCAST>), grid, dim3(kRBlock), 0, s, l, r, d, a); break;
+        default: hipLaunchKernelGGL((bin_rows_kernel<T, OP, LM, M_ELEM>), grid, dim3(kRBlock), 0, s, l, r, d, a); break;
     }
 }
 template <class T, int OP>
@@ -294,9 +264,11 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
     const int rank = dsc.rank;
 
     // (1) one unit-stride run in all three operands
-    if (rank <= 1 && (rank == 0 || (dsc.stride[0][0] == 1 && dsc.stride[1][0] == 1 && dsc.stride[2][0] == 1))) {
+    // (for the gather op the right operand is a placeholder that is never read: treat it as a twin of the left one)
+    const bool r_unit = (OP == kOpCopy) || rank == 0 || dsc.stride[1][0] == 1;
+    if (rank <= 1 && (rank == 0 || (dsc.stride[0][0] == 1 && r_unit && dsc.stride[2][0] == 1))) {
         const T* lp = l + dsc.offset[0];
-        const T* rp = r + dsc.offset[1];
+        const T* rp = (OP == kOpCopy) ? lp : r + dsc.offset[1];
         T* dp = d + dsc.offset[2];
         uintptr_t al = reinterpret_cast<uintptr_t>(lp) & 15, ar = reinterpret_cast<uintptr_t>(rp) & 15, ad = reinterpret_cast<uintptr_t>(dp) & 15;
         if (al == ar && ar == ad) {
@@ -305,9 +277,9 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
             if (head > n) head = n;
             size_t nvec = (n - head) / N, tail = n - head - nvec * N;
             if (nvec) {
-                size_t blocks = (nvec + (size_t)kBlock * 4 - 1) / ((size_t)kBlock * 4);
+                size_t blocks = (nvec + (size_t)kRBlock - 1) / (size_t)kRBlock;
                 if (blocks > 0x7fffffffull) return rt_fail(RT_E_INVALID, "broadcast: %zu elements is too long for one launch", n);
-                hipLaunchKernelGGL((bin_contig_kernel<T, OP>), dim3((unsigned)blocks), dim3(kBlock), 0, s,
+                hipLaunchKernelGGL((bin_contig_kernel<T, OP>), dim3((unsigned)blocks), dim3(kRBlock), 0, s,
                                    reinterpret_cast<const Vec16<T>*>(lp + head), reinterpret_cast<const Vec16<T>*>(rp + head),
                                    reinterpret_cast<Vec16<T>*>(dp + head), nvec);
             }
@@ -334,11 +306,27 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
         a.L = (uint32_t)dsc.shape[rank - 1];
         a.istride[0] = dsc.stride[0][rank - 1];
         a.istride[1] = dsc.stride[1][rank - 1];
-        // loop dim: the largest outer dim along which one input does not move; else the innermost outer dim
-        int gdim = -1;
-        for (int k = 0; k < rank - 1; ++k)
-            if ((dsc.stride[0][k] == 0 || dsc.stride[1][k] == 0) && (gdim < 0 || dsc.shape[k] > dsc.shape[gdim])) gdim = k;
-        if (gdim < 0 && rank >= 2) gdim = rank - 2;
+        auto mode = [&](int o, const T* base) -> int {
+            int64_t is = dsc.stride[o][rank - 1];
+            if (is == 0) return (int)M_BCAST;
+            if (is == 1 && vec_ok<T>(base, dsc, o)) return (int)M_VEC;
+            return (int)M_ELEM;
+        };
+        const int lm = mode(0, l), rm = (OP == kOpCopy) ? (int)M_BCAST : mode(1, r);
+        // Loop dim.  Default: the innermost outer dim, two steps per lane (measured best on MI355X: enough work to
+        // amortise the per-block index arithmetic, short enough that the chip is covered by ~10^5..10^6 small blocks;
+        // a broadcast operand is re-read from L2, which its reuse distance fits).  Exception: an operand that needs
+        // element-wise gathers (inner stride not 0/1) and does not move along some outer dim is fetched once and kept
+        // in registers while the block walks that dim.
+        int gdim = rank >= 2 ? rank - 2 : -1;
+        uint32_t steps = 2;
+        for (int o = 0; o < 2; ++o) {
+            if ((o == 0 ? lm : rm) != M_ELEM) continue;
+            int best = -1;
+            for (int k = 0; k < rank - 1; ++k)
+                if (dsc.stride[o][k] == 0 && (best < 0 || dsc.shape[k] > dsc.shape[best])) best = k;
+            if (best >= 0) { gdim = best; steps = 16; }
+        }
         a.G = gdim >= 0 ? (uint32_t)dsc.shape[gdim] : 1;
         for (int o = 0; o < 3; ++o) a.gstride[o] = gdim >= 0 ? dsc.stride[o][gdim] : 0;
         a.nouter = 0;
@@ -355,29 +343,27 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
         // lanes per row: enough for one vector per lane, at most a block
         uint32_t vecs = (uint32_t)((a.L + N - 1) / N);
         uint32_t tpr = 1;
-        while (tpr < vecs && tpr < (uint32_t)kBlock) tpr <<= 1;
+        while (tpr < vecs && tpr < (uint32_t)kRBlock) tpr <<= 1;
         a.tpr = tpr;
         a.tiles = (vecs + tpr - 1) / tpr;
-        const uint32_t gy = kBlock / tpr;
-        // loop-dim iterations per block: as long as possible (an operand that does not move along the loop dim is
-        // then fetched once per block), shortened until there are enough blocks to fill the chip
-        uint32_t gchunk = a.G;
-        const uint64_t want_blocks = (uint64_t)ctx->num_cus * 8;
-        while (gchunk > gy * kGU && outer * a.tiles * ((a.G + gchunk - 1) / gchunk) < want_blocks) gchunk = (gchunk + 1) / 2;
+        const uint32_t gy = kRBlock / tpr;
+        uint32_t gchunk = gy * steps;
+        if (gchunk > a.G) gchunk = a.G;
         if (gchunk < 1) gchunk = 1;
         a.gchunk = gchunk;
         a.nchunks = (a.G + gchunk - 1) / gchunk;
         a.tiles_div = make_fastdiv(a.tiles);
         a.nchunks_div = make_fastdiv(a.nchunks);
+        // an input is "streamed" when each of its elements is used once: no zero stride over a dim of size > 1
+        a.nt_mask = 0;
+        for (int o = 0; o < 2; ++o) {
+            bool streamed = true;
+            for (int k = 0; k < rank; ++k) streamed = streamed && dsc.stride[o][k] != 0;
+            if (streamed) a.nt_mask |= (1u << o);
+        }
         const uint64_t blocks = outer * a.nchunks * a.tiles;
         if (blocks < (1ull << 31)) {
-            auto mode = [&](int o, const T* base) -> int {
-                int64_t is = dsc.stride[o][rank - 1];
-                if (is == 0) return (int)M_BCAST;
-                if (is == 1 && vec_ok<T>(base, dsc, o)) return (int)M_VEC;
-                return (int)M_ELEM;
-            };
-            launch_rows<T, OP>(mode(0, l), mode(1, r), dim3((unsigned)blocks), s, l + dsc.offset[0], r + dsc.offset[1], d + dsc.offset[2], a);
+            launch_rows<T, OP>(lm, rm, dim3((unsigned)blocks), s, l + dsc.offset[0], r + dsc.offset[1], d + dsc.offset[2], a);
             RT_HIP(hipGetLastError());
             return RT_OK;
         }

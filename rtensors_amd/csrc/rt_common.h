@@ -94,6 +94,24 @@ int32_t rt_collapse(int nops, int rank, const uint64_t* shape, const int64_t* co
 // ---- device helpers ------------------------------------------------------------------------------------------------
 #define RT_WAVE 64
 
+// 16-byte global accesses.  The non-temporal forms mark data that is touched once (streamed operands, outputs):
+// measured on MI355X they lift a read-modify-write pass from ~5.5 to ~6.7 TB/s and a read-only pass from ~5.5 to
+// ~7.0 TB/s, because streamed lines no longer displace each other in L2 / Infinity Cache.
+typedef uint32_t rt_u32x4 __attribute__((ext_vector_type(4)));
+template <class V> __device__ __forceinline__ V rt_ld16(const V* p) {
+    static_assert(sizeof(V) == 16, "16-byte vector expected");
+    return *p;
+}
+template <class V> __device__ __forceinline__ V rt_ld16_nt(const V* p) {
+    static_assert(sizeof(V) == 16, "16-byte vector expected");
+    rt_u32x4 r = __builtin_nontemporal_load(reinterpret_cast<const rt_u32x4*>(p));
+    return __builtin_bit_cast(V, r);
+}
+template <class V> __device__ __forceinline__ void rt_st16_nt(V* p, const V& v) {
+    static_assert(sizeof(V) == 16, "16-byte vector expected");
+    __builtin_nontemporal_store(__builtin_bit_cast(rt_u32x4, v), reinterpret_cast<rt_u32x4*>(p));
+}
+
 // Division of a 32-bit numerator by a runtime-constant divisor via multiply-high (round-up method); exact for
 // every n < 2^31 and 1 <= d < 2^31.
 struct FastDiv32 {

@@ -171,39 +171,23 @@ template <class T> struct FillF {
 template <class T> struct alignas(16) Vec16 { T e[16 / sizeof(T)]; };
 
 constexpr int kBlock = 256;
-constexpr int kUnroll = 4;      // 16-byte accesses in flight per lane
+constexpr int kUnroll = 4;      // 16-byte accesses per lane in the row kernel
+constexpr int kCBlock = 128;    // contiguous kernel: one 16-byte vector per lane, 128 lanes per block
 
-// Body: `nvec` 16-byte vectors starting at the 16-byte aligned address `p`.
+// Body: `nvec` 16-byte vectors starting at the 16-byte aligned address `p`.  One vector per lane and small blocks:
+// on MI355X this shape (with non-temporal accesses for read-modify-write, plain stores for write-only) was the
+// fastest of the block-size / unroll / grid-stride variants tried, ~6.7 TB/s in place and ~6.8 TB/s for fill.
 template <class T, class F>
-__global__ __launch_bounds__(kBlock) void ew_contig_kernel(Vec16<T>* __restrict__ p, size_t nvec, F f) {
+__global__ __launch_bounds__(256) void ew_contig_kernel(Vec16<T>* __restrict__ p, size_t nvec, F f) {
     constexpr int N = 16 / sizeof(T);
-    const size_t base = (size_t)blockIdx.x * (kBlock * kUnroll) + threadIdx.x;
-    Vec16<T> v[kUnroll];
-    if (base + (size_t)(kUnroll - 1) * kBlock < nvec) {       // whole tile inside: no per-access predicate
-        if constexpr (F::kReads) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= nvec) return;
+    Vec16<T> v;
+    if constexpr (F::kReads) v = rt_ld16_nt(p + i);
 #pragma unroll
-            for (int u = 0; u < kUnroll; ++u) v[u] = p[base + (size_t)u * kBlock];
-        }
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-#pragma unroll
-            for (int j = 0; j < N; ++j) v[u].e[j] = f(v[u].e[j]);
-        }
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) p[base + (size_t)u * kBlock] = v[u];
-    } else {
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            const size_t i = base + (size_t)u * kBlock;
-            if (i < nvec) {
-                Vec16<T> w;
-                if constexpr (F::kReads) w = p[i];
-#pragma unroll
-                for (int j = 0; j < N; ++j) w.e[j] = f(w.e[j]);
-                p[i] = w;
-            }
-        }
-    }
+    for (int j = 0; j < N; ++j) v.e[j] = f(v.e[j]);
+    if constexpr (F::kReads) rt_st16_nt(p + i, v);
+    else p[i] = v;
 }
 
 // Edges of a contiguous run that do not fill a 16-byte vector, and 1-D strided views: one element per lane.
@@ -334,9 +318,10 @@ int32_t launch_contig(rt_ctx* ctx, T* p, size_t n, F f) {
     size_t nvec = (n - head) / N;
     size_t tail = n - head - nvec * N;
     if (nvec) {
-        size_t blocks = (nvec + (size_t)kBlock * kUnroll - 1) / ((size_t)kBlock * kUnroll);
+        const size_t bs = F::kReads ? (size_t)kCBlock : (size_t)256;      // pure stores: 256 lanes measured best
+        size_t blocks = (nvec + bs - 1) / bs;
         if (blocks > 0x7fffffffull) return rt_fail(RT_E_INVALID, "contiguous run of %zu elements is too long for one launch", n);
-        hipLaunchKernelGGL((ew_contig_kernel<T, F>), dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream,
+        hipLaunchKernelGGL((ew_contig_kernel<T, F>), dim3((unsigned)blocks), dim3((unsigned)bs), 0, ctx->stream,
                            reinterpret_cast<Vec16<T>*>(p + head), nvec, f);
     }
     if (head) hipLaunchKernelGGL((ew_strided_kernel<T, F>), dim3(1), dim3(kBlock), 0, ctx->stream, p, (int64_t)1, head, f);

@@ -156,7 +156,7 @@ __device__ __forceinline__ void fold_run(Acc<OP, T>& a, const T* __restrict__ p,
     for (; i + (uint64_t)(U - 1) * nthreads < nvec; i += (uint64_t)U * nthreads) {
         Vec16<T> v[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) v[u] = pv[i + (uint64_t)u * nthreads];
+        for (int u = 0; u < U; ++u) v[u] = rt_ld16_nt(pv + i + (uint64_t)u * nthreads);
 #pragma unroll
         for (int u = 0; u < U; ++u) {
 #pragma unroll
@@ -164,7 +164,7 @@ __device__ __forceinline__ void fold_run(Acc<OP, T>& a, const T* __restrict__ p,
         }
     }
     for (; i < nvec; i += nthreads) {
-        Vec16<T> v = pv[i];
+        Vec16<T> v = rt_ld16_nt(pv + i);
 #pragma unroll
         for (uint32_t j = 0; j < N; ++j) a.push(v.e[j], vb + i * N + j);
     }
@@ -224,6 +224,16 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(const T* __restrict
                                                              uint32_t tiles, uint32_t splits, uint64_t seglen, uint64_t count, int last) {
     constexpr int U = 4;
     struct alignas(sizeof(T) * VW) VecW { T e[VW]; };
+    // the source is read exactly once: non-temporal loads
+    auto load = [](const T* q) -> VecW {
+        if constexpr (sizeof(VecW) == 16) {
+            return rt_ld16_nt(reinterpret_cast<const VecW*>(q));
+        } else {
+            VecW w;
+            w.e[0] = __builtin_nontemporal_load(q);
+            return w;
+        }
+    };
     uint64_t b = blockIdx.x;
     const uint32_t tile = (uint32_t)(b % tiles);
     b /= tiles;
@@ -245,7 +255,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(const T* __restrict
         for (; k + (uint64_t)(U - 1) * kWaves < end; k += (uint64_t)U * kWaves) {
             VecW v[U];
 #pragma unroll
-            for (int u = 0; u < U; ++u) v[u] = *reinterpret_cast<const VecW*>(p + (k + (uint64_t)u * kWaves) * inner);
+            for (int u = 0; u < U; ++u) v[u] = load(p + (k + (uint64_t)u * kWaves) * inner);
 #pragma unroll
             for (int u = 0; u < U; ++u) {
 #pragma unroll
@@ -253,7 +263,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(const T* __restrict
             }
         }
         for (; k < end; k += kWaves) {
-            VecW v = *reinterpret_cast<const VecW*>(p + k * inner);
+            VecW v = load(p + k * inner);
 #pragma unroll
             for (int j = 0; j < VW; ++j) a[j].push(v.e[j], k);
         }
