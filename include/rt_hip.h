@@ -61,7 +61,12 @@ typedef enum rt_unary_op {
     RT_U_NEG = 0, RT_U_RELU, RT_U_SIGMOID, RT_U_SILU, RT_U_TANH, RT_U_ABS, RT_U_SQRT, RT_U_LN, RT_U_EXPM1, RT_U_LN1P,
     RT_U_FLOOR, RT_U_CEIL, RT_U_ROUND, RT_U_TRUNC, RT_U_SIN, RT_U_COS, RT_U_TAN, RT_U_ASIN, RT_U_ACOS, RT_U_ATAN,
     RT_U_SINH, RT_U_COSH, RT_U_ASINH, RT_U_ACOSH, RT_U_ATANH, RT_U_RSQRT, RT_U_RECIPROCAL, RT_U_SQUARE, RT_U_CUBE,
-    RT_U_EXP, RT_U_SIGN, RT_U_COUNT
+    RT_U_EXP, RT_U_SIGN, RT_U_COUNT,
+    /* Two maps with no op of their own in the reference: its autograd builds them one element at a time with get/set
+     * (ops/unary/mod.rs:213-252), which on a device backend is one round trip per element. */
+    RT_U_STEP = 31,      /* x > 0 ? 1 : 0   -- the ReLU gradient map (ops/unary/mod.rs:234-252) */
+    RT_U_ABS_GRAD = 32,  /* x > 0 ? 1 : -1  -- the Abs gradient map  (ops/unary/mod.rs:213-232) */
+    RT_U_EXT_COUNT = 33
 } rt_unary_op;
 
 /* ops/reduction/mod.rs:161-175 (codes 6-10 -- variance, logsumexp, norm, argmax, argmin -- are outside this path) */

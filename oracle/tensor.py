@@ -206,3 +206,50 @@ def mean_l1_loss(y: OTensor, target: OTensor):
     n = np.float32(diff.meta.size())                                      # T::from_usize goes through f32
     grad_map = gmap.unary("sign") / cpu.NP_DTYPE[y.dtype].type(n)
     return loss, grad_map
+
+
+def relu_grad_map(inp: OTensor) -> OTensor:
+    """ops/unary/mod.rs:234-252: zeros, then 1 where `input > 0` (the reference does it with one get/set per element)."""
+    vals = inp.to_numpy().reshape(-1)
+    out = np.where(vals > 0, 1, 0).astype(vals.dtype)
+    return OTensor(inp.dtype, out, MetaTensor.row_major(inp.meta.shape))
+
+
+def inverse_broadcast_gradient(grad: OTensor, strides, shape, mode: str) -> OTensor:
+    """grad/backwards.rs:516-538.  mode 'reference_literal' keeps only the *metadata* of `grad.sum_at(dim)` (line 527);
+    mode 'sum' keeps the summed tensor, which is what the function's doc comment describes."""
+    differential = grad.meta.rank() - len(shape)
+    for dim, stride in enumerate(strides):
+        if stride == 0:
+            summed = grad.sum_at(dim)
+            if mode == "sum":
+                grad = summed
+            else:
+                grad = OTensor(grad.dtype, grad.buf, MetaTensor(list(summed.meta.shape), list(summed.meta.strides), summed.meta.offset), grad.is_view)
+    for dim in range(len(strides) - 1, -1, -1):
+        if strides[dim] == 0 and (dim < differential or shape[dim - differential] != 1):
+            sq = grad.squeeze_at(dim)
+            grad = OTensor(grad.dtype, grad.buf, sq.meta, grad.is_view)
+    return grad
+
+
+def train_step(x: OTensor, bias: OTensor, target: OTensor, lr: float, mode: str = "sum", seed_with_loss: bool = True):
+    """One step of y = relu(x + bias), loss = mean_l1_loss(y, target), backward to d(bias), SGD, as the reference's engine
+    sequences it (grad/mod.rs:432-495, grad/backwards.rs:7-42,148-161,229-239, grad/optim.rs:28-50).  `bias` is updated
+    in place; returns (loss, d_bias)."""
+    out_shape, stra, strb = compute_broadcasted_params(x.meta, bias.meta)
+    pre = x + bias                                        # BroadcastAdd node
+    y = pre.owned()
+    gmap_relu = relu_grad_map(pre)                        # ReLU node
+    y.unary_inplace("relu")
+    loss, gmap_l1 = mean_l1_loss(y, target)               # L1 node
+    upstream = loss.owned() if seed_with_loss else OTensor.from_buf(loss.dtype, [1], [])   # grad/mod.rs:442-447
+    d_y = gmap_l1 * upstream                              # backwards_l1
+    d_pre = gmap_relu * d_y                               # backwards_relu
+    d_bias = inverse_broadcast_gradient(d_pre.owned(), strb, bias.meta.shape, mode)       # backwards_add, rhs
+    grad = d_bias.owned() if not d_bias.is_view else d_bias                               # accumulate_grad: first assignment clones
+    grad_values = OTensor(grad.dtype, cpu.gather(grad.dtype, grad.buf, grad.meta), MetaTensor.row_major(grad.meta.shape))
+    update = grad_values * cpu.NP_DTYPE[grad.dtype].type(lr)                               # grad * lr
+    v = bias.view()
+    v -= update
+    return loss, grad_values

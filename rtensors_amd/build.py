@@ -79,5 +79,25 @@ def build(force: bool = False, jobs: int = 8) -> None:
             print(f"[build] linked {lib}", file=sys.stderr)
 
 
+    _build_host(force)
+
+
+def _build_host(force: bool) -> None:
+    """librt_host.so: the C++ host layer.  Built with g++ against include/rt_hip.h only (no HIP headers) and linked to
+    librt_hip.so, the way a foreign-language binding would use the C ABI."""
+    host = os.path.join(HERE, "host")
+    src = os.path.join(host, "rt_host_capi.cpp")
+    out = os.path.join(LIB, "librt_host.so")
+    deps = [src] + [os.path.join(host, h) for h in ("rt_meta.hpp", "rt_backend.hpp", "rt_tensor.hpp", "rt_grad.hpp")] + HEADERS[1:]
+    if force or _stale(out, deps + [os.path.join(LIB, "librt_hip.so")]):
+        cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra", "-o", out, src, "-L" + LIB, "-lrt_hip", "-Wl,-rpath,$ORIGIN"]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"g++ failed on the host layer:\n{r.stdout + r.stderr}")
+        if (r.stdout + r.stderr).strip():
+            print((r.stdout + r.stderr).strip(), file=sys.stderr)
+        print("[build] linked librt_host.so", file=sys.stderr)
+
+
 if __name__ == "__main__":
     build(force="--force" in sys.argv)

@@ -107,6 +107,11 @@ template <int OP, class T> struct UnaryF {
             if constexpr (is_flt<T>::value) return m_abs(x);
             else if constexpr (is_sint<T>::value) return x < 0 ? w_sub<T>((T)0, x) : x;
             else return x;
+        } else if constexpr (OP == RT_U_STEP) {                           // ops/unary/mod.rs:234-252
+            if constexpr (is_bool<T>::value) return x;
+            else return gt0(x) ? (T)1 : (T)0;
+        } else if constexpr (OP == RT_U_ABS_GRAD) {                       // ops/unary/mod.rs:213-232
+            return gt0(x) ? (T)1 : (T)-1;
         } else if constexpr (OP == RT_U_NEG) {                            // cpu.rs:644-647
             if constexpr (is_flt<T>::value) return -x;
             else return w_sub<T>(zero_of<T>(), x);
@@ -443,7 +448,7 @@ int32_t unary_float(rt_ctx* ctx, int op, void* buf, uint64_t buf_len, uint64_t o
         RT_UCASE(RT_U_ROUND); RT_UCASE(RT_U_TRUNC); RT_UCASE(RT_U_SIN); RT_UCASE(RT_U_COS); RT_UCASE(RT_U_TAN); RT_UCASE(RT_U_ASIN);
         RT_UCASE(RT_U_ACOS); RT_UCASE(RT_U_ATAN); RT_UCASE(RT_U_SINH); RT_UCASE(RT_U_COSH); RT_UCASE(RT_U_ASINH); RT_UCASE(RT_U_ACOSH);
         RT_UCASE(RT_U_ATANH); RT_UCASE(RT_U_RSQRT); RT_UCASE(RT_U_RECIPROCAL); RT_UCASE(RT_U_SQUARE); RT_UCASE(RT_U_CUBE);
-        RT_UCASE(RT_U_EXP); RT_UCASE(RT_U_SIGN);
+        RT_UCASE(RT_U_EXP); RT_UCASE(RT_U_SIGN); RT_UCASE(RT_U_STEP); RT_UCASE(RT_U_ABS_GRAD);
     }
 #undef RT_UCASE
     return rt_fail(RT_E_INVALID, "unary: unknown op code %d", op);
@@ -452,11 +457,13 @@ int32_t unary_float(rt_ctx* ctx, int op, void* buf, uint64_t buf_len, uint64_t o
 // Non-float dtypes: relu and abs for every dtype, neg for the signed ones (trait bounds, backend/mod.rs:311-355).
 template <class T>
 int32_t unary_other(rt_ctx* ctx, int op, void* buf, uint64_t buf_len, uint64_t offset, int rank, const uint64_t* shape, const int64_t* strides) {
-    if (op < 0 || op >= RT_U_COUNT) return rt_fail(RT_E_INVALID, "unary: unknown op code %d", op);
+    if (op < 0 || op >= RT_U_EXT_COUNT) return rt_fail(RT_E_INVALID, "unary: unknown op code %d", op);
     if (op == RT_U_RELU) return unary_go<T, RT_U_RELU>(ctx, buf, buf_len, offset, rank, shape, strides);
+    if (op == RT_U_STEP) return unary_go<T, RT_U_STEP>(ctx, buf, buf_len, offset, rank, shape, strides);
     if (op == RT_U_ABS) return unary_go<T, RT_U_ABS>(ctx, buf, buf_len, offset, rank, shape, strides);
     if constexpr (is_sint<T>::value) {
         if (op == RT_U_NEG) return unary_go<T, RT_U_NEG>(ctx, buf, buf_len, offset, rank, shape, strides);
+        if (op == RT_U_ABS_GRAD) return unary_go<T, RT_U_ABS_GRAD>(ctx, buf, buf_len, offset, rank, shape, strides);
     }
     return rt_fail(RT_E_DTYPE, "unary op %d is not defined for this dtype (the reference bounds it on f32/f64)", op);
 }

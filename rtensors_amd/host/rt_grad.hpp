@@ -1,0 +1,219 @@
+// Reverse-mode tape for the broadcast/reduce training step (no matmul): y = relu(x + bias), loss = mean_l1_loss(y, t),
+// backward to d(bias), SGD update.  Follows the reference's engine: grad/mod.rs:269-308 (context, attach), 432-495
+// (backwards: toposort, upstream accumulation), grad/backwards.rs:7-42, 148-161, 229-239, 516-538 (node rules),
+// ops/broadcast/l1.rs:16-84 (L1 loss and its gradient map), ops/unary/mod.rs:234-252 (ReLU gradient map),
+// grad/optim.rs:28-50 (SGD).  Every arithmetic step is a backend call issued through rt::Tensor.
+#pragma once
+
+#include <map>
+#include <memory>
+#include <set>
+#include <vector>
+
+#include "rt_tensor.hpp"
+
+namespace rt {
+namespace grad {
+
+// How `inverse_broadcast_gradient` treats a broadcast dim.
+//   Sum              : d(operand) = sum of the upstream gradient over the dim (what the function's own doc comment and
+//                      the maths say).
+//   ReferenceLiteral : what grad/backwards.rs:527 executes -- `grad.meta = grad.sum_at(dim)?.meta`: the sum is computed,
+//                      its buffer dropped, and only its metadata kept, so the stored gradient is the first slice of the
+//                      upstream buffer.  Kept so the divergence can be shown in a test.
+enum class BroadcastGradMode { Sum, ReferenceLiteral };
+
+enum class NodeKind { None, Leaf, BroadcastAdd, BroadcastSub, ReLU, L1 };
+
+struct Node {
+    NodeKind kind = NodeKind::None;
+    std::vector<int> parents;            // -1 = no gradient flows there (GradNode::None sentinel)
+    Strides lhs_strides, rhs_strides;    // BroadcastAdd / BroadcastSub
+    Shape lhs_shape, rhs_shape;
+    Tensor grad_map;                     // ReLU, L1
+    Tensor loss;                         // L1
+    std::shared_ptr<Tensor> grad;        // Leaf: accumulated gradient (null until the first backward pass)
+};
+
+struct Var {
+    Tensor t;
+    int node = -1;
+};
+
+class GradContext {
+  public:
+    BroadcastGradMode mode = BroadcastGradMode::Sum;
+    bool seed_with_loss = true;   // grad/mod.rs:442-447 seeds the root with the loss tensor itself, not with 1
+
+    Var input(const Tensor& t) { return Var{t, -1}; }
+    Var param(const Tensor& t) {                        // TensorBase::param + GradNode::Leaf
+        Node n;
+        n.kind = NodeKind::Leaf;
+        nodes_.push_back(n);
+        return Var{t, (int)nodes_.size() - 1};
+    }
+
+    // ops/broadcast/add.rs:173-208 + attach_broadcast_add_grad (586-607)
+    Var add(const Var& a, const Var& b) { return broadcast(a, b, BinaryOpType::Add, NodeKind::BroadcastAdd); }
+    Var sub(const Var& a, const Var& b) { return broadcast(a, b, BinaryOpType::Sub, NodeKind::BroadcastSub); }
+
+    // ops/unary/mod.rs:114-126 (relu = owned + relu_inplace) with the gradient map of 234-252: 1 where input > 0
+    Var relu(const Var& a) {
+        Tensor result = a.t.owned();
+        Tensor gmap;
+        const bool track = a.node >= 0;
+        if (track) gmap = result.owned();
+        result.relu_inplace();
+        if (!track) return Var{result, -1};
+        gmap.unary_inplace(RT_U_STEP);
+        Node n;
+        n.kind = NodeKind::ReLU;
+        n.parents = {a.node};
+        n.grad_map = gmap;
+        nodes_.push_back(n);
+        return Var{result, (int)nodes_.size() - 1};
+    }
+
+    // ops/broadcast/l1.rs:49-84 with ReductionType::Mean
+    Var mean_l1_loss(const Var& y, const Var& target) {
+        Tensor diff = y.t - target.t;
+        Tensor gmap = diff.sign();
+        diff.abs_inplace();
+        Tensor loss = diff.mean();
+        // attach_l1_grad (l1.rs:16-46): grad_map = sign(gmap) / T::from_usize(N), from_usize going through f32
+        Tensor grad_map = gmap.sign() / (double)(float)diff.size();
+        Node n;
+        n.kind = NodeKind::L1;
+        n.parents = {y.node, target.node};
+        n.grad_map = grad_map;
+        n.loss = loss;
+        nodes_.push_back(n);
+        return Var{loss, (int)nodes_.size() - 1};
+    }
+
+    // grad/mod.rs:432-495
+    void backwards(const Var& root) {
+        if (root.node < 0 || nodes_[(size_t)root.node].kind != NodeKind::L1)
+            throw TensorError(ErrorKind::GradError, "Root node does not contain a loss.");
+        std::vector<int> order;
+        std::set<int> seen;
+        toposort(root.node, seen, order);
+        std::map<int, std::vector<Tensor>> acc;
+        const Tensor& loss = nodes_[(size_t)root.node].loss;
+        acc[root.node].push_back(seed_with_loss ? loss.owned() : Tensor::ones(loss.backend(), loss.dtype(), loss.shape()));
+        for (size_t i = order.size(); i-- > 0;) {
+            const int key = order[i];
+            std::vector<Tensor>& ups = acc[key];
+            if (ups.empty()) continue;
+            Tensor dldy = ups[0];
+            for (size_t k = 1; k < ups.size(); ++k) dldy = dldy + ups[k];
+            Node& n = nodes_[(size_t)key];
+            std::vector<Tensor> down = node_backwards(n, dldy);
+            for (size_t p = 0; p < n.parents.size() && p < down.size(); ++p)
+                if (n.parents[p] >= 0) acc[n.parents[p]].push_back(down[p]);
+            acc.erase(key);
+        }
+    }
+
+    std::shared_ptr<Tensor> grad_of(const Var& v) const { return v.node >= 0 ? nodes_[(size_t)v.node].grad : nullptr; }
+    void clear_grad(const Var& v) { if (v.node >= 0) nodes_[(size_t)v.node].grad.reset(); }
+
+  private:
+    Var broadcast(const Var& a, const Var& b, BinaryOpType op, NodeKind kind) {
+        Tensor result = a.t.binary(b.t, op);
+        if (a.node < 0 && b.node < 0) return Var{result, -1};
+        BroadcastParams p = compute_broadcasted_params(a.t.meta(), b.t.meta());
+        Node n;
+        n.kind = kind;
+        n.parents = {a.node, b.node};
+        n.lhs_strides = p.a;
+        n.rhs_strides = p.b;
+        n.lhs_shape = a.t.shape();
+        n.rhs_shape = b.t.shape();
+        nodes_.push_back(n);
+        return Var{result, (int)nodes_.size() - 1};
+    }
+
+    void toposort(int key, std::set<int>& seen, std::vector<int>& order) {
+        if (key < 0 || seen.count(key)) return;
+        seen.insert(key);
+        for (int p : nodes_[(size_t)key].parents) toposort(p, seen, order);
+        order.push_back(key);
+    }
+
+    // grad/backwards.rs:516-538
+    void inverse_broadcast_gradient(Tensor& g, const Strides& strides, const Shape& shape) const {
+        const size_t differential = g.rank() - shape.size();
+        for (size_t dim = 0; dim < strides.size(); ++dim) {
+            if (strides[dim] != 0) continue;
+            Tensor summed = g.sum_at(dim);
+            if (mode == BroadcastGradMode::Sum) g = summed;
+            else g.set_meta(summed.meta());
+        }
+        for (size_t dim = strides.size(); dim-- > 0;) {
+            if (strides[dim] == 0 && (dim < differential || shape[dim - differential] != 1)) {
+                Tensor sq = g.squeeze_at(dim);
+                g.set_meta(sq.meta());
+            }
+        }
+    }
+
+    std::vector<Tensor> node_backwards(Node& n, const Tensor& up) {
+        switch (n.kind) {
+            case NodeKind::Leaf:                                         // accumulate_grad, backwards.rs:7-25
+                if (n.grad) *n.grad += up;
+                else n.grad = std::make_shared<Tensor>(up.owned());
+                return {};
+            case NodeKind::L1: {                                         // backwards_l1, backwards.rs:148-161
+                std::vector<Tensor> out(2);
+                if (n.parents[0] >= 0) out[0] = n.grad_map * up;
+                if (n.parents[1] >= 0) out[1] = (-n.grad_map) * up;
+                return out;
+            }
+            case NodeKind::ReLU:                                         // backwards_relu, backwards.rs:229-239
+                return {n.grad_map * up};
+            case NodeKind::BroadcastAdd:                                 // backwards_add / backwards_sub, backwards.rs:27-60
+            case NodeKind::BroadcastSub: {
+                std::vector<Tensor> out(2);
+                if (n.parents[0] >= 0) { out[0] = up.owned(); inverse_broadcast_gradient(out[0], n.lhs_strides, n.lhs_shape); }
+                if (n.parents[1] >= 0) {
+                    out[1] = n.kind == NodeKind::BroadcastSub ? -up : up.owned();
+                    inverse_broadcast_gradient(out[1], n.rhs_strides, n.rhs_shape);
+                }
+                return out;
+            }
+            default:
+                return {};
+        }
+    }
+
+    std::vector<Node> nodes_;
+};
+
+// grad/optim.rs:14-50
+class SGD {
+  public:
+    explicit SGD(double learning_rate) : lr_(learning_rate) {}
+    void register_parameter(GradContext& ctx, Var& param) {
+        if (param.node < 0) throw TensorError(ErrorKind::GradError, "Only leaf tensors can be registered as parameters.");
+        ctx_ = &ctx;
+        params_.push_back(&param);
+    }
+    void step() {
+        for (Var* p : params_) {
+            std::shared_ptr<Tensor> g = ctx_->grad_of(*p);
+            if (!g) continue;
+            Tensor update = *g * lr_;           // grad * lr: owned copy + in-place scalar mul, rounded to T
+            ctx_->clear_grad(*p);
+            Tensor v = p->t.view();
+            v -= update;                        // in-place broadcast sub through a mutable view
+        }
+    }
+  private:
+    double lr_;
+    GradContext* ctx_ = nullptr;
+    std::vector<Var*> params_;
+};
+
+}  // namespace grad
+}  // namespace rt

@@ -1,0 +1,306 @@
+"""The C++ host layer (tensors, views, operators, reductions, autograd step) on the GPU against the oracle, and the
+BASELINE configurations at their full sizes through size-independent properties."""
+import numpy as np
+import pytest
+
+import golden_dsl
+from oracle import cpu
+from oracle.meta import Slice as OSlice, TensorError as OErr
+from oracle.tensor import OTensor, train_step as oracle_train_step
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def T():
+    from rtensors_amd import tensor
+    return tensor
+
+
+@pytest.fixture(scope="module")
+def be(T):
+    return T.Backend(0)
+
+
+CASES = golden_dsl.load("reference_vectors.json") + golden_dsl.load("reference_meta_vectors.json")
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: c["name"])
+def test_reference_vectors_through_host_layer(T, be, case):
+    def slice_cls(start, end, step):
+        return T.Slice(start, end, step)
+    slice_cls.range = T.Slice.range
+    slice_cls.range_inclusive = T.Slice.range_inclusive
+    slice_cls.index = T.Slice.index
+    env, err = golden_dsl.run_case(case, lambda dt, v, s: T.Tensor.from_buf(be, dt, v, s), slice_cls, T.TensorError)
+    for exp in case["expect"]:
+        exp.pop("path", None)
+
+    def meta_of(t):
+        i = t._info()
+        return i["shape"], i["strides"], i["offset"], i["contiguous"]
+    golden_dsl.check_case(case, env, err, lambda t: t.to_numpy(), lambda t, idx: t.get(idx), meta_of)
+
+
+def rand_values(dtype, n, rng):
+    npd = cpu.NP_DTYPE[cpu.DTYPE_BY_NAME[dtype]]
+    if npd.kind == "f":
+        return rng.standard_normal(n).astype(npd)
+    return rng.integers(-100, 100, size=n).astype(npd)
+
+
+def test_random_programs_match_oracle(T, be):
+    rng = np.random.default_rng(21)
+    for trial in range(60):
+        dtype = ["f32", "f64", "i32", "i64"][trial % 4]
+        rank = int(rng.integers(1, 5))
+        shape = [int(rng.integers(1, 9)) for _ in range(rank)]
+        sb = [d if rng.random() < 0.6 else 1 for d in shape][int(rng.integers(0, rank)):]
+        va, vb = rand_values(dtype, int(np.prod(shape)), rng), rand_values(dtype, int(np.prod(sb)), rng)
+        o, g = OTensor.from_buf(dtype, va, shape), T.Tensor.from_buf(be, dtype, va, shape)
+        ob, gb = OTensor.from_buf(dtype, vb, sb), T.Tensor.from_buf(be, dtype, vb, sb)
+        ov, gv = o, g
+        for _ in range(int(rng.integers(0, 3))):
+            r = len(ov.meta.shape)
+            d = int(rng.integers(0, r))
+            k = int(rng.integers(0, 3))
+            if k == 0 and ov.meta.strides[d] > 0 and ov.meta.shape[d] > 1:
+                step = int(rng.choice([1, 2, -1]))
+                ov, gv = ov.slice(d, OSlice(None, None, step)), gv.slice(d, T.Slice(None, None, step))
+            elif k == 1 and r > 1:
+                p = [int(v) for v in rng.permutation(r)]
+                ov, gv = ov.permute(p), gv.permute(p)
+            else:
+                ov, gv = ov.unsqueeze_at(d), gv.unsqueeze_at(d)
+        try:
+            want = ((ov + ob) * 3 - ob).unary("relu")
+        except OErr:
+            continue
+        got = ((gv + gb) * 3 - gb).unary("relu")
+        assert got.shape == want.meta.shape
+        assert got.to_numpy().tobytes() == want.to_numpy().tobytes(), (trial, dtype, ov.meta, sb)
+        if ov.meta.shape == want.meta.shape and not (ov.meta.is_contiguous() and any(s < 0 for s in ov.meta.strides)):
+            ov -= ob; gv -= gb
+            ov.unary_inplace("abs"); gv.unary_inplace("abs")
+            assert g.dump_buffer().tobytes() == o.buf.tobytes()
+        if want.meta.rank() and dtype in ("i32", "i64"):
+            for ax in range(want.meta.rank()):
+                assert got.sum_at(ax).to_numpy().tobytes() == want.sum_at(ax).to_numpy().tobytes()
+            assert got.max().to_numpy().tobytes() == want.max().to_numpy().tobytes()
+
+
+def test_reduce_of_noncontiguous_and_reversed_views(T, be):
+    x = np.arange(24, dtype=np.float64) * 0.5 - 3
+    o, g = OTensor.from_buf("f64", x, [2, 3, 4]), T.Tensor.from_buf(be, "f64", x, [2, 3, 4])
+    assert np.array_equal(g.transpose().sum_at(0).to_numpy(), o.transpose().sum_at(0).to_numpy())
+    assert np.array_equal(g.permute([1, 2, 0]).max_at(1).to_numpy(), o.permute([1, 2, 0]).max_at(1).to_numpy())
+    # a reversed view is |stride|-contiguous; the reference then reduces from the wrong offset (Cpu: ignores it).  Here it
+    # is gathered first, so the result is the reduction of the viewed values.
+    rv = g.slice(0, T.Slice(None, None, -1))
+    assert np.array_equal(rv.sum_at(2).to_numpy().reshape(2, 3), x.reshape(2, 3, 4)[::-1].sum(axis=2))
+
+
+def test_out_of_scope_methods_report_unsupported(T, be):
+    g = T.Tensor.from_buf(be, "f32", np.ones(4, np.float32), [4])
+    with pytest.raises(T.TensorError) as e:
+        g._new(T._h.rth_reduce, 6, T.C.c_int64(-1))           # variance
+    assert e.value.kind == "UnsupportedOperation"
+
+
+# ---- autograd step (config 5 at reduced size) ---------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["f32", "f64"])
+@pytest.mark.parametrize("mode", ["sum", "reference_literal"])
+@pytest.mark.parametrize("seed_with_loss", [True, False])
+def test_train_step_matches_oracle(T, be, dtype, mode, seed_with_loss):
+    from rtensors_amd import datagen
+    npd = cpu.NP_DTYPE[cpu.DTYPE_BY_NAME[dtype]]
+    n, d = 384, 96
+    x = datagen.normal(npd, n * d, 4, 0)
+    bias = datagen.normal(npd, d, 4, 1, 0.1)
+    target = datagen.uniform(npd, n * d, 4, 2)
+    ox, ob, ot = OTensor.from_buf(dtype, x, [n, d]), OTensor.from_buf(dtype, bias, [d]), OTensor.from_buf(dtype, target, [n, d])
+    gx, gb, gt = T.Tensor.from_buf(be, dtype, x, [n, d]), T.Tensor.from_buf(be, dtype, bias, [d]), T.Tensor.from_buf(be, dtype, target, [n, d])
+    oloss, ograd = oracle_train_step(ox, ob, ot, 0.01, mode, seed_with_loss)
+    gloss, ggrad = T.train_step(gx, gb, gt, 0.01, mode, seed_with_loss)
+    tol = (1e-5 if dtype == "f32" else 1e-12)
+    # loss = mean |y - t|: a float reduction, within rel tol of sum|x|/N
+    absdiff_sum = float(np.abs(np.maximum(x.reshape(n, d).astype(np.float64) + bias, 0) - target.reshape(n, d)).sum())
+    assert abs(float(gloss.to_numpy()) - float(oloss.buf[0])) <= tol * absdiff_sum / (n * d) + 1e-30
+    assert ggrad.shape == ograd.meta.shape == [d]
+    # d(bias): elementwise maps are bit-exact; the column sum is a float reduction (tolerance relative to sum|g|)
+    scale = abs(float(oloss.buf[0])) if seed_with_loss else 1.0
+    gtol = tol * scale * n / (n * d) * 4 + 1e-30 if mode == "sum" else 1e-6 * scale
+    assert np.max(np.abs(ggrad.to_numpy().astype(np.float64) - ograd.buf.astype(np.float64))) <= gtol
+    assert np.max(np.abs(gb.to_numpy().astype(np.float64) - ob.buf.astype(np.float64))) <= 0.01 * gtol + np.finfo(npd).eps
+    if mode == "sum" and not seed_with_loss:
+        # closed form: d(bias)[j] = (1/N) * sum_i [x_ij + b_j > 0] * sign(y_ij - t_ij),  N = n*d
+        pre = (x.reshape(n, d) + bias.astype(npd)).astype(npd)
+        y = np.maximum(pre, 0)
+        closed = ((pre > 0) * np.sign((y - target.reshape(n, d)).astype(npd))).astype(np.float64).sum(axis=0) / (n * d)
+        assert np.max(np.abs(ggrad.to_numpy() - closed)) < 1e-6
+    if mode == "reference_literal":
+        # the literal engine keeps row 0 of the upstream gradient instead of the batch sum
+        ob2 = OTensor.from_buf(dtype, bias, [d])
+        _, gsum = oracle_train_step(OTensor.from_buf(dtype, x, [n, d]), ob2, OTensor.from_buf(dtype, target, [n, d]), 0.01, "sum", seed_with_loss)
+        assert not np.allclose(gsum.buf, ograd.buf)
+
+
+# ---- BASELINE configurations at full size ---------------------------------------------------------------------------------------
+def test_config1_full_vs_oracle(be, T):
+    from rtensors_amd import datagen
+    n = 4096
+    for dtype in ("f32", "i32"):
+        if dtype == "f32":
+            a, b = datagen.uniform(np.float32, n, 0, 0), datagen.uniform(np.float32, n, 0, 1)
+        else:
+            a, b = datagen.integers(n, 0, 2, -1000, 1000), datagen.integers(n, 0, 3, -1000, 1000)
+        oc = OTensor.from_buf(dtype, a, [1, n]) + OTensor.from_buf(dtype, b, [n, 1])
+        gc = T.Tensor.from_buf(be, dtype, a, [1, n]) + T.Tensor.from_buf(be, dtype, b, [n, 1])
+        assert gc.shape == [n, n] and gc.to_numpy().tobytes() == oc.buf.tobytes()
+        os_, gs = oc.sum_at(1), gc.sum_at(1)
+        assert gs.shape == [n, 1]
+        if dtype == "i32":
+            assert gs.to_numpy().tobytes() == os_.buf.tobytes()
+            assert np.array_equal(gs.to_numpy().reshape(-1).astype(np.int64), a.astype(np.int64).sum() + n * b.astype(np.int64))   # closed form
+        else:
+            tol = 1e-5 * np.abs(oc.buf.astype(np.float64)).reshape(n, n).sum(axis=1)
+            assert np.all(np.abs(gs.to_numpy().reshape(-1).astype(np.float64) - os_.buf.astype(np.float64)) <= tol)
+
+
+def test_config2_chain_full_size(be, T):
+    """c = relu(a * 3 + b); c -= 1 at 2^28 f32 (2^27 f64, 2^28 i32): a strided sample of the result is compared with the
+    same chain in numpy (each step is one IEEE / wrapping operation, so the comparison is bit-exact)."""
+    from rtensors_amd import datagen
+    for dtype, n in (("f32", 1 << 28), ("f64", 1 << 27), ("i32", 1 << 28)):
+        npd = cpu.NP_DTYPE[cpu.DTYPE_BY_NAME[dtype]]
+        chunk = 1 << 22
+        def gen(stream, start, m):
+            if dtype == "i32":
+                return datagen.integers(m, 1, stream, -(1 << 20), 1 << 20, start)
+            return datagen.normal(npd, m, 1, stream, 1.0, start)
+        # only the sampled windows are generated on the host; the device tensors come from the device generator
+        from rtensors_amd import hip as H
+        hb = H.Hip.new(0)
+        code = H.DTYPE_BY_NAME[dtype]
+        da, db = hb.alloc_uninit(code, n), hb.alloc_uninit(code, n)
+        if dtype == "i32":
+            datagen.fill_device(da, "int", 1, 0, -(1 << 20), 1 << 20); datagen.fill_device(db, "int", 1, 1, -(1 << 20), 1 << 20)
+        else:
+            datagen.fill_device(da, "normal", 1, 0); datagen.fill_device(db, "normal", 1, 1)
+        three, one = (3, 1) if dtype == "i32" else (3.0, 1.0)
+        t = hb.copy(da)                                   # `a * 3.0` = owned() + in-place mul
+        hb.scalar_contiguous("mul", t, three, 0, n)
+        u = hb.alloc_uninit(code, n)
+        m = (0, [n], [1])
+        hb.broadcast((t, m), (db, m), (u, m), "add")
+        c = hb.copy(u)                                    # `.relu()` = owned() + in-place relu
+        hb.unary_contiguous("relu", c, 0, n)
+        hb.scalar_contiguous("sub", c, one, 0, n)
+        for start in (0, 12345 * 4, n // 2 + 3, n - chunk):
+            tmp = hb.alloc_uninit(code, chunk)
+            hb.copy_range_within(tmp, c, 0, start, chunk)
+            got = hb.dump(tmp)
+            ha, hbv = gen(0, start, chunk), gen(1, start, chunk)
+            with np.errstate(over="ignore"):
+                want = (np.maximum((ha * npd.type(three)).astype(npd) + hbv, 0).astype(npd) - npd.type(one)).astype(npd)
+            assert got.tobytes() == want.tobytes(), (dtype, start)
+        del da, db, t, u, c
+        hb.sync()
+
+
+def test_config3_both_variants_agree_and_match_formula(be, T):
+    """z = x + y -> (16,64,512,1024) with x contiguous, and with x given as the permuted / reversed / unsqueezed view of a
+    (16,1024,512) tensor holding the same values: both must produce the same 2 GiB, checked on sampled rows against
+    numpy, and checked equal to each other in full on the device."""
+    from rtensors_amd import datagen, hip as H
+    hb = H.Hip.new(0)
+    B, J, K, L = 16, 64, 512, 1024
+    x = datagen.normal(np.float32, B * K * L, 2, 0).reshape(B, K, L)
+    y = datagen.uniform(np.float32, J * L, 2, 1).reshape(J, L)
+    gx = hb.alloc_from_slice(H.F32, x.reshape(-1))
+    gy = hb.alloc_from_slice(H.F32, y.reshape(-1))
+    shape = [B, J, K, L]
+    zs = [J * K * L, K * L, L, 1]
+    z1 = hb.alloc_uninit(H.F32, B * J * K * L)
+    hb.broadcast((gx, (0, shape, [K * L, 0, L, 1])), (gy, (0, shape, [0, L, 0, 1])), (z1, (0, shape, zs)), "add")
+    # variant b: base[b, l, K-1-k] = x[b, k, l]; view = base.permute([0,2,1]).slice(1, step -1).unsqueeze_at(1)
+    base = np.ascontiguousarray(np.transpose(x, (0, 2, 1))[:, :, ::-1])
+    gbase = hb.alloc_from_slice(H.F32, base.reshape(-1))
+    from oracle.meta import MetaTensor                                # metadata only: derive the view's layout with the oracle rules
+    mv = OTensor(cpu.F32, np.zeros(1, np.float32), MetaTensor.row_major([B, L, K])).permute([0, 2, 1]).slice(1, OSlice(None, None, -1)).unsqueeze_at(1)
+    assert mv.meta.shape == [B, 1, K, L] and mv.meta.strides == [K * L, -K, -1, K] and mv.meta.offset == K - 1
+    z2 = hb.alloc_uninit(H.F32, B * J * K * L)
+    hb.broadcast((gbase, (mv.meta.offset, shape, [K * L, 0, -1, K])), (gy, (0, shape, [0, L, 0, 1])), (z2, (0, shape, zs)), "add")
+    assert z1 == z2                                                   # device-side equality over all 2^29 elements
+    rng = np.random.default_rng(0)
+    for _ in range(64):
+        b, j, k = int(rng.integers(0, B)), int(rng.integers(0, J)), int(rng.integers(0, K))
+        row = hb.alloc_uninit(H.F32, L)
+        hb.copy_range_within(row, z1, 0, ((b * J + j) * K + k) * L, L)
+        assert hb.dump(row).tobytes() == (x[b, k] + y[j]).tobytes()
+    hb.sync()
+
+
+def test_config4_full_size_reductions(be, T):
+    from rtensors_amd import datagen, hip as H
+    hb = H.Hip.new(0)
+    R, Cc = 8192, 32768
+    t = hb.alloc_uninit(H.F32, R * Cc)
+    datagen.fill_device(t, "normal", 3, 0)
+    host = hb.dump(t).reshape(R, Cc)
+    h64 = host.astype(np.float64)
+    meta = (0, [R, Cc], [Cc, 1])
+    def run(op, dim, n_out):
+        out = hb.alloc(H.F32, n_out)
+        hb.apply_reduce_contiguous_nd((t, meta), out, dim, op)
+        return hb.dump(out)
+    rows_abs = np.abs(h64).sum(axis=1); cols_abs = np.abs(h64).sum(axis=0)
+    assert np.all(np.abs(run("sum", 1, R) - h64.sum(axis=1)) <= 1e-5 * rows_abs)
+    assert np.all(np.abs(run("mean", 1, R) - h64.mean(axis=1)) <= 1e-5 * rows_abs / Cc + 1e-12)
+    assert run("max", 1, R).tobytes() == host.max(axis=1).tobytes()
+    assert np.all(np.abs(run("sum", 0, Cc) - h64.sum(axis=0)) <= 1e-5 * cols_abs)
+    out = hb.alloc(H.F32, 1)
+    hb.apply_reduce_contiguous_flat(t, out, 0, R * Cc, "sum")
+    assert abs(float(hb.dump(out)[0]) - h64.sum()) <= 1e-5 * np.abs(h64).sum()
+    # a checksum of checksums: summing the row sums equals summing the column sums equals the full sum, within tolerance
+    assert abs(run("sum", 1, R).astype(np.float64).sum() - run("sum", 0, Cc).astype(np.float64).sum()) <= 2e-5 * np.abs(h64).sum()
+    del host, h64
+    ti = hb.alloc_uninit(H.I32, R * Cc)
+    datagen.fill_device(ti, "int", 3, 1, -1000, 1000)
+    hi = hb.dump(ti).reshape(R, Cc)
+    def runi(op, dim, n_out):
+        out = hb.alloc(H.I32, n_out)
+        hb.apply_reduce_contiguous_nd((ti, meta), out, dim, op)
+        return hb.dump(out)
+    assert np.array_equal(runi("sum", 1, R), hi.sum(axis=1, dtype=np.int64).astype(np.int32))
+    assert np.array_equal(runi("sum", 0, Cc), hi.sum(axis=0, dtype=np.int64).astype(np.int32))
+    assert np.array_equal(runi("max", 1, R), hi.max(axis=1)) and np.array_equal(runi("min", 0, Cc), hi.min(axis=0))
+    assert np.array_equal(runi("min", 1, R), hi.min(axis=1)) and np.array_equal(runi("max", 0, Cc), hi.max(axis=0))
+    hb.sync()
+
+
+def test_config5_full_size_step(be, T):
+    """x (65536,4096), bias (4096,), target (65536,4096), lr 0.01: d(bias) against the closed form evaluated in numpy."""
+    from rtensors_amd import datagen
+    n, d = 65536, 4096
+    x = datagen.normal(np.float32, n * d, 4, 0)
+    bias = datagen.normal(np.float32, d, 4, 1, 0.1)
+    target = datagen.uniform(np.float32, n * d, 4, 2)
+    gx, gb, gt = T.Tensor.from_buf(be, "f32", x, [n, d]), T.Tensor.from_buf(be, "f32", bias, [d]), T.Tensor.from_buf(be, "f32", target, [n, d])
+    gloss, ggrad = T.train_step(gx, gb, gt, 0.01, "sum", True)
+    pre = x.reshape(n, d) + bias
+    y = np.maximum(pre, 0)
+    diff = y - target.reshape(n, d)
+    loss = np.abs(diff.astype(np.float64)).mean()
+    got_loss = float(gloss.to_numpy())
+    assert abs(got_loss - loss) <= 1e-5 * loss
+    N = np.float32(np.float32(n * d))
+    gm = (np.sign(diff) / N).astype(np.float32)                       # sign(sign(d)) / N
+    up = (gm * np.float32(got_loss)).astype(np.float32) * (pre > 0)   # L1 backward seeded with the loss, then ReLU backward
+    closed = up.astype(np.float64).sum(axis=0)
+    tol = 1e-5 * np.abs(up.astype(np.float64)).sum(axis=0) + 1e-30
+    g = ggrad.to_numpy().astype(np.float64)
+    assert np.all(np.abs(g - closed) <= tol)
+    new_bias = gb.to_numpy()
+    want_bias = bias - (ggrad.to_numpy() * np.float32(0.01)).astype(np.float32)
+    assert new_bias.tobytes() == want_bias.astype(np.float32).tobytes()
