@@ -117,7 +117,7 @@ __device__ __forceinline__ Vec16<T> load_vec(const T* __restrict__ rowp, uint32_
     return v;
 }
 
-template <class T, int OP, int LM, int RM>
+template <class T, int OP, int LM, int RM, int GU>
 __global__ __launch_bounds__(kRBlock) void bin_rows_kernel(const T* l, const T* r, T* d, RowArgs a) {
     constexpr int N = 16 / sizeof(T);
     // blockIdx -> (outer index, chunk of the loop dim, column tile); all uniform, computed on the scalar unit
@@ -154,14 +154,50 @@ __global__ __launch_bounds__(kRBlock) void bin_rows_kernel(const T* l, const T* 
         Vec16<T> lh, rh;                                        // operands that do not move along the loop dim
         if (l_fixed) lh = load_vec<T, LM>(l + ol, c, a.istride[0], false);
         if (r_fixed) rh = load_vec<T, RM>(r + orr, c, a.istride[1], false);
-        for (uint32_t g = g_begin + ty; g < g_end; g += gy) {
-            Vec16<T> x = l_fixed ? lh : load_vec<T, LM>(l + ol + (int64_t)g * a.gstride[0], c, a.istride[0], ntl);
-            Vec16<T> y;
-            if constexpr (OP == kOpCopy) y = x;
-            else y = r_fixed ? rh : load_vec<T, RM>(r + orr + (int64_t)g * a.gstride[1], c, a.istride[1], ntr);
+        if constexpr (GU == 1) {
+            // short loop (two steps per lane by default): load, combine, store
+            for (uint32_t g = g_begin + ty; g < g_end; g += gy) {
+                Vec16<T> x = l_fixed ? lh : load_vec<T, LM>(l + ol + (int64_t)g * a.gstride[0], c, a.istride[0], ntl);
+                Vec16<T> y;
+                if constexpr (OP == kOpCopy) y = x;
+                else y = r_fixed ? rh : load_vec<T, RM>(r + orr + (int64_t)g * a.gstride[1], c, a.istride[1], ntr);
 #pragma unroll
-            for (int j = 0; j < N; ++j) x.e[j] = bin_apply<OP, T>(x.e[j], y.e[j]);
-            rt_st16_nt(reinterpret_cast<Vec16<T>*>(d + od + (int64_t)g * a.gstride[2] + c), x);
+                for (int j = 0; j < N; ++j) x.e[j] = bin_apply<OP, T>(x.e[j], y.e[j]);
+                rt_st16_nt(reinterpret_cast<Vec16<T>*>(d + od + (int64_t)g * a.gstride[2] + c), x);
+            }
+        } else {
+            // long loop (an expensive operand is held in registers while the block walks the loop dim): GU steps per
+            // batch, the next batch's loads issued before this batch's stores.  Loads and stores retire in issue order,
+            // so a load issued after a store would wait for that store's acknowledgement.
+            Vec16<T> xn[GU], yn[GU];
+            auto load_batch = [&](uint32_t g0) {
+#pragma unroll
+                for (int u = 0; u < GU; ++u) {
+                    const uint32_t g = min(g0 + u * gy, g_end - 1);
+                    if (!l_fixed) xn[u] = load_vec<T, LM>(l + ol + (int64_t)g * a.gstride[0], c, a.istride[0], ntl);
+                    if constexpr (OP != kOpCopy) { if (!r_fixed) yn[u] = load_vec<T, RM>(r + orr + (int64_t)g * a.gstride[1], c, a.istride[1], ntr); }
+                }
+            };
+            uint32_t g0 = g_begin + ty;
+            if (g0 < g_end) load_batch(g0);
+            for (; g0 < g_end; g0 += gy * GU) {
+                Vec16<T> x[GU], y[GU];
+#pragma unroll
+                for (int u = 0; u < GU; ++u) {
+                    x[u] = l_fixed ? lh : xn[u];
+                    if constexpr (OP == kOpCopy) y[u] = x[u]; else y[u] = r_fixed ? rh : yn[u];
+                }
+                if (g0 + gy * GU < g_end) load_batch(g0 + gy * GU);
+#pragma unroll
+                for (int u = 0; u < GU; ++u) {
+                    const uint32_t g = g0 + u * gy;
+                    if (g < g_end) {
+#pragma unroll
+                        for (int j = 0; j < N; ++j) x[u].e[j] = bin_apply<OP, T>(x[u].e[j], y[u].e[j]);
+                        rt_st16_nt(reinterpret_cast<Vec16<T>*>(d + od + (int64_t)g * a.gstride[2] + c), x[u]);
+                    }
+                }
+            }
         }
     } else {
         // ragged end of a row: element accesses
@@ -171,6 +207,146 @@ __global__ __launch_bounds__(kRBlock) void bin_rows_kernel(const T* l, const T* 
             T* dp = d + od + (int64_t)g * a.gstride[2];
             for (uint32_t k = c; k < a.L; ++k)
                 dp[k] = bin_apply<OP, T>(lp[(int64_t)k * a.istride[0]], rp[(int64_t)k * a.istride[1]]);
+        }
+    }
+}
+
+// ---- tile (one operand transposed) ---------------------------------------------------------------------------------------
+// One input has its unit-|stride| dim somewhere other than dst's inner dim (a permuted, possibly reversed view): reading
+// it along dst's inner dim would touch one cache line per element.  A block instead gathers a (kTK x TL) tile of it with
+// lanes running along *its* unit-stride dim `t` (one 128-byte line per 32 lanes), transposes through LDS, keeps its
+// share of the tile in registers, and then walks the loop dim g (an outer dim along which that operand does not move,
+// if there is one) writing full rows of dst with 16-byte non-temporal stores.
+constexpr int kTBlock = 256;
+constexpr int kTK = 32;                      // tile extent along the transposed operand's unit-stride dim
+constexpr int kTRows = kTK / (kTBlock / RT_WAVE);   // rows of the tile each lane keeps (8)
+
+struct TileArgs {
+    uint32_t L, K, G;               // inner length, extent of dim t, extent of the loop dim (1 if none)
+    uint32_t gchunk, nchunks, ktiles, ltiles;
+    FastDiv32 ltiles_div, ktiles_div, nchunks_div;
+    int nouter;
+    uint32_t oshape[RT_MAX_RANK];
+    FastDiv32 odiv[RT_MAX_RANK];
+    int64_t ostride[3][RT_MAX_RANK];
+    int64_t gstride[3], tstride[3], istride[3];   // per operand (0 left, 1 right, 2 dst): loop dim, dim t, inner dim
+    uint32_t nt_other;              // the non-transposed input is streamed -> non-temporal loads
+};
+
+// XT = index (0/1) of the transposed input; OM = access mode of the other input along the inner dim.
+template <class T, int OP, int XT, int OM>
+__global__ __launch_bounds__(kTBlock) void bin_tile_kernel(const T* l, const T* r, T* d, TileArgs a) {
+    constexpr int N = 16 / sizeof(T);
+    constexpr int TL = RT_WAVE * N;           // tile extent along dst's inner dim: one 16-byte vector per lane of a wave
+    __shared__ alignas(16) T tile[kTK][TL + N];
+    uint32_t b = blockIdx.x;
+    uint32_t q = fd_div(b, a.ltiles_div);
+    const uint32_t ltile = b - q * a.ltiles;
+    b = q;
+    q = fd_div(b, a.ktiles_div);
+    const uint32_t ktile = b - q * a.ktiles;
+    b = q;
+    q = fd_div(b, a.nchunks_div);
+    const uint32_t chunk = b - q * a.nchunks;
+    uint32_t rem = q;
+    int64_t off[3] = {0, 0, 0};
+#pragma unroll
+    for (int k = RT_MAX_RANK - 1; k >= 0; --k) {
+        if (k < a.nouter) {
+            uint32_t qq = fd_div(rem, a.odiv[k]);
+            uint32_t c = rem - qq * a.oshape[k];
+#pragma unroll
+            for (int o = 0; o < 3; ++o) off[o] += (int64_t)c * a.ostride[o][k];
+            rem = qq;
+        }
+    }
+    const T* xt = (XT == 0 ? l : r) + off[XT];
+    const T* xo = (XT == 0 ? r : l) + off[1 - XT];
+    constexpr int O = 1 - XT;
+    T* dp = d + off[2];
+    const uint32_t k0 = ktile * kTK, l0 = ltile * TL;
+    const uint32_t g_begin = chunk * a.gchunk;
+    const uint32_t g_end = min(a.G, g_begin + a.gchunk);
+    const bool xt_fixed = a.gstride[XT] == 0;
+
+    const uint32_t lane = threadIdx.x & (RT_WAVE - 1), wv = threadIdx.x / RT_WAVE;
+    const uint32_t c = l0 + lane * N;                        // first inner column of this lane's vectors
+    Vec16<T> xv[kTRows];
+    Vec16<T> ov[kTRows];                                     // other operand, fetched one loop step ahead
+
+    const bool o_fixed = a.tstride[O] == 0;
+    if (c + N <= a.L && g_begin < g_end) {
+        // first step's rows of the other operand: issued before the gather so that both are in flight together
+        const T* orow0 = xo + (int64_t)g_begin * a.gstride[O];
+#pragma unroll
+        for (int i = 0; i < kTRows; ++i) {
+            const uint32_t k = min(k0 + wv + i * (kTBlock / RT_WAVE), a.K - 1);
+            if (i == 0 || !o_fixed) ov[i] = load_vec<T, OM>(orow0 + (int64_t)k * a.tstride[O], c, a.istride[O], a.nt_other != 0);
+        }
+    }
+
+    for (uint32_t g = g_begin; g < g_end; ++g) {
+        if (g == g_begin || !xt_fixed) {
+            if (g != g_begin) __syncthreads();
+            // gather: lanes along dim t (32 consecutive lanes read one 128-byte line of the transposed operand); each
+            // lane collects the N elements of one 16-byte group of a tile row, all loads in flight before the first LDS
+            // write, and writes the group with one 16-byte LDS store (row stride = 4 words mod 32: conflict free).
+            const uint32_t tk = threadIdx.x % kTK, grp0 = threadIdx.x / kTK;
+            constexpr int kGroupsPerLane = RT_WAVE / (kTBlock / kTK);          // 64 groups per row / 8 lanes-rows = 8
+            const T* src = xt + (int64_t)g * a.gstride[XT] + (int64_t)min(k0 + tk, a.K - 1) * a.tstride[XT];
+            Vec16<T> grp[kGroupsPerLane];
+#pragma unroll
+            for (int i = 0; i < kGroupsPerLane; ++i) {
+                const uint32_t col = l0 + (grp0 + i * (kTBlock / kTK)) * N;
+#pragma unroll
+                for (int j = 0; j < N; ++j) grp[i].e[j] = src[(int64_t)min(col + j, a.L - 1) * a.istride[XT]];
+            }
+#pragma unroll
+            for (int i = 0; i < kGroupsPerLane; ++i)
+                *reinterpret_cast<Vec16<T>*>(&tile[tk][(grp0 + i * (kTBlock / kTK)) * N]) = grp[i];
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < kTRows; ++i) xv[i] = *reinterpret_cast<const Vec16<T>*>(&tile[wv + i * (kTBlock / RT_WAVE)][lane * N]);
+        }
+        if (c >= a.L) continue;
+        const T* orow = xo + (int64_t)g * a.gstride[O];
+        T* drow = dp + (int64_t)g * a.gstride[2];
+        if (c + N <= a.L) {
+            // Loads and stores retire in issue order on this hardware, so waiting for a load that was issued after a
+            // batch of stores also waits for those stores to be acknowledged.  The other operand is therefore fetched one
+            // loop step ahead: its wait only covers loads.
+            Vec16<T> cur[kTRows];
+#pragma unroll
+            for (int i = 0; i < kTRows; ++i) cur[i] = ov[o_fixed ? 0 : i];
+            if (g + 1 < g_end && a.gstride[O] != 0) {
+                const T* nrow = xo + (int64_t)(g + 1) * a.gstride[O];
+#pragma unroll
+                for (int i = 0; i < kTRows; ++i) {
+                    const uint32_t k = min(k0 + wv + i * (kTBlock / RT_WAVE), a.K - 1);
+                    if (i == 0 || !o_fixed) ov[i] = load_vec<T, OM>(nrow + (int64_t)k * a.tstride[O], c, a.istride[O], a.nt_other != 0);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < kTRows; ++i) {
+                const uint32_t k = k0 + wv + i * (kTBlock / RT_WAVE);
+                if (k < a.K) {
+                    Vec16<T> out;
+#pragma unroll
+                    for (int j = 0; j < N; ++j) out.e[j] = XT == 0 ? bin_apply<OP, T>(xv[i].e[j], cur[i].e[j]) : bin_apply<OP, T>(cur[i].e[j], xv[i].e[j]);
+                    rt_st16_nt(reinterpret_cast<Vec16<T>*>(drow + (int64_t)k * a.tstride[2] + c), out);
+                }
+            }
+        } else {
+            for (int i = 0; i < kTRows; ++i) {
+                const uint32_t k = k0 + wv + i * (kTBlock / RT_WAVE);
+                if (k < a.K) {
+                    for (uint32_t cc = c; cc < a.L; ++cc) {
+                        T xe = xv[i].e[cc - c];
+                        T oe = (orow + (int64_t)k * a.tstride[O])[(int64_t)cc * a.istride[O]];
+                        drow[(int64_t)k * a.tstride[2] + cc] = XT == 0 ? bin_apply<OP, T>(xe, oe) : bin_apply<OP, T>(oe, xe);
+                    }
+                }
+            }
         }
     }
 }
@@ -225,20 +401,28 @@ __global__ __launch_bounds__(kBlock) void bin_generic64_kernel(const T* l, const
 }
 
 // ---- host: kernel choice ----------------------------------------------------------------------------------------------
+template <class T, int OP, int LM, int RM>
+void launch_rows_g(bool batched, dim3 grid, hipStream_t s, const T* l, const T* r, T* d, const RowArgs& a) {
+    // the batched long-loop form is only ever chosen when one input is gathered element-wise
+    if constexpr (LM == M_ELEM || RM == M_ELEM) {
+        if (batched) { hipLaunchKernelGGL((bin_rows_kernel<T, OP, LM, RM, 4>), grid, dim3(kRBlock), 0, s, l, r, d, a); return; }
+    }
+    hipLaunchKernelGGL((bin_rows_kernel<T, OP, LM, RM, 1>), grid, dim3(kRBlock), 0, s, l, r, d, a);
+}
 template <class T, int OP, int LM>
-void launch_rows_r(int rm, dim3 grid, hipStream_t s, const T* l, const T* r, T* d, const RowArgs& a) {
+void launch_rows_r(int rm, bool batched, dim3 grid, hipStream_t s, const T* l, const T* r, T* d, const RowArgs& a) {
     switch (rm) {
-        case M_VEC: hipLaunchKernelGGL((bin_rows_kernel<T, OP, LM, M_VEC>), grid, dim3(kRBlock), 0, s, l, r, d, a); break;
-        case M_BCAST: hipLaunchKernelGGL((bin_rows_kernel<T, OP, LM, M_BCAST>), grid, dim3(kRBlock), 0, s, l, r, d, a); break;
-        default: hipLaunchKernelGGL((bin_rows_kernel<T, OP, LM, M_ELEM>), grid, dim3(kRBlock), 0, s, l, r, d, a); break;
+        case M_VEC: launch_rows_g<T, OP, LM, M_VEC>(batched, grid, s, l, r, d, a); break;
+        case M_BCAST: launch_rows_g<T, OP, LM, M_BCAST>(batched, grid, s, l, r, d, a); break;
+        default: launch_rows_g<T, OP, LM, M_ELEM>(batched, grid, s, l, r, d, a); break;
     }
 }
 template <class T, int OP>
-void launch_rows(int lm, int rm, dim3 grid, hipStream_t s, const T* l, const T* r, T* d, const RowArgs& a) {
+void launch_rows(int lm, int rm, bool batched, dim3 grid, hipStream_t s, const T* l, const T* r, T* d, const RowArgs& a) {
     switch (lm) {
-        case M_VEC: launch_rows_r<T, OP, M_VEC>(rm, grid, s, l, r, d, a); break;
-        case M_BCAST: launch_rows_r<T, OP, M_BCAST>(rm, grid, s, l, r, d, a); break;
-        default: launch_rows_r<T, OP, M_ELEM>(rm, grid, s, l, r, d, a); break;
+        case M_VEC: launch_rows_r<T, OP, M_VEC>(rm, batched, grid, s, l, r, d, a); break;
+        case M_BCAST: launch_rows_r<T, OP, M_BCAST>(rm, batched, grid, s, l, r, d, a); break;
+        default: launch_rows_r<T, OP, M_ELEM>(rm, batched, grid, s, l, r, d, a); break;
     }
 }
 
@@ -296,6 +480,86 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
             if (tail) edge(head + nvec * N, tail);
             RT_HIP(hipGetLastError());
             return RT_OK;
+        }
+    }
+
+    // (2a) tile: exactly one input is "transposed" (inner stride neither 0 nor 1, unit |stride| along another dim)
+    if (OP != kOpCopy && rank >= 2 && count < (1ull << 31) && dsc.stride[2][rank - 1] == 1 && dsc.shape[rank - 1] >= 2 * N && vec_ok<T>(d, dsc, 2)) {
+        auto transposed_dim = [&](int o) -> int {
+            int64_t is = dsc.stride[o][rank - 1];
+            if (is == 0 || is == 1) return -1;
+            for (int k = rank - 2; k >= 0; --k)
+                if ((dsc.stride[o][k] == 1 || dsc.stride[o][k] == -1) && dsc.shape[k] >= 16) return k;
+            return -1;
+        };
+        const int tl = transposed_dim(0), tr = transposed_dim(1);
+        // When the transposed input does not move along some long outer dim, the row kernel gathers it once per block
+        // and reuses it from registers for 16 output rows, which measured faster than the tile kernel; the tile kernel
+        // is for the case without such reuse (e.g. a + b.transpose()).
+        auto hoistable = [&](int o) {
+            for (int k = 0; k < rank - 1; ++k)
+                if (dsc.stride[o][k] == 0 && dsc.shape[k] >= 8) return true;
+            return false;
+        };
+        if ((tl >= 0) != (tr >= 0) && !hoistable(tl >= 0 ? 0 : 1)) {
+            const int xt = tl >= 0 ? 0 : 1, o = 1 - xt, tdim = tl >= 0 ? tl : tr;
+            int om;
+            {
+                int64_t is = dsc.stride[o][rank - 1];
+                const T* base = o == 0 ? l : r;
+                om = is == 0 ? (int)M_BCAST : ((is == 1 && vec_ok<T>(base, dsc, o)) ? (int)M_VEC : (int)M_ELEM);
+            }
+            TileArgs a;
+            memset(&a, 0, sizeof(a));
+            a.L = (uint32_t)dsc.shape[rank - 1];
+            a.K = (uint32_t)dsc.shape[tdim];
+            int gdim = -1;
+            for (int k = 0; k < rank - 1; ++k)
+                if (k != tdim && dsc.stride[xt][k] == 0 && (gdim < 0 || dsc.shape[k] > dsc.shape[gdim])) gdim = k;
+            a.G = gdim >= 0 ? (uint32_t)dsc.shape[gdim] : 1;
+            for (int q = 0; q < 3; ++q) {
+                a.gstride[q] = gdim >= 0 ? dsc.stride[q][gdim] : 0;
+                a.tstride[q] = dsc.stride[q][tdim];
+                a.istride[q] = dsc.stride[q][rank - 1];
+            }
+            uint64_t outer = 1;
+            for (int k = 0; k < rank - 1; ++k) {
+                if (k == gdim || k == tdim) continue;
+                a.oshape[a.nouter] = (uint32_t)dsc.shape[k];
+                a.odiv[a.nouter] = make_fastdiv((uint32_t)dsc.shape[k]);
+                for (int q = 0; q < 3; ++q) a.ostride[q][a.nouter] = dsc.stride[q][k];
+                outer *= (uint64_t)dsc.shape[k];
+                a.nouter++;
+            }
+            for (int k = a.nouter; k < RT_MAX_RANK; ++k) { a.oshape[k] = 1; a.odiv[k] = make_fastdiv(1); }
+            const uint32_t TL = RT_WAVE * (uint32_t)N;
+            a.ktiles = (a.K + kTK - 1) / kTK;
+            a.ltiles = (a.L + TL - 1) / TL;
+            // loop-dim steps per block: the gathered tile is reused for all of them; keep enough blocks to fill the chip
+            uint32_t gchunk = a.G;
+            const uint64_t want_blocks = (uint64_t)ctx->num_cus * 16;
+            while (gchunk > 8 && outer * a.ktiles * a.ltiles * ((a.G + gchunk - 1) / gchunk) < want_blocks) gchunk = (gchunk + 1) / 2;
+            a.gchunk = gchunk;
+            a.nchunks = (a.G + gchunk - 1) / gchunk;
+            a.ltiles_div = make_fastdiv(a.ltiles);
+            a.ktiles_div = make_fastdiv(a.ktiles);
+            a.nchunks_div = make_fastdiv(a.nchunks);
+            bool streamed = true;
+            for (int k = 0; k < rank; ++k) streamed = streamed && dsc.stride[o][k] != 0;
+            a.nt_other = streamed ? 1u : 0u;
+            const uint64_t blocks = outer * a.nchunks * a.ktiles * a.ltiles;
+            if (blocks < (1ull << 31)) {
+                const T* lp = l + dsc.offset[0];
+                const T* rp = r + dsc.offset[1];
+                T* dp = d + dsc.offset[2];
+                dim3 grid((unsigned)blocks), blk(kTBlock);
+#define RT_TILE(XT, OM) hipLaunchKernelGGL((bin_tile_kernel<T, OP, XT, OM>), grid, blk, 0, s, lp, rp, dp, a)
+                if (xt == 0) { if (om == M_VEC) RT_TILE(0, M_VEC); else if (om == M_BCAST) RT_TILE(0, M_BCAST); else RT_TILE(0, M_ELEM); }
+                else         { if (om == M_VEC) RT_TILE(1, M_VEC); else if (om == M_BCAST) RT_TILE(1, M_BCAST); else RT_TILE(1, M_ELEM); }
+#undef RT_TILE
+                RT_HIP(hipGetLastError());
+                return RT_OK;
+            }
         }
     }
 
@@ -363,7 +627,7 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
         }
         const uint64_t blocks = outer * a.nchunks * a.tiles;
         if (blocks < (1ull << 31)) {
-            launch_rows<T, OP>(lm, rm, dim3((unsigned)blocks), s, l + dsc.offset[0], r + dsc.offset[1], d + dsc.offset[2], a);
+            launch_rows<T, OP>(lm, rm, steps > 2, dim3((unsigned)blocks), s, l + dsc.offset[0], r + dsc.offset[1], d + dsc.offset[2], a);
             RT_HIP(hipGetLastError());
             return RT_OK;
         }

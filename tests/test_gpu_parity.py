@@ -473,3 +473,37 @@ def test_convert(hip):
     with pytest.raises(H.TensorError) as e:
         hip.convert(isrc, hip.alloc(H.F32, 3))
     assert e.value.kind == "SizeMismatch"
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64", "i32", "u8", "i16"])
+def test_broadcast_with_transposed_operand(hip, dtype):
+    """One input is a permuted (and possibly reversed / strided) view whose unit-stride dim is not the output's inner dim:
+    the LDS-transpose tile kernel.  Ragged tile edges, both operand positions, broadcast and in-place forms."""
+    rng = np.random.default_rng(abs(hash(dtype)) % 2 ** 31)
+    shapes = [(3, 40, 70), (2, 5, 33, 130), (64, 257), (1, 100, 36), (4, 17, 1030), (2, 3, 16, 16)]
+    for shape in shapes:
+        r = len(shape)
+        perm = list(range(r)); perm[-1], perm[-2] = perm[-2], perm[-1]
+        base_shape = [shape[p] for p in perm]                 # base laid out so that permuting it gives `shape`
+        vx = rand_values(dtype, int(np.prod(shape)), rng)
+        ox, gx = OTensor.from_buf(dtype, vx, base_shape), G(hip, dtype, vx, base_shape)
+        for variant in range(4):
+            oxv, gxv = ox.permute(perm), gx.permute(perm)
+            if variant & 1:                                    # reverse the dim that is unit-stride in memory
+                oxv, gxv = oxv.slice(r - 2, Slice(None, None, -1)), gxv.slice(r - 2, Slice(None, None, -1))
+            if variant & 2 and r >= 3:                         # the other operand broadcasts along dim 0
+                sy = [1] + list(oxv.meta.shape[1:])
+            else:
+                sy = list(oxv.meta.shape)
+            vy = rand_values(dtype, int(np.prod(sy)), rng)
+            oy, gy = OTensor.from_buf(dtype, vy, sy), G(hip, dtype, vy, sy)
+            for op in ("add", "sub", "mul"):
+                f = {"add": "__add__", "sub": "__sub__", "mul": "__mul__"}[op]
+                with np.errstate(all="ignore"):
+                    w1, w2 = getattr(oxv, f)(oy), getattr(oy, f)(oxv)
+                g1, g2 = getattr(gxv, f)(gy), getattr(gy, f)(gxv)
+                assert g1.dump().tobytes() == w1.buf.tobytes(), (dtype, shape, variant, op, "x op y")
+                assert g2.dump().tobytes() == w2.buf.tobytes(), (dtype, shape, variant, op, "y op x")
+            if sy == list(oxv.meta.shape):                     # in place: y (contiguous) += transposed x
+                oy += oxv; gy += gxv
+                assert gy.dump().tobytes() == oy.buf.tobytes(), (dtype, shape, variant, "inplace")
