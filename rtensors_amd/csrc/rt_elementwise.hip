@@ -17,12 +17,16 @@ struct boolean_t { uint8_t v; };      // core/value.rs:650-765: + is OR, - is XO
 
 template <class T> struct is_flt : std::integral_constant<bool, std::is_same<T, float>::value || std::is_same<T, double>::value> {};
 template <class T> struct is_bool : std::is_same<T, boolean_t> {};
-template <class T> struct is_sint : std::integral_constant<bool, std::is_integral<T>::value && std::is_signed<T>::value> {};
-template <class T> struct is_uint : std::integral_constant<bool, std::is_integral<T>::value && std::is_unsigned<T>::value> {};
+typedef unsigned __int128 u128_t;      // core/value.rs: u128 / i128 (no division on the device: there is no 128-bit divide routine)
+typedef __int128 i128_t;
+template <class T> struct is_sint : std::integral_constant<bool, (std::is_integral<T>::value && std::is_signed<T>::value) || std::is_same<T, i128_t>::value> {};
+template <class T> struct is_uint : std::integral_constant<bool, (std::is_integral<T>::value && std::is_unsigned<T>::value) || std::is_same<T, u128_t>::value> {};
+template <class T> struct is_int : std::integral_constant<bool, is_sint<T>::value || is_uint<T>::value> {};
 
 template <class T, class E = void> struct carrier { typedef T type; };
-template <class T> struct carrier<T, typename std::enable_if<std::is_integral<T>::value && sizeof(T) <= 4>::type> { typedef uint32_t type; };
-template <class T> struct carrier<T, typename std::enable_if<std::is_integral<T>::value && sizeof(T) == 8>::type> { typedef uint64_t type; };
+template <class T> struct carrier<T, typename std::enable_if<is_int<T>::value && sizeof(T) <= 4>::type> { typedef uint32_t type; };
+template <class T> struct carrier<T, typename std::enable_if<is_int<T>::value && sizeof(T) == 8>::type> { typedef uint64_t type; };
+template <class T> struct carrier<T, typename std::enable_if<is_int<T>::value && sizeof(T) == 16>::type> { typedef u128_t type; };
 
 // wrapping integer arithmetic (Rust release semantics) through an unsigned carrier; IEEE for floats
 template <class T> __device__ __forceinline__ T w_add(T a, T b) {
@@ -45,6 +49,7 @@ template <class T> __device__ __forceinline__ T w_mul(T a, T b) {
 template <class T> __device__ __forceinline__ T w_div(T a, T b) {
     if constexpr (is_flt<T>::value) return a / b;
     else if constexpr (is_bool<T>::value) return boolean_t{0};
+    else if constexpr (sizeof(T) == 16) return (T)0;                      // refused on the host
     else if constexpr (is_sint<T>::value) {
         if (b == 0) return 0;
         if (b == (T)-1) return w_sub<T>((T)0, a);
@@ -415,6 +420,8 @@ template <class T> T load_scalar(const void* v) { T x; memcpy(&x, v, sizeof(T));
         case RT_I32: { typedef int32_t T; BODY; } break;                    \
         case RT_U64: { typedef uint64_t T; BODY; } break;                   \
         case RT_I64: { typedef int64_t T; BODY; } break;                    \
+        case RT_U128: { typedef u128_t T; BODY; } break;                    \
+        case RT_I128: { typedef i128_t T; BODY; } break;                    \
         case RT_F32: { typedef float T; BODY; } break;                      \
         case RT_F64: { typedef double T; BODY; } break;                     \
         case RT_BOOL: { typedef boolean_t T; BODY; } break;                 \
@@ -422,7 +429,6 @@ template <class T> T load_scalar(const void* v) { T x; memcpy(&x, v, sizeof(T));
     }
 
 int32_t no_dtype(const char* what, int dtype) {
-    if (dtype == RT_U128 || dtype == RT_I128) return rt_fail(RT_E_DTYPE, "%s: 128-bit integers are not built for the device", what);
     return rt_fail(RT_E_DTYPE, "%s: unknown dtype code %d", what, dtype);
 }
 
@@ -494,6 +500,8 @@ int32_t scalar_typed(rt_ctx* ctx, int op, void* buf, uint64_t buf_len, const voi
         case RT_S_DIV:
             if constexpr (is_bool<T>::value) {
                 return rt_fail(RT_E_ARITH, "scalar div: division is not implemented for boolean in the reference (todo!())");
+            } else if constexpr (sizeof(T) == 16) {
+                return rt_fail(RT_E_DTYPE, "scalar div: 128-bit integer division is not built for the device");
             } else {
                 if constexpr (!is_flt<T>::value) {
                     if (load_scalar<T>(value) == (T)0) return rt_fail(RT_E_ARITH, "scalar div: integer division by zero (the reference panics)");

@@ -507,3 +507,72 @@ def test_broadcast_with_transposed_operand(hip, dtype):
             if sy == list(oxv.meta.shape):                     # in place: y (contiguous) += transposed x
                 oy += oxv; gy += gxv
                 assert gy.dump().tobytes() == oy.buf.tobytes(), (dtype, shape, variant, "inplace")
+
+
+def test_128bit_integers(hip):
+    """u128 / i128: fill, + - * (tensor and scalar), relu / abs / neg, leaky_relu, gather, equality; division is refused."""
+    from rtensors_amd import hip as H
+    rng = np.random.default_rng(128)
+    vals_a = [int(rng.integers(-2 ** 62, 2 ** 62)) * int(rng.integers(1, 2 ** 62)) for _ in range(600)]
+    vals_b = [int(rng.integers(-2 ** 62, 2 ** 62)) * int(rng.integers(1, 2 ** 40)) for _ in range(600)]
+    vals_a[:4] = [2 ** 127 - 1, -2 ** 127, 0, -1]
+    for name, code in (("i128", cpu.I128), ("u128", cpu.U128)):
+        a, b = cpu.from_ints(code, vals_a), cpu.from_ints(code, vals_b)
+        oa, ob = OTensor.from_buf(name, a, [20, 30]), OTensor.from_buf(name, b, [20, 30])
+        ga, gb = G(hip, name, a, [20, 30]), G(hip, name, b, [20, 30])
+        gv = ga.transpose().slice(0, Slice(None, None, -1)); ov = oa.transpose().slice(0, Slice(None, None, -1))
+        for op in ("__add__", "__sub__", "__mul__"):
+            assert getattr(ga, op)(gb).dump().tobytes() == getattr(oa, op)(ob).buf.tobytes(), (name, op)
+            assert getattr(gv, op)(gb.transpose()).dump().tobytes() == getattr(ov, op)(ob.transpose()).buf.tobytes(), (name, op, "view")
+        row = OTensor.from_buf(name, b[:30], [30]); grow = G(hip, name, b[:30], [30])
+        assert (ga + grow).dump().tobytes() == (oa + row).buf.tobytes()
+        assert gv.to_numpy().tobytes() == ov.to_numpy().tobytes()
+        for uop in (("relu", "abs", "neg") if name == "i128" else ("relu", "abs")):
+            assert ga.unary(uop).dump().tobytes() == oa.unary(uop).buf.tobytes(), (name, uop)
+        o2, g2 = oa.owned(), ga.owned()
+        o2 += 12345678901234567890123; g2 += 12345678901234567890123
+        o2 *= 3; g2 *= 3
+        o2.scalar_op_inplace("leaky_relu", 7); g2.scalar_op_inplace("leaky_relu", 7)
+        o2.slice(1, Slice(None, None, 2)).fill(5); g2.slice(1, Slice(None, None, 2)).fill(5)
+        assert g2.dump().tobytes() == o2.buf.tobytes()
+        assert g2.buf == hip.copy(g2.buf) and not (g2.buf == ga.buf)
+        with pytest.raises(H.TensorError) as e:
+            ga / gb
+        assert e.value.kind == "UnsupportedOperation"
+
+
+def test_allocation_failure_is_an_error_not_an_abort(hip):
+    from rtensors_amd import hip as H
+    with pytest.raises(H.TensorError) as e:
+        hip.alloc_uninit(H.F32, 1 << 46)            # 256 TiB
+    assert e.value.kind == "HipError"
+    b = hip.alloc(H.F32, 16)                        # the context keeps working afterwards
+    assert not hip.dump(b).any()
+
+
+def test_one_context_from_several_threads(hip):
+    import threading
+    from rtensors_amd import hip as H
+    errors = []
+
+    def worker(seed):
+        try:
+            rng = np.random.default_rng(seed)
+            for _ in range(30):
+                n = int(rng.integers(1000, 200000))
+                x = rng.standard_normal(n).astype(np.float32)
+                b = hip.alloc_from_slice(H.F32, x)
+                hip.scalar_contiguous("mul", b, 2.0, 0, n)
+                hip.unary_contiguous("relu", b, 0, n)
+                out = hip.alloc(H.F32, 1)
+                hip.apply_reduce_contiguous_flat(b, out, 0, n, "max")
+                want = np.maximum(x * np.float32(2.0), 0)
+                if hip.dump(b).tobytes() != want.tobytes() or hip.dump(out)[0] != max(want.max(), np.finfo(np.float32).min):
+                    errors.append(seed)
+        except Exception as ex:          # noqa: BLE001
+            errors.append(repr(ex))
+
+    ts = [threading.Thread(target=worker, args=(s,)) for s in range(6)]
+    [t.start() for t in ts]
+    [t.join() for t in ts]
+    assert not errors, errors
