@@ -43,7 +43,7 @@ struct rt_ctx {
     // scratch for two-stage reductions (partials), grown on demand, reused across calls
     void* scratch = nullptr;
     size_t scratch_bytes = 0;
-    // one pinned 8-byte cell + device flag used by rt_equal / rt_read
+    // device flag written by the equality kernel and read back by rt_equal
     int32_t* flag_dev = nullptr;
     int num_cus = 256;
 };

@@ -3,9 +3,9 @@
 // Element definitions follow the reference's Cpu backend (backend/cpu.rs:485-724), which is the parity target:
 // e.g. relu is `x > 0 ? x : 0` (NaN -> 0, -0.0 -> +0.0) and sign(0) = 0.
 //
-// Memory behaviour: the contiguous kernel moves 16 bytes per lane per access (global_load/store_dwordx4), a whole
-// wavefront touching 1 KiB of consecutive addresses, UNROLL independent accesses in flight per lane.  Algorithmic
-// traffic is 2*N*sizeof(T) for read-modify-write ops and N*sizeof(T) for fill.
+// Memory behaviour: the contiguous kernel moves one 16-byte vector per lane (global_load/store_dwordx4), a whole
+// wavefront touching 1 KiB of consecutive addresses, in many small blocks.  Algorithmic traffic is 2*N*sizeof(T) for
+// read-modify-write ops and N*sizeof(T) for fill.
 #include "rt_common.h"
 
 #include <type_traits>

@@ -576,3 +576,65 @@ def test_one_context_from_several_threads(hip):
     [t.start() for t in ts]
     [t.join() for t in ts]
     assert not errors, errors
+
+
+def test_rank_limits(hip):
+    from rtensors_amd import hip as H
+    # 12 dims that collapse to one contiguous run: fine
+    shape = [2] * 12
+    strides = [1 << (11 - i) for i in range(12)]
+    x = np.arange(4096, dtype=np.float32) - 2000
+    g = hip.alloc_from_slice(H.F32, x)
+    hip.unary_nd("relu", g, 0, shape, strides)
+    assert np.array_equal(hip.dump(g), np.maximum(x, 0))
+    # 10 dims of a (3^10)-buffer, every dim sliced with step 2: nothing merges, more than 8 dims remain -> refused, not launched
+    n = 3
+    full = [n] * 10
+    st = [n ** (9 - i) * 2 for i in range(10)]
+    big = hip.alloc(H.F32, n ** 10 * 2)
+    with pytest.raises(H.TensorError) as e:
+        hip.unary_nd("relu", big, 0, [2] * 10, st)
+    assert e.value.kind == "UnsupportedOperation"
+    # rank 0 and empty views
+    one = hip.alloc_from_slice(H.F32, np.array([-3.0], np.float32))
+    hip.unary_nd("neg", one, 0, [], [])
+    assert hip.dump(one)[0] == 3.0
+    hip.broadcast((one, (0, [], [])), (one, (0, [], [])), (one, (0, [], [])), "mul")
+    assert hip.dump(one)[0] == 9.0
+    hip.unary_nd("neg", one, 0, [0, 5], [5, 1])
+    hip.broadcast((one, (0, [4, 0], [0, 0])), (one, (0, [4, 0], [0, 0])), (one, (0, [4, 0], [0, 1])), "add")
+    out = hip.alloc(H.F32, 1)
+    hip.apply_reduce_contiguous_flat(one, out, 0, 0, "sum")           # empty reduction: the accumulator's initial value
+    assert hip.dump(out)[0] == 0.0
+    hip.apply_reduce_contiguous_flat(one, out, 0, 0, "max")
+    assert hip.dump(out)[0] == np.finfo(np.float32).min
+
+
+def test_more_than_2_31_elements(hip):
+    """Views and broadcasts with 2^31 + 2^20 elements take the 64-bit index kernels; u8 keeps the buffers at 2-4 GiB."""
+    from rtensors_amd import hip as H
+    n = (1 << 31) + (1 << 20)
+    a = hip.alloc(H.U8, 2 * n)                    # viewed with stride 2
+    hip.fill_contiguous(a, 3, 0, 2 * n)
+    hip.fill_1d_strided(a, 7, 1, 2, n)            # odd positions = 7 (1-D strided kernel, > 2^31 elements)
+    b = hip.alloc(H.U8, n)
+    hip.fill_contiguous(b, 10, 0, n)
+    hip.fill_nd(b, 20, 0, [n // 2, 1], [2, 1])    # even positions = 20
+    d = hip.alloc(H.U8, n)
+    # d[i] = a[2i + 1] + b[i]: left operand strided -> generic 64-bit kernel
+    hip.broadcast((a, (1, [n], [2])), (b, (0, [n], [1])), (d, (0, [n], [1])), "add")
+    host = hip.dump(d)
+    want = np.full(n, 17, dtype=np.uint8); want[0::2] = 27
+    assert np.array_equal(host, want)
+    del host, want
+    # N-d view over 2^31+ elements that is not one run: rows of 2^20 with a gap after each
+    rows, cols = n // (1 << 20), 1 << 20
+    hip.unary_nd("relu", a, 0, [rows, cols - 1], [cols, 1])
+    # contiguous path, 2-D in-place binary over everything, then a device-side reduction as checksum
+    hip.broadcast((d, (0, [n], [1])), (b, (0, [n], [1])), (d, (0, [n], [1])), "sub")
+    out = hip.alloc(H.U8, 1)
+    hip.apply_reduce_contiguous_flat(d, out, 0, n, "max")
+    assert hip.dump(out)[0] == 7
+    hip.apply_reduce_contiguous_flat(d, out, 0, n, "min")
+    assert hip.dump(out)[0] == 7
+    hip.sync()
