@@ -160,6 +160,13 @@ class Workloads:
     def copy(self): return self._c2("copy")
     def fill(self): return self._c2("fill")
 
+    def view_relu(self):
+        # in-place relu on the left half of a (16384,16384) f32 matrix: a non-contiguous view with unit-stride rows
+        H = self.H
+        n = 16384
+        a = self._gen("c2a", H.F32, 1 << 28, "normal", 1, 0)
+        return (lambda: self.hip.unary_nd("relu", a, 0, [n, n // 2], [n, 1])), 2 * n * (n // 2) * 4, n * (n // 2)
+
     def tr_add(self):
         # z = a + b.transpose() on (16384,16384) f32: the right operand's unit-stride dim is the output's row dim
         H = self.H

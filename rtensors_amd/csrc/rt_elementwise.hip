@@ -180,8 +180,7 @@ template <class T> struct FillF {
 // ---- kernels ------------------------------------------------------------------------------------------------------
 template <class T> struct alignas(16) Vec16 { T e[16 / sizeof(T)]; };
 
-constexpr int kBlock = 256;
-constexpr int kUnroll = 4;      // 16-byte accesses per lane in the row kernel
+constexpr int kBlock = 256;     // element-per-lane kernels
 constexpr int kCBlock = 128;    // contiguous kernel: one 16-byte vector per lane, 128 lanes per block
 
 // Body: `nvec` 16-byte vectors starting at the 16-byte aligned address `p`.  One vector per lane and small blocks:
@@ -244,53 +243,58 @@ __global__ __launch_bounds__(kBlock) void ew_nd_kernel(T* __restrict__ p, NdArgs
     }
 }
 
-// N-d view whose innermost collapsed dim is unit-stride: a block walks one row segment with 16-byte accesses when
-// the segment start is 16-byte aligned, element accesses otherwise.  grid.x enumerates (row, column tile).
+// N-d view whose innermost collapsed dim is unit-stride (row ranges, sub-blocks of a matrix ...).  Same work shape as the
+// broadcast row kernel: 128-lane blocks, one 16-byte vector per lane and step, two steps along the innermost outer dim
+// per block; (outer index, chunk, column tile) from blockIdx by multiply-high division on the scalar unit.
+struct RowsArgs {
+    uint32_t L, G, gchunk, nchunks, tiles, tpr;
+    FastDiv32 tiles_div, nchunks_div;
+    int nouter;
+    uint32_t oshape[RT_MAX_RANK];
+    FastDiv32 odiv[RT_MAX_RANK];
+    int64_t ostride[RT_MAX_RANK];
+    int64_t gstride;
+};
+
 template <class T, class F>
-__global__ __launch_bounds__(kBlock) void ew_rows_kernel(T* __restrict__ p, NdArgs a, uint32_t tiles_per_row, FastDiv32 tdiv, F f) {
+__global__ __launch_bounds__(kCBlock) void ew_rows_kernel(T* __restrict__ p, RowsArgs a, F f) {
     constexpr int N = 16 / sizeof(T);
-    const uint32_t row = fd_div(blockIdx.x, tdiv);
-    const uint32_t tile = blockIdx.x - row * tiles_per_row;
-    uint32_t rem = row;
+    uint32_t b = blockIdx.x;
+    uint32_t q = fd_div(b, a.tiles_div);
+    const uint32_t tile = b - q * a.tiles;
+    b = q;
+    q = fd_div(b, a.nchunks_div);
+    const uint32_t chunk = b - q * a.nchunks;
+    uint32_t rem = q;
     int64_t off = 0;
 #pragma unroll
-    for (int d = RT_MAX_RANK - 2; d >= 0; --d) {
-        if (d < a.rank - 1) {
-            uint32_t q = fd_div(rem, a.div[d]);
-            uint32_t c = rem - q * a.shape[d];
-            off += (int64_t)c * a.stride[d];
-            rem = q;
+    for (int k = RT_MAX_RANK - 1; k >= 0; --k) {
+        if (k < a.nouter) {
+            uint32_t qq = fd_div(rem, a.odiv[k]);
+            off += (int64_t)(rem - qq * a.oshape[k]) * a.ostride[k];
+            rem = qq;
         }
     }
-    const uint32_t L = a.shape[a.rank - 1];
-    T* rowp = p + off;
-    const uint32_t col0 = tile * (kBlock * N * kUnroll);
-    const bool aligned = ((reinterpret_cast<uintptr_t>(rowp) & 15) == 0);
-    if (aligned) {
+    const uint32_t tx = threadIdx.x & (a.tpr - 1), ty = threadIdx.x / a.tpr, gy = kCBlock / a.tpr;
+    const uint32_t c = (tile * a.tpr + tx) * N;
+    if (c >= a.L) return;
+    const uint32_t g_begin = chunk * a.gchunk, g_end = min(a.G, g_begin + a.gchunk);
+    for (uint32_t g = g_begin + ty; g < g_end; g += gy) {
+        T* rowp = p + off + (int64_t)g * a.gstride;
+        if (c + N <= a.L) {
+            Vec16<T>* v = reinterpret_cast<Vec16<T>*>(rowp + c);
+            Vec16<T> w;
+            if constexpr (F::kReads) w = rt_ld16_nt(v);
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            const uint32_t c = col0 + (u * kBlock + threadIdx.x) * N;
-            if (c + N <= L) {
-                Vec16<T>* q = reinterpret_cast<Vec16<T>*>(rowp + c);
-                Vec16<T> w;
-                if constexpr (F::kReads) w = *q;
-#pragma unroll
-                for (int j = 0; j < N; ++j) w.e[j] = f(w.e[j]);
-                *q = w;
-            } else {
-                for (uint32_t k = c; k < L && k < c + N; ++k) {
-                    T x = zero_of<T>();
-                    if constexpr (F::kReads) x = rowp[k];
-                    rowp[k] = f(x);
-                }
+            for (int j = 0; j < N; ++j) w.e[j] = f(w.e[j]);
+            if constexpr (F::kReads) rt_st16_nt(v, w);
+            else *v = w;
+        } else {
+            for (uint32_t k = c; k < a.L; ++k) {
+                T x = zero_of<T>();
+                if constexpr (F::kReads) x = rowp[k];
+                rowp[k] = f(x);
             }
-        }
-    } else {
-        const uint32_t end = min(L, col0 + kBlock * N * kUnroll);
-        for (uint32_t k = col0 + threadIdx.x; k < end; k += kBlock) {
-            T x = zero_of<T>();
-            if constexpr (F::kReads) x = rowp[k];
-            rowp[k] = f(x);
         }
     }
 }
@@ -368,15 +372,40 @@ int32_t launch_view(rt_ctx* ctx, T* base, const NdDesc& d, uint64_t count, F f) 
         a.stride[i] = i < d.rank ? d.stride[0][i] : 0;
         a.div[i] = make_fastdiv(a.shape[i]);
     }
-    constexpr uint32_t N = 16 / sizeof(T);
-    const uint32_t L = a.shape[d.rank - 1];
-    if (d.stride[0][d.rank - 1] == 1 && L >= 4 * N) {
-        const uint32_t per_tile = kBlock * N * kUnroll;
-        const uint32_t tiles = (L + per_tile - 1) / per_tile;
-        const uint64_t rows = count / L;
-        if (rows * tiles < (1ull << 31)) {
-            hipLaunchKernelGGL((ew_rows_kernel<T, F>), dim3((unsigned)(rows * tiles)), dim3(kBlock), 0, ctx->stream,
-                               p, a, tiles, make_fastdiv(tiles), f);
+    constexpr int64_t N = 16 / sizeof(T);
+    // rows form: unit-stride inner dim of at least two vectors, every row start 16-byte aligned
+    bool rows_ok = d.stride[0][d.rank - 1] == 1 && d.shape[d.rank - 1] >= 2 * N && (reinterpret_cast<uintptr_t>(p) & 15) == 0;
+    for (int k = 0; k < d.rank - 1; ++k) rows_ok = rows_ok && (d.stride[0][k] % N == 0);
+    if (rows_ok) {
+        RowsArgs r;
+        memset(&r, 0, sizeof(r));
+        const int gdim = d.rank - 2;
+        r.L = (uint32_t)d.shape[d.rank - 1];
+        r.G = (uint32_t)d.shape[gdim];
+        r.gstride = d.stride[0][gdim];
+        uint64_t outer = 1;
+        for (int k = 0; k < gdim; ++k) {
+            r.oshape[r.nouter] = (uint32_t)d.shape[k];
+            r.odiv[r.nouter] = make_fastdiv((uint32_t)d.shape[k]);
+            r.ostride[r.nouter] = d.stride[0][k];
+            outer *= (uint64_t)d.shape[k];
+            r.nouter++;
+        }
+        for (int k = r.nouter; k < RT_MAX_RANK; ++k) { r.oshape[k] = 1; r.odiv[k] = make_fastdiv(1); }
+        const uint32_t vecs = (uint32_t)((r.L + N - 1) / N);
+        uint32_t tpr = 1;
+        while (tpr < vecs && tpr < (uint32_t)kCBlock) tpr <<= 1;
+        r.tpr = tpr;
+        r.tiles = (vecs + tpr - 1) / tpr;
+        uint32_t gchunk = (kCBlock / tpr) * 2;
+        if (gchunk > r.G) gchunk = r.G;
+        r.gchunk = gchunk;
+        r.nchunks = (r.G + gchunk - 1) / gchunk;
+        r.tiles_div = make_fastdiv(r.tiles);
+        r.nchunks_div = make_fastdiv(r.nchunks);
+        const uint64_t blocks = outer * r.nchunks * r.tiles;
+        if (blocks < (1ull << 31)) {
+            hipLaunchKernelGGL((ew_rows_kernel<T, F>), dim3((unsigned)blocks), dim3(kCBlock), 0, ctx->stream, p, r, f);
             RT_HIP(hipGetLastError());
             return RT_OK;
         }
