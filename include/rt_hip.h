@@ -53,7 +53,10 @@ typedef enum rt_binary_op { RT_ADD = 0, RT_SUB = 1, RT_MUL = 2, RT_DIV = 3 } rt_
 
 /* backend/remote/protocol.rs:226-232 */
 typedef enum rt_scalar_op {
-    RT_S_ADD = 0, RT_S_SUB = 1, RT_S_MUL = 2, RT_S_DIV = 3, RT_S_LOG = 4, RT_S_LOG1P = 5, RT_S_LEAKY_RELU = 6, RT_S_ELU = 7
+    RT_S_ADD = 0, RT_S_SUB = 1, RT_S_MUL = 2, RT_S_DIV = 3, RT_S_LOG = 4, RT_S_LOG1P = 5, RT_S_LEAKY_RELU = 6, RT_S_ELU = 7,
+    /* No op of its own in the reference: x > 0 ? 1 : s, the leaky-ReLU gradient map its autograd builds one element at a
+     * time with get/set (ops/scalar/mod.rs:149-166). */
+    RT_S_LEAKY_GRAD = 8
 } rt_scalar_op;
 
 /* backend/remote/protocol.rs:213-224 */

@@ -318,7 +318,7 @@ unary_impl(int op, T* buf, size_t buflen, const Meta& m, int* path) {
 }
 
 // ---- scalar functions: backend/cpu.rs:677-724 -------------------------------------------------------------------
-enum : int { S_ADD = 0, S_SUB, S_MUL, S_DIV, S_LOG, S_LOG1P, S_LEAKY_RELU, S_ELU, S_COUNT };   // protocol.rs:226-232
+enum : int { S_ADD = 0, S_SUB, S_MUL, S_DIV, S_LOG, S_LOG1P, S_LEAKY_RELU, S_ELU, S_LEAKY_GRAD, S_COUNT };   // protocol.rs:226-232; S_LEAKY_GRAD: ops/scalar/mod.rs:149-166
 
 template <class T> inline typename std::enable_if<is_float<T>::value, bool>::type
 scalar_float_only(int op, T& x, T v) {
@@ -343,6 +343,9 @@ int scalar_impl(int op, T* buf, size_t buflen, T v, const Meta& m, int* path) {
         case S_DIV: rc = visit(buf, buflen, m, path, [v, &fault](T& x) { x = dvd(x, v, fault); }); break;
         case S_LEAKY_RELU:                                                            // cpu.rs:708-715
             rc = visit(buf, buflen, m, path, [v](T& x) { x = gt(x, consts<T>::zero()) ? x : mul(x, v); });
+            break;
+        case S_LEAKY_GRAD:                                                            // ops/scalar/mod.rs:152-160: 1 where input > 0, else the slope
+            rc = visit(buf, buflen, m, path, [v](T& x) { x = gt(x, consts<T>::zero()) ? consts<T>::one() : v; });
             break;
         case S_LOG: case S_LOG1P: case S_ELU:
             if (!is_float<T>::value) return ORC_E_DTYPE;

@@ -67,6 +67,10 @@ template <class T> __device__ __forceinline__ T zero_of() {
     if constexpr (is_bool<T>::value) return boolean_t{0};
     else return (T)0;
 }
+template <class T> __device__ __forceinline__ T one_of() {
+    if constexpr (is_bool<T>::value) return boolean_t{1};
+    else return (T)1;
+}
 
 // libm spellings per precision
 __device__ __forceinline__ float m_exp(float x) { return expf(x); }
@@ -167,6 +171,7 @@ template <int OP, class T> struct ScalarF {
         else if constexpr (OP == RT_S_LOG) return m_log(x) / m_log(v);                            // f32::log(base)
         else if constexpr (OP == RT_S_LOG1P) return m_log1p(x) / m_log(v);                        // core/value.rs vlog1p
         else if constexpr (OP == RT_S_ELU) return x >= (T)0 ? x : v * m_expm1(x);                 // cpu.rs:717-724
+        else if constexpr (OP == RT_S_LEAKY_GRAD) return gt0(x) ? one_of<T>() : v;                // ops/scalar/mod.rs:149-166
         else return x;
     }
 };
@@ -526,6 +531,7 @@ int32_t scalar_typed(rt_ctx* ctx, int op, void* buf, uint64_t buf_len, const voi
         case RT_S_SUB: return scalar_go<T, RT_S_SUB>(ctx, buf, buf_len, value, offset, rank, shape, strides);
         case RT_S_MUL: return scalar_go<T, RT_S_MUL>(ctx, buf, buf_len, value, offset, rank, shape, strides);
         case RT_S_LEAKY_RELU: return scalar_go<T, RT_S_LEAKY_RELU>(ctx, buf, buf_len, value, offset, rank, shape, strides);
+        case RT_S_LEAKY_GRAD: return scalar_go<T, RT_S_LEAKY_GRAD>(ctx, buf, buf_len, value, offset, rank, shape, strides);
         case RT_S_DIV:
             if constexpr (is_bool<T>::value) {
                 return rt_fail(RT_E_ARITH, "scalar div: division is not implemented for boolean in the reference (todo!())");

@@ -25,7 +25,7 @@ DTYPE_BY_NAME = {"u8": U8, "i8": I8, "u16": U16, "i16": I16, "u32": U32, "u128":
 UNARY = {n: i for i, n in enumerate(
     "neg relu sigmoid silu tanh abs sqrt ln expm1 ln1p floor ceil round trunc sin cos tan asin acos atan sinh cosh "
     "asinh acosh atanh rsqrt reciprocal square cube exp sign step abs_grad".split())}
-SCALAR = {n: i for i, n in enumerate("add sub mul div log log1p leaky_relu elu".split())}
+SCALAR = {n: i for i, n in enumerate("add sub mul div log log1p leaky_relu elu leaky_grad".split())}
 BINARY = {"add": 0, "sub": 1, "mul": 2, "div": 3}
 REDUCE = {"sum": 1, "prod": 2, "max": 3, "min": 4, "mean": 5}
 

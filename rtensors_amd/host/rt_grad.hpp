@@ -74,6 +74,31 @@ class GradContext {
         return Var{result, (int)nodes_.size() - 1};
     }
 
+    // ops/scalar/mod.rs:149-166: leaky_relu shares GradNode::ReLU; its map is 1 where input > 0 and the slope elsewhere
+    Var leaky_relu(const Var& a, double slope) {
+        Tensor result = a.t.owned();
+        Tensor gmap;
+        const bool track = a.node >= 0;
+        if (track) gmap = result.owned();
+        result.leaky_relu_inplace(slope);
+        if (!track) return Var{result, -1};
+        gmap.scalar_assign(RT_S_LEAKY_GRAD, slope);
+        return map_node(result, gmap, a.node);
+    }
+
+    // ops/unary/mod.rs:213-232: Abs keeps a map of +1 where input > 0 and -1 elsewhere; backwards_abs (backwards.rs:267-276)
+    // multiplies it into the upstream gradient exactly as backwards_relu does
+    Var abs(const Var& a) {
+        Tensor result = a.t.owned();
+        Tensor gmap;
+        const bool track = a.node >= 0;
+        if (track) gmap = result.owned();
+        result.abs_inplace();
+        if (!track) return Var{result, -1};
+        gmap.unary_inplace(RT_U_ABS_GRAD);
+        return map_node(result, gmap, a.node);
+    }
+
     // ops/broadcast/l1.rs:49-84 with ReductionType::Mean
     Var mean_l1_loss(const Var& y, const Var& target) {
         Tensor diff = y.t - target.t;
@@ -156,6 +181,15 @@ class GradContext {
                 g.set_meta(sq.meta());
             }
         }
+    }
+
+    Var map_node(const Tensor& result, const Tensor& gmap, int parent) {
+        Node n;
+        n.kind = NodeKind::ReLU;
+        n.parents = {parent};
+        n.grad_map = gmap;
+        nodes_.push_back(n);
+        return Var{result, (int)nodes_.size() - 1};
     }
 
     std::vector<Tensor> node_backwards(Node& n, const Tensor& up) {

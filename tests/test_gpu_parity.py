@@ -217,6 +217,42 @@ def test_scalar_and_fill_contiguous(hip, dtype):
     assert hip.dump(g).tobytes() == want.tobytes()
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f64", "i32", "i64", "i8"])
+def test_gradient_maps(hip, dtype):
+    """The three maps the reference's autograd fills with one get/set per element (ops/unary/mod.rs:213-252,
+    ops/scalar/mod.rs:149-166): relu -> x > 0 ? 1 : 0, abs -> x > 0 ? 1 : -1, leaky_relu -> x > 0 ? 1 : slope."""
+    rng = np.random.default_rng(21)
+    code = cpu.DTYPE_BY_NAME[dtype]
+    npd = cpu.NP_DTYPE[code]
+    n = 40_003
+    x = rand_values(dtype, n, rng)
+    if dtype[0] == "f":
+        x[:6] = [0.0, -0.0, np.nan, np.inf, -np.inf, np.finfo(npd).tiny / 2]
+    else:
+        x[:3] = [0, 1, -1]
+    slope = npd.type(0.125) if dtype[0] == "f" else npd.type(-3)
+    one = npd.type(1)
+    with np.errstate(invalid="ignore"):
+        pos = x > 0
+    cases = {"step": np.where(pos, one, npd.type(0)), "abs_grad": np.where(pos, one, npd.type(-1)), "leaky_grad": np.where(pos, one, slope)}
+    for name, full in cases.items():
+        full = full.astype(npd)
+        for (off, shape, strides) in (([0], [n], [1]), ([5], [(n - 5) // 3], [3]), ([n - 99], [200, 50], [-150, 2])):
+            m = MetaTensor(shape, strides, off[0])
+            want = x.copy()
+            idx = (off[0] + np.add.outer(*[np.arange(sz) * st for sz, st in zip(shape, strides)])).reshape(-1) if len(shape) == 2 \
+                else off[0] + np.arange(shape[0]) * strides[0]
+            want[idx] = full[idx]
+            g = hip.alloc_from_slice(code, x)
+            if name == "leaky_grad":
+                hip.scalar_nd(name, g, slope, m.offset, m.shape, m.strides)
+                chk = x.copy(); cpu.scalar(code, name, chk, slope, m)
+                assert chk.tobytes() == want.tobytes()
+            else:
+                hip.unary_nd(name, g, m.offset, m.shape, m.strides)
+            assert hip.dump(g).tobytes() == want.tobytes(), (name, shape, strides)
+
+
 @pytest.mark.parametrize("dtype", ["f32", "f64", "i32", "u8", "i64", "i16"])
 def test_inplace_ops_over_random_views(hip, dtype):
     rng = np.random.default_rng(4)

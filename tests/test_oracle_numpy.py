@@ -167,6 +167,24 @@ def test_special_values(oracle_lib):
     assert i.unary("relu").buf.tolist() == [0, 0, 0, 7]
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f64", "i32", "i64", "u8"])
+def test_leaky_relu_gradient_map(dtype, oracle_lib):
+    # ops/scalar/mod.rs:149-166: `if val > 0 { 1 } else { scalar }`, element by element
+    npd = cpu.NP_DTYPE[cpu.DTYPE_BY_NAME[dtype]]
+    x = np.array([3, 0, 1, 0, 7, 2, 0, 9], dtype=npd) if dtype == "u8" else np.array([3, -2, 0, -0.0, 7, -9, 1, -1], dtype=npd)
+    s = npd.type(0.25) if dtype[0] == "f" else npd.type(5)
+    if dtype[0] == "f":
+        x[5] = np.nan                                        # NaN > 0 is false -> slope
+    t = OTensor.from_buf(dtype, x, [8])
+    got = t.scalar_op_inplace("leaky_grad", s).buf
+    want = np.where(x > 0, npd.type(1), s).astype(npd)
+    assert got.tobytes() == want.tobytes()
+    v = OTensor.from_buf(dtype, x, [8]).slice(0, Slice(None, None, -3))      # elements 7, 4, 1 through a reversed view
+    v.scalar_op_inplace("leaky_grad", s)
+    want2 = x.copy(); want2[[7, 4, 1]] = want[[7, 4, 1]]
+    assert v.buf.tobytes() == want2.tobytes()
+
+
 @pytest.mark.parametrize("dtype", ["f32", "f64"])
 def test_transcendental_unary_within_reference_tolerance(dtype, oracle_lib):
     # bit parity of these is unpinned (platform libm on both sides); the reference's own tests use 1e-5
