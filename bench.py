@@ -240,6 +240,40 @@ def time_kernel(hip, fn, iters, warmup):
     return float(np.mean(times)), float(np.median(times)), float(np.min(times))
 
 
+def api_overhead(hip):
+    """Host-side cost of the calls around the kernels, in microseconds per call as seen from this process (the ctypes hop,
+    roughly 1-2 us, is included): a cached allocate + free, the asynchronous enqueue of an elementwise, a broadcast and an
+    axis-reduce call on tiny operands, and the launch-to-completion round trip of one tiny call."""
+    from rtensors_amd import hip as H
+    n = 2000
+    out = {}
+    b = hip.alloc(H.F32, 1 << 18); del b
+    hip.sync()
+    t0 = time.perf_counter()
+    for _ in range(n):
+        b = hip.alloc_uninit(H.F32, 1 << 18); del b
+    out["alloc_free_cached_1MiB_us"] = round((time.perf_counter() - t0) / n * 1e6, 2)
+    a = hip.alloc(H.F32, 64); c = hip.alloc(H.F32, 64 * 64); r = hip.alloc(H.F32, 64)
+    shape = [64, 64]
+    calls = {
+        "enqueue_scalar_contiguous_us": lambda: hip.scalar_contiguous("add", a, 1.0, 0, 64),
+        "enqueue_broadcast_rank2_us": lambda: hip.broadcast((a, (0, shape, [0, 1])), (a, (0, shape, [1, 0])), (c, (0, shape, [64, 1])), "add"),
+        "enqueue_reduce_axis_us": lambda: hip.apply_reduce_contiguous_nd((c, (0, shape, [64, 1])), r, 1, "sum"),
+    }
+    for name, fn in calls.items():
+        fn(); hip.sync()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        out[name] = round((time.perf_counter() - t0) / n * 1e6, 2)
+        hip.sync()
+    t0 = time.perf_counter()
+    for _ in range(200):
+        hip.scalar_contiguous("add", a, 1.0, 0, 64); hip.sync()
+    out["round_trip_tiny_call_plus_sync_us"] = round((time.perf_counter() - t0) / 200 * 1e6, 2)
+    return out
+
+
 def cpu_baseline():
     """The CPU oracle (C++ restatement of the reference's single-threaded Cpu backend) timed on a bounded sample of the
     headline step: 4 of the 16 batch slices of the config-3 broadcast add, and the whole config-4 axis sum."""
@@ -332,6 +366,8 @@ def main():
             detail[name] = {"ms": round(mean, 4), "GBps": round(nbytes / (mean * 1e-3) / 1e9, 1),
                             "frac": round(nbytes / (mean * 1e-3) / PEAK_HBM, 4), "Gelem_s": round(nelem / (mean * 1e-3) / 1e9, 2)}
     w.drop()
+    if not args.no_detail:
+        detail["api_overhead"] = api_overhead(hip)
 
     out = {
         "metric": "achieved HBM GB/s (% of peak) for broadcast-add + axis-sum, f32, 1 MI355X",
