@@ -27,7 +27,7 @@ PEAK_HBM = 8.0e12   # bytes/s, MI355X HBM3E
 # HBM bytes per launch of the config-3 broadcast-add kernel, from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE, each
 # scaled by what the same counter reads for the 1 GiB copy kernel (x2.000 and x1.000); see
 # profiles/bin_rows_kernel_config3_broadcast_add.txt.  Algorithmic bytes are 2181300224: nothing is re-read.
-MEASURED_TRAFFIC_C3A = 2181208987
+MEASURED_TRAFFIC_C3A = 2181097179
 
 
 def row_major(shape):
@@ -212,7 +212,7 @@ class Workloads:
 HEADLINE = ["c3a_add", "c4_sum1"]
 DETAIL = ["copy", "fill", "c1_add", "c1_sum1", "c2_mul", "c2_add", "c2_relu", "c2_sub", "c2_f64_mul", "c2_f64_add", "c2_i32_mul", "c2_i32_add",
           "c3a_add", "c3b_add", "c4_sum1", "c4_mean1", "c4_max1", "c4_sum0", "c4_sum_all", "c4_i32_sum1", "c4_i32_max1", "c4_i32_min0",
-          "c5_bias_add", "c5_colsum"]
+          "c5_bias_add", "c5_colsum", "view_relu", "tr_add"]
 KIND = {"copy": "elementwise", "fill": "elementwise"}
 
 
