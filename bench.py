@@ -177,6 +177,14 @@ class Workloads:
         return (lambda: self.hip.broadcast((a, (0, shape, [n, 1])), (b, (0, shape, [1, n])), (c, (0, shape, [n, 1])), "add")), 3 * n * n * 4, n * n
 
     # ---- config 1 -------------------------------------------------------------------------------------------------------------
+    def tr_copy(self):
+        """Row-major copy of a transposed 16384 x 16384 f32 view (`contiguous()` of `m.transpose()`)."""
+        H = self.H
+        n = 16384
+        a = self._gen("c2a", H.F32, n * n, "normal", 1, 0)
+        c = self._out("c2cf32", H.F32, n * n)
+        return (lambda: self.hip.gather(a, (0, [n, n], [1, n]), c)), 2 * n * n * 4, n * n
+
     def c1_add(self):
         H = self.H
         a = self._gen("c1a", H.F32, 4096, "uniform", 0, 0); b = self._gen("c1b", H.F32, 4096, "uniform", 0, 1)
@@ -212,7 +220,7 @@ class Workloads:
 HEADLINE = ["c3a_add", "c4_sum1"]
 DETAIL = ["copy", "fill", "c1_add", "c1_sum1", "c2_mul", "c2_add", "c2_relu", "c2_sub", "c2_f64_mul", "c2_f64_add", "c2_i32_mul", "c2_i32_add",
           "c3a_add", "c3b_add", "c4_sum1", "c4_mean1", "c4_max1", "c4_sum0", "c4_sum_all", "c4_i32_sum1", "c4_i32_max1", "c4_i32_min0",
-          "c5_bias_add", "c5_colsum", "view_relu", "tr_add"]
+          "c5_bias_add", "c5_colsum", "view_relu", "tr_add", "tr_copy"]
 KIND = {"copy": "elementwise", "fill": "elementwise"}
 
 

@@ -14,58 +14,11 @@
 //            blockIdx by multiply-high division on the scalar unit; no per-element index arithmetic.
 //   generic: anything else, one element per lane, per-element multiply-high index decomposition.
 // Algorithmic traffic: (|left|_unique + |right|_unique + N) * sizeof(T).
-#include "rt_common.h"
+#include "rt_broadcast_common.h"
 
-#include <type_traits>
+using namespace rtb;
 
 namespace {
-
-struct boolean_t { uint8_t v; };
-template <class T> struct is_flt : std::integral_constant<bool, std::is_same<T, float>::value || std::is_same<T, double>::value> {};
-template <class T> struct is_bool : std::is_same<T, boolean_t> {};
-
-typedef unsigned __int128 u128_t;
-template <class T, class E = void> struct carrier { typedef T type; };
-template <class T> struct carrier<T, typename std::enable_if<std::is_integral<T>::value && sizeof(T) <= 4>::type> { typedef uint32_t type; };
-template <class T> struct carrier<T, typename std::enable_if<std::is_integral<T>::value && sizeof(T) == 8>::type> { typedef uint64_t type; };
-
-// ops/base.rs:27-37 on T; integers wrap (release build), integer division truncates toward zero
-constexpr int kOpCopy = 4;      // internal: dst = left (strided gather); right is ignored
-
-template <int OP, class T> __device__ __forceinline__ T bin_apply(T a, T b) {
-    if constexpr (OP == kOpCopy) {
-        return a;
-    } else if constexpr (is_flt<T>::value) {
-        if constexpr (OP == RT_ADD) return a + b;
-        else if constexpr (OP == RT_SUB) return a - b;
-        else if constexpr (OP == RT_MUL) return a * b;
-        else return a / b;
-    } else if constexpr (is_bool<T>::value) {
-        if constexpr (OP == RT_ADD) return boolean_t{(uint8_t)(a.v | b.v)};            // core/value.rs:708-713 (OR)
-        else if constexpr (OP == RT_SUB) return boolean_t{(uint8_t)(a.v ^ b.v)};       // core/value.rs:715-720 (XOR)
-        else return boolean_t{(uint8_t)(a.v & b.v)};                                   // core/value.rs:722-727 (AND)
-    } else {
-        typedef typename carrier<T>::type W;
-        if constexpr (OP == RT_ADD) return (T)(W)((W)a + (W)b);
-        else if constexpr (OP == RT_SUB) return (T)(W)((W)a - (W)b);
-        else if constexpr (OP == RT_MUL) return (T)(W)((W)a * (W)b);
-        else {
-            // the reference panics on b == 0 and MIN / -1; the device yields 0 and MIN there and raises no error
-            if (b == 0) return (T)0;
-            if constexpr (std::is_signed<T>::value) {
-                if (b == (T)-1) return (T)(W)((W)0 - (W)a);
-            }
-            return (T)(a / b);
-        }
-    }
-}
-
-template <class T> struct alignas(16) Vec16 { T e[16 / sizeof(T)]; };
-
-constexpr int kBlock = 256;     // generic kernels
-constexpr int kRBlock = 128;    // contig / rows kernels: small blocks, one 16-byte vector per lane per step
-
-enum Mode : int { M_VEC = 0, M_BCAST = 1, M_ELEM = 2 };
 
 // ---- contig ---------------------------------------------------------------------------------------------------------
 // One vector per lane, non-temporal loads and stores: every byte is touched exactly once.
@@ -99,24 +52,6 @@ struct RowArgs {
     int64_t gstride[3];
     int64_t istride[2];             // inner strides of left, right (dst: 1)
 };
-
-template <class T, int MODE>
-__device__ __forceinline__ Vec16<T> load_vec(const T* __restrict__ rowp, uint32_t c, int64_t istride, bool nt) {
-    constexpr int N = 16 / sizeof(T);
-    Vec16<T> v;
-    if constexpr (MODE == M_VEC) {
-        const Vec16<T>* q = reinterpret_cast<const Vec16<T>*>(rowp + c);
-        v = nt ? rt_ld16_nt(q) : rt_ld16(q);
-    } else if constexpr (MODE == M_BCAST) {
-        T x = rowp[0];
-#pragma unroll
-        for (int j = 0; j < N; ++j) v.e[j] = x;
-    } else {
-#pragma unroll
-        for (int j = 0; j < N; ++j) v.e[j] = rowp[(int64_t)(c + j) * istride];
-    }
-    return v;
-}
 
 template <class T, int OP, int LM, int RM, int GU>
 __global__ __launch_bounds__(kRBlock) void bin_rows_kernel(const T* l, const T* r, T* d, RowArgs a) {
@@ -212,146 +147,6 @@ __global__ __launch_bounds__(kRBlock) void bin_rows_kernel(const T* l, const T* 
     }
 }
 
-// ---- tile (one operand transposed) ---------------------------------------------------------------------------------------
-// One input has its unit-|stride| dim somewhere other than dst's inner dim (a permuted, possibly reversed view): reading
-// it along dst's inner dim would touch one cache line per element.  A block instead gathers a (kTK x TL) tile of it with
-// lanes running along *its* unit-stride dim `t` (one 128-byte line per 32 lanes), transposes through LDS, keeps its
-// share of the tile in registers, and then walks the loop dim g (an outer dim along which that operand does not move,
-// if there is one) writing full rows of dst with 16-byte non-temporal stores.
-constexpr int kTBlock = 256;
-constexpr int kTK = 32;                      // tile extent along the transposed operand's unit-stride dim
-constexpr int kTRows = kTK / (kTBlock / RT_WAVE);   // rows of the tile each lane keeps (8)
-
-struct TileArgs {
-    uint32_t L, K, G;               // inner length, extent of dim t, extent of the loop dim (1 if none)
-    uint32_t gchunk, nchunks, ktiles, ltiles;
-    FastDiv32 ltiles_div, ktiles_div, nchunks_div;
-    int nouter;
-    uint32_t oshape[RT_MAX_RANK];
-    FastDiv32 odiv[RT_MAX_RANK];
-    int64_t ostride[3][RT_MAX_RANK];
-    int64_t gstride[3], tstride[3], istride[3];   // per operand (0 left, 1 right, 2 dst): loop dim, dim t, inner dim
-    uint32_t nt_other;              // the non-transposed input is streamed -> non-temporal loads
-};
-
-// XT = index (0/1) of the transposed input; OM = access mode of the other input along the inner dim.
-template <class T, int OP, int XT, int OM>
-__global__ __launch_bounds__(kTBlock) void bin_tile_kernel(const T* l, const T* r, T* d, TileArgs a) {
-    constexpr int N = 16 / sizeof(T);
-    constexpr int TL = RT_WAVE * N;           // tile extent along dst's inner dim: one 16-byte vector per lane of a wave
-    __shared__ alignas(16) T tile[kTK][TL + N];
-    uint32_t b = blockIdx.x;
-    uint32_t q = fd_div(b, a.ltiles_div);
-    const uint32_t ltile = b - q * a.ltiles;
-    b = q;
-    q = fd_div(b, a.ktiles_div);
-    const uint32_t ktile = b - q * a.ktiles;
-    b = q;
-    q = fd_div(b, a.nchunks_div);
-    const uint32_t chunk = b - q * a.nchunks;
-    uint32_t rem = q;
-    int64_t off[3] = {0, 0, 0};
-#pragma unroll
-    for (int k = RT_MAX_RANK - 1; k >= 0; --k) {
-        if (k < a.nouter) {
-            uint32_t qq = fd_div(rem, a.odiv[k]);
-            uint32_t c = rem - qq * a.oshape[k];
-#pragma unroll
-            for (int o = 0; o < 3; ++o) off[o] += (int64_t)c * a.ostride[o][k];
-            rem = qq;
-        }
-    }
-    const T* xt = (XT == 0 ? l : r) + off[XT];
-    const T* xo = (XT == 0 ? r : l) + off[1 - XT];
-    constexpr int O = 1 - XT;
-    T* dp = d + off[2];
-    const uint32_t k0 = ktile * kTK, l0 = ltile * TL;
-    const uint32_t g_begin = chunk * a.gchunk;
-    const uint32_t g_end = min(a.G, g_begin + a.gchunk);
-    const bool xt_fixed = a.gstride[XT] == 0;
-
-    const uint32_t lane = threadIdx.x & (RT_WAVE - 1), wv = threadIdx.x / RT_WAVE;
-    const uint32_t c = l0 + lane * N;                        // first inner column of this lane's vectors
-    Vec16<T> xv[kTRows];
-    Vec16<T> ov[kTRows];                                     // other operand, fetched one loop step ahead
-
-    const bool o_fixed = a.tstride[O] == 0;
-    if (c + N <= a.L && g_begin < g_end) {
-        // first step's rows of the other operand: issued before the gather so that both are in flight together
-        const T* orow0 = xo + (int64_t)g_begin * a.gstride[O];
-#pragma unroll
-        for (int i = 0; i < kTRows; ++i) {
-            const uint32_t k = min(k0 + wv + i * (kTBlock / RT_WAVE), a.K - 1);
-            if (i == 0 || !o_fixed) ov[i] = load_vec<T, OM>(orow0 + (int64_t)k * a.tstride[O], c, a.istride[O], a.nt_other != 0);
-        }
-    }
-
-    for (uint32_t g = g_begin; g < g_end; ++g) {
-        if (g == g_begin || !xt_fixed) {
-            if (g != g_begin) __syncthreads();
-            // gather: lanes along dim t (32 consecutive lanes read one 128-byte line of the transposed operand); each
-            // lane collects the N elements of one 16-byte group of a tile row, all loads in flight before the first LDS
-            // write, and writes the group with one 16-byte LDS store (row stride = 4 words mod 32: conflict free).
-            const uint32_t tk = threadIdx.x % kTK, grp0 = threadIdx.x / kTK;
-            constexpr int kGroupsPerLane = RT_WAVE / (kTBlock / kTK);          // 64 groups per row / 8 lanes-rows = 8
-            const T* src = xt + (int64_t)g * a.gstride[XT] + (int64_t)min(k0 + tk, a.K - 1) * a.tstride[XT];
-            Vec16<T> grp[kGroupsPerLane];
-#pragma unroll
-            for (int i = 0; i < kGroupsPerLane; ++i) {
-                const uint32_t col = l0 + (grp0 + i * (kTBlock / kTK)) * N;
-#pragma unroll
-                for (int j = 0; j < N; ++j) grp[i].e[j] = src[(int64_t)min(col + j, a.L - 1) * a.istride[XT]];
-            }
-#pragma unroll
-            for (int i = 0; i < kGroupsPerLane; ++i)
-                *reinterpret_cast<Vec16<T>*>(&tile[tk][(grp0 + i * (kTBlock / kTK)) * N]) = grp[i];
-            __syncthreads();
-#pragma unroll
-            for (int i = 0; i < kTRows; ++i) xv[i] = *reinterpret_cast<const Vec16<T>*>(&tile[wv + i * (kTBlock / RT_WAVE)][lane * N]);
-        }
-        if (c >= a.L) continue;
-        const T* orow = xo + (int64_t)g * a.gstride[O];
-        T* drow = dp + (int64_t)g * a.gstride[2];
-        if (c + N <= a.L) {
-            // Loads and stores retire in issue order on this hardware, so waiting for a load that was issued after a
-            // batch of stores also waits for those stores to be acknowledged.  The other operand is therefore fetched one
-            // loop step ahead: its wait only covers loads.
-            Vec16<T> cur[kTRows];
-#pragma unroll
-            for (int i = 0; i < kTRows; ++i) cur[i] = ov[o_fixed ? 0 : i];
-            if (g + 1 < g_end && a.gstride[O] != 0) {
-                const T* nrow = xo + (int64_t)(g + 1) * a.gstride[O];
-#pragma unroll
-                for (int i = 0; i < kTRows; ++i) {
-                    const uint32_t k = min(k0 + wv + i * (kTBlock / RT_WAVE), a.K - 1);
-                    if (i == 0 || !o_fixed) ov[i] = load_vec<T, OM>(nrow + (int64_t)k * a.tstride[O], c, a.istride[O], a.nt_other != 0);
-                }
-            }
-#pragma unroll
-            for (int i = 0; i < kTRows; ++i) {
-                const uint32_t k = k0 + wv + i * (kTBlock / RT_WAVE);
-                if (k < a.K) {
-                    Vec16<T> out;
-#pragma unroll
-                    for (int j = 0; j < N; ++j) out.e[j] = XT == 0 ? bin_apply<OP, T>(xv[i].e[j], cur[i].e[j]) : bin_apply<OP, T>(cur[i].e[j], xv[i].e[j]);
-                    rt_st16_nt(reinterpret_cast<Vec16<T>*>(drow + (int64_t)k * a.tstride[2] + c), out);
-                }
-            }
-        } else {
-            for (int i = 0; i < kTRows; ++i) {
-                const uint32_t k = k0 + wv + i * (kTBlock / RT_WAVE);
-                if (k < a.K) {
-                    for (uint32_t cc = c; cc < a.L; ++cc) {
-                        T xe = xv[i].e[cc - c];
-                        T oe = (orow + (int64_t)k * a.tstride[O])[(int64_t)cc * a.istride[O]];
-                        drow[(int64_t)k * a.tstride[2] + cc] = XT == 0 ? bin_apply<OP, T>(xe, oe) : bin_apply<OP, T>(oe, xe);
-                    }
-                }
-            }
-        }
-    }
-}
-
 // ---- generic ------------------------------------------------------------------------------------------------------------
 struct GenArgs {
     int rank;
@@ -427,18 +222,6 @@ void launch_rows(int lm, int rm, bool batched, dim3 grid, hipStream_t s, const T
     }
 }
 
-static inline bool mult_of(int64_t v, int64_t n) { return v % n == 0; }
-
-// Can operand `o` be read with aligned 16-byte loads at every (outer, g, column-vector) position?
-template <class T>
-static bool vec_ok(const T* base, const NdDesc& dsc, int o) {
-    constexpr int64_t N = 16 / sizeof(T);
-    if ((reinterpret_cast<uintptr_t>(base + dsc.offset[o]) & 15) != 0) return false;
-    for (int k = 0; k < dsc.rank - 1; ++k)
-        if (!mult_of(dsc.stride[o][k], N)) return false;
-    return true;
-}
-
 template <class T, int OP>
 int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const void* lv, const void* rv, void* dv) {
     const T* l = (const T*)lv;
@@ -484,84 +267,10 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
         }
     }
 
-    // (2a) tile: exactly one input is "transposed" (inner stride neither 0 nor 1, unit |stride| along another dim)
-    if (OP != kOpCopy && rank >= 2 && count < (1ull << 31) && dsc.stride[2][rank - 1] == 1 && dsc.shape[rank - 1] >= 2 * N && vec_ok<T>(d, dsc, 2)) {
-        auto transposed_dim = [&](int o) -> int {
-            int64_t is = dsc.stride[o][rank - 1];
-            if (is == 0 || is == 1) return -1;
-            for (int k = rank - 2; k >= 0; --k)
-                if ((dsc.stride[o][k] == 1 || dsc.stride[o][k] == -1) && dsc.shape[k] >= 16) return k;
-            return -1;
-        };
-        const int tl = transposed_dim(0), tr = transposed_dim(1);
-        // When the transposed input does not move along some long outer dim, the row kernel gathers it once per block
-        // and reuses it from registers for 16 output rows, which measured faster than the tile kernel; the tile kernel
-        // is for the case without such reuse (e.g. a + b.transpose()).
-        auto hoistable = [&](int o) {
-            for (int k = 0; k < rank - 1; ++k)
-                if (dsc.stride[o][k] == 0 && dsc.shape[k] >= 8) return true;
-            return false;
-        };
-        if ((tl >= 0) != (tr >= 0) && !hoistable(tl >= 0 ? 0 : 1)) {
-            const int xt = tl >= 0 ? 0 : 1, o = 1 - xt, tdim = tl >= 0 ? tl : tr;
-            int om;
-            {
-                int64_t is = dsc.stride[o][rank - 1];
-                const T* base = o == 0 ? l : r;
-                om = is == 0 ? (int)M_BCAST : ((is == 1 && vec_ok<T>(base, dsc, o)) ? (int)M_VEC : (int)M_ELEM);
-            }
-            TileArgs a;
-            memset(&a, 0, sizeof(a));
-            a.L = (uint32_t)dsc.shape[rank - 1];
-            a.K = (uint32_t)dsc.shape[tdim];
-            int gdim = -1;
-            for (int k = 0; k < rank - 1; ++k)
-                if (k != tdim && dsc.stride[xt][k] == 0 && (gdim < 0 || dsc.shape[k] > dsc.shape[gdim])) gdim = k;
-            a.G = gdim >= 0 ? (uint32_t)dsc.shape[gdim] : 1;
-            for (int q = 0; q < 3; ++q) {
-                a.gstride[q] = gdim >= 0 ? dsc.stride[q][gdim] : 0;
-                a.tstride[q] = dsc.stride[q][tdim];
-                a.istride[q] = dsc.stride[q][rank - 1];
-            }
-            uint64_t outer = 1;
-            for (int k = 0; k < rank - 1; ++k) {
-                if (k == gdim || k == tdim) continue;
-                a.oshape[a.nouter] = (uint32_t)dsc.shape[k];
-                a.odiv[a.nouter] = make_fastdiv((uint32_t)dsc.shape[k]);
-                for (int q = 0; q < 3; ++q) a.ostride[q][a.nouter] = dsc.stride[q][k];
-                outer *= (uint64_t)dsc.shape[k];
-                a.nouter++;
-            }
-            for (int k = a.nouter; k < RT_MAX_RANK; ++k) { a.oshape[k] = 1; a.odiv[k] = make_fastdiv(1); }
-            const uint32_t TL = RT_WAVE * (uint32_t)N;
-            a.ktiles = (a.K + kTK - 1) / kTK;
-            a.ltiles = (a.L + TL - 1) / TL;
-            // loop-dim steps per block: the gathered tile is reused for all of them; keep enough blocks to fill the chip
-            uint32_t gchunk = a.G;
-            const uint64_t want_blocks = (uint64_t)ctx->num_cus * 16;
-            while (gchunk > 8 && outer * a.ktiles * a.ltiles * ((a.G + gchunk - 1) / gchunk) < want_blocks) gchunk = (gchunk + 1) / 2;
-            a.gchunk = gchunk;
-            a.nchunks = (a.G + gchunk - 1) / gchunk;
-            a.ltiles_div = make_fastdiv(a.ltiles);
-            a.ktiles_div = make_fastdiv(a.ktiles);
-            a.nchunks_div = make_fastdiv(a.nchunks);
-            bool streamed = true;
-            for (int k = 0; k < rank; ++k) streamed = streamed && dsc.stride[o][k] != 0;
-            a.nt_other = streamed ? 1u : 0u;
-            const uint64_t blocks = outer * a.nchunks * a.ktiles * a.ltiles;
-            if (blocks < (1ull << 31)) {
-                const T* lp = l + dsc.offset[0];
-                const T* rp = r + dsc.offset[1];
-                T* dp = d + dsc.offset[2];
-                dim3 grid((unsigned)blocks), blk(kTBlock);
-#define RT_TILE(XT, OM) hipLaunchKernelGGL((bin_tile_kernel<T, OP, XT, OM>), grid, blk, 0, s, lp, rp, dp, a)
-                if (xt == 0) { if (om == M_VEC) RT_TILE(0, M_VEC); else if (om == M_BCAST) RT_TILE(0, M_BCAST); else RT_TILE(0, M_ELEM); }
-                else         { if (om == M_VEC) RT_TILE(1, M_VEC); else if (om == M_BCAST) RT_TILE(1, M_BCAST); else RT_TILE(1, M_ELEM); }
-#undef RT_TILE
-                RT_HIP(hipGetLastError());
-                return RT_OK;
-            }
-        }
+    // (2a) tile: exactly one input is "transposed" (rt_broadcast_tile.hip)
+    {
+        int32_t status = RT_OK;
+        if (tile_try<T, OP>(ctx, dsc, count, l, r, d, &status)) return status;
     }
 
     // (2) rows: dst inner dim unit-stride, rows 16-byte aligned, everything indexable in 32 bits

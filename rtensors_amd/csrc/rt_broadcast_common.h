@@ -1,0 +1,95 @@
+// Shared by the broadcast translation units (rt_broadcast.hip: planning, contiguous / row / generic kernels;
+// rt_broadcast_tile.hip: the LDS-transpose kernel): element types, the binary op on T, 16-byte vectors, operand access modes.
+#pragma once
+
+#include "rt_common.h"
+
+#include <type_traits>
+
+namespace rtb {
+
+struct boolean_t { uint8_t v; };
+template <class T> struct is_flt : std::integral_constant<bool, std::is_same<T, float>::value || std::is_same<T, double>::value> {};
+template <class T> struct is_bool : std::is_same<T, boolean_t> {};
+
+typedef unsigned __int128 u128_t;
+template <class T, class E = void> struct carrier { typedef T type; };
+template <class T> struct carrier<T, typename std::enable_if<std::is_integral<T>::value && sizeof(T) <= 4>::type> { typedef uint32_t type; };
+template <class T> struct carrier<T, typename std::enable_if<std::is_integral<T>::value && sizeof(T) == 8>::type> { typedef uint64_t type; };
+
+// ops/base.rs:27-37 on T; integers wrap (release build), integer division truncates toward zero
+constexpr int kOpCopy = 4;      // internal: dst = left (strided gather); right is ignored
+
+template <int OP, class T> __device__ __forceinline__ T bin_apply(T a, T b) {
+    if constexpr (OP == kOpCopy) {
+        return a;
+    } else if constexpr (is_flt<T>::value) {
+        if constexpr (OP == RT_ADD) return a + b;
+        else if constexpr (OP == RT_SUB) return a - b;
+        else if constexpr (OP == RT_MUL) return a * b;
+        else return a / b;
+    } else if constexpr (is_bool<T>::value) {
+        if constexpr (OP == RT_ADD) return boolean_t{(uint8_t)(a.v | b.v)};            // core/value.rs:708-713 (OR)
+        else if constexpr (OP == RT_SUB) return boolean_t{(uint8_t)(a.v ^ b.v)};       // core/value.rs:715-720 (XOR)
+        else return boolean_t{(uint8_t)(a.v & b.v)};                                   // core/value.rs:722-727 (AND)
+    } else {
+        typedef typename carrier<T>::type W;
+        if constexpr (OP == RT_ADD) return (T)(W)((W)a + (W)b);
+        else if constexpr (OP == RT_SUB) return (T)(W)((W)a - (W)b);
+        else if constexpr (OP == RT_MUL) return (T)(W)((W)a * (W)b);
+        else {
+            // the reference panics on b == 0 and MIN / -1; the device yields 0 and MIN there and raises no error
+            if (b == 0) return (T)0;
+            if constexpr (std::is_signed<T>::value) {
+                if (b == (T)-1) return (T)(W)((W)0 - (W)a);
+            }
+            return (T)(a / b);
+        }
+    }
+}
+
+template <class T> struct alignas(16) Vec16 { T e[16 / sizeof(T)]; };
+
+constexpr int kBlock = 256;     // generic kernels
+constexpr int kRBlock = 128;    // contig / rows kernels: small blocks, one 16-byte vector per lane per step
+
+enum Mode : int { M_VEC = 0, M_BCAST = 1, M_ELEM = 2 };
+
+template <class T, int MODE>
+__device__ __forceinline__ Vec16<T> load_vec(const T* __restrict__ rowp, uint32_t c, int64_t istride, bool nt) {
+    constexpr int N = 16 / sizeof(T);
+    Vec16<T> v;
+    if constexpr (MODE == M_VEC) {
+        const Vec16<T>* q = reinterpret_cast<const Vec16<T>*>(rowp + c);
+        v = nt ? rt_ld16_nt(q) : rt_ld16(q);
+    } else if constexpr (MODE == M_BCAST) {
+        T x = rowp[0];
+#pragma unroll
+        for (int j = 0; j < N; ++j) v.e[j] = x;
+    } else {
+#pragma unroll
+        for (int j = 0; j < N; ++j) v.e[j] = rowp[(int64_t)(c + j) * istride];
+    }
+    return v;
+}
+
+static inline bool mult_of(int64_t v, int64_t n) { return v % n == 0; }
+
+// Can operand `o` be read with aligned 16-byte loads at every (outer, g, column-vector) position?
+template <class T>
+static bool vec_ok(const T* base, const NdDesc& dsc, int o) {
+    constexpr int64_t N = 16 / sizeof(T);
+    if ((reinterpret_cast<uintptr_t>(base + dsc.offset[o]) & 15) != 0) return false;
+    for (int k = 0; k < dsc.rank - 1; ++k)
+        if (!mult_of(dsc.stride[o][k], N)) return false;
+    return true;
+}
+
+// Launches the LDS-transpose kernel when the operation fits it: exactly one input is "transposed" (its inner stride is
+// neither 0 nor 1 and it has unit |stride| along another dim) and there is no long stride-0 dim over which the row kernel
+// could hoist it.  Returns true when the operation was taken (then *status is its result), false when another kernel
+// should run it.  Instantiated in rt_broadcast_tile.hip for every (T, OP) that rt_broadcast.hip uses.
+template <class T, int OP>
+bool tile_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* l, const T* r, T* d, int32_t* status);
+
+}  // namespace rtb

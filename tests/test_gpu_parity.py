@@ -480,6 +480,28 @@ def test_gather_views(hip):
             assert gv.to_numpy().tobytes() == ov.to_numpy().tobytes(), (dtype, ov.meta)
 
 
+@pytest.mark.parametrize("dtype", ["f32", "u8", "i16", "f64"])
+def test_gather_transposed_views(hip, dtype):
+    """Row-major copy (`owned()` / `contiguous()`) of permuted, reversed and stepped views large enough for the
+    LDS-transpose copy kernel, with ragged tile edges."""
+    rng = np.random.default_rng(17)
+    for shape in [(64, 257), (3, 40, 70), (2, 5, 33, 130), (4, 17, 1030), (100, 36), (2, 3, 16, 16), (7, 300, 9)]:
+        r = len(shape)
+        vals = rand_values(dtype, int(np.prod(shape)), rng)
+        o, g = OTensor.from_buf(dtype, vals, list(shape)), G(hip, dtype, vals, list(shape))
+        perms = [list(range(r - 2)) + [r - 1, r - 2]]
+        if r >= 3:
+            perms.append([r - 1] + list(range(1, r - 1)) + [0])
+        for perm in perms:
+            for variant in range(3):
+                ov, gv = o.permute(perm), g.permute(perm)
+                if variant == 1:
+                    ov, gv = ov.slice(r - 2, Slice(None, None, -1)), gv.slice(r - 2, Slice(None, None, -1))
+                if variant == 2:
+                    ov, gv = ov.slice(r - 1, Slice(1, None, 2)), gv.slice(r - 1, Slice(1, None, 2))
+                assert gv.contiguous().dump().tobytes() == ov.to_numpy().tobytes(), (dtype, shape, perm, variant)
+
+
 def test_convert(hip):
     from rtensors_amd import hip as H
     rng = np.random.default_rng(8)
