@@ -176,6 +176,23 @@ class Workloads:
         shape = [n, n]
         return (lambda: self.hip.broadcast((a, (0, shape, [n, 1])), (b, (0, shape, [1, n])), (c, (0, shape, [n, 1])), "add")), 3 * n * n * 4, n * n
 
+    # ---- matmul (behind the same trait; MFMA-bound, not part of the headline) ---------------------------------------------------------
+    def _mm(self, dtype_name, n):
+        H = self.H
+        dt = H.DTYPE_BY_NAME[dtype_name]
+        dist = "normal" if dtype_name[0] == "f" else "int"
+        a = self._gen(f"mma_{dtype_name}", dt, n * n, dist, 7, 0, -1000, 1000) if dist == "int" else self._gen(f"mma_{dtype_name}", dt, n * n, dist, 7, 0)
+        b = self._gen(f"mmb_{dtype_name}", dt, n * n, dist, 7, 1, -1000, 1000) if dist == "int" else self._gen(f"mmb_{dtype_name}", dt, n * n, dist, 7, 1)
+        c = self._out(f"mmc_{dtype_name}", dt, n * n)
+        meta = (0, [n, n], [n, 1])
+        fn = lambda: self.hip.matmul((a, meta, "row_major"), (b, meta, "row_major"), c, 1, n, n, n)
+        fn.flops = 2 * n ** 3
+        return fn, 3 * n * n * H.NP_DTYPE[dt].itemsize, n * n
+
+    def mm_f32(self): return self._mm("f32", 8192)
+    def mm_f64(self): return self._mm("f64", 4096)
+    def mm_i32(self): return self._mm("i32", 4096)
+
     # ---- config 1 -------------------------------------------------------------------------------------------------------------
     def tr_copy(self):
         """Row-major copy of a transposed 16384 x 16384 f32 view (`contiguous()` of `m.transpose()`)."""
@@ -338,8 +355,11 @@ def main():
         fn, nbytes, nelem = getattr(w, args.kernel)()
         preheat(hip, [fn], args.preheat)
         mean, med, mn = time_kernel(hip, fn, args.steps, args.warmup)
-        print(json.dumps({"kernel": args.kernel, "ms_mean": mean, "ms_median": med, "ms_min": mn, "bytes": nbytes,
-                          "GBps": nbytes / (mean * 1e-3) / 1e9, "frac_of_peak": nbytes / (mean * 1e-3) / PEAK_HBM}))
+        rec = {"kernel": args.kernel, "ms_mean": mean, "ms_median": med, "ms_min": mn, "bytes": nbytes,
+               "GBps": nbytes / (mean * 1e-3) / 1e9, "frac_of_peak": nbytes / (mean * 1e-3) / PEAK_HBM}
+        if hasattr(fn, "flops"):
+            rec["TFLOPs"] = fn.flops / (mean * 1e-3) / 1e12
+        print(json.dumps(rec))
         return
 
     # ---- headline step ---------------------------------------------------------------------------------------------------

@@ -157,6 +157,24 @@ int32_t rt_reduce_nd(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, ui
                      uint64_t offset, int32_t rank, const uint64_t* shape, const int64_t* strides,
                      void* dst, uint64_t dst_len, int32_t dim);
 
+/* ---- matmul ------------------------------------------------------------------------------------------------------
+ * BackendMatMul::matmul (backend/mod.rs:474-485; Cpu backend/cpu.rs:725-951), argument list of protocol Op::Matmul
+ * (backend/remote/protocol.rs:269-277): dst[b] = lhs[b] (m x k) * rhs[b] (k x n) for every batch, dst row-major and
+ * contiguous from element 0 (b*m*n elements).  Each operand comes with its meta and the layout the caller found for its
+ * last two dims (core/meta.rs:744-750, ops/linalg/matmul.rs:200-251): row-major = column stride 1, column-major = row
+ * stride 1; batch dims must collapse into one stride; strides must not be negative.  The checks are those of
+ * backend/remote/server.rs:299-334 and 605-636 (RT_E_INVALID / RT_E_OUT_OF_BOUNDS); dst must not be one of the inputs.
+ * f32/f64 run on rocBLAS (loaded on first use), every other dtype -- all 13 are accepted, as the Cpu backend's generic
+ * loop does -- on a tiled kernel with the reference's wrapping `sum += a * b`.  Mixed layouts are accepted for every dtype
+ * (the Cpu backend has them for f32/f64 only). */
+typedef enum rt_contiguity { RT_ROW_MAJOR = 0, RT_COLUMN_MAJOR = 1, RT_CONTIGUITY_NONE = 2 } rt_contiguity;
+int32_t rt_matmul(rt_ctx* ctx, int32_t dtype,
+                  const void* lhs, uint64_t lhs_len, uint64_t lhs_offset, int32_t lhs_rank, const uint64_t* lhs_shape,
+                  const int64_t* lhs_strides, int32_t lhs_contiguity,
+                  const void* rhs, uint64_t rhs_len, uint64_t rhs_offset, int32_t rhs_rank, const uint64_t* rhs_shape,
+                  const int64_t* rhs_strides, int32_t rhs_contiguity,
+                  void* dst, uint64_t dst_len, uint64_t b, uint64_t m, uint64_t k, uint64_t n);
+
 /* ---- strided gather (what TensorView::owned / contiguous need, core/tensor.rs:299-325: the reference issues one
  * copy_range_within per forward-contiguous run; this is the same result in one launch) ------------------------- */
 int32_t rt_gather(rt_ctx* ctx, int32_t dtype, const void* src, uint64_t src_len, uint64_t offset, int32_t rank,

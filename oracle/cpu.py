@@ -60,6 +60,7 @@ def lib():
             build()
         L = C.CDLL(_SO)
         sz, i64p, szp, vp, ip = C.c_size_t, C.POINTER(C.c_int64), C.POINTER(C.c_size_t), C.c_void_p, C.POINTER(C.c_int)
+        i64 = C.c_int64
         L.orc_dtype_size.argtypes = [C.c_int]
         L.orc_is_contiguous.argtypes = [sz, C.c_int, szp, i64p]
         L.orc_unary.argtypes = [C.c_int, C.c_int, vp, sz, sz, C.c_int, szp, i64p, ip]
@@ -71,6 +72,7 @@ def lib():
         L.orc_reduce_nd.argtypes = [C.c_int, C.c_int, vp, sz, sz, C.c_int, szp, i64p, vp, sz, C.c_int, C.c_int]
         L.orc_gather.argtypes = [C.c_int, vp, sz, sz, C.c_int, szp, i64p, vp, sz]
         L.orc_equal.argtypes = [C.c_int, vp, vp, sz]
+        L.orc_matmul.argtypes = [C.c_int, vp, sz, sz, i64, i64, i64, vp, sz, sz, i64, i64, i64, vp, sz, sz, sz, sz, sz]
         _lib = L
     return _lib
 
@@ -188,6 +190,20 @@ def gather(dtype: int, src: np.ndarray, meta: MetaTensor) -> np.ndarray:
     rc = lib().orc_gather(dtype, _ptr(src), src.size, meta.offset, meta.rank(), _shape_arr(meta.shape),
                           _stride_arr(meta.strides), _ptr(dst), dst.size)
     _check(rc, "gather")
+    return dst
+
+
+def matmul(dtype: int, lhs: np.ndarray, lhs_meta: MetaTensor, rhs: np.ndarray, rhs_meta: MetaTensor, b: int, m: int, k: int, n: int) -> np.ndarray:
+    """`BackendMatMul::matmul` of the Cpu backend (backend/cpu.rs:725-951): dst[batch] = lhs[batch] @ rhs[batch], dst row-major.
+    The batch stride is `strides[rank - 3]` (0 for rank 2), rows / columns step by the last two strides."""
+    def parts(meta):
+        r = meta.rank()
+        return meta.offset, meta.strides[r - 2], meta.strides[r - 1], (meta.strides[r - 3] if r > 2 else 0)
+    lo, lrs, lcs, lbs = parts(lhs_meta)
+    ro, rrs, rcs, rbs = parts(rhs_meta)
+    dst = np.zeros(b * m * n, dtype=NP_DTYPE[dtype])
+    rc = lib().orc_matmul(dtype, _ptr(lhs), lhs.size, lo, lrs, lcs, lbs, _ptr(rhs), rhs.size, ro, rrs, rcs, rbs, _ptr(dst), dst.size, b, m, k, n)
+    _check(rc, "matmul")
     return dst
 
 

@@ -538,6 +538,39 @@ template <class T> int equal_impl(const T* a, const T* b, size_t n) {
         default: return ORC_E_DTYPE;                            \
     }
 
+// ---- matmul: backend/cpu.rs:857-939 (generic_backend_matmul) -------------------------------------------------------------------
+// dst[batch][row][col] = sum over inner, ascending, of lhs * rhs with `sum += a * b` on T (wrapping integers, OR/AND for
+// boolean); dst is row-major from element 0.  The reference writes the loop twice, for two row-major and for two
+// column-major operands (lhs_idx = batch + row*lda + inner / batch + row + inner*lda, ...); with (row stride, column stride)
+// per operand both are the one loop below.  For f32/f64 the reference calls OpenBLAS gemm (backend/cpu.rs:725-855; OpenBLAS
+// 0.3.30, build.rs:76-169, not vendored), whose summation order is not part of its interface: for those two dtypes this loop
+// is the textbook definition, exact whenever every partial sum is representable (all of the reference's own test vectors)
+// and otherwise only a tolerance reference -- bit parity for float matmul is unpinned.
+template <class T>
+int matmul_impl(const T* lhs, size_t lhs_len, size_t l_off, int64_t l_rs, int64_t l_cs, int64_t l_bs,
+                const T* rhs, size_t rhs_len, size_t r_off, int64_t r_rs, int64_t r_cs, int64_t r_bs,
+                T* dst, size_t dst_len, size_t b, size_t m, size_t k, size_t n) {
+    if (l_rs < 0 || l_cs < 0 || l_bs < 0 || r_rs < 0 || r_cs < 0 || r_bs < 0) return ORC_E_OOB;
+    if (b * m * n > dst_len) return ORC_E_OOB;
+    if (b && m && k && l_off + (b - 1) * (size_t)l_bs + (m - 1) * (size_t)l_rs + (k - 1) * (size_t)l_cs >= lhs_len) return ORC_E_OOB;
+    if (b && k && n && r_off + (b - 1) * (size_t)r_bs + (k - 1) * (size_t)r_rs + (n - 1) * (size_t)r_cs >= rhs_len) return ORC_E_OOB;
+    for (size_t batch = 0; batch < b; ++batch) {
+        const size_t lhs_batch = l_off + batch * (size_t)l_bs, rhs_batch = r_off + batch * (size_t)r_bs, out_batch = batch * m * n;
+        for (size_t row = 0; row < m; ++row) {
+            for (size_t col = 0; col < n; ++col) {
+                T sum = consts<T>::zero();
+                for (size_t inner = 0; inner < k; ++inner) {
+                    const T a = lhs[lhs_batch + row * (size_t)l_rs + inner * (size_t)l_cs];
+                    const T c = rhs[rhs_batch + inner * (size_t)r_rs + col * (size_t)r_cs];
+                    sum = add(sum, mul(a, c));
+                }
+                dst[out_batch + row * n + col] = sum;
+            }
+        }
+    }
+    return ORC_OK;
+}
+
 template <class T> inline T load_value(const void* p) { T v; std::memcpy(&v, p, sizeof(T)); return v; }
 
 }  // namespace
@@ -600,6 +633,13 @@ int orc_gather(int dtype, const void* src, size_t srclen, size_t offset, int ran
                const int64_t* strides, void* dst, size_t dstlen) {
     Meta m{offset, rank, shape, strides};
     ORC_DISPATCH(dtype, return gather_impl<T>((const T*)src, srclen, m, (T*)dst, dstlen));
+}
+
+int orc_matmul(int dtype, const void* lhs, size_t lhs_len, size_t l_off, int64_t l_rs, int64_t l_cs, int64_t l_bs,
+               const void* rhs, size_t rhs_len, size_t r_off, int64_t r_rs, int64_t r_cs, int64_t r_bs,
+               void* dst, size_t dst_len, size_t b, size_t m, size_t k, size_t n) {
+    ORC_DISPATCH(dtype, return matmul_impl<T>((const T*)lhs, lhs_len, l_off, l_rs, l_cs, l_bs, (const T*)rhs, rhs_len, r_off, r_rs, r_cs, r_bs,
+                                              (T*)dst, dst_len, b, m, k, n));
 }
 
 int orc_equal(int dtype, const void* a, const void* b, size_t n) {

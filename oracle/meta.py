@@ -66,6 +66,20 @@ class MetaTensor:
                 expected *= dim
         return True
 
+    def is_flat(self) -> bool:
+        """core/meta.rs:543-561: contiguity that allows an innermost |stride| other than 1 (used for matmul batch dims)."""
+        if len(self.shape) == 0 or 0 in self.shape:
+            return True
+        if len(self.shape) != len(self.strides):
+            return False
+        expected = abs(self.strides[-1])
+        for dim, s in zip(reversed(self.shape), reversed(self.strides)):
+            if dim != 1:
+                if abs(s) != expected:
+                    return False
+                expected *= dim
+        return True
+
     def non_singleton_dims(self) -> List[Tuple[int, int, int]]:
         """core/meta.rs:618-625: (index, size, stride) of dims with size > 1."""
         return [(i, d, s) for i, (d, s) in enumerate(zip(self.shape, self.strides)) if d > 1]
@@ -255,3 +269,21 @@ def logical_to_buffer_idx(idx: Sequence[int], strides: Sequence[int], offset: in
     if b < 0:
         raise TensorError("IdxOutOfBounds", "buffer index is negative")
     return b
+
+
+def contiguity_type(meta: MetaTensor) -> str:
+    """ops/linalg/matmul.rs:200-251: layout of the last two dims as gemm sees it ("row_major": last stride 1; "column_major":
+    second-to-last stride 1; else "none"), "none" as well when several batch dims do not collapse into one stride."""
+    r = meta.rank()
+    if r < 2:
+        return "row_major"
+    if meta.strides[r - 1] == 1:
+        inner = "row_major"
+    elif meta.strides[r - 2] == 1:
+        inner = "column_major"
+    else:
+        inner = "none"
+    batch = MetaTensor(list(meta.shape[:r - 2]), list(meta.strides[:r - 2]), 0)
+    if batch.rank() > 1 and not batch.is_flat():
+        return "none"
+    return inner

@@ -14,7 +14,7 @@ from typing import Optional, Sequence
 import numpy as np
 
 from . import cpu
-from .meta import (MetaTensor, Slice, TensorError, compute_broadcasted_params, compute_permuted_parameters,
+from .meta import (MetaTensor, Slice, TensorError, compute_broadcasted_params, compute_permuted_parameters, contiguity_type,
                    compute_sliced_parameters, compute_squeezed_parameters, compute_unsqueezed_parameters,
                    logical_to_buffer_idx, reduction_output_meta, shape_to_stride)
 
@@ -114,6 +114,48 @@ class OTensor:
     def to_numpy(self) -> np.ndarray:
         """Row-major values of the elements this tensor/view addresses, shaped like the tensor."""
         return cpu.gather(self.dtype, self.buf, self.meta).reshape(self.meta.shape)
+
+    # ---- matmul / dot / outer: ops/linalg/matmul.rs:5-180 ------------------------------------------------------------------
+    def matmul(self, other: "OTensor") -> "OTensor":
+        lhs, rhs = self, other
+        if lhs.meta.rank() < 2:
+            raise TensorError("InvalidShape", "LHS tensor must have rank >= 2 for matmul")
+        if rhs.meta.rank() < 2:
+            raise TensorError("InvalidShape", "RHS tensor must have rank >= 2 for matmul")
+        # an operand whose last two dims have no unit stride (or whose batch dims do not collapse) is made row-major first;
+        # negative strides are treated the same way here (the reference casts them to usize)
+        def prepared(t):
+            ct = contiguity_type(t.meta)
+            if ct == "none" or any(s < 0 for s in t.meta.strides):
+                return t.contiguous()
+            return t
+        lhs, rhs = prepared(lhs), prepared(rhs)
+        lr, rr = lhs.meta.rank(), rhs.meta.rank()
+        if lr != rr:
+            raise TensorError("InvalidShape", f"Both tensors must have the same rank >= 2, got lhs rank {lr} and rhs rank {rr}")
+        lb, rb = list(lhs.meta.shape[:lr - 2]), list(rhs.meta.shape[:rr - 2])
+        if lb != rb:
+            raise TensorError("SizeMismatch", f"Batch dimensions must match for matmul, got {lb} and {rb}")
+        b = 1
+        for d in lb:
+            b *= d
+        m, k_l = lhs.meta.shape[lr - 2], lhs.meta.shape[lr - 1]
+        k_r, n = rhs.meta.shape[rr - 2], rhs.meta.shape[rr - 1]
+        if k_l != k_r:
+            raise TensorError("SizeMismatch", f"Inner matrix dimensions must match for matmul, got lhs K={k_l} and rhs K={k_r}")
+        # the kernels step through batches by strides[rank - 3] alone: collapse flat batch dims to that stride
+        out = cpu.matmul(self.dtype, lhs.buf, lhs.meta, rhs.buf, rhs.meta, b, m, k_l, n)
+        return OTensor(self.dtype, out, MetaTensor.row_major(lb + [m, n]))
+
+    def dot(self, other: "OTensor") -> "OTensor":
+        if self.meta.rank() != 1 or other.meta.rank() != 1:
+            raise TensorError("InvalidShape", "Dot product is only defined for 1-D tensors")
+        return self.unsqueeze_at(0).matmul(other.unsqueeze_at(1)).squeeze()
+
+    def outer(self, other: "OTensor") -> "OTensor":
+        if self.meta.rank() != 1 or other.meta.rank() != 1:
+            raise TensorError("InvalidShape", "Outer product is only defined for 1-D tensors")
+        return self.unsqueeze_at(1).matmul(other.unsqueeze_at(0))
 
     # ---- broadcast binary operators: ops/broadcast/add.rs:7-478 (sub/mul/div are textual twins) ---------------------
     def _binary(self, other: "OTensor", op: str) -> "OTensor":

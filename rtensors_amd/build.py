@@ -27,7 +27,7 @@ FLAGS = [
 ]
 
 LIBS = {
-    "librt_hip.so": ["rt_runtime.hip", "rt_layout.hip", "rt_elementwise.hip", "rt_broadcast.hip", "rt_broadcast_tile.hip", "rt_reduce.hip", "rt_misc.hip"],
+    "librt_hip.so": ["rt_runtime.hip", "rt_layout.hip", "rt_elementwise.hip", "rt_broadcast.hip", "rt_broadcast_tile.hip", "rt_reduce.hip", "rt_misc.hip", "rt_matmul.hip"],
     "librt_datagen.so": ["rt_datagen.hip"],
 }
 HEADERS = [os.path.join(CSRC, "rt_common.h"), os.path.join(CSRC, "rt_broadcast_common.h"), os.path.join(HERE, "..", "include", "rt_hip.h")]
@@ -73,7 +73,7 @@ def build(force: bool = False, jobs: int = 8) -> None:
         out = os.path.join(LIB, lib)
         deps = [objs[s] for s in ss]
         if force or _stale(out, deps):
-            r = subprocess.run(["hipcc", f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", out] + deps, capture_output=True, text=True)
+            r = subprocess.run(["hipcc", f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", out] + deps + ["-ldl"], capture_output=True, text=True)
             if r.returncode != 0:
                 raise RuntimeError(f"link of {lib} failed:\n{_filter(r.stdout + r.stderr)}")
             print(f"[build] linked {lib}", file=sys.stderr)

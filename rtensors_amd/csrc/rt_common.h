@@ -43,6 +43,9 @@ struct rt_ctx {
     // scratch for two-stage reductions (partials), grown on demand, reused across calls
     void* scratch = nullptr;
     size_t scratch_bytes = 0;
+    // rocBLAS handle bound to `stream` (created by the first f32/f64 matmul) and the function that destroys it
+    void* blas = nullptr;
+    int (*blas_destroy)(void*) = nullptr;
     // device flag written by the equality kernel and read back by rt_equal
     int32_t* flag_dev = nullptr;
     int num_cus = 256;

@@ -83,6 +83,7 @@ extern "C" int32_t rt_ctx_destroy(rt_ctx* ctx) {
         for (auto& kv : ctx->free_blocks) (void)hipFree(kv.second);
         for (auto& kv : ctx->live) (void)hipFree(kv.first);
         if (ctx->scratch) (void)hipFree(ctx->scratch);
+        if (ctx->blas && ctx->blas_destroy) (void)ctx->blas_destroy(ctx->blas);
         if (ctx->flag_dev) (void)hipFree(ctx->flag_dev);
         (void)hipStreamDestroy(ctx->stream);
     }

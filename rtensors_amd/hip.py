@@ -26,6 +26,7 @@ UNARY = {n: i for i, n in enumerate(
     "neg relu sigmoid silu tanh abs sqrt ln expm1 ln1p floor ceil round trunc sin cos tan asin acos atan sinh cosh "
     "asinh acosh atanh rsqrt reciprocal square cube exp sign step abs_grad".split())}
 SCALAR = {n: i for i, n in enumerate("add sub mul div log log1p leaky_relu elu leaky_grad".split())}
+CONTIGUITY = {"row_major": 0, "column_major": 1, "none": 2}     # core/meta.rs:744-750
 BINARY = {"add": 0, "sub": 1, "mul": 2, "div": 3}
 REDUCE = {"sum": 1, "prod": 2, "max": 3, "min": 4, "mean": 5}
 
@@ -222,6 +223,13 @@ class Hip:
     def gather(self, src: HipBuf, meta, dst: HipBuf):
         off, shape, strides = meta
         _check(lib.rt_gather(self._ctx, src.dtype, src.ptr, src.len, off, len(shape), _u64s(shape), _i64s(strides), dst.ptr, dst.len))
+
+    # ---- matmul (backend/mod.rs:474-485) ----------------------------------------------------------------------------------
+    def matmul(self, lhs: Tuple[HipBuf, tuple, str], rhs: Tuple[HipBuf, tuple, str], dst: HipBuf, b: int, m: int, k: int, n: int):
+        """lhs / rhs = (buffer, (offset, shape, strides), "row_major" | "column_major" | "none")."""
+        (lb, (loff, lshape, lstr), lc), (rb, (roff, rshape, rstr), rc) = lhs, rhs
+        _check(lib.rt_matmul(self._ctx, dst.dtype, lb.ptr, lb.len, loff, len(lshape), _u64s(lshape), _i64s(lstr), CONTIGUITY[lc],
+                             rb.ptr, rb.len, roff, len(rshape), _u64s(rshape), _i64s(rstr), CONTIGUITY[rc], dst.ptr, dst.len, b, m, k, n))
 
     # ---- timing -----------------------------------------------------------------------------------------------------------
     def event(self):

@@ -214,13 +214,20 @@ class Hip {
         if (sm.rank() == 1) apply_reduce_contiguous_flat(src, dst, sm.offset, sm.size(), op);
         else apply_reduce_contiguous_nd(src, sm, dst, dim, op);
     }
-    // argmax / conv2d / matmul sit behind the same trait but outside this path; they report an error instead of the
+    // argmax / conv2d sit behind the same trait but outside this path; they report an error instead of the
     // Cpu backend's todo!() panic (backend/cpu.rs:452-481).
     void apply_argmax(const HipBuf&, const MetaTensor&, HipBuf&, size_t, ReductionOpTypes) const {
         throw TensorError(ErrorKind::UnsupportedOperation, "argmax/argmin are not implemented by the Hip backend");
     }
     void apply_conv_2d() const { throw TensorError(ErrorKind::UnsupportedOperation, "conv2d is not implemented by the Hip backend"); }
-    void matmul() const { throw TensorError(ErrorKind::UnsupportedOperation, "matmul is not implemented by the Hip backend"); }
+
+    // ---- BackendMatMul::matmul (backend/mod.rs:474-485) ---------------------------------------------------------------------
+    void matmul(const HipBuf& lhs, const MetaTensor& lm, ContiguityTypes lc, const HipBuf& rhs, const MetaTensor& rm, ContiguityTypes rc, HipBuf& dst,
+                uint64_t b, uint64_t m, uint64_t k, uint64_t n) const {
+        check(rt_matmul(raw(), dst.dtype(), lhs.ptr(), lhs.len(), lm.offset, (int32_t)lm.rank(), lm.shape.data(), lm.strides.data(), (int32_t)lc,
+                        rhs.ptr(), rhs.len(), rm.offset, (int32_t)rm.rank(), rm.shape.data(), rm.strides.data(), (int32_t)rc, dst.ptr(), dst.len(),
+                        b, m, k, n));
+    }
 
     // row-major copy of a view (what TensorView::owned needs, core/tensor.rs:299-325) in one launch
     void gather(const HipBuf& src, const MetaTensor& m, HipBuf& dst) const {

@@ -75,6 +75,7 @@ int rth_meta_broadcast(int ranka, const uint64_t* shapea, const int64_t* strides
         for (size_t i = 0; i < p.shape.size(); ++i) { oshape[i] = p.shape[i]; ostra[i] = p.a[i]; ostrb[i] = p.b[i]; }
     });
 }
+int rth_meta_contiguity_type(int rank, const uint64_t* shape, const int64_t* strides) { return (int)contiguity_type(make_meta(rank, shape, strides, 0)); }
 int rth_meta_is_contiguous(int rank, const uint64_t* shape, const int64_t* strides) { return make_meta(rank, shape, strides, 0).is_contiguous() ? 1 : 0; }
 
 // ---- backend / tensors ---------------------------------------------------------------------------------------------------
@@ -116,6 +117,9 @@ int rth_contiguous(void* t, void** out) { return guarded([&] { *out = new Tensor
 
 int rth_binary(void* a, void* b, int op, void** out) { return guarded([&] { *out = new Tensor(((Tensor*)a)->binary(*(Tensor*)b, (BinaryOpType)op)); }); }
 int rth_binary_assign(void* a, void* b, int op) { return guarded([&] { ((Tensor*)a)->binary_assign(*(Tensor*)b, (BinaryOpType)op); }); }
+int rth_matmul(void* a, void* b, void** out) { return guarded([&] { *out = new Tensor(((Tensor*)a)->matmul(*(Tensor*)b)); }); }
+int rth_dot(void* a, void* b, void** out) { return guarded([&] { *out = new Tensor(((Tensor*)a)->dot(*(Tensor*)b)); }); }
+int rth_outer(void* a, void* b, void** out) { return guarded([&] { *out = new Tensor(((Tensor*)a)->outer(*(Tensor*)b)); }); }
 int rth_scalar(void* a, int op, double v, void** out) { return guarded([&] { *out = new Tensor(((Tensor*)a)->scalar(op, v)); }); }
 int rth_scalar_assign(void* a, int op, double v) { return guarded([&] { ((Tensor*)a)->scalar_assign(op, v); }); }
 int rth_unary(void* a, int op, void** out) { return guarded([&] { *out = new Tensor(((Tensor*)a)->unary(op)); }); }

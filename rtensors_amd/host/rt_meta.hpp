@@ -98,6 +98,22 @@ struct MetaTensor {
         }
         return true;
     }
+    // core/meta.rs:543-561: contiguity that allows an innermost |stride| other than 1 (matmul batch dims)
+    bool is_flat() const {
+        if (shape.empty()) return true;
+        for (uint64_t d : shape) if (d == 0) return true;
+        if (shape.size() != strides.size()) return false;
+        auto mag = [](int64_t s) { return s < 0 ? (uint64_t)(-(s + 1)) + 1 : (uint64_t)s; };
+        uint64_t expected = mag(strides.back());
+        for (size_t i = shape.size(); i-- > 0;) {
+            if (shape[i] != 1) {
+                if (mag(strides[i]) != expected) return false;
+                uint64_t p;
+                expected = __builtin_mul_overflow(expected, shape[i], &p) ? UINT64_MAX : p;
+            }
+        }
+        return true;
+    }
     // Forward row-major run: what a kernel may treat as `offset .. offset + size` (signed strides).
     bool is_forward_contiguous() const {
         int64_t expected = 1;
@@ -255,6 +271,21 @@ inline MetaTensor reduction_output_meta(const MetaTensor& in, std::optional<size
     Shape s;
     for (size_t d = 0; d < in.rank(); ++d) s.push_back(d == *axis ? 1 : in.shape[d]);
     return MetaTensor::row_major(s);
+}
+
+// core/meta.rs:744-750; codes equal rt_contiguity of the C ABI
+enum class ContiguityTypes { RowMajor = 0, ColumnMajor = 1, None = 2 };
+
+// ops/linalg/matmul.rs:200-251: the layout gemm sees in the last two dims; None as well when several batch dims do not
+// collapse into one stride
+inline ContiguityTypes contiguity_type(const MetaTensor& meta) {
+    const size_t r = meta.rank();
+    if (r < 2) return ContiguityTypes::RowMajor;
+    ContiguityTypes inner = meta.strides[r - 1] == 1 ? ContiguityTypes::RowMajor
+                          : meta.strides[r - 2] == 1 ? ContiguityTypes::ColumnMajor : ContiguityTypes::None;
+    MetaTensor batch(Shape(meta.shape.begin(), meta.shape.end() - 2), Strides(meta.strides.begin(), meta.strides.end() - 2), 0);
+    if (batch.rank() > 1 && !batch.is_flat()) return ContiguityTypes::None;
+    return inner;
 }
 
 }  // namespace rt

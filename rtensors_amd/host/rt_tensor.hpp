@@ -157,6 +157,45 @@ class Tensor {
     RT_TENSOR_UNARY(square, RT_U_SQUARE) RT_TENSOR_UNARY(cube, RT_U_CUBE) RT_TENSOR_UNARY(exp, RT_U_EXP) RT_TENSOR_UNARY(sign, RT_U_SIGN)
 #undef RT_TENSOR_UNARY
 
+    // ---- matmul / dot / outer (ops/linalg/matmul.rs:5-180) ------------------------------------------------------------------------------
+    // (..., M, K) @ (..., K, N) -> (..., M, N); batch dims must match exactly.  An operand whose last two dims have no unit
+    // stride, or whose batch dims do not collapse into one stride, is made row-major first (matmul.rs:42-62); so is one with
+    // a negative stride, which the reference would cast to usize.
+    Tensor matmul(const Tensor& rhs) const {
+        if (rank() < 2) throw TensorError(ErrorKind::InvalidShape, "LHS tensor must have rank >= 2 for matmul");
+        if (rhs.rank() < 2) throw TensorError(ErrorKind::InvalidShape, "RHS tensor must have rank >= 2 for matmul");
+        auto prepared = [](const Tensor& t) {
+            bool negative = false;
+            for (int64_t s : t.meta_.strides) negative = negative || s < 0;
+            return (negative || contiguity_type(t.meta_) == ContiguityTypes::None) ? t.gathered() : t;
+        };
+        const Tensor l = prepared(*this), r = prepared(rhs);
+        const size_t lr = l.rank(), rr = r.rank();
+        if (lr != rr) throw TensorError(ErrorKind::InvalidShape, "Both tensors must have the same rank >= 2");
+        Shape batch(l.meta_.shape.begin(), l.meta_.shape.end() - 2);
+        if (batch != Shape(r.meta_.shape.begin(), r.meta_.shape.end() - 2))
+            throw TensorError(ErrorKind::SizeMismatch, "Batch dimensions must match for matmul");
+        uint64_t b = 1;
+        for (uint64_t d : batch) b *= d;
+        const uint64_t m = l.meta_.shape[lr - 2], k = l.meta_.shape[lr - 1], kr = r.meta_.shape[rr - 2], n = r.meta_.shape[rr - 1];
+        if (k != kr) throw TensorError(ErrorKind::SizeMismatch, "Inner matrix dimensions must match for matmul");
+        Shape out_shape = batch;
+        out_shape.push_back(m);
+        out_shape.push_back(n);
+        MetaTensor om = MetaTensor::row_major(out_shape);
+        Tensor out(*backend_, backend_->alloc_uninit(dtype(), om.size()), om);
+        backend_->matmul(*l.buf_, l.meta_, contiguity_type(l.meta_), *r.buf_, r.meta_, contiguity_type(r.meta_), *out.buf_, b, m, k, n);
+        return out;
+    }
+    Tensor dot(const Tensor& rhs) const {
+        if (rank() != 1 || rhs.rank() != 1) throw TensorError(ErrorKind::InvalidShape, "Dot product is only defined for 1-D tensors");
+        return unsqueeze_at(0).matmul(rhs.unsqueeze_at(1)).squeeze();
+    }
+    Tensor outer(const Tensor& rhs) const {
+        if (rank() != 1 || rhs.rank() != 1) throw TensorError(ErrorKind::InvalidShape, "Outer product is only defined for 1-D tensors");
+        return unsqueeze_at(1).matmul(rhs.unsqueeze_at(0));
+    }
+
     // ---- reductions ----------------------------------------------------------------------------------------------------------------------
     // Non-contiguous inputs are copied first (ops/reduction/mod.rs:346-408).  "Contiguous" here means a forward
     // row-major run: a reversed view is |stride|-contiguous for the reference and would reach its kernels with the

@@ -111,6 +111,10 @@ def meta_broadcast(shape_a, strides_a, shape_b, strides_b):
     return list(sh[:n]), list(sa[:n]), list(sb[:n])
 
 
+def meta_contiguity_type(shape, strides) -> str:
+    return ("row_major", "column_major", "none")[_h.rth_meta_contiguity_type(len(shape), _u64(shape), _i64(strides))]
+
+
 def meta_is_contiguous(shape, strides) -> bool:
     return bool(_h.rth_meta_is_contiguous(len(shape), _u64(shape), _i64(strides)))
 
@@ -216,6 +220,10 @@ class Tensor:
     def relu(self): return self.unary("relu")
     def sign(self): return self.unary("sign")
     def abs(self): return self.unary("abs")
+
+    def matmul(self, o): return self._new(_h.rth_matmul, o._p)
+    def dot(self, o): return self._new(_h.rth_dot, o._p)
+    def outer(self, o): return self._new(_h.rth_outer, o._p)
 
     def reduce(self, op, axis=None): return self._new(_h.rth_reduce, REDUCE[op], C.c_int64(-1 if axis is None else axis))
     def sum_at(self, a): return self.reduce("sum", a)

@@ -2,7 +2,7 @@
 
 A case is `inputs` (named row-major tensors), a `program` (one step per line: [result, op, operands...]) and
 `expect` entries.  The same case runs against any tensor implementation that offers the reference's surface
-(from_buf, slice, permute, transpose, unsqueeze_at, squeeze, + - * /, in-place forms, unary, reductions);
+(from_buf, slice, permute, transpose, unsqueeze_at, squeeze, + - * /, in-place forms, unary, reductions, matmul);
 `factory(dtype_name, values, shape)` creates an owned tensor, `TensorError` is that implementation's error type.
 """
 import json
@@ -67,6 +67,8 @@ def run_case(case, factory, SliceCls, ErrorCls):
                 paths[dst] = getattr(env[dst], "last_path", None)
             elif op == "scalar_inplace":
                 env[dst] = env[args[0]].scalar_op_inplace(args[1], args[2])
+            elif op in ("matmul", "dot", "outer"):
+                env[dst] = getattr(env[args[0]], op)(env[args[1]])
             elif op in ("sum", "mean", "max", "min", "prod"):
                 env[dst] = env[args[0]].reduce(op, args[1])
             else:

@@ -5,7 +5,7 @@ from __future__ import annotations
 
 import numpy as np
 
-from oracle.meta import (MetaTensor, Slice, TensorError, compute_broadcasted_params, compute_permuted_parameters,
+from oracle.meta import (MetaTensor, Slice, TensorError, compute_broadcasted_params, compute_permuted_parameters, contiguity_type,
                          compute_sliced_parameters, compute_squeezed_parameters, compute_unsqueezed_parameters,
                          logical_to_buffer_idx, reduction_output_meta)
 from rtensors_amd import hip as H
@@ -126,6 +126,37 @@ class GTensor:
         return self
 
     def fill(self, v): self.backend.fill(self.buf, v, _m(self.meta))
+
+    def matmul(self, other):
+        """ops/linalg/matmul.rs:5-139 over the C ABI's rt_matmul."""
+        if self.meta.rank() < 2 or other.meta.rank() < 2:
+            raise TensorError("InvalidShape", "matmul operands need rank >= 2")
+        def prepared(t):
+            return t.contiguous() if contiguity_type(t.meta) == "none" or any(s < 0 for s in t.meta.strides) else t
+        l, r = prepared(self), prepared(other)
+        if l.meta.rank() != r.meta.rank():
+            raise TensorError("InvalidShape", "rank mismatch")
+        batch = list(l.meta.shape[:-2])
+        if batch != list(r.meta.shape[:-2]):
+            raise TensorError("SizeMismatch", "batch dims")
+        m, k, kr, n = l.meta.shape[-2], l.meta.shape[-1], r.meta.shape[-2], r.meta.shape[-1]
+        if k != kr:
+            raise TensorError("SizeMismatch", "inner dims")
+        b = int(np.prod(batch, dtype=np.int64)) if batch else 1
+        om = MetaTensor.row_major(batch + [m, n])
+        out = self.backend.alloc_uninit(self.dtype, max(om.size(), 1))
+        self.backend.matmul((l.buf, _m(l.meta), contiguity_type(l.meta)), (r.buf, _m(r.meta), contiguity_type(r.meta)), out, b, m, k, n)
+        return GTensor(self.backend, out, om)
+
+    def dot(self, other):
+        if self.meta.rank() != 1 or other.meta.rank() != 1:
+            raise TensorError("InvalidShape", "Dot product is only defined for 1-D tensors")
+        return self.unsqueeze_at(0).matmul(other.unsqueeze_at(1)).squeeze()
+
+    def outer(self, other):
+        if self.meta.rank() != 1 or other.meta.rank() != 1:
+            raise TensorError("InvalidShape", "Outer product is only defined for 1-D tensors")
+        return self.unsqueeze_at(1).matmul(other.unsqueeze_at(0))
 
     def reduce(self, op, axis=None):
         t = self if self.meta.is_contiguous() and all(s >= 0 for s in self.meta.strides) else self.contiguous()

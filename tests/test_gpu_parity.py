@@ -291,7 +291,7 @@ def test_reversed_view_is_walked_backwards_not_out_of_bounds(hip):
         o.slice(0, Slice(None, None, -1)).unary_inplace("relu")
 
 
-CASES = golden_dsl.load("reference_vectors.json")
+CASES = golden_dsl.load("reference_vectors.json") + golden_dsl.load("reference_matmul_vectors.json")
 
 
 @pytest.mark.parametrize("case", CASES, ids=lambda c: c["name"])
@@ -696,3 +696,112 @@ def test_more_than_2_31_elements(hip):
     hip.apply_reduce_contiguous_flat(d, out, 0, n, "min")
     assert hip.dump(out)[0] == 7
     hip.sync()
+
+
+# ---- matmul (BackendMatMul::matmul, backend/mod.rs:474-485) --------------------------------------------------------------------------
+MM_SHAPES = [(1, 1, 1, 1), (1, 5, 7, 3), (3, 64, 64, 64), (2, 70, 33, 129), (1, 130, 16, 65), (4, 1, 40, 1), (1, 2, 1, 200)]
+
+
+def _mm_operand(make, dtype, rng, b, rows, cols, layout, lo=-1000, hi=1000):
+    """An operand of logical shape (b, rows, cols) [or (rows, cols) when b == 1 and layout is even] in one of four layouts:
+    0 row-major contiguous, 1 row-major rows of a wider matrix at an offset, 2 column-major (transposed base),
+    3 column-major with a padded leading dim.  Returns what `make(values, shape)` gives, viewed accordingly."""
+    if layout == 0:
+        return make(rand_values(dtype, b * rows * cols, rng, lo, hi), [b, rows, cols])
+    if layout == 1:
+        t = make(rand_values(dtype, b * (rows + 2) * (cols + 5), rng, lo, hi), [b, rows + 2, cols + 5])
+        return t.slice(1, Slice(1, rows + 1, 1)).slice(2, Slice(3, cols + 3, 1))
+    if layout == 2:
+        return make(rand_values(dtype, b * rows * cols, rng, lo, hi), [b, cols, rows]).permute([0, 2, 1])
+    t = make(rand_values(dtype, b * (cols + 1) * (rows + 3), rng, lo, hi), [b, cols + 1, rows + 3])
+    return t.slice(1, Slice(0, cols, 1)).slice(2, Slice(2, rows + 2, 1)).permute([0, 2, 1])
+
+
+@pytest.mark.parametrize("dtype", ["i32", "u8", "i64", "i16", "u32", "bool"])
+def test_matmul_integers_bit_exact(hip, dtype):
+    """The tiled kernel against the Cpu backend's triple loop (backend/cpu.rs:857-939): wrapping sums, every pairing of
+    row-/column-major operands (the reference itself has mixed pairings for f32/f64 only), padded leading dims, offsets,
+    batches, ragged tiles."""
+    seed = abs(hash(dtype)) % 2 ** 31
+    lo, hi = (-2 ** 31, 2 ** 31 - 1) if dtype in ("i64", "u32", "i32") else (-1000, 1000)      # products overflow and wrap
+    for (b, m, k, n) in MM_SHAPES:
+        for ll in range(4):
+            for rl in range(4):
+                r1, r2 = np.random.default_rng(seed), np.random.default_rng(seed)
+                ol = _mm_operand(lambda v, s: OTensor.from_buf(dtype, v, s), dtype, r1, b, m, k, ll, lo, hi)
+                orr = _mm_operand(lambda v, s: OTensor.from_buf(dtype, v, s), dtype, r1, b, k, n, rl, lo, hi)
+                gl = _mm_operand(lambda v, s: G(hip, dtype, v, s), dtype, r2, b, m, k, ll, lo, hi)
+                gr = _mm_operand(lambda v, s: G(hip, dtype, v, s), dtype, r2, b, k, n, rl, lo, hi)
+                with np.errstate(all="ignore"):
+                    want = ol.matmul(orr)
+                got = gl.matmul(gr)
+                assert list(got.meta.shape) == list(want.meta.shape) == [b, m, n]
+                assert got.dump().tobytes() == want.buf.tobytes(), (dtype, (b, m, k, n), ll, rl)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64"])
+def test_matmul_floats_within_tolerance(hip, dtype):
+    """rocBLAS gemm against the textbook dot product in ascending k.  The reference's own f32/f64 path is OpenBLAS, whose
+    summation order is not specified, so bit parity is unpinned; the bound is rel * sum_k |a_ik * b_kj| with rel = 1e-5 (f32)
+    / 1e-12 (f64), and the result is cross-checked against numpy in f64."""
+    rel = 1e-5 if dtype == "f32" else 1e-12
+    seed = 99
+    for (b, m, k, n) in MM_SHAPES + [(2, 300, 517, 260)]:
+        for ll in range(4):
+            for rl in range(4):
+                if (b, m, k, n) == (2, 300, 517, 260) and (ll, rl) not in ((0, 0), (1, 3), (2, 1), (3, 2)):
+                    continue
+                r1, r2 = np.random.default_rng(seed), np.random.default_rng(seed)
+                ol = _mm_operand(lambda v, s: OTensor.from_buf(dtype, v, s), dtype, r1, b, m, k, ll)
+                orr = _mm_operand(lambda v, s: OTensor.from_buf(dtype, v, s), dtype, r1, b, k, n, rl)
+                gl = _mm_operand(lambda v, s: G(hip, dtype, v, s), dtype, r2, b, m, k, ll)
+                gr = _mm_operand(lambda v, s: G(hip, dtype, v, s), dtype, r2, b, k, n, rl)
+                want = ol.matmul(orr).buf.reshape(b, m, n).astype(np.float64)
+                got = gl.matmul(gr).dump().reshape(b, m, n).astype(np.float64)
+                A, B = ol.to_numpy().astype(np.float64), orr.to_numpy().astype(np.float64)
+                bound = rel * (np.abs(A) @ np.abs(B)) + 1e-300
+                assert (np.abs(got - want) <= bound).all(), (dtype, (b, m, k, n), ll, rl, np.abs(got - want).max())
+                assert (np.abs(got - A @ B) <= bound).all(), (dtype, (b, m, k, n), ll, rl)
+
+
+def test_matmul_128_bit_and_rank2(hip):
+    vals_a, vals_b = [2 ** 100 + 7, 3, 5, 2 ** 64 + 1, 11, 13], [1, 2 ** 90, 3, 4, 2 ** 127 - 1, 6]
+    for name in ("u128", "i128"):
+        oa, ob = OTensor.from_buf(name, vals_a, [2, 3]), OTensor.from_buf(name, vals_b, [3, 2])
+        ga, gb = G(hip, name, cpu.from_ints(cpu.DTYPE_BY_NAME[name], vals_a), [2, 3]), G(hip, name, cpu.from_ints(cpu.DTYPE_BY_NAME[name], vals_b), [3, 2])
+        assert ga.matmul(gb).dump().tobytes() == oa.matmul(ob).buf.tobytes()
+        assert ga.matmul(ga.transpose()).dump().tobytes() == oa.matmul(oa.transpose()).buf.tobytes()
+    x, y = np.arange(1, 6, dtype=np.float32), np.arange(2, 7, dtype=np.float32)
+    gx, gy = G(hip, "f32", x, [5]), G(hip, "f32", y, [5])
+    assert gx.dot(gy).dump().tolist() == [float(x @ y)] and gx.dot(gy).meta.shape == []
+    assert gx.outer(gy).dump().tobytes() == np.outer(x, y).astype(np.float32).tobytes()
+
+
+def test_matmul_descriptor_checks(hip):
+    """backend/remote/server.rs:299-334, 605-636: a bad operand is an error code, never a launch."""
+    from rtensors_amd import hip as H
+    a = hip.alloc_from_slice(H.F32, np.arange(12, dtype=np.float32))
+    b = hip.alloc_from_slice(H.F32, np.arange(12, dtype=np.float32))
+    d = hip.alloc(H.F32, 16)
+    ok_l, ok_r = (a, (0, [3, 4], [4, 1]), "row_major"), (b, (0, [4, 3], [3, 1]), "row_major")
+    hip.matmul(ok_l, ok_r, d, 1, 3, 4, 3)
+    want = (np.arange(12, dtype=np.float32).reshape(3, 4) @ np.arange(12, dtype=np.float32).reshape(4, 3)).reshape(-1)
+    assert hip.dump(d)[:9].tolist() == want.tolist()
+    bad = [
+        ((a, (0, [3, 4], [4, 1]), "row_major"), (b, (0, [4, 3], [3, 1]), "row_major"), a, (1, 3, 4, 3), "alias"),
+        ((a, (0, [3, 4], [4, 1]), "column_major"), ok_r, d, (1, 3, 4, 3), "layout code does not match strides"),
+        ((a, (0, [3, 4], [4, 1]), "none"), ok_r, d, (1, 3, 4, 3), "layout none"),
+        ((a, (11, [3, 4], [-4, 1]), "row_major"), ok_r, d, (1, 3, 4, 3), "negative stride"),
+        ((a, (1, [3, 4], [4, 1]), "row_major"), ok_r, d, (1, 3, 4, 3), "extent past the end"),
+        ((a, (0, [3, 4], [4, 1]), "row_major"), ok_r, d, (1, 3, 4, 4), "shape does not match m, k, n"),
+        ((a, (0, [1, 3, 4], [12, 4, 1]), "row_major"), ok_r, d, (1, 3, 4, 3), "rank mismatch"),
+        ((a, (0, [3, 4], [4, 1]), "row_major"), ok_r, hip.alloc(H.F32, 8), (1, 3, 4, 3), "dst too small"),
+        ((a, (0, [2, 1, 3, 2], [6, 3, 2, 1]), "row_major"), (b, (0, [2, 1, 2, 3], [3, 6, 3, 1]), "row_major"), d, (2, 3, 2, 3), "batch dims not collapsible"),
+    ]
+    for l, r, dst, (bb, m, k, n), why in bad:
+        with pytest.raises(H.TensorError):
+            hip.matmul(l, r, dst, bb, m, k, n)
+    # k == 0: empty sums
+    hip.fill_contiguous(d, 7.0, 0, 16)
+    hip.matmul((a, (0, [3, 0], [0, 1]), "row_major"), (b, (0, [0, 3], [3, 1]), "row_major"), d, 1, 3, 0, 3)
+    assert hip.dump(d).tolist() == [0.0] * 9 + [7.0] * 7
