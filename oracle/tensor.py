@@ -295,3 +295,21 @@ def train_step(x: OTensor, bias: OTensor, target: OTensor, lr: float, mode: str 
     v = bias.view()
     v -= update
     return loss, grad_values
+
+
+def linear_step(x: OTensor, w: OTensor, target: OTensor, lr: float, seed_with_loss: bool = True):
+    """One step of y = x @ w, loss = mean_l1_loss(y, target), backward to d(w), SGD (ops/linalg/matmul.rs:5-139, 182-198;
+    backwards_matmul, grad/backwards.rs:493-510: d(rhs) = lhs^T @ upstream with only the last two dims swapped).  `w` is
+    updated in place; returns (loss, d_w)."""
+    y = x.matmul(w)                                       # MatMul node keeps contiguous copies of both inputs
+    left = x.contiguous()
+    loss, gmap_l1 = mean_l1_loss(y, target)               # L1 node
+    upstream = loss.owned() if seed_with_loss else OTensor.from_buf(loss.dtype, [1], [])   # grad/mod.rs:442-447
+    d_y = gmap_l1 * upstream                              # backwards_l1
+    r = left.meta.rank()
+    perm = list(range(r - 2)) + [r - 1, r - 2]
+    d_w = left.permute(perm).matmul(d_y)                  # backwards_matmul, rhs
+    update = d_w * cpu.NP_DTYPE[d_w.dtype].type(lr)
+    v = w.view()
+    v -= update
+    return loss, d_w

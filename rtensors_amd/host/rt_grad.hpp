@@ -23,7 +23,7 @@ namespace grad {
 //                      upstream buffer.  Kept so the divergence can be shown in a test.
 enum class BroadcastGradMode { Sum, ReferenceLiteral };
 
-enum class NodeKind { None, Leaf, BroadcastAdd, BroadcastSub, ReLU, L1 };
+enum class NodeKind { None, Leaf, BroadcastAdd, BroadcastSub, ReLU, L1, MatMul };
 
 struct Node {
     NodeKind kind = NodeKind::None;
@@ -31,6 +31,7 @@ struct Node {
     Strides lhs_strides, rhs_strides;    // BroadcastAdd / BroadcastSub
     Shape lhs_shape, rhs_shape;
     Tensor grad_map;                     // ReLU, L1
+    Tensor left_input, right_input;      // MatMul (row-major copies, ops/linalg/matmul.rs:126-130)
     Tensor loss;                         // L1
     std::shared_ptr<Tensor> grad;        // Leaf: accumulated gradient (null until the first backward pass)
 };
@@ -97,6 +98,19 @@ class GradContext {
         if (!track) return Var{result, -1};
         gmap.unary_inplace(RT_U_ABS_GRAD);
         return map_node(result, gmap, a.node);
+    }
+
+    // ops/linalg/matmul.rs:5-139 + attach_matmul_grad (182-198): the node keeps contiguous copies of both inputs
+    Var matmul(const Var& a, const Var& b) {
+        Tensor result = a.t.matmul(b.t);
+        if (a.node < 0 && b.node < 0) return Var{result, -1};
+        Node n;
+        n.kind = NodeKind::MatMul;
+        n.parents = {a.node, b.node};
+        n.left_input = a.t.contiguous();
+        n.right_input = b.t.contiguous();
+        nodes_.push_back(n);
+        return Var{result, (int)nodes_.size() - 1};
     }
 
     // ops/broadcast/l1.rs:49-84 with ReductionType::Mean
@@ -214,6 +228,19 @@ class GradContext {
                     out[1] = n.kind == NodeKind::BroadcastSub ? -up : up.owned();
                     inverse_broadcast_gradient(out[1], n.rhs_strides, n.rhs_shape);
                 }
+                return out;
+            }
+            case NodeKind::MatMul: {                                     // backwards_matmul, backwards.rs:493-510
+                // d(lhs) = upstream @ rhs^T, d(rhs) = lhs^T @ upstream; only the last two dims are swapped
+                auto swap_last_two = [](const Tensor& t) {
+                    std::vector<size_t> dims(t.rank());
+                    for (size_t i = 0; i < dims.size(); ++i) dims[i] = i;
+                    std::swap(dims[dims.size() - 1], dims[dims.size() - 2]);
+                    return t.permute(dims);
+                };
+                std::vector<Tensor> out(2);
+                if (n.parents[0] >= 0) out[0] = up.matmul(swap_last_two(n.right_input));
+                if (n.parents[1] >= 0) out[1] = swap_last_two(n.left_input).matmul(up);
                 return out;
             }
             default:

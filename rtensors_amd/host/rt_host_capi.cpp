@@ -163,4 +163,24 @@ int rth_train_step(void* x, void* bias, void* target, double lr, int mode, int s
     });
 }
 
+// y = x @ w; loss = mean_l1_loss(y, target); backward; SGD(lr) on w (updated in place).  Outputs: loss and d(w).
+int rth_linear_step(void* x, void* w, void* target, double lr, int seed_with_loss, void** out_loss, void** out_grad) {
+    return guarded([&] {
+        grad::GradContext ctx;
+        ctx.seed_with_loss = seed_with_loss != 0;
+        grad::Var vx = ctx.input(*(Tensor*)x);
+        grad::Var vw = ctx.param(*(Tensor*)w);
+        grad::Var vt = ctx.input(*(Tensor*)target);
+        grad::SGD opt(lr);
+        opt.register_parameter(ctx, vw);
+        grad::Var loss = ctx.mean_l1_loss(ctx.matmul(vx, vw), vt);
+        ctx.backwards(loss);
+        std::shared_ptr<Tensor> g = ctx.grad_of(vw);
+        if (!g) throw TensorError(ErrorKind::GradError, "no gradient reached the parameter");
+        *out_grad = new Tensor(g->contiguous());
+        *out_loss = new Tensor(loss.t);
+        opt.step();
+    });
+}
+
 }  // extern "C"

@@ -269,3 +269,10 @@ def train_step(x: Tensor, bias: Tensor, target: Tensor, lr: float, mode: str = "
     pl, pg = C.c_void_p(), C.c_void_p()
     _ck(_h.rth_train_step(x._p, bias._p, target._p, C.c_double(lr), 0 if mode == "sum" else 1, 1 if seed_with_loss else 0, C.byref(pl), C.byref(pg)))
     return Tensor(pl, x.backend), Tensor(pg, x.backend)
+
+
+def linear_step(x: Tensor, w: Tensor, target: Tensor, lr: float, seed_with_loss: bool = True):
+    """y = x @ w; loss = mean_l1_loss(y, target); backward; SGD(lr) on w in place.  Returns (loss, d_w)."""
+    pl, pg = C.c_void_p(), C.c_void_p()
+    _ck(_h.rth_linear_step(x._p, w._p, target._p, C.c_double(lr), 1 if seed_with_loss else 0, C.byref(pl), C.byref(pg)))
+    return Tensor(pl, x.backend), Tensor(pg, x.backend)

@@ -146,6 +146,37 @@ def test_train_step_matches_oracle(T, be, dtype, mode, seed_with_loss):
         assert not np.allclose(gsum.buf, ograd.buf)
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f64"])
+@pytest.mark.parametrize("seed_with_loss", [True, False])
+def test_linear_step_matches_oracle(T, be, dtype, seed_with_loss):
+    """y = x @ w, mean L1 loss, backward through the MatMul node (d(w) = x^T @ upstream), SGD on w."""
+    from rtensors_amd import datagen
+    from oracle.tensor import linear_step as oracle_linear_step
+    npd = cpu.NP_DTYPE[cpu.DTYPE_BY_NAME[dtype]]
+    n, d, h = 200, 48, 24
+    x = datagen.normal(npd, n * d, 5, 0)
+    w = datagen.normal(npd, d * h, 5, 1, 0.2)
+    target = datagen.uniform(npd, n * h, 5, 2)
+    ox, ow, ot = OTensor.from_buf(dtype, x, [n, d]), OTensor.from_buf(dtype, w, [d, h]), OTensor.from_buf(dtype, target, [n, h])
+    gx, gw, gt = T.Tensor.from_buf(be, dtype, x, [n, d]), T.Tensor.from_buf(be, dtype, w, [d, h]), T.Tensor.from_buf(be, dtype, target, [n, h])
+    oloss, ograd = oracle_linear_step(ox, ow, ot, 0.01, seed_with_loss)
+    gloss, ggrad = T.linear_step(gx, gw, gt, 0.01, seed_with_loss)
+    tol = 1e-5 if dtype == "f32" else 1e-12
+    X, W, Tg = x.reshape(n, d).astype(np.float64), w.reshape(d, h).astype(np.float64), target.reshape(n, h).astype(np.float64)
+    Y = X @ W
+    assert abs(float(gloss.to_numpy()) - float(oloss.buf[0])) <= 50 * tol * (np.abs(X) @ np.abs(W) + np.abs(Tg)).sum() / (n * h)
+    assert ggrad.shape == ograd.meta.shape == [d, h]
+    scale = abs(float(oloss.buf[0])) if seed_with_loss else 1.0
+    bound = 50 * tol * scale * np.abs(X).sum(axis=0)[:, None] / (n * h) + 1e-30
+    # sign(y - t) can flip where a float matmul result lands on the other side of the target: compare away from such ties
+    stable = np.abs(Y - Tg) > 1e-3
+    if stable.all():
+        assert (np.abs(ggrad.to_numpy().astype(np.float64) - ograd.buf.reshape(d, h).astype(np.float64)) <= bound).all()
+    closed = scale * (X.T @ np.sign(Y - Tg)) / (n * h)
+    assert np.max(np.abs(ggrad.to_numpy().astype(np.float64) - closed)) <= 1e-4 * scale * (1.0 + (~stable).sum())
+    assert np.max(np.abs(gw.to_numpy().astype(np.float64) - (W - 0.01 * closed))) <= 1e-5 * (1.0 + (~stable).sum())
+
+
 # ---- BASELINE configurations at full size ---------------------------------------------------------------------------------------
 def test_config1_full_vs_oracle(be, T):
     from rtensors_amd import datagen
