@@ -299,6 +299,50 @@ def api_overhead(hip):
     return out
 
 
+def host_layer_runs(iters=10):
+    """Whole operator sequences issued through the C++ host layer (allocation of every result and temporary included), wall
+    clock per iteration: the config-2 chain c = relu(a * 3 + b); c -= 1 and the config-5 training step at full size
+    (65536 x 4096).  The reference's operators issue the chain as two clones + four kernels (13 x 1 GiB of traffic); the host
+    layer runs `a * 3` and `relu(u)` as one out-of-place pass each, so its four kernels move 2 + 3 + 2 + 2 = 9 x 1 GiB."""
+    from rtensors_amd import tensor as T
+    be = T.Backend(0)
+    rng = np.random.default_rng(0)
+    out = {}
+    n = 1 << 28
+    a = T.Tensor.from_buf(be, "f32", rng.standard_normal(n, dtype=np.float32), [n])
+    b = T.Tensor.from_buf(be, "f32", rng.standard_normal(n, dtype=np.float32), [n])
+
+    def chain():
+        c = ((a * 3.0) + b).relu()
+        c -= 1.0
+        return c
+    for _ in range(3):
+        chain()
+    be.sync()
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        chain()
+    be.sync()
+    ms = (time.perf_counter() - t0) / iters * 1e3
+    out["c2_chain_ms"] = round(ms, 4)
+    out["c2_chain_GBps"] = round(9 * n * 4 / (ms * 1e-3) / 1e9, 1)             # bytes its four kernels move
+    out["c2_chain_bytes"] = 9 * n * 4
+    del a, b
+    rows, cols = 65536, 4096
+    x = T.Tensor.from_buf(be, "f32", rng.standard_normal(rows * cols, dtype=np.float32), [rows, cols])
+    target = T.Tensor.from_buf(be, "f32", rng.random(rows * cols, dtype=np.float32) * 2 - 1, [rows, cols])
+    bias = T.Tensor.from_buf(be, "f32", rng.standard_normal(cols, dtype=np.float32) * 0.1, [cols])
+    for _ in range(2):
+        T.train_step(x, bias, target, 0.01)
+    be.sync()
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        T.train_step(x, bias, target, 0.01)
+    be.sync()
+    out["c5_train_step_ms"] = round((time.perf_counter() - t0) / iters * 1e3, 4)
+    return out
+
+
 def cpu_baseline():
     """The CPU oracle (C++ restatement of the reference's single-threaded Cpu backend) timed on a bounded sample of the
     headline step: 4 of the 16 batch slices of the config-3 broadcast add, and the whole config-4 axis sum."""
@@ -396,6 +440,7 @@ def main():
     w.drop()
     if not args.no_detail:
         detail["api_overhead"] = api_overhead(hip)
+        detail["host_layer"] = host_layer_runs()
 
     out = {
         "metric": "achieved HBM GB/s (% of peak) for broadcast-add + axis-sum, f32, 1 MI355X",

@@ -157,6 +157,18 @@ int32_t rt_reduce_nd(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, ui
                      uint64_t offset, int32_t rank, const uint64_t* shape, const int64_t* strides,
                      void* dst, uint64_t dst_len, int32_t dim);
 
+/* ---- out-of-place unary / scalar ops ---------------------------------------------------------------------------------
+ * dst[0 .. len) = op(src[start .. start + len)); the source is only read.  The trait has in-place ops only: `tensor.relu()`,
+ * `tensor * 3.0` and the other value-returning forms clone the tensor and then run the in-place op (ops/unary/mod.rs:114-126,
+ * ops/scalar/add.rs:93-97), i.e. 4 * N * sizeof(T) of traffic in two passes.  These two entry points give the same result in
+ * one pass over 2 * N * sizeof(T) for a contiguous source (gather other views first); op codes, dtype rules and errors are
+ * those of rt_unary_* / rt_scalar_*.  RT_E_WRONG_DIMS is never returned here (the run is contiguous by construction);
+ * RT_E_OUT_OF_BOUNDS when the run leaves src or len exceeds dst_len. */
+int32_t rt_unary_to(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, uint64_t src_len, uint64_t start, uint64_t len,
+                    void* dst, uint64_t dst_len);
+int32_t rt_scalar_to(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, uint64_t src_len, const void* value,
+                     uint64_t start, uint64_t len, void* dst, uint64_t dst_len);
+
 /* ---- matmul ------------------------------------------------------------------------------------------------------
  * BackendMatMul::matmul (backend/mod.rs:474-485; Cpu backend/cpu.rs:725-951), argument list of protocol Op::Matmul
  * (backend/remote/protocol.rs:269-277): dst[b] = lhs[b] (m x k) * rhs[b] (k x n) for every batch, dst row-major and

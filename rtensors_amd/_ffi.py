@@ -16,7 +16,7 @@ SYMBOLS = [
     "rt_read", "rt_write", "rt_copy", "rt_dump", "rt_equal", "rt_convert",
     "rt_fill_contiguous", "rt_fill_1d_strided", "rt_fill_nd",
     "rt_unary_contiguous", "rt_unary_1d_strided", "rt_unary_nd",
-    "rt_scalar_contiguous", "rt_scalar_1d_strided", "rt_scalar_nd",
+    "rt_scalar_contiguous", "rt_scalar_1d_strided", "rt_scalar_nd", "rt_unary_to", "rt_scalar_to",
     "rt_broadcast", "rt_reduce_flat", "rt_reduce_nd", "rt_gather", "rt_matmul",
     "rt_event_create", "rt_event_record", "rt_event_elapsed_ms", "rt_event_destroy", "rt_mem_stats", "rt_mem_trim",
 ]
@@ -37,6 +37,7 @@ _SIGS = {
     "rt_unary_nd": [vp, i32, i32, vp, u64, u64, i32, u64p, i64p],
     "rt_scalar_contiguous": [vp, i32, i32, vp, u64, vp, u64, u64], "rt_scalar_1d_strided": [vp, i32, i32, vp, u64, vp, u64, i64, u64],
     "rt_scalar_nd": [vp, i32, i32, vp, u64, vp, u64, i32, u64p, i64p],
+    "rt_unary_to": [vp, i32, i32, vp, u64, u64, u64, vp, u64], "rt_scalar_to": [vp, i32, i32, vp, u64, vp, u64, u64, vp, u64],
     "rt_broadcast": [vp, i32, i32, i32, u64p, vp, u64, u64, i64p, vp, u64, u64, i64p, vp, u64, u64, i64p],
     "rt_reduce_flat": [vp, i32, i32, vp, u64, vp, u64, u64, u64],
     "rt_reduce_nd": [vp, i32, i32, vp, u64, u64, i32, u64p, i64p, vp, u64, i32],

@@ -191,6 +191,14 @@ class Hip:
         _check(lib.rt_scalar_nd(self._ctx, buf.dtype, SCALAR[op], buf.ptr, buf.len, v.ctypes.data_as(C.c_void_p), offset, len(shape),
                                 _u64s(shape), _i64s(strides)))
 
+    # out-of-place forms (no counterpart in the trait): dst[0 .. length) = op(src[start .. start + length))
+    def unary_to(self, op: str, src, start, length, dst):
+        _check(lib.rt_unary_to(self._ctx, src.dtype, UNARY[op], src.ptr, src.len, start, length, dst.ptr, dst.len))
+
+    def scalar_to(self, op: str, src, value, start, length, dst):
+        v = _value(src.dtype, value)
+        _check(lib.rt_scalar_to(self._ctx, src.dtype, SCALAR[op], src.ptr, src.len, v.ctypes.data_as(C.c_void_p), start, length, dst.ptr, dst.len))
+
     # The trait's default methods pick one of the three layouts from |stride| contiguity (backend/mod.rs:15-213), which
     # sends a fully reversed view to the `_contiguous` loop with the offset of its *last* element.  Here the whole
     # (offset, shape, strides) goes down and the C side canonicalises it with signed strides.

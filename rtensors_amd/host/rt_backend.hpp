@@ -175,6 +175,13 @@ class Hip {
     void scalar_apply(int op, HipBuf& buf, const Scalar& v, const MetaTensor& m) const {
         check(rt_scalar_nd(raw(), buf.dtype(), op, buf.ptr(), buf.len(), v.bytes, m.offset, (int32_t)m.rank(), m.shape.data(), m.strides.data()));
     }
+    // out-of-place forms over a contiguous run: dst[0 .. len) = op(src[start .. start + len)) in one pass
+    void apply_unary_to(int op, const HipBuf& src, uint64_t start, uint64_t len, HipBuf& dst) const {
+        check(rt_unary_to(raw(), src.dtype(), op, src.ptr(), src.len(), start, len, dst.ptr(), dst.len()));
+    }
+    void scalar_apply_to(int op, const HipBuf& src, const Scalar& v, uint64_t start, uint64_t len, HipBuf& dst) const {
+        check(rt_scalar_to(raw(), src.dtype(), op, src.ptr(), src.len(), v.bytes, start, len, dst.ptr(), dst.len()));
+    }
     // the trait's named methods (apply_relu, scalar_apply_add, ...) in terms of the op codes
 #define RT_UNARY_METHOD(name, CODE) void apply_##name(HipBuf& buf, const MetaTensor& m) const { apply_unary(CODE, buf, m); }
     RT_UNARY_METHOD(neg, RT_U_NEG) RT_UNARY_METHOD(relu, RT_U_RELU) RT_UNARY_METHOD(sigmoid, RT_U_SIGMOID) RT_UNARY_METHOD(silu, RT_U_SILU)

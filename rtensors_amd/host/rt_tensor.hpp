@@ -79,6 +79,17 @@ class Tensor {
     }
     void fill(const Scalar& v) { backend_->fill(*buf_, v, meta_); }
 
+    // Would owned() give a row-major tensor holding exactly this tensor's elements in order?  Then `op(owned())` can be
+    // computed in one pass from this tensor's run into a fresh buffer.  A view: whenever it is a forward contiguous run
+    // (owned() gathers it).  An owner: only when its buffer is that run and nothing else (owned() clones the whole buffer
+    // and keeps the meta).
+    bool one_pass_ok() const {
+        if (size() == 0 || !meta_.is_forward_contiguous()) return false;
+        if (is_view_) return true;
+        return meta_.offset == 0 && buf_->len() == size() && meta_.strides == shape_to_stride(meta_.shape);
+    }
+    Tensor like_row_major() const { return Tensor(*backend_, backend_->alloc_uninit(dtype(), size()), MetaTensor::row_major(meta_.shape)); }
+
     // ---- owned / contiguous -------------------------------------------------------------------------------------------------------
     // TensorBase::owned = Clone: the whole buffer, same meta.  A view's owned() gathers into a fresh row-major buffer.
     Tensor owned() const {
@@ -122,9 +133,19 @@ class Tensor {
     Tensor& operator*=(const Tensor& o) { return binary_assign(o, BinaryOpType::Mul); }
     Tensor& operator/=(const Tensor& o) { return binary_assign(o, BinaryOpType::Div); }
 
-    // ---- scalar operators: `t op= s` is one in-place kernel, `t op s` is owned() + in-place (ops/scalar/add.rs:84-113) ----------------
+    // ---- scalar operators: `t op= s` is one in-place kernel; `t op s` is owned() + in-place in the reference
+    // (ops/scalar/add.rs:84-113), here one out-of-place pass when the operand is a forward contiguous run -----------------------------
     Tensor& scalar_assign(int op, const Scalar& v) { backend_->scalar_apply(op, *buf_, v, meta_); return *this; }
-    Tensor scalar(int op, const Scalar& v) const { Tensor r = owned(); r.scalar_assign(op, v); return r; }
+    Tensor scalar(int op, const Scalar& v) const {
+        if (one_pass_ok()) {
+            Tensor r = like_row_major();
+            backend_->scalar_apply_to(op, *buf_, v, meta_.offset, size(), *r.buf_);
+            return r;
+        }
+        Tensor r = owned();
+        r.scalar_assign(op, v);
+        return r;
+    }
     Tensor& scalar_assign(int op, double v) { return scalar_assign(op, Scalar::from_double(dtype(), v)); }
     Tensor scalar(int op, double v) const { return scalar(op, Scalar::from_double(dtype(), v)); }
     Tensor operator+(double s) const { return scalar(RT_S_ADD, s); }
@@ -140,9 +161,19 @@ class Tensor {
     Tensor& log_inplace(double base) { return scalar_assign(RT_S_LOG, base); }
     Tensor& log1p_inplace(double base) { return scalar_assign(RT_S_LOG1P, base); }
 
-    // ---- unary ops: `t.f()` = owned() + `t.f_inplace()` (ops/unary/mod.rs:114-126) ------------------------------------------------------
+    // ---- unary ops: `t.f()` = owned() + `t.f_inplace()` in the reference (ops/unary/mod.rs:114-126), here one out-of-place pass
+    // when the operand is a forward contiguous run ----------------------------------------------------------------------------------------
     Tensor& unary_inplace(int op) { backend_->apply_unary(op, *buf_, meta_); return *this; }
-    Tensor unary(int op) const { Tensor r = owned(); r.unary_inplace(op); return r; }
+    Tensor unary(int op) const {
+        if (one_pass_ok()) {
+            Tensor r = like_row_major();
+            backend_->apply_unary_to(op, *buf_, meta_.offset, size(), *r.buf_);
+            return r;
+        }
+        Tensor r = owned();
+        r.unary_inplace(op);
+        return r;
+    }
     Tensor operator-() const { return unary(RT_U_NEG); }
 #define RT_TENSOR_UNARY(name, CODE)                            \
     Tensor name() const { return unary(CODE); }                \

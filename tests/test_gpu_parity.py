@@ -698,6 +698,57 @@ def test_more_than_2_31_elements(hip):
     hip.sync()
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f64", "i32", "u8", "i64"])
+def test_out_of_place_unary_and_scalar(hip, dtype):
+    """rt_unary_to / rt_scalar_to: one pass from a contiguous run into a fresh buffer must equal clone + in-place op
+    (ops/unary/mod.rs:114-126, ops/scalar/add.rs:93-97), leave the source untouched, and refuse what the in-place forms refuse."""
+    from rtensors_amd import hip as H
+    rng = np.random.default_rng(31)
+    code = cpu.DTYPE_BY_NAME[dtype]
+    n = 70_001
+    x = rand_values(dtype, n, rng)
+    src = hip.alloc_from_slice(code, x)
+    unary_ops = ["relu", "abs", "neg", "square", "sign", "step", "sigmoid"] if dtype[0] == "f" else (["relu", "abs", "step"] + (["neg"] if dtype[0] == "i" else []))
+    scalar_ops = {"add": 3, "sub": 7, "mul": 3, "div": 3, "leaky_relu": 2, "leaky_grad": 2}
+    for start, length in ((0, n), (4, n - 9), (5, 1000), (n - 3, 3), (16, 0)):
+        m = MetaTensor([length], [1], start)
+        for op in unary_ops:
+            if op in ("step",):
+                with np.errstate(invalid="ignore"):
+                    want = np.where(x[start:start + length] > 0, 1, 0).astype(x.dtype)
+            else:
+                full = x.copy()
+                with np.errstate(all="ignore"):
+                    cpu.unary(code, op, full, m)
+                want = full[start:start + length]
+            dst = hip.alloc(code, max(length, 1) + 2)
+            hip.unary_to(op, src, start, length, dst)
+            got = hip.dump(dst)
+            if op == "sigmoid":
+                assert np.allclose(got[:length], want, rtol=1e-5, atol=1e-5)
+            else:
+                assert got[:length].tobytes() == want.tobytes(), (op, start, length)
+            assert not got[length:].any()                                    # nothing written past the run
+        for op, v in scalar_ops.items():
+            full = x.copy()
+            with np.errstate(all="ignore"):
+                cpu.scalar(code, op, full, v, m)
+            dst = hip.alloc(code, max(length, 1))
+            hip.scalar_to(op, src, v, start, length, dst)
+            assert hip.dump(dst)[:length].tobytes() == full[start:start + length].tobytes(), (op, start, length)
+    assert hip.dump(src).tobytes() == x.tobytes()                            # the source is only read
+    small = hip.alloc(code, 10)
+    for bad in (lambda: hip.unary_to("relu", src, 0, 11, small), lambda: hip.unary_to("relu", src, n - 5, 6, small),
+                lambda: hip.unary_to("relu", src, 0, n, src), lambda: hip.scalar_to("add", src, 1, 0, 11, small)):
+        with pytest.raises(H.TensorError):
+            bad()
+    if dtype[0] != "f":
+        with pytest.raises(H.TensorError):
+            hip.unary_to("sigmoid", src, 0, 10, small)                        # bounded on f32/f64 in the reference
+        with pytest.raises(H.TensorError):
+            hip.scalar_to("div", src, 0, 0, 10, small)                       # integer / 0 scalar
+
+
 # ---- matmul (BackendMatMul::matmul, backend/mod.rs:474-485) --------------------------------------------------------------------------
 MM_SHAPES = [(1, 1, 1, 1), (1, 5, 7, 3), (3, 64, 64, 64), (2, 70, 33, 129), (1, 130, 16, 65), (4, 1, 40, 1), (1, 2, 1, 200)]
 
