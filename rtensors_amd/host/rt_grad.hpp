@@ -60,13 +60,9 @@ class GradContext {
 
     // ops/unary/mod.rs:114-126 (relu = owned + relu_inplace) with the gradient map of 234-252: 1 where input > 0
     Var relu(const Var& a) {
-        Tensor result = a.t.owned();
-        Tensor gmap;
-        const bool track = a.node >= 0;
-        if (track) gmap = result.owned();
-        result.relu_inplace();
-        if (!track) return Var{result, -1};
-        gmap.unary_inplace(RT_U_STEP);
+        Tensor result = a.t.relu();
+        if (a.node < 0) return Var{result, -1};
+        Tensor gmap = a.t.unary(RT_U_STEP);
         Node n;
         n.kind = NodeKind::ReLU;
         n.parents = {a.node};
@@ -77,27 +73,17 @@ class GradContext {
 
     // ops/scalar/mod.rs:149-166: leaky_relu shares GradNode::ReLU; its map is 1 where input > 0 and the slope elsewhere
     Var leaky_relu(const Var& a, double slope) {
-        Tensor result = a.t.owned();
-        Tensor gmap;
-        const bool track = a.node >= 0;
-        if (track) gmap = result.owned();
-        result.leaky_relu_inplace(slope);
-        if (!track) return Var{result, -1};
-        gmap.scalar_assign(RT_S_LEAKY_GRAD, slope);
-        return map_node(result, gmap, a.node);
+        Tensor result = a.t.scalar(RT_S_LEAKY_RELU, slope);
+        if (a.node < 0) return Var{result, -1};
+        return map_node(result, a.t.scalar(RT_S_LEAKY_GRAD, slope), a.node);
     }
 
     // ops/unary/mod.rs:213-232: Abs keeps a map of +1 where input > 0 and -1 elsewhere; backwards_abs (backwards.rs:267-276)
     // multiplies it into the upstream gradient exactly as backwards_relu does
     Var abs(const Var& a) {
-        Tensor result = a.t.owned();
-        Tensor gmap;
-        const bool track = a.node >= 0;
-        if (track) gmap = result.owned();
-        result.abs_inplace();
-        if (!track) return Var{result, -1};
-        gmap.unary_inplace(RT_U_ABS_GRAD);
-        return map_node(result, gmap, a.node);
+        Tensor result = a.t.abs();
+        if (a.node < 0) return Var{result, -1};
+        return map_node(result, a.t.unary(RT_U_ABS_GRAD), a.node);
     }
 
     // ops/linalg/matmul.rs:5-139 + attach_matmul_grad (182-198): the node keeps contiguous copies of both inputs
@@ -119,8 +105,10 @@ class GradContext {
         Tensor gmap = diff.sign();
         diff.abs_inplace();
         Tensor loss = diff.mean();
-        // attach_l1_grad (l1.rs:16-46): grad_map = sign(gmap) / T::from_usize(N), from_usize going through f32
-        Tensor grad_map = gmap.sign() / (double)(float)diff.size();
+        // attach_l1_grad (l1.rs:16-46): grad_map = sign(gmap) / T::from_usize(N), from_usize going through f32.  gmap is
+        // already a sign map and sign(sign(x)) == sign(x) bit for bit (-1, +0, +1; NaN and -0.0 went to +0 the first time),
+        // so the second sign pass is not issued.
+        Tensor grad_map = gmap / (double)(float)diff.size();
         Node n;
         n.kind = NodeKind::L1;
         n.parents = {y.node, target.node};
@@ -223,9 +211,11 @@ class GradContext {
             case NodeKind::BroadcastAdd:                                 // backwards_add / backwards_sub, backwards.rs:27-60
             case NodeKind::BroadcastSub: {
                 std::vector<Tensor> out(2);
-                if (n.parents[0] >= 0) { out[0] = up.owned(); inverse_broadcast_gradient(out[0], n.lhs_strides, n.lhs_shape); }
+                // The reference clones the upstream gradient first (backwards.rs:36-37).  Nothing downstream writes into a
+                // gradient it was handed (the leaf accumulates into its own buffer), so the handle is shared instead.
+                if (n.parents[0] >= 0) { out[0] = up; inverse_broadcast_gradient(out[0], n.lhs_strides, n.lhs_shape); }
                 if (n.parents[1] >= 0) {
-                    out[1] = n.kind == NodeKind::BroadcastSub ? -up : up.owned();
+                    out[1] = n.kind == NodeKind::BroadcastSub ? -up : up;
                     inverse_broadcast_gradient(out[1], n.rhs_strides, n.rhs_shape);
                 }
                 return out;
