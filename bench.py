@@ -39,7 +39,7 @@ def row_major(shape):
 
 class Workloads:
     """Builds the device tensors of configs 1-5 lazily and exposes each kernel as a closure `() -> None` plus its
-    algorithmic bytes (BASELINE.md section 3: unique input elements + output elements, times sizeof)."""
+    algorithmic bytes (unique input elements + output elements, times sizeof)."""
 
     def __init__(self, hip):
         from rtensors_amd import datagen, hip as H
@@ -175,6 +175,26 @@ class Workloads:
         c = self._out("c2cf32", H.F32, 1 << 28)
         shape = [n, n]
         return (lambda: self.hip.broadcast((a, (0, shape, [n, 1])), (b, (0, shape, [1, n])), (c, (0, shape, [n, 1])), "add")), 3 * n * n * 4, n * n
+
+    # ---- buffer equality and dtype conversion (PartialEq of Backend::Buf, Backend::convert) ------------------------------------------
+    def equal_f32(self):
+        H = self.H
+        a = self._gen("c2a", H.F32, 1 << 28, "normal", 1, 0)
+        b = self._out("c2eq", H.F32, 1 << 28)
+        self.hip.copy_range_within(b, a, 0, 0, 1 << 28)
+        return (lambda: self.hip.equal(a, b)), 2 * (1 << 28) * 4, 1 << 28
+
+    def convert_f32_f64(self):
+        H = self.H
+        a = self._gen("c2a", H.F32, 1 << 28, "normal", 1, 0)
+        d = self._out("cvt64", H.F64, 1 << 28)
+        return (lambda: self.hip.convert(a, d)), (1 << 28) * 12, 1 << 28
+
+    def convert_f32_i32(self):
+        H = self.H
+        a = self._gen("c2a", H.F32, 1 << 28, "normal", 1, 0)
+        d = self._out("cvt32", H.I32, 1 << 28)
+        return (lambda: self.hip.convert(a, d)), (1 << 28) * 8, 1 << 28
 
     # ---- matmul (behind the same trait; MFMA-bound, not part of the headline) ---------------------------------------------------------
     def _mm(self, dtype_name, n):

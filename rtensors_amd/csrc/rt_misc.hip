@@ -10,8 +10,23 @@ constexpr int kBlock = 256;
 
 __global__ void set_flag_kernel(int32_t* flag, int32_t v) { *flag = v; }
 
+template <class T> struct alignas(16) Vec16 { T e[16 / sizeof(T)]; };
+constexpr int kVBlock = 128;    // vector kernels: one 16-byte vector (or one group of vectors) per lane
+
 // `==` per element: NaN != NaN, -0.0 == 0.0 (what Box<[T]> == Box<[T]> gives; the reference's device version is
-// K/kernels/utils/buffer_equal.cu:7-39).  All lanes that see a mismatch store the same value.
+// K/kernels/utils/buffer_equal.cu:7-39).  All lanes that see a mismatch store the same value.  Both buffers are read
+// exactly once: one 16-byte vector per lane, non-temporal loads.
+template <class T>
+__global__ __launch_bounds__(kVBlock) void equal_vec_kernel(const Vec16<T>* __restrict__ a, const Vec16<T>* __restrict__ b, size_t nvec, int32_t* flag) {
+    constexpr int N = 16 / sizeof(T);
+    const size_t i = (size_t)blockIdx.x * kVBlock + threadIdx.x;
+    if (i >= nvec) return;
+    const Vec16<T> x = rt_ld16_nt(a + i), y = rt_ld16_nt(b + i);
+    bool bad = false;
+#pragma unroll
+    for (int j = 0; j < N; ++j) bad = bad || !(x.e[j] == y.e[j]);
+    if (bad) *flag = 0;
+}
 template <class T>
 __global__ __launch_bounds__(kBlock) void equal_kernel(const T* __restrict__ a, const T* __restrict__ b, size_t n, int32_t* flag) {
     size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
@@ -23,10 +38,22 @@ __global__ __launch_bounds__(kBlock) void equal_kernel(const T* __restrict__ a, 
 
 template <class T>
 int32_t equal_typed(rt_ctx* ctx, const void* a, const void* b, size_t n) {
-    size_t blocks = (n + kBlock - 1) / kBlock;
-    size_t cap = (size_t)ctx->num_cus * 32;
-    hipLaunchKernelGGL((equal_kernel<T>), dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(kBlock), 0, ctx->stream,
-                       (const T*)a, (const T*)b, n, ctx->flag_dev);
+    constexpr size_t N = 16 / sizeof(T);
+    const bool aligned = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15) == 0;
+    const size_t nvec = aligned ? n / N : 0;
+    if (nvec) {
+        const size_t blocks = (nvec + kVBlock - 1) / kVBlock;
+        if (blocks > 0x7fffffffull) return rt_fail(RT_E_INVALID, "rt_equal: %zu elements is too long for one launch", n);
+        hipLaunchKernelGGL((equal_vec_kernel<T>), dim3((unsigned)blocks), dim3(kVBlock), 0, ctx->stream, (const Vec16<T>*)a, (const Vec16<T>*)b, nvec,
+                           ctx->flag_dev);
+    }
+    const size_t rest = n - nvec * N;
+    if (rest) {
+        size_t blocks = (rest + kBlock - 1) / kBlock;
+        size_t cap = (size_t)ctx->num_cus * 32;
+        hipLaunchKernelGGL((equal_kernel<T>), dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(kBlock), 0, ctx->stream,
+                           (const T*)a + nvec * N, (const T*)b + nvec * N, rest, ctx->flag_dev);
+    }
     RT_HIP(hipGetLastError());
     return RT_OK;
 }
@@ -66,12 +93,57 @@ __global__ __launch_bounds__(kBlock) void convert_kernel(const S* __restrict__ s
     for (; i < n; i += step) d[i] = convert_one<D, S>(s[i]);
 }
 
+// Non-temporal access of a naturally aligned pack of 1, 2, 4, 8 or 16 bytes.
+template <int BYTES> struct pack_word;
+template <> struct pack_word<1> { typedef uint8_t type; };
+template <> struct pack_word<2> { typedef uint16_t type; };
+template <> struct pack_word<4> { typedef uint32_t type; };
+template <> struct pack_word<8> { typedef uint64_t type; };
+template <> struct pack_word<16> { typedef rt_u32x4 type; };
+template <class P> __device__ __forceinline__ P pack_ld_nt(const P* p) {
+    typedef typename pack_word<sizeof(P)>::type W;
+    return __builtin_bit_cast(P, __builtin_nontemporal_load(reinterpret_cast<const W*>(p)));
+}
+template <class P> __device__ __forceinline__ void pack_st_nt(P* p, const P& v) {
+    typedef typename pack_word<sizeof(P)>::type W;
+    __builtin_nontemporal_store(__builtin_bit_cast(W, v), reinterpret_cast<W*>(p));
+}
+
+// A lane converts E = 16 / max(sizeof S, sizeof D) elements: one 16-byte vector of the wider type and one 16-, 8-, 4-, 2-
+// or 1-byte pack of the narrower one, so that every load and every store instruction of a wave covers one contiguous run.
+// (Giving each lane 16 bytes of the narrower type and several vectors of the wider one leaves every wide access
+// half-coalesced: f32 -> f64 measured 4.0 TB/s that way against 4.8 TB/s for one element per lane.)
+template <class S, class D>
+__global__ __launch_bounds__(kVBlock) void convert_vec_kernel(const S* __restrict__ s, D* __restrict__ d, size_t ngroups) {
+    constexpr int E = 16 / (sizeof(S) > sizeof(D) ? sizeof(S) : sizeof(D));
+    struct alignas(E * sizeof(S)) SP { S e[E]; };
+    struct alignas(E * sizeof(D)) DP { D e[E]; };
+    const size_t i = (size_t)blockIdx.x * kVBlock + threadIdx.x;
+    if (i >= ngroups) return;
+    const SP in = pack_ld_nt(reinterpret_cast<const SP*>(s) + i);
+    DP out;
+#pragma unroll
+    for (int k = 0; k < E; ++k) out.e[k] = convert_one<D, S>(in.e[k]);
+    pack_st_nt(reinterpret_cast<DP*>(d) + i, out);
+}
+
 template <class S, class D>
 int32_t convert_go(rt_ctx* ctx, const void* s, void* d, size_t n) {
-    size_t blocks = (n + kBlock - 1) / kBlock;
-    size_t cap = (size_t)ctx->num_cus * 32;
-    hipLaunchKernelGGL((convert_kernel<S, D>), dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(kBlock), 0, ctx->stream,
-                       (const S*)s, (D*)d, n);
+    constexpr size_t E = 16 / (sizeof(S) > sizeof(D) ? sizeof(S) : sizeof(D));
+    const bool aligned = ((reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) & 15) == 0;
+    const size_t ngroups = aligned ? n / E : 0;
+    if (ngroups) {
+        const size_t blocks = (ngroups + kVBlock - 1) / kVBlock;
+        if (blocks > 0x7fffffffull) return rt_fail(RT_E_INVALID, "convert: %zu elements is too long for one launch", n);
+        hipLaunchKernelGGL((convert_vec_kernel<S, D>), dim3((unsigned)blocks), dim3(kVBlock), 0, ctx->stream, (const S*)s, (D*)d, ngroups);
+    }
+    const size_t rest = n - ngroups * E;
+    if (rest) {
+        size_t blocks = (rest + kBlock - 1) / kBlock;
+        size_t cap = (size_t)ctx->num_cus * 32;
+        hipLaunchKernelGGL((convert_kernel<S, D>), dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(kBlock), 0, ctx->stream,
+                           (const S*)s + ngroups * E, (D*)d + ngroups * E, rest);
+    }
     RT_HIP(hipGetLastError());
     return RT_OK;
 }
