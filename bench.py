@@ -176,6 +176,29 @@ class Workloads:
         shape = [n, n]
         return (lambda: self.hip.broadcast((a, (0, shape, [n, 1])), (b, (0, shape, [1, n])), (c, (0, shape, [n, 1])), "add")), 3 * n * n * 4, n * n
 
+    # ---- layouts without a unit-stride inner dim (one element per lane kernels) --------------------------------------------------------
+    def strided1d_relu(self):
+        """In-place relu on every second element of a 2^28 f32 buffer: every cache line is read and written, half of it is used."""
+        H = self.H
+        c = self._out("c2cf32", H.F32, 1 << 28)
+        return (lambda: self.hip.unary_1d_strided("relu", c, 0, 2, 1 << 27)), 2 * (1 << 27) * 4, 1 << 27
+
+    def nd_step2_relu(self):
+        """In-place relu on m[:, ::2] of a 16384 x 16384 f32 matrix."""
+        H = self.H
+        n = 16384
+        c = self._out("c2cf32", H.F32, n * n)
+        return (lambda: self.hip.unary_nd("relu", c, 0, [n, n // 2], [n, 2])), 2 * (n * n // 2) * 4, n * n // 2
+
+    def generic_step2_add(self):
+        """z[:, ::2] = x[:, ::2] + y[:, ::2] on 16384 x 16384 f32 matrices: no operand has a unit-stride inner dim."""
+        H = self.H
+        n = 16384
+        a = self._gen("c2a", H.F32, n * n, "normal", 1, 0); b = self._gen("c2b", H.F32, n * n, "normal", 1, 1)
+        c = self._out("c2cf32", H.F32, n * n)
+        m = (0, [n, n // 2], [n, 2])
+        return (lambda: self.hip.broadcast((a, m), (b, m), (c, m), "add")), 3 * (n * n // 2) * 4, n * n // 2
+
     # ---- buffer equality and dtype conversion (PartialEq of Backend::Buf, Backend::convert) ------------------------------------------
     def equal_f32(self):
         H = self.H

@@ -155,25 +155,39 @@ struct GenArgs {
     int64_t stride[3][RT_MAX_RANK];
 };
 
+constexpr int kGU = 4;          // elements in flight per lane in the generic kernel
+
 template <class T, int OP>
 __global__ __launch_bounds__(kBlock) void bin_generic_kernel(const T* l, const T* r, T* d, GenArgs a, uint32_t n) {
-    uint32_t i = blockIdx.x * kBlock + threadIdx.x;
-    const uint32_t step = gridDim.x * kBlock;
-    for (; i < n; i += step) {
-        uint32_t rem = i;
-        int64_t ol = 0, orr = 0, od = 0;
+    // a block owns kGU * kBlock consecutive elements per trip, lane t the elements t, t + kBlock, ...; all loads are issued
+    // before the first store
+    constexpr uint32_t span = kGU * kBlock, step = kBlock;
+    for (uint64_t base = (uint64_t)blockIdx.x * span; base < n; base += (uint64_t)gridDim.x * span) {
+        const uint32_t i = (uint32_t)base + threadIdx.x;
+        int64_t od[kGU];
+        T x[kGU], y[kGU];
 #pragma unroll
-        for (int k = RT_MAX_RANK - 1; k >= 0; --k) {
-            if (k < a.rank) {
-                uint32_t q = fd_div(rem, a.div[k]);
-                uint32_t c = rem - q * a.shape[k];
-                ol += (int64_t)c * a.stride[0][k];
-                orr += (int64_t)c * a.stride[1][k];
-                od += (int64_t)c * a.stride[2][k];
-                rem = q;
+        for (int u = 0; u < kGU; ++u) {
+            uint32_t rem = min(i + u * step, n - 1);     // lanes past the end recompute the last element and do not store it
+            int64_t ol = 0, orr = 0;
+            od[u] = 0;
+#pragma unroll
+            for (int k = RT_MAX_RANK - 1; k >= 0; --k) {
+                if (k < a.rank) {
+                    uint32_t q = fd_div(rem, a.div[k]);
+                    uint32_t c = rem - q * a.shape[k];
+                    ol += (int64_t)c * a.stride[0][k];
+                    orr += (int64_t)c * a.stride[1][k];
+                    od[u] += (int64_t)c * a.stride[2][k];
+                    rem = q;
+                }
             }
+            x[u] = l[ol];
+            if constexpr (OP != kOpCopy) y[u] = r[orr]; else y[u] = x[u];
         }
-        d[od] = bin_apply<OP, T>(l[ol], r[orr]);
+#pragma unroll
+        for (int u = 0; u < kGU; ++u)
+            if (i + u * step < n) d[od[u]] = bin_apply<OP, T>(x[u], y[u]);
     }
 }
 
@@ -352,9 +366,8 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
             g.div[k] = make_fastdiv(g.shape[k]);
             for (int o = 0; o < 3; ++o) g.stride[o][k] = k < rank ? dsc.stride[o][k] : 0;
         }
-        size_t blocks = ((size_t)count + kBlock - 1) / kBlock;
-        size_t cap = (size_t)ctx->num_cus * 64;
-        hipLaunchKernelGGL((bin_generic_kernel<T, OP>), dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(kBlock), 0, s,
+        size_t blocks = ((size_t)count + kGU * kBlock - 1) / (kGU * kBlock);
+        hipLaunchKernelGGL((bin_generic_kernel<T, OP>), dim3((unsigned)blocks), dim3(kBlock), 0, s,
                            l + dsc.offset[0], r + dsc.offset[1], d + dsc.offset[2], g, (uint32_t)count);
     } else {
         size_t cap = (size_t)ctx->num_cus * 64;

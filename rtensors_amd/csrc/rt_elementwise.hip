@@ -187,6 +187,7 @@ template <class T> struct alignas(16) Vec16 { T e[16 / sizeof(T)]; };
 
 constexpr int kBlock = 256;     // element-per-lane kernels
 constexpr int kCBlock = 128;    // contiguous kernel: one 16-byte vector per lane, 128 lanes per block
+constexpr int kEU = 4;          // element-per-lane kernels: elements in flight per lane
 
 // Body: `nvec` 16-byte vectors starting at the 16-byte aligned address `p`.  One vector per lane and small blocks:
 // on MI355X this shape (with non-temporal accesses for read-modify-write, plain stores for write-only) was the
@@ -207,13 +208,23 @@ __global__ __launch_bounds__(256) void ew_contig_kernel(Vec16<T>* __restrict__ p
 // Edges of a contiguous run that do not fill a 16-byte vector, and 1-D strided views: one element per lane.
 template <class T, class F>
 __global__ __launch_bounds__(kBlock) void ew_strided_kernel(T* __restrict__ p, int64_t stride, size_t n, F f) {
-    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    const size_t step = (size_t)gridDim.x * kBlock;
-    for (; i < n; i += step) {
-        T* q = p + (int64_t)i * stride;
-        T x = zero_of<T>();
-        if constexpr (F::kReads) x = *q;
-        *q = f(x);
+    // A block owns kEU * kBlock consecutive elements per trip, lane t the elements t, t + kBlock, ...; all loads are issued
+    // before the first store (loads and stores retire in issue order, so a load -> store -> load chain would wait for
+    // every store)
+    const size_t span = (size_t)kEU * kBlock;
+    for (size_t base = (size_t)blockIdx.x * span; base < n; base += (size_t)gridDim.x * span) {
+        T x[kEU];
+#pragma unroll
+        for (int u = 0; u < kEU; ++u) {
+            const size_t i = base + (size_t)u * kBlock + threadIdx.x;
+            x[u] = zero_of<T>();
+            if constexpr (F::kReads) { if (i < n) x[u] = p[(int64_t)i * stride]; }
+        }
+#pragma unroll
+        for (int u = 0; u < kEU; ++u) {
+            const size_t i = base + (size_t)u * kBlock + threadIdx.x;
+            if (i < n) p[(int64_t)i * stride] = f(x[u]);
+        }
     }
 }
 
@@ -227,24 +238,32 @@ struct NdArgs {
 // N-d view, fewer than 2^31 elements: lane i handles the i-th element in row-major order of the collapsed dims.
 template <class T, class F>
 __global__ __launch_bounds__(kBlock) void ew_nd_kernel(T* __restrict__ p, NdArgs a, uint32_t n, F f) {
-    uint32_t i = blockIdx.x * kBlock + threadIdx.x;
-    const uint32_t step = gridDim.x * kBlock;
-    for (; i < n; i += step) {
-        uint32_t rem = i;
-        int64_t off = 0;
+    // a block owns kEU * kBlock consecutive elements per trip (n < 2^31, so base + span does not wrap)
+    constexpr uint32_t span = kEU * kBlock;
+    for (uint64_t base = (uint64_t)blockIdx.x * span; base < n; base += (uint64_t)gridDim.x * span) {
+        const uint32_t i = (uint32_t)base + threadIdx.x;
+        constexpr uint32_t step = kBlock;
+        int64_t off[kEU];
+        T x[kEU];
 #pragma unroll
-        for (int d = RT_MAX_RANK - 1; d >= 0; --d) {
-            if (d < a.rank) {
-                uint32_t q = fd_div(rem, a.div[d]);
-                uint32_t c = rem - q * a.shape[d];
-                off += (int64_t)c * a.stride[d];
-                rem = q;
+        for (int u = 0; u < kEU; ++u) {
+            uint32_t rem = min(i + u * step, n - 1);
+            off[u] = 0;
+#pragma unroll
+            for (int d = RT_MAX_RANK - 1; d >= 0; --d) {
+                if (d < a.rank) {
+                    uint32_t q = fd_div(rem, a.div[d]);
+                    uint32_t c = rem - q * a.shape[d];
+                    off[u] += (int64_t)c * a.stride[d];
+                    rem = q;
+                }
             }
+            x[u] = zero_of<T>();
+            if constexpr (F::kReads) { if (i + u * step < n) x[u] = p[off[u]]; }
         }
-        T* q = p + off;
-        T x = zero_of<T>();
-        if constexpr (F::kReads) x = *q;
-        *q = f(x);
+#pragma unroll
+        for (int u = 0; u < kEU; ++u)
+            if (i + u * step < n) p[off[u]] = f(x[u]);
     }
 }
 
@@ -397,8 +416,8 @@ int32_t launch_view(rt_ctx* ctx, T* base, const NdDesc& d, uint64_t count, F f) 
     if (d.rank == 0) return launch_contig<T, F>(ctx, p, 1, f);
     if (d.rank == 1) {
         if (d.stride[0][0] == 1) return launch_contig<T, F>(ctx, p, (size_t)d.shape[0], f);
-        size_t blocks = ((size_t)d.shape[0] + kBlock - 1) / kBlock;
-        hipLaunchKernelGGL((ew_strided_kernel<T, F>), dim3(capped_grid(blocks, (size_t)ctx->num_cus * 32)), dim3(kBlock), 0, ctx->stream,
+        size_t blocks = ((size_t)d.shape[0] + kEU * kBlock - 1) / (kEU * kBlock);
+        hipLaunchKernelGGL((ew_strided_kernel<T, F>), dim3(capped_grid(blocks, 0x7fffffffull)), dim3(kBlock), 0, ctx->stream,
                            p, d.stride[0][0], (size_t)d.shape[0], f);
         RT_HIP(hipGetLastError());
         return RT_OK;
@@ -455,8 +474,8 @@ int32_t launch_view(rt_ctx* ctx, T* base, const NdDesc& d, uint64_t count, F f) 
             return RT_OK;
         }
     }
-    size_t blocks = ((size_t)count + kBlock - 1) / kBlock;
-    hipLaunchKernelGGL((ew_nd_kernel<T, F>), dim3(capped_grid(blocks, (size_t)ctx->num_cus * 64)), dim3(kBlock), 0, ctx->stream,
+    size_t blocks = ((size_t)count + kEU * kBlock - 1) / (kEU * kBlock);
+    hipLaunchKernelGGL((ew_nd_kernel<T, F>), dim3(capped_grid(blocks, 0x7fffffffull)), dim3(kBlock), 0, ctx->stream,
                        p, a, (uint32_t)count, f);
     RT_HIP(hipGetLastError());
     return RT_OK;
