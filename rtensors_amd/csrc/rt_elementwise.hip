@@ -303,17 +303,30 @@ __global__ __launch_bounds__(kCBlock) void ew_rows_kernel(T* __restrict__ p, Row
     const uint32_t c = (tile * a.tpr + tx) * N;
     if (c >= a.L) return;
     const uint32_t g_begin = chunk * a.gchunk, g_end = min(a.G, g_begin + a.gchunk);
-    for (uint32_t g = g_begin + ty; g < g_end; g += gy) {
-        T* rowp = p + off + (int64_t)g * a.gstride;
-        if (c + N <= a.L) {
-            Vec16<T>* v = reinterpret_cast<Vec16<T>*>(rowp + c);
-            Vec16<T> w;
-            if constexpr (F::kReads) w = rt_ld16_nt(v);
+    if (c + N <= a.L) {
+        // two rows per trip, both loads issued before the first store
+        for (uint32_t g = g_begin + ty; g < g_end; g += 2 * gy) {
+            const bool two = g + gy < g_end;
+            Vec16<T>* v0 = reinterpret_cast<Vec16<T>*>(p + off + (int64_t)g * a.gstride + c);
+            Vec16<T>* v1 = reinterpret_cast<Vec16<T>*>(p + off + (int64_t)(two ? g + gy : g) * a.gstride + c);
+            Vec16<T> w0 = {}, w1 = {};
+            if constexpr (F::kReads) {
+                w0 = rt_ld16_nt(v0);
+                if (two) w1 = rt_ld16_nt(v1);
+            }
 #pragma unroll
-            for (int j = 0; j < N; ++j) w.e[j] = f(w.e[j]);
-            if constexpr (F::kReads) rt_st16_nt(v, w);
-            else *v = w;
-        } else {
+            for (int j = 0; j < N; ++j) { w0.e[j] = f(w0.e[j]); w1.e[j] = f(w1.e[j]); }
+            if constexpr (F::kReads) {
+                rt_st16_nt(v0, w0);
+                if (two) rt_st16_nt(v1, w1);
+            } else {
+                *v0 = w0;
+                if (two) *v1 = w1;
+            }
+        }
+    } else {
+        for (uint32_t g = g_begin + ty; g < g_end; g += gy) {
+            T* rowp = p + off + (int64_t)g * a.gstride;
             for (uint32_t k = c; k < a.L; ++k) {
                 T x = zero_of<T>();
                 if constexpr (F::kReads) x = rowp[k];
