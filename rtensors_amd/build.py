@@ -73,7 +73,7 @@ def build(force: bool = False, jobs: int = 8) -> None:
         out = os.path.join(LIB, lib)
         deps = [objs[s] for s in ss]
         if force or _stale(out, deps):
-            r = subprocess.run(["hipcc", f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", out] + deps + ["-ldl"], capture_output=True, text=True)
+            r = subprocess.run(["hipcc", f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", out] + deps + ["-ldl", "-lpthread"], capture_output=True, text=True)
             if r.returncode != 0:
                 raise RuntimeError(f"link of {lib} failed:\n{_filter(r.stdout + r.stderr)}")
             print(f"[build] linked {lib}", file=sys.stderr)

@@ -43,6 +43,9 @@ struct rt_ctx {
     // scratch for two-stage reductions (partials), grown on demand, reused across calls
     void* scratch = nullptr;
     size_t scratch_bytes = 0;
+    // pinned staging ring for large host<->device transfers (allocated by the first one), one event per slot
+    void* stage[4] = {nullptr, nullptr, nullptr, nullptr};
+    hipEvent_t stage_ev[4] = {nullptr, nullptr, nullptr, nullptr};
     // rocBLAS handle bound to `stream` (created by the first f32/f64 matmul) and the function that destroys it
     void* blas = nullptr;
     int (*blas_destroy)(void*) = nullptr;

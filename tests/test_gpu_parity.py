@@ -119,6 +119,40 @@ def test_allocator_reuses_blocks(hip):
     assert hip.mem_stats()["device_allocs"] == before
 
 
+def test_large_transfers_round_trip(hip):
+    """Host <-> device copies above 4 MiB go through the pinned staging ring in 8 MiB chunks split over four copy threads:
+    sizes on and around every boundary must come back byte for byte, also when several threads transfer at once."""
+    import threading
+    from rtensors_amd import hip as H
+    rng = np.random.default_rng(77)
+    mib = 1 << 20
+    sizes = [4 * mib - 1, 4 * mib, 4 * mib + 1, 8 * mib - 64, 8 * mib, 8 * mib + 3, 32 * mib, 32 * mib + 5, 41 * mib + 777]
+    for n in sizes:
+        x = rng.integers(0, 256, size=n, dtype=np.uint8)
+        b = hip.alloc_from_slice(H.U8, x)
+        assert hip.dump(b).tobytes() == x.tobytes(), n
+        y = rng.integers(0, 256, size=n, dtype=np.uint8)
+        hip.copy_from_slice(b, y)
+        assert hip.dump(b).tobytes() == y.tobytes(), n
+    x64 = rng.standard_normal(3 * mib + 11)                     # 24 MiB + 88 bytes of f64
+    assert hip.dump(hip.alloc_from_slice(H.F64, x64)).tobytes() == x64.tobytes()
+    errors = []
+    def worker(seed):
+        try:
+            r = np.random.default_rng(seed)
+            be = H.Hip.new(0)                                   # own context: own staging ring, shared copy threads
+            for _ in range(3):
+                v = r.integers(0, 256, size=9 * mib + seed, dtype=np.uint8)
+                if be.dump(be.alloc_from_slice(H.U8, v)).tobytes() != v.tobytes():
+                    errors.append(seed)
+        except Exception as e:                                  # noqa: BLE001
+            errors.append(repr(e))
+    ts = [threading.Thread(target=worker, args=(s,)) for s in (1, 2, 3)]
+    [t.start() for t in ts]
+    [t.join() for t in ts]
+    assert not errors, errors
+
+
 UNARY_EXACT = ["neg", "relu", "abs", "sqrt", "floor", "ceil", "round", "trunc", "reciprocal", "square", "cube", "sign"]
 UNARY_TOL = ["sigmoid", "silu", "tanh", "ln", "expm1", "ln1p", "sin", "cos", "tan", "asin", "acos", "atan", "sinh", "cosh", "asinh",
              "acosh", "atanh", "rsqrt", "exp"]
