@@ -160,6 +160,18 @@ class Workloads:
     def copy(self): return self._c2("copy")
     def fill(self): return self._c2("fill")
 
+    def clone(self):
+        """Backend::copy of a 1 GiB buffer (what TensorBase::clone / owned() issue), allocation from the cache included."""
+        H = self.H
+        a = self._gen("c2a", H.F32, 1 << 28, "normal", 1, 0)
+        return (lambda: self.hip.copy(a)), 2 * (1 << 28) * 4, 1 << 28
+
+    def copy_range(self):
+        H = self.H
+        a = self._gen("c2a", H.F32, 1 << 28, "normal", 1, 0)
+        c = self._out("c2cf32", H.F32, 1 << 28)
+        return (lambda: self.hip.copy_range_within(c, a, 0, 0, 1 << 28)), 2 * (1 << 28) * 4, 1 << 28
+
     def view_relu(self):
         # in-place relu on the left half of a (16384,16384) f32 matrix: a non-contiguous view with unit-stride rows
         H = self.H

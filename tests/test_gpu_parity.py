@@ -102,6 +102,15 @@ def test_buffers_and_transfers(hip):
             hip.write(b, 1000, x[0])
         with pytest.raises(H.TensorError):
             hip.copy_range_within(c, b, 950, 0, 100)
+    # device copies large enough for the vector copy kernel: equal and unequal 16-byte phases, ragged ends
+    big = rng.integers(0, 256, size=100_003, dtype=np.uint8)
+    src = hip.alloc_from_slice(H.U8, big)
+    assert hip.dump(hip.copy(src)).tobytes() == big.tobytes()
+    for dst_off, src_off, length in ((0, 0, 100_003), (16, 32, 70_001), (5, 21, 50_000), (3, 4, 60_000), (7, 7, 99_990), (1, 17, 4096), (9, 9, 15)):
+        dst = hip.alloc(H.U8, 100_003)
+        hip.copy_range_within(dst, src, dst_off, src_off, length)
+        want = np.zeros(100_003, dtype=np.uint8); want[dst_off:dst_off + length] = big[src_off:src_off + length]
+        assert hip.dump(dst).tobytes() == want.tobytes(), (dst_off, src_off, length)
     nan = hip.alloc_from_slice(H.F32, np.array([1.0, np.nan], np.float32))
     assert not (nan == hip.copy(nan))                                     # NaN != NaN, like Box<[f32]> ==
     pz = hip.alloc_from_slice(H.F32, np.array([0.0], np.float32)); nz = hip.alloc_from_slice(H.F32, np.array([-0.0], np.float32))
