@@ -188,6 +188,21 @@ class Workloads:
         shape = [n, n]
         return (lambda: self.hip.broadcast((a, (0, shape, [n, 1])), (b, (0, shape, [1, n])), (c, (0, shape, [n, 1])), "add")), 3 * n * n * 4, n * n
 
+    # ---- reductions over short rows / narrow columns / a short middle axis (1 GiB f32 each) -------------------------------------------
+    def _red(self, outer, R, inner):
+        H = self.H
+        a = self._gen("c2a", H.F32, 1 << 28, "normal", 1, 0)
+        d = self._out("redout", H.F32, 1 << 26)
+        shape, strides = [outer, R, inner], [R * inner, inner, 1]
+        return (lambda: self.hip.apply_reduce_contiguous_nd((a, (0, shape, strides)), d, 1, "sum")), (outer * R * inner + outer * inner) * 4, outer * R * inner
+
+    def red_rows32(self): return self._red(1 << 23, 32, 1)
+    def red_rows256(self): return self._red(1 << 20, 256, 1)
+    def red_inner3(self): return self._red(1, (1 << 28) // 3, 3)
+    def red_inner100(self): return self._red(1, (1 << 28) // 100, 100)
+    def red_mid64(self): return self._red(65536, 64, 64)
+    def red_mid4(self): return self._red(1 << 20, 4, 64)
+
     # ---- layouts without a unit-stride inner dim (one element per lane kernels) --------------------------------------------------------
     def strided1d_relu(self):
         """In-place relu on every second element of a 2^28 f32 buffer: every cache line is read and written, half of it is used."""

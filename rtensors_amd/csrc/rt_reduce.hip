@@ -295,11 +295,210 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(const T* __restrict
     }
 }
 
+// ---- short rows: 1 <= R <= 1024 ----------------------------------------------------------------------------------------------
+// One lane (or wave) per row reads a short row with a stride of R elements between lanes: at R = 32 that measured 0.32 TB/s.
+// Here a block copies the contiguous run holding its rows into LDS with 16-byte coalesced loads (row r at pitch R | 1, so that
+// lanes walking different rows hit different banks), then groups of T lanes fold one row each from LDS.
+constexpr uint32_t kRowsTileBytes = 32768;
+struct RowsTileArgs {
+    uint64_t rows;
+    uint32_t R, pitch, rpb, T;          // row length, LDS pitch, rows per block, lanes per row (power of two <= 64)
+    FastDiv32 r_div;
+};
+
+template <int OP, class T>
+__global__ __launch_bounds__(kBlock) void reduce_rows_tile_kernel(const T* __restrict__ src, T* __restrict__ out, RowsTileArgs a, uint64_t count) {
+    constexpr uint32_t N = 16 / sizeof(T);
+    __shared__ alignas(16) T tile[kRowsTileBytes / sizeof(T)];
+    const uint64_t row0 = (uint64_t)blockIdx.x * a.rpb;
+    const uint32_t nrows = (uint32_t)(a.rows - row0 < a.rpb ? a.rows - row0 : a.rpb);
+    const uint32_t ne = nrows * a.R;
+    const T* p = src + row0 * a.R;
+    auto put = [&](uint32_t e, T v) {
+        const uint32_t r = fd_div(e, a.r_div);
+        tile[r * a.pitch + (e - r * a.R)] = v;
+    };
+    uint32_t head = (uint32_t)(((16 - (reinterpret_cast<uintptr_t>(p) & 15)) & 15) / sizeof(T));
+    if (head > ne) head = ne;
+    if (threadIdx.x < head) put(threadIdx.x, p[threadIdx.x]);
+    const uint32_t nvec = (ne - head) / N;
+    const Vec16<T>* pv = reinterpret_cast<const Vec16<T>*>(p + head);
+    constexpr int U = 4;
+    for (uint32_t v0 = threadIdx.x; v0 < nvec; v0 += U * kBlock) {
+        Vec16<T> x[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (v0 + u * kBlock < nvec) x[u] = rt_ld16_nt(pv + v0 + u * kBlock);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (v0 + u * kBlock < nvec) {
+#pragma unroll
+                for (uint32_t j = 0; j < N; ++j) put(head + (v0 + u * kBlock) * N + j, x[u].e[j]);
+            }
+        }
+    }
+    const uint32_t tb = head + nvec * N;
+    if (tb + threadIdx.x < ne) put(tb + threadIdx.x, p[tb + threadIdx.x]);
+    __syncthreads();
+    const uint32_t g = threadIdx.x / a.T, j = threadIdx.x & (a.T - 1), groups = kBlock / a.T;
+    for (uint32_t r = g; r < nrows; r += groups) {
+        Acc<OP, T> acc;
+        acc.init();
+        const T* row = tile + r * a.pitch;
+        for (uint32_t k = j; k < a.R; k += a.T) acc.push(row[k], k);
+        for (uint32_t d = a.T / 2; d >= 1; d >>= 1) {
+            Acc<OP, T> o;
+            o.v = shfl_down_t<T>(acc.v, (int)d);
+            if constexpr (Acc<OP, T>::kTrack) o.pos = shfl_down_t<uint64_t>(acc.pos, (int)d); else o.pos = 0;
+            if (j + d < a.T) acc.merge(o);
+        }
+        if (j == 0) out[row0 + r] = finalize<OP, T>(acc.v, count);
+    }
+}
+
+// ---- narrow columns: inner < 128, long R ------------------------------------------------------------------------------------
+// With lanes along `inner` only `inner` of 64 lanes would work.  Here the (R, inner) slab of one outer index is read as one
+// contiguous stream in tiles of S = Tn * VW elements, S a multiple of inner, so that lane t always meets the same VW columns
+// (element t*VW + j of every tile) and rows tile*L + (t*VW + j) / inner, L = S / inner rows per tile, in ascending order.  The
+// lanes that share a column are combined through LDS at the end (ties by position, so the first extremum still wins).
+struct ColsNarrowArgs {
+    uint64_t R, outer;
+    uint32_t inner, Tn, L, splits;      // columns, active lanes, rows per tile, segments per outer index
+    uint64_t seg_tiles;                 // tiles per segment
+    FastDiv32 inner_div;
+};
+
+template <int OP, class T, int VW>
+__global__ __launch_bounds__(kBlock) void reduce_cols_narrow_kernel(const T* __restrict__ src, T* __restrict__ out, ColsNarrowArgs a, uint64_t count,
+                                                                    int last) {
+    constexpr bool kTrack = Acc<OP, T>::kTrack;
+    struct alignas(sizeof(T) * VW) VecW { T e[VW]; };
+    __shared__ T sv[kBlock * VW];
+    __shared__ uint64_t sp[kTrack ? kBlock * VW : 1];
+    const uint64_t o = blockIdx.x / a.splits;
+    const uint32_t seg = (uint32_t)(blockIdx.x - o * a.splits);
+    const uint32_t t = threadIdx.x;
+    const uint32_t S = a.Tn * VW;
+    const uint64_t slab = a.R * a.inner;                       // elements of one outer index
+    const T* base = src + o * slab;
+    Acc<OP, T> acc[VW];
+    uint32_t krow[VW];
+#pragma unroll
+    for (int j = 0; j < VW; ++j) { acc[j].init(); krow[j] = fd_div(t * VW + j, a.inner_div); }
+    if (t < a.Tn) {
+        const uint64_t tile_begin = (uint64_t)seg * a.seg_tiles;
+        uint64_t tile_end = tile_begin + a.seg_tiles;
+        const uint64_t ntiles = (a.R + a.L - 1) / a.L;
+        if (tile_end > ntiles) tile_end = ntiles;
+        constexpr int U = 4;
+        for (uint64_t tl = tile_begin; tl < tile_end; tl += U) {
+            VecW x[U];
+            bool full[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const uint64_t e = (tl + u) * S + (uint64_t)t * VW;
+                full[u] = tl + u < tile_end && e + VW <= slab;
+                if (full[u]) {
+                    if constexpr (sizeof(VecW) == 16) x[u] = rt_ld16_nt(reinterpret_cast<const VecW*>(base + e));
+                    else x[u].e[0] = __builtin_nontemporal_load(base + e);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const uint64_t k0 = (tl + u) * a.L;
+                if (full[u]) {
+#pragma unroll
+                    for (int j = 0; j < VW; ++j) acc[j].push(x[u].e[j], k0 + krow[j]);
+                } else if (tl + u < tile_end) {                // the slab ends inside this lane's vector
+                    const uint64_t e = (tl + u) * S + (uint64_t)t * VW;
+#pragma unroll
+                    for (int j = 0; j < VW; ++j)
+                        if (e + j < slab) acc[j].push(base[e + j], k0 + krow[j]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < VW; ++j) {
+        sv[t * VW + j] = acc[j].v;
+        if constexpr (kTrack) sp[t * VW + j] = acc[j].pos;
+    }
+    __syncthreads();
+    if (t < a.inner) {
+        Acc<OP, T> r;
+        r.v = sv[t];
+        r.pos = kTrack ? sp[t] : 0;
+        for (uint32_t q = 1; q < a.L; ++q) {
+            Acc<OP, T> x;
+            x.v = sv[t + q * a.inner];
+            x.pos = kTrack ? sp[t + q * a.inner] : 0;
+            r.merge(x);
+        }
+        out[((uint64_t)seg * a.outer + o) * a.inner + t] = last ? finalize<OP, T>(r.v, count) : r.v;
+    }
+}
+
+// ---- short reduced axis: R <= 32, any inner -----------------------------------------------------------------------------------
+// One lane per VW neighbouring outputs walks the R inputs of each (they are `inner` apart); consecutive lanes read consecutive
+// addresses, and everything one outer index needs is one contiguous slab, so every cache line is fetched once.
+template <int OP, class T, int VW>
+__global__ __launch_bounds__(kBlock) void reduce_cols_short_kernel(const T* __restrict__ src, T* __restrict__ out, uint32_t R, uint64_t inner,
+                                                                   uint32_t inner_vecs, FastDiv32 iv_div, uint64_t nvec_out, uint64_t count) {
+    struct alignas(sizeof(T) * VW) VecW { T e[VW]; };
+    const uint64_t idx = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (idx >= nvec_out) return;
+    const uint32_t o = fd_div((uint32_t)idx, iv_div);           // nvec_out < 2^32 on this path
+    const uint32_t iv = (uint32_t)idx - o * inner_vecs;
+    const T* p = src + (uint64_t)o * R * inner + (uint64_t)iv * VW;
+    Acc<OP, T> acc[VW];
+#pragma unroll
+    for (int j = 0; j < VW; ++j) acc[j].init();
+    constexpr int U = 4;
+    for (uint32_t k = 0; k < R; k += U) {
+        VecW x[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (k + u < R) {
+                if constexpr (sizeof(VecW) == 16) x[u] = rt_ld16_nt(reinterpret_cast<const VecW*>(p + (uint64_t)(k + u) * inner));
+                else x[u].e[0] = __builtin_nontemporal_load(p + (uint64_t)(k + u) * inner);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (k + u < R) {
+#pragma unroll
+                for (int j = 0; j < VW; ++j) acc[j].push(x[u].e[j], k + u);
+            }
+        }
+    }
+    T* q = out + (uint64_t)o * inner + (uint64_t)iv * VW;
+#pragma unroll
+    for (int j = 0; j < VW; ++j) q[j] = finalize<OP, T>(acc[j].v, count);
+}
+
+constexpr uint64_t kRowsTileMaxR = 1024;
+
 // ---- host planning ------------------------------------------------------------------------------------------------------
 template <int OP, class T>
 int32_t rows_stage(rt_ctx* ctx, const T* src, T* out, uint64_t rows, uint64_t R, uint64_t count, bool allow_split) {
     hipStream_t s = ctx->stream;
     if (rows == 0) return RT_OK;
+    if (R >= 1 && R <= kRowsTileMaxR && count == R) {          // short rows (not the second stage of a split reduction)
+        RowsTileArgs a;
+        a.rows = rows;
+        a.R = (uint32_t)R;
+        a.pitch = a.R | 1u;
+        a.rpb = (uint32_t)(kRowsTileBytes / sizeof(T)) / a.pitch;
+        a.r_div = make_fastdiv(a.R);
+        uint32_t t = 1;                                           // lanes per row: fill the block, at most one wave, at most R
+        while (t < 64 && (uint64_t)t * 2 * a.rpb <= (uint64_t)kBlock && t * 2 <= a.R) t <<= 1;
+        a.T = t;
+        const uint64_t blocks = (rows + a.rpb - 1) / a.rpb;
+        if (blocks >= (1ull << 31)) return rt_fail(RT_E_INVALID, "reduce: too many rows for one launch");
+        hipLaunchKernelGGL((reduce_rows_tile_kernel<OP, T>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, out, a, count);
+        RT_HIP(hipGetLastError());
+        return RT_OK;
+    }
     if (R < 64) {
         uint64_t blocks = (rows + kBlock - 1) / kBlock;
         if (blocks >= (1ull << 31)) return rt_fail(RT_E_INVALID, "reduce: too many rows for one launch");
@@ -398,11 +597,74 @@ int32_t cols_launch(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t 
 }
 
 template <int OP, class T>
+int32_t cols_narrow(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t R, uint64_t inner) {
+    constexpr uint32_t N = 16 / sizeof(T);
+    const bool vec = (reinterpret_cast<uintptr_t>(src) & 15) == 0 && (outer == 1 || (R * inner) % N == 0);
+    const uint32_t vw = vec ? N : 1;
+    uint32_t g = (uint32_t)inner, h = vw;                      // gcd(inner, vw)
+    while (h) { uint32_t t = g % h; g = h; h = t; }
+    const uint32_t innerp = (uint32_t)inner / g;               // lanes per period: Tn * vw must be a multiple of inner
+    ColsNarrowArgs a;
+    a.R = R;
+    a.outer = outer;
+    a.inner = (uint32_t)inner;
+    a.Tn = (uint32_t)kBlock / innerp * innerp;
+    a.L = a.Tn * vw / (uint32_t)inner;
+    a.inner_div = make_fastdiv((uint32_t)inner);
+    const uint64_t ntiles = (R + a.L - 1) / a.L;
+    const uint64_t want = (uint64_t)ctx->num_cus * 4;
+    uint64_t splits = outer >= want ? 1 : (want + outer - 1) / outer;
+    if (splits > ntiles / 8) splits = ntiles / 8;              // at least 8 tiles per block
+    if (splits < 1) splits = 1;
+    a.seg_tiles = (ntiles + splits - 1) / splits;
+    splits = (ntiles + a.seg_tiles - 1) / a.seg_tiles;
+    a.splits = (uint32_t)splits;
+    const uint64_t blocks = outer * splits;
+    if (blocks >= (1ull << 31)) return rt_fail(RT_E_INVALID, "reduce: too many outputs for one launch");
+    T* dst1 = out;
+    if (splits > 1) {
+        void* scratch = nullptr;
+        RT_TRY(rt_scratch(ctx, (size_t)(splits * outer * inner) * sizeof(T), &scratch));
+        dst1 = (T*)scratch;
+    }
+    const int last = splits == 1 ? 1 : 0;
+    if (vec) hipLaunchKernelGGL((reduce_cols_narrow_kernel<OP, T, N>), dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream, src, dst1, a, R, last);
+    else hipLaunchKernelGGL((reduce_cols_narrow_kernel<OP, T, 1>), dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream, src, dst1, a, R, last);
+    RT_HIP(hipGetLastError());
+    if (splits == 1) return RT_OK;
+    // second stage: the partials are (splits, outer * inner); fold the segments in order (mean divides by the original count)
+    const uint64_t inner2 = outer * inner;
+    const uint64_t tiles2 = (inner2 + RT_WAVE - 1) / RT_WAVE;
+    hipLaunchKernelGGL((reduce_cols_kernel<OP, T, 1>), dim3((unsigned)tiles2), dim3(kBlock), 0, ctx->stream, dst1, out, (uint64_t)splits, inner2, (uint64_t)1,
+                       (uint32_t)tiles2, 1u, (uint64_t)splits, R, 1);
+    RT_HIP(hipGetLastError());
+    return RT_OK;
+}
+
+template <int OP, class T>
 int32_t reduce_typed(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t R, uint64_t inner) {
     if (outer == 0 || inner == 0) return RT_OK;
     if (OP == RT_R_MEAN && !is_flt<T>::value && R == 0) return rt_fail(RT_E_ARITH, "reduce: integer mean over an empty axis divides by zero");
     if (inner == 1) return rows_stage<OP, T>(ctx, src, out, outer, R, R, true);
     constexpr int N = 16 / sizeof(T);
+    // Which kernel: measured on MI355X over 1 GiB of f32 (sum), TB/s -- rows of 8 / 32 / 100 / 256 elements 4.8 / 5.2 / 5.4 / 5.7;
+    // columns with inner 3 / 17 / 100 5.0 / 5.0 / 4.8; (65536, 64, 64) 6.4; (2^20, 4, 64) 5.4.  One lane or one wave per short row
+    // gave 0.3-2.3, lanes along a narrow inner 0.2-1.2.
+    if (R <= 32 && inner <= 1024) {                                             // short reduced axis: a lane per output vector
+        const bool v = (inner % N == 0) && ((reinterpret_cast<uintptr_t>(src) & 15) == 0);
+        const uint64_t ivecs = v ? inner / N : inner;
+        if (ivecs < (1ull << 31) && outer * ivecs < (1ull << 31)) {
+            const uint64_t nvec_out = outer * ivecs;
+            const uint64_t blocks = (nvec_out + kBlock - 1) / kBlock;
+            if (v) hipLaunchKernelGGL((reduce_cols_short_kernel<OP, T, N>), dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream, src, out, (uint32_t)R, inner,
+                                      (uint32_t)ivecs, make_fastdiv((uint32_t)ivecs), nvec_out, R);
+            else hipLaunchKernelGGL((reduce_cols_short_kernel<OP, T, 1>), dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream, src, out, (uint32_t)R, inner,
+                                    (uint32_t)ivecs, make_fastdiv((uint32_t)ivecs), nvec_out, R);
+            RT_HIP(hipGetLastError());
+            return RT_OK;
+        }
+    }
+    if (inner < 128 && R >= 64 && outer < (1ull << 20)) return cols_narrow<OP, T>(ctx, src, out, outer, R, inner);
     const bool vec = (inner % N == 0) && ((reinterpret_cast<uintptr_t>(src) & 15) == 0) && ((reinterpret_cast<uintptr_t>(out) & 15) == 0);
     if (vec) return cols_launch<OP, T, N>(ctx, src, out, outer, R, inner, R, true);
     return cols_launch<OP, T, 1>(ctx, src, out, outer, R, inner, R, true);

@@ -741,6 +741,56 @@ def test_more_than_2_31_elements(hip):
     hip.sync()
 
 
+def _check_reduce(hip, dtype, outer, R, inner, rng, offset=0):
+    """All five ops over (outer, R, inner) along the middle axis, against the oracle (which folds in index order)."""
+    code = cpu.DTYPE_BY_NAME[dtype]
+    npd = cpu.NP_DTYPE[code]
+    n = outer * R * inner
+    x = rand_values(dtype, n + offset, rng, -50, 50)
+    if dtype[0] == "f" and n >= 8:
+        x[offset:offset + 4] = [0.0, -0.0, np.nan, -0.0]
+        x[offset + n - 2:offset + n] = [-0.0, 0.0]
+    src = hip.alloc_from_slice(code, x)
+    shape = [outer, R, inner]
+    m = MetaTensor(shape, [R * inner, inner, 1], offset)
+    ops = ("sum", "max", "min", "mean", "prod") if dtype[0] == "f" else ("sum", "max", "min")
+    for op in ops:
+        with np.errstate(all="ignore"):
+            want = cpu.reduce_nd(code, op, x, m, 1, honour_offset=True)
+        dst = hip.alloc(code, outer * inner)
+        hip.apply_reduce_contiguous_nd((src, (offset, shape, [R * inner, inner, 1])), dst, 1, op)
+        got = hip.dump(dst)
+        if dtype[0] != "f" or op in ("max", "min"):
+            assert got.tobytes() == want.tobytes(), (dtype, op, outer, R, inner, offset)
+        elif op == "prod":
+            ok = np.isclose(got.astype(np.float64), want.astype(np.float64), rtol=1e-4 if dtype == "f32" else 1e-10, atol=0, equal_nan=True)
+            assert ok.all() or R > 64, (dtype, op, outer, R, inner)
+        else:
+            rel = 1e-5 if dtype == "f32" else 1e-12
+            v = np.nan_to_num(np.abs(x[offset:offset + n].astype(np.float64))).reshape(outer, R, inner).sum(axis=1).reshape(-1)
+            scale = v / (R if op == "mean" else 1)
+            fin = np.isfinite(want.astype(np.float64))
+            assert (np.isnan(got) == np.isnan(want)).all(), (dtype, op, outer, R, inner)
+            assert (np.abs(got.astype(np.float64) - want.astype(np.float64))[fin] <= rel * scale[fin] + 1e-300).all(), (dtype, op, outer, R, inner)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64", "i32", "u8", "i64"])
+def test_reduction_shapes_short_rows_narrow_columns_short_axis(hip, dtype):
+    """The shapes that have kernels of their own: rows of 1..1025 elements (LDS-tiled), narrow inner dims (streamed with the
+    lanes pinned to columns), reduced axes of at most 32 elements (a lane per output); odd counts, unaligned offsets, and the
+    hand-over points to the general kernels."""
+    rng = np.random.default_rng(abs(hash(dtype)) % 2 ** 31)
+    for R in (1, 2, 3, 7, 8, 31, 32, 33, 63, 64, 65, 100, 255, 256, 1000, 1023, 1024, 1025):
+        for rows in (1, 77, 1000):
+            _check_reduce(hip, dtype, rows, R, 1, rng, offset=int(rng.integers(0, 5)))
+    for inner in (2, 3, 4, 5, 17, 64, 100, 127, 128):
+        for R, outer in ((64, 3), (1000, 1), (5003, 2), (70001, 1)):
+            _check_reduce(hip, dtype, outer, R, inner, rng, offset=int(rng.integers(0, 5)))
+    for R in (1, 2, 4, 5, 16, 31, 32, 33):
+        for inner, outer in ((2, 1000), (3, 1), (64, 50), (100, 7), (1024, 3), (1028, 2)):
+            _check_reduce(hip, dtype, outer, R, inner, rng, offset=int(rng.integers(0, 5)))
+
+
 @pytest.mark.parametrize("dtype", ["f32", "f64", "i32", "u8", "i64"])
 def test_out_of_place_unary_and_scalar(hip, dtype):
     """rt_unary_to / rt_scalar_to: one pass from a contiguous run into a fresh buffer must equal clone + in-place op
