@@ -92,4 +92,10 @@ static bool vec_ok(const T* base, const NdDesc& dsc, int o) {
 template <class T, int OP>
 bool tile_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* l, const T* r, T* d, int32_t* status);
 
+// Row-major copy of a view whose second-to-last dim is short (2..64) and unit-stride in the source while the last dim steps
+// by exactly that extent: interleaved -> planar, e.g. (H*W, C) pixels into (C, H*W) planes.  Returns true when taken.
+// Instantiated in rt_broadcast_tile.hip for the four word sizes the gather uses.
+template <class T>
+bool planar_copy_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* src, T* dst, int32_t* status);
+
 }  // namespace rtb

@@ -545,6 +545,23 @@ def test_gather_transposed_views(hip, dtype):
                 assert gv.contiguous().dump().tobytes() == ov.to_numpy().tobytes(), (dtype, shape, perm, variant)
 
 
+@pytest.mark.parametrize("dtype", ["f32", "u8", "i16", "f64"])
+def test_gather_interleaved_to_planar(hip, dtype):
+    """(.., M, C) -> (.., C, M) with a short C (pixels to planes): the LDS-staged planar copy, with odd plane lengths, a batch
+    dim, an offset start, and C at both ends of its range; C = 65 and a strided channel dim go to the general kernels."""
+    rng = np.random.default_rng(23)
+    for (batch, M, C) in [(1, 1000, 3), (2, 4099, 4), (3, 257, 2), (1, 300, 64), (1, 700, 65), (2, 1 << 15, 3), (1, 5000, 17)]:
+        vals = rand_values(dtype, batch * M * C + 5, rng)
+        o, g = OTensor.from_buf(dtype, vals, [batch * M * C + 5]), G(hip, dtype, vals, [batch * M * C + 5])
+        for start in (0, 5):
+            ov = o.slice(0, Slice(start, start + batch * M * C, 1)); gv = g.slice(0, Slice(start, start + batch * M * C, 1))
+            ov = OTensor(ov.dtype, ov.buf, MetaTensor([batch, M, C], [M * C, C, 1], start), is_view=True).permute([0, 2, 1])
+            gv = type(g)(g.backend, g.buf, MetaTensor([batch, M, C], [M * C, C, 1], start), is_view=True).permute([0, 2, 1])
+            assert gv.contiguous().dump().tobytes() == ov.to_numpy().tobytes(), (dtype, batch, M, C, start)
+            ov2, gv2 = ov.slice(1, Slice(0, None, 2)), gv.slice(1, Slice(0, None, 2))          # every second channel: not this kernel
+            assert gv2.contiguous().dump().tobytes() == ov2.to_numpy().tobytes(), (dtype, batch, M, C, start, "strided")
+
+
 def test_convert(hip):
     from rtensors_amd import hip as H
     rng = np.random.default_rng(8)
