@@ -280,7 +280,10 @@ struct RowsArgs {
     int64_t gstride;
 };
 
-template <class T, class F>
+// NT: every row covers whole 128-byte lines, so the view is streamed with non-temporal accesses.  Rows that share cache lines
+// with elements outside the view go through the cache normally, so that the partly written lines are merged in L2 instead of
+// being written to memory piece by piece ((2^24, 16)[:, :15] f32 relu: 0.92 ms non-temporal, 0.62 ms cached).
+template <class T, class F, bool NT>
 __global__ __launch_bounds__(kCBlock) void ew_rows_kernel(T* __restrict__ p, RowsArgs a, F f) {
     constexpr int N = 16 / sizeof(T);
     uint32_t b = blockIdx.x;
@@ -311,12 +314,17 @@ __global__ __launch_bounds__(kCBlock) void ew_rows_kernel(T* __restrict__ p, Row
             Vec16<T>* v1 = reinterpret_cast<Vec16<T>*>(p + off + (int64_t)(two ? g + gy : g) * a.gstride + c);
             Vec16<T> w0 = {}, w1 = {};
             if constexpr (F::kReads) {
-                w0 = rt_ld16_nt(v0);
-                if (two) w1 = rt_ld16_nt(v1);
+                if constexpr (NT) {
+                    w0 = rt_ld16_nt(v0);
+                    if (two) w1 = rt_ld16_nt(v1);
+                } else {
+                    w0 = *v0;
+                    if (two) w1 = *v1;
+                }
             }
 #pragma unroll
             for (int j = 0; j < N; ++j) { w0.e[j] = f(w0.e[j]); w1.e[j] = f(w1.e[j]); }
-            if constexpr (F::kReads) {
+            if constexpr (F::kReads && NT) {
                 rt_st16_nt(v0, w0);
                 if (two) rt_st16_nt(v1, w1);
             } else {
@@ -460,11 +468,13 @@ int32_t launch_view(rt_ctx* ctx, T* base, const NdDesc& d, uint64_t count, F f) 
         r.L = (uint32_t)d.shape[d.rank - 1];
         r.G = (uint32_t)d.shape[gdim];
         r.gstride = d.stride[0][gdim];
+        bool whole_lines = ((uint64_t)r.L * sizeof(T)) % 128 == 0 && (reinterpret_cast<uintptr_t>(p) & 127) == 0 && (r.gstride * (int64_t)sizeof(T)) % 128 == 0;
         uint64_t outer = 1;
         for (int k = 0; k < gdim; ++k) {
             r.oshape[r.nouter] = (uint32_t)d.shape[k];
             r.odiv[r.nouter] = make_fastdiv((uint32_t)d.shape[k]);
             r.ostride[r.nouter] = d.stride[0][k];
+            if ((d.stride[0][k] * (int64_t)sizeof(T)) % 128 != 0) whole_lines = false;
             outer *= (uint64_t)d.shape[k];
             r.nouter++;
         }
@@ -482,7 +492,8 @@ int32_t launch_view(rt_ctx* ctx, T* base, const NdDesc& d, uint64_t count, F f) 
         r.nchunks_div = make_fastdiv(r.nchunks);
         const uint64_t blocks = outer * r.nchunks * r.tiles;
         if (blocks < (1ull << 31)) {
-            hipLaunchKernelGGL((ew_rows_kernel<T, F>), dim3((unsigned)blocks), dim3(kCBlock), 0, ctx->stream, p, r, f);
+            if (whole_lines) hipLaunchKernelGGL((ew_rows_kernel<T, F, true>), dim3((unsigned)blocks), dim3(kCBlock), 0, ctx->stream, p, r, f);
+            else hipLaunchKernelGGL((ew_rows_kernel<T, F, false>), dim3((unsigned)blocks), dim3(kCBlock), 0, ctx->stream, p, r, f);
             RT_HIP(hipGetLastError());
             return RT_OK;
         }
