@@ -24,14 +24,12 @@ namespace {
 // One vector per lane, non-temporal loads and stores: every byte is touched exactly once.
 template <class T, int OP>
 __global__ __launch_bounds__(kRBlock) void bin_contig_kernel(const Vec16<T>* l, const Vec16<T>* r, Vec16<T>* d, size_t nvec) {
-    constexpr int N = 16 / sizeof(T);
     const size_t i = (size_t)blockIdx.x * kRBlock + threadIdx.x;
     if (i >= nvec) return;
     Vec16<T> a = rt_ld16_nt(l + i);
     Vec16<T> b;
     if constexpr (OP != kOpCopy) b = rt_ld16_nt(r + i); else b = a;
-#pragma unroll
-    for (int j = 0; j < N; ++j) a.e[j] = bin_apply<OP, T>(a.e[j], b.e[j]);
+    bin_apply_vec<OP, T>(a, b);
     rt_st16_nt(d + i, a);
 }
 
@@ -87,37 +85,45 @@ __global__ __launch_bounds__(kRBlock) void bin_rows_kernel(const T* l, const T* 
 
     if (c + N <= a.L) {
         const bool l_fixed = (a.gstride[0] == 0), r_fixed = (a.gstride[1] == 0);
-        Vec16<T> lh, rh;                                        // operands that do not move along the loop dim
-        if (l_fixed) lh = load_vec<T, LM>(l + ol, c, a.istride[0], false);
-        if (r_fixed) rh = load_vec<T, RM>(r + orr, c, a.istride[1], false);
+        // Vectors cross the control flow below as four 32-bit words: held as arrays of 1-byte elements they would be split into
+        // sixteen separate registers at every select and re-packed before the store.
+        typedef rt_u32x4 Raw;
+        auto ldl = [&](int64_t off, bool nt) { return load_raw<T, LM>(l + off, c, a.istride[0], nt); };
+        auto ldr = [&](int64_t off, bool nt) { return load_raw<T, RM>(r + off, c, a.istride[1], nt); };
+        auto combine_store = [&](Raw x, Raw y, uint32_t g) {
+            Vec16<T> xv = __builtin_bit_cast(Vec16<T>, x);
+            bin_apply_vec<OP, T>(xv, __builtin_bit_cast(Vec16<T>, y));
+            rt_st16_nt(reinterpret_cast<Vec16<T>*>(d + od + (int64_t)g * a.gstride[2] + c), xv);
+        };
+        Raw lh = {}, rh = {};                                   // operands that do not move along the loop dim
+        if (l_fixed) lh = ldl(ol, false);
+        if (r_fixed) rh = ldr(orr, false);
         if constexpr (GU == 1) {
             // short loop (two steps per lane by default): load, combine, store
             for (uint32_t g = g_begin + ty; g < g_end; g += gy) {
-                Vec16<T> x = l_fixed ? lh : load_vec<T, LM>(l + ol + (int64_t)g * a.gstride[0], c, a.istride[0], ntl);
-                Vec16<T> y;
+                Raw x = l_fixed ? lh : ldl(ol + (int64_t)g * a.gstride[0], ntl);
+                Raw y;
                 if constexpr (OP == kOpCopy) y = x;
-                else y = r_fixed ? rh : load_vec<T, RM>(r + orr + (int64_t)g * a.gstride[1], c, a.istride[1], ntr);
-#pragma unroll
-                for (int j = 0; j < N; ++j) x.e[j] = bin_apply<OP, T>(x.e[j], y.e[j]);
-                rt_st16_nt(reinterpret_cast<Vec16<T>*>(d + od + (int64_t)g * a.gstride[2] + c), x);
+                else y = r_fixed ? rh : ldr(orr + (int64_t)g * a.gstride[1], ntr);
+                combine_store(x, y, g);
             }
         } else {
             // long loop (an expensive operand is held in registers while the block walks the loop dim): GU steps per
             // batch, the next batch's loads issued before this batch's stores.  Loads and stores retire in issue order,
             // so a load issued after a store would wait for that store's acknowledgement.
-            Vec16<T> xn[GU], yn[GU];
+            Raw xn[GU], yn[GU];
             auto load_batch = [&](uint32_t g0) {
 #pragma unroll
                 for (int u = 0; u < GU; ++u) {
                     const uint32_t g = min(g0 + u * gy, g_end - 1);
-                    if (!l_fixed) xn[u] = load_vec<T, LM>(l + ol + (int64_t)g * a.gstride[0], c, a.istride[0], ntl);
-                    if constexpr (OP != kOpCopy) { if (!r_fixed) yn[u] = load_vec<T, RM>(r + orr + (int64_t)g * a.gstride[1], c, a.istride[1], ntr); }
+                    if (!l_fixed) xn[u] = ldl(ol + (int64_t)g * a.gstride[0], ntl);
+                    if constexpr (OP != kOpCopy) { if (!r_fixed) yn[u] = ldr(orr + (int64_t)g * a.gstride[1], ntr); }
                 }
             };
             uint32_t g0 = g_begin + ty;
             if (g0 < g_end) load_batch(g0);
             for (; g0 < g_end; g0 += gy * GU) {
-                Vec16<T> x[GU], y[GU];
+                Raw x[GU], y[GU];
 #pragma unroll
                 for (int u = 0; u < GU; ++u) {
                     x[u] = l_fixed ? lh : xn[u];
@@ -127,11 +133,7 @@ __global__ __launch_bounds__(kRBlock) void bin_rows_kernel(const T* l, const T* 
 #pragma unroll
                 for (int u = 0; u < GU; ++u) {
                     const uint32_t g = g0 + u * gy;
-                    if (g < g_end) {
-#pragma unroll
-                        for (int j = 0; j < N; ++j) x[u].e[j] = bin_apply<OP, T>(x[u].e[j], y[u].e[j]);
-                        rt_st16_nt(reinterpret_cast<Vec16<T>*>(d + od + (int64_t)g * a.gstride[2] + c), x[u]);
-                    }
+                    if (g < g_end) combine_store(x[u], y[u], g);
                 }
             }
         }
@@ -222,8 +224,7 @@ __global__ __launch_bounds__(kRBlock) void bin_flat_kernel(const T* l, const T* 
         }
     }
     if constexpr (OP == kOpCopy) y = x;
-#pragma unroll
-    for (int j = 0; j < N; ++j) x.e[j] = bin_apply<OP, T>(x.e[j], y.e[j]);
+    bin_apply_vec<OP, T>(x, y);
     rt_st16_nt(reinterpret_cast<Vec16<T>*>(d) + v, x);
 }
 

@@ -50,27 +50,52 @@ template <int OP, class T> __device__ __forceinline__ T bin_apply(T a, T b) {
 
 template <class T> struct alignas(16) Vec16 { T e[16 / sizeof(T)]; };
 
+// x = x OP y on a whole vector.  1-byte add / subtract (and every bool op) run on four elements per 32-bit word.
+template <int OP, class T> __device__ __forceinline__ void bin_apply_vec(Vec16<T>& x, const Vec16<T>& y) {
+    if constexpr (sizeof(T) == 1 && (OP == RT_ADD || OP == RT_SUB || (OP == RT_MUL && is_bool<T>::value))) {
+        rt_words4 a = __builtin_bit_cast(rt_words4, x);
+        const rt_words4 b = __builtin_bit_cast(rt_words4, y);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if constexpr (is_bool<T>::value) a.w[j] = OP == RT_ADD ? (a.w[j] | b.w[j]) : (OP == RT_SUB ? (a.w[j] ^ b.w[j]) : (a.w[j] & b.w[j]));
+            else a.w[j] = OP == RT_ADD ? rt_add_4x8(a.w[j], b.w[j]) : rt_sub_4x8(a.w[j], b.w[j]);
+        }
+        x = __builtin_bit_cast(Vec16<T>, a);
+    } else {
+#pragma unroll
+        for (int j = 0; j < (int)(16 / sizeof(T)); ++j) x.e[j] = bin_apply<OP, T>(x.e[j], y.e[j]);
+    }
+}
+
 constexpr int kBlock = 256;     // generic kernels
 constexpr int kRBlock = 128;    // contig / rows kernels: small blocks, one 16-byte vector per lane per step
 
 enum Mode : int { M_VEC = 0, M_BCAST = 1, M_ELEM = 2 };
 
+// One 16-byte vector of an operand's row as four 32-bit words (the form that crosses selects and loops without being split into
+// per-element registers), and the same as elements.
+template <class T, int MODE>
+__device__ __forceinline__ rt_u32x4 load_raw(const T* __restrict__ rowp, uint32_t c, int64_t istride, bool nt) {
+    constexpr int N = 16 / sizeof(T);
+    if constexpr (MODE == M_VEC) {
+        const rt_u32x4* q = reinterpret_cast<const rt_u32x4*>(rowp + c);
+        return nt ? __builtin_nontemporal_load(q) : *q;
+    } else {
+        Vec16<T> v;
+        if constexpr (MODE == M_BCAST) {
+            T x = rowp[0];
+#pragma unroll
+            for (int j = 0; j < N; ++j) v.e[j] = x;
+        } else {
+#pragma unroll
+            for (int j = 0; j < N; ++j) v.e[j] = rowp[(int64_t)(c + j) * istride];
+        }
+        return __builtin_bit_cast(rt_u32x4, v);
+    }
+}
 template <class T, int MODE>
 __device__ __forceinline__ Vec16<T> load_vec(const T* __restrict__ rowp, uint32_t c, int64_t istride, bool nt) {
-    constexpr int N = 16 / sizeof(T);
-    Vec16<T> v;
-    if constexpr (MODE == M_VEC) {
-        const Vec16<T>* q = reinterpret_cast<const Vec16<T>*>(rowp + c);
-        v = nt ? rt_ld16_nt(q) : rt_ld16(q);
-    } else if constexpr (MODE == M_BCAST) {
-        T x = rowp[0];
-#pragma unroll
-        for (int j = 0; j < N; ++j) v.e[j] = x;
-    } else {
-#pragma unroll
-        for (int j = 0; j < N; ++j) v.e[j] = rowp[(int64_t)(c + j) * istride];
-    }
-    return v;
+    return __builtin_bit_cast(Vec16<T>, load_raw<T, MODE>(rowp, c, istride, nt));
 }
 
 static inline bool mult_of(int64_t v, int64_t n) { return v % n == 0; }

@@ -157,8 +157,8 @@ __global__ __launch_bounds__(kTBlock) void bin_tile_kernel(const T* xt, const T*
                 if (k0 + kk < a.K) {
                     const Vec16<T> xv = *reinterpret_cast<const Vec16<T>*>(&tile[kk][lane * N]);
                     Vec16<T> out;
-#pragma unroll
-                    for (int j = 0; j < N; ++j) out.e[j] = x_left ? bin_apply<OP, T>(xv.e[j], ov[i].e[j]) : bin_apply<OP, T>(ov[i].e[j], xv.e[j]);
+                    if (x_left) { out = xv; bin_apply_vec<OP, T>(out, ov[i]); }
+                    else { out = ov[i]; bin_apply_vec<OP, T>(out, xv); }
                     rt_st16_nt(reinterpret_cast<Vec16<T>*>(drow + (int64_t)(k0 + kk) * a.tstride[2] + c), out);
                 }
             }

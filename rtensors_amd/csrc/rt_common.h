@@ -118,6 +118,23 @@ template <class V> __device__ __forceinline__ void rt_st16_nt(V* p, const V& v) 
     __builtin_nontemporal_store(__builtin_bit_cast(rt_u32x4, v), reinterpret_cast<rt_u32x4*>(p));
 }
 
+// Four 1-byte integers packed in a 32-bit word, wrapping add / subtract of every byte at once: the low seven bits are
+// combined with the top bits masked so that no carry or borrow crosses a byte, then the top bits are restored by xor.
+// Per-byte code (sub-dword selects and re-packing) costs about twice the vector instructions per 16-byte vector, enough
+// to pull a streaming pass over 1-byte elements from ~6.55 down to ~6.1 TB/s on MI355X.
+__device__ __forceinline__ uint32_t rt_add_4x8(uint32_t a, uint32_t b) {
+    return ((a & 0x7f7f7f7fu) + (b & 0x7f7f7f7fu)) ^ ((a ^ b) & 0x80808080u);
+}
+__device__ __forceinline__ uint32_t rt_sub_4x8(uint32_t a, uint32_t b) {
+    return ((a | 0x80808080u) - (b & 0x7f7f7f7fu)) ^ ((a ^ ~b) & 0x80808080u);
+}
+// bytes with the sign bit set -> 0xff, others -> 0x00
+__device__ __forceinline__ uint32_t rt_negmask_4x8(uint32_t a) {
+    uint32_t s = (a >> 7) & 0x01010101u;
+    return (s << 8) - s;
+}
+struct rt_words4 { uint32_t w[4]; };
+
 // Division of a 32-bit numerator by a runtime-constant divisor via multiply-high (round-up method); exact for
 // every n < 2^31 and 1 <= d < 2^31.
 struct FastDiv32 {

@@ -107,8 +107,21 @@ __device__ __forceinline__ float m_abs(float x) { return fabsf(x); }
 __device__ __forceinline__ double m_abs(double x) { return fabs(x); }
 
 // ---- functors ---------------------------------------------------------------------------------------------------
+// A functor over 1-byte elements may offer `packed`: the same op on four elements in one 32-bit word (rt_common.h).
 template <int OP, class T> struct UnaryF {
     static constexpr bool kReads = true;
+    static constexpr bool kPacked = sizeof(T) == 1 && (OP == RT_U_RELU || OP == RT_U_NEG || OP == RT_U_ABS);
+    __device__ __forceinline__ uint32_t packed(uint32_t w) const {
+        if constexpr (!is_sint<T>::value) {
+            // unsigned and bool: relu and abs are the identity; bool negation is 0 ^ x
+            if constexpr (OP == RT_U_NEG && is_uint<T>::value) return rt_sub_4x8(0u, w);
+            else return w;
+        } else {
+            if constexpr (OP == RT_U_RELU) return w & ~rt_negmask_4x8(w);
+            else if constexpr (OP == RT_U_NEG) return rt_sub_4x8(0u, w);
+            else { const uint32_t m = rt_negmask_4x8(w); return rt_sub_4x8(w ^ m, m); }   // two's complement of the negative bytes
+        }
+    }
     __device__ __forceinline__ T operator()(T x) const {
         if constexpr (OP == RT_U_RELU) {                                  // cpu.rs:650-657
             return gt0(x) ? x : zero_of<T>();
@@ -161,7 +174,15 @@ template <int OP, class T> struct UnaryF {
 
 template <int OP, class T> struct ScalarF {
     static constexpr bool kReads = true;
+    static constexpr bool kPacked = sizeof(T) == 1 && (OP == RT_S_ADD || OP == RT_S_SUB || (OP == RT_S_MUL && is_bool<T>::value));
     T v;
+    __device__ __forceinline__ uint32_t packed(uint32_t w) const {
+        uint8_t b;
+        __builtin_memcpy(&b, &v, 1);
+        const uint32_t v4 = (uint32_t)b * 0x01010101u;
+        if constexpr (is_bool<T>::value) return OP == RT_S_ADD ? (w | v4) : (OP == RT_S_SUB ? (w ^ v4) : (w & v4));
+        else return OP == RT_S_ADD ? rt_add_4x8(w, v4) : rt_sub_4x8(w, v4);
+    }
     __device__ __forceinline__ T operator()(T x) const {
         if constexpr (OP == RT_S_ADD) return w_add<T>(x, v);                                      // cpu.rs:678-696
         else if constexpr (OP == RT_S_SUB) return w_sub<T>(x, v);
@@ -178,12 +199,25 @@ template <int OP, class T> struct ScalarF {
 
 template <class T> struct FillF {
     static constexpr bool kReads = false;
+    static constexpr bool kPacked = false;
     T v;
     __device__ __forceinline__ T operator()(T) const { return v; }
 };
 
 // ---- kernels ------------------------------------------------------------------------------------------------------
 template <class T> struct alignas(16) Vec16 { T e[16 / sizeof(T)]; };
+
+template <class T, class F> __device__ __forceinline__ void apply_vec(Vec16<T>& v, const F& f) {
+    if constexpr (F::kPacked) {
+        rt_words4 w = __builtin_bit_cast(rt_words4, v);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) w.w[j] = f.packed(w.w[j]);
+        v = __builtin_bit_cast(Vec16<T>, w);
+    } else {
+#pragma unroll
+        for (int j = 0; j < (int)(16 / sizeof(T)); ++j) v.e[j] = f(v.e[j]);
+    }
+}
 
 constexpr int kBlock = 256;     // element-per-lane kernels
 constexpr int kCBlock = 128;    // contiguous kernel: one 16-byte vector per lane, 128 lanes per block
@@ -194,13 +228,11 @@ constexpr int kEU = 4;          // element-per-lane kernels: elements in flight 
 // fastest of the block-size / unroll / grid-stride variants tried, ~6.7 TB/s in place and ~6.8 TB/s for fill.
 template <class T, class F>
 __global__ __launch_bounds__(256) void ew_contig_kernel(Vec16<T>* __restrict__ p, size_t nvec, F f) {
-    constexpr int N = 16 / sizeof(T);
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= nvec) return;
     Vec16<T> v;
     if constexpr (F::kReads) v = rt_ld16_nt(p + i);
-#pragma unroll
-    for (int j = 0; j < N; ++j) v.e[j] = f(v.e[j]);
+    apply_vec(v, f);
     if constexpr (F::kReads) rt_st16_nt(p + i, v);
     else p[i] = v;
 }
@@ -310,23 +342,27 @@ __global__ __launch_bounds__(kCBlock) void ew_rows_kernel(T* __restrict__ p, Row
         // two rows per trip, both loads issued before the first store
         for (uint32_t g = g_begin + ty; g < g_end; g += 2 * gy) {
             const bool two = g + gy < g_end;
-            Vec16<T>* v0 = reinterpret_cast<Vec16<T>*>(p + off + (int64_t)g * a.gstride + c);
-            Vec16<T>* v1 = reinterpret_cast<Vec16<T>*>(p + off + (int64_t)(two ? g + gy : g) * a.gstride + c);
-            Vec16<T> w0 = {}, w1 = {};
+            // vectors stay four 32-bit words across the conditional loads (arrays of 1-byte elements would be split up and re-packed)
+            rt_u32x4* v0 = reinterpret_cast<rt_u32x4*>(p + off + (int64_t)g * a.gstride + c);
+            rt_u32x4* v1 = reinterpret_cast<rt_u32x4*>(p + off + (int64_t)(two ? g + gy : g) * a.gstride + c);
+            rt_u32x4 w0 = {}, w1 = {};
             if constexpr (F::kReads) {
                 if constexpr (NT) {
-                    w0 = rt_ld16_nt(v0);
-                    if (two) w1 = rt_ld16_nt(v1);
+                    w0 = __builtin_nontemporal_load(v0);
+                    if (two) w1 = __builtin_nontemporal_load(v1);
                 } else {
                     w0 = *v0;
                     if (two) w1 = *v1;
                 }
             }
-#pragma unroll
-            for (int j = 0; j < N; ++j) { w0.e[j] = f(w0.e[j]); w1.e[j] = f(w1.e[j]); }
+            Vec16<T> e0 = __builtin_bit_cast(Vec16<T>, w0), e1 = __builtin_bit_cast(Vec16<T>, w1);
+            apply_vec(e0, f);
+            apply_vec(e1, f);
+            w0 = __builtin_bit_cast(rt_u32x4, e0);
+            w1 = __builtin_bit_cast(rt_u32x4, e1);
             if constexpr (F::kReads && NT) {
-                rt_st16_nt(v0, w0);
-                if (two) rt_st16_nt(v1, w1);
+                __builtin_nontemporal_store(w0, v0);
+                if (two) __builtin_nontemporal_store(w1, v1);
             } else {
                 *v0 = w0;
                 if (two) *v1 = w1;
@@ -393,12 +429,10 @@ int32_t launch_contig(rt_ctx* ctx, T* p, size_t n, F f) {
 // traffic (2 * N * sizeof(T) instead of 4 * N * sizeof(T)).
 template <class T, class F>
 __global__ __launch_bounds__(kCBlock) void ew_contig_out_kernel(const Vec16<T>* __restrict__ s, Vec16<T>* __restrict__ d, size_t nvec, F f) {
-    constexpr int N = 16 / sizeof(T);
     const size_t i = (size_t)blockIdx.x * kCBlock + threadIdx.x;
     if (i >= nvec) return;
     Vec16<T> v = rt_ld16_nt(s + i);
-#pragma unroll
-    for (int j = 0; j < N; ++j) v.e[j] = f(v.e[j]);
+    apply_vec(v, f);
     rt_st16_nt(d + i, v);
 }
 template <class T, class F>

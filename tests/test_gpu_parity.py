@@ -199,6 +199,74 @@ def test_unary_contiguous_float(hip, dtype):
                 assert got[:start].tobytes() == xi[:start].tobytes() and got[n - 2:].tobytes() == xi[n - 2:].tobytes()
 
 
+@pytest.mark.parametrize("dtype", ["u8", "i8", "bool"])
+def test_one_byte_types_every_pair(hip, dtype):
+    """The vector kernels handle 1-byte elements four to a 32-bit word.  Every (a, b) byte pair, so every carry / borrow / sign
+    combination inside a word: binary ops (contiguous, row-broadcast and in-place-row kernels), scalar ops and relu / neg / abs,
+    against two's-complement arithmetic in numpy and against the oracle."""
+    from rtensors_amd import hip as H
+    code = cpu.DTYPE_BY_NAME[dtype]
+    npd = cpu.NP_DTYPE[code]
+    if dtype == "bool":
+        a = np.repeat(np.arange(2, dtype=np.uint8), 2).astype(np.bool_); a = np.tile(a, 4096)
+        b = np.tile(np.arange(2, dtype=np.uint8), 2).astype(np.bool_); b = np.tile(b, 4096)
+        closed = {"add": a | b, "sub": a ^ b, "mul": a & b}
+    else:
+        a = np.repeat(np.arange(256, dtype=np.uint8), 256).view(npd)
+        b = np.tile(np.arange(256, dtype=np.uint8), 256).view(npd)
+        w = {"add": a.astype(np.int32) + b, "sub": a.astype(np.int32) - b, "mul": a.astype(np.int32) * b}
+        closed = {k: v.astype(np.uint8 if dtype == "u8" else np.int8) for k, v in w.items()}      # astype wraps modulo 256
+    n = a.size
+    ga, gb = hip.alloc_from_slice(code, a), hip.alloc_from_slice(code, b)
+    flat = (0, [n], [1])
+    for op in ("add", "sub", "mul"):
+        want = np.zeros(n, dtype=npd)
+        cpu.broadcast(code, op, a.copy(), MetaTensor([n], [1], 0), b.copy(), MetaTensor([n], [1], 0), want, MetaTensor([n], [1], 0))
+        assert want.tobytes() == closed[op].tobytes(), op                  # the oracle agrees with the closed form
+        gd = hip.alloc(code, n)
+        hip.broadcast((ga, flat), (gb, flat), (gd, flat), op)
+        assert hip.dump(gd).tobytes() == want.tobytes(), op
+        # rows kernel: right operand is one row of 256 repeated (b is exactly that)
+        rows = (0, [n // 256, 256], [256, 1])
+        gd2 = hip.alloc(code, n)
+        hip.broadcast((ga, rows), (gb, (0, [n // 256, 256], [0, 1])), (gd2, rows), op)
+        assert hip.dump(gd2).tobytes() == want.tobytes(), op
+    if dtype != "bool":
+        x = np.tile(np.arange(256, dtype=np.uint8), 64).view(npd)
+        for v in (0, 1, 3, 127, 128, 200, 255):
+            sv = int(np.array([v], dtype=np.uint8).view(npd)[0])
+            for op in ("add", "sub"):
+                g = hip.alloc_from_slice(code, x)
+                hip.scalar_contiguous(op, g, sv, 0, x.size)
+                wide = x.astype(np.int32) + sv if op == "add" else x.astype(np.int32) - sv
+                assert hip.dump(g).tobytes() == wide.astype(npd).tobytes(), (op, v)
+                # a view of whole rows inside a wider buffer takes the in-place row kernel
+                g = hip.alloc_from_slice(code, x)
+                hip.scalar_nd(op, g, sv, 16, [x.size // 64, 32], [64, 1])
+                want = x.copy()
+                cpu.scalar(code, op, want, sv, MetaTensor([x.size // 64, 32], [64, 1], 16))
+                assert hip.dump(g).tobytes() == want.tobytes(), (op, v)
+        for op in ("relu", "neg", "abs"):
+            want = x.copy()
+            try:
+                cpu.unary(code, op, want, MetaTensor([x.size], [1], 0))
+            except OErr:
+                continue
+            g = hip.alloc_from_slice(code, x)
+            hip.unary_contiguous(op, g, 0, x.size)
+            assert hip.dump(g).tobytes() == want.tobytes(), op
+            xi = x.astype(np.int32)
+            fixed = {"relu": np.maximum(xi, 0), "neg": -xi, "abs": np.abs(xi)}[op].astype(npd)
+            assert want.tobytes() == fixed.tobytes(), op
+    else:
+        x = np.tile(np.array([0, 1, 1, 0, 1], dtype=np.bool_), 4000)
+        for v in (False, True):
+            for op, f in (("add", np.logical_or), ("sub", np.logical_xor), ("mul", np.logical_and)):
+                g = hip.alloc_from_slice(code, x)
+                hip.scalar_contiguous(op, g, v, 0, x.size)
+                assert hip.dump(g).tobytes() == f(x, v).tobytes(), (op, v)
+
+
 @pytest.mark.parametrize("dtype", [d for d in ALL_DTYPES if d not in ("f32", "f64")])
 def test_unary_contiguous_int(hip, dtype):
     from rtensors_amd import hip as H
