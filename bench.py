@@ -114,6 +114,49 @@ class Workloads:
     def c4_i32_max1(self): return self._c4_axis("i32", "max", 1)
     def c4_i32_min0(self): return self._c4_axis("i32", "min", 0)
 
+    # statistics and index reductions on the config-4 tensor (the Cuda backend's other reduction kinds)
+    def _c4_stat(self, op, dim):
+        H = self.H
+        t = self._c4("f32")
+        arg = op in ("argmax", "argmin")
+        if dim is None:
+            out = self._out("c4sall" + ("u64" if arg else ""), H.U64 if arg else t.dtype, 1)
+            f = self.hip.apply_argmax_contiguous_flat if arg else self.hip.apply_reduce_contiguous_flat
+            return (lambda: f(t, out, 0, t.len, op)), t.len * 4 + (8 if arg else 4), t.len
+        shape = [8192, 32768]
+        nout = shape[1 - dim]
+        out = self._out(f"c4s{dim}" + ("u64" if arg else ""), H.U64 if arg else t.dtype, nout)
+        src = (t, (0, shape, [32768, 1]))
+        f = self.hip.apply_argmax_contiguous_nd if arg else self.hip.apply_reduce_contiguous_nd
+        return (lambda: f(src, out, dim, op)), t.len * 4 + nout * (8 if arg else 4), t.len
+
+    def c4_var1(self): return self._c4_stat("var", 1)
+    def c4_std0(self): return self._c4_stat("std", 0)
+    def c4_var_all(self): return self._c4_stat("var", None)
+    def c4_lse1(self): return self._c4_stat("logsumexp", 1)
+    def c4_lse0(self): return self._c4_stat("logsumexp", 0)
+    def c4_l2norm1(self): return self._c4_stat("l2_norm", 1)
+    def c4_l1norm0(self): return self._c4_stat("l1_norm", 0)
+    def c4_argmax1(self): return self._c4_stat("argmax", 1)
+    def c4_argmin0(self): return self._c4_stat("argmin", 0)
+    def c4_argmax_all(self): return self._c4_stat("argmax", None)
+
+    def _stat_shape(self, op, outer, R, inner):
+        H = self.H
+        a = self._gen("c2a", H.F32, 1 << 28, "normal", 1, 0)
+        arg = op in ("argmax", "argmin")
+        d = self._out("statout" + ("u64" if arg else ""), H.U64 if arg else H.F32, 1 << 26 if not arg else 1 << 25)
+        shape, strides = [outer, R, inner], [R * inner, inner, 1]
+        f = self.hip.apply_argmax_contiguous_nd if arg else self.hip.apply_reduce_contiguous_nd
+        return (lambda: f((a, (0, shape, strides)), d, 1, op)), outer * R * inner * 4 + outer * inner * (8 if arg else 4), outer * R * inner
+
+    def lse_rows10(self): return self._stat_shape("logsumexp", (1 << 28) // 10, 10, 1)       # class scores: rows of 10
+    def argmax_rows10(self): return self._stat_shape("argmax", (1 << 28) // 10, 10, 1)
+    def lse_rows1000(self): return self._stat_shape("logsumexp", (1 << 28) // 1000, 1000, 1)
+    def var_rows256(self): return self._stat_shape("var", 1 << 20, 256, 1)
+    def var_inner3(self): return self._stat_shape("var", 1, (1 << 28) // 3, 3)                # per-channel statistics of pixels
+    def var_mid64(self): return self._stat_shape("var", 65536, 64, 64)
+
     def c4_sum_all(self):
         t = self._c4("f32")
         out = self._out("c4oall", t.dtype, 1)

@@ -72,8 +72,20 @@ typedef enum rt_unary_op {
     RT_U_EXT_COUNT = 33
 } rt_unary_op;
 
-/* ops/reduction/mod.rs:161-175 (codes 6-10 -- variance, logsumexp, norm, argmax, argmin -- are outside this path) */
-typedef enum rt_reduce_op { RT_R_SUM = 1, RT_R_PROD = 2, RT_R_MAX = 3, RT_R_MIN = 4, RT_R_MEAN = 5 } rt_reduce_op;
+/* ReductionOpTypes::get_code, ops/reduction/mod.rs:161-175.  The low byte is the reference's code; the variants that carry a
+ * payload (Variance { unbiased }, Stdev { unbiased }, Norm(L1 | L2)) put it into the flag bits, the same three facts that
+ * populate_reduction_settings (backend/cuda.rs:1750-1774) hands to the reference's kernels as `ReductionSettings`. */
+#define RT_R_FLAG_UNBIASED 0x100 /* divide by n - 1 (var_at, std_at(.., true)); without it by n (pop_var_at) */
+#define RT_R_FLAG_STD 0x200      /* square root of the variance */
+#define RT_R_FLAG_L1 0x100       /* norm: sum |x| */
+#define RT_R_FLAG_L2 0x200       /* norm: sqrt(sum x^2) */
+typedef enum rt_reduce_op {
+    RT_R_SUM = 1, RT_R_PROD = 2, RT_R_MAX = 3, RT_R_MIN = 4, RT_R_MEAN = 5,
+    RT_R_VARIANCE = 6,           /* | RT_R_FLAG_UNBIASED | RT_R_FLAG_STD */
+    RT_R_LOGSUMEXP = 7,
+    RT_R_NORM = 8,               /* | RT_R_FLAG_L1 or RT_R_FLAG_L2 (one of them is required) */
+    RT_R_ARGMAX = 9, RT_R_ARGMIN = 10 /* rt_argmax_flat / rt_argmax_nd only */
+} rt_reduce_op;
 
 #define RT_MAX_RANK 8        /* dims a kernel descriptor holds after size-1 removal and merging of adjacent dims */
 #define RT_MAX_INPUT_RANK 128 /* the reference's own cap on rank (core/primitives.rs:377-383) */
@@ -156,6 +168,29 @@ int32_t rt_reduce_flat(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, 
 int32_t rt_reduce_nd(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, uint64_t src_len,
                      uint64_t offset, int32_t rank, const uint64_t* shape, const int64_t* strides,
                      void* dst, uint64_t dst_len, int32_t dim);
+/* The same two entry points also take the statistics the reference's Cuda backend offers and its Cpu backend panics on
+ * (ops/reduction/mod.rs:185; kernels K/kernels/reduction/reduce.cu:167-213 variance, 641-735 logsumexp, 66-97 norms), f32/f64 only:
+ *   RT_R_VARIANCE [| RT_R_FLAG_UNBIASED] [| RT_R_FLAG_STD]   m2 / (n - 1 | n), m2 = sum (x - mean)^2 merged pairwise
+ *                                                           (Chan's update, never sum x^2 - n mean^2); n = 1 unbiased gives NaN
+ *   RT_R_LOGSUMEXP                                           max + log(sum exp(x - max)); -inf for an empty or all -inf run, +inf
+ *                                                           when +inf occurs (the reference's flat launcher has no case for it
+ *                                                           and leaves dst unwritten, reduce.cu:795-832; here flat works too)
+ *   RT_R_NORM | RT_R_FLAG_L1 / RT_R_FLAG_L2                  sum |x| / sqrt(sum x^2)
+ * Results are within 1e-5 (f32) / 1e-12 (f64), relative, of the same quantity accumulated in higher precision.
+ * RT_R_ARGMAX / RT_R_ARGMIN are refused here with RT_E_INVALID (kinds cannot be swapped between entry points,
+ * backend/remote/remote_tests.rs:857-859). */
+
+/* Backend::apply_argmax_contiguous_flat / apply_argmax_contiguous_nd (backend/mod.rs:412-463; the Cpu backend has todo!() there,
+ * backend/cpu.rs:451-471; Cuda: reduce.cu:843-990).  dst holds u64 indices: for the flat form the position inside the run
+ * (0 = element `start`), for the nd form the coordinate along `dim` of each of the outer * inner outputs.  The smallest index of
+ * the extremum wins; NaN never wins; 0 for an empty run and when no element beats the starting value (T::MIN / T::MAX, as in
+ * the reference's kernel).  op is RT_R_ARGMAX or RT_R_ARGMIN, anything else is RT_E_INVALID.  f32/f64 as in the reference, plus
+ * the 8..64-bit integers.  Same validation as rt_reduce_flat / rt_reduce_nd. */
+int32_t rt_argmax_flat(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, uint64_t src_len,
+                       uint64_t* dst, uint64_t dst_len, uint64_t start, uint64_t len);
+int32_t rt_argmax_nd(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, uint64_t src_len,
+                     uint64_t offset, int32_t rank, const uint64_t* shape, const int64_t* strides,
+                     uint64_t* dst, uint64_t dst_len, int32_t dim);
 
 /* ---- out-of-place unary / scalar ops ---------------------------------------------------------------------------------
  * dst[0 .. len) = op(src[start .. start + len)); the source is only read.  The trait has in-place ops only: `tensor.relu()`,

@@ -38,7 +38,12 @@ UNARY = {n: i for i, n in enumerate(
     "asinh acosh atanh rsqrt reciprocal square cube exp sign".split())}
 SCALAR = {n: i for i, n in enumerate("add sub mul div log log1p leaky_relu elu leaky_grad".split())}
 BINARY = {"add": 0, "sub": 1, "mul": 2, "div": 3}
-REDUCE = {"sum": 1, "prod": 2, "max": 3, "min": 4, "mean": 5}
+REDUCE = {"sum": 1, "prod": 2, "max": 3, "min": 4, "mean": 5,
+          # the Cuda backend's other kinds (ops/reduction/mod.rs:161-175; payload of Variance / Stdev / Norm in the flag bits)
+          "pop_var": 6, "var": 6 | 0x100, "pop_std": 6 | 0x200, "std": 6 | 0x300, "logsumexp": 7, "l1_norm": 8 | 0x100, "l2_norm": 8 | 0x200,
+          "argmax": 9, "argmin": 10}
+STAT_OPS = ("pop_var", "var", "pop_std", "std", "logsumexp", "l1_norm", "l2_norm")
+ARG_OPS = ("argmax", "argmin")
 
 _ERR = {1: "UnsupportedOperation", 2: "IdxOutOfBounds(panic)", 3: "ArithmeticPanic", 4: "WrongDims", 5: "UnsupportedOp"}
 
@@ -71,6 +76,8 @@ def lib():
         L.orc_reduce_flat.argtypes = [C.c_int, C.c_int, vp, sz, vp, sz, sz, sz]
         L.orc_reduce_nd.argtypes = [C.c_int, C.c_int, vp, sz, sz, C.c_int, szp, i64p, vp, sz, C.c_int, C.c_int]
         L.orc_gather.argtypes = [C.c_int, vp, sz, sz, C.c_int, szp, i64p, vp, sz]
+        L.orc_reduce_stat.argtypes = [C.c_int, C.c_int, vp, sz, sz, sz, sz, sz, vp, sz]
+        L.orc_argmax.argtypes = [C.c_int, C.c_int, vp, sz, sz, sz, sz, sz, vp, sz]
         L.orc_equal.argtypes = [C.c_int, vp, vp, sz]
         L.orc_matmul.argtypes = [C.c_int, vp, sz, sz, i64, i64, i64, vp, sz, sz, i64, i64, i64, vp, sz, sz, sz, sz, sz]
         _lib = L
@@ -182,6 +189,34 @@ def reduce_nd(dtype: int, op: str, src: np.ndarray, meta: MetaTensor, dim: int, 
                              _stride_arr(meta.strides), _ptr(dst), dst.size, dim, 1 if honour_offset else 0)
     _check(rc, f"reduce_nd {op}")
     return dst
+
+
+def _outer_r_inner(meta: MetaTensor, dim: Optional[int]):
+    """(outer, R, inner) of a contiguous view reduced over `dim` (None: everything, the flat form)."""
+    if dim is None:
+        return 1, meta.size(), 1
+    if not meta.is_contiguous():
+        raise TensorError("WrongDims", "Reduction over non-contiguous tensors is not implemented yet.")
+    return meta.outer_dimensions(dim), meta.shape[dim], meta.inner_dimensions(dim)
+
+
+def reduce_stat(dtype: int, op: str, src: np.ndarray, meta: MetaTensor, dim: Optional[int]) -> np.ndarray:
+    """Variance / stdev / logsumexp / norms over `dim` (None: the whole contiguous view): the per-element rules of the reference's Cuda
+    kernels applied in index order (oracle/cpu_oracle.cpp)."""
+    outer, r, inner = _outer_r_inner(meta, dim)
+    dst = np.zeros(max(outer * inner, 1), dtype=NP_DTYPE[dtype])
+    rc = lib().orc_reduce_stat(dtype, REDUCE[op], _ptr(src), src.size, meta.offset, outer, r, inner, _ptr(dst), dst.size)
+    _check(rc, f"reduce {op}")
+    return dst[:outer * inner]
+
+
+def argmax(dtype: int, op: str, src: np.ndarray, meta: MetaTensor, dim: Optional[int]) -> np.ndarray:
+    """`apply_argmax_contiguous_flat` / `_nd`: u64 index of the first extremum along `dim` (None: inside the whole view)."""
+    outer, r, inner = _outer_r_inner(meta, dim)
+    dst = np.zeros(max(outer * inner, 1), dtype=np.uint64)
+    rc = lib().orc_argmax(dtype, REDUCE[op], _ptr(src), src.size, meta.offset, outer, r, inner, _ptr(dst), dst.size)
+    _check(rc, op)
+    return dst[:outer * inner]
 
 
 def gather(dtype: int, src: np.ndarray, meta: MetaTensor) -> np.ndarray:

@@ -13,6 +13,8 @@
 //                                                 as_strided evaluation
 //   reduce flat / nd (sum,prod,max,min,mean)    : reference known-answer vectors (incl. the order-sensitive
 //                                                 f64 sum 1.0999999999999999) + numpy sequential accumulate
+//   variance / stdev / logsumexp / norms / arg  : the Cuda backend's known-answer vectors (backend/cuda.rs:2321-2590) + numpy
+//                                                 float64 var / logaddexp.reduce / norm / argmax (ties, NaN cases by hand)
 //   integer reductions                          : not in the reference (WeightValue is f32/f64 only); pinned by
 //                                                 the closed form "sum mod 2^w", min/max by numpy
 //   transcendental unaries (exp, ln, sin ...)   : PARITY UNPINNED bit-for-bit (Rust std -> platform libm);
@@ -494,6 +496,97 @@ int reduce_nd_impl(int op, const T* src, size_t srclen, const Meta& sm, T* dst, 
     return ORC_OK;
 }
 
+// ---- statistics and index reductions -------------------------------------------------------------------------------------
+// The reference's Cpu backend has no accumulator for these (ops/reduction/mod.rs:185 panics, backend/cpu.rs:451-471 is todo!());
+// its Cuda backend defines them in cuda/kernels/reduction/reduce.cu.  Restated here are that file's per-element rules, applied
+// in ascending index order by one thread (the Cuda kernels combine the same states in tree order):
+//   variance / stdev  welford_update 181-189, finalize 385-402: m2 / (n - 1 | n), optional sqrt
+//   logsumexp         lse_from_value / lse_combine 654-673, result m + log(s) 731-733; x == max counts as exp(0) = 1, so that
+//                     infinite inputs give +-inf instead of the NaN of exp(inf - inf)
+//   norms             L1SumOp 66-75 (sum |x|), L2SumOp 88-97 + PostSqrt 143-152 (sqrt(sum x^2))
+//   argmax / argmin   strict comparison starting from lowest() / max() with index 0, 893-905: the first extremum wins, NaN never
+// The source is viewed as (outer, R, inner) from `offset`, as apply_reduce_contiguous_nd does (backend/cpu.rs:413-449).
+enum : int { R_VARIANCE = 6, R_LOGSUMEXP = 7, R_NORM = 8, R_ARGMAX = 9, R_ARGMIN = 10, RF_UNBIASED = 0x100, RF_STD = 0x200, RF_L1 = 0x100, RF_L2 = 0x200 };
+
+template <class T>
+int reduce_stat_impl(int op, const T* src, size_t srclen, size_t offset, size_t outer, size_t r, size_t inner, T* dst, size_t dstlen) {
+    const int code = op & 0xff, flags = op & ~0xff;
+    if (code == R_VARIANCE) { if (flags & ~(RF_UNBIASED | RF_STD)) return ORC_E_OP; }
+    else if (code == R_LOGSUMEXP) { if (flags) return ORC_E_OP; }
+    else if (code == R_NORM) { if (flags != RF_L1 && flags != RF_L2) return ORC_E_OP; }
+    else return ORC_E_OP;
+    if (outer * inner > dstlen) return ORC_E_OOB;
+    if (outer * r * inner > 0 && (offset > srclen || outer * r * inner > srclen - offset)) return ORC_E_OOB;
+    for (size_t o = 0; o < outer; ++o) {
+        for (size_t i = 0; i < inner; ++i) {
+            const T* base = src + offset + o * r * inner + i;
+            T out;
+            if (code == R_VARIANCE) {
+                T mean = (T)0, m2 = (T)0;
+                long count = 0;
+                for (size_t k = 0; k < r; ++k) {
+                    const T x = base[k * inner];
+                    count += 1;
+                    const T delta = x - mean;
+                    mean += delta / (T)count;
+                    const T delta2 = x - mean;
+                    m2 += delta * delta2;
+                }
+                const T denom = (flags & RF_UNBIASED) ? (T)(count - 1) : (T)count;
+                out = m2 / denom;
+                if (flags & RF_STD) out = std::sqrt(out);
+            } else if (code == R_LOGSUMEXP) {
+                T m = -std::numeric_limits<T>::infinity(), sum = (T)0;
+                for (size_t k = 0; k < r; ++k) {
+                    const T x = base[k * inner];
+                    const T top = (x > m) ? x : m;                                   // NaN never becomes the maximum
+                    const T keep = (m == top) ? (T)1 : std::exp(m - top);
+                    const T add = (x == top) ? (T)1 : std::exp(x - top);
+                    sum = sum * keep + add;
+                    m = top;
+                }
+                out = (sum == (T)0) ? m : m + std::log(sum);
+            } else {
+                T sum = (T)0;
+                for (size_t k = 0; k < r; ++k) {
+                    const T x = base[k * inner];
+                    sum += (flags == RF_L1) ? std::fabs(x) : x * x;
+                }
+                out = (flags == RF_L1) ? sum : std::sqrt(sum);
+            }
+            dst[o * inner + i] = out;
+        }
+    }
+    return ORC_OK;
+}
+
+template <class T, class E = void> struct arg_ok : std::false_type {};
+template <class T> struct arg_ok<T, typename std::enable_if<std::is_arithmetic<T>::value && sizeof(T) <= 8>::type> : std::true_type {};
+
+template <class T>
+typename std::enable_if<arg_ok<T>::value, int>::type
+argmax_impl(int op, const T* src, size_t srclen, size_t offset, size_t outer, size_t r, size_t inner, uint64_t* dst, size_t dstlen) {
+    if (op != R_ARGMAX && op != R_ARGMIN) return ORC_E_OP;
+    if (outer * inner > dstlen) return ORC_E_OOB;
+    if (outer * r * inner > 0 && (offset > srclen || outer * r * inner > srclen - offset)) return ORC_E_OOB;
+    for (size_t o = 0; o < outer; ++o) {
+        for (size_t i = 0; i < inner; ++i) {
+            const T* base = src + offset + o * r * inner + i;
+            T best = op == R_ARGMAX ? std::numeric_limits<T>::lowest() : std::numeric_limits<T>::max();
+            uint64_t at = 0;
+            for (size_t k = 0; k < r; ++k) {
+                const T x = base[k * inner];
+                if (op == R_ARGMAX ? x > best : x < best) { best = x; at = k; }
+            }
+            dst[o * inner + i] = at;
+        }
+    }
+    return ORC_OK;
+}
+template <class T>
+typename std::enable_if<!arg_ok<T>::value, int>::type
+argmax_impl(int, const T*, size_t, size_t, size_t, size_t, size_t, uint64_t*, size_t) { return ORC_E_DTYPE; }
+
 // ---- view_to_contiguous: core/tensor.rs:299-325 with core/meta.rs:263-307, 506-521 ------------------------------
 // Copies forward-contiguous runs (negative strides never form a run) into a fresh row-major buffer.
 template <class T>
@@ -627,6 +720,16 @@ int orc_reduce_nd(int dtype, int op, const void* src, size_t srclen, size_t offs
                   const int64_t* strides, void* dst, size_t dstlen, int dim, int honour_offset) {
     Meta m{offset, rank, shape, strides};
     ORC_DISPATCH(dtype, return reduce_nd_impl<T>(op, (const T*)src, srclen, m, (T*)dst, dstlen, dim, honour_offset));
+}
+
+int orc_reduce_stat(int dtype, int op, const void* src, size_t srclen, size_t offset, size_t outer, size_t r, size_t inner, void* dst, size_t dstlen) {
+    if (dtype == F32) return reduce_stat_impl<float>(op, (const float*)src, srclen, offset, outer, r, inner, (float*)dst, dstlen);
+    if (dtype == F64) return reduce_stat_impl<double>(op, (const double*)src, srclen, offset, outer, r, inner, (double*)dst, dstlen);
+    return ORC_E_DTYPE;                                                  // T: WeightValue
+}
+
+int orc_argmax(int dtype, int op, const void* src, size_t srclen, size_t offset, size_t outer, size_t r, size_t inner, uint64_t* dst, size_t dstlen) {
+    ORC_DISPATCH(dtype, return argmax_impl<T>(op, (const T*)src, srclen, offset, outer, r, inner, dst, dstlen));
 }
 
 int orc_gather(int dtype, const void* src, size_t srclen, size_t offset, int rank, const size_t* shape,

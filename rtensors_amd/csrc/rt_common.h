@@ -65,6 +65,14 @@ int32_t rt_alloc_bytes(rt_ctx* ctx, size_t bytes, void** out);       // caller h
 int32_t rt_free_locked(rt_ctx* ctx, void* p);
 int32_t rt_scratch(rt_ctx* ctx, size_t bytes, void** out);           // caller holds ctx->mu
 
+// Validation shared by the reduce and argmax entry points.  *run == false after RT_OK: there are no outputs, launch nothing.
+int32_t rt_check_reduce_flat(uint64_t src_len, const void* src, const void* dst, uint64_t dst_len, uint64_t start, uint64_t len);
+int32_t rt_check_reduce_nd(uint64_t src_len, const void* src, uint64_t offset, int32_t rank, const uint64_t* shape, const int64_t* strides,
+                           const void* dst, uint64_t dst_len, int32_t dim, uint64_t* outer, uint64_t* inner, bool* run);
+// variance / stdev / logsumexp / norms (out: T*) and argmax / argmin (out: uint64_t*) of src viewed as (outer, R, inner); caller
+// holds ctx->mu
+int32_t rt_reduce_stat(rt_ctx* ctx, int dtype, int op, const void* src, void* out, uint64_t outer, uint64_t R, uint64_t inner);
+
 static inline int rt_elem_size(int dtype) {
     switch (dtype) {
         case RT_U8: case RT_I8: case RT_BOOL: return 1;

@@ -679,7 +679,7 @@ int32_t reduce_ops(rt_ctx* ctx, int op, const void* src, void* out, uint64_t out
         case RT_R_MIN: return reduce_typed<RT_R_MIN, T>(ctx, (const T*)src, (T*)out, outer, R, inner);
         case RT_R_MEAN: return reduce_typed<RT_R_MEAN, T>(ctx, (const T*)src, (T*)out, outer, R, inner);
     }
-    return rt_fail(RT_E_INVALID, "reduce: op code %d has no accumulator (the reference panics, ops/reduction/mod.rs:185)", op);
+    return rt_fail(RT_E_INVALID, "reduce: op 0x%x is not a reduction op code with valid flags", op);
 }
 
 int32_t reduce_any(rt_ctx* ctx, int dtype, int op, const void* src, void* out, uint64_t outer, uint64_t R, uint64_t inner) {
@@ -700,27 +700,20 @@ int32_t reduce_any(rt_ctx* ctx, int dtype, int op, const void* src, void* out, u
 
 }  // namespace
 
-extern "C" int32_t rt_reduce_flat(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, uint64_t src_len, void* dst, uint64_t dst_len,
-                                  uint64_t start, uint64_t len) {
-    RT_TRY(rt_ctx_enter(ctx));
-    int es = rt_elem_size(dtype);
-    if (!es) return rt_fail(RT_E_DTYPE, "reduce: unknown dtype code %d", dtype);
-    // check_reduce_flat, backend/remote/server.rs:375-380
+// check_reduce_flat, backend/remote/server.rs:375-380
+int32_t rt_check_reduce_flat(uint64_t src_len, const void* src, const void* dst, uint64_t dst_len, uint64_t start, uint64_t len) {
     if (start > src_len || len > src_len - start)
         return rt_fail(RT_E_OUT_OF_BOUNDS, "reduction source: elements %llu..%llu of a buffer with %llu elements",
                        (unsigned long long)start, (unsigned long long)(start + len), (unsigned long long)src_len);
     if (dst_len == 0) return rt_fail(RT_E_OUT_OF_BOUNDS, "reduction output buffer is empty");
     if (!dst || (!src && len)) return rt_fail(RT_E_INVALID, "reduce: null buffer");
-    CtxGuard g(ctx);
-    return reduce_any(ctx, dtype, op, (const char*)src + start * es, dst, 1, len, 1);
+    return RT_OK;
 }
 
-extern "C" int32_t rt_reduce_nd(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, uint64_t src_len, uint64_t offset, int32_t rank,
-                                const uint64_t* shape, const int64_t* strides, void* dst, uint64_t dst_len, int32_t dim) {
-    RT_TRY(rt_ctx_enter(ctx));
-    int es = rt_elem_size(dtype);
-    if (!es) return rt_fail(RT_E_DTYPE, "reduce: unknown dtype code %d", dtype);
-    // check_reduce_nd, backend/remote/server.rs:327-373
+// check_reduce_nd, backend/remote/server.rs:327-373
+int32_t rt_check_reduce_nd(uint64_t src_len, const void* src, uint64_t offset, int32_t rank, const uint64_t* shape, const int64_t* strides,
+                           const void* dst, uint64_t dst_len, int32_t dim, uint64_t* outer_out, uint64_t* inner_out, bool* run) {
+    *run = false;
     if (rank < 1 || rank > RT_MAX_INPUT_RANK || !shape || !strides) return rt_fail(RT_E_INVALID, "reduce: bad rank %d or null shape", rank);
     if (dim < 0 || dim >= rank) return rt_fail(RT_E_INVALID, "reduction dim %d out of range for rank %d", dim, rank);
     unsigned __int128 size = 1, outer = 1, inner = 1;
@@ -750,6 +743,39 @@ extern "C" int32_t rt_reduce_nd(rt_ctx* ctx, int32_t dtype, int32_t op, const vo
         return rt_fail(RT_E_OUT_OF_BOUNDS, "reduction output needs %llu elements, buffer has %llu", (unsigned long long)(outer * inner),
                        (unsigned long long)dst_len);
     if (!dst || !src) return rt_fail(RT_E_INVALID, "reduce: null buffer");
+    *outer_out = (uint64_t)outer;
+    *inner_out = (uint64_t)inner;
+    *run = true;
+    return RT_OK;
+}
+
+static int32_t reduce_dispatch(rt_ctx* ctx, int dtype, int op, const void* src, void* out, uint64_t outer, uint64_t R, uint64_t inner) {
+    const int code = op & 0xff;
+    if (code == RT_R_ARGMAX || code == RT_R_ARGMIN)
+        return rt_fail(RT_E_INVALID, "reduce: argmax / argmin produce indices, use rt_argmax_flat / rt_argmax_nd");
+    if (code == RT_R_VARIANCE || code == RT_R_LOGSUMEXP || code == RT_R_NORM) return rt_reduce_stat(ctx, dtype, op, src, out, outer, R, inner);
+    return reduce_any(ctx, dtype, op, src, out, outer, R, inner);
+}
+
+extern "C" int32_t rt_reduce_flat(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, uint64_t src_len, void* dst, uint64_t dst_len,
+                                  uint64_t start, uint64_t len) {
+    RT_TRY(rt_ctx_enter(ctx));
+    int es = rt_elem_size(dtype);
+    if (!es) return rt_fail(RT_E_DTYPE, "reduce: unknown dtype code %d", dtype);
+    RT_TRY(rt_check_reduce_flat(src_len, src, dst, dst_len, start, len));
     CtxGuard g(ctx);
-    return reduce_any(ctx, dtype, op, (const char*)src + offset * es, dst, (uint64_t)outer, shape[dim], (uint64_t)inner);
+    return reduce_dispatch(ctx, dtype, op, (const char*)src + start * es, dst, 1, len, 1);
+}
+
+extern "C" int32_t rt_reduce_nd(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, uint64_t src_len, uint64_t offset, int32_t rank,
+                                const uint64_t* shape, const int64_t* strides, void* dst, uint64_t dst_len, int32_t dim) {
+    RT_TRY(rt_ctx_enter(ctx));
+    int es = rt_elem_size(dtype);
+    if (!es) return rt_fail(RT_E_DTYPE, "reduce: unknown dtype code %d", dtype);
+    uint64_t outer = 0, inner = 0;
+    bool run = false;
+    RT_TRY(rt_check_reduce_nd(src_len, src, offset, rank, shape, strides, dst, dst_len, dim, &outer, &inner, &run));
+    if (!run) return RT_OK;
+    CtxGuard g(ctx);
+    return reduce_dispatch(ctx, dtype, op, (const char*)src + offset * es, dst, outer, shape[dim], inner);
 }

@@ -1,0 +1,694 @@
+// Reductions whose running state is more than one value of T: variance / standard deviation, logsumexp, L1 / L2 norm, argmax /
+// argmin, full (flat) and along one axis of a row-major contiguous tensor viewed as (outer, R, inner).  The reference offers them
+// on its Cuda backend only (K/kernels/reduction/reduce.cu: Welford states 167-213 and 324-460, logsumexp 641-735, norms 66-97 and
+// 291-321, argmax 843-990); its Cpu backend panics or has todo!() for them (ops/reduction/mod.rs:185, backend/cpu.rs:451-471).
+//
+// Every kernel is written once over a state type S with init / push / push_block / merge / result:
+//   MomentState   (mean, m2, n)   blocks of 8-16 elements are folded exactly (mean of the block, squared deviations from it) and
+//                                 merged into the running state with Chan's update -- the reference's welford_combine; one
+//                                 division per block instead of one per element
+//   LseState      (max, sum)      sum of exp(x - max), rescaled when the maximum moves; one exp per element plus one per block
+//   NormState     (sum)           sum |x| or sum x^2
+//   ArgState      (value, index)  strict comparison against T::MIN / T::MAX, smallest index among equals
+// Kernels (HBM-bound, algorithmic traffic N_in * sizeof(T) + N_out * sizeof(out)):
+//   rows  (inner == 1): block per row segment / wave per row / LDS-staged short rows, as in rt_reduce.hip
+//   cols  (inner  > 1): lanes along `inner` with 16-byte loads; a narrow `inner` is streamed as one contiguous run instead
+//   Partial states of split reductions go to the context's scratch buffer and a merge kernel folds them (two launches, no atomics).
+#include "rt_common.h"
+
+#include <limits>
+#include <type_traits>
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kWaves = kBlock / RT_WAVE;
+
+template <class T> struct is_flt : std::integral_constant<bool, std::is_same<T, float>::value || std::is_same<T, double>::value> {};
+template <class T> struct alignas(16) Vec16 { T e[16 / sizeof(T)]; };
+
+__device__ __forceinline__ float m_exp(float x) { return expf(x); }
+__device__ __forceinline__ double m_exp(double x) { return exp(x); }
+__device__ __forceinline__ float m_log(float x) { return logf(x); }
+__device__ __forceinline__ double m_log(double x) { return log(x); }
+__device__ __forceinline__ float m_sqrt(float x) { return sqrtf(x); }
+__device__ __forceinline__ double m_sqrt(double x) { return sqrt(x); }
+__device__ __forceinline__ float m_abs(float x) { return fabsf(x); }
+__device__ __forceinline__ double m_abs(double x) { return fabs(x); }
+__device__ __forceinline__ float m_max(float a, float b) { return fmaxf(a, b); }
+__device__ __forceinline__ double m_max(double a, double b) { return fmax(a, b); }
+
+// ---- states -----------------------------------------------------------------------------------------------------------
+// push(x, pos): one element at position `pos` of the reduced axis; push_block<K>(x, pos0, step): K elements at positions pos0,
+// pos0 + step, ...; merge(o): another partial state, any relative order; result(flags): the output value.
+
+template <class T> struct MomentState {
+    typedef T Out;
+    T mean, m2;
+    uint64_t n;
+    __device__ __forceinline__ void init() { mean = (T)0; m2 = (T)0; n = 0; }
+    __device__ __forceinline__ void absorb(T omean, T om2, uint64_t on) {          // welford_combine, reduce.cu:191-213
+        if (on == 0) return;
+        if (n == 0) { mean = omean; m2 = om2; n = on; return; }
+        const uint64_t nn = n + on;
+        const T delta = omean - mean;
+        const T w = (T)on / (T)nn;
+        mean = mean + delta * w;
+        m2 = m2 + om2 + (delta * delta) * ((T)n * w);
+        n = nn;
+    }
+    __device__ __forceinline__ void push(T x, uint64_t) { absorb(x, (T)0, 1); }
+    template <int K> __device__ __forceinline__ void push_block(const T* x, uint64_t, uint64_t) {
+        T s = (T)0;
+#pragma unroll
+        for (int i = 0; i < K; ++i) s = s + x[i];
+        const T bm = s * ((T)1 / (T)K);                                              // K is a power of two: exact scaling
+        T q = (T)0;
+#pragma unroll
+        for (int i = 0; i < K; ++i) { const T d = x[i] - bm; q = q + d * d; }
+        absorb(bm, q, K);
+    }
+    __device__ __forceinline__ void merge(const MomentState& o) { absorb(o.mean, o.m2, o.n); }
+    __device__ __forceinline__ T result(int flags) const {                          // finalize_var_kernel_ptr, reduce.cu:385-402
+        const T denom = (flags & RT_R_FLAG_UNBIASED) ? (T)n - (T)1 : (T)n;
+        const T v = m2 / denom;
+        return (flags & RT_R_FLAG_STD) ? m_sqrt(v) : v;
+    }
+};
+
+template <class T> struct LseState {
+    typedef T Out;
+    T m, s;
+    __device__ __forceinline__ void init() { m = -std::numeric_limits<T>::infinity(); s = (T)0; }
+    // exp(x - top), with x == top giving 1 also when both are infinite
+    static __device__ __forceinline__ T term(T x, T top) { return x == top ? (T)1 : m_exp(x - top); }
+    __device__ __forceinline__ void push(T x, uint64_t) {
+        const T top = m_max(m, x);
+        s = s * term(m, top) + term(x, top);
+        m = top;
+    }
+    template <int K> __device__ __forceinline__ void push_block(const T* x, uint64_t, uint64_t) {
+        T top = m;
+#pragma unroll
+        for (int i = 0; i < K; ++i) top = m_max(top, x[i]);
+        T acc = s * term(m, top);
+#pragma unroll
+        for (int i = 0; i < K; ++i) acc = acc + term(x[i], top);
+        s = acc;
+        m = top;
+    }
+    __device__ __forceinline__ void merge(const LseState& o) {                      // lse_combine, reduce.cu:660-673
+        const T top = m_max(m, o.m);
+        s = s * term(m, top) + o.s * term(o.m, top);
+        m = top;
+    }
+    __device__ __forceinline__ T result(int) const { return s == (T)0 ? m : m + m_log(s); }
+};
+
+template <class T, bool SQ> struct NormState {
+    typedef T Out;
+    T s;
+    __device__ __forceinline__ void init() { s = (T)0; }
+    __device__ __forceinline__ void push(T x, uint64_t) { s = s + (SQ ? x * x : m_abs(x)); }
+    template <int K> __device__ __forceinline__ void push_block(const T* x, uint64_t, uint64_t) {
+        T b = (T)0;
+#pragma unroll
+        for (int i = 0; i < K; ++i) b = b + (SQ ? x[i] * x[i] : m_abs(x[i]));
+        s = s + b;
+    }
+    __device__ __forceinline__ void merge(const NormState& o) { s = s + o.s; }
+    __device__ __forceinline__ T result(int) const { return SQ ? m_sqrt(s) : s; }
+};
+
+template <class T, bool MAX> struct ArgState {
+    typedef uint64_t Out;
+    T v;
+    uint64_t idx;
+    __device__ __forceinline__ void init() {
+        v = MAX ? std::numeric_limits<T>::lowest() : std::numeric_limits<T>::max();
+        idx = ~0ull;
+    }
+    static __device__ __forceinline__ bool beats(T a, T b) { return MAX ? a > b : a < b; }
+    __device__ __forceinline__ void push(T x, uint64_t pos) {
+        if (beats(x, v)) { v = x; idx = pos; }                                      // NaN never wins, the first of equals stays
+    }
+    template <int K> __device__ __forceinline__ void push_block(const T* x, uint64_t pos0, uint64_t step) {
+#pragma unroll
+        for (int i = 0; i < K; ++i) push(x[i], pos0 + (uint64_t)i * step);
+    }
+    __device__ __forceinline__ void merge(const ArgState& o) {
+        if (beats(o.v, v) || (o.v == v && o.idx < idx)) { v = o.v; idx = o.idx; }
+    }
+    __device__ __forceinline__ uint64_t result(int) const { return idx == ~0ull ? 0 : idx; }
+};
+
+// a state moved between lanes as 32-bit words
+template <class S> __device__ __forceinline__ S shfl_down_state(const S& s, int d) {
+    static_assert(sizeof(S) % 4 == 0, "state is a whole number of words");
+    constexpr int W = sizeof(S) / 4;
+    uint32_t w[W];
+    __builtin_memcpy(w, &s, sizeof(S));                                             // states may hold padding: no bit_cast
+#pragma unroll
+    for (int i = 0; i < W; ++i) w[i] = (uint32_t)__shfl_down((int)w[i], d, RT_WAVE);
+    S r;
+    __builtin_memcpy(&r, w, sizeof(S));
+    return r;
+}
+
+// lanes [0, width) of each aligned group of `width` lanes fold into the group's first lane (width: power of two <= 64)
+template <class S> __device__ __forceinline__ void group_reduce(S& a, uint32_t width, uint32_t lane_in_group) {
+    for (uint32_t d = width / 2; d >= 1; d >>= 1) {
+        S o = shfl_down_state(a, (int)d);
+        if (lane_in_group + d < width) a.merge(o);
+    }
+}
+
+template <class S> __device__ __forceinline__ void block_reduce(S& a) {
+    __shared__ S part[kWaves];
+    const uint32_t lane = threadIdx.x & (RT_WAVE - 1), w = threadIdx.x / RT_WAVE;
+    group_reduce(a, RT_WAVE, lane);
+    if (lane == 0) part[w] = a;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int k = 1; k < kWaves; ++k) a.merge(part[k]);
+    }
+}
+
+// fold elements [begin, end) of the contiguous run `p`; positions are relative to `p`
+template <class S, class T>
+__device__ __forceinline__ void fold_run(S& a, const T* __restrict__ p, uint64_t begin, uint64_t end, uint32_t tid, uint32_t nthreads) {
+    constexpr uint32_t N = 16 / sizeof(T);
+    constexpr int U = 4;
+    if (begin >= end) return;
+    uint64_t head = ((16 - (reinterpret_cast<uintptr_t>(p + begin) & 15)) & 15) / sizeof(T);
+    if (head > end - begin) head = end - begin;
+    if (tid < head) a.push(p[begin + tid], begin + tid);
+    const uint64_t vb = begin + head;
+    const uint64_t nvec = (end - vb) / N;
+    const Vec16<T>* pv = reinterpret_cast<const Vec16<T>*>(p + vb);
+    uint64_t i = tid;
+    for (; i + (uint64_t)(U - 1) * nthreads < nvec; i += (uint64_t)U * nthreads) {
+        Vec16<T> v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = rt_ld16_nt(pv + i + (uint64_t)u * nthreads);
+        if constexpr (std::is_same<typename S::Out, uint64_t>::value) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) a.template push_block<N>(v[u].e, vb + (i + (uint64_t)u * nthreads) * N, 1);
+        } else {
+            T x[U * N];                                                             // positions are irrelevant: one block of U * N
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+#pragma unroll
+                for (uint32_t j = 0; j < N; ++j) x[u * N + j] = v[u].e[j];
+            }
+            a.template push_block<U * N>(x, 0, 0);
+        }
+    }
+    for (; i < nvec; i += nthreads) {
+        Vec16<T> v = rt_ld16_nt(pv + i);
+        a.template push_block<N>(v.e, vb + i * N, 1);
+    }
+    const uint64_t tb = vb + nvec * N;
+    if (tb + tid < end) a.push(p[tb + tid], tb + tid);
+}
+
+// ---- rows -------------------------------------------------------------------------------------------------------------
+// grid.x = rows * splits; block b folds segment (b % splits) of row (b / splits) -> part[b] (state) or out[row] (result)
+template <class S, class T>
+__global__ __launch_bounds__(kBlock) void st_rows_block_kernel(const T* __restrict__ src, typename S::Out* __restrict__ out, S* __restrict__ part,
+                                                               uint64_t R, uint32_t splits, uint64_t seglen, int flags) {
+    const uint64_t row = blockIdx.x / splits;
+    const uint32_t seg = blockIdx.x - (uint32_t)(row * splits);
+    const uint64_t begin = (uint64_t)seg * seglen;
+    uint64_t end = begin + seglen;
+    if (end > R) end = R;
+    S a;
+    a.init();
+    fold_run<S, T>(a, src + row * R, begin, end, threadIdx.x, kBlock);
+    block_reduce(a);
+    if (threadIdx.x == 0) {
+        if (part) part[blockIdx.x] = a;
+        else out[row] = a.result(flags);
+    }
+}
+
+// one wave per row
+template <class S, class T>
+__global__ __launch_bounds__(kBlock) void st_rows_wave_kernel(const T* __restrict__ src, typename S::Out* __restrict__ out, uint64_t rows, uint64_t R, int flags) {
+    const uint64_t row = (uint64_t)blockIdx.x * kWaves + threadIdx.x / RT_WAVE;
+    if (row >= rows) return;
+    const uint32_t lane = threadIdx.x & (RT_WAVE - 1);
+    S a;
+    a.init();
+    fold_run<S, T>(a, src + row * R, 0, R, lane, RT_WAVE);
+    group_reduce(a, RT_WAVE, lane);
+    if (lane == 0) out[row] = a.result(flags);
+}
+
+// short rows (1 <= R <= 1024): the block's rows are one contiguous run, copied into LDS with coalesced 16-byte loads (row pitch R | 1
+// keeps lanes that walk different rows on different banks), then groups of G lanes fold one row each.
+constexpr uint32_t kTileBytes = 32768;
+constexpr uint64_t kTileMaxR = 1024;
+struct TileArgs {
+    uint64_t rows;
+    uint32_t R, pitch, rpb, G;
+    FastDiv32 r_div;
+};
+
+template <class S, class T>
+__global__ __launch_bounds__(kBlock) void st_rows_tile_kernel(const T* __restrict__ src, typename S::Out* __restrict__ out, TileArgs a, int flags) {
+    constexpr uint32_t N = 16 / sizeof(T);
+    __shared__ alignas(16) T tile[kTileBytes / sizeof(T)];
+    const uint64_t row0 = (uint64_t)blockIdx.x * a.rpb;
+    const uint32_t nrows = (uint32_t)(a.rows - row0 < a.rpb ? a.rows - row0 : a.rpb);
+    const uint32_t ne = nrows * a.R;
+    const T* p = src + row0 * a.R;
+    auto put = [&](uint32_t e, T v) {
+        const uint32_t r = fd_div(e, a.r_div);
+        tile[r * a.pitch + (e - r * a.R)] = v;
+    };
+    uint32_t head = (uint32_t)(((16 - (reinterpret_cast<uintptr_t>(p) & 15)) & 15) / sizeof(T));
+    if (head > ne) head = ne;
+    if (threadIdx.x < head) put(threadIdx.x, p[threadIdx.x]);
+    const uint32_t nvec = (ne - head) / N;
+    const Vec16<T>* pv = reinterpret_cast<const Vec16<T>*>(p + head);
+    constexpr int U = 4;
+    for (uint32_t v0 = threadIdx.x; v0 < nvec; v0 += U * kBlock) {
+        Vec16<T> x[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (v0 + u * kBlock < nvec) x[u] = rt_ld16_nt(pv + v0 + u * kBlock);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (v0 + u * kBlock < nvec) {
+#pragma unroll
+                for (uint32_t j = 0; j < N; ++j) put(head + (v0 + u * kBlock) * N + j, x[u].e[j]);
+            }
+        }
+    }
+    const uint32_t tb = head + nvec * N;
+    if (tb + threadIdx.x < ne) put(tb + threadIdx.x, p[tb + threadIdx.x]);
+    __syncthreads();
+    const uint32_t g = threadIdx.x / a.G, j = threadIdx.x & (a.G - 1), groups = kBlock / a.G;
+    for (uint32_t r0 = 0; r0 < nrows; r0 += groups) {              // every lane runs every trip: the shuffles below need the whole wave
+        const uint32_t r = r0 + g;
+        S acc;
+        acc.init();
+        if (r < nrows) {
+            const T* row = tile + r * a.pitch;
+            uint32_t k = j;
+            for (; k + 3 * a.G < a.R; k += 4 * a.G) {
+                T x[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) x[u] = row[k + u * a.G];
+                acc.template push_block<4>(x, k, a.G);
+            }
+            for (; k < a.R; k += a.G) acc.push(row[k], k);
+        }
+        group_reduce(acc, a.G, j);
+        if (j == 0 && r < nrows) out[row0 + r] = acc.result(flags);
+    }
+}
+
+// ---- cols -------------------------------------------------------------------------------------------------------------
+// src viewed as (outer, R, inner).  blockIdx.x -> (o, seg, tile); lane tx covers columns (tile * 64 + tx) * VW ..; wave ty takes
+// k = begin + ty, + kWaves, ...  Results go to out[o * inner + col], partial states to part[(seg * outer + o) * inner + col].
+template <class S, class T, int VW>
+__global__ __launch_bounds__(kBlock) void st_cols_kernel(const T* __restrict__ src, typename S::Out* __restrict__ out, S* __restrict__ part, uint64_t R,
+                                                         uint64_t inner, uint64_t outer, uint32_t tiles, uint32_t splits, uint64_t seglen, int flags) {
+    constexpr int U = 4;
+    struct alignas(sizeof(T) * VW) VecW { T e[VW]; };
+    auto load = [](const T* q) -> VecW {
+        if constexpr (sizeof(VecW) == 16) {
+            return rt_ld16_nt(reinterpret_cast<const VecW*>(q));
+        } else {
+            VecW w;
+            w.e[0] = __builtin_nontemporal_load(q);
+            return w;
+        }
+    };
+    uint64_t b = blockIdx.x;
+    const uint32_t tile = (uint32_t)(b % tiles);
+    b /= tiles;
+    const uint32_t seg = (uint32_t)(b % splits);
+    const uint64_t o = b / splits;
+    const uint32_t tx = threadIdx.x & (RT_WAVE - 1), ty = threadIdx.x / RT_WAVE;
+    const uint64_t col = ((uint64_t)tile * RT_WAVE + tx) * VW;
+    const bool active = col < inner;                           // inner is a multiple of VW
+    const uint64_t begin = (uint64_t)seg * seglen;
+    uint64_t end = begin + seglen;
+    if (end > R) end = R;
+
+    S a[VW];
+#pragma unroll
+    for (int j = 0; j < VW; ++j) a[j].init();
+    if (active) {
+        const T* p = src + o * R * inner + col;
+        uint64_t k = begin + ty;
+        for (; k + (uint64_t)(U - 1) * kWaves < end; k += (uint64_t)U * kWaves) {
+            VecW v[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) v[u] = load(p + (k + (uint64_t)u * kWaves) * inner);
+#pragma unroll
+            for (int j = 0; j < VW; ++j) {
+                T x[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) x[u] = v[u].e[j];
+                a[j].template push_block<U>(x, k, kWaves);
+            }
+        }
+        for (; k < end; k += kWaves) {
+            VecW v = load(p + k * inner);
+#pragma unroll
+            for (int j = 0; j < VW; ++j) a[j].push(v.e[j], k);
+        }
+    }
+    __shared__ S sm[kWaves - 1][RT_WAVE][VW];
+    if (ty > 0) {
+#pragma unroll
+        for (int j = 0; j < VW; ++j) sm[ty - 1][tx][j] = a[j];
+    }
+    __syncthreads();
+    if (ty == 0 && active) {
+        const uint64_t at = ((uint64_t)seg * outer + o) * inner + col;
+#pragma unroll
+        for (int j = 0; j < VW; ++j) {
+#pragma unroll
+            for (int w = 0; w < kWaves - 1; ++w) a[j].merge(sm[w][tx][j]);
+            if (part) part[at + j] = a[j];
+            else out[at + j] = a[j].result(flags);
+        }
+    }
+}
+
+// narrow inner (inner < 64) with a long reduced axis: the (R, inner) slab of one outer index is streamed as one contiguous run.
+// Lane t < Tn (Tn a multiple of inner) reads elements t, t + Tn, ... of the segment, which all lie in column t % inner, in ascending
+// row order; the lanes that share a column are merged through LDS.
+struct NarrowArgs {
+    uint64_t R, outer, seg_rows;        // rows per segment (a multiple of L)
+    uint32_t inner, Tn, L, splits;      // columns, active lanes, rows per trip, segments per outer index
+};
+
+template <class S, class T>
+__global__ __launch_bounds__(kBlock) void st_cols_narrow_kernel(const T* __restrict__ src, typename S::Out* __restrict__ out, S* __restrict__ part, NarrowArgs a,
+                                                                int flags) {
+    constexpr int U = 8;
+    const uint64_t o = blockIdx.x / a.splits;
+    const uint32_t seg = blockIdx.x - (uint32_t)(o * a.splits);
+    const uint64_t row_begin = (uint64_t)seg * a.seg_rows;
+    uint64_t row_end = row_begin + a.seg_rows;
+    if (row_end > a.R) row_end = a.R;
+    const uint32_t t = threadIdx.x;
+    S acc;
+    acc.init();
+    if (t < a.Tn && row_begin < row_end) {
+        const uint32_t lr = t / a.inner;                                     // row of this lane inside a trip
+        const T* p = src + (o * a.R + row_begin) * a.inner + t;             // element of trip 0
+        const uint64_t nrows = row_end - row_begin;
+        const uint64_t full = nrows / a.L;                                   // trips in which every lane has an element
+        uint64_t trip = 0;
+        for (; trip + U <= full; trip += U) {
+            T x[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) x[u] = __builtin_nontemporal_load(p + (trip + u) * a.Tn);
+            acc.template push_block<U>(x, row_begin + trip * a.L + lr, a.L);
+        }
+        for (; trip < full; ++trip) acc.push(__builtin_nontemporal_load(p + trip * a.Tn), row_begin + trip * a.L + lr);
+        if (full * a.L + lr < nrows) acc.push(__builtin_nontemporal_load(p + full * a.Tn), row_begin + full * a.L + lr);
+    }
+    __shared__ S sm[kBlock];
+    sm[t] = acc;
+    __syncthreads();
+    if (t < a.inner) {
+        for (uint32_t q = t + a.inner; q < a.Tn; q += a.inner) acc.merge(sm[q]);
+        const uint64_t at = ((uint64_t)seg * a.outer + o) * a.inner + t;
+        if (part) part[at] = acc;
+        else out[at] = acc.result(flags);
+    }
+}
+
+// ---- second stage -------------------------------------------------------------------------------------------------------
+// part[o * splits + k], one wave per output
+template <class S>
+__global__ __launch_bounds__(kBlock) void st_merge_rows_kernel(const S* __restrict__ part, typename S::Out* __restrict__ out, uint64_t nout, uint32_t splits, int flags) {
+    const uint64_t o = (uint64_t)blockIdx.x * kWaves + threadIdx.x / RT_WAVE;
+    if (o >= nout) return;
+    const uint32_t lane = threadIdx.x & (RT_WAVE - 1);
+    S a;
+    a.init();
+    for (uint32_t k = lane; k < splits; k += RT_WAVE) a.merge(part[o * splits + k]);
+    group_reduce(a, RT_WAVE, lane);
+    if (lane == 0) out[o] = a.result(flags);
+}
+// part[k * nout + o], one lane per output
+template <class S>
+__global__ __launch_bounds__(kBlock) void st_merge_cols_kernel(const S* __restrict__ part, typename S::Out* __restrict__ out, uint64_t nout, uint32_t splits, int flags) {
+    const uint64_t o = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (o >= nout) return;
+    S a = part[o];
+    for (uint32_t k = 1; k < splits; ++k) a.merge(part[(uint64_t)k * nout + o]);
+    out[o] = a.result(flags);
+}
+
+// an output with nothing to fold (R == 0)
+template <class S>
+__global__ __launch_bounds__(kBlock) void st_empty_kernel(typename S::Out* __restrict__ out, uint64_t nout, int flags) {
+    const uint64_t o = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (o >= nout) return;
+    S a;
+    a.init();
+    out[o] = a.result(flags);
+}
+
+// ---- host planning ------------------------------------------------------------------------------------------------------
+static int32_t too_many() { return rt_fail(RT_E_INVALID, "reduce: too many outputs for one launch"); }
+
+template <class S, class T>
+int32_t rows_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t rows, uint64_t R, int flags) {
+    hipStream_t s = ctx->stream;
+    if (R <= kTileMaxR) {
+        TileArgs a;
+        a.rows = rows;
+        a.R = (uint32_t)R;
+        a.pitch = a.R | 1u;
+        a.rpb = (uint32_t)(kTileBytes / sizeof(T)) / a.pitch;
+        a.r_div = make_fastdiv(a.R);
+        uint32_t g = 1;                                           // lanes per row: fill the block, at most one wave, at most R
+        while (g < 64 && (uint64_t)g * 2 * a.rpb <= (uint64_t)kBlock && g * 2 <= a.R) g <<= 1;
+        a.G = g;
+        const uint64_t blocks = (rows + a.rpb - 1) / a.rpb;
+        if (blocks >= (1ull << 31)) return too_many();
+        hipLaunchKernelGGL((st_rows_tile_kernel<S, T>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, out, a, flags);
+        RT_HIP(hipGetLastError());
+        return RT_OK;
+    }
+    const uint64_t want = (uint64_t)ctx->num_cus * 8;
+    if (R < 4096 && rows >= want / 2) {
+        const uint64_t blocks = (rows + kWaves - 1) / kWaves;
+        if (blocks >= (1ull << 31)) return too_many();
+        hipLaunchKernelGGL((st_rows_wave_kernel<S, T>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, out, rows, R, flags);
+        RT_HIP(hipGetLastError());
+        return RT_OK;
+    }
+    uint32_t splits = 1;
+    if (rows < want) {
+        const uint64_t min_seg = 16384;                           // elements; below this a split is not worth a second pass
+        const uint64_t by_size = R / min_seg, by_need = (want + rows - 1) / rows;
+        uint64_t sp = by_need < by_size ? by_need : by_size;
+        if (sp > 4096) sp = 4096;
+        if (sp > 1) splits = (uint32_t)sp;
+    }
+    if (rows * splits >= (1ull << 31)) return too_many();
+    if (splits == 1) {
+        hipLaunchKernelGGL((st_rows_block_kernel<S, T>), dim3((unsigned)rows), dim3(kBlock), 0, s, src, out, (S*)nullptr, R, 1u, R, flags);
+        RT_HIP(hipGetLastError());
+        return RT_OK;
+    }
+    constexpr uint64_t N = 16 / sizeof(T);
+    uint64_t seglen = (R + splits - 1) / splits;
+    seglen = (seglen + N * kBlock - 1) / (N * kBlock) * (N * kBlock);           // whole 16-byte vectors per lane
+    splits = (uint32_t)((R + seglen - 1) / seglen);
+    void* scratch = nullptr;
+    RT_TRY(rt_scratch(ctx, (size_t)(rows * splits) * sizeof(S), &scratch));
+    S* part = (S*)scratch;
+    hipLaunchKernelGGL((st_rows_block_kernel<S, T>), dim3((unsigned)(rows * splits)), dim3(kBlock), 0, s, src, out, part, R, splits, seglen, flags);
+    RT_HIP(hipGetLastError());
+    hipLaunchKernelGGL((st_merge_rows_kernel<S>), dim3((unsigned)((rows + kWaves - 1) / kWaves)), dim3(kBlock), 0, s, part, out, rows, splits, flags);
+    RT_HIP(hipGetLastError());
+    return RT_OK;
+}
+
+template <class S, class T, int VW>
+int32_t cols_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t outer, uint64_t R, uint64_t inner, int flags) {
+    hipStream_t s = ctx->stream;
+    const uint64_t per_tile = (uint64_t)RT_WAVE * VW;
+    const uint64_t tiles = (inner + per_tile - 1) / per_tile;
+    const uint64_t want = (uint64_t)ctx->num_cus * 2;           // two blocks per CU, as for the plain column reductions
+    uint32_t splits = 1;
+    if (outer * tiles < want) {
+        const uint64_t min_seg = 64;
+        const uint64_t by_size = R / min_seg, by_need = (want + outer * tiles - 1) / (outer * tiles);
+        uint64_t sp = by_need < by_size ? by_need : by_size;
+        if (sp > 1024) sp = 1024;
+        if (sp > 1) splits = (uint32_t)sp;
+    }
+    uint64_t seglen = (R + splits - 1) / splits;
+    if (splits > 1) {
+        seglen = (seglen + 4 * kWaves - 1) / (4 * kWaves) * (4 * kWaves);
+        splits = (uint32_t)((R + seglen - 1) / seglen);
+    }
+    const uint64_t blocks = outer * splits * tiles;
+    if (blocks >= (1ull << 31) || tiles >= (1ull << 31)) return too_many();
+    S* part = nullptr;
+    if (splits > 1) {
+        void* scratch = nullptr;
+        RT_TRY(rt_scratch(ctx, (size_t)(splits * outer * inner) * sizeof(S), &scratch));
+        part = (S*)scratch;
+    }
+    hipLaunchKernelGGL((st_cols_kernel<S, T, VW>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, out, part, R, inner, outer, (uint32_t)tiles, splits, seglen,
+                       flags);
+    RT_HIP(hipGetLastError());
+    if (splits > 1) {
+        const uint64_t nout = outer * inner;
+        const uint64_t mb = (nout + kBlock - 1) / kBlock;
+        if (mb >= (1ull << 31)) return too_many();
+        hipLaunchKernelGGL((st_merge_cols_kernel<S>), dim3((unsigned)mb), dim3(kBlock), 0, s, part, out, nout, splits, flags);
+        RT_HIP(hipGetLastError());
+    }
+    return RT_OK;
+}
+
+template <class S, class T>
+int32_t narrow_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t outer, uint64_t R, uint64_t inner, int flags) {
+    NarrowArgs a;
+    a.R = R;
+    a.outer = outer;
+    a.inner = (uint32_t)inner;
+    a.Tn = (uint32_t)kBlock / a.inner * a.inner;
+    a.L = a.Tn / a.inner;
+    const uint64_t trips = (R + a.L - 1) / a.L;
+    const uint64_t want = (uint64_t)ctx->num_cus * 4;
+    uint64_t splits = outer >= want ? 1 : (want + outer - 1) / outer;
+    if (splits > trips / 16) splits = trips / 16;               // at least 16 trips per block
+    if (splits < 1) splits = 1;
+    const uint64_t seg_trips = (trips + splits - 1) / splits;
+    splits = (trips + seg_trips - 1) / seg_trips;
+    a.seg_rows = seg_trips * a.L;
+    a.splits = (uint32_t)splits;
+    const uint64_t blocks = outer * splits;
+    if (blocks >= (1ull << 31)) return too_many();
+    S* part = nullptr;
+    if (splits > 1) {
+        void* scratch = nullptr;
+        RT_TRY(rt_scratch(ctx, (size_t)(splits * outer * inner) * sizeof(S), &scratch));
+        part = (S*)scratch;
+    }
+    hipLaunchKernelGGL((st_cols_narrow_kernel<S, T>), dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream, src, out, part, a, flags);
+    RT_HIP(hipGetLastError());
+    if (splits > 1) {
+        const uint64_t nout = outer * inner;
+        hipLaunchKernelGGL((st_merge_cols_kernel<S>), dim3((unsigned)((nout + kBlock - 1) / kBlock)), dim3(kBlock), 0, ctx->stream, part, out, nout,
+                           (uint32_t)splits, flags);
+        RT_HIP(hipGetLastError());
+    }
+    return RT_OK;
+}
+
+template <class S, class T>
+int32_t plan(rt_ctx* ctx, const void* src_v, void* out_v, uint64_t outer, uint64_t R, uint64_t inner, int flags) {
+    const T* src = (const T*)src_v;
+    typename S::Out* out = (typename S::Out*)out_v;
+    if (outer == 0 || inner == 0) return RT_OK;
+    const uint64_t nout = outer * inner;
+    if (R == 0) {
+        const uint64_t blocks = (nout + kBlock - 1) / kBlock;
+        if (blocks >= (1ull << 31)) return too_many();
+        hipLaunchKernelGGL((st_empty_kernel<S>), dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream, out, nout, flags);
+        RT_HIP(hipGetLastError());
+        return RT_OK;
+    }
+    if (inner == 1) return rows_plan<S, T>(ctx, src, out, outer, R, flags);
+    if (inner < 64 && R >= 64 && outer < (1ull << 20)) return narrow_plan<S, T>(ctx, src, out, outer, R, inner, flags);
+    constexpr int N = 16 / sizeof(T);
+    const bool vec = (inner % N == 0) && ((reinterpret_cast<uintptr_t>(src) & 15) == 0);
+    if (vec) return cols_plan<S, T, N>(ctx, src, out, outer, R, inner, flags);
+    return cols_plan<S, T, 1>(ctx, src, out, outer, R, inner, flags);
+}
+
+template <class T>
+int32_t stat_ops(rt_ctx* ctx, int op, const void* src, void* out, uint64_t outer, uint64_t R, uint64_t inner) {
+    const int code = op & 0xff, flags = op & ~0xff;
+    switch (code) {
+        case RT_R_VARIANCE:
+            if (flags & ~(RT_R_FLAG_UNBIASED | RT_R_FLAG_STD)) break;
+            return plan<MomentState<T>, T>(ctx, src, out, outer, R, inner, flags);
+        case RT_R_LOGSUMEXP:
+            if (flags) break;
+            return plan<LseState<T>, T>(ctx, src, out, outer, R, inner, flags);
+        case RT_R_NORM:
+            if (flags == RT_R_FLAG_L1) return plan<NormState<T, false>, T>(ctx, src, out, outer, R, inner, flags);
+            if (flags == RT_R_FLAG_L2) return plan<NormState<T, true>, T>(ctx, src, out, outer, R, inner, flags);
+            return rt_fail(RT_E_INVALID, "reduce: norm needs exactly one of RT_R_FLAG_L1 / RT_R_FLAG_L2 (op 0x%x)", op);
+    }
+    return rt_fail(RT_E_INVALID, "reduce: op 0x%x is not a reduction op code with valid flags", op);
+}
+
+template <class T>
+int32_t arg_ops(rt_ctx* ctx, int op, const void* src, void* out, uint64_t outer, uint64_t R, uint64_t inner) {
+    if (op == RT_R_ARGMAX) return plan<ArgState<T, true>, T>(ctx, src, out, outer, R, inner, 0);
+    return plan<ArgState<T, false>, T>(ctx, src, out, outer, R, inner, 0);
+}
+
+}  // namespace
+
+int32_t rt_reduce_stat(rt_ctx* ctx, int dtype, int op, const void* src, void* out, uint64_t outer, uint64_t R, uint64_t inner) {
+    const int code = op & 0xff;
+    if (code == RT_R_ARGMAX || code == RT_R_ARGMIN) {
+        if (op != code) return rt_fail(RT_E_INVALID, "argmax: op 0x%x carries flags", op);
+        switch (dtype) {
+            case RT_U8: return arg_ops<uint8_t>(ctx, op, src, out, outer, R, inner);
+            case RT_I8: return arg_ops<int8_t>(ctx, op, src, out, outer, R, inner);
+            case RT_U16: return arg_ops<uint16_t>(ctx, op, src, out, outer, R, inner);
+            case RT_I16: return arg_ops<int16_t>(ctx, op, src, out, outer, R, inner);
+            case RT_U32: return arg_ops<uint32_t>(ctx, op, src, out, outer, R, inner);
+            case RT_I32: return arg_ops<int32_t>(ctx, op, src, out, outer, R, inner);
+            case RT_U64: return arg_ops<uint64_t>(ctx, op, src, out, outer, R, inner);
+            case RT_I64: return arg_ops<int64_t>(ctx, op, src, out, outer, R, inner);
+            case RT_F32: return arg_ops<float>(ctx, op, src, out, outer, R, inner);
+            case RT_F64: return arg_ops<double>(ctx, op, src, out, outer, R, inner);
+        }
+        return rt_fail(RT_E_DTYPE, "argmax: dtype code %d has no order to search (f32/f64 in the reference, 8..64-bit integers added here)", dtype);
+    }
+    switch (dtype) {
+        case RT_F32: return stat_ops<float>(ctx, op, src, out, outer, R, inner);
+        case RT_F64: return stat_ops<double>(ctx, op, src, out, outer, R, inner);
+    }
+    return rt_fail(RT_E_DTYPE, "reduce: variance, logsumexp and norms are defined for f32 / f64 (the reference bounds them on WeightValue), not dtype code %d",
+                   dtype);
+}
+
+extern "C" int32_t rt_argmax_flat(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, uint64_t src_len, uint64_t* dst, uint64_t dst_len,
+                                  uint64_t start, uint64_t len) {
+    RT_TRY(rt_ctx_enter(ctx));
+    const int es = rt_elem_size(dtype);
+    if (!es) return rt_fail(RT_E_DTYPE, "argmax: unknown dtype code %d", dtype);
+    if (op != RT_R_ARGMAX && op != RT_R_ARGMIN) return rt_fail(RT_E_INVALID, "argmax: op code %d is neither argmax (9) nor argmin (10)", op);
+    RT_TRY(rt_check_reduce_flat(src_len, src, dst, dst_len, start, len));
+    CtxGuard g(ctx);
+    return rt_reduce_stat(ctx, dtype, op, (const char*)src + start * es, dst, 1, len, 1);
+}
+
+extern "C" int32_t rt_argmax_nd(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, uint64_t src_len, uint64_t offset, int32_t rank,
+                                const uint64_t* shape, const int64_t* strides, uint64_t* dst, uint64_t dst_len, int32_t dim) {
+    RT_TRY(rt_ctx_enter(ctx));
+    const int es = rt_elem_size(dtype);
+    if (!es) return rt_fail(RT_E_DTYPE, "argmax: unknown dtype code %d", dtype);
+    if (op != RT_R_ARGMAX && op != RT_R_ARGMIN) return rt_fail(RT_E_INVALID, "argmax: op code %d is neither argmax (9) nor argmin (10)", op);
+    uint64_t outer = 0, inner = 0;
+    bool run = false;
+    RT_TRY(rt_check_reduce_nd(src_len, src, offset, rank, shape, strides, dst, dst_len, dim, &outer, &inner, &run));
+    if (!run) return RT_OK;
+    CtxGuard g(ctx);
+    return rt_reduce_stat(ctx, dtype, op, (const char*)src + offset * es, dst, outer, shape[dim], inner);
+}

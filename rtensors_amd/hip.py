@@ -28,7 +28,10 @@ UNARY = {n: i for i, n in enumerate(
 SCALAR = {n: i for i, n in enumerate("add sub mul div log log1p leaky_relu elu leaky_grad".split())}
 CONTIGUITY = {"row_major": 0, "column_major": 1, "none": 2}     # core/meta.rs:744-750
 BINARY = {"add": 0, "sub": 1, "mul": 2, "div": 3}
-REDUCE = {"sum": 1, "prod": 2, "max": 3, "min": 4, "mean": 5}
+# ReductionOpTypes::get_code (ops/reduction/mod.rs:161-175) in the low byte; the payload of Variance / Stdev / Norm in the flag bits
+REDUCE = {"sum": 1, "prod": 2, "max": 3, "min": 4, "mean": 5,
+          "pop_var": 6, "var": 6 | 0x100, "pop_std": 6 | 0x200, "std": 6 | 0x300, "logsumexp": 7, "l1_norm": 8 | 0x100, "l2_norm": 8 | 0x200,
+          "argmax": 9, "argmin": 10}
 
 # rt_status -> TensorError variant (core/tensor.rs:11-53; HipError stands where CudaError stands)
 _KIND = {1: "InvalidArgument", 2: "UnsupportedOperation", 3: "IdxOutOfBounds", 4: "HipError", 5: "HipError",
@@ -226,6 +229,19 @@ class Hip:
     def apply_reduce_contiguous_nd(self, src: Tuple[HipBuf, tuple], dst: HipBuf, dim: int, op: str):
         sb, (off, shape, strides) = src
         _check(lib.rt_reduce_nd(self._ctx, sb.dtype, REDUCE[op], sb.ptr, sb.len, off, len(shape), _u64s(shape), _i64s(strides),
+                                dst.ptr, dst.len, dim))
+
+    # Backend::apply_argmax_contiguous_flat / _nd (backend/mod.rs:412-463): dst is a u64 buffer
+    def apply_argmax_contiguous_flat(self, src: HipBuf, dst: HipBuf, start: int, length: int, op: str):
+        if dst.dtype != U64:
+            raise TensorError(1, "argmax writes u64 indices")
+        _check(lib.rt_argmax_flat(self._ctx, src.dtype, REDUCE[op], src.ptr, src.len, dst.ptr, dst.len, start, length))
+
+    def apply_argmax_contiguous_nd(self, src: Tuple[HipBuf, tuple], dst: HipBuf, dim: int, op: str):
+        if dst.dtype != U64:
+            raise TensorError(1, "argmax writes u64 indices")
+        sb, (off, shape, strides) = src
+        _check(lib.rt_argmax_nd(self._ctx, sb.dtype, REDUCE[op], sb.ptr, sb.len, off, len(shape), _u64s(shape), _i64s(strides),
                                 dst.ptr, dst.len, dim))
 
     def gather(self, src: HipBuf, meta, dst: HipBuf):

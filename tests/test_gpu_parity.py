@@ -1,6 +1,7 @@
 """GPU parity: every kernel family of the HIP backend, called through the C ABI, against the CPU oracle on the same
 seeded inputs.  Bit-exact for integers, for f32/f64 elementwise results, and for max/min; float sum/prod/mean within
 rel 1e-5 (f32) / 1e-12 (f64) of sum|x|; transcendental unaries within the reference's own 1e-5."""
+import os
 import numpy as np
 import pytest
 
@@ -558,8 +559,8 @@ def test_reduce_offset_and_errors(hip):
     with pytest.raises(H.TensorError):
         hip.apply_reduce_contiguous_nd((g, (0, [4, 6], [6, 1])), hip.alloc(H.F64, 4), 2, "sum")
     f = hip.alloc_from_slice(H.F32, np.zeros(4, np.float32))
-    with pytest.raises(H.TensorError):                                           # variance etc. are outside this path
-        lib_status = __import__("rtensors_amd._ffi", fromlist=["lib"]).lib.rt_reduce_flat(hip._ctx, H.F32, 6, f.ptr, 4, f.ptr, 4, 0, 4)
+    with pytest.raises(H.TensorError):                                           # not a reduction op code
+        lib_status = __import__("rtensors_amd._ffi", fromlist=["lib"]).lib.rt_reduce_flat(hip._ctx, H.F32, 11, f.ptr, 4, f.ptr, 4, 0, 4)
         H._check(lib_status)
 
 
@@ -874,6 +875,144 @@ def test_reduction_shapes_short_rows_narrow_columns_short_axis(hip, dtype):
     for R in (1, 2, 4, 5, 16, 31, 32, 33):
         for inner, outer in ((2, 1000), (3, 1), (64, 50), (100, 7), (1024, 3), (1028, 2)):
             _check_reduce(hip, dtype, outer, R, inner, rng, offset=int(rng.integers(0, 5)))
+
+
+def _check_stat(hip, dtype, outer, R, inner, rng, offset=0):
+    """Variance / stdev / logsumexp / norms along the middle axis of (outer, R, inner).  The GPU folds in tree order, the oracle in
+    index order, so the comparison is by tolerance: within 1e-5 (f32) / 1e-12 (f64), relative, of the oracle run in float64 on the
+    same values (for f64 that is the oracle itself)."""
+    code = cpu.DTYPE_BY_NAME[dtype]
+    n = outer * R * inner
+    x = (rng.normal(size=n + offset) * 3 + 10).astype(cpu.NP_DTYPE[code])
+    src = hip.alloc_from_slice(code, x)
+    shape, strides = [outer, R, inner], [R * inner, inner, 1]
+    m = MetaTensor(shape, strides, offset)
+    x64 = x.astype(np.float64)
+    rel = 1e-5 if dtype == "f32" else 1e-12
+    for op in cpu.STAT_OPS:
+        with np.errstate(all="ignore"):
+            want = cpu.reduce_stat(cpu.F64, op, x64, m, 1)
+        dst = hip.alloc(code, outer * inner)
+        hip.apply_reduce_contiguous_nd((src, (offset, shape, strides)), dst, 1, op)
+        got = hip.dump(dst).astype(np.float64)
+        assert (np.isnan(got) == np.isnan(want)).all(), (dtype, op, outer, R, inner)
+        fin = np.isfinite(want)
+        assert (np.abs(got - want)[fin] <= rel * np.abs(want)[fin] + 1e-300).all(), (dtype, op, outer, R, inner, offset, got[:4], want[:4])
+
+
+def _check_arg(hip, dtype, outer, R, inner, rng, offset=0):
+    """argmax / argmin: exact.  Values from a small set so that ties are everywhere; floats also carry NaN."""
+    code = cpu.DTYPE_BY_NAME[dtype]
+    n = outer * R * inner
+    if dtype[0] == "f":
+        x = np.round(rng.normal(size=n + offset) * 2).astype(cpu.NP_DTYPE[code])
+        x[rng.integers(0, n + offset, size=max(1, (n + offset) // 50))] = np.nan
+    else:
+        lo = 0 if dtype[0] == "u" else -5
+        x = rng.integers(lo, lo + 11, size=n + offset).astype(cpu.NP_DTYPE[code])
+    src = hip.alloc_from_slice(code, x)
+    shape, strides = [outer, R, inner], [R * inner, inner, 1]
+    m = MetaTensor(shape, strides, offset)
+    for op in cpu.ARG_OPS:
+        want = cpu.argmax(code, op, x, m, 1)
+        dst = hip.alloc(cpu.U64, outer * inner)
+        hip.apply_argmax_contiguous_nd((src, (offset, shape, strides)), dst, 1, op)
+        got = hip.dump(dst)
+        assert got.tolist() == want.tolist(), (dtype, op, outer, R, inner, offset)
+
+
+STAT_SHAPES = ([(rows, R, 1) for R in (1, 2, 3, 7, 8, 31, 32, 33, 64, 65, 100, 255, 256, 1000, 1024, 1025, 2000, 4095) for rows in (1, 77, 1500)]
+               + [(3, 70001, 1), (1, 300000, 1), (1100, 4100, 1)]
+               + [(outer, R, inner) for inner in (2, 3, 5, 17, 63, 64, 100, 128) for R, outer in ((64, 3), (1000, 1), (5003, 2), (70001, 1))]
+               + [(outer, R, inner) for R in (1, 2, 5, 16, 33) for inner, outer in ((2, 1000), (3, 1), (64, 50), (1028, 2))]
+               + [(1, 300, 5000), (2, 4000, 260), (1, 70, 2052)])
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64"])
+def test_statistic_reductions_shapes(hip, dtype):
+    rng = np.random.default_rng(abs(hash(dtype)) % 2 ** 31)
+    for outer, R, inner in STAT_SHAPES:
+        _check_stat(hip, dtype, outer, R, inner, rng, offset=int(rng.integers(0, 5)))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64", "i32", "u8", "i64", "i16"])
+def test_argmax_argmin_shapes(hip, dtype):
+    rng = np.random.default_rng(abs(hash(dtype)) % 2 ** 31)
+    for outer, R, inner in STAT_SHAPES:
+        _check_arg(hip, dtype, outer, R, inner, rng, offset=int(rng.integers(0, 5)))
+
+
+def test_statistic_reductions_known_answers_and_edges(hip):
+    """The reference's Cuda known answers through the C ABI, the flat entry points, and the edge cases the oracle tests pin."""
+    import json
+    from rtensors_amd import hip as H
+    cases = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_reduce_stat_vectors.json")))["cases"]
+    for c in cases:
+        code = cpu.DTYPE_BY_NAME[c["dtype"]]
+        x = np.array(c["data"], dtype=cpu.NP_DTYPE[code])
+        src = hip.alloc_from_slice(code, x)
+        shape = c["shape"]
+        strides = [shape[1], 1]
+        arg = c["op"] in cpu.ARG_OPS
+        nout = 1 if c["dim"] is None else int(np.prod(shape)) // shape[c["dim"]]
+        dst = hip.alloc(cpu.U64 if arg else code, nout)
+        if c["dim"] is None:
+            (hip.apply_argmax_contiguous_flat if arg else hip.apply_reduce_contiguous_flat)(src, dst, 0, x.size, c["op"])
+        else:
+            (hip.apply_argmax_contiguous_nd if arg else hip.apply_reduce_contiguous_nd)((src, (0, shape, strides)), dst, c["dim"], c["op"])
+        got = hip.dump(dst)
+        if arg:
+            assert got.tolist() == c["want"], c
+        else:
+            assert np.allclose(got.astype(np.float64), c["want"], rtol=1e-6 if c["dtype"] == "f32" else 1e-14, atol=0), (c, got)
+    nan, inf = float("nan"), float("inf")
+
+    def flat(dtype, op, values, start=0, length=None):
+        code = cpu.DTYPE_BY_NAME[dtype]
+        x = np.array(values, dtype=cpu.NP_DTYPE[code])
+        src = hip.alloc_from_slice(code, x) if x.size else hip.alloc(code, 1)
+        arg = op in cpu.ARG_OPS
+        dst = hip.alloc(cpu.U64 if arg else code, 1)
+        (hip.apply_argmax_contiguous_flat if arg else hip.apply_reduce_contiguous_flat)(src, dst, start, x.size - start if length is None else length, op)
+        return hip.dump(dst)[0]
+    assert flat("f64", "argmax", [1, 5, 5, 2]) == 1 and flat("f64", "argmin", [3, 1, 1, 2]) == 1
+    assert flat("f64", "argmax", [nan, 2, nan, 7, 7]) == 3 and flat("f64", "argmax", [nan, nan]) == 0 and flat("f64", "argmax", [-inf, -inf]) == 0
+    assert flat("f32", "argmin", [inf, 4, -inf, -inf]) == 2
+    assert flat("f64", "argmax", [9, 1, 5, 5, 2], start=1) == 1                 # positions count from `start`
+    assert flat("i32", "argmax", [3, -7, 9, 9, 0]) == 2 and flat("u8", "argmin", [3, 0, 9, 0]) == 1
+    assert flat("f64", "logsumexp", [-inf, -inf]) == -inf and flat("f64", "logsumexp", [1.0, inf, 2.0]) == inf
+    assert np.isnan(flat("f64", "logsumexp", [1.0, nan]))
+    assert flat("f64", "logsumexp", [], length=0) == -inf and flat("f64", "argmax", [], length=0) == 0 and flat("f64", "l2_norm", [], length=0) == 0
+    assert np.isclose(flat("f64", "logsumexp", [1000.0, 1000.0]), 1000.0 + np.log(2.0), rtol=1e-15)
+    assert np.isclose(flat("f32", "logsumexp", [-1000.0, -1001.0]), -1000.0 + np.log1p(np.exp(-1.0)), rtol=1e-6)
+    assert flat("f64", "pop_var", [4.0]) == 0.0 and np.isnan(flat("f64", "var", [4.0]))
+    assert np.isclose(flat("f64", "var", [1e9, 1e9 + 1, 1e9 + 2]), 1.0, rtol=1e-12)
+    big = 1e9 + np.arange(100001, dtype=np.float64) % 3                            # a large common offset must not cancel
+    assert np.isclose(flat("f64", "pop_var", big), big.var(), rtol=1e-11)
+    # what the entry points refuse
+    f = hip.alloc_from_slice(H.F32, np.arange(8, dtype=np.float32))
+    i = hip.alloc_from_slice(H.I32, np.arange(8, dtype=np.int32))
+    o32, o64 = hip.alloc(H.F32, 8), hip.alloc(H.U64, 8)
+    with pytest.raises(H.TensorError) as e:
+        hip.apply_reduce_contiguous_flat(f, o32, 0, 8, "argmax")                   # kinds are not swapped between entry points
+    assert e.value.kind == "InvalidArgument"
+    with pytest.raises(H.TensorError) as e:
+        hip.apply_argmax_contiguous_flat(f, o64, 0, 8, "sum")
+    assert e.value.kind == "InvalidArgument"
+    with pytest.raises(H.TensorError) as e:
+        hip.apply_reduce_contiguous_flat(i, hip.alloc(H.I32, 1), 0, 8, "var")       # WeightValue kinds on an integer
+    assert e.value.kind == "UnsupportedOperation"
+    lib = __import__("rtensors_amd._ffi", fromlist=["lib"]).lib
+    for bad in (8, 8 | 0x300, 7 | 0x100, 6 | 0x400, 11, 0):
+        with pytest.raises(H.TensorError):
+            H._check(lib.rt_reduce_flat(hip._ctx, H.F32, bad, f.ptr, 8, o32.ptr, 8, 0, 8))
+    with pytest.raises(H.TensorError) as e:
+        hip.apply_argmax_contiguous_nd((f, (0, [2, 4], [1, 2])), o64, 0, "argmax")
+    assert e.value.kind == "WrongDims"
+    with pytest.raises(H.TensorError) as e:
+        hip.apply_argmax_contiguous_nd((f, (0, [2, 4], [4, 1])), hip.alloc(H.U64, 3), 0, "argmax")
+    assert e.value.kind == "IdxOutOfBounds"
+    hip.sync()
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f64", "i32", "u8", "i64"])
