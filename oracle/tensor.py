@@ -217,6 +217,13 @@ class OTensor:
     # ---- reductions: ops/reduction/mod.rs:262-302, 346-408 ------------------------------------------------------------
     def reduce(self, op: str, axis: Optional[int] = None, honour_offset: bool = True) -> "OTensor":
         t = self if self.meta.is_contiguous() else self.contiguous()
+        if op in cpu.STAT_OPS or op in cpu.ARG_OPS:                        # do_reduce / do_argmax with the Cuda backend's kinds
+            arg = op in cpu.ARG_OPS
+            if axis is not None and not (0 <= axis < t.meta.rank()):
+                raise TensorError("InvalidDim", "reduction axis out of range")
+            out = (cpu.argmax if arg else cpu.reduce_stat)(t.dtype, op, t.buf, t.meta, axis)
+            out_meta = MetaTensor([], [], 0) if axis is None else reduction_output_meta(t.meta, axis)
+            return OTensor(cpu.U64 if arg else t.dtype, out, out_meta)
         if axis is None:                                                  # Idx::Item
             out = cpu.reduce_flat(t.dtype, op, t.buf, t.meta.offset, t.meta.size())
             return OTensor(t.dtype, out, MetaTensor([], [], 0))
@@ -237,6 +244,20 @@ class OTensor:
     def max(self): return self.reduce("max")
     def min(self): return self.reduce("min")
     def prod(self): return self.reduce("prod")
+    def var_at(self, axis): return self.reduce("var", axis)
+    def pop_var_at(self, axis): return self.reduce("pop_var", axis)
+    def std_at(self, axis, unbiased): return self.reduce("std" if unbiased else "pop_std", axis)
+    def norm_at(self, axis, norm): return self.reduce({"L1": "l1_norm", "L2": "l2_norm"}[norm], axis)
+    def logsumexp_at(self, axis): return self.reduce("logsumexp", axis)
+    def argmax_at(self, axis): return self.reduce("argmax", axis)
+    def argmin_at(self, axis): return self.reduce("argmin", axis)
+    def var(self): return self.reduce("var")
+    def pop_var(self): return self.reduce("pop_var")
+    def std(self, unbiased): return self.reduce("std" if unbiased else "pop_std")
+    def norm(self, norm): return self.reduce({"L1": "l1_norm", "L2": "l2_norm"}[norm])
+    def logsumexp(self): return self.reduce("logsumexp")
+    def argmax(self): return self.reduce("argmax")
+    def argmin(self): return self.reduce("argmin")
 
 
 def mean_l1_loss(y: OTensor, target: OTensor):

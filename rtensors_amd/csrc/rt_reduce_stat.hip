@@ -44,6 +44,7 @@ __device__ __forceinline__ double m_max(double a, double b) { return fmax(a, b);
 
 template <class T> struct MomentState {
     typedef T Out;
+    static constexpr int kColsBlocksPerCU = 2;
     T mean, m2;
     uint64_t n;
     __device__ __forceinline__ void init() { mean = (T)0; m2 = (T)0; n = 0; }
@@ -78,6 +79,7 @@ template <class T> struct MomentState {
 
 template <class T> struct LseState {
     typedef T Out;
+    static constexpr int kColsBlocksPerCU = 4;                  // one exp per element: more waves per CU to hide it (0.215 -> 0.180 ms on 1 GiB)
     T m, s;
     __device__ __forceinline__ void init() { m = -std::numeric_limits<T>::infinity(); s = (T)0; }
     // exp(x - top), with x == top giving 1 also when both are infinite
@@ -107,6 +109,7 @@ template <class T> struct LseState {
 
 template <class T, bool SQ> struct NormState {
     typedef T Out;
+    static constexpr int kColsBlocksPerCU = 2;
     T s;
     __device__ __forceinline__ void init() { s = (T)0; }
     __device__ __forceinline__ void push(T x, uint64_t) { s = s + (SQ ? x * x : m_abs(x)); }
@@ -122,6 +125,7 @@ template <class T, bool SQ> struct NormState {
 
 template <class T, bool MAX> struct ArgState {
     typedef uint64_t Out;
+    static constexpr int kColsBlocksPerCU = 2;
     T v;
     uint64_t idx;
     __device__ __forceinline__ void init() {
@@ -382,72 +386,116 @@ __global__ __launch_bounds__(kBlock) void st_cols_kernel(const T* __restrict__ s
     }
 }
 
-// narrow inner (inner < 64) with a long reduced axis: the (R, inner) slab of one outer index is streamed as one contiguous run.
-// Lane t < Tn (Tn a multiple of inner) reads elements t, t + Tn, ... of the segment, which all lie in column t % inner, in ascending
-// row order; the lanes that share a column are merged through LDS.
+// Narrow inner (fewer columns than a wave of vectors covers): the (R, inner) slab of one outer index is read as one contiguous stream
+// in tiles of Tn * VW elements, a multiple of inner, so that lane t always meets the same VW columns (element t * VW + j of every
+// tile, column (t * VW + j) % inner) in rows tile * L + (t * VW + j) / inner, L rows per tile, ascending.  The lanes that share a
+// column are merged through LDS at the end.
 struct NarrowArgs {
-    uint64_t R, outer, seg_rows;        // rows per segment (a multiple of L)
-    uint32_t inner, Tn, L, splits;      // columns, active lanes, rows per trip, segments per outer index
+    uint64_t R, outer, seg_tiles;       // tiles per segment
+    uint32_t inner, Tn, L, splits, G;   // columns, active lanes, rows per tile, segments per outer index, lanes per column in the final merge
+    FastDiv32 inner_div;
 };
 
-template <class S, class T>
+template <class S, class T, int VW>
 __global__ __launch_bounds__(kBlock) void st_cols_narrow_kernel(const T* __restrict__ src, typename S::Out* __restrict__ out, S* __restrict__ part, NarrowArgs a,
                                                                 int flags) {
-    constexpr int U = 8;
+    struct alignas(sizeof(T) * VW) VecW { T e[VW]; };
+    constexpr int U = 4;
+    __shared__ S sm[kBlock * VW];
     const uint64_t o = blockIdx.x / a.splits;
-    const uint32_t seg = blockIdx.x - (uint32_t)(o * a.splits);
-    const uint64_t row_begin = (uint64_t)seg * a.seg_rows;
-    uint64_t row_end = row_begin + a.seg_rows;
-    if (row_end > a.R) row_end = a.R;
+    const uint32_t seg = (uint32_t)(blockIdx.x - o * a.splits);
     const uint32_t t = threadIdx.x;
-    S acc;
-    acc.init();
-    if (t < a.Tn && row_begin < row_end) {
-        const uint32_t lr = t / a.inner;                                     // row of this lane inside a trip
-        const T* p = src + (o * a.R + row_begin) * a.inner + t;             // element of trip 0
-        const uint64_t nrows = row_end - row_begin;
-        const uint64_t full = nrows / a.L;                                   // trips in which every lane has an element
-        uint64_t trip = 0;
-        for (; trip + U <= full; trip += U) {
-            T x[U];
+    const uint32_t tile_elems = a.Tn * VW;
+    const uint64_t slab = a.R * a.inner;
+    const T* base = src + o * slab;
+    S acc[VW];
+    uint32_t krow[VW];
 #pragma unroll
-            for (int u = 0; u < U; ++u) x[u] = __builtin_nontemporal_load(p + (trip + u) * a.Tn);
-            acc.template push_block<U>(x, row_begin + trip * a.L + lr, a.L);
+    for (int j = 0; j < VW; ++j) { acc[j].init(); krow[j] = fd_div(t * VW + j, a.inner_div); }
+    if (t < a.Tn) {
+        const uint64_t tile_begin = (uint64_t)seg * a.seg_tiles;
+        uint64_t tile_end = tile_begin + a.seg_tiles;
+        const uint64_t ntiles = (a.R + a.L - 1) / a.L;
+        if (tile_end > ntiles) tile_end = ntiles;
+        auto load = [&](uint64_t e) -> VecW {
+            if constexpr (sizeof(VecW) == 16) {
+                return rt_ld16_nt(reinterpret_cast<const VecW*>(base + e));
+            } else {
+                VecW w;
+                w.e[0] = __builtin_nontemporal_load(base + e);
+                return w;
+            }
+        };
+        uint64_t tl = tile_begin;
+        // batches of U tiles that this lane's vector lies inside completely
+        for (; tl + U <= tile_end && (tl + U - 1) * tile_elems + (uint64_t)t * VW + VW <= slab; tl += U) {
+            VecW x[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) x[u] = load((tl + u) * tile_elems + (uint64_t)t * VW);
+#pragma unroll
+            for (int j = 0; j < VW; ++j) {
+                T col[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) col[u] = x[u].e[j];
+                acc[j].template push_block<U>(col, tl * a.L + krow[j], a.L);
+            }
         }
-        for (; trip < full; ++trip) acc.push(__builtin_nontemporal_load(p + trip * a.Tn), row_begin + trip * a.L + lr);
-        if (full * a.L + lr < nrows) acc.push(__builtin_nontemporal_load(p + full * a.Tn), row_begin + full * a.L + lr);
+        for (; tl < tile_end; ++tl) {                          // the last tiles, element by element where the slab ends inside a vector
+            const uint64_t e = tl * tile_elems + (uint64_t)t * VW;
+#pragma unroll
+            for (int j = 0; j < VW; ++j)
+                if (e + j < slab) acc[j].push(base[e + j], tl * a.L + krow[j]);
+        }
     }
-    __shared__ S sm[kBlock];
-    sm[t] = acc;
+#pragma unroll
+    for (int j = 0; j < VW; ++j) sm[t * VW + j] = acc[j];
     __syncthreads();
-    if (t < a.inner) {
-        for (uint32_t q = t + a.inner; q < a.Tn; q += a.inner) acc.merge(sm[q]);
-        const uint64_t at = ((uint64_t)seg * a.outer + o) * a.inner + t;
-        if (part) part[at] = acc;
-        else out[at] = acc.result(flags);
+    // column c is held by the L states c, c + inner, ...: G lanes per column (a power of two, inner * G <= kBlock) share them
+    const uint32_t c = t / a.G, j = t & (a.G - 1);
+    S r;
+    r.init();
+    if (c < a.inner) {
+        for (uint32_t q = j; q < a.L; q += a.G) r.merge(sm[c + q * a.inner]);
+    }
+    group_reduce(r, a.G, j);
+    if (c < a.inner && j == 0) {
+        const uint64_t at = ((uint64_t)seg * a.outer + o) * a.inner + c;
+        if (part) part[at] = r;
+        else out[at] = r.result(flags);
     }
 }
 
 // ---- second stage -------------------------------------------------------------------------------------------------------
-// part[o * splits + k], one wave per output
+// Partial state k of output o lies at part[o * ostride + k * kstride] (rows: ostride = splits, kstride = 1; columns: ostride = 1,
+// kstride = number of outputs).  One wave per output, the lanes spread over k: few outputs with many partials each must not be
+// folded by one lane in one long chain of dependent loads.
 template <class S>
-__global__ __launch_bounds__(kBlock) void st_merge_rows_kernel(const S* __restrict__ part, typename S::Out* __restrict__ out, uint64_t nout, uint32_t splits, int flags) {
+__global__ __launch_bounds__(kBlock) void st_merge_wave_kernel(const S* __restrict__ part, typename S::Out* __restrict__ out, uint64_t nout, uint32_t splits,
+                                                               uint64_t ostride, uint64_t kstride, int flags) {
     const uint64_t o = (uint64_t)blockIdx.x * kWaves + threadIdx.x / RT_WAVE;
     if (o >= nout) return;
     const uint32_t lane = threadIdx.x & (RT_WAVE - 1);
     S a;
     a.init();
-    for (uint32_t k = lane; k < splits; k += RT_WAVE) a.merge(part[o * splits + k]);
+    for (uint32_t k = lane; k < splits; k += RT_WAVE) a.merge(part[o * ostride + (uint64_t)k * kstride]);
     group_reduce(a, RT_WAVE, lane);
     if (lane == 0) out[o] = a.result(flags);
 }
-// part[k * nout + o], one lane per output
+// many outputs, few partials each (column layout): one lane per output, coalesced over the outputs
 template <class S>
-__global__ __launch_bounds__(kBlock) void st_merge_cols_kernel(const S* __restrict__ part, typename S::Out* __restrict__ out, uint64_t nout, uint32_t splits, int flags) {
+__global__ __launch_bounds__(kBlock) void st_merge_lane_kernel(const S* __restrict__ part, typename S::Out* __restrict__ out, uint64_t nout, uint32_t splits, int flags) {
     const uint64_t o = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
     if (o >= nout) return;
     S a = part[o];
-    for (uint32_t k = 1; k < splits; ++k) a.merge(part[(uint64_t)k * nout + o]);
+    uint32_t k = 1;
+    for (; k + 4 <= splits; k += 4) {                           // four loads in flight
+        S p[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) p[u] = part[(uint64_t)(k + u) * nout + o];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) a.merge(p[u]);
+    }
+    for (; k < splits; ++k) a.merge(part[(uint64_t)k * nout + o]);
     out[o] = a.result(flags);
 }
 
@@ -464,10 +512,24 @@ __global__ __launch_bounds__(kBlock) void st_empty_kernel(typename S::Out* __res
 // ---- host planning ------------------------------------------------------------------------------------------------------
 static int32_t too_many() { return rt_fail(RT_E_INVALID, "reduce: too many outputs for one launch"); }
 
+template <class S>
+int32_t merge_cols(rt_ctx* ctx, const S* part, typename S::Out* out, uint64_t nout, uint32_t splits, int flags) {
+    if (splits >= 8 && nout <= 16384) {
+        hipLaunchKernelGGL((st_merge_wave_kernel<S>), dim3((unsigned)((nout + kWaves - 1) / kWaves)), dim3(kBlock), 0, ctx->stream, part, out, nout, splits,
+                           (uint64_t)1, nout, flags);
+    } else {
+        const uint64_t mb = (nout + kBlock - 1) / kBlock;
+        if (mb >= (1ull << 31)) return too_many();
+        hipLaunchKernelGGL((st_merge_lane_kernel<S>), dim3((unsigned)mb), dim3(kBlock), 0, ctx->stream, part, out, nout, splits, flags);
+    }
+    RT_HIP(hipGetLastError());
+    return RT_OK;
+}
+
 template <class S, class T>
 int32_t rows_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t rows, uint64_t R, int flags) {
     hipStream_t s = ctx->stream;
-    if (R <= kTileMaxR) {
+    if (R <= kTileMaxR) {                                          // measured against a wave per row: R = 256 0.22 / 0.56 ms, R = 1000 0.28 / 0.33 ms
         TileArgs a;
         a.rows = rows;
         a.R = (uint32_t)R;
@@ -514,7 +576,8 @@ int32_t rows_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t rows
     S* part = (S*)scratch;
     hipLaunchKernelGGL((st_rows_block_kernel<S, T>), dim3((unsigned)(rows * splits)), dim3(kBlock), 0, s, src, out, part, R, splits, seglen, flags);
     RT_HIP(hipGetLastError());
-    hipLaunchKernelGGL((st_merge_rows_kernel<S>), dim3((unsigned)((rows + kWaves - 1) / kWaves)), dim3(kBlock), 0, s, part, out, rows, splits, flags);
+    hipLaunchKernelGGL((st_merge_wave_kernel<S>), dim3((unsigned)((rows + kWaves - 1) / kWaves)), dim3(kBlock), 0, s, part, out, rows, splits,
+                       (uint64_t)splits, (uint64_t)1, flags);
     RT_HIP(hipGetLastError());
     return RT_OK;
 }
@@ -524,7 +587,7 @@ int32_t cols_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t oute
     hipStream_t s = ctx->stream;
     const uint64_t per_tile = (uint64_t)RT_WAVE * VW;
     const uint64_t tiles = (inner + per_tile - 1) / per_tile;
-    const uint64_t want = (uint64_t)ctx->num_cus * 2;           // two blocks per CU, as for the plain column reductions
+    const uint64_t want = (uint64_t)ctx->num_cus * S::kColsBlocksPerCU;       // resident blocks per CU (2 measured best for the cheap states)
     uint32_t splits = 1;
     if (outer * tiles < want) {
         const uint64_t min_seg = 64;
@@ -549,32 +612,35 @@ int32_t cols_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t oute
     hipLaunchKernelGGL((st_cols_kernel<S, T, VW>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, out, part, R, inner, outer, (uint32_t)tiles, splits, seglen,
                        flags);
     RT_HIP(hipGetLastError());
-    if (splits > 1) {
-        const uint64_t nout = outer * inner;
-        const uint64_t mb = (nout + kBlock - 1) / kBlock;
-        if (mb >= (1ull << 31)) return too_many();
-        hipLaunchKernelGGL((st_merge_cols_kernel<S>), dim3((unsigned)mb), dim3(kBlock), 0, s, part, out, nout, splits, flags);
-        RT_HIP(hipGetLastError());
-    }
+    if (splits > 1) RT_TRY(merge_cols<S>(ctx, part, out, outer * inner, splits, flags));
     return RT_OK;
 }
 
 template <class S, class T>
 int32_t narrow_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t outer, uint64_t R, uint64_t inner, int flags) {
+    constexpr uint32_t N = 16 / sizeof(T);
+    // vector loads for 4- and 8-byte elements (more lanes' worth of states would not fit in LDS)
+    const bool vec = sizeof(T) >= 4 && (reinterpret_cast<uintptr_t>(src) & 15) == 0 && (outer == 1 || (R * inner) % N == 0);
+    const uint32_t vw = vec ? N : 1;
+    uint32_t g = (uint32_t)inner, h = vw;                      // gcd(inner, vw)
+    while (h) { uint32_t r = g % h; g = h; h = r; }
+    const uint32_t innerp = (uint32_t)inner / g;               // lanes per period: Tn * vw must be a multiple of inner
     NarrowArgs a;
     a.R = R;
     a.outer = outer;
     a.inner = (uint32_t)inner;
-    a.Tn = (uint32_t)kBlock / a.inner * a.inner;
-    a.L = a.Tn / a.inner;
-    const uint64_t trips = (R + a.L - 1) / a.L;
+    a.Tn = (uint32_t)kBlock / innerp * innerp;
+    a.L = a.Tn * vw / (uint32_t)inner;
+    a.inner_div = make_fastdiv((uint32_t)inner);
+    a.G = 1;
+    while (a.G < 64 && (uint64_t)a.G * 2 * inner <= (uint64_t)kBlock && a.G * 2 <= a.L) a.G <<= 1;
+    const uint64_t ntiles = (R + a.L - 1) / a.L;
     const uint64_t want = (uint64_t)ctx->num_cus * 4;
     uint64_t splits = outer >= want ? 1 : (want + outer - 1) / outer;
-    if (splits > trips / 16) splits = trips / 16;               // at least 16 trips per block
+    if (splits > ntiles / 8) splits = ntiles / 8;              // at least 8 tiles per block
     if (splits < 1) splits = 1;
-    const uint64_t seg_trips = (trips + splits - 1) / splits;
-    splits = (trips + seg_trips - 1) / seg_trips;
-    a.seg_rows = seg_trips * a.L;
+    a.seg_tiles = (ntiles + splits - 1) / splits;
+    splits = (ntiles + a.seg_tiles - 1) / a.seg_tiles;
     a.splits = (uint32_t)splits;
     const uint64_t blocks = outer * splits;
     if (blocks >= (1ull << 31)) return too_many();
@@ -584,14 +650,10 @@ int32_t narrow_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t ou
         RT_TRY(rt_scratch(ctx, (size_t)(splits * outer * inner) * sizeof(S), &scratch));
         part = (S*)scratch;
     }
-    hipLaunchKernelGGL((st_cols_narrow_kernel<S, T>), dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream, src, out, part, a, flags);
+    if (vec) hipLaunchKernelGGL((st_cols_narrow_kernel<S, T, (sizeof(T) >= 4 ? (int)N : 1)>), dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream, src, out, part, a, flags);
+    else hipLaunchKernelGGL((st_cols_narrow_kernel<S, T, 1>), dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream, src, out, part, a, flags);
     RT_HIP(hipGetLastError());
-    if (splits > 1) {
-        const uint64_t nout = outer * inner;
-        hipLaunchKernelGGL((st_merge_cols_kernel<S>), dim3((unsigned)((nout + kBlock - 1) / kBlock)), dim3(kBlock), 0, ctx->stream, part, out, nout,
-                           (uint32_t)splits, flags);
-        RT_HIP(hipGetLastError());
-    }
+    if (splits > 1) RT_TRY(merge_cols<S>(ctx, part, out, outer * inner, (uint32_t)splits, flags));
     return RT_OK;
 }
 
@@ -609,8 +671,10 @@ int32_t plan(rt_ctx* ctx, const void* src_v, void* out_v, uint64_t outer, uint64
         return RT_OK;
     }
     if (inner == 1) return rows_plan<S, T>(ctx, src, out, outer, R, flags);
-    if (inner < 64 && R >= 64 && outer < (1ull << 20)) return narrow_plan<S, T>(ctx, src, out, outer, R, inner, flags);
     constexpr int N = 16 / sizeof(T);
+    // fewer columns than the vectors of one wave cover: stream the slab instead of leaving lanes idle
+    if (inner < (uint64_t)RT_WAVE * (sizeof(T) >= 4 ? N : 1) && inner <= (uint64_t)kBlock && R * inner >= 1024 && outer * inner < (1ull << 31))
+        return narrow_plan<S, T>(ctx, src, out, outer, R, inner, flags);
     const bool vec = (inner % N == 0) && ((reinterpret_cast<uintptr_t>(src) & 15) == 0);
     if (vec) return cols_plan<S, T, N>(ctx, src, out, outer, R, inner, flags);
     return cols_plan<S, T, 1>(ctx, src, out, outer, R, inner, flags);

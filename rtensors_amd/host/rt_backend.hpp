@@ -74,8 +74,16 @@ inline void check(int32_t st) {
 
 // ops/base.rs:7-12, ops/reduction/mod.rs:141-175
 enum class BinaryOpType : int { Add = RT_ADD, Sub = RT_SUB, Mul = RT_MUL, Div = RT_DIV };
-enum class ReductionOpTypes : int { Sum = RT_R_SUM, Prod = RT_R_PROD, Max = RT_R_MAX, Min = RT_R_MIN, Mean = RT_R_MEAN,
-                                    Variance = 6, LogSumExp = 7, Norm = 8, ArgMax = 9, ArgMin = 10 };
+// ReductionOpTypes (ops/reduction/mod.rs:141-175).  The variants that carry a payload there -- Variance { unbiased },
+// Stdev { unbiased }, Norm(L1 | L2) -- are spelled out, with the payload in the flag bits the C ABI takes.
+enum class ReductionOpTypes : int {
+    Sum = RT_R_SUM, Prod = RT_R_PROD, Max = RT_R_MAX, Min = RT_R_MIN, Mean = RT_R_MEAN,
+    PopVariance = RT_R_VARIANCE, Variance = RT_R_VARIANCE | RT_R_FLAG_UNBIASED,
+    PopStdev = RT_R_VARIANCE | RT_R_FLAG_STD, Stdev = RT_R_VARIANCE | RT_R_FLAG_STD | RT_R_FLAG_UNBIASED,
+    LogSumExp = RT_R_LOGSUMEXP, NormL1 = RT_R_NORM | RT_R_FLAG_L1, NormL2 = RT_R_NORM | RT_R_FLAG_L2,
+    ArgMax = RT_R_ARGMAX, ArgMin = RT_R_ARGMIN
+};
+enum class NormType { L1, L2 };                                   // ops/reduction/mod.rs:203-206
 
 class Hip;
 
@@ -221,11 +229,23 @@ class Hip {
         if (sm.rank() == 1) apply_reduce_contiguous_flat(src, dst, sm.offset, sm.size(), op);
         else apply_reduce_contiguous_nd(src, sm, dst, dim, op);
     }
-    // argmax / conv2d sit behind the same trait but outside this path; they report an error instead of the
-    // Cpu backend's todo!() panic (backend/cpu.rs:452-481).
-    void apply_argmax(const HipBuf&, const MetaTensor&, HipBuf&, size_t, ReductionOpTypes) const {
-        throw TensorError(ErrorKind::UnsupportedOperation, "argmax/argmin are not implemented by the Hip backend");
+    // Backend::apply_argmax_contiguous_flat / _nd / apply_argmax (backend/mod.rs:412-463): dst is a u64 buffer
+    void apply_argmax_contiguous_flat(const HipBuf& src, HipBuf& dst, uint64_t start, uint64_t len, ReductionOpTypes op) const {
+        if (dst.dtype() != RT_U64) throw TensorError(ErrorKind::UnsupportedOperation, "argmax writes u64 indices");
+        check(rt_argmax_flat(raw(), src.dtype(), (int)op, src.ptr(), src.len(), (uint64_t*)dst.ptr(), dst.len(), start, len));
     }
+    void apply_argmax_contiguous_nd(const HipBuf& src, const MetaTensor& sm, HipBuf& dst, size_t dim, ReductionOpTypes op) const {
+        if (dst.dtype() != RT_U64) throw TensorError(ErrorKind::UnsupportedOperation, "argmax writes u64 indices");
+        check(rt_argmax_nd(raw(), src.dtype(), (int)op, src.ptr(), src.len(), sm.offset, (int32_t)sm.rank(), sm.shape.data(), sm.strides.data(),
+                           (uint64_t*)dst.ptr(), dst.len(), (int32_t)dim));
+    }
+    void apply_argmax(const HipBuf& src, const MetaTensor& sm, HipBuf& dst, size_t dim, ReductionOpTypes op) const {
+        if (!sm.is_contiguous()) throw TensorError(ErrorKind::WrongDims, "Reduction over non-contiguous tensors is not implemented yet.");
+        if (sm.rank() == 1) apply_argmax_contiguous_flat(src, dst, sm.offset, sm.size(), op);
+        else apply_argmax_contiguous_nd(src, sm, dst, dim, op);
+    }
+    // conv2d sits behind the same trait but outside this path; it reports an error instead of the Cpu backend's todo!() panic
+    // (backend/cpu.rs:473-481).
     void apply_conv_2d() const { throw TensorError(ErrorKind::UnsupportedOperation, "conv2d is not implemented by the Hip backend"); }
 
     // ---- BackendMatMul::matmul (backend/mod.rs:474-485) ---------------------------------------------------------------------

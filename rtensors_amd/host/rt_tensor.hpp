@@ -232,8 +232,7 @@ class Tensor {
     // row-major run: a reversed view is |stride|-contiguous for the reference and would reach its kernels with the
     // offset of the last element; it is gathered instead.
     Tensor reduce(ReductionOpTypes op, std::optional<size_t> axis) const {
-        if ((int)op > (int)ReductionOpTypes::Mean)
-            throw TensorError(ErrorKind::UnsupportedOperation, "this reduction is not implemented by the Hip backend");
+        if (op == ReductionOpTypes::ArgMax || op == ReductionOpTypes::ArgMin) return arg_reduce(op, axis);
         if (!meta_.is_forward_contiguous()) return gathered().reduce(op, axis);
         if (!axis) {                                                           // Idx::Item (ops/reduction/mod.rs:272-285)
             Tensor out(*backend_, backend_->alloc_uninit(dtype(), 1), MetaTensor({}, {}, 0));
@@ -256,6 +255,41 @@ class Tensor {
     Tensor max() const { return reduce(ReductionOpTypes::Max, std::nullopt); }
     Tensor min() const { return reduce(ReductionOpTypes::Min, std::nullopt); }
     Tensor mean() const { return reduce(ReductionOpTypes::Mean, std::nullopt); }
+    // the kinds only the reference's Cuda backend implements (ops/reduction/mod.rs:411-500)
+    Tensor var_at(size_t a) const { return reduce(ReductionOpTypes::Variance, a); }
+    Tensor pop_var_at(size_t a) const { return reduce(ReductionOpTypes::PopVariance, a); }
+    Tensor std_at(size_t a, bool unbiased) const { return reduce(unbiased ? ReductionOpTypes::Stdev : ReductionOpTypes::PopStdev, a); }
+    Tensor norm_at(size_t a, NormType n) const { return reduce(n == NormType::L1 ? ReductionOpTypes::NormL1 : ReductionOpTypes::NormL2, a); }
+    Tensor l1_norm_at(size_t a) const { return norm_at(a, NormType::L1); }
+    Tensor l2_norm_at(size_t a) const { return norm_at(a, NormType::L2); }
+    Tensor logsumexp_at(size_t a) const { return reduce(ReductionOpTypes::LogSumExp, a); }
+    Tensor argmax_at(size_t a) const { return arg_reduce(ReductionOpTypes::ArgMax, a); }
+    Tensor argmin_at(size_t a) const { return arg_reduce(ReductionOpTypes::ArgMin, a); }
+    Tensor var() const { return reduce(ReductionOpTypes::Variance, std::nullopt); }
+    Tensor pop_var() const { return reduce(ReductionOpTypes::PopVariance, std::nullopt); }
+    Tensor std(bool unbiased) const { return reduce(unbiased ? ReductionOpTypes::Stdev : ReductionOpTypes::PopStdev, std::nullopt); }
+    Tensor norm(NormType n) const { return reduce(n == NormType::L1 ? ReductionOpTypes::NormL1 : ReductionOpTypes::NormL2, std::nullopt); }
+    Tensor l1_norm() const { return norm(NormType::L1); }
+    Tensor l2_norm() const { return norm(NormType::L2); }
+    Tensor logsumexp() const { return reduce(ReductionOpTypes::LogSumExp, std::nullopt); }
+    Tensor argmax() const { return arg_reduce(ReductionOpTypes::ArgMax, std::nullopt); }
+    Tensor argmin() const { return arg_reduce(ReductionOpTypes::ArgMin, std::nullopt); }
+    // do_argmax (ops/reduction/mod.rs:305-342): a u64 tensor of positions, rank-0 for the total form
+    Tensor arg_reduce(ReductionOpTypes op, std::optional<size_t> axis) const {
+        if (op != ReductionOpTypes::ArgMax && op != ReductionOpTypes::ArgMin)
+            throw TensorError(ErrorKind::UnsupportedOperation, "arg_reduce takes ArgMax or ArgMin");
+        if (!meta_.is_forward_contiguous()) return gathered().arg_reduce(op, axis);
+        if (!axis) {
+            Tensor out(*backend_, backend_->alloc_uninit(RT_U64, 1), MetaTensor({}, {}, 0));
+            backend_->apply_argmax_contiguous_flat(*buf_, *out.buf_, meta_.offset, meta_.size(), op);
+            return out;
+        }
+        if (*axis >= rank()) throw TensorError(ErrorKind::InvalidDim, "reduction axis out of range");
+        MetaTensor om = reduction_output_meta(meta_, axis);
+        Tensor out(*backend_, backend_->alloc_uninit(RT_U64, om.size()), om);
+        backend_->apply_argmax(*buf_, meta_, *out.buf_, *axis, op);
+        return out;
+    }
 
     // PartialEq of tensors: same shape and the same addressed values
     bool equals(const Tensor& o) const {

@@ -234,6 +234,23 @@ class Tensor:
     def mean(self): return self.reduce("mean")
     def max(self): return self.reduce("max")
     def min(self): return self.reduce("min")
+    # the kinds only the reference's Cuda backend implements (ops/reduction/mod.rs:411-500); argmax / argmin give u64 tensors
+    def var_at(self, a): return self.reduce("var", a)
+    def pop_var_at(self, a): return self.reduce("pop_var", a)
+    def std_at(self, a, unbiased): return self.reduce("std" if unbiased else "pop_std", a)
+    def norm_at(self, a, norm): return self.reduce({"L1": "l1_norm", "L2": "l2_norm"}[norm], a)
+    def l1_norm_at(self, a): return self.reduce("l1_norm", a)
+    def l2_norm_at(self, a): return self.reduce("l2_norm", a)
+    def logsumexp_at(self, a): return self.reduce("logsumexp", a)
+    def argmax_at(self, a): return self.reduce("argmax", a)
+    def argmin_at(self, a): return self.reduce("argmin", a)
+    def var(self): return self.reduce("var")
+    def pop_var(self): return self.reduce("pop_var")
+    def std(self, unbiased): return self.reduce("std" if unbiased else "pop_std")
+    def norm(self, norm): return self.reduce({"L1": "l1_norm", "L2": "l2_norm"}[norm])
+    def logsumexp(self): return self.reduce("logsumexp")
+    def argmax(self): return self.reduce("argmax")
+    def argmin(self): return self.reduce("argmin")
 
     def fill(self, v): _ck(_h.rth_fill(self._p, C.c_double(v)))
 

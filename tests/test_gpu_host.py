@@ -101,11 +101,49 @@ def test_reduce_of_noncontiguous_and_reversed_views(T, be):
     assert np.array_equal(rv.sum_at(2).to_numpy().reshape(2, 3), x.reshape(2, 3, 4)[::-1].sum(axis=2))
 
 
+def test_statistic_and_index_reductions_through_host_layer(T, be):
+    """var / pop_var / std / norm / logsumexp / argmax / argmin (ops/reduction/mod.rs:411-500): shapes of the outputs (kept dim, rank-0
+    totals, u64 for the index kinds), views gathered first, and the reference's Cuda known answers."""
+    import json, os
+    cases = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_reduce_stat_vectors.json")))["cases"]
+    for c in cases:
+        x = np.array(c["data"], dtype=cpu.NP_DTYPE[cpu.DTYPE_BY_NAME[c["dtype"]]])
+        g, o = T.Tensor.from_buf(be, c["dtype"], x, c["shape"]), OTensor.from_buf(c["dtype"], x, c["shape"])
+        got, want = g.reduce(c["op"], c["dim"]), o.reduce(c["op"], c["dim"])
+        assert list(got.shape) == list(want.meta.shape) == ([] if c["dim"] is None else [1, 2])
+        if c["op"] in cpu.ARG_OPS:
+            assert got.dtype == cpu.U64 and got.to_numpy().reshape(-1).tolist() == c["want"]
+        else:
+            assert np.allclose(got.to_numpy().reshape(-1).astype(np.float64), c["want"], rtol=1e-6 if c["dtype"] == "f32" else 1e-14, atol=0)
+    rng = np.random.default_rng(9)
+    x = (rng.normal(size=(6, 5, 7)) * 2 + 4)
+    g, o = T.Tensor.from_buf(be, "f64", x.reshape(-1), [6, 5, 7]), OTensor.from_buf("f64", x.reshape(-1), [6, 5, 7])
+    gv, ov = g.permute([2, 0, 1]).slice(1, T.Slice(None, None, -2)), o.permute([2, 0, 1]).slice(1, OSlice(None, None, -2))
+    for axis in (0, 1, 2):
+        for name, args in (("var_at", ()), ("pop_var_at", ()), ("std_at", (True,)), ("std_at", (False,)), ("norm_at", ("L1",)), ("norm_at", ("L2",)),
+                           ("logsumexp_at", ())):
+            got, want = getattr(gv, name)(axis, *args), getattr(ov, name)(axis, *args)
+            assert list(got.shape) == list(want.meta.shape)
+            assert np.allclose(got.to_numpy(), want.to_numpy(), rtol=1e-12, atol=0), (name, axis)
+        for name in ("argmax_at", "argmin_at"):
+            got, want = getattr(gv, name)(axis), getattr(ov, name)(axis)
+            assert np.array_equal(got.to_numpy(), want.to_numpy()), (name, axis)
+    assert np.isclose(gv.var().to_numpy(), ov.var().to_numpy(), rtol=1e-12) and np.isclose(gv.std(False).to_numpy(), ov.std(False).to_numpy(), rtol=1e-12)
+    assert np.isclose(gv.logsumexp().to_numpy(), ov.logsumexp().to_numpy(), rtol=1e-12) and np.isclose(gv.norm("L2").to_numpy(), ov.norm("L2").to_numpy(), rtol=1e-12)
+    assert int(gv.argmax().to_numpy()) == int(ov.argmax().to_numpy()) and int(gv.argmin().to_numpy()) == int(ov.argmin().to_numpy())
+    # closed form on the viewed values
+    xv = x.transpose(2, 0, 1)[:, ::-2]
+    assert np.allclose(gv.var_at(2).to_numpy().reshape(xv.shape[0], xv.shape[1]), xv.var(axis=2, ddof=1), rtol=1e-12)
+    assert np.array_equal(gv.argmax_at(1).to_numpy().reshape(xv.shape[0], xv.shape[2]), xv.argmax(axis=1))
+
+
 def test_out_of_scope_methods_report_unsupported(T, be):
-    g = T.Tensor.from_buf(be, "f32", np.ones(4, np.float32), [4])
+    g = T.Tensor.from_buf(be, "i32", np.ones(4, np.int32), [4])
     with pytest.raises(T.TensorError) as e:
-        g._new(T._h.rth_reduce, 6, T.C.c_int64(-1))           # variance
+        g.var()                                               # WeightValue kinds on an integer tensor
     assert e.value.kind == "UnsupportedOperation"
+    with pytest.raises(T.TensorError):
+        g._new(T._h.rth_reduce, 11, T.C.c_int64(-1))          # not a reduction op code
 
 
 # ---- autograd step (config 5 at reduced size) ---------------------------------------------------------------------------------

@@ -2,6 +2,7 @@
 seeded inputs.  Bit-exact for integers, for f32/f64 elementwise results, and for max/min; float sum/prod/mean within
 rel 1e-5 (f32) / 1e-12 (f64) of sum|x|; transcendental unaries within the reference's own 1e-5."""
 import os
+import zlib
 import numpy as np
 import pytest
 
@@ -419,7 +420,7 @@ def test_reference_vectors_on_gpu(hip, case):
 @pytest.mark.parametrize("dtype", ALL_DTYPES)
 @pytest.mark.parametrize("op", ["add", "sub", "mul", "div"])
 def test_broadcast_random_vs_oracle(hip, dtype, op):
-    rng = np.random.default_rng(abs(hash((dtype, op))) % 2 ** 31)
+    rng = np.random.default_rng(zlib.crc32((dtype + op).encode()))
     if dtype == "bool" and op == "div":
         pytest.skip("boolean division is todo!() in the reference")
     for trial in range(25):
@@ -482,7 +483,7 @@ def _tol(dtype, x):
 @pytest.mark.parametrize("dtype", ["f32", "f64", "i32", "i64", "u8", "i16", "u32"])
 @pytest.mark.parametrize("op", ["sum", "prod", "max", "min", "mean"])
 def test_reduce_random_vs_oracle(hip, dtype, op):
-    rng = np.random.default_rng(abs(hash((dtype, op))) % 2 ** 31)
+    rng = np.random.default_rng(zlib.crc32((dtype + op).encode()))
     shapes = [[1], [7], [63], [64], [1000], [70001], [4, 5], [3, 4, 5], [2, 3, 4, 5], [1, 6], [6, 1], [257, 3], [3, 257], [2, 4100],
               [4100, 2], [5, 64, 7], [300, 260], [17, 1024], [2, 1, 3], [33, 40000], [40000, 33], [3, 2048, 8]]
     for shape in shapes:
@@ -666,7 +667,7 @@ def test_convert(hip):
 def test_broadcast_with_transposed_operand(hip, dtype):
     """One input is a permuted (and possibly reversed / strided) view whose unit-stride dim is not the output's inner dim:
     the LDS-transpose tile kernel.  Ragged tile edges, both operand positions, broadcast and in-place forms."""
-    rng = np.random.default_rng(abs(hash(dtype)) % 2 ** 31)
+    rng = np.random.default_rng(zlib.crc32(dtype.encode()))
     shapes = [(3, 40, 70), (2, 5, 33, 130), (64, 257), (1, 100, 36), (4, 17, 1030), (2, 3, 16, 16)]
     for shape in shapes:
         r = len(shape)
@@ -865,7 +866,7 @@ def test_reduction_shapes_short_rows_narrow_columns_short_axis(hip, dtype):
     """The shapes that have kernels of their own: rows of 1..1025 elements (LDS-tiled), narrow inner dims (streamed with the
     lanes pinned to columns), reduced axes of at most 32 elements (a lane per output); odd counts, unaligned offsets, and the
     hand-over points to the general kernels."""
-    rng = np.random.default_rng(abs(hash(dtype)) % 2 ** 31)
+    rng = np.random.default_rng(zlib.crc32(dtype.encode()))
     for R in (1, 2, 3, 7, 8, 31, 32, 33, 63, 64, 65, 100, 255, 256, 1000, 1023, 1024, 1025):
         for rows in (1, 77, 1000):
             _check_reduce(hip, dtype, rows, R, 1, rng, offset=int(rng.integers(0, 5)))
@@ -897,7 +898,15 @@ def _check_stat(hip, dtype, outer, R, inner, rng, offset=0):
         got = hip.dump(dst).astype(np.float64)
         assert (np.isnan(got) == np.isnan(want)).all(), (dtype, op, outer, R, inner)
         fin = np.isfinite(want)
-        assert (np.abs(got - want)[fin] <= rel * np.abs(want)[fin] + 1e-300).all(), (dtype, op, outer, R, inner, offset, got[:4], want[:4])
+        tol = rel * np.abs(want)
+        if op in ("var", "pop_var", "std", "pop_std"):
+            # a variance is conditioned by kappa = sqrt(1 + mean^2 / var): two samples 1e-3 apart around 10 lose four digits in any
+            # arithmetic, the oracle's included
+            xs = x64[offset:offset + n].reshape(outer, R, inner)
+            with np.errstate(all="ignore"):
+                kappa = np.sqrt(1 + xs.mean(axis=1) ** 2 / xs.var(axis=1)).reshape(-1)
+            tol = tol * np.where(np.isfinite(kappa), kappa, 1.0)
+        assert (np.abs(got - want)[fin] <= tol[fin] + 1e-300).all(), (dtype, op, outer, R, inner, offset, got[:4], want[:4])
 
 
 def _check_arg(hip, dtype, outer, R, inner, rng, offset=0):
@@ -930,14 +939,14 @@ STAT_SHAPES = ([(rows, R, 1) for R in (1, 2, 3, 7, 8, 31, 32, 33, 64, 65, 100, 2
 
 @pytest.mark.parametrize("dtype", ["f32", "f64"])
 def test_statistic_reductions_shapes(hip, dtype):
-    rng = np.random.default_rng(abs(hash(dtype)) % 2 ** 31)
+    rng = np.random.default_rng(zlib.crc32(dtype.encode()))
     for outer, R, inner in STAT_SHAPES:
         _check_stat(hip, dtype, outer, R, inner, rng, offset=int(rng.integers(0, 5)))
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f64", "i32", "u8", "i64", "i16"])
 def test_argmax_argmin_shapes(hip, dtype):
-    rng = np.random.default_rng(abs(hash(dtype)) % 2 ** 31)
+    rng = np.random.default_rng(zlib.crc32(dtype.encode()))
     for outer, R, inner in STAT_SHAPES:
         _check_arg(hip, dtype, outer, R, inner, rng, offset=int(rng.integers(0, 5)))
 
@@ -1090,7 +1099,7 @@ def test_matmul_integers_bit_exact(hip, dtype):
     """The tiled kernel against the Cpu backend's triple loop (backend/cpu.rs:857-939): wrapping sums, every pairing of
     row-/column-major operands (the reference itself has mixed pairings for f32/f64 only), padded leading dims, offsets,
     batches, ragged tiles."""
-    seed = abs(hash(dtype)) % 2 ** 31
+    seed = zlib.crc32(dtype.encode())
     lo, hi = (-2 ** 31, 2 ** 31 - 1) if dtype in ("i64", "u32", "i32") else (-1000, 1000)      # products overflow and wrap
     for (b, m, k, n) in MM_SHAPES:
         for ll in range(4):
