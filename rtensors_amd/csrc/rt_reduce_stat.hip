@@ -42,23 +42,27 @@ __device__ __forceinline__ double m_max(double a, double b) { return fmax(a, b);
 // push(x, pos): one element at position `pos` of the reduced axis; push_block<K>(x, pos0, step): K elements at positions pos0,
 // pos0 + step, ...; merge(o): another partial state, any relative order; result(flags): the output value.
 
+// 1 / x for a weight: the hardware reciprocal (1 ulp) is enough for f32, where a correctly rounded division costs ~10 instructions
+__device__ __forceinline__ float m_recip(float x) { return __builtin_amdgcn_rcpf(x); }
+__device__ __forceinline__ double m_recip(double x) { return 1.0 / x; }
+
 template <class T> struct MomentState {
     typedef T Out;
     static constexpr int kColsBlocksPerCU = 2;
     T mean, m2;
-    uint64_t n;
-    __device__ __forceinline__ void init() { mean = (T)0; m2 = (T)0; n = 0; }
-    __device__ __forceinline__ void absorb(T omean, T om2, uint64_t on) {          // welford_combine, reduce.cu:191-213
-        if (on == 0) return;
-        if (n == 0) { mean = omean; m2 = om2; n = on; return; }
-        const uint64_t nn = n + on;
+    double n;                                                   // a count, exact up to 2^53; as a double it converts to T in one instruction
+    __device__ __forceinline__ void init() { mean = (T)0; m2 = (T)0; n = 0.0; }
+    // welford_combine, reduce.cu:191-213.  An empty receiver needs no special case: delta = omean, w = 1, n * w = 0.
+    __device__ __forceinline__ void absorb(T omean, T om2, double on) {
+        if (on == 0.0) return;
+        const double nn = n + on;
         const T delta = omean - mean;
-        const T w = (T)on / (T)nn;
+        const T w = (T)on * m_recip((T)nn);
         mean = mean + delta * w;
         m2 = m2 + om2 + (delta * delta) * ((T)n * w);
         n = nn;
     }
-    __device__ __forceinline__ void push(T x, uint64_t) { absorb(x, (T)0, 1); }
+    __device__ __forceinline__ void push(T x, uint64_t) { absorb(x, (T)0, 1.0); }
     template <int K> __device__ __forceinline__ void push_block(const T* x, uint64_t, uint64_t) {
         T s = (T)0;
 #pragma unroll
@@ -67,11 +71,11 @@ template <class T> struct MomentState {
         T q = (T)0;
 #pragma unroll
         for (int i = 0; i < K; ++i) { const T d = x[i] - bm; q = q + d * d; }
-        absorb(bm, q, K);
+        absorb(bm, q, (double)K);
     }
     __device__ __forceinline__ void merge(const MomentState& o) { absorb(o.mean, o.m2, o.n); }
     __device__ __forceinline__ T result(int flags) const {                          // finalize_var_kernel_ptr, reduce.cu:385-402
-        const T denom = (flags & RT_R_FLAG_UNBIASED) ? (T)n - (T)1 : (T)n;
+        const T denom = (flags & RT_R_FLAG_UNBIASED) ? (T)(n - 1.0) : (T)n;
         const T v = m2 / denom;
         return (flags & RT_R_FLAG_STD) ? m_sqrt(v) : v;
     }
@@ -82,8 +86,13 @@ template <class T> struct LseState {
     static constexpr int kColsBlocksPerCU = 4;                  // one exp per element: more waves per CU to hide it (0.215 -> 0.180 ms on 1 GiB)
     T m, s;
     __device__ __forceinline__ void init() { m = -std::numeric_limits<T>::infinity(); s = (T)0; }
-    // exp(x - top), with x == top giving 1 also when both are infinite
-    static __device__ __forceinline__ T term(T x, T top) { return x == top ? (T)1 : m_exp(x - top); }
+    // exp(x - top), with x == top giving 1 also when both are infinite.  The argument is never positive, so for f32 the hardware
+    // exponential (2^(x log2 e), a few ulp for the arguments near 0 that carry the sum) stays inside the 1e-5 of the result; the
+    // library routine costs about four times the instructions and made short-row logsumexp compute-bound.
+    static __device__ __forceinline__ T term(T x, T top) {
+        if constexpr (std::is_same<T, float>::value) return x == top ? 1.0f : __expf(x - top);
+        else return x == top ? (T)1 : m_exp(x - top);
+    }
     __device__ __forceinline__ void push(T x, uint64_t) {
         const T top = m_max(m, x);
         s = s * term(m, top) + term(x, top);
