@@ -363,7 +363,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_tile_kernel(const T* __res
 // lanes that share a column are combined through LDS at the end (ties by position, so the first extremum still wins).
 struct ColsNarrowArgs {
     uint64_t R, outer;
-    uint32_t inner, Tn, L, splits;      // columns, active lanes, rows per tile, segments per outer index
+    uint32_t inner, Tn, L, splits, G;   // columns, active lanes, rows per tile, segments per outer index, lanes per column in the final merge
     uint64_t seg_tiles;                 // tiles per segment
     FastDiv32 inner_div;
 };
@@ -424,18 +424,25 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_narrow_kernel(const T* __r
         if constexpr (kTrack) sp[t * VW + j] = acc[j].pos;
     }
     __syncthreads();
-    if (t < a.inner) {
-        Acc<OP, T> r;
-        r.v = sv[t];
-        r.pos = kTrack ? sp[t] : 0;
-        for (uint32_t q = 1; q < a.L; ++q) {
+    // column c is held by the L values c, c + inner, ...: G lanes per column (a power of two, inner * G <= kBlock) share them
+    const uint32_t c = t / a.G, j = t & (a.G - 1);
+    Acc<OP, T> r;
+    r.init();
+    if (c < a.inner) {
+        for (uint32_t q = j; q < a.L; q += a.G) {
             Acc<OP, T> x;
-            x.v = sv[t + q * a.inner];
-            x.pos = kTrack ? sp[t + q * a.inner] : 0;
+            x.v = sv[c + q * a.inner];
+            x.pos = kTrack ? sp[c + q * a.inner] : 0;
             r.merge(x);
         }
-        out[((uint64_t)seg * a.outer + o) * a.inner + t] = last ? finalize<OP, T>(r.v, count) : r.v;
     }
+    for (uint32_t d = a.G / 2; d >= 1; d >>= 1) {
+        Acc<OP, T> x;
+        x.v = shfl_down_t<T>(r.v, (int)d);
+        if constexpr (kTrack) x.pos = shfl_down_t<uint64_t>(r.pos, (int)d); else x.pos = 0;
+        if (j + d < a.G) r.merge(x);
+    }
+    if (c < a.inner && j == 0) out[((uint64_t)seg * a.outer + o) * a.inner + c] = last ? finalize<OP, T>(r.v, count) : r.v;
 }
 
 // ---- short reduced axis: R <= 32, any inner -----------------------------------------------------------------------------------
@@ -477,6 +484,28 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_short_kernel(const T* __re
 }
 
 constexpr uint64_t kRowsTileMaxR = 1024;
+
+// ---- second stage of a split column reduction with few outputs ----------------------------------------------------------------
+// part[k * nout + o], k < splits.  One wave per output with the lanes spread over k: a lane per output would walk its `splits`
+// partials in one chain of dependent loads (1 GiB sum over 3 columns: 0.209 -> 0.17 ms).
+template <int OP, class T>
+__global__ __launch_bounds__(kBlock) void reduce_merge_wave_kernel(const T* __restrict__ part, T* __restrict__ out, uint64_t nout, uint32_t splits, uint64_t count) {
+    const uint64_t o = (uint64_t)blockIdx.x * kWaves + threadIdx.x / RT_WAVE;
+    if (o >= nout) return;
+    const uint32_t lane = threadIdx.x & (RT_WAVE - 1);
+    Acc<OP, T> a;
+    a.init();
+    for (uint32_t k = lane; k < splits; k += RT_WAVE) a.push(part[(uint64_t)k * nout + o], k);       // partials arrive in segment order
+    wave_reduce<OP, T>(a);
+    if (lane == 0) out[o] = finalize<OP, T>(a.v, count);
+}
+template <int OP, class T>
+bool merge_few_outputs(rt_ctx* ctx, const T* part, T* out, uint64_t nout, uint32_t splits, uint64_t count) {
+    if (splits < 8 || nout > 16384) return false;
+    hipLaunchKernelGGL((reduce_merge_wave_kernel<OP, T>), dim3((unsigned)((nout + kWaves - 1) / kWaves)), dim3(kBlock), 0, ctx->stream, part, out, nout, splits,
+                       count);
+    return true;
+}
 
 // ---- host planning ------------------------------------------------------------------------------------------------------
 template <int OP, class T>
@@ -588,6 +617,7 @@ int32_t cols_launch(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t 
     RT_HIP(hipGetLastError());
     // second stage: partials are (splits, outer*inner): a column reduce with R = splits
     const uint64_t inner2 = outer * inner;
+    if (merge_few_outputs<OP, T>(ctx, part, out, inner2, splits, count)) { RT_HIP(hipGetLastError()); return RT_OK; }
     const uint64_t tiles2 = (inner2 + per_tile - 1) / per_tile;
     if (tiles2 >= (1ull << 31)) return rt_fail(RT_E_INVALID, "reduce: too many outputs for one launch");
     hipLaunchKernelGGL((reduce_cols_kernel<OP, T, VW>), dim3((unsigned)tiles2), dim3(kBlock), 0, s, part, out, (uint64_t)splits, inner2, (uint64_t)1,
@@ -611,6 +641,8 @@ int32_t cols_narrow(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t 
     a.Tn = (uint32_t)kBlock / innerp * innerp;
     a.L = a.Tn * vw / (uint32_t)inner;
     a.inner_div = make_fastdiv((uint32_t)inner);
+    a.G = 1;
+    while (a.G < 64 && (uint64_t)a.G * 2 * inner <= (uint64_t)kBlock && a.G * 2 <= a.L) a.G <<= 1;
     const uint64_t ntiles = (R + a.L - 1) / a.L;
     const uint64_t want = (uint64_t)ctx->num_cus * 4;
     uint64_t splits = outer >= want ? 1 : (want + outer - 1) / outer;
@@ -634,6 +666,7 @@ int32_t cols_narrow(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t 
     if (splits == 1) return RT_OK;
     // second stage: the partials are (splits, outer * inner); fold the segments in order (mean divides by the original count)
     const uint64_t inner2 = outer * inner;
+    if (merge_few_outputs<OP, T>(ctx, dst1, out, inner2, (uint32_t)splits, R)) { RT_HIP(hipGetLastError()); return RT_OK; }
     const uint64_t tiles2 = (inner2 + RT_WAVE - 1) / RT_WAVE;
     hipLaunchKernelGGL((reduce_cols_kernel<OP, T, 1>), dim3((unsigned)tiles2), dim3(kBlock), 0, ctx->stream, dst1, out, (uint64_t)splits, inner2, (uint64_t)1,
                        (uint32_t)tiles2, 1u, (uint64_t)splits, R, 1);
