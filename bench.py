@@ -350,7 +350,7 @@ class Workloads:
 HEADLINE = ["c3a_add", "c4_sum1"]
 DETAIL = ["copy", "fill", "c1_add", "c1_sum1", "c2_mul", "c2_add", "c2_relu", "c2_sub", "c2_f64_mul", "c2_f64_add", "c2_i32_mul", "c2_i32_add",
           "c3a_add", "c3b_add", "c4_sum1", "c4_mean1", "c4_max1", "c4_sum0", "c4_sum_all", "c4_i32_sum1", "c4_i32_max1", "c4_i32_min0",
-          "c5_bias_add", "c5_colsum", "view_relu", "tr_add", "tr_copy"]
+          "c4_var1", "c4_std0", "c4_lse1", "c4_argmax1", "c5_bias_add", "c5_colsum", "view_relu", "tr_add", "tr_copy"]
 KIND = {"copy": "elementwise", "fill": "elementwise"}
 
 

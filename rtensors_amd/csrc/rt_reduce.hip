@@ -165,10 +165,20 @@ __device__ __forceinline__ void fold_run(Acc<OP, T>& a, const T* __restrict__ p,
             for (uint32_t j = 0; j < N; ++j) a.push(v[u].e[j], vb + (i + (uint64_t)u * nthreads) * N + j);
         }
     }
-    for (; i < nvec; i += nthreads) {
-        Vec16<T> v = rt_ld16_nt(pv + i);
+    if (i < nvec) {
+        // the last 1 .. U-1 vectors of this lane, again all loads issued before the first is used: a wave takes as long as its
+        // slowest lane, and one load at a time here tripled the time of rows of 250 vectors
+        Vec16<T> v[U - 1];
 #pragma unroll
-        for (uint32_t j = 0; j < N; ++j) a.push(v.e[j], vb + i * N + j);
+        for (int u = 0; u < U - 1; ++u)
+            if (i + (uint64_t)u * nthreads < nvec) v[u] = rt_ld16_nt(pv + i + (uint64_t)u * nthreads);
+#pragma unroll
+        for (int u = 0; u < U - 1; ++u) {
+            if (i + (uint64_t)u * nthreads < nvec) {
+#pragma unroll
+                for (uint32_t j = 0; j < N; ++j) a.push(v[u].e[j], vb + (i + (uint64_t)u * nthreads) * N + j);
+            }
+        }
     }
     const uint64_t tb = vb + nvec * N;
     if (tb + tid < end) a.push(p[tb + tid], tb + tid);
@@ -512,7 +522,9 @@ template <int OP, class T>
 int32_t rows_stage(rt_ctx* ctx, const T* src, T* out, uint64_t rows, uint64_t R, uint64_t count, bool allow_split) {
     hipStream_t s = ctx->stream;
     if (rows == 0) return RT_OK;
-    if (R >= 1 && R <= kRowsTileMaxR && count == R) {          // short rows (not the second stage of a split reduction)
+    // short rows (not the second stage of a split reduction).  From 2 KiB per row a wave per row is faster (f32 sum, 1 GiB: rows of
+    // 512 elements 0.183 ms staged / 0.155 ms direct, 1024: 0.188 / 0.159; below that the staged form wins, 256: 0.185 / 0.222)
+    if (R >= 1 && R <= kRowsTileMaxR && R * sizeof(T) < 2048 && count == R) {
         RowsTileArgs a;
         a.rows = rows;
         a.R = (uint32_t)R;

@@ -218,9 +218,14 @@ __device__ __forceinline__ void fold_run(S& a, const T* __restrict__ p, uint64_t
             a.template push_block<U * N>(x, 0, 0);
         }
     }
-    for (; i < nvec; i += nthreads) {
-        Vec16<T> v = rt_ld16_nt(pv + i);
-        a.template push_block<N>(v.e, vb + i * N, 1);
+    if (i < nvec) {                                             // the last 1 .. U-1 vectors of this lane, loads first
+        Vec16<T> v[U - 1];
+#pragma unroll
+        for (int u = 0; u < U - 1; ++u)
+            if (i + (uint64_t)u * nthreads < nvec) v[u] = rt_ld16_nt(pv + i + (uint64_t)u * nthreads);
+#pragma unroll
+        for (int u = 0; u < U - 1; ++u)
+            if (i + (uint64_t)u * nthreads < nvec) a.template push_block<N>(v[u].e, vb + (i + (uint64_t)u * nthreads) * N, 1);
     }
     const uint64_t tb = vb + nvec * N;
     if (tb + tid < end) a.push(p[tb + tid], tb + tid);
@@ -538,7 +543,7 @@ int32_t merge_cols(rt_ctx* ctx, const S* part, typename S::Out* out, uint64_t no
 template <class S, class T>
 int32_t rows_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t rows, uint64_t R, int flags) {
     hipStream_t s = ctx->stream;
-    if (R <= kTileMaxR) {                                          // measured against a wave per row: R = 256 0.22 / 0.56 ms, R = 1000 0.28 / 0.33 ms
+    if (R <= kTileMaxR && R * sizeof(T) < 2048) {                // from 2 KiB per row a wave per row is faster (f32 rows of 1024: 0.194 / 0.157 ms)
         TileArgs a;
         a.rows = rows;
         a.R = (uint32_t)R;
