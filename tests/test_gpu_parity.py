@@ -825,6 +825,17 @@ def test_more_than_2_31_elements(hip):
     assert hip.dump(out)[0] == 7
     hip.apply_reduce_contiguous_flat(d, out, 0, n, "min")
     assert hip.dump(out)[0] == 7
+    # positions beyond 2^31 come back whole from the index reductions
+    p_max, p_min = (1 << 31) + 12345, (1 << 31) + 77
+    hip.write(d, p_max, 9); hip.write(d, p_max + 5, 9); hip.write(d, p_min, 2)
+    idx = hip.alloc(H.U64, rows)
+    hip.apply_argmax_contiguous_flat(d, idx, 0, n, "argmax")
+    assert int(hip.dump(idx)[0]) == p_max
+    hip.apply_argmax_contiguous_flat(d, idx, 0, n, "argmin")
+    assert int(hip.dump(idx)[0]) == p_min
+    hip.apply_argmax_contiguous_nd((d, (0, [rows, cols], [cols, 1])), idx, 1, "argmax")
+    got = hip.dump(idx)
+    assert int(got[p_max // cols]) == p_max % cols and int(got.sum()) == p_max % cols
     hip.sync()
 
 
