@@ -237,8 +237,15 @@ __global__ __launch_bounds__(kRBlock) void bin_flat_row_kernel(const T* __restri
     const uint32_t v = blockIdx.x * kRBlock + threadIdx.x;
     if (v >= nvec) return;
     Vec16<T> x = rt_ld16_nt(reinterpret_cast<const Vec16<T>*>(flat) + v);
-    const uint32_t c = v - fd_div(v, row_div) * row_vecs;
-    Vec16<T> y = rt_ld16(reinterpret_cast<const Vec16<T>*>(row) + c);
+    Vec16<T> y;
+    if (row_vecs == 0) {                                          // the "row" is a single element (tensor op one-element tensor)
+        const T e = row[0];
+#pragma unroll
+        for (int j = 0; j < (int)(16 / sizeof(T)); ++j) y.e[j] = e;
+    } else {
+        const uint32_t c = v - fd_div(v, row_div) * row_vecs;
+        y = rt_ld16(reinterpret_cast<const Vec16<T>*>(row) + c);
+    }
     if constexpr (ROW_IS_LEFT) { bin_apply_vec<OP, T>(y, x); rt_st16_nt(reinterpret_cast<Vec16<T>*>(d) + v, y); }
     else { bin_apply_vec<OP, T>(x, y); rt_st16_nt(reinterpret_cast<Vec16<T>*>(d) + v, x); }
 }
@@ -359,23 +366,27 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
     bool prefer_flat = rank >= 2 && ((uint64_t)dsc.shape[rank - 1] * sizeof(T)) % 128 != 0 && row_major_run(2);
     for (int o = 0; o < (OP == kOpCopy ? 1 : 2) && prefer_flat; ++o)
         prefer_flat = row_major_run(o) || dsc.stride[o][rank - 1] == 0;
-    // (2b) bias add: dst and one input are one aligned run, the other input is a single row repeated.  Measured against the row
+    // (2b) bias add / tensor op one-element tensor: dst and one input are one aligned run, the other input is a single row (or a
+    // single element) repeated.  Measured against the row
     // kernel on 1 GiB f32: rows of 256 B 0.347 -> 0.338 ms, 16 KiB 0.355 -> 0.335, 128 KiB 0.340 -> 0.328, in place 0.368 -> 0.333;
     // level at 4 MiB rows, slower (0.384 -> 0.455 ms) at 64 MiB, where the row no longer stays in cache between its uses.
     if constexpr (OP != kOpCopy) {
-        if (rank >= 2 && count < (1ull << 31) && (uint64_t)dsc.shape[rank - 1] * sizeof(T) <= (1u << 20) && row_major_run(2) && dsc.shape[rank - 1] % N == 0 && count % N == 0 &&
-            (reinterpret_cast<uintptr_t>(d + dsc.offset[2]) & 15) == 0) {
+        if (rank >= 1 && count < (1ull << 31) && row_major_run(2) && count % N == 0 && (reinterpret_cast<uintptr_t>(d + dsc.offset[2]) & 15) == 0) {
             for (int o = 0; o < 2; ++o) {
-                const int p = 1 - o;                                   // o: the streamed input, p: the row
-                bool is_row = dsc.stride[p][rank - 1] == 1;
+                const int p = 1 - o;                                   // o: the streamed input, p: the row (or the single element)
+                bool is_row = rank >= 2 && dsc.stride[p][rank - 1] == 1 && dsc.shape[rank - 1] % N == 0 &&
+                              (uint64_t)dsc.shape[rank - 1] * sizeof(T) <= (1u << 20);
+                bool is_scalar = true;
                 for (int k = 0; k < rank - 1; ++k) is_row = is_row && dsc.stride[p][k] == 0;
+                for (int k = 0; k < rank; ++k) is_scalar = is_scalar && dsc.stride[p][k] == 0;
                 const T* fo = (o == 0 ? l : r) + dsc.offset[o];
                 const T* ro = (p == 0 ? l : r) + dsc.offset[p];
-                if (!is_row || !row_major_run(o) || (reinterpret_cast<uintptr_t>(fo) & 15) || (reinterpret_cast<uintptr_t>(ro) & 15)) continue;
-                const uint32_t nvec = (uint32_t)(count / N), row_vecs = (uint32_t)(dsc.shape[rank - 1] / N);
+                if (!(is_row || is_scalar) || !row_major_run(o) || (reinterpret_cast<uintptr_t>(fo) & 15)) continue;
+                if (!is_scalar && (reinterpret_cast<uintptr_t>(ro) & 15)) continue;
+                const uint32_t nvec = (uint32_t)(count / N), row_vecs = is_scalar ? 0u : (uint32_t)(dsc.shape[rank - 1] / N);
                 dim3 grid((nvec + kRBlock - 1) / kRBlock), blk(kRBlock);
-                if (p == 0) hipLaunchKernelGGL((bin_flat_row_kernel<T, OP, true>), grid, blk, 0, s, fo, ro, d + dsc.offset[2], nvec, row_vecs, make_fastdiv(row_vecs));
-                else hipLaunchKernelGGL((bin_flat_row_kernel<T, OP, false>), grid, blk, 0, s, fo, ro, d + dsc.offset[2], nvec, row_vecs, make_fastdiv(row_vecs));
+                if (p == 0) hipLaunchKernelGGL((bin_flat_row_kernel<T, OP, true>), grid, blk, 0, s, fo, ro, d + dsc.offset[2], nvec, row_vecs, make_fastdiv(row_vecs ? row_vecs : 1u));
+                else hipLaunchKernelGGL((bin_flat_row_kernel<T, OP, false>), grid, blk, 0, s, fo, ro, d + dsc.offset[2], nvec, row_vecs, make_fastdiv(row_vecs ? row_vecs : 1u));
                 RT_HIP(hipGetLastError());
                 return RT_OK;
             }
