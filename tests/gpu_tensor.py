@@ -160,14 +160,18 @@ class GTensor:
 
     def reduce(self, op, axis=None):
         t = self if self.meta.is_contiguous() and all(s >= 0 for s in self.meta.strides) else self.contiguous()
+        arg = op in ("argmax", "argmin")                          # do_argmax (ops/reduction/mod.rs:305-342): u64 output
+        flat = self.backend.apply_argmax_contiguous_flat if arg else self.backend.apply_reduce_contiguous_flat
+        nd = self.backend.apply_argmax_contiguous_nd if arg else self.backend.apply_reduce_contiguous_nd
+        odt = H.U64 if arg else t.dtype
         if axis is None:
-            out = self.backend.alloc(t.dtype, 1)
-            self.backend.apply_reduce_contiguous_flat(t.buf, out, t.meta.offset, t.meta.size(), op)
+            out = self.backend.alloc(odt, 1)
+            flat(t.buf, out, t.meta.offset, t.meta.size(), op)
             return GTensor(self.backend, out, MetaTensor([], [], 0))
         om = reduction_output_meta(t.meta, axis)
-        out = self.backend.alloc(t.dtype, om.size())
+        out = self.backend.alloc(odt, om.size())
         if t.meta.rank() == 1:
-            self.backend.apply_reduce_contiguous_flat(t.buf, out, t.meta.offset, t.meta.size(), op)
+            flat(t.buf, out, t.meta.offset, t.meta.size(), op)
         else:
-            self.backend.apply_reduce_contiguous_nd((t.buf, _m(t.meta)), out, axis, op)
+            nd((t.buf, _m(t.meta)), out, axis, op)
         return GTensor(self.backend, out, om)
