@@ -366,6 +366,41 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_tile_kernel(const T* __res
     }
 }
 
+// ---- short rows whose length is a power-of-two number of 16-byte vectors (16 B .. 1 KiB per row, aligned) -----------------------------
+// No staging: the rows of a block are one contiguous run, lane t reads vector t of it (four such loads in flight), the VR lanes
+// that hold one row are neighbours inside a wave and fold with log2(VR) shuffles.
+template <int OP, class T>
+__global__ __launch_bounds__(kBlock) void reduce_rows_pow2_kernel(const T* __restrict__ src, T* __restrict__ out, uint64_t nvec, uint32_t VR, uint32_t vr_shift,
+                                                                  uint64_t count) {
+    constexpr uint32_t N = 16 / sizeof(T);
+    constexpr int U = 4;
+    const Vec16<T>* pv = reinterpret_cast<const Vec16<T>*>(src);
+    const uint64_t v0 = (uint64_t)blockIdx.x * (kBlock * U) + threadIdx.x;
+    Vec16<T> x[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+        if (v0 + (uint64_t)u * kBlock < nvec) x[u] = rt_ld16_nt(pv + v0 + (uint64_t)u * kBlock);
+    const uint32_t j = threadIdx.x & (VR - 1);                    // position of this lane's vector inside its row
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const uint64_t v = v0 + (uint64_t)u * kBlock;
+        Acc<OP, T> a;
+        a.init();
+        if (v < nvec) {
+#pragma unroll
+            for (uint32_t e = 0; e < N; ++e) a.push(x[u].e[e], (uint64_t)j * N + e);
+        }
+        for (uint32_t d = VR / 2; d >= 1; d >>= 1) {
+            Acc<OP, T> o;
+            o.v = shfl_down_t<T>(a.v, (int)d);
+            // positions inside a row fit 32 bits here (one shuffle instead of two); "none yet" stays the largest value
+            if constexpr (Acc<OP, T>::kTrack) o.pos = (uint64_t)(uint32_t)__shfl_down((int)(uint32_t)a.pos, (int)d, RT_WAVE); else o.pos = 0;
+            if (j + d < VR) a.merge(o);
+        }
+        if (j == 0 && v < nvec) out[v >> vr_shift] = finalize<OP, T>(a.v, count);
+    }
+}
+
 // ---- narrow columns: inner < 128, long R ------------------------------------------------------------------------------------
 // With lanes along `inner` only `inner` of 64 lanes would work.  Here the (R, inner) slab of one outer index is read as one
 // contiguous stream in tiles of S = Tn * VW elements, S a multiple of inner, so that lane t always meets the same VW columns
@@ -522,6 +557,26 @@ template <int OP, class T>
 int32_t rows_stage(rt_ctx* ctx, const T* src, T* out, uint64_t rows, uint64_t R, uint64_t count, bool allow_split) {
     hipStream_t s = ctx->stream;
     if (rows == 0) return RT_OK;
+    {
+        constexpr uint64_t N = 16 / sizeof(T);
+        const uint64_t vr = R / N;
+        // (small inputs stay with the staged kernel, where few rows mean one lane per row: a sum in index order, bit for bit the
+        // sequential result)
+        // float max / min carry a position through every shuffle step: with 8-byte values that only pays up to 16 lanes per row
+        const uint64_t vr_max = (Acc<OP, T>::kTrack && sizeof(T) == 8) ? 16 : 64;
+        if (count == R && R % N == 0 && vr >= 1 && vr <= vr_max && (vr & (vr - 1)) == 0 && rows * vr >= 4096 &&
+            (reinterpret_cast<uintptr_t>(src) & 15) == 0) {
+            const uint64_t nvec = rows * vr;
+            const uint64_t blocks = (nvec + (uint64_t)kBlock * 4 - 1) / ((uint64_t)kBlock * 4);
+            if (blocks < (1ull << 31)) {
+                uint32_t shift = 0;
+                while ((1ull << shift) < vr) ++shift;
+                hipLaunchKernelGGL((reduce_rows_pow2_kernel<OP, T>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, out, nvec, (uint32_t)vr, shift, count);
+                RT_HIP(hipGetLastError());
+                return RT_OK;
+            }
+        }
+    }
     // short rows (not the second stage of a split reduction).  From 2 KiB per row a wave per row is faster (f32 sum, 1 GiB: rows of
     // 512 elements 0.183 ms staged / 0.155 ms direct, 1024: 0.188 / 0.159; below that the staged form wins, 256: 0.185 / 0.222)
     if (R >= 1 && R <= kRowsTileMaxR && R * sizeof(T) < 2048 && count == R) {

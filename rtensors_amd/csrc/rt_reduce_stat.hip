@@ -329,6 +329,31 @@ __global__ __launch_bounds__(kBlock) void st_rows_tile_kernel(const T* __restric
     }
 }
 
+// rows of 1, 2 or 4 aligned 16-byte vectors: no staging, lane t reads vector t of the block's run (four loads in flight) and the
+// lanes of a row, neighbours inside a wave, merge with one or two shuffle steps
+template <class S, class T>
+__global__ __launch_bounds__(kBlock) void st_rows_pow2_kernel(const T* __restrict__ src, typename S::Out* __restrict__ out, uint64_t nvec, uint32_t VR,
+                                                              uint32_t vr_shift, int flags) {
+    constexpr uint32_t N = 16 / sizeof(T);
+    constexpr int U = 4;
+    const Vec16<T>* pv = reinterpret_cast<const Vec16<T>*>(src);
+    const uint64_t v0 = (uint64_t)blockIdx.x * (kBlock * U) + threadIdx.x;
+    Vec16<T> x[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+        if (v0 + (uint64_t)u * kBlock < nvec) x[u] = rt_ld16_nt(pv + v0 + (uint64_t)u * kBlock);
+    const uint32_t j = threadIdx.x & (VR - 1);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const uint64_t v = v0 + (uint64_t)u * kBlock;
+        S a;
+        a.init();
+        if (v < nvec) a.template push_block<N>(x[u].e, (uint64_t)j * N, 1);
+        group_reduce(a, VR, j);
+        if (j == 0 && v < nvec) out[v >> vr_shift] = a.result(flags);
+    }
+}
+
 // ---- cols -------------------------------------------------------------------------------------------------------------
 // src viewed as (outer, R, inner).  blockIdx.x -> (o, seg, tile); lane tx covers columns (tile * 64 + tx) * VW ..; wave ty takes
 // k = begin + ty, + kWaves, ...  Results go to out[o * inner + col], partial states to part[(seg * outer + o) * inner + col].
@@ -543,6 +568,20 @@ int32_t merge_cols(rt_ctx* ctx, const S* part, typename S::Out* out, uint64_t no
 template <class S, class T>
 int32_t rows_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t rows, uint64_t R, int flags) {
     hipStream_t s = ctx->stream;
+    {
+        constexpr uint64_t N = 16 / sizeof(T);
+        const uint64_t vr = R / N;
+        if (R % N == 0 && (vr == 1 || vr == 2 || vr == 4) && rows * vr >= 4096 && (reinterpret_cast<uintptr_t>(src) & 15) == 0) {
+            const uint64_t nvec = rows * vr;
+            const uint64_t blocks = (nvec + (uint64_t)kBlock * 4 - 1) / ((uint64_t)kBlock * 4);
+            if (blocks < (1ull << 31)) {
+                hipLaunchKernelGGL((st_rows_pow2_kernel<S, T>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, out, nvec, (uint32_t)vr,
+                                   vr == 1 ? 0u : (vr == 2 ? 1u : 2u), flags);
+                RT_HIP(hipGetLastError());
+                return RT_OK;
+            }
+        }
+    }
     if (R <= kTileMaxR && R * sizeof(T) < 2048) {                // from 2 KiB per row a wave per row is faster (f32 rows of 1024: 0.194 / 0.157 ms)
         TileArgs a;
         a.rows = rows;

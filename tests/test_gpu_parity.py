@@ -881,6 +881,10 @@ def test_reduction_shapes_short_rows_narrow_columns_short_axis(hip, dtype):
     for R in (1, 2, 3, 7, 8, 31, 32, 33, 63, 64, 65, 100, 255, 256, 1000, 1023, 1024, 1025):
         for rows in (1, 77, 1000):
             _check_reduce(hip, dtype, rows, R, 1, rng, offset=int(rng.integers(0, 5)))
+    # many short rows of a power-of-two number of 16-byte vectors: the kernel without staging (aligned and unaligned starts)
+    for R in (2, 4, 8, 16, 32, 64, 128, 256, 512, 1024):
+        for offset in (0, 4, 16, 3):
+            _check_reduce(hip, dtype, 70000 if R <= 64 else 5000, R, 1, rng, offset=offset)
     for inner in (2, 3, 4, 5, 17, 64, 100, 127, 128):
         for R, outer in ((64, 3), (1000, 1), (5003, 2), (70001, 1)):
             _check_reduce(hip, dtype, outer, R, inner, rng, offset=int(rng.integers(0, 5)))
@@ -943,6 +947,7 @@ def _check_arg(hip, dtype, outer, R, inner, rng, offset=0):
 
 STAT_SHAPES = ([(rows, R, 1) for R in (1, 2, 3, 7, 8, 31, 32, 33, 64, 65, 100, 255, 256, 1000, 1024, 1025, 2000, 4095) for rows in (1, 77, 1500)]
                + [(3, 70001, 1), (1, 300000, 1), (1100, 4100, 1)]
+               + [(30000, R, 1) for R in (1, 2, 4, 8, 16, 32, 64)]
                + [(outer, R, inner) for inner in (2, 3, 5, 17, 63, 64, 100, 128) for R, outer in ((64, 3), (1000, 1), (5003, 2), (70001, 1))]
                + [(outer, R, inner) for R in (1, 2, 5, 16, 33) for inner, outer in ((2, 1000), (3, 1), (64, 50), (1028, 2))]
                + [(1, 300, 5000), (2, 4000, 260), (1, 70, 2052)])
@@ -953,6 +958,9 @@ def test_statistic_reductions_shapes(hip, dtype):
     rng = np.random.default_rng(zlib.crc32(dtype.encode()))
     for outer, R, inner in STAT_SHAPES:
         _check_stat(hip, dtype, outer, R, inner, rng, offset=int(rng.integers(0, 5)))
+    for R in (2, 4, 8, 16):                                       # aligned starts reach the kernel without staging
+        _check_stat(hip, dtype, 30000, R, 1, rng, offset=0)
+        _check_stat(hip, dtype, 30000, R, 1, rng, offset=8)
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f64", "i32", "u8", "i64", "i16"])
@@ -960,6 +968,9 @@ def test_argmax_argmin_shapes(hip, dtype):
     rng = np.random.default_rng(zlib.crc32(dtype.encode()))
     for outer, R, inner in STAT_SHAPES:
         _check_arg(hip, dtype, outer, R, inner, rng, offset=int(rng.integers(0, 5)))
+    for R in (2, 4, 8, 16, 32, 64):
+        _check_arg(hip, dtype, 30000, R, 1, rng, offset=0)
+        _check_arg(hip, dtype, 30000, R, 1, rng, offset=16)
 
 
 def test_statistic_reductions_known_answers_and_edges(hip):
