@@ -282,9 +282,17 @@ __global__ __launch_bounds__(kBlock) void st_rows_tile_kernel(const T* __restric
     const uint32_t nrows = (uint32_t)(a.rows - row0 < a.rpb ? a.rows - row0 : a.rpb);
     const uint32_t ne = nrows * a.R;
     const T* p = src + row0 * a.R;
+    // 1- and 2-byte elements: the run is copied as it lies, with 16-byte LDS stores (an element-wise scatter would issue 8 or 16
+    // sub-word stores per vector: u8 rows of 100 ran at 1.9 TB/s); `mis` keeps the 16-byte phase of the global address
+    constexpr bool kVerbatim = sizeof(T) < 4;
+    const uint32_t mis = kVerbatim ? (uint32_t)((reinterpret_cast<uintptr_t>(p) & 15) / sizeof(T)) : 0u;
     auto put = [&](uint32_t e, T v) {
-        const uint32_t r = fd_div(e, a.r_div);
-        tile[r * a.pitch + (e - r * a.R)] = v;
+        if constexpr (kVerbatim) {
+            tile[mis + e] = v;
+        } else {
+            const uint32_t r = fd_div(e, a.r_div);
+            tile[r * a.pitch + (e - r * a.R)] = v;
+        }
     };
     uint32_t head = (uint32_t)(((16 - (reinterpret_cast<uintptr_t>(p) & 15)) & 15) / sizeof(T));
     if (head > ne) head = ne;
@@ -300,8 +308,12 @@ __global__ __launch_bounds__(kBlock) void st_rows_tile_kernel(const T* __restric
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             if (v0 + u * kBlock < nvec) {
+                if constexpr (kVerbatim) {
+                    *reinterpret_cast<Vec16<T>*>(&tile[mis + head + (v0 + u * kBlock) * N]) = x[u];
+                } else {
 #pragma unroll
-                for (uint32_t j = 0; j < N; ++j) put(head + (v0 + u * kBlock) * N + j, x[u].e[j]);
+                    for (uint32_t j = 0; j < N; ++j) put(head + (v0 + u * kBlock) * N + j, x[u].e[j]);
+                }
             }
         }
     }
@@ -314,7 +326,7 @@ __global__ __launch_bounds__(kBlock) void st_rows_tile_kernel(const T* __restric
         S acc;
         acc.init();
         if (r < nrows) {
-            const T* row = tile + r * a.pitch;
+            const T* row = tile + mis + r * a.pitch;              // pitch == R in the verbatim layout
             uint32_t k = j;
             for (; k + 3 * a.G < a.R; k += 4 * a.G) {
                 T x[4];
@@ -586,8 +598,8 @@ int32_t rows_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t rows
         TileArgs a;
         a.rows = rows;
         a.R = (uint32_t)R;
-        a.pitch = a.R | 1u;
-        a.rpb = (uint32_t)(kTileBytes / sizeof(T)) / a.pitch;
+        a.pitch = sizeof(T) < 4 ? a.R : (a.R | 1u);
+        a.rpb = (uint32_t)(kTileBytes / sizeof(T) - (sizeof(T) < 4 ? 16 / sizeof(T) : 0)) / a.pitch;
         a.r_div = make_fastdiv(a.R);
         uint32_t g = 1;                                           // lanes per row: fill the block, at most one wave, at most R
         while (g < 64 && (uint64_t)g * 2 * a.rpb <= (uint64_t)kBlock && g * 2 <= a.R) g <<= 1;
