@@ -196,15 +196,56 @@ __global__ __launch_bounds__(kBlock) void bin_generic_kernel(const T* l, const T
 // dst is one forward contiguous run but its rows are too short (or not 16-byte aligned) for the row kernel, e.g. (2^26, 4) + (4,)
 // or rows of 1001 elements: a lane owns one 16-byte vector of dst, an input laid out like dst (LV / RV) is read with one vector
 // load, any other input element by element through the index decomposition (it is a broadcast operand: its lines stay in cache).
-template <class T, int OP, bool LV, bool RV>
+// Operand modes of the flat kernel: F_VEC laid out like dst (one vector load), F_ROW one row of `a.shape[rank - 1]` elements
+// repeated for every row (stride 1 along the last dim, 0 along the others), F_ELEM anything else.
+enum FlatMode : int { F_ELEM = 0, F_VEC = 1, F_ROW = 2 };
+
+// 16 bytes of a repeated row starting at column c0 = (first element of the vector) mod L.  Inside the row that is one 16-byte
+// load from an address that is only element-aligned (the hardware runs in unaligned-access mode); a vector that wraps around the
+// end of the row is put together element by element.  Without this a 1-byte row needed sixteen index decompositions per lane
+// (u8 (N, 1000) + (1000,): 2.3 TB/s).
+template <class T>
+__device__ __forceinline__ Vec16<T> load_row_vec(const T* __restrict__ row, uint32_t first, uint32_t L, const FastDiv32& l_div) {
+    constexpr uint32_t N = 16 / sizeof(T);
+    uint32_t c = first - fd_div(first, l_div) * L;
+    Vec16<T> y;
+    if (c + N <= L) {
+        __builtin_memcpy(&y, row + c, 16);
+    } else if (L >= N) {
+        // the vector holds the last k elements of the row and then its first N - k: two loads that stay inside the row, joined
+        // by a 128-bit funnel shift (nearly every wave of a 1000-byte row has one such lane; sixteen dependent byte loads there
+        // held the whole wave back)
+        const uint32_t k = L - c;                                 // 1 .. N - 1
+        unsigned __int128 tail, head;
+        __builtin_memcpy(&tail, row + (L - N), 16);
+        __builtin_memcpy(&head, row, 16);
+        const unsigned __int128 both = (tail >> ((N - k) * sizeof(T) * 8)) | (head << (k * sizeof(T) * 8));
+        __builtin_memcpy(&y, &both, 16);
+    } else {
+#pragma unroll
+        for (uint32_t j = 0; j < N; ++j) {
+            y.e[j] = row[c];
+            c = (c + 1 == L) ? 0u : c + 1;
+        }
+    }
+    return y;
+}
+
+template <class T, int OP, int LMODE, int RMODE>
 __global__ __launch_bounds__(kRBlock) void bin_flat_kernel(const T* l, const T* r, T* d, GenArgs a, uint32_t nvec) {
     constexpr int N = 16 / sizeof(T);
+    constexpr bool LE = LMODE == F_ELEM, RE = RMODE == F_ELEM && OP != kOpCopy;
     const uint32_t v = blockIdx.x * kRBlock + threadIdx.x;
     if (v >= nvec) return;
     Vec16<T> x, y;
-    if constexpr (LV) x = rt_ld16_nt(reinterpret_cast<const Vec16<T>*>(l) + v);
-    if constexpr (RV) y = rt_ld16_nt(reinterpret_cast<const Vec16<T>*>(r) + v);
-    if constexpr (!LV || (!RV && OP != kOpCopy)) {
+    const uint32_t L = a.shape[a.rank - 1];
+    if constexpr (LMODE == F_VEC) x = rt_ld16_nt(reinterpret_cast<const Vec16<T>*>(l) + v);
+    if constexpr (LMODE == F_ROW) x = load_row_vec<T>(l, v * N, L, a.div[a.rank - 1]);
+    if constexpr (OP != kOpCopy) {
+        if constexpr (RMODE == F_VEC) y = rt_ld16_nt(reinterpret_cast<const Vec16<T>*>(r) + v);
+        if constexpr (RMODE == F_ROW) y = load_row_vec<T>(r, v * N, L, a.div[a.rank - 1]);
+    }
+    if constexpr (LE || RE) {
 #pragma unroll
         for (int j = 0; j < N; ++j) {
             uint32_t rem = v * N + j;
@@ -214,13 +255,13 @@ __global__ __launch_bounds__(kRBlock) void bin_flat_kernel(const T* l, const T* 
                 if (k < a.rank) {
                     uint32_t q = fd_div(rem, a.div[k]);
                     uint32_t c = rem - q * a.shape[k];
-                    if constexpr (!LV) ol += (int64_t)c * a.stride[0][k];
-                    if constexpr (!RV) orr += (int64_t)c * a.stride[1][k];
+                    if constexpr (LE) ol += (int64_t)c * a.stride[0][k];
+                    if constexpr (RE) orr += (int64_t)c * a.stride[1][k];
                     rem = q;
                 }
             }
-            if constexpr (!LV) x.e[j] = l[ol];
-            if constexpr (!RV && OP != kOpCopy) y.e[j] = r[orr];
+            if constexpr (LE) x.e[j] = l[ol];
+            if constexpr (RE) y.e[j] = r[orr];
         }
     }
     if constexpr (OP == kOpCopy) y = x;
@@ -486,11 +527,21 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
         if (flat(2, dp) && count >= (uint64_t)N) {
             const uint32_t nvec = (uint32_t)(count / N);
             const bool lv = flat(0, lp), rv = OP != kOpCopy && flat(1, rp);
+            // a repeated row: stride 1 along the last dim, 0 along every other one
+            auto row_like = [&](int o) {
+                if (rank < 2 || dsc.stride[o][rank - 1] != 1) return false;
+                for (int k = 0; k < rank - 1; ++k)
+                    if (dsc.stride[o][k] != 0) return false;
+                return true;
+            };
+            const bool lrow = !lv && rv && row_like(0), rrow = lv && !rv && OP != kOpCopy && row_like(1);
             dim3 grid((nvec + kRBlock - 1) / kRBlock), blk(kRBlock);
-            if (lv && rv) hipLaunchKernelGGL((bin_flat_kernel<T, OP, true, true>), grid, blk, 0, s, lp, rp, dp, g, nvec);
-            else if (lv) hipLaunchKernelGGL((bin_flat_kernel<T, OP, true, false>), grid, blk, 0, s, lp, rp, dp, g, nvec);
-            else if (rv) hipLaunchKernelGGL((bin_flat_kernel<T, OP, false, true>), grid, blk, 0, s, lp, rp, dp, g, nvec);
-            else hipLaunchKernelGGL((bin_flat_kernel<T, OP, false, false>), grid, blk, 0, s, lp, rp, dp, g, nvec);
+            if (lrow) hipLaunchKernelGGL((bin_flat_kernel<T, OP, F_ROW, F_VEC>), grid, blk, 0, s, lp, rp, dp, g, nvec);
+            else if (rrow) hipLaunchKernelGGL((bin_flat_kernel<T, OP, F_VEC, F_ROW>), grid, blk, 0, s, lp, rp, dp, g, nvec);
+            else if (lv && rv) hipLaunchKernelGGL((bin_flat_kernel<T, OP, F_VEC, F_VEC>), grid, blk, 0, s, lp, rp, dp, g, nvec);
+            else if (lv) hipLaunchKernelGGL((bin_flat_kernel<T, OP, F_VEC, F_ELEM>), grid, blk, 0, s, lp, rp, dp, g, nvec);
+            else if (rv) hipLaunchKernelGGL((bin_flat_kernel<T, OP, F_ELEM, F_VEC>), grid, blk, 0, s, lp, rp, dp, g, nvec);
+            else hipLaunchKernelGGL((bin_flat_kernel<T, OP, F_ELEM, F_ELEM>), grid, blk, 0, s, lp, rp, dp, g, nvec);
             first = nvec * (uint32_t)N;                          // the last count % N elements go to the element kernel
         }
         if (first < count) {

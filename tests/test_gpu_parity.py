@@ -452,6 +452,28 @@ def test_broadcast_random_vs_oracle(hip, dtype, op):
         assert got.dump().tobytes() == want.buf.tobytes(), (trial, dtype, op, ova.meta, ovb.meta)
 
 
+@pytest.mark.parametrize("dtype", ["u8", "i8", "i16", "f32", "f64", "bool"])
+def test_broadcast_repeated_row_any_length(hip, dtype):
+    """(rows, L) op (L,) for row lengths that are not a whole number of 16-byte vectors, so that vectors of the output straddle the
+    end of the row (unaligned row loads, the two-load wrap-around, rows shorter than a vector), both operand orders, out of place
+    and in place; plus the aligned lengths that take the flat row kernel."""
+    rng = np.random.default_rng(zlib.crc32(dtype.encode()) + 5)
+    for L in (1, 2, 3, 5, 7, 15, 16, 17, 31, 33, 100, 250, 1000, 1001, 1024, 4099):
+        rows = max(3, 40000 // L)
+        va, vb = rand_values(dtype, rows * L, rng), rand_values(dtype, L, rng)
+        oa, ob = OTensor.from_buf(dtype, va, [rows, L]), OTensor.from_buf(dtype, vb, [L])
+        ga, gb = G(hip, dtype, va, [rows, L]), G(hip, dtype, vb, [L])
+        for f in ("__add__", "__sub__", "__mul__"):
+            with np.errstate(all="ignore"):
+                w1, w2 = getattr(oa, f)(ob), getattr(ob, f)(oa)
+            assert getattr(ga, f)(gb).dump().tobytes() == w1.buf.tobytes(), (dtype, L, f, "x op row")
+            assert getattr(gb, f)(ga).dump().tobytes() == w2.buf.tobytes(), (dtype, L, f, "row op x")
+        with np.errstate(all="ignore"):
+            oa += ob
+        ga += gb
+        assert ga.dump().tobytes() == oa.buf.tobytes(), (dtype, L, "in place")
+
+
 @pytest.mark.parametrize("dtype", ["f32", "i32", "f64", "u8"])
 def test_broadcast_inplace_random(hip, dtype):
     rng = np.random.default_rng(17)
