@@ -60,6 +60,10 @@ def run_case(case, factory, SliceCls, ErrorCls):
                 a = env[args[0]]
                 env[dst] = {"add_scalar": a.__add__, "sub_scalar": a.__sub__, "mul_scalar": a.__mul__,
                             "div_scalar": a.__truediv__}[op](args[1])
+            elif op in ("iadd_scalar", "isub_scalar", "imul_scalar", "idiv_scalar"):            # `view += 5` and friends
+                a = env[args[0]]
+                env[dst] = {"iadd_scalar": a.__iadd__, "isub_scalar": a.__isub__, "imul_scalar": a.__imul__,
+                            "idiv_scalar": a.__itruediv__}[op](args[1])
             elif op == "unary":
                 env[dst] = env[args[0]].unary(args[1])
             elif op == "unary_inplace":
