@@ -61,6 +61,9 @@ class GTensor:
     def get(self, idx):
         return self.backend.read(self.buf, logical_to_buffer_idx(list(idx), self.meta.strides, self.meta.offset))
 
+    def set(self, idx, value):
+        self.backend.write(self.buf, logical_to_buffer_idx(list(idx), self.meta.strides, self.meta.offset), value)
+
     def dump(self): return self.backend.dump(self.buf)
 
     def owned(self):
