@@ -64,6 +64,11 @@ def run_case(case, factory, SliceCls, ErrorCls):
                 a = env[args[0]]
                 env[dst] = {"iadd_scalar": a.__iadd__, "isub_scalar": a.__isub__, "imul_scalar": a.__imul__,
                             "idiv_scalar": a.__itruediv__}[op](args[1])
+            elif op == "fill":                                                                   # view.fill(value)
+                env[args[0]].fill(args[1])
+                env[dst] = env[args[0]]
+            elif op == "owned":
+                env[dst] = env[args[0]].owned()
             elif op == "set":                                                                    # view.set(coord, value)
                 env[args[0]].set(args[1], args[2])
                 env[dst] = env[args[0]]
