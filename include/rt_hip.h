@@ -123,7 +123,9 @@ int32_t rt_copy(rt_ctx* ctx, int32_t dtype, const void* src, uint64_t len, void*
 int32_t rt_dump(rt_ctx* ctx, int32_t dtype, const void* src, uint64_t len, void* host_dst);
 /* PartialEq of Backend::Buf (backend/cuda.rs:59-141): lengths equal and all elements `==` (NaN != NaN). */
 int32_t rt_equal(rt_ctx* ctx, int32_t dtype, const void* a, uint64_t a_len, const void* b, uint64_t b_len, int32_t* out_equal);
-/* Backend::convert: elementwise dtype conversion between equally long buffers (core/value.rs:255-462). */
+/* Backend::convert: elementwise dtype conversion between equally long buffers (core/value.rs:255-462), every pair of the 13 dtypes:
+ * Rust `as` between integers, float -> integer rounds half away from zero and saturates (NaN -> 0), integer -> float rounds to
+ * nearest (u128 -> f32 overflows to +inf), anything -> bool is x != 0. */
 int32_t rt_convert(rt_ctx* ctx, int32_t src_dtype, const void* src, uint64_t src_len, int32_t dst_dtype, void* dst, uint64_t dst_len);
 
 /* ---- fill (Backend::fill_contiguous / fill_1d_strided / fill_nd, backend/mod.rs:270-294) ----------------------- */

@@ -66,7 +66,51 @@ struct boolean_t { uint8_t v; };
 template <class T> struct is_flt : std::integral_constant<bool, std::is_same<T, float>::value || std::is_same<T, double>::value> {};
 template <class T> struct is_bool : std::is_same<T, boolean_t> {};
 
+typedef unsigned __int128 u128_t;
+typedef __int128 i128_t;
+template <class T> struct is_128 : std::integral_constant<bool, std::is_same<T, u128_t>::value || std::is_same<T, i128_t>::value> {};
+
+// u128 -> f32 / f64, correctly rounded (Rust `as`): the 64 leading bits go through the hardware's u64 conversion with the bits
+// shifted out folded into the lowest one (it lies far below the rounding position), then an exact power-of-two scaling.  A value
+// of 2^128 - 2^103 and above becomes +inf in f32, as in Rust.
+template <class F> __device__ __forceinline__ F u128_to_float(u128_t x) {
+    const uint64_t hi = (uint64_t)(x >> 64), lo = (uint64_t)x;
+    if (hi == 0) return (F)lo;
+    const int lz = __builtin_clzll(hi);
+    const u128_t v = x << lz;
+    uint64_t m = (uint64_t)(v >> 64);
+    if ((uint64_t)v != 0) m |= 1;
+    if constexpr (std::is_same<F, float>::value) return ldexpf((float)m, 64 - lz);
+    else return ldexp((double)m, 64 - lz);
+}
+// f32 / f64 (already rounded to an integer, finite, 0 <= r < 2^128) -> u128, exact
+template <class F> __device__ __forceinline__ u128_t float_to_u128(F r) {
+    const F two64 = (F)18446744073709551616.0;
+    if (r < two64) return (u128_t)(uint64_t)r;
+    const uint64_t hi = (uint64_t)(r / two64);                  // a power-of-two quotient: exact, then truncated
+    const uint64_t lo = (uint64_t)(r - (F)hi * two64);
+    return ((u128_t)hi << 64) | lo;
+}
+
 template <class D, class S> __device__ __forceinline__ D convert_one(S x) {
+    if constexpr (is_128<D>::value && is_flt<S>::value) {
+        // round half away from zero, then Rust's saturating `as` (NaN -> 0)
+        S r = std::is_same<S, float>::value ? (S)roundf((float)x) : (S)round((double)x);
+        if (r != r) return (D)0;
+        const S two127 = (S)170141183460469231731687303715884105728.0;
+        if constexpr (std::is_same<D, u128_t>::value) {
+            if (r <= (S)0) return (D)0;
+            if (r >= two127 * (S)2) return ~(u128_t)0;          // also +inf (2^128 itself is not finite in f32)
+            return float_to_u128<S>(r);
+        } else {
+            if (r <= -two127) return (i128_t)((u128_t)1 << 127);
+            if (r >= two127) return (i128_t)(~(u128_t)0 >> 1);
+            return r < (S)0 ? -(i128_t)float_to_u128<S>(-r) : (i128_t)float_to_u128<S>(r);
+        }
+    } else if constexpr (is_128<S>::value && is_flt<D>::value) {
+        if constexpr (std::is_same<S, u128_t>::value) return u128_to_float<D>(x);
+        else return x < 0 ? -u128_to_float<D>((u128_t)0 - (u128_t)x) : u128_to_float<D>((u128_t)x);
+    } else
     if constexpr (is_bool<D>::value) {
         if constexpr (is_bool<S>::value) return x;
         else return boolean_t{(uint8_t)(x != (S)0)};
@@ -161,6 +205,8 @@ int32_t convert_go(rt_ctx* ctx, const void* s, void* d, size_t n) {
         case RT_F32: return convert_go<S, float>(ctx, s, d, n);                    \
         case RT_F64: return convert_go<S, double>(ctx, s, d, n);                   \
         case RT_BOOL: return convert_go<S, boolean_t>(ctx, s, d, n);               \
+        case RT_U128: return convert_go<S, u128_t>(ctx, s, d, n);                  \
+        case RT_I128: return convert_go<S, i128_t>(ctx, s, d, n);                  \
     }                                                                              \
     break;
 
@@ -177,6 +223,8 @@ int32_t convert_any(rt_ctx* ctx, int sd, const void* s, int dd, void* d, size_t 
         case RT_F32: RT_DST_CASES(float)
         case RT_F64: RT_DST_CASES(double)
         case RT_BOOL: RT_DST_CASES(boolean_t)
+        case RT_U128: RT_DST_CASES(u128_t)
+        case RT_I128: RT_DST_CASES(i128_t)
     }
     return rt_fail(RT_E_DTYPE, "convert: dtype pair (%d -> %d) is not built for the device", sd, dd);
 }

@@ -685,6 +685,86 @@ def test_convert(hip):
     assert e.value.kind == "SizeMismatch"
 
 
+def test_convert_128bit_integers(hip):
+    """`T::convert::<N>` with u128 / i128 on either side (core/value.rs:255-462): Rust `as` between integers (truncate / extend), round half
+    away from zero + saturating cast from floats, correctly rounded casts to floats; checked against Python's exact integers."""
+    import struct
+    from rtensors_amd import hip as H
+    rng = np.random.default_rng(1280)
+    M = 1 << 128
+
+    def wrap(v, code):                                                   # Rust `as` to a 128-bit type from any integer
+        v %= M
+        return v - M if code == cpu.I128 and v >= M >> 1 else v
+    ints = [0, 1, -1, 2 ** 63, -2 ** 63, 2 ** 64, 2 ** 64 - 1, 2 ** 127 - 1, -2 ** 127, 2 ** 127, 2 ** 128 - 1, 255, 256, -129, 2 ** 100 + 2 ** 76, 2 ** 100 + 2 ** 76 + 1,
+            2 ** 100 + 3 * 2 ** 76, 2 ** 128 - 2 ** 103, 2 ** 128 - 2 ** 103 - 1, 2 ** 120 + 2 ** 66, 2 ** 120 + 2 ** 66 + 1]
+    ints += [int(rng.integers(0, 2 ** 63)) * int(rng.integers(0, 2 ** 63)) * int(rng.choice([1, -1])) * int(rng.integers(1, 8)) for _ in range(300)]
+    for code in (cpu.U128, cpu.I128):
+        vals = [wrap(v, code) for v in ints]
+        src = hip.alloc_from_slice(code, cpu.from_ints(code, vals))
+        # to the narrower integers and bool: truncation
+        for name in ("u8", "i8", "u16", "i16", "u32", "i32", "u64", "i64"):
+            dcode = cpu.DTYPE_BY_NAME[name]
+            dst = hip.alloc(dcode, len(vals)); hip.convert(src, dst)
+            bits = cpu.NP_DTYPE[dcode].itemsize * 8
+            want = [(v % (1 << bits)) - ((1 << bits) if name[0] == "i" and (v % (1 << bits)) >= 1 << (bits - 1) else 0) for v in vals]
+            assert [int(x) for x in hip.dump(dst)] == want, (code, name)
+        dst = hip.alloc(cpu.BOOL, len(vals)); hip.convert(src, dst)
+        assert hip.dump(dst).tolist() == [v != 0 for v in vals]
+        other = cpu.I128 if code == cpu.U128 else cpu.U128
+        dst = hip.alloc(other, len(vals)); hip.convert(src, dst)
+        assert cpu.to_ints(other, hip.dump(dst)) == [wrap(v, other) for v in vals]
+        # to f64: Python's int -> float is correctly rounded; to f32: nearest of the two neighbours, ties to even, by exact integer arithmetic
+        dst = hip.alloc(cpu.F64, len(vals)); hip.convert(src, dst)
+        assert hip.dump(dst).tolist() == [float(v) for v in vals], code
+
+        def to_f32(v):
+            if v == 0: return 0.0
+            sgn, a = (-1 if v < 0 else 1), abs(v)
+            e = a.bit_length() - 24
+            if e <= 0: return float(v)
+            q, r = a >> e, a & ((1 << e) - 1)
+            half = 1 << (e - 1)
+            if r > half or (r == half and q & 1): q += 1
+            f = q << e
+            return sgn * (float("inf") if f >= (1 << 128) - (1 << 103) and f.bit_length() > 128 or f >= 1 << 128 else float(f))
+        dst = hip.alloc(cpu.F32, len(vals)); hip.convert(src, dst)
+        got = hip.dump(dst).astype(np.float64).tolist()
+        assert got == [to_f32(v) for v in vals], [(v, g, to_f32(v)) for v, g in zip(vals, got) if g != to_f32(v)][:3]
+    # from the other types
+    for name in ("u8", "i8", "i16", "u32", "i64", "u64", "bool"):
+        scode = cpu.DTYPE_BY_NAME[name]
+        x = rand_values(name, 500, rng, -2 ** 62, 2 ** 62)
+        if name not in ("bool",):
+            info = np.iinfo(x.dtype); x[:2] = [info.min, info.max]
+        src = hip.alloc_from_slice(scode, x)
+        for code in (cpu.U128, cpu.I128):
+            dst = hip.alloc(code, x.size); hip.convert(src, dst)
+            assert cpu.to_ints(code, hip.dump(dst)) == [wrap(int(v), code) for v in x], (name, code)
+    for fname, npd in (("f32", np.float32), ("f64", np.float64)):
+        f = np.concatenate([rng.standard_normal(200) * 10.0 ** rng.integers(0, 39, size=200),
+                            [0.0, -0.0, 0.5, -0.5, 1.5, 2.5, -2.5, np.nan, np.inf, -np.inf, 2.0 ** 64, 2.0 ** 64 - 2 ** 12, 2.0 ** 127, -2.0 ** 127, 2.0 ** 126,
+                             3.4e38, -3.4e38, 1e30, -1e30, 2.0 ** 63, 2.0 ** 100]]).astype(npd)
+        src = hip.alloc_from_slice(cpu.DTYPE_BY_NAME[fname], f)
+
+        def rust_cast(v, code):
+            v = float(v)
+            if v != v: return 0
+            if v in (float("inf"), float("-inf")):
+                r = v
+            else:
+                r = int(np.sign(v)) * int(np.floor(abs(v) + 0.5)) if abs(v) < 2 ** 60 else int(v)     # round half away from zero; large values are integers
+            lo, hi = (0, M - 1) if code == cpu.U128 else (-(M >> 1), (M >> 1) - 1)
+            if r == float("inf"): return hi
+            if r == float("-inf"): return lo
+            return min(max(r, lo), hi)
+        for code in (cpu.U128, cpu.I128):
+            dst = hip.alloc(code, f.size); hip.convert(src, dst)
+            got = cpu.to_ints(code, hip.dump(dst))
+            want = [rust_cast(v, code) for v in f]
+            assert got == want, [(float(v), g, w) for v, g, w in zip(f, got, want) if g != w][:3]
+
+
 @pytest.mark.parametrize("dtype", ["f32", "f64", "i32", "u8", "i16"])
 def test_broadcast_with_transposed_operand(hip, dtype):
     """One input is a permuted (and possibly reversed / strided) view whose unit-stride dim is not the output's inner dim:
