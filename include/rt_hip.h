@@ -178,7 +178,8 @@ int32_t rt_reduce_nd(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, ui
  *                                                           when +inf occurs (the reference's flat launcher has no case for it
  *                                                           and leaves dst unwritten, reduce.cu:795-832; here flat works too)
  *   RT_R_NORM | RT_R_FLAG_L1 / RT_R_FLAG_L2                  sum |x| / sqrt(sum x^2)
- * Results are within 1e-5 (f32) / 1e-12 (f64), relative, of the same quantity accumulated in higher precision.
+ * Results are within 1e-5 (f32) / 1e-12 (f64), relative, of the same quantity accumulated in higher precision (variance: times its
+ * condition number sqrt(1 + mean^2 / var); logsumexp: relative to max(|result|, |largest element|), the two terms it adds).
  * RT_R_ARGMAX / RT_R_ARGMIN are refused here with RT_E_INVALID (kinds cannot be swapped between entry points,
  * backend/remote/remote_tests.rs:857-859). */
 
