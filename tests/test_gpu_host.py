@@ -22,7 +22,7 @@ def be(T):
     return T.Backend(0)
 
 
-CASES = (golden_dsl.load("reference_vectors.json") + golden_dsl.load("reference_scalar_vectors.json") + golden_dsl.load("reference_view_vectors.json") + golden_dsl.load("reference_meta_vectors.json") +
+CASES = (golden_dsl.load("reference_vectors.json") + golden_dsl.load("reference_scalar_vectors.json") + golden_dsl.load("reference_view_vectors.json") + golden_dsl.load("reference_operand_vectors.json") + golden_dsl.load("reference_meta_vectors.json") +
          golden_dsl.load("reference_matmul_vectors.json"))
 
 

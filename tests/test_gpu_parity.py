@@ -404,7 +404,7 @@ def test_reversed_view_is_walked_backwards_not_out_of_bounds(hip):
         o.slice(0, Slice(None, None, -1)).unary_inplace("relu")
 
 
-CASES = golden_dsl.load("reference_vectors.json") + golden_dsl.load("reference_scalar_vectors.json") + golden_dsl.load("reference_view_vectors.json") + golden_dsl.load("reference_matmul_vectors.json")
+CASES = golden_dsl.load("reference_vectors.json") + golden_dsl.load("reference_scalar_vectors.json") + golden_dsl.load("reference_view_vectors.json") + golden_dsl.load("reference_operand_vectors.json") + golden_dsl.load("reference_matmul_vectors.json")
 
 
 @pytest.mark.parametrize("case", CASES, ids=lambda c: c["name"])

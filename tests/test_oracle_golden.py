@@ -8,7 +8,7 @@ from oracle import cpu
 from oracle.meta import Slice, TensorError
 from oracle.tensor import OTensor
 
-CASES = golden_dsl.load("reference_vectors.json") + golden_dsl.load("reference_scalar_vectors.json") + golden_dsl.load("reference_view_vectors.json") + golden_dsl.load("reference_matmul_vectors.json")
+CASES = golden_dsl.load("reference_vectors.json") + golden_dsl.load("reference_scalar_vectors.json") + golden_dsl.load("reference_view_vectors.json") + golden_dsl.load("reference_operand_vectors.json") + golden_dsl.load("reference_matmul_vectors.json")
 META_CASES = golden_dsl.load("reference_meta_vectors.json")
 
 
