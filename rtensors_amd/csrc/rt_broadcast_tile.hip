@@ -1,7 +1,7 @@
 // LDS-transpose kernel of the broadcast family (see rt_broadcast.hip for the family and rt_broadcast_common.h for the
 // shared definitions).  One input has its unit-|stride| dim `t` somewhere other than dst's inner dim (a permuted, possibly
 // reversed view, e.g. `a + b.transpose()` or the row-major copy of a permuted tensor): reading it along dst's inner dim would
-// touch one cache line per element.  A block instead gathers a (kTK x TL) tile of it along *its* unit-stride dim with
+// touch one cache line per element.  A block instead gathers a (TK x TL) tile of it along *its* unit-stride dim with
 // 16-byte loads (full 128-byte lines), scatters the elements into LDS transposed, and then writes full rows of dst with
 // 16-byte non-temporal stores, combining with the other input on the way.
 //
@@ -16,9 +16,20 @@ using namespace rtb;
 namespace {
 
 constexpr int kTBlock = 256;
-constexpr int kTK = 32;                      // tile extent along the transposed operand's unit-stride dim
 constexpr int kTWaves = kTBlock / RT_WAVE;
-constexpr int kTRows = kTK / kTWaves;        // dst rows of the tile written by each wave (8)
+constexpr int kTSteps = 8;                   // 16-byte vectors of dst written by each lane per tile
+
+// Tile geometry by element size.  4 bytes and more: 32 elements along the transposed operand's unit-stride dim (a 128-byte line
+// of f32) by 64 vectors along dst's inner dim, so a wave writes 1 KiB of one dst row per instruction.  1-byte elements: 64 by 32
+// vectors (512 bytes of two dst rows per wave instruction), because 32 elements along t would gather only a quarter of a line
+// per inner-dim position (32768^2 u8 add with a transposed operand: 5.5 TB/s against 4.8 with the 32 x 64 shape).  2-byte
+// elements keep 32 x 64: the 64 x 32 shape measured +1 % on that add and -7 % on the transposing copy.
+template <class T> struct TileGeom {
+    static constexpr int LPR = sizeof(T) == 1 ? 32 : 64;           // lanes (vectors) per tile row
+    static constexpr int RPI = RT_WAVE / LPR;                       // dst rows per wave instruction
+    static constexpr int TK = kTSteps * kTWaves * RPI;              // tile extent along dim t
+    static constexpr int TL = LPR * (16 / (int)sizeof(T));          // tile extent along dst's inner dim
+};
 
 struct TileArgs {
     uint32_t L, K, G;               // inner length, extent of dim t, extent of the loop dim (1 if none)
@@ -40,8 +51,8 @@ struct TileArgs {
 template <class T, int OP, int OM, bool VG>
 __global__ __launch_bounds__(kTBlock) void bin_tile_kernel(const T* xt, const T* xo, T* d, TileArgs a) {
     constexpr int N = 16 / sizeof(T);
-    constexpr int TL = RT_WAVE * N;           // tile extent along dst's inner dim: one 16-byte vector per lane of a wave
-    __shared__ alignas(16) T tile[kTK][TL + N];
+    constexpr int LPR = TileGeom<T>::LPR, RPI = TileGeom<T>::RPI, TK = TileGeom<T>::TK, TL = TileGeom<T>::TL;
+    __shared__ alignas(16) T tile[TK][TL + N];
     // blockIdx -> (outer index, chunk of the loop dim, tile along t, tile along the inner dim); the last is the fastest so
     // that blocks running together write neighbouring 1 KiB pieces of the same dst rows
     uint32_t b = blockIdx.x;
@@ -69,7 +80,7 @@ __global__ __launch_bounds__(kTBlock) void bin_tile_kernel(const T* xt, const T*
     xt += offx;
     xo += offo;
     T* dp = d + offd;
-    const uint32_t k0 = ktile * kTK, l0 = ltile * TL;
+    const uint32_t k0 = ktile * TK, l0 = ltile * TL;
     const uint32_t g_begin = chunk * a.gchunk;
     const uint32_t g_end = min(a.G, g_begin + a.gchunk);
     const bool xt_fixed = a.gstride[0] == 0;
@@ -77,19 +88,20 @@ __global__ __launch_bounds__(kTBlock) void bin_tile_kernel(const T* xt, const T*
     const bool x_left = a.x_is_left != 0;
 
     const uint32_t lane = threadIdx.x & (RT_WAVE - 1), wv = threadIdx.x / RT_WAVE;
-    const uint32_t c = l0 + lane * N;                        // first inner column of this lane's vectors
+    const uint32_t c = l0 + (lane % LPR) * N;                // first inner column of this lane's vectors
+    const uint32_t krow = wv * RPI + lane / LPR;             // this lane's tile row in step 0; step i adds i * kTWaves * RPI
     const bool full_vec = c + N <= a.L;
 
     for (uint32_t g = g_begin; g < g_end; ++g) {
         // rows of the other operand for this step: issued before the gather so that both are in flight together (issuing them
         // after the gather's LDS writes saves 40 VGPRs and reaches four waves per SIMD instead of three, but measured 3 % slower)
-        Vec16<T> ov[kTRows] = {};
+        Vec16<T> ov[kTSteps] = {};
         if constexpr (OP != kOpCopy) {
             if (full_vec) {
                 const T* orow = xo + (int64_t)g * a.gstride[1];
 #pragma unroll
-                for (int i = 0; i < kTRows; ++i) {
-                    const uint32_t k = min(k0 + wv + i * kTWaves, a.K - 1);
+                for (int i = 0; i < kTSteps; ++i) {
+                    const uint32_t k = min(k0 + krow + i * kTWaves * RPI, a.K - 1);
                     if (i == 0 || !o_fixed) ov[i] = load_vec<T, OM>(orow + (int64_t)k * a.tstride[1], c, a.istride[1], a.nt_other != 0);
                     else ov[i] = ov[0];
                 }
@@ -98,10 +110,61 @@ __global__ __launch_bounds__(kTBlock) void bin_tile_kernel(const T* xt, const T*
         if (g == g_begin || !xt_fixed) {
             if (g != g_begin) __syncthreads();
             const T* xg = xt + (int64_t)g * a.gstride[0];
-            if constexpr (VG) {
+            if constexpr (VG && sizeof(T) < 4) {
+                // 1- and 2-byte elements: a lane loads the vectors of P = 4 / sizeof(T) neighbouring inner-dim positions and
+                // transposes P x P blocks in registers (byte permutes), so that every LDS write carries a full 32-bit word of P
+                // neighbouring columns of one tile row.  One LDS write per element, as the 4-byte path does, costs 2x / 4x the
+                // LDS instructions per byte moved and held a 16384^2 add with a transposed operand at 4.5 (i16) / 2.5 (u8) TB/s
+                // (now 5.7 / 5.5).
+                constexpr int P = 4 / sizeof(T);
+                constexpr int VT = TK / N;                     // vectors per tile row along t
+                constexpr int GPI = kTBlock / VT;              // groups of P inner-dim positions covered per iteration
+                constexpr int IT = TL / (GPI * P);
+                const uint32_t tq = threadIdx.x % VT, lg = threadIdx.x / VT;
+                const uint32_t t0 = k0 + tq * N;
+                const bool fwd = a.tstride[0] > 0;
+                const T* src = xg + (fwd ? (int64_t)t0 : -(int64_t)(t0 + N - 1));
+                rt_u32x4 grp[IT][P];
+#pragma unroll
+                for (int i = 0; i < IT; ++i) {
+#pragma unroll
+                    for (int p = 0; p < P; ++p) {
+                        const uint32_t col = min(l0 + (lg + i * GPI) * P + p, a.L - 1);
+                        if (t0 < a.K) {                        // K is a multiple of N on this path
+                            const rt_u32x4* q4 = reinterpret_cast<const rt_u32x4*>(src + (int64_t)col * a.istride[0]);
+                            grp[i][p] = a.nt_xt ? rt_ld16_nt(q4) : rt_ld16(q4);
+                        } else {
+                            grp[i][p] = rt_u32x4{0, 0, 0, 0};
+                        }
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < IT; ++i) {
+                    const uint32_t colw = (lg + i * GPI) * P;
+                    auto put = [&](int j, uint32_t w) {       // word of the P columns at element j of the loaded vectors
+                        *reinterpret_cast<uint32_t*>(&tile[tq * N + (fwd ? j : N - 1 - j)][colw]) = w;
+                    };
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        if constexpr (P == 2) {
+                            put(2 * k, __builtin_amdgcn_perm(grp[i][1][k], grp[i][0][k], 0x05040100u));
+                            put(2 * k + 1, __builtin_amdgcn_perm(grp[i][1][k], grp[i][0][k], 0x07060302u));
+                        } else {
+                            const uint32_t p0 = __builtin_amdgcn_perm(grp[i][1][k], grp[i][0][k], 0x05010400u);   // a0 b0 a1 b1
+                            const uint32_t p1 = __builtin_amdgcn_perm(grp[i][1][k], grp[i][0][k], 0x07030602u);   // a2 b2 a3 b3
+                            const uint32_t q0 = __builtin_amdgcn_perm(grp[i][3][k], grp[i][2][k], 0x05010400u);   // c0 d0 c1 d1
+                            const uint32_t q1 = __builtin_amdgcn_perm(grp[i][3][k], grp[i][2][k], 0x07030602u);   // c2 d2 c3 d3
+                            put(4 * k, __builtin_amdgcn_perm(q0, p0, 0x05040100u));
+                            put(4 * k + 1, __builtin_amdgcn_perm(q0, p0, 0x07060302u));
+                            put(4 * k + 2, __builtin_amdgcn_perm(q1, p1, 0x05040100u));
+                            put(4 * k + 3, __builtin_amdgcn_perm(q1, p1, 0x07060302u));
+                        }
+                    }
+                }
+            } else if constexpr (VG) {
                 // 16-byte loads along dim t: 8 lanes cover one 128-byte line of 4-byte elements, a wave instruction covers 8
                 // tile rows; the N elements of a vector go to N different tile rows, one LDS write each
-                constexpr int VT = kTK / N;                    // vectors per tile row along t
+                constexpr int VT = TK / N;                     // vectors per tile row along t
                 constexpr int LPI = kTBlock / VT;              // inner-dim positions covered per iteration
                 constexpr int IT = TL / LPI;
                 const uint32_t tq = threadIdx.x % VT, ls = threadIdx.x / VT;
@@ -128,8 +191,8 @@ __global__ __launch_bounds__(kTBlock) void bin_tile_kernel(const T* xt, const T*
             } else {
                 // element loads with lanes along dim t (32 consecutive lanes read one 128-byte line of 4-byte elements); each
                 // lane collects the N elements of one 16-byte group of a tile row and writes the group with one LDS store
-                const uint32_t tk = threadIdx.x % kTK, grp0 = threadIdx.x / kTK;
-                constexpr int kGroups = RT_WAVE / (kTBlock / kTK);                 // 64 groups per row / 8 rows of lanes = 8
+                const uint32_t tk = threadIdx.x % TK, grp0 = threadIdx.x / TK;
+                constexpr int kGroups = LPR / (kTBlock / TK);                      // groups per tile row / rows of lanes = 8
                 constexpr int kBatch = sizeof(T) >= 4 ? 4 : 1;                     // groups in flight per lane
                 const T* src = xg + (int64_t)min(k0 + tk, a.K - 1) * a.tstride[0];
 #pragma unroll 1
@@ -137,13 +200,13 @@ __global__ __launch_bounds__(kTBlock) void bin_tile_kernel(const T* xt, const T*
                     Vec16<T> grp[kBatch];
 #pragma unroll
                     for (int i = 0; i < kBatch; ++i) {
-                        const uint32_t col = l0 + (grp0 + (i0 + i) * (kTBlock / kTK)) * N;
+                        const uint32_t col = l0 + (grp0 + (i0 + i) * (kTBlock / TK)) * N;
 #pragma unroll
                         for (int j = 0; j < N; ++j) grp[i].e[j] = src[(int64_t)min(col + j, a.L - 1) * a.istride[0]];
                     }
 #pragma unroll
                     for (int i = 0; i < kBatch; ++i)
-                        *reinterpret_cast<Vec16<T>*>(&tile[tk][(grp0 + (i0 + i) * (kTBlock / kTK)) * N]) = grp[i];
+                        *reinterpret_cast<Vec16<T>*>(&tile[tk][(grp0 + (i0 + i) * (kTBlock / TK)) * N]) = grp[i];
                 }
             }
             __syncthreads();
@@ -152,10 +215,10 @@ __global__ __launch_bounds__(kTBlock) void bin_tile_kernel(const T* xt, const T*
         T* drow = dp + (int64_t)g * a.gstride[2];
         if (full_vec) {
 #pragma unroll
-            for (int i = 0; i < kTRows; ++i) {
-                const uint32_t kk = wv + i * kTWaves;
+            for (int i = 0; i < kTSteps; ++i) {
+                const uint32_t kk = krow + i * kTWaves * RPI;
                 if (k0 + kk < a.K) {
-                    const Vec16<T> xv = *reinterpret_cast<const Vec16<T>*>(&tile[kk][lane * N]);
+                    const Vec16<T> xv = *reinterpret_cast<const Vec16<T>*>(&tile[kk][(lane % LPR) * N]);
                     Vec16<T> out;
                     if (x_left) { out = xv; bin_apply_vec<OP, T>(out, ov[i]); }
                     else { out = ov[i]; bin_apply_vec<OP, T>(out, xv); }
@@ -165,8 +228,8 @@ __global__ __launch_bounds__(kTBlock) void bin_tile_kernel(const T* xt, const T*
         } else {
             // ragged end of a row: element accesses
             const T* orow = xo + (int64_t)g * a.gstride[1];
-            for (int i = 0; i < kTRows; ++i) {
-                const uint32_t kk = wv + i * kTWaves;
+            for (int i = 0; i < kTSteps; ++i) {
+                const uint32_t kk = krow + i * kTWaves * RPI;
                 if (k0 + kk < a.K) {
                     for (uint32_t cc = c; cc < a.L; ++cc) {
                         T xe = tile[kk][cc - l0];
@@ -188,8 +251,8 @@ template <class T, int OP>
 bool tile_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* l, const T* r, T* d, int32_t* status) {
     constexpr int64_t N = 16 / sizeof(T);
     const int rank = dsc.rank;
-    // rows shorter than a quarter of the tile's 64 * N columns would leave most lanes of every wave idle
-    if (!(rank >= 2 && count < (1ull << 31) && dsc.stride[2][rank - 1] == 1 && dsc.shape[rank - 1] >= 16 * N && vec_ok<T>(d, dsc, 2))) return false;
+    // rows shorter than a quarter of the tile's columns would leave most lanes of every wave idle
+    if (!(rank >= 2 && count < (1ull << 31) && dsc.stride[2][rank - 1] == 1 && dsc.shape[rank - 1] >= TileGeom<T>::TL / 4 && vec_ok<T>(d, dsc, 2))) return false;
     auto transposed_dim = [&](int o) -> int {
         int64_t is = dsc.stride[o][rank - 1];
         if (is == 0 || is == 1) return -1;
@@ -241,8 +304,8 @@ bool tile_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* l, const 
         a.nouter++;
     }
     for (int k = a.nouter; k < RT_MAX_RANK; ++k) { a.oshape[k] = 1; a.odiv[k] = make_fastdiv(1); }
-    const uint32_t TL = RT_WAVE * (uint32_t)N;
-    a.ktiles = (a.K + kTK - 1) / kTK;
+    const uint32_t TL = TileGeom<T>::TL, TK = TileGeom<T>::TK;
+    a.ktiles = (a.K + TK - 1) / TK;
     a.ltiles = (a.L + TL - 1) / TL;
     // loop-dim steps per block: the gathered tile is reused for all of them; keep enough blocks to fill the chip
     uint32_t gchunk = a.G;
@@ -262,7 +325,7 @@ bool tile_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* l, const 
         const int64_t ts = dsc.stride[xt][tdim];
         // every vector starts at (base + multiples of N) for an ascending dim t, and ends there for a descending one
         const T* first = ts > 0 ? xbase : xbase - (N - 1);
-        bool ok = (reinterpret_cast<uintptr_t>(first) & 15) == 0 && (a.K % (uint32_t)N) == 0 && kTK % N == 0;
+        bool ok = (reinterpret_cast<uintptr_t>(first) & 15) == 0 && (a.K % (uint32_t)N) == 0 && TK % (uint32_t)N == 0;
         bool xstream = true;
         for (int k = 0; k < rank; ++k) {
             if (k != tdim) ok = ok && mult_of(dsc.stride[xt][k], N);

@@ -620,7 +620,7 @@ def test_gather_transposed_views(hip, dtype):
     """Row-major copy (`owned()` / `contiguous()`) of permuted, reversed and stepped views large enough for the
     LDS-transpose copy kernel, with ragged tile edges."""
     rng = np.random.default_rng(17)
-    for shape in [(64, 257), (3, 40, 70), (2, 5, 33, 130), (4, 17, 1030), (100, 36), (2, 3, 16, 16), (7, 300, 9)]:
+    for shape in [(64, 257), (3, 40, 70), (2, 5, 33, 130), (4, 17, 1030), (100, 36), (2, 3, 16, 16), (7, 300, 9), (48, 2100), (2, 32, 1040), (160, 520)]:
         r = len(shape)
         vals = rand_values(dtype, int(np.prod(shape)), rng)
         o, g = OTensor.from_buf(dtype, vals, list(shape)), G(hip, dtype, vals, list(shape))
@@ -770,7 +770,7 @@ def test_broadcast_with_transposed_operand(hip, dtype):
     """One input is a permuted (and possibly reversed / strided) view whose unit-stride dim is not the output's inner dim:
     the LDS-transpose tile kernel.  Ragged tile edges, both operand positions, broadcast and in-place forms."""
     rng = np.random.default_rng(zlib.crc32(dtype.encode()))
-    shapes = [(3, 40, 70), (2, 5, 33, 130), (64, 257), (1, 100, 36), (4, 17, 1030), (2, 3, 16, 16)]
+    shapes = [(3, 40, 70), (2, 5, 33, 130), (64, 257), (1, 100, 36), (4, 17, 1030), (2, 3, 16, 16), (48, 2100), (2, 32, 1040), (160, 520)]
     for shape in shapes:
         r = len(shape)
         perm = list(range(r)); perm[-1], perm[-2] = perm[-2], perm[-1]
