@@ -27,7 +27,7 @@ PEAK_HBM = 8.0e12   # bytes/s, MI355X HBM3E
 # HBM bytes per launch of the config-3 broadcast-add kernel, from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE, each
 # scaled by what the same counter reads for the 1 GiB copy kernel (x2.000 and x1.000); see
 # profiles/bin_rows_kernel_config3_broadcast_add.txt.  Algorithmic bytes are 2181300224: nothing is re-read.
-MEASURED_TRAFFIC_C3A = 2181169159
+MEASURED_TRAFFIC_C3A = 2181192501
 
 
 def row_major(shape):

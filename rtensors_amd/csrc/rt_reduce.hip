@@ -623,6 +623,10 @@ int32_t rows_stage(rt_ctx* ctx, const T* src, T* out, uint64_t rows, uint64_t R,
         return RT_OK;
     }
     // block per (row, segment); split long rows when there are too few of them
+    // The first-stage launches ask for kRtFourBlocksLds bytes of LDS they never touch, which holds a CU to four resident blocks
+    // instead of eight: fewer concurrent streams keep more DRAM pages open.  1 GiB f32: full sum 0.167 -> 0.159 ms, sum and max
+    // over rows of 32768 0.159 -> 0.158 and 0.163 -> 0.158 ms.  (The same cap on the one-vector-per-lane elementwise kernels,
+    // which need every wave slot to cover latency, and on the wave-per-row kernel only lost time.)
     uint32_t splits = 1;
     if (allow_split && rows < want) {
         const uint64_t min_seg = 16384;                       // elements; below this a split is not worth a second pass
@@ -634,7 +638,7 @@ int32_t rows_stage(rt_ctx* ctx, const T* src, T* out, uint64_t rows, uint64_t R,
     }
     if (rows * splits >= (1ull << 31)) return rt_fail(RT_E_INVALID, "reduce: too many rows for one launch");
     if (splits == 1) {
-        hipLaunchKernelGGL((reduce_rows_block_kernel<OP, T>), dim3((unsigned)rows), dim3(kBlock), 0, s, src, out, R, 1u, R, count, 1);
+        hipLaunchKernelGGL((reduce_rows_block_kernel<OP, T>), dim3((unsigned)rows), dim3(kBlock), kRtFourBlocksLds, s, src, out, R, 1u, R, count, 1);
         RT_HIP(hipGetLastError());
         return RT_OK;
     }
@@ -645,7 +649,7 @@ int32_t rows_stage(rt_ctx* ctx, const T* src, T* out, uint64_t rows, uint64_t R,
     void* scratch = nullptr;
     RT_TRY(rt_scratch(ctx, (size_t)(rows * splits) * sizeof(T), &scratch));
     T* part = (T*)scratch;
-    hipLaunchKernelGGL((reduce_rows_block_kernel<OP, T>), dim3((unsigned)(rows * splits)), dim3(kBlock), 0, s, src, part, R, splits, seglen, count, 0);
+    hipLaunchKernelGGL((reduce_rows_block_kernel<OP, T>), dim3((unsigned)(rows * splits)), dim3(kBlock), kRtFourBlocksLds, s, src, part, R, splits, seglen, count, 0);
     RT_HIP(hipGetLastError());
     // second stage: each row of `splits` partials -> one output (mean divides by the original count)
     if (splits < 64) {

@@ -628,7 +628,7 @@ int32_t rows_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t rows
     }
     if (rows * splits >= (1ull << 31)) return too_many();
     if (splits == 1) {
-        hipLaunchKernelGGL((st_rows_block_kernel<S, T>), dim3((unsigned)rows), dim3(kBlock), 0, s, src, out, (S*)nullptr, R, 1u, R, flags);
+        hipLaunchKernelGGL((st_rows_block_kernel<S, T>), dim3((unsigned)rows), dim3(kBlock), kRtFourBlocksLds, s, src, out, (S*)nullptr, R, 1u, R, flags);
         RT_HIP(hipGetLastError());
         return RT_OK;
     }
@@ -639,7 +639,7 @@ int32_t rows_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t rows
     void* scratch = nullptr;
     RT_TRY(rt_scratch(ctx, (size_t)(rows * splits) * sizeof(S), &scratch));
     S* part = (S*)scratch;
-    hipLaunchKernelGGL((st_rows_block_kernel<S, T>), dim3((unsigned)(rows * splits)), dim3(kBlock), 0, s, src, out, part, R, splits, seglen, flags);
+    hipLaunchKernelGGL((st_rows_block_kernel<S, T>), dim3((unsigned)(rows * splits)), dim3(kBlock), kRtFourBlocksLds, s, src, out, part, R, splits, seglen, flags);
     RT_HIP(hipGetLastError());
     hipLaunchKernelGGL((st_merge_wave_kernel<S>), dim3((unsigned)((rows + kWaves - 1) / kWaves)), dim3(kBlock), 0, s, part, out, rows, splits,
                        (uint64_t)splits, (uint64_t)1, flags);
