@@ -4,6 +4,7 @@
 // layer builds with a plain host compiler, the way a Rust FFI binding would.
 #pragma once
 
+#include <limits>
 #include <cstring>
 #include <memory>
 #include <string>
@@ -43,6 +44,21 @@ struct Scalar {
             case RT_U128: return of<u128>((u128)x); case RT_I128: return of<i128>((i128)x);
             case RT_F32: return of<float>((float)x); case RT_F64: return of<double>(x);
             case RT_BOOL: return of<boolean>(boolean{(uint8_t)(x != 0)});
+        }
+        throw TensorError(ErrorKind::UnsupportedOperation, "unknown dtype code");
+    }
+    // T::MIN / T::MAX of the element type (core/value.rs:496-508, 703-704): the lowest / highest finite value for floats
+    static Scalar limit(int dtype, bool highest) {
+        switch (dtype) {
+            case RT_U8: return of<uint8_t>(highest ? UINT8_MAX : 0); case RT_I8: return of<int8_t>(highest ? INT8_MAX : INT8_MIN);
+            case RT_U16: return of<uint16_t>(highest ? UINT16_MAX : 0); case RT_I16: return of<int16_t>(highest ? INT16_MAX : INT16_MIN);
+            case RT_U32: return of<uint32_t>(highest ? UINT32_MAX : 0); case RT_I32: return of<int32_t>(highest ? INT32_MAX : INT32_MIN);
+            case RT_U64: return of<uint64_t>(highest ? UINT64_MAX : 0); case RT_I64: return of<int64_t>(highest ? INT64_MAX : INT64_MIN);
+            case RT_U128: return of<u128>(highest ? ~(u128)0 : (u128)0);
+            case RT_I128: return of<i128>(highest ? (i128)(~(u128)0 >> 1) : -(i128)(~(u128)0 >> 1) - 1);
+            case RT_F32: return of<float>(highest ? std::numeric_limits<float>::max() : std::numeric_limits<float>::lowest());
+            case RT_F64: return of<double>(highest ? std::numeric_limits<double>::max() : std::numeric_limits<double>::lowest());
+            case RT_BOOL: return of<boolean>(boolean{(uint8_t)(highest ? 1 : 0)});
         }
         throw TensorError(ErrorKind::UnsupportedOperation, "unknown dtype code");
     }

@@ -92,6 +92,13 @@ int rth_zeros(void* backend, int dtype, int rank, const uint64_t* shape, void** 
 int rth_ones(void* backend, int dtype, int rank, const uint64_t* shape, void** out) {
     return guarded([&] { *out = new Tensor(Tensor::ones(*(Hip*)backend, dtype, Shape(shape, shape + rank))); });
 }
+int rth_limit(void* backend, int dtype, int highest, int rank, const uint64_t* shape, void** out) {
+    return guarded([&] {
+        Shape sh(shape, shape + rank);
+        *out = new Tensor(highest ? Tensor::max(*(Hip*)backend, dtype, sh) : Tensor::min(*(Hip*)backend, dtype, sh));
+    });
+}
+int rth_into_dtype(void* t, int dtype, void** out) { return guarded([&] { *out = new Tensor(((Tensor*)t)->into_dtype(dtype)); }); }
 void rth_free(void* t) { delete (Tensor*)t; }
 
 int rth_info(void* t, int* rank, uint64_t* shape, int64_t* strides, uint64_t* offset, int* dtype, int* is_view, int* contiguous, uint64_t* buf_len) {

@@ -43,6 +43,20 @@ class Tensor {
         return Tensor(backend, backend.alloc(dtype, m.size()), m);
     }
     static Tensor ones(const Hip& backend, int dtype, const Shape& shape) { return full(backend, dtype, shape, Scalar::from_double(dtype, 1.0)); }
+    // TensorBase::max / ::min (core/primitives.rs:490-506): every element T::MAX / T::MIN, filled on the device
+    static Tensor max(const Hip& backend, int dtype, const Shape& shape) { return full(backend, dtype, shape, Scalar::limit(dtype, true)); }
+    static Tensor min(const Hip& backend, int dtype, const Shape& shape) { return full(backend, dtype, shape, Scalar::limit(dtype, false)); }
+    // TensorBase::scalar / ::column / ::row (core/primitives.rs:418-444): shapes [], [n] and [1, n]
+    static Tensor scalar(const Hip& backend, const Scalar& v) { return from_buf(backend, v.dtype, v.bytes, 1, Shape{}); }
+    static Tensor column(const Hip& backend, int dtype, const void* host, uint64_t n) { return from_buf(backend, dtype, host, n, Shape{n}); }
+    static Tensor row(const Hip& backend, int dtype, const void* host, uint64_t n) { return from_buf(backend, dtype, host, n, Shape{1, n}); }
+    // TensorBase::into_dtype (core/primitives.rs:527-539): a new buffer of meta.size() elements of the other type, the whole
+    // source buffer converted into it (SizeMismatch when the two lengths differ, as for a view of part of a buffer), same meta
+    Tensor into_dtype(int new_dtype) const {
+        Buf nb = backend_->alloc_uninit(new_dtype, meta_.size());
+        backend_->convert(*buf_, *nb);
+        return Tensor(*backend_, nb, meta_);
+    }
 
     // ---- accessors ------------------------------------------------------------------------------------------------------
     const MetaTensor& meta() const { return meta_; }
@@ -333,6 +347,12 @@ class TensorBase : public Tensor {
     }
     static TensorBase zeros(const Hip& b, const Shape& s) { return TensorBase(Tensor::zeros(b, dtype_of<T>::value, s)); }
     static TensorBase ones(const Hip& b, const Shape& s) { return TensorBase(Tensor::ones(b, dtype_of<T>::value, s)); }
+    static TensorBase max(const Hip& b, const Shape& s) { return TensorBase(Tensor::max(b, dtype_of<T>::value, s)); }
+    static TensorBase min(const Hip& b, const Shape& s) { return TensorBase(Tensor::min(b, dtype_of<T>::value, s)); }
+    static TensorBase scalar(const Hip& b, T v) { return TensorBase(Tensor::scalar(b, Scalar::of<T>(v))); }
+    static TensorBase column(const Hip& b, const std::vector<T>& v) { return TensorBase(Tensor::column(b, dtype_of<T>::value, v.data(), v.size())); }
+    static TensorBase row(const Hip& b, const std::vector<T>& v) { return TensorBase(Tensor::row(b, dtype_of<T>::value, v.data(), v.size())); }
+    template <class N> TensorBase<N> into_dtype() const { return TensorBase<N>(Tensor::into_dtype(dtype_of<N>::value)); }
     std::vector<T> to_vec() const {
         std::vector<T> out(size());
         to_host(out.data());

@@ -161,6 +161,32 @@ class Tensor:
         code = DTYPE_BY_NAME[dtype] if isinstance(dtype, str) else dtype
         p = C.c_void_p(); _ck(_h.rth_ones(backend._p, code, len(shape), _u64(shape), C.byref(p))); return Tensor(p, backend)
 
+    @staticmethod
+    def max_of(backend, dtype, shape):
+        """`TensorBase::max(shape)` (core/primitives.rs:490-495): every element T::MAX."""
+        code = DTYPE_BY_NAME[dtype] if isinstance(dtype, str) else dtype
+        p = C.c_void_p(); _ck(_h.rth_limit(backend._p, code, 1, len(shape), _u64(shape), C.byref(p))); return Tensor(p, backend)
+
+    @staticmethod
+    def min_of(backend, dtype, shape):
+        """`TensorBase::min(shape)` (core/primitives.rs:501-506): every element T::MIN."""
+        code = DTYPE_BY_NAME[dtype] if isinstance(dtype, str) else dtype
+        p = C.c_void_p(); _ck(_h.rth_limit(backend._p, code, 0, len(shape), _u64(shape), C.byref(p))); return Tensor(p, backend)
+
+    @staticmethod
+    def scalar(backend, dtype, value): return Tensor.from_buf(backend, dtype, [value], [])            # core/primitives.rs:418-420
+
+    @staticmethod
+    def column(backend, dtype, values): return Tensor.from_buf(backend, dtype, values, [len(values)])  # core/primitives.rs:428-432
+
+    @staticmethod
+    def row(backend, dtype, values): return Tensor.from_buf(backend, dtype, values, [1, len(values)])  # core/primitives.rs:440-444
+
+    def into_dtype(self, dtype):
+        """`TensorBase::into_dtype::<N>()` (core/primitives.rs:527-539): the whole buffer converted, same meta."""
+        code = DTYPE_BY_NAME[dtype] if isinstance(dtype, str) else dtype
+        return self._new(_h.rth_into_dtype, C.c_int(code))
+
     def _info(self):
         r, sh, st, off = _meta_out()
         dt, iv, cg, bl = C.c_int(0), C.c_int(0), C.c_int(0), C.c_uint64(0)

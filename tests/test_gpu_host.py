@@ -137,6 +137,36 @@ def test_statistic_and_index_reductions_through_host_layer(T, be):
     assert np.array_equal(gv.argmax_at(1).to_numpy().reshape(xv.shape[0], xv.shape[2]), xv.argmax(axis=1))
 
 
+def test_constructors_and_into_dtype(T, be):
+    """`scalar`, `column`, `row`, `max`, `min`, `zeros`, `ones` (core/primitives.rs:418-506; the reference's tests core/mod.rs:839-867 hold
+    the shapes) and `into_dtype` (core/primitives.rs:527-539: whole buffer converted, meta kept, a partial view refused)."""
+    col, row, sc = T.Tensor.column(be, "i32", [1, 2, 3]), T.Tensor.row(be, "i32", [1, 2, 3]), T.Tensor.scalar(be, "i32", 42)
+    assert list(col.shape) == [3] and [col.get([i]) for i in range(3)] == [1, 2, 3]                       # core/mod.rs:839-845
+    assert list(row.shape) == [1, 3] and [row.get([0, i]) for i in range(3)] == [1, 2, 3]                 # core/mod.rs:848-856
+    assert list(sc.shape) == [] and sc.get([]) == 42                                                       # core/mod.rs:859-867
+    for name in ("u8", "i8", "u16", "i16", "u32", "i32", "u64", "i64"):
+        info = np.iinfo(cpu.NP_DTYPE[cpu.DTYPE_BY_NAME[name]])
+        assert T.Tensor.max_of(be, name, [2, 3]).to_numpy().reshape(-1).tolist() == [info.max] * 6
+        assert T.Tensor.min_of(be, name, [5]).to_numpy().reshape(-1).tolist() == [info.min] * 5
+    for name in ("f32", "f64"):
+        info = np.finfo(cpu.NP_DTYPE[cpu.DTYPE_BY_NAME[name]])
+        assert T.Tensor.max_of(be, name, [4]).to_numpy().tolist() == [info.max] * 4 and T.Tensor.min_of(be, name, [4]).to_numpy().tolist() == [info.min] * 4
+    assert T.Tensor.max_of(be, "bool", [3]).to_numpy().astype(np.uint8).tolist() == [1, 1, 1]
+    assert T.Tensor.zeros(be, "f64", [2, 2]).to_numpy().reshape(-1).tolist() == [0.0] * 4 and T.Tensor.ones(be, "u16", [3]).to_numpy().tolist() == [1, 1, 1]
+    x = np.array([0.4, 0.5, 1.5, -0.5, -1.5, 300.7, -2.5, 1e10, -1e10, 7.0, np.nan, 2.5], dtype=np.float32)
+    t = T.Tensor.from_buf(be, "f32", x, [3, 4])
+    as_i32 = t.into_dtype("i32")
+    assert as_i32.dtype == cpu.I32 and list(as_i32.shape) == [3, 4] and list(as_i32.strides) == [4, 1]
+    assert as_i32.to_numpy().reshape(-1).tolist() == [0, 1, 2, -1, -2, 301, -3, 2 ** 31 - 1, -2 ** 31, 7, 0, 3]   # round half away from zero, saturate, NaN -> 0
+    assert t.into_dtype("f64").to_numpy().reshape(-1).tobytes() == x.astype(np.float64).tobytes()
+    tv = t.transpose()                                                  # a view of the whole buffer keeps its meta
+    tvi = tv.into_dtype("i64")
+    assert list(tvi.shape) == [4, 3] and list(tvi.strides) == [1, 4] and tvi.get([1, 2]) == 7
+    with pytest.raises(T.TensorError) as e:                             # a view of part of the buffer: size != buffer length
+        t.slice(0, T.Slice(0, 2, 1)).into_dtype("i32")
+    assert e.value.kind == "SizeMismatch"
+
+
 def test_out_of_scope_methods_report_unsupported(T, be):
     g = T.Tensor.from_buf(be, "i32", np.ones(4, np.int32), [4])
     with pytest.raises(T.TensorError) as e:
