@@ -222,6 +222,19 @@ def compute_squeezed_parameters(shape, strides, dim: Optional[int]):
     return new_shape, new_strides
 
 
+def compute_view_as_parameters(meta: "MetaTensor", new_shape):
+    """core/tensor.rs:328-355 (`view_as_inner`): the layout must pass the relaxed contiguity check and the element counts must agree;
+    the result has the new shape's row-major strides and the same offset (whatever the signs of the old strides were)."""
+    if not meta.is_contiguous():
+        raise TensorError("ContiguityError", "cannot view_as a non-contiguous tensor")
+    n = 1
+    for d in new_shape:
+        n *= d
+    if n != meta.size():
+        raise TensorError("InvalidShape", f"invalid size {n} for initial size {meta.size()}")
+    return list(new_shape), shape_to_stride(list(new_shape)), meta.offset
+
+
 def compute_broadcasted_params(a: MetaTensor, b: MetaTensor):
     """ops/broadcast/mod.rs:13-55: (out_shape, a_strides, b_strides)."""
     sa, sb = list(a.shape), list(b.shape)

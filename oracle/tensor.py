@@ -15,7 +15,7 @@ import numpy as np
 
 from . import cpu
 from .meta import (MetaTensor, Slice, TensorError, compute_broadcasted_params, compute_permuted_parameters, contiguity_type,
-                   compute_sliced_parameters, compute_squeezed_parameters, compute_unsqueezed_parameters,
+                   compute_sliced_parameters, compute_squeezed_parameters, compute_unsqueezed_parameters, compute_view_as_parameters,
                    logical_to_buffer_idx, reduction_output_meta, shape_to_stride)
 
 
@@ -78,6 +78,16 @@ class OTensor:
     def squeeze(self) -> "OTensor":
         shape, strides = compute_squeezed_parameters(self.meta.shape, self.meta.strides, None)
         return self._view(shape, strides, self.meta.offset)
+
+    def view_as(self, shape) -> "OTensor":
+        """core/tensor.rs:120-122, 328-355: reinterpret a contiguous layout under another shape (no copy)."""
+        return self._view(*compute_view_as_parameters(self.meta, list(shape)))
+
+    def reshape(self, shape) -> "OTensor":
+        """core/tensor.rs:238-243: `contiguous()` then the `view_as` meta on the new owner."""
+        c = self.contiguous()
+        sh, st, off = compute_view_as_parameters(c.meta, list(shape))
+        return OTensor(c.dtype, c.buf, MetaTensor(sh, st, off))
 
     # ---- element access: core/tensor.rs:535-541, 665-682; backend/cpu.rs:185-207 -----------------------------------
     def get(self, idx):

@@ -119,6 +119,12 @@ int rth_unsqueeze(void* t, uint64_t dim, void** out) { return guarded([&] { *out
 int rth_squeeze(void* t, int64_t dim, void** out) {
     return guarded([&] { *out = new Tensor(dim < 0 ? ((Tensor*)t)->squeeze() : ((Tensor*)t)->squeeze_at((size_t)dim)); });
 }
+int rth_view_as(void* t, int rank, const uint64_t* shape, void** out) {
+    return guarded([&] { *out = new Tensor(((Tensor*)t)->view_as(Shape(shape, shape + rank))); });
+}
+int rth_reshape(void* t, int rank, const uint64_t* shape, void** out) {
+    return guarded([&] { *out = new Tensor(((Tensor*)t)->reshape(Shape(shape, shape + rank))); });
+}
 int rth_owned(void* t, void** out) { return guarded([&] { *out = new Tensor(((Tensor*)t)->owned()); }); }
 int rth_contiguous(void* t, void** out) { return guarded([&] { *out = new Tensor(((Tensor*)t)->contiguous()); }); }
 

@@ -16,7 +16,8 @@ namespace rt {
 // TensorError (core/tensor.rs:11-53); HipError stands where the cfg-gated CudaError stands.
 enum class ErrorKind {
     InvalidShape, InvalidDim, IdxOutOfBounds, WrongDims, BroadcastError, SizeMismatch, UnsupportedOperation, GradError, HipError,
-    Panic   // where the reference's operator sugar unwraps / panics (e.g. in-place op that would have to grow the lhs)
+    Panic,  // where the reference's operator sugar unwraps / panics (e.g. in-place op that would have to grow the lhs)
+    ContiguityError
 };
 
 inline const char* kind_name(ErrorKind k) {
@@ -31,6 +32,7 @@ inline const char* kind_name(ErrorKind k) {
         case ErrorKind::GradError: return "GradError";
         case ErrorKind::HipError: return "HipError";
         case ErrorKind::Panic: return "Panic";
+        case ErrorKind::ContiguityError: return "ContiguityError";
     }
     return "?";
 }
@@ -232,6 +234,26 @@ inline MetaTensor compute_squeezed_parameters(const MetaTensor& m, std::optional
         out.shape.erase(out.shape.begin() + (long)d);
         out.strides.erase(out.strides.begin() + (long)d);
     }
+    return out;
+}
+
+// core/tensor.rs:328-355 (`view_as_inner`): a layout that passes the relaxed contiguity check is given another shape of the same
+// element count, with that shape's row-major strides and the same offset.  The reference does this whatever the signs of the old
+// strides are, which for a reversed view (|stride| contiguous, offset at its first element = the run's last address) describes
+// memory past the run.  Here a view whose non-singleton strides are all negative gets the negated row-major strides, so that
+// element k of the new shape is still element k of the old one; mixed signs cannot be expressed by strides and are refused.
+inline MetaTensor compute_view_as_parameters(const MetaTensor& m, const Shape& shape) {
+    if (!m.is_contiguous()) throw TensorError(ErrorKind::ContiguityError, "Cannot view_as non contiguous tensor");
+    uint64_t n = 1;
+    for (uint64_t d : shape) n *= d;
+    if (n != m.size()) throw TensorError(ErrorKind::InvalidShape, "Invalid size " + std::to_string(n) + " for initial shape " + std::to_string(m.size()));
+    bool neg = false, pos = false;
+    for (size_t d = 0; d < m.shape.size(); ++d)
+        if (m.shape[d] > 1) (m.strides[d] < 0 ? neg : pos) = true;
+    if (neg && pos && n > 0) throw TensorError(ErrorKind::ContiguityError, "Cannot view_as a view reversed along some of its dims only");
+    MetaTensor out = MetaTensor::row_major(shape);
+    out.offset = m.offset;
+    if (neg) for (auto& st : out.strides) st = -st;
     return out;
 }
 

@@ -312,6 +312,14 @@ class Tensor {
         return backend_->equal(*a.buf_, *b.buf_);
     }
 
+    // AsView::view_as (core/tensor.rs:120-122, 328-355): another shape over the same contiguous elements, no copy
+    Tensor view_as(const Shape& shape) const { return with_meta(compute_view_as_parameters(meta_, shape)); }
+    // AsTensor::reshape (core/tensor.rs:238-243): contiguous() and then the view_as meta on the new owner
+    Tensor reshape(const Shape& shape) const {
+        Tensor c = contiguous();
+        c.meta_ = compute_view_as_parameters(c.meta_, shape);
+        return c;
+    }
     // metadata rewrite used by the autograd step (grad/backwards.rs:516-538 mutates `grad.meta` in place)
     void set_meta(const MetaTensor& m) { meta_ = m; }
 

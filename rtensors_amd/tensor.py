@@ -21,7 +21,7 @@ for _n in ("rth_backend_destroy", "rth_free"):
     getattr(_h, _n).argtypes = [C.c_void_p]
 
 _KINDS = ["InvalidShape", "InvalidDim", "IdxOutOfBounds", "WrongDims", "BroadcastError", "SizeMismatch", "UnsupportedOperation",
-          "GradError", "HipError", "Panic"]
+          "GradError", "HipError", "Panic", "ContiguityError"]
 MAX_RANK = 128
 
 
@@ -218,6 +218,8 @@ class Tensor:
     def unsqueeze_at(self, d): return self._new(_h.rth_unsqueeze, C.c_uint64(d))
     def squeeze_at(self, d): return self._new(_h.rth_squeeze, C.c_int64(d))
     def squeeze(self): return self._new(_h.rth_squeeze, C.c_int64(-1))
+    def view_as(self, shape): return self._new(_h.rth_view_as, len(shape), _u64(shape))       # core/tensor.rs:120-122
+    def reshape(self, shape): return self._new(_h.rth_reshape, len(shape), _u64(shape))       # core/tensor.rs:238-243
     def owned(self): return self._new(_h.rth_owned)
     def contiguous(self): return self._new(_h.rth_contiguous)
 

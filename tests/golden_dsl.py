@@ -2,7 +2,7 @@
 
 A case is `inputs` (named row-major tensors), a `program` (one step per line: [result, op, operands...]) and
 `expect` entries.  The same case runs against any tensor implementation that offers the reference's surface
-(from_buf, slice, permute, transpose, unsqueeze_at, squeeze, + - * /, in-place forms, unary, reductions, matmul);
+(from_buf, slice, view_as, reshape, permute, transpose, unsqueeze_at, squeeze, + - * /, in-place forms, unary, reductions, matmul);
 `factory(dtype_name, values, shape)` creates an owned tensor, `TensorError` is that implementation's error type.
 """
 import json
@@ -48,6 +48,10 @@ def run_case(case, factory, SliceCls, ErrorCls):
                 env[dst] = env[args[0]].transpose()
             elif op == "unsqueeze":
                 env[dst] = env[args[0]].unsqueeze_at(args[1])
+            elif op == "view_as":
+                env[dst] = env[args[0]].view_as(args[1])
+            elif op == "reshape":
+                env[dst] = env[args[0]].reshape(args[1])
             elif op == "squeeze":
                 env[dst] = env[args[0]].squeeze() if len(args) == 1 else env[args[0]].squeeze_at(args[1])
             elif op in ("add", "sub", "mul", "div"):

@@ -6,7 +6,7 @@ from __future__ import annotations
 import numpy as np
 
 from oracle.meta import (MetaTensor, Slice, TensorError, compute_broadcasted_params, compute_permuted_parameters, contiguity_type,
-                         compute_sliced_parameters, compute_squeezed_parameters, compute_unsqueezed_parameters,
+                         compute_sliced_parameters, compute_squeezed_parameters, compute_unsqueezed_parameters, compute_view_as_parameters,
                          logical_to_buffer_idx, reduction_output_meta)
 from rtensors_amd import hip as H
 
@@ -57,6 +57,14 @@ class GTensor:
     def squeeze(self):
         shape, strides = compute_squeezed_parameters(self.meta.shape, self.meta.strides, None)
         return self._view(shape, strides, self.meta.offset)
+
+    def view_as(self, shape):
+        return self._view(*compute_view_as_parameters(self.meta, list(shape)))
+
+    def reshape(self, shape):
+        c = self.contiguous()
+        sh, st, off = compute_view_as_parameters(c.meta, list(shape))
+        return GTensor(c.backend, c.buf, MetaTensor(sh, st, off))
 
     def get(self, idx):
         return self.backend.read(self.buf, logical_to_buffer_idx(list(idx), self.meta.strides, self.meta.offset))

@@ -167,6 +167,40 @@ def test_constructors_and_into_dtype(T, be):
     assert e.value.kind == "SizeMismatch"
 
 
+def test_view_as_and_reshape(T, be):
+    """`view_as` (core/tensor.rs:328-355) and `reshape` (238-243) through the host layer: shared storage, the two error kinds, reshape of
+    permuted views, and the one place where the host layer departs from the reference: a fully reversed view keeps its element order."""
+    x = np.arange(24, dtype=np.int32)
+    t = T.Tensor.from_buf(be, "i32", x, [2, 3, 4])
+    v = t.view_as([6, 4])
+    assert list(v.shape) == [6, 4] and list(v.strides) == [4, 1] and np.array_equal(v.to_numpy(), x.reshape(6, 4))
+    v.set([5, 3], 99)                                                    # same storage
+    assert t.get([1, 2, 3]) == 99
+    v.set([5, 3], 23)
+    row = t.slice(0, 1).slice(0, 2)                                      # contiguous run at an offset
+    assert np.array_equal(row.view_as([2, 2]).to_numpy(), x.reshape(2, 3, 4)[1, 2].reshape(2, 2)) and row.view_as([2, 2]).offset == 20
+    with pytest.raises(T.TensorError) as e:
+        t.transpose().view_as([24])
+    assert e.value.kind == "ContiguityError"
+    with pytest.raises(T.TensorError) as e:
+        t.view_as([5, 5])
+    assert e.value.kind == "InvalidShape"
+    r = t.transpose().reshape([6, 4])                                    # gathers first
+    assert not r._info()["is_view"]
+    assert np.array_equal(r.to_numpy(), x.reshape(2, 3, 4).transpose(2, 1, 0).reshape(6, 4)) and list(r.strides) == [4, 1]
+    assert np.array_equal(t.reshape([4, 6]).to_numpy(), x.reshape(4, 6))
+    flat = T.Tensor.from_buf(be, "i32", x, [24])
+    rev = flat.slice(0, T.Slice(None, None, -1))                         # |stride| contiguous, offset 23
+    rv = rev.view_as([4, 6])
+    assert list(rv.strides) == [-6, -1] and rv.offset == 23 and np.array_equal(rv.to_numpy(), x[::-1].reshape(4, 6))
+    assert np.array_equal(rev.reshape([2, 12]).to_numpy(), x[::-1].reshape(2, 12))
+    half = t.slice(2, T.Slice(None, None, -1))                           # reversed along the last dim only
+    with pytest.raises(T.TensorError) as e:
+        half.view_as([24])
+    assert e.value.kind == "ContiguityError"
+    assert np.array_equal(half.reshape([24]).to_numpy(), x.reshape(2, 3, 4)[:, :, ::-1].reshape(24))
+
+
 def test_out_of_scope_methods_report_unsupported(T, be):
     g = T.Tensor.from_buf(be, "i32", np.ones(4, np.int32), [4])
     with pytest.raises(T.TensorError) as e:
