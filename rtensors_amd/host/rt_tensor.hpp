@@ -83,6 +83,13 @@ class Tensor {
     Tensor unsqueeze_at(size_t dim) const { return with_meta(compute_unsqueezed_parameters(meta_, dim)); }
     Tensor squeeze_at(size_t dim) const { return with_meta(compute_squeezed_parameters(meta_, dim)); }
     Tensor squeeze() const { return with_meta(compute_squeezed_parameters(meta_, std::nullopt)); }
+    // TensorAccess::slice_at / ::unsqueeze (core/tensor.rs:443-445, 462-464)
+    Tensor slice_at(size_t dim, uint64_t at) const { return slice(dim, Slice::index(at)); }
+    Tensor unsqueeze() const { return unsqueeze_at(0); }
+    // the in-place metadata forms of an owner (core/primitives.rs:509-524)
+    void squeeze_inplace() { meta_ = compute_squeezed_parameters(meta_, std::nullopt); }
+    void unsqueeze_at_inplace(size_t dim) { meta_ = compute_unsqueezed_parameters(meta_, dim); }
+    void unsqueeze_inplace() { unsqueeze_at_inplace(0); }
 
     // ---- element access (core/tensor.rs:535-541, 665-688) ----------------------------------------------------------------------
     Scalar get(const std::vector<uint64_t>& idx) const { return backend_->read(*buf_, logical_to_buffer_idx(idx, meta_.strides, meta_.offset)); }
