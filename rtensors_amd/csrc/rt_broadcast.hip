@@ -93,7 +93,7 @@ __global__ __launch_bounds__(kRBlock) void bin_rows_kernel(const T* l, const T* 
         auto combine_store = [&](Raw x, Raw y, uint32_t g) {
             Vec16<T> xv = __builtin_bit_cast(Vec16<T>, x);
             bin_apply_vec<OP, T>(xv, __builtin_bit_cast(Vec16<T>, y));
-            rt_st16_nt(reinterpret_cast<Vec16<T>*>(d + od + (int64_t)g * a.gstride[2] + c), xv);
+            rt_st16u_nt<T>(d + od + (int64_t)g * a.gstride[2] + c, __builtin_bit_cast(rt_u32x4, xv));
         };
         Raw lh = {}, rh = {};                                   // operands that do not move along the loop dim
         if (l_fixed) lh = ldl(ol, false);
@@ -239,10 +239,10 @@ __global__ __launch_bounds__(kRBlock) void bin_flat_kernel(const T* l, const T* 
     if (v >= nvec) return;
     Vec16<T> x, y;
     const uint32_t L = a.shape[a.rank - 1];
-    if constexpr (LMODE == F_VEC) x = rt_ld16_nt(reinterpret_cast<const Vec16<T>*>(l) + v);
+    if constexpr (LMODE == F_VEC) x = __builtin_bit_cast(Vec16<T>, rt_ld16u<T>(l + (size_t)v * N, true));     // a run like dst, from any element
     if constexpr (LMODE == F_ROW) x = load_row_vec<T>(l, v * N, L, a.div[a.rank - 1]);
     if constexpr (OP != kOpCopy) {
-        if constexpr (RMODE == F_VEC) y = rt_ld16_nt(reinterpret_cast<const Vec16<T>*>(r) + v);
+        if constexpr (RMODE == F_VEC) y = __builtin_bit_cast(Vec16<T>, rt_ld16u<T>(r + (size_t)v * N, true));
         if constexpr (RMODE == F_ROW) y = load_row_vec<T>(r, v * N, L, a.div[a.rank - 1]);
     }
     if constexpr (LE || RE) {
@@ -391,7 +391,8 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
         if (tile_try<T, OP>(ctx, dsc, count, l, r, d, &status)) return status;
     }
 
-    // (2) rows: dst inner dim unit-stride, rows 16-byte aligned, everything indexable in 32 bits
+    // (2) rows: dst inner dim unit-stride (rows may start at any element: 16-byte accesses at element alignment), everything
+    // indexable in 32 bits
     // Rows whose pitch is not a whole number of 128-byte lines make every block of the row kernel start and end inside a line it
     // shares with its neighbours; when dst is one contiguous run and every input is either laid out like dst or constant along
     // the row (a per-row scalar), the flat kernel below writes whole aligned spans instead: (2^18, 1000) + (2^18, 1) f32 takes
@@ -433,19 +434,37 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
             }
         }
     }
-    if (rank >= 1 && !prefer_flat && count < (1ull << 31) && dsc.stride[2][rank - 1] == 1 && dsc.shape[rank - 1] >= 2 * N && vec_ok<T>(d, dsc, 2)) {
+    // dst rows that do not start on 16-byte boundaries (an odd row length, a column slice): when dst is one aligned contiguous run
+    // and every input is a run like dst, a repeated row or a single element, the flat kernel below keeps all of dst's stores
+    // aligned and is faster (65536 rows of 4095 f32 plus a row: 0.34 ms there, 0.46 ms here); with any other input the row kernel's
+    // unaligned vectors beat the flat kernel's element gathers (8192 x 32767 out of `m[:, 1:]` plus a row: 0.41 against 0.54 ms).
+    auto rows_aligned = [&](int o, const T* base) {
+        if ((reinterpret_cast<uintptr_t>(base + dsc.offset[o]) & 15) != 0) return false;
+        for (int k = 0; k < rank - 1; ++k)
+            if (!mult_of(dsc.stride[o][k], N)) return false;
+        return true;
+    };
+    auto repeated_row_or_element = [&](int o) {
+        for (int k = 0; k < rank - 1; ++k)
+            if (dsc.stride[o][k] != 0) return false;
+        return rank >= 1 && (dsc.stride[o][rank - 1] == 1 || dsc.stride[o][rank - 1] == 0);
+    };
+    bool flat_good = count >= (uint64_t)N && row_major_run(2) && (reinterpret_cast<uintptr_t>(d + dsc.offset[2]) & 15) == 0;
+    for (int o = 0; o < (OP == kOpCopy ? 1 : 2) && flat_good; ++o) flat_good = row_major_run(o) || repeated_row_or_element(o);
+    if (rank >= 1 && !prefer_flat && count < (1ull << 31) && dsc.stride[2][rank - 1] == 1 && dsc.shape[rank - 1] >= 2 * N &&
+        (rows_aligned(2, d) || !flat_good)) {
         RowArgs a;
         memset(&a, 0, sizeof(a));
         a.L = (uint32_t)dsc.shape[rank - 1];
         a.istride[0] = dsc.stride[0][rank - 1];
         a.istride[1] = dsc.stride[1][rank - 1];
-        auto mode = [&](int o, const T* base) -> int {
+        auto mode = [&](int o) -> int {
             int64_t is = dsc.stride[o][rank - 1];
             if (is == 0) return (int)M_BCAST;
-            if (is == 1 && vec_ok<T>(base, dsc, o)) return (int)M_VEC;
+            if (is == 1) return (int)M_VEC;
             return (int)M_ELEM;
         };
-        const int lm = mode(0, l), rm = (OP == kOpCopy) ? (int)M_BCAST : mode(1, r);
+        const int lm = mode(0), rm = (OP == kOpCopy) ? (int)M_BCAST : mode(1);
         // Loop dim.  Default: the innermost outer dim, two steps per lane (measured best on MI355X: enough work to
         // amortise the per-block index arithmetic, short enough that the chip is covered by ~10^5..10^6 small blocks;
         // a broadcast operand is re-read from L2, which its reuse distance fits).  Exception: an operand that needs
@@ -514,19 +533,12 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
         const T* lp = l + dsc.offset[0];
         const T* rp = r + dsc.offset[1];
         T* dp = d + dsc.offset[2];
-        // does operand o walk memory exactly like a row-major run over the collapsed shape, from a 16-byte aligned address?
-        auto flat = [&](int o, const T* base) {
-            int64_t acc = 1;
-            for (int k = rank - 1; k >= 0; --k) {
-                if (dsc.stride[o][k] != acc) return false;
-                acc *= dsc.shape[k];
-            }
-            return (reinterpret_cast<uintptr_t>(base) & 15) == 0;
-        };
+        // dst must walk memory exactly like a row-major run over the collapsed shape from a 16-byte aligned address; an input that
+        // walks the same way (from any element) is read with one vector load per lane
         uint32_t first = 0;
-        if (flat(2, dp) && count >= (uint64_t)N) {
+        if (row_major_run(2) && (reinterpret_cast<uintptr_t>(dp) & 15) == 0 && count >= (uint64_t)N) {
             const uint32_t nvec = (uint32_t)(count / N);
-            const bool lv = flat(0, lp), rv = OP != kOpCopy && flat(1, rp);
+            const bool lv = row_major_run(0), rv = OP != kOpCopy && row_major_run(1);
             // a repeated row: stride 1 along the last dim, 0 along every other one
             auto row_like = [&](int o) {
                 if (rank < 2 || dsc.stride[o][rank - 1] != 1) return false;

@@ -70,6 +70,7 @@ template <int OP, class T> __device__ __forceinline__ void bin_apply_vec(Vec16<T
 constexpr int kBlock = 256;     // generic kernels
 constexpr int kRBlock = 128;    // contig / rows kernels: small blocks, one 16-byte vector per lane per step
 
+// M_VEC: unit stride along the row (16-byte accesses at element alignment), M_BCAST: stride 0, M_ELEM: any other stride
 enum Mode : int { M_VEC = 0, M_BCAST = 1, M_ELEM = 2 };
 
 // One 16-byte vector of an operand's row as four 32-bit words (the form that crosses selects and loops without being split into
@@ -78,8 +79,7 @@ template <class T, int MODE>
 __device__ __forceinline__ rt_u32x4 load_raw(const T* __restrict__ rowp, uint32_t c, int64_t istride, bool nt) {
     constexpr int N = 16 / sizeof(T);
     if constexpr (MODE == M_VEC) {
-        const rt_u32x4* q = reinterpret_cast<const rt_u32x4*>(rowp + c);
-        return nt ? __builtin_nontemporal_load(q) : *q;
+        return rt_ld16u<T>(rowp + c, nt);                    // unit stride along the row; the row may start at any element
     } else {
         Vec16<T> v;
         if constexpr (MODE == M_BCAST) {
@@ -99,16 +99,6 @@ __device__ __forceinline__ Vec16<T> load_vec(const T* __restrict__ rowp, uint32_
 }
 
 static inline bool mult_of(int64_t v, int64_t n) { return v % n == 0; }
-
-// Can operand `o` be read with aligned 16-byte loads at every (outer, g, column-vector) position?
-template <class T>
-static bool vec_ok(const T* base, const NdDesc& dsc, int o) {
-    constexpr int64_t N = 16 / sizeof(T);
-    if ((reinterpret_cast<uintptr_t>(base + dsc.offset[o]) & 15) != 0) return false;
-    for (int k = 0; k < dsc.rank - 1; ++k)
-        if (!mult_of(dsc.stride[o][k], N)) return false;
-    return true;
-}
 
 // Launches the LDS-transpose kernel when the operation fits it: exactly one input is "transposed" (its inner stride is
 // neither 0 nor 1 and it has unit |stride| along another dim) and there is no long stride-0 dim over which the row kernel

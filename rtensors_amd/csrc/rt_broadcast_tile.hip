@@ -222,7 +222,7 @@ __global__ __launch_bounds__(kTBlock) void bin_tile_kernel(const T* xt, const T*
                     Vec16<T> out;
                     if (x_left) { out = xv; bin_apply_vec<OP, T>(out, ov[i]); }
                     else { out = ov[i]; bin_apply_vec<OP, T>(out, xv); }
-                    rt_st16_nt(reinterpret_cast<Vec16<T>*>(drow + (int64_t)(k0 + kk) * a.tstride[2] + c), out);
+                    rt_st16u_nt<T>(drow + (int64_t)(k0 + kk) * a.tstride[2] + c, __builtin_bit_cast(rt_u32x4, out));
                 }
             }
         } else {
@@ -252,7 +252,7 @@ bool tile_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* l, const 
     constexpr int64_t N = 16 / sizeof(T);
     const int rank = dsc.rank;
     // rows shorter than a quarter of the tile's columns would leave most lanes of every wave idle
-    if (!(rank >= 2 && count < (1ull << 31) && dsc.stride[2][rank - 1] == 1 && dsc.shape[rank - 1] >= TileGeom<T>::TL / 4 && vec_ok<T>(d, dsc, 2))) return false;
+    if (!(rank >= 2 && count < (1ull << 31) && dsc.stride[2][rank - 1] == 1 && dsc.shape[rank - 1] >= TileGeom<T>::TL / 4)) return false;
     auto transposed_dim = [&](int o) -> int {
         int64_t is = dsc.stride[o][rank - 1];
         if (is == 0 || is == 1) return -1;
@@ -276,8 +276,7 @@ bool tile_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* l, const 
     int om;
     {
         int64_t is = dsc.stride[o][rank - 1];
-        const T* base = o == 0 ? l : r;
-        om = is == 0 ? (int)M_BCAST : ((is == 1 && vec_ok<T>(base, dsc, o)) ? (int)M_VEC : (int)M_ELEM);
+        om = is == 0 ? (int)M_BCAST : (is == 1 ? (int)M_VEC : (int)M_ELEM);
     }
     TileArgs a;
     memset(&a, 0, sizeof(a));

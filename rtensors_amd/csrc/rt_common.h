@@ -130,6 +130,33 @@ template <class V> __device__ __forceinline__ void rt_st16_nt(V* p, const V& v) 
     __builtin_nontemporal_store(__builtin_bit_cast(rt_u32x4, v), reinterpret_cast<rt_u32x4*>(p));
 }
 
+// 16-byte accesses at element alignment.  The hardware runs in unaligned-access mode: the same global_load / global_store
+// dwordx4 serves any address, so a row that starts 4 bytes past a 16-byte boundary (a column slice `m[:, 1:]`, an odd row length)
+// still moves one vector per lane; a wave's 1 KiB then touches nine 128-byte lines instead of eight.  The pointee types below
+// only tell the compiler not to assume more than the element's own alignment.
+typedef uint32_t rt_u32x4_a1 __attribute__((ext_vector_type(4), aligned(1)));
+typedef uint32_t rt_u32x4_a2 __attribute__((ext_vector_type(4), aligned(2)));
+typedef uint32_t rt_u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+template <int ES> struct rt_uvec { typedef rt_u32x4_a4 type; };
+template <> struct rt_uvec<1> { typedef rt_u32x4_a1 type; };
+template <> struct rt_uvec<2> { typedef rt_u32x4_a2 type; };
+template <class T> __device__ __forceinline__ rt_u32x4 rt_ld16u(const T* p, bool nt) {
+    typedef typename rt_uvec<(int)sizeof(T)>::type U;
+    const U* q = reinterpret_cast<const U*>(p);
+    U r = nt ? __builtin_nontemporal_load(q) : *q;
+    return rt_u32x4{r.x, r.y, r.z, r.w};
+}
+template <class T> __device__ __forceinline__ void rt_st16u(T* p, rt_u32x4 v) {
+    typedef typename rt_uvec<(int)sizeof(T)>::type U;
+    U r = {v.x, v.y, v.z, v.w};
+    *reinterpret_cast<U*>(p) = r;
+}
+template <class T> __device__ __forceinline__ void rt_st16u_nt(T* p, rt_u32x4 v) {
+    typedef typename rt_uvec<(int)sizeof(T)>::type U;
+    U r = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(r, reinterpret_cast<U*>(p));
+}
+
 // Four 1-byte integers packed in a 32-bit word, wrapping add / subtract of every byte at once: the low seven bits are
 // combined with the top bits masked so that no carry or borrow crosses a byte, then the top bits are restored by xor.
 // Per-byte code (sub-dword selects and re-packing) costs about twice the vector instructions per 16-byte vector, enough

@@ -343,17 +343,13 @@ __global__ __launch_bounds__(kCBlock) void ew_rows_kernel(T* __restrict__ p, Row
         for (uint32_t g = g_begin + ty; g < g_end; g += 2 * gy) {
             const bool two = g + gy < g_end;
             // vectors stay four 32-bit words across the conditional loads (arrays of 1-byte elements would be split up and re-packed)
-            rt_u32x4* v0 = reinterpret_cast<rt_u32x4*>(p + off + (int64_t)g * a.gstride + c);
-            rt_u32x4* v1 = reinterpret_cast<rt_u32x4*>(p + off + (int64_t)(two ? g + gy : g) * a.gstride + c);
+            // rows may start at any element: 16-byte accesses at element alignment
+            T* v0 = p + off + (int64_t)g * a.gstride + c;
+            T* v1 = p + off + (int64_t)(two ? g + gy : g) * a.gstride + c;
             rt_u32x4 w0 = {}, w1 = {};
             if constexpr (F::kReads) {
-                if constexpr (NT) {
-                    w0 = __builtin_nontemporal_load(v0);
-                    if (two) w1 = __builtin_nontemporal_load(v1);
-                } else {
-                    w0 = *v0;
-                    if (two) w1 = *v1;
-                }
+                w0 = rt_ld16u<T>(v0, NT);
+                if (two) w1 = rt_ld16u<T>(v1, NT);
             }
             Vec16<T> e0 = __builtin_bit_cast(Vec16<T>, w0), e1 = __builtin_bit_cast(Vec16<T>, w1);
             apply_vec(e0, f);
@@ -361,11 +357,11 @@ __global__ __launch_bounds__(kCBlock) void ew_rows_kernel(T* __restrict__ p, Row
             w0 = __builtin_bit_cast(rt_u32x4, e0);
             w1 = __builtin_bit_cast(rt_u32x4, e1);
             if constexpr (F::kReads && NT) {
-                __builtin_nontemporal_store(w0, v0);
-                if (two) __builtin_nontemporal_store(w1, v1);
+                rt_st16u_nt<T>(v0, w0);
+                if (two) rt_st16u_nt<T>(v1, w1);
             } else {
-                *v0 = w0;
-                if (two) *v1 = w1;
+                rt_st16u<T>(v0, w0);
+                if (two) rt_st16u<T>(v1, w1);
             }
         }
     } else {
@@ -492,9 +488,9 @@ int32_t launch_view(rt_ctx* ctx, T* base, const NdDesc& d, uint64_t count, F f) 
         a.div[i] = make_fastdiv(a.shape[i]);
     }
     constexpr int64_t N = 16 / sizeof(T);
-    // rows form: unit-stride inner dim of at least two vectors, every row start 16-byte aligned
-    bool rows_ok = d.stride[0][d.rank - 1] == 1 && d.shape[d.rank - 1] >= 2 * N && (reinterpret_cast<uintptr_t>(p) & 15) == 0;
-    for (int k = 0; k < d.rank - 1; ++k) rows_ok = rows_ok && (d.stride[0][k] % N == 0);
+    // rows form: unit-stride inner dim of at least two vectors; the rows may start at any element (`m[:, 1:]` of a 8192 x 32768
+    // f32 matrix: relu in place 0.57 ms element by element, 0.36 ms with unaligned vectors)
+    const bool rows_ok = d.stride[0][d.rank - 1] == 1 && d.shape[d.rank - 1] >= 2 * N;
     if (rows_ok) {
         RowsArgs r;
         memset(&r, 0, sizeof(r));

@@ -993,6 +993,11 @@ def test_reduction_shapes_short_rows_narrow_columns_short_axis(hip, dtype):
     for R in (1, 2, 4, 5, 16, 31, 32, 33):
         for inner, outer in ((2, 1000), (3, 1), (64, 50), (100, 7), (1024, 3), (1028, 2)):
             _check_reduce(hip, dtype, outer, R, inner, rng, offset=int(rng.integers(0, 5)))
+    # wide rows whose length is not a multiple of the 16-byte vector (and starts that are not aligned): every lane still loads
+    # whole vectors, the last one overlapping its neighbour
+    for outer, R, inner in ((2, 300, 257), (1, 5003, 1001), (3, 100, 129), (1, 2000, 1030), (1, 70, 4099), (2, 40, 131)):
+        for offset in (0, 1, 3):
+            _check_reduce(hip, dtype, outer, R, inner, rng, offset=offset)
 
 
 def _check_stat(hip, dtype, outer, R, inner, rng, offset=0):
@@ -1052,7 +1057,7 @@ STAT_SHAPES = ([(rows, R, 1) for R in (1, 2, 3, 7, 8, 31, 32, 33, 64, 65, 100, 2
                + [(30000, R, 1) for R in (1, 2, 4, 8, 16, 32, 64)]
                + [(outer, R, inner) for inner in (2, 3, 5, 17, 63, 64, 100, 128) for R, outer in ((64, 3), (1000, 1), (5003, 2), (70001, 1))]
                + [(outer, R, inner) for R in (1, 2, 5, 16, 33) for inner, outer in ((2, 1000), (3, 1), (64, 50), (1028, 2))]
-               + [(1, 300, 5000), (2, 4000, 260), (1, 70, 2052)])
+               + [(1, 300, 5000), (2, 4000, 260), (1, 70, 2052), (2, 300, 257), (1, 5003, 1001), (3, 100, 129), (1, 2000, 1030), (1, 70, 4099), (2, 40, 131)])
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f64"])
