@@ -23,8 +23,19 @@ namespace {
 // ---- contig ---------------------------------------------------------------------------------------------------------
 // One vector per lane, non-temporal loads and stores: every byte is touched exactly once.
 template <class T, int OP>
-__global__ __launch_bounds__(kRBlock) void bin_contig_kernel(const Vec16<T>* l, const Vec16<T>* r, Vec16<T>* d, size_t nvec) {
+__global__ __launch_bounds__(kRBlock) void bin_contig_kernel(const Vec16<T>* l, const Vec16<T>* r, Vec16<T>* d, size_t nvec, uint32_t head,
+                                                             uint32_t tail) {
     const size_t i = (size_t)blockIdx.x * kRBlock + threadIdx.x;
+    // the `head` elements before and the `tail` elements after the aligned body (fewer than a vector each; all three operands
+    // share the phase) are taken by lanes of the first and the last block instead of launches of their own
+    auto edge = [&](int64_t e) {
+        const T x = *(reinterpret_cast<const T*>(l) + e);
+        T y = x;
+        if constexpr (OP != kOpCopy) y = *(reinterpret_cast<const T*>(r) + e);
+        *(reinterpret_cast<T*>(d) + e) = bin_apply<OP, T>(x, y);
+    };
+    if (blockIdx.x == 0 && threadIdx.x < head) edge((int64_t)threadIdx.x - (int64_t)head);
+    if (blockIdx.x == gridDim.x - 1 && threadIdx.x < tail) edge((int64_t)(nvec * (16 / sizeof(T))) + (int64_t)threadIdx.x);
     if (i >= nvec) return;
     Vec16<T> a = rt_ld16_nt(l + i);
     Vec16<T> b;
@@ -355,27 +366,17 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
         uintptr_t al = reinterpret_cast<uintptr_t>(lp) & 15, ar = reinterpret_cast<uintptr_t>(rp) & 15, ad = reinterpret_cast<uintptr_t>(dp) & 15;
         if (al == ar && ar == ad) {
             size_t n = (size_t)count;
-            size_t head = ((16 - ad) & 15) / sizeof(T);
+            // the body starts where dst reaches a 128-byte line (the inputs, in phase with dst modulo 16, are then 16-byte aligned):
+            // a wave's 1 KiB of stores covers eight whole lines instead of sharing its first and last line with a neighbour
+            size_t head = ((128 - (reinterpret_cast<uintptr_t>(dp) & 127)) & 127) / sizeof(T);
             if (head > n) head = n;
             size_t nvec = (n - head) / N, tail = n - head - nvec * N;
-            if (nvec) {
-                size_t blocks = (nvec + (size_t)kRBlock - 1) / (size_t)kRBlock;
-                if (blocks > 0x7fffffffull) return rt_fail(RT_E_INVALID, "broadcast: %zu elements is too long for one launch", n);
-                hipLaunchKernelGGL((bin_contig_kernel<T, OP>), dim3((unsigned)blocks), dim3(kRBlock), 0, s,
-                                   reinterpret_cast<const Vec16<T>*>(lp + head), reinterpret_cast<const Vec16<T>*>(rp + head),
-                                   reinterpret_cast<Vec16<T>*>(dp + head), nvec);
-            }
-            // the few elements before / after the 16-byte aligned body
-            auto edge = [&](size_t first, size_t len) {
-                NdDesc e;
-                memset(&e, 0, sizeof(e));
-                e.rank = 1;
-                e.shape[0] = (int64_t)len;
-                e.stride[0][0] = e.stride[1][0] = e.stride[2][0] = 1;
-                hipLaunchKernelGGL((bin_generic64_kernel<T, OP>), dim3(1), dim3(kBlock), 0, s, lp + first, rp + first, dp + first, e, (uint64_t)len);
-            };
-            if (head) edge(0, head);
-            if (tail) edge(head + nvec * N, tail);
+            size_t blocks = (nvec + (size_t)kRBlock - 1) / (size_t)kRBlock;
+            if (blocks < 1) blocks = 1;                            // fewer elements than a vector: edges only
+            if (blocks > 0x7fffffffull) return rt_fail(RT_E_INVALID, "broadcast: %zu elements is too long for one launch", n);
+            hipLaunchKernelGGL((bin_contig_kernel<T, OP>), dim3((unsigned)blocks), dim3(kRBlock), 0, s,
+                               reinterpret_cast<const Vec16<T>*>(lp + head), reinterpret_cast<const Vec16<T>*>(rp + head),
+                               reinterpret_cast<Vec16<T>*>(dp + head), nvec, (uint32_t)head, (uint32_t)tail);
             RT_HIP(hipGetLastError());
             return RT_OK;
         }

@@ -227,8 +227,23 @@ constexpr int kEU = 4;          // element-per-lane kernels: elements in flight 
 // on MI355X this shape (with non-temporal accesses for read-modify-write, plain stores for write-only) was the
 // fastest of the block-size / unroll / grid-stride variants tried, ~6.7 TB/s in place and ~6.8 TB/s for fill.
 template <class T, class F>
-__global__ __launch_bounds__(256) void ew_contig_kernel(Vec16<T>* __restrict__ p, size_t nvec, F f) {
+__global__ __launch_bounds__(256) void ew_contig_kernel(Vec16<T>* __restrict__ p, size_t nvec, uint32_t head, uint32_t tail, F f) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    // The `head` elements before and the `tail` elements after the 16-byte aligned body (fewer than a vector each) are taken by
+    // lanes of the first and the last block: launches of their own cost a run that starts off a 16-byte boundary 9 % (1 GiB f32
+    // `+= 1`: 0.363 ms with three launches against 0.331 ms aligned).
+    if (blockIdx.x == 0 && threadIdx.x < head) {
+        T* e = reinterpret_cast<T*>(p) - head + threadIdx.x;
+        T x = zero_of<T>();
+        if constexpr (F::kReads) x = *e;
+        *e = f(x);
+    }
+    if (blockIdx.x == gridDim.x - 1 && threadIdx.x < tail) {
+        T* e = reinterpret_cast<T*>(p + nvec) + threadIdx.x;
+        T x = zero_of<T>();
+        if constexpr (F::kReads) x = *e;
+        *e = f(x);
+    }
     if (i >= nvec) return;
     Vec16<T> v;
     if constexpr (F::kReads) v = rt_ld16_nt(p + i);
@@ -397,26 +412,27 @@ __global__ __launch_bounds__(kBlock) void ew_nd64_kernel(T* __restrict__ p, NdDe
 }
 
 // ---- launch logic ---------------------------------------------------------------------------------------------------
+constexpr uintptr_t kBodyAlign = 128;        // at most 127 one-byte elements before the body: fewer than the lanes of a block
 static inline unsigned capped_grid(size_t blocks, size_t cap) { return (unsigned)(blocks < 1 ? 1 : (blocks > cap ? cap : blocks)); }
 
 template <class T, class F>
 int32_t launch_contig(rt_ctx* ctx, T* p, size_t n, F f) {
     if (n == 0) return RT_OK;
     constexpr size_t N = 16 / sizeof(T);
+    // The vector body starts on a 128-byte line, not merely on a 16-byte boundary, so that a wave's 1 KiB covers eight whole
+    // lines; with the body 16 bytes into a line every wave shares its first and last line with a neighbour and the pass is 9 %
+    // slower (1 GiB f32 `+= 1` from element 1: 0.361 ms, aligned 0.331 ms).  The up to 127 bytes before it are edge elements.
     uintptr_t addr = reinterpret_cast<uintptr_t>(p);
-    size_t head = ((16 - (addr & 15)) & 15) / sizeof(T);
+    size_t head = ((kBodyAlign - (addr & (kBodyAlign - 1))) & (kBodyAlign - 1)) / sizeof(T);
     if (head > n) head = n;
     size_t nvec = (n - head) / N;
     size_t tail = n - head - nvec * N;
-    if (nvec) {
-        const size_t bs = F::kReads ? (size_t)kCBlock : (size_t)256;      // pure stores: 256 lanes measured best
-        size_t blocks = (nvec + bs - 1) / bs;
-        if (blocks > 0x7fffffffull) return rt_fail(RT_E_INVALID, "contiguous run of %zu elements is too long for one launch", n);
-        hipLaunchKernelGGL((ew_contig_kernel<T, F>), dim3((unsigned)blocks), dim3((unsigned)bs), 0, ctx->stream,
-                           reinterpret_cast<Vec16<T>*>(p + head), nvec, f);
-    }
-    if (head) hipLaunchKernelGGL((ew_strided_kernel<T, F>), dim3(1), dim3(kBlock), 0, ctx->stream, p, (int64_t)1, head, f);
-    if (tail) hipLaunchKernelGGL((ew_strided_kernel<T, F>), dim3(1), dim3(kBlock), 0, ctx->stream, p + head + nvec * N, (int64_t)1, tail, f);
+    const size_t bs = F::kReads ? (size_t)kCBlock : (size_t)256;          // pure stores: 256 lanes measured best
+    size_t blocks = (nvec + bs - 1) / bs;
+    if (blocks < 1) blocks = 1;                                           // a run shorter than a vector: edges only
+    if (blocks > 0x7fffffffull) return rt_fail(RT_E_INVALID, "contiguous run of %zu elements is too long for one launch", n);
+    hipLaunchKernelGGL((ew_contig_kernel<T, F>), dim3((unsigned)blocks), dim3((unsigned)bs), 0, ctx->stream,
+                       reinterpret_cast<Vec16<T>*>(p + head), nvec, (uint32_t)head, (uint32_t)tail, f);
     RT_HIP(hipGetLastError());
     return RT_OK;
 }
