@@ -440,37 +440,32 @@ int32_t launch_contig(rt_ctx* ctx, T* p, size_t n, F f) {
 // Out of place: dst[i] = f(src[i]) for a contiguous run; what `tensor.op()` needs instead of clone + in-place op, at half the
 // traffic (2 * N * sizeof(T) instead of 4 * N * sizeof(T)).
 template <class T, class F>
-__global__ __launch_bounds__(kCBlock) void ew_contig_out_kernel(const Vec16<T>* __restrict__ s, Vec16<T>* __restrict__ d, size_t nvec, F f) {
+__global__ __launch_bounds__(kCBlock) void ew_contig_out_kernel(const T* __restrict__ s, T* __restrict__ d, size_t nvec, uint32_t head, uint32_t tail, F f) {
+    constexpr size_t N = 16 / sizeof(T);
     const size_t i = (size_t)blockIdx.x * kCBlock + threadIdx.x;
+    // s and d point at the vector body, which starts on a 128-byte line of d; the `head` elements before it and the `tail`
+    // elements after it go to lanes of the first and the last block
+    if (blockIdx.x == 0 && threadIdx.x < head) { const int64_t e = (int64_t)threadIdx.x - (int64_t)head; d[e] = f(s[e]); }
+    if (blockIdx.x == gridDim.x - 1 && threadIdx.x < tail) { const size_t e = nvec * N + threadIdx.x; d[e] = f(s[e]); }
     if (i >= nvec) return;
-    Vec16<T> v = rt_ld16_nt(s + i);
+    Vec16<T> v = __builtin_bit_cast(Vec16<T>, rt_ld16u<T>(s + i * N, true));          // the source may be in any phase
     apply_vec(v, f);
-    rt_st16_nt(d + i, v);
-}
-template <class T, class F>
-__global__ __launch_bounds__(kBlock) void ew_elem_out_kernel(const T* __restrict__ s, T* __restrict__ d, size_t n, F f) {
-    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    const size_t step = (size_t)gridDim.x * kBlock;
-    for (; i < n; i += step) d[i] = f(s[i]);
+    rt_st16_nt(reinterpret_cast<Vec16<T>*>(d) + i, v);
 }
 
 template <class T, class F>
 int32_t launch_contig_out(rt_ctx* ctx, const T* s, T* d, size_t n, F f) {
     constexpr size_t N = 16 / sizeof(T);
-    const bool aligned = ((reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) & 15) == 0;
-    const size_t nvec = aligned ? n / N : 0;
-    if (nvec) {
-        size_t blocks = (nvec + kCBlock - 1) / kCBlock;
-        if (blocks > 0x7fffffffull) return rt_fail(RT_E_INVALID, "contiguous run of %zu elements is too long for one launch", n);
-        hipLaunchKernelGGL((ew_contig_out_kernel<T, F>), dim3((unsigned)blocks), dim3(kCBlock), 0, ctx->stream,
-                           reinterpret_cast<const Vec16<T>*>(s), reinterpret_cast<Vec16<T>*>(d), nvec, f);
-    }
-    const size_t rest = n - nvec * N;
-    if (rest) {
-        size_t blocks = (rest + kBlock - 1) / kBlock;
-        hipLaunchKernelGGL((ew_elem_out_kernel<T, F>), dim3(capped_grid(blocks, (size_t)ctx->num_cus * 32)), dim3(kBlock), 0, ctx->stream,
-                           s + nvec * N, d + nvec * N, rest, f);
-    }
+    if (n == 0) return RT_OK;
+    const uintptr_t addr = reinterpret_cast<uintptr_t>(d);
+    size_t head = ((kBodyAlign - (addr & (kBodyAlign - 1))) & (kBodyAlign - 1)) / sizeof(T);
+    if (head > n) head = n;
+    const size_t nvec = (n - head) / N, tail = n - head - nvec * N;
+    size_t blocks = (nvec + kCBlock - 1) / kCBlock;
+    if (blocks < 1) blocks = 1;
+    if (blocks > 0x7fffffffull) return rt_fail(RT_E_INVALID, "contiguous run of %zu elements is too long for one launch", n);
+    hipLaunchKernelGGL((ew_contig_out_kernel<T, F>), dim3((unsigned)blocks), dim3(kCBlock), 0, ctx->stream, s + head, d + head, nvec, (uint32_t)head,
+                       (uint32_t)tail, f);
     RT_HIP(hipGetLastError());
     return RT_OK;
 }

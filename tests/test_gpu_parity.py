@@ -120,6 +120,31 @@ def test_buffers_and_transfers(hip):
     assert not (hip.alloc(H.F32, 3) == hip.alloc(H.F32, 4))
 
 
+@pytest.mark.parametrize("dtype", ["u8", "i16", "f32", "f64"])
+def test_copy_range_within_any_phase(hip, dtype):
+    """`copy_range_within` (backend/mod.rs:227-229) with source and destination ranges in every 16-byte phase relative to each other and
+    to the 128-byte lines the copy kernel aligns its body to; lengths from a single element to several blocks; the bytes outside the
+    destination range stay untouched."""
+    code = cpu.DTYPE_BY_NAME[dtype]
+    rng = np.random.default_rng(zlib.crc32(dtype.encode()) + 5)
+    n = 6000
+    x = rand_values(dtype, n, rng)
+    src = hip.alloc_from_slice(code, x)
+    for trial in range(60):
+        ln = int(rng.choice([1, 2, 3, 15, 16, 17, 31, 127, 128, 129, 1000, 4097, 5000]))
+        do, so = int(rng.integers(0, n - ln + 1)), int(rng.integers(0, n - ln + 1))
+        if trial < 20:
+            do, so = trial % 5, (trial * 3) % 7                                 # small offsets: every phase pair near the buffer start
+            ln = min(ln, n - 8)
+        y = rand_values(dtype, n, rng)
+        dst = hip.alloc_from_slice(code, y)
+        hip.copy_range_within(dst, src, do, so, ln)
+        want = y.copy(); want[do:do + ln] = x[so:so + ln]
+        assert hip.dump(dst).tobytes() == want.tobytes(), (dtype, do, so, ln)
+    with pytest.raises(Exception):
+        hip.copy_range_within(src, src, n - 3, 0, 4)
+
+
 def test_allocator_reuses_blocks(hip):
     from rtensors_amd import hip as H
     hip.sync()
