@@ -76,10 +76,13 @@ enum Mode : int { M_VEC = 0, M_BCAST = 1, M_ELEM = 2 };
 // One 16-byte vector of an operand's row as four 32-bit words (the form that crosses selects and loops without being split into
 // per-element registers), and the same as elements.
 template <class T, int MODE>
-__device__ __forceinline__ rt_u32x4 load_raw(const T* __restrict__ rowp, uint32_t c, int64_t istride, bool nt) {
+__device__ __forceinline__ rt_u32x4 load_raw(const T* __restrict__ rowp, uint32_t c, int64_t istride) {
     constexpr int N = 16 / sizeof(T);
     if constexpr (MODE == M_VEC) {
-        return rt_ld16u<T>(rowp + c, nt);                    // unit stride along the row; the row may start at any element
+        // Unit stride along the row; the row may start at any element.  Plain (cached) loads also for operands that are read only
+        // once: a non-temporal hint chosen at run time measured no gain on them (a column-sliced 1 GiB operand plus a row, the
+        // transposed add) and its second code path cost the config-3 add 4 %.
+        return rt_ld16u<T, false>(rowp + c);
     } else {
         Vec16<T> v;
         if constexpr (MODE == M_BCAST) {
@@ -94,8 +97,8 @@ __device__ __forceinline__ rt_u32x4 load_raw(const T* __restrict__ rowp, uint32_
     }
 }
 template <class T, int MODE>
-__device__ __forceinline__ Vec16<T> load_vec(const T* __restrict__ rowp, uint32_t c, int64_t istride, bool nt) {
-    return __builtin_bit_cast(Vec16<T>, load_raw<T, MODE>(rowp, c, istride, nt));
+__device__ __forceinline__ Vec16<T> load_vec(const T* __restrict__ rowp, uint32_t c, int64_t istride) {
+    return __builtin_bit_cast(Vec16<T>, load_raw<T, MODE>(rowp, c, istride));
 }
 
 static inline bool mult_of(int64_t v, int64_t n) { return v % n == 0; }

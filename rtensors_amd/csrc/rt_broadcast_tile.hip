@@ -42,8 +42,6 @@ struct TileArgs {
     // strides by role: 0 = the transposed input, 1 = the other input, 2 = dst
     int64_t gstride[3], tstride[3], istride[3];   // loop dim, dim t, inner dim
     uint32_t x_is_left;             // the transposed input is the left operand of the op
-    uint32_t nt_other;              // the non-transposed input is streamed -> non-temporal loads
-    uint32_t nt_xt;                 // the transposed input is streamed
 };
 
 // xt / xo: the transposed and the other input.  OM = access mode of the other input along the inner dim; VG = the transposed
@@ -102,7 +100,7 @@ __global__ __launch_bounds__(kTBlock) void bin_tile_kernel(const T* xt, const T*
 #pragma unroll
                 for (int i = 0; i < kTSteps; ++i) {
                     const uint32_t k = min(k0 + krow + i * kTWaves * RPI, a.K - 1);
-                    if (i == 0 || !o_fixed) ov[i] = load_vec<T, OM>(orow + (int64_t)k * a.tstride[1], c, a.istride[1], a.nt_other != 0);
+                    if (i == 0 || !o_fixed) ov[i] = load_vec<T, OM>(orow + (int64_t)k * a.tstride[1], c, a.istride[1]);
                     else ov[i] = ov[0];
                 }
             }
@@ -132,7 +130,7 @@ __global__ __launch_bounds__(kTBlock) void bin_tile_kernel(const T* xt, const T*
                         const uint32_t col = min(l0 + (lg + i * GPI) * P + p, a.L - 1);
                         if (t0 < a.K) {                        // K is a multiple of N on this path
                             const rt_u32x4* q4 = reinterpret_cast<const rt_u32x4*>(src + (int64_t)col * a.istride[0]);
-                            grp[i][p] = a.nt_xt ? rt_ld16_nt(q4) : rt_ld16(q4);
+                            grp[i][p] = rt_ld16(q4);
                         } else {
                             grp[i][p] = rt_u32x4{0, 0, 0, 0};
                         }
@@ -178,7 +176,7 @@ __global__ __launch_bounds__(kTBlock) void bin_tile_kernel(const T* xt, const T*
                     const uint32_t col = min(l0 + ls + i * LPI, a.L - 1);
                     if (t0 < a.K) {                            // K is a multiple of N on this path
                         const Vec16<T>* p = reinterpret_cast<const Vec16<T>*>(src + (int64_t)col * a.istride[0]);
-                        grp[i] = a.nt_xt ? rt_ld16_nt(p) : rt_ld16(p);
+                        grp[i] = rt_ld16(p);
                     } else {
                         grp[i] = Vec16<T>{};
                     }
@@ -315,9 +313,6 @@ bool tile_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* l, const 
     a.ltiles_div = make_fastdiv(a.ltiles);
     a.ktiles_div = make_fastdiv(a.ktiles);
     a.nchunks_div = make_fastdiv(a.nchunks);
-    bool streamed = true;
-    for (int k = 0; k < rank; ++k) streamed = streamed && dsc.stride[o][k] != 0;
-    a.nt_other = streamed ? 1u : 0u;
     bool vec_gather = false;
     {
         const T* xbase = (xt == 0 ? l : r) + dsc.offset[xt];
@@ -325,13 +320,9 @@ bool tile_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* l, const 
         // every vector starts at (base + multiples of N) for an ascending dim t, and ends there for a descending one
         const T* first = ts > 0 ? xbase : xbase - (N - 1);
         bool ok = (reinterpret_cast<uintptr_t>(first) & 15) == 0 && (a.K % (uint32_t)N) == 0 && TK % (uint32_t)N == 0;
-        bool xstream = true;
-        for (int k = 0; k < rank; ++k) {
+        for (int k = 0; k < rank; ++k)
             if (k != tdim) ok = ok && mult_of(dsc.stride[xt][k], N);
-            xstream = xstream && dsc.stride[xt][k] != 0;
-        }
         vec_gather = ok;
-        a.nt_xt = xstream ? 1u : 0u;
     }
     const uint64_t blocks = outer * a.nchunks * a.ktiles * a.ltiles;
     if (blocks >= (1ull << 31)) return false;

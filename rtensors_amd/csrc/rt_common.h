@@ -140,10 +140,13 @@ typedef uint32_t rt_u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 template <int ES> struct rt_uvec { typedef rt_u32x4_a4 type; };
 template <> struct rt_uvec<1> { typedef rt_u32x4_a1 type; };
 template <> struct rt_uvec<2> { typedef rt_u32x4_a2 type; };
-template <class T> __device__ __forceinline__ rt_u32x4 rt_ld16u(const T* p, bool nt) {
+// NT is a compile-time choice on purpose: written as `nt ? nontemporal_load(q) : *q` the two loads of one address are merged
+// into a single plain load and the hint is lost.
+template <class T, bool NT> __device__ __forceinline__ rt_u32x4 rt_ld16u(const T* p) {
     typedef typename rt_uvec<(int)sizeof(T)>::type U;
     const U* q = reinterpret_cast<const U*>(p);
-    U r = nt ? __builtin_nontemporal_load(q) : *q;
+    U r;
+    if constexpr (NT) r = __builtin_nontemporal_load(q); else r = *q;
     return rt_u32x4{r.x, r.y, r.z, r.w};
 }
 template <class T> __device__ __forceinline__ void rt_st16u(T* p, rt_u32x4 v) {

@@ -363,8 +363,8 @@ __global__ __launch_bounds__(kCBlock) void ew_rows_kernel(T* __restrict__ p, Row
             T* v1 = p + off + (int64_t)(two ? g + gy : g) * a.gstride + c;
             rt_u32x4 w0 = {}, w1 = {};
             if constexpr (F::kReads) {
-                w0 = rt_ld16u<T>(v0, NT);
-                if (two) w1 = rt_ld16u<T>(v1, NT);
+                w0 = rt_ld16u<T, NT>(v0);
+                if (two) w1 = rt_ld16u<T, NT>(v1);
             }
             Vec16<T> e0 = __builtin_bit_cast(Vec16<T>, w0), e1 = __builtin_bit_cast(Vec16<T>, w1);
             apply_vec(e0, f);
@@ -448,7 +448,7 @@ __global__ __launch_bounds__(kCBlock) void ew_contig_out_kernel(const T* __restr
     if (blockIdx.x == 0 && threadIdx.x < head) { const int64_t e = (int64_t)threadIdx.x - (int64_t)head; d[e] = f(s[e]); }
     if (blockIdx.x == gridDim.x - 1 && threadIdx.x < tail) { const size_t e = nvec * N + threadIdx.x; d[e] = f(s[e]); }
     if (i >= nvec) return;
-    Vec16<T> v = __builtin_bit_cast(Vec16<T>, rt_ld16u<T>(s + i * N, true));          // the source may be in any phase
+    Vec16<T> v = __builtin_bit_cast(Vec16<T>, rt_ld16u<T, true>(s + i * N));          // the source may be in any phase
     apply_vec(v, f);
     rt_st16_nt(reinterpret_cast<Vec16<T>*>(d) + i, v);
 }

@@ -253,7 +253,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(const T* __restrict
     // the source is read exactly once: non-temporal loads; rows may start at any element (unaligned 16-byte loads)
     auto load = [](const T* q) -> VecW {
         if constexpr (sizeof(VecW) == 16) {
-            return __builtin_bit_cast(VecW, rt_ld16u<T>(q, true));
+            return __builtin_bit_cast(VecW, rt_ld16u<T, true>(q));
         } else {
             VecW w;
             w.e[0] = __builtin_nontemporal_load(q);
@@ -384,7 +384,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_tile_kernel(const T* __res
     }
 }
 
-// ---- short rows whose length is a power-of-two number of 16-byte vectors (16 B .. 1 KiB per row, aligned) -----------------------------
+// ---- short rows whose length is a power-of-two number of 16-byte vectors (16 B .. 1 KiB per row) -----------------------------------
 // No staging: the rows of a block are one contiguous run, lane t reads vector t of it (four such loads in flight), the VR lanes
 // that hold one row are neighbours inside a wave and fold with log2(VR) shuffles.
 template <int OP, class T>
@@ -392,12 +392,11 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_pow2_kernel(const T* __res
                                                                   uint64_t count) {
     constexpr uint32_t N = 16 / sizeof(T);
     constexpr int U = 4;
-    const Vec16<T>* pv = reinterpret_cast<const Vec16<T>*>(src);
-    const uint64_t v0 = (uint64_t)blockIdx.x * (kBlock * U) + threadIdx.x;
+    const uint64_t v0 = (uint64_t)blockIdx.x * (kBlock * U) + threadIdx.x;           // the run may start at any element
     Vec16<T> x[U];
 #pragma unroll
     for (int u = 0; u < U; ++u)
-        if (v0 + (uint64_t)u * kBlock < nvec) x[u] = rt_ld16_nt(pv + v0 + (uint64_t)u * kBlock);
+        if (v0 + (uint64_t)u * kBlock < nvec) x[u] = __builtin_bit_cast(Vec16<T>, rt_ld16u<T, true>(src + (v0 + (uint64_t)u * kBlock) * N));
     const uint32_t j = threadIdx.x & (VR - 1);                    // position of this lane's vector inside its row
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -462,7 +461,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_narrow_kernel(const T* __r
                 const uint64_t e = (tl + u) * S + (uint64_t)t * VW;
                 full[u] = tl + u < tile_end && e + VW <= slab;
                 if (full[u]) {
-                    if constexpr (sizeof(VecW) == 16) x[u] = rt_ld16_nt(reinterpret_cast<const VecW*>(base + e));
+                    if constexpr (sizeof(VecW) == 16) x[u] = __builtin_bit_cast(VecW, rt_ld16u<T, true>(base + e));     // any phase
                     else x[u].e[0] = __builtin_nontemporal_load(base + e);
                 }
             }
@@ -529,7 +528,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_short_kernel(const T* __re
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             if (k + u < R) {
-                if constexpr (sizeof(VecW) == 16) x[u] = rt_ld16_nt(reinterpret_cast<const VecW*>(p + (uint64_t)(k + u) * inner));
+                if constexpr (sizeof(VecW) == 16) x[u] = __builtin_bit_cast(VecW, rt_ld16u<T, true>(p + (uint64_t)(k + u) * inner));
                 else x[u].e[0] = __builtin_nontemporal_load(p + (uint64_t)(k + u) * inner);
             }
         }
@@ -582,8 +581,7 @@ int32_t rows_stage(rt_ctx* ctx, const T* src, T* out, uint64_t rows, uint64_t R,
         // sequential result)
         // float max / min carry a position through every shuffle step: with 8-byte values that only pays up to 16 lanes per row
         const uint64_t vr_max = (Acc<OP, T>::kTrack && sizeof(T) == 8) ? 16 : 64;
-        if (count == R && R % N == 0 && vr >= 1 && vr <= vr_max && (vr & (vr - 1)) == 0 && rows * vr >= 4096 &&
-            (reinterpret_cast<uintptr_t>(src) & 15) == 0) {
+        if (count == R && R % N == 0 && vr >= 1 && vr <= vr_max && (vr & (vr - 1)) == 0 && rows * vr >= 4096) {
             const uint64_t nvec = rows * vr;
             const uint64_t blocks = (nvec + (uint64_t)kBlock * 4 - 1) / ((uint64_t)kBlock * 4);
             if (blocks < (1ull << 31)) {
@@ -718,8 +716,7 @@ int32_t cols_launch(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t 
 template <int OP, class T>
 int32_t cols_narrow(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t R, uint64_t inner) {
     constexpr uint32_t N = 16 / sizeof(T);
-    const bool vec = (reinterpret_cast<uintptr_t>(src) & 15) == 0 && (outer == 1 || (R * inner) % N == 0);
-    const uint32_t vw = vec ? N : 1;
+    const uint32_t vw = N;                                     // 16-byte loads at element alignment: any phase of the slabs
     uint32_t g = (uint32_t)inner, h = vw;                      // gcd(inner, vw)
     while (h) { uint32_t t = g % h; g = h; h = t; }
     const uint32_t innerp = (uint32_t)inner / g;               // lanes per period: Tn * vw must be a multiple of inner
@@ -749,8 +746,7 @@ int32_t cols_narrow(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t 
         dst1 = (T*)scratch;
     }
     const int last = splits == 1 ? 1 : 0;
-    if (vec) hipLaunchKernelGGL((reduce_cols_narrow_kernel<OP, T, N>), dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream, src, dst1, a, R, last);
-    else hipLaunchKernelGGL((reduce_cols_narrow_kernel<OP, T, 1>), dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream, src, dst1, a, R, last);
+    hipLaunchKernelGGL((reduce_cols_narrow_kernel<OP, T, N>), dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream, src, dst1, a, R, last);
     RT_HIP(hipGetLastError());
     if (splits == 1) return RT_OK;
     // second stage: the partials are (splits, outer * inner); fold the segments in order (mean divides by the original count)
@@ -773,7 +769,7 @@ int32_t reduce_typed(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t
     // columns with inner 3 / 17 / 100 5.0 / 5.0 / 4.8; (65536, 64, 64) 6.4; (2^20, 4, 64) 5.4.  One lane or one wave per short row
     // gave 0.3-2.3, lanes along a narrow inner 0.2-1.2.
     if (R <= 32 && inner <= 1024) {                                             // short reduced axis: a lane per output vector
-        const bool v = (inner % N == 0) && ((reinterpret_cast<uintptr_t>(src) & 15) == 0);
+        const bool v = inner % N == 0;                                          // rows may start at any element
         const uint64_t ivecs = v ? inner / N : inner;
         if (ivecs < (1ull << 31) && outer * ivecs < (1ull << 31)) {
             const uint64_t nvec_out = outer * ivecs;

@@ -348,12 +348,11 @@ __global__ __launch_bounds__(kBlock) void st_rows_pow2_kernel(const T* __restric
                                                               uint32_t vr_shift, int flags) {
     constexpr uint32_t N = 16 / sizeof(T);
     constexpr int U = 4;
-    const Vec16<T>* pv = reinterpret_cast<const Vec16<T>*>(src);
-    const uint64_t v0 = (uint64_t)blockIdx.x * (kBlock * U) + threadIdx.x;
+    const uint64_t v0 = (uint64_t)blockIdx.x * (kBlock * U) + threadIdx.x;           // the run may start at any element
     Vec16<T> x[U];
 #pragma unroll
     for (int u = 0; u < U; ++u)
-        if (v0 + (uint64_t)u * kBlock < nvec) x[u] = rt_ld16_nt(pv + v0 + (uint64_t)u * kBlock);
+        if (v0 + (uint64_t)u * kBlock < nvec) x[u] = __builtin_bit_cast(Vec16<T>, rt_ld16u<T, true>(src + (v0 + (uint64_t)u * kBlock) * N));
     const uint32_t j = threadIdx.x & (VR - 1);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -391,7 +390,7 @@ __global__ __launch_bounds__(kBlock) void st_cols_kernel(const T* __restrict__ s
     // rows may start at any element: unaligned 16-byte loads
     auto load = [](const T* q) -> VecW {
         if constexpr (sizeof(VecW) == 16) {
-            return __builtin_bit_cast(VecW, rt_ld16u<T>(q, true));
+            return __builtin_bit_cast(VecW, rt_ld16u<T, true>(q));
         } else {
             VecW w;
             w.e[0] = __builtin_nontemporal_load(q);
@@ -478,7 +477,7 @@ __global__ __launch_bounds__(kBlock) void st_cols_narrow_kernel(const T* __restr
         if (tile_end > ntiles) tile_end = ntiles;
         auto load = [&](uint64_t e) -> VecW {
             if constexpr (sizeof(VecW) == 16) {
-                return rt_ld16_nt(reinterpret_cast<const VecW*>(base + e));
+                return __builtin_bit_cast(VecW, rt_ld16u<T, true>(base + e));          // any phase
             } else {
                 VecW w;
                 w.e[0] = __builtin_nontemporal_load(base + e);
@@ -591,7 +590,7 @@ int32_t rows_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t rows
     {
         constexpr uint64_t N = 16 / sizeof(T);
         const uint64_t vr = R / N;
-        if (R % N == 0 && (vr == 1 || vr == 2 || vr == 4) && rows * vr >= 4096 && (reinterpret_cast<uintptr_t>(src) & 15) == 0) {
+        if (R % N == 0 && (vr == 1 || vr == 2 || vr == 4) && rows * vr >= 4096) {
             const uint64_t nvec = rows * vr;
             const uint64_t blocks = (nvec + (uint64_t)kBlock * 4 - 1) / ((uint64_t)kBlock * 4);
             if (blocks < (1ull << 31)) {
@@ -693,7 +692,7 @@ template <class S, class T>
 int32_t narrow_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t outer, uint64_t R, uint64_t inner, int flags) {
     constexpr uint32_t N = 16 / sizeof(T);
     // vector loads for 4- and 8-byte elements (more lanes' worth of states would not fit in LDS)
-    const bool vec = sizeof(T) >= 4 && (reinterpret_cast<uintptr_t>(src) & 15) == 0 && (outer == 1 || (R * inner) % N == 0);
+    const bool vec = sizeof(T) >= 4;
     const uint32_t vw = vec ? N : 1;
     uint32_t g = (uint32_t)inner, h = vw;                      // gcd(inner, vw)
     while (h) { uint32_t r = g % h; g = h; h = r; }

@@ -320,7 +320,7 @@ __global__ __launch_bounds__(128) void rt_copy_vec_kernel(const uint8_t* __restr
     const size_t i = (size_t)blockIdx.x * 128 + threadIdx.x;
     if (blockIdx.x == 0 && threadIdx.x < head) { const int64_t e = (int64_t)threadIdx.x - (int64_t)head; d[e] = s[e]; }
     if (blockIdx.x == gridDim.x - 1 && threadIdx.x < tail) { const size_t e = nvec * 16 + threadIdx.x; d[e] = s[e]; }
-    if (i < nvec) __builtin_nontemporal_store(rt_ld16u<uint8_t>(s + i * 16, true), reinterpret_cast<rt_u32x4*>(d) + i);
+    if (i < nvec) __builtin_nontemporal_store(rt_ld16u<uint8_t, true>(s + i * 16), reinterpret_cast<rt_u32x4*>(d) + i);
 }
 
 static int32_t device_copy(rt_ctx* ctx, void* dst, const void* src, size_t bytes) {      // caller holds ctx->mu
