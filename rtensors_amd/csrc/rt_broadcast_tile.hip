@@ -42,6 +42,7 @@ struct TileArgs {
     // strides by role: 0 = the transposed input, 1 = the other input, 2 = dst
     int64_t gstride[3], tstride[3], istride[3];   // loop dim, dim t, inner dim
     uint32_t x_is_left;             // the transposed input is the left operand of the op
+    uint32_t nt_xt;                 // every element of the transposed input is used once -> non-temporal gather (tr_add 0.536 -> 0.509 ms)
 };
 
 // xt / xo: the transposed and the other input.  OM = access mode of the other input along the inner dim; VG = the transposed
@@ -130,7 +131,7 @@ __global__ __launch_bounds__(kTBlock) void bin_tile_kernel(const T* xt, const T*
                         const uint32_t col = min(l0 + (lg + i * GPI) * P + p, a.L - 1);
                         if (t0 < a.K) {                        // K is a multiple of N on this path
                             const rt_u32x4* q4 = reinterpret_cast<const rt_u32x4*>(src + (int64_t)col * a.istride[0]);
-                            grp[i][p] = rt_ld16(q4);
+                            grp[i][p] = rt_ld16_dyn(q4, a.nt_xt != 0);
                         } else {
                             grp[i][p] = rt_u32x4{0, 0, 0, 0};
                         }
@@ -176,7 +177,7 @@ __global__ __launch_bounds__(kTBlock) void bin_tile_kernel(const T* xt, const T*
                     const uint32_t col = min(l0 + ls + i * LPI, a.L - 1);
                     if (t0 < a.K) {                            // K is a multiple of N on this path
                         const Vec16<T>* p = reinterpret_cast<const Vec16<T>*>(src + (int64_t)col * a.istride[0]);
-                        grp[i] = rt_ld16(p);
+                        grp[i] = rt_ld16_dyn(p, a.nt_xt != 0);
                     } else {
                         grp[i] = Vec16<T>{};
                     }
@@ -320,9 +321,13 @@ bool tile_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* l, const 
         // every vector starts at (base + multiples of N) for an ascending dim t, and ends there for a descending one
         const T* first = ts > 0 ? xbase : xbase - (N - 1);
         bool ok = (reinterpret_cast<uintptr_t>(first) & 15) == 0 && (a.K % (uint32_t)N) == 0 && TK % (uint32_t)N == 0;
-        for (int k = 0; k < rank; ++k)
+        bool xstream = true;
+        for (int k = 0; k < rank; ++k) {
             if (k != tdim) ok = ok && mult_of(dsc.stride[xt][k], N);
+            xstream = xstream && dsc.stride[xt][k] != 0;
+        }
         vec_gather = ok;
+        a.nt_xt = xstream ? 1u : 0u;
     }
     const uint64_t blocks = outer * a.nchunks * a.ktiles * a.ltiles;
     if (blocks >= (1ull << 31)) return false;

@@ -140,8 +140,7 @@ typedef uint32_t rt_u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 template <int ES> struct rt_uvec { typedef rt_u32x4_a4 type; };
 template <> struct rt_uvec<1> { typedef rt_u32x4_a1 type; };
 template <> struct rt_uvec<2> { typedef rt_u32x4_a2 type; };
-// NT is a compile-time choice on purpose: written as `nt ? nontemporal_load(q) : *q` the two loads of one address are merged
-// into a single plain load and the hint is lost.
+// NT is a compile-time choice on purpose (see rt_ld16_dyn for why a plain ternary will not do).
 template <class T, bool NT> __device__ __forceinline__ rt_u32x4 rt_ld16u(const T* p) {
     typedef typename rt_uvec<(int)sizeof(T)>::type U;
     const U* q = reinterpret_cast<const U*>(p);
@@ -158,6 +157,18 @@ template <class T> __device__ __forceinline__ void rt_st16u_nt(T* p, rt_u32x4 v)
     typedef typename rt_uvec<(int)sizeof(T)>::type U;
     U r = {v.x, v.y, v.z, v.w};
     __builtin_nontemporal_store(r, reinterpret_cast<U*>(p));
+}
+
+// Aligned 16-byte load whose non-temporal hint is a wave-uniform run-time flag: two real branches.  The pointer of the
+// non-temporal branch passes through an empty asm statement, because written as `nt ? nontemporal_load(q) : *q` the two loads of
+// one address can be merged into a single plain load.
+template <class V> __device__ __forceinline__ V rt_ld16_dyn(const V* p, bool nt) {
+    if (nt) {
+        const V* q = p;
+        asm volatile("" : "+v"(q));
+        return rt_ld16_nt(q);
+    }
+    return rt_ld16(p);
 }
 
 // Four 1-byte integers packed in a 32-bit word, wrapping add / subtract of every byte at once: the low seven bits are
