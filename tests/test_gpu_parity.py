@@ -1016,7 +1016,7 @@ def test_reduction_shapes_short_rows_narrow_columns_short_axis(hip, dtype):
         for R, outer in ((64, 3), (1000, 1), (5003, 2), (70001, 1)):
             _check_reduce(hip, dtype, outer, R, inner, rng, offset=int(rng.integers(0, 5)))
     for R in (1, 2, 4, 5, 16, 31, 32, 33):
-        for inner, outer in ((2, 1000), (3, 1), (64, 50), (100, 7), (1024, 3), (1028, 2)):
+        for inner, outer in ((2, 1000), (3, 1), (64, 50), (100, 7), (1024, 3), (1028, 2), (5, 9), (7, 3), (257, 4), (1001, 2), (19, 40)):
             _check_reduce(hip, dtype, outer, R, inner, rng, offset=int(rng.integers(0, 5)))
     # wide rows whose length is not a multiple of the 16-byte vector (and starts that are not aligned): every lane still loads
     # whole vectors, the last one overlapping its neighbour
