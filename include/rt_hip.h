@@ -195,6 +195,20 @@ int32_t rt_argmax_nd(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, ui
                      uint64_t offset, int32_t rank, const uint64_t* shape, const int64_t* strides,
                      uint64_t* dst, uint64_t dst_len, int32_t dim);
 
+/* ---- reduction that allocates nothing -----------------------------------------------------------------------------------
+ * No counterpart in the reference.  For callers that cannot allocate device memory: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  Same arguments, validation, kernels and results (bit for bit) as rt_reduce_nd, but the
+ * partial results of a split reduction go to a workspace of RT_STATIC_SCRATCH_BYTES that is part of the library's device image
+ * (every device the library runs on holds it until the process ends) instead of the context's on-demand scratch buffer; the call
+ * performs no hipMalloc / hipFree.  A reduction whose partials do not fit is refused with RT_E_INVALID before anything is launched
+ * (partials = splits * outer * inner elements: sum / prod / max / min / mean of any shape stay below 1 MiB, e.g. 512 KiB for the
+ * axis-0 sum of (8192, 32768) f32; the statistics keep states of 8 .. 24 bytes per partial and can exceed it when many columns are
+ * split).  All calls on one device share the workspace: calls that overlap on one device (two contexts) race on it. */
+#define RT_STATIC_SCRATCH_BYTES (1u << 20)
+int32_t rt_reduce_nd_static(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, uint64_t src_len,
+                            uint64_t offset, int32_t rank, const uint64_t* shape, const int64_t* strides,
+                            void* dst, uint64_t dst_len, int32_t dim);
+
 /* ---- out-of-place unary / scalar ops ---------------------------------------------------------------------------------
  * dst[0 .. len) = op(src[start .. start + len)); the source is only read.  The trait has in-place ops only: `tensor.relu()`,
  * `tensor * 3.0` and the other value-returning forms clone the tensor and then run the in-place op (ops/unary/mod.rs:114-126,

@@ -43,6 +43,11 @@ struct rt_ctx {
     // scratch for two-stage reductions (partials), grown on demand, reused across calls
     void* scratch = nullptr;
     size_t scratch_bytes = 0;
+    // While `fixed_only` is set (for the duration of one call of the entry point that allocates nothing, under `mu`) rt_scratch hands
+    // out `fixed_scratch` (fixed_scratch_bytes long) and refuses anything larger instead of growing `scratch`.
+    void* fixed_scratch = nullptr;
+    size_t fixed_scratch_bytes = 0;
+    bool fixed_only = false;
     // pinned staging ring for large host<->device transfers (allocated by the first one), one event per slot
     void* stage[4] = {nullptr, nullptr, nullptr, nullptr};
     hipEvent_t stage_ev[4] = {nullptr, nullptr, nullptr, nullptr};

@@ -159,6 +159,13 @@ int32_t rt_free_locked(rt_ctx* ctx, void* p) {
 }
 
 int32_t rt_scratch(rt_ctx* ctx, size_t bytes, void** out) {
+    if (ctx->fixed_only) {
+        if (bytes > ctx->fixed_scratch_bytes)
+            return rt_fail(RT_E_INVALID, "this reduction needs %zu bytes of partial results; the built-in workspace of the entry point "
+                           "that allocates nothing holds %zu (use rt_reduce_nd)", bytes, ctx->fixed_scratch_bytes);
+        *out = ctx->fixed_scratch;
+        return RT_OK;
+    }
     if (bytes > ctx->scratch_bytes) {
         if (ctx->scratch) {
             RT_HIP(hipStreamSynchronize(ctx->stream));

@@ -231,6 +231,12 @@ class Hip:
         _check(lib.rt_reduce_nd(self._ctx, sb.dtype, REDUCE[op], sb.ptr, sb.len, off, len(shape), _u64s(shape), _i64s(strides),
                                 dst.ptr, dst.len, dim))
 
+    def apply_reduce_contiguous_nd_static(self, src: Tuple[HipBuf, tuple], dst: HipBuf, dim: int, op: str):
+        """rt_reduce_nd_static: the same reduction with its partial results in the library's built-in workspace (no allocation)."""
+        sb, (off, shape, strides) = src
+        _check(lib.rt_reduce_nd_static(self._ctx, sb.dtype, REDUCE[op], sb.ptr, sb.len, off, len(shape), _u64s(shape), _i64s(strides),
+                                       dst.ptr, dst.len, dim))
+
     # Backend::apply_argmax_contiguous_flat / _nd (backend/mod.rs:412-463): dst is a u64 buffer
     def apply_argmax_contiguous_flat(self, src: HipBuf, dst: HipBuf, start: int, length: int, op: str):
         if dst.dtype != U64:
