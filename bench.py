@@ -509,14 +509,15 @@ def main():
     w = Workloads(hip)
 
     if args.kernel:
-        fn, nbytes, nelem = getattr(w, args.kernel)()
-        preheat(hip, [fn], args.preheat)
-        mean, med, mn = time_kernel(hip, fn, args.steps, args.warmup)
-        rec = {"kernel": args.kernel, "ms_mean": mean, "ms_median": med, "ms_min": mn, "bytes": nbytes,
-               "GBps": nbytes / (mean * 1e-3) / 1e9, "frac_of_peak": nbytes / (mean * 1e-3) / PEAK_HBM}
-        if hasattr(fn, "flops"):
-            rec["TFLOPs"] = fn.flops / (mean * 1e-3) / 1e12
-        print(json.dumps(rec))
+        for name in args.kernel.split(","):                    # several names: one after the other in this process
+            fn, nbytes, nelem = getattr(w, name)()
+            preheat(hip, [fn], args.preheat)
+            mean, med, mn = time_kernel(hip, fn, args.steps, args.warmup)
+            rec = {"kernel": name, "ms_mean": mean, "ms_median": med, "ms_min": mn, "bytes": nbytes,
+                   "GBps": nbytes / (mean * 1e-3) / 1e9, "frac_of_peak": nbytes / (mean * 1e-3) / PEAK_HBM}
+            if hasattr(fn, "flops"):
+                rec["TFLOPs"] = fn.flops / (mean * 1e-3) / 1e12
+            print(json.dumps(rec), flush=True)
         return
 
     # ---- headline step ---------------------------------------------------------------------------------------------------

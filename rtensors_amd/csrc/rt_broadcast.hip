@@ -22,10 +22,10 @@ namespace {
 
 // ---- contig ---------------------------------------------------------------------------------------------------------
 // One vector per lane, non-temporal loads and stores: every byte is touched exactly once.
+constexpr int kCBlock2 = 256;
 template <class T, int OP>
-__global__ __launch_bounds__(kRBlock) void bin_contig_kernel(const Vec16<T>* l, const Vec16<T>* r, Vec16<T>* d, size_t nvec, uint32_t head,
-                                                             uint32_t tail) {
-    const size_t i = (size_t)blockIdx.x * kRBlock + threadIdx.x;
+__global__ __launch_bounds__(kCBlock2) void bin_contig_kernel(const Vec16<T>* l, const Vec16<T>* r, Vec16<T>* d, size_t nvec, uint32_t head,
+                                                              uint32_t tail, TileMap m) {
     // the `head` elements before and the `tail` elements after the aligned body (fewer than a vector each; all three operands
     // share the phase) are taken by lanes of the first and the last block instead of launches of their own
     auto edge = [&](int64_t e) {
@@ -36,7 +36,8 @@ __global__ __launch_bounds__(kRBlock) void bin_contig_kernel(const Vec16<T>* l, 
     };
     if (blockIdx.x == 0 && threadIdx.x < head) edge((int64_t)threadIdx.x - (int64_t)head);
     if (blockIdx.x == gridDim.x - 1 && threadIdx.x < tail) edge((int64_t)(nvec * (16 / sizeof(T))) + (int64_t)threadIdx.x);
-    if (i >= nvec) return;
+    size_t i;
+    if (!rt_tile_index(m, blockIdx.x, kCBlock2, threadIdx.x, nvec, &i)) return;     // a block owns a quarter of four pages (see TileMap)
     Vec16<T> a = rt_ld16_nt(l + i);
     Vec16<T> b;
     if constexpr (OP != kOpCopy) b = rt_ld16_nt(r + i); else b = a;
@@ -63,7 +64,7 @@ struct RowArgs {
 };
 
 template <class T, int OP, int LM, int RM, int GU>
-__global__ __launch_bounds__(kRBlock) void bin_rows_kernel(const T* l, const T* r, T* d, RowArgs a) {
+__global__ __launch_bounds__(256) void bin_rows_kernel(const T* l, const T* r, T* d, RowArgs a) {
     constexpr int N = 16 / sizeof(T);
     // blockIdx -> (outer index, chunk of the loop dim, column tile); all uniform, computed on the scalar unit
     uint32_t b = blockIdx.x;
@@ -72,22 +73,12 @@ __global__ __launch_bounds__(kRBlock) void bin_rows_kernel(const T* l, const T* 
     b = q;
     q = fd_div(b, a.nchunks_div);
     const uint32_t chunk = b - q * a.nchunks;
-    uint32_t rem = q;
-    int64_t ol = 0, orr = 0, od = 0;
-#pragma unroll
-    for (int k = RT_MAX_RANK - 1; k >= 0; --k) {
-        if (k < a.nouter) {
-            uint32_t qq = fd_div(rem, a.odiv[k]);
-            uint32_t c = rem - qq * a.oshape[k];
-            ol += (int64_t)c * a.ostride[0][k];
-            orr += (int64_t)c * a.ostride[1][k];
-            od += (int64_t)c * a.ostride[2][k];
-            rem = qq;
-        }
-    }
+    int64_t off3[3];
+    rt_outer_offsets<3>(q, a.nouter, a.oshape, a.odiv, a.ostride, off3);
+    const int64_t ol = off3[0], orr = off3[1], od = off3[2];
     const uint32_t tx = threadIdx.x & (a.tpr - 1);
     const uint32_t ty = threadIdx.x / a.tpr;
-    const uint32_t gy = kRBlock / a.tpr;
+    const uint32_t gy = blockDim.x / a.tpr;
     const uint32_t c = (tile * a.tpr + tx) * N;                 // first column of this lane's vector
     if (c >= a.L) return;
     const uint32_t g_begin = chunk * a.gchunk;
@@ -157,6 +148,59 @@ __global__ __launch_bounds__(kRBlock) void bin_rows_kernel(const T* l, const T* 
                 dp[k] = bin_apply<OP, T>(lp[(int64_t)k * a.istride[0]], rp[(int64_t)k * a.istride[1]]);
         }
     }
+}
+
+// ---- rows, lean form ------------------------------------------------------------------------------------------------------
+// The common case of the row kernel -- rows of at least 1 KiB, no gathered input, at most two outer dims besides the loop dim,
+// rows not shifted to a line boundary -- with as little work per wave as possible: a 256-lane block owns the same 1 KiB piece of
+// four consecutive rows, one wave per row, one vector per lane, and the next block owns the next piece of the same rows (the tiled
+// order described at TileMap).  All kernel arguments are fetched in one batch, the row index is wave-uniform and every offset is
+// computed on the scalar unit.  Config 3 (x (16,1,512,1024) + y (1,64,1,1024), 2 GiB out): 0.90 of peak in this shape when a
+// wave's life is one load-add-store; the general kernel above spends longer decoding its descriptor than a wave may live.
+struct Rows4Args {
+    uint32_t L, G, tiles;
+    FastDiv32 tiles_div;
+    int32_t gs[3], o0s[3], o1s[3];       // strides of left, right, dst along the loop dim and the two outer dims (inner one first)
+};
+
+// grid: x = column tile + tiles * (chunk of four rows), y = index along the inner outer dim, z = index along the outer one.  Every
+// offset inside an operand fits 32 bits (checked on the host).
+template <class T, int OP, int LM, int RM>
+__global__ __launch_bounds__(256) void bin_rows4_kernel(const T* l, const T* r, T* d, Rows4Args a) {
+    constexpr int N = 16 / sizeof(T);
+    uint32_t L = a.L, G = a.G, tiles = a.tiles, tm = a.tiles_div.mul, ts = a.tiles_div.shift;
+    int32_t g0 = a.gs[0], g1 = a.gs[1], g2 = a.gs[2], p0 = a.o0s[0], p1 = a.o0s[1], p2 = a.o0s[2], q0 = a.o1s[0], q1 = a.o1s[1], q2 = a.o1s[2];
+    RT_PIN(L); RT_PIN(G); RT_PIN(tiles); RT_PIN(tm); RT_PIN(ts);
+    RT_PIN(g0); RT_PIN(g1); RT_PIN(g2); RT_PIN(p0); RT_PIN(p1); RT_PIN(p2); RT_PIN(q0); RT_PIN(q1); RT_PIN(q2);
+    RT_TOUCH(l); RT_TOUCH(r); RT_TOUCH(d);
+    const uint32_t chunk = (uint32_t)(((uint64_t)__umulhi(blockIdx.x, tm) + blockIdx.x) >> ts);
+    const uint32_t tile = blockIdx.x - chunk * tiles;
+    const int32_t i0 = (int32_t)blockIdx.y, i1 = (int32_t)blockIdx.z;
+    const uint32_t g = chunk * 4 + (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    if (g >= G) return;
+    const T* lp = l + (i1 * q0 + i0 * p0 + (int32_t)g * g0);
+    const T* rp = r + (i1 * q1 + i0 * p1 + (int32_t)g * g1);
+    T* dp = d + (i1 * q2 + i0 * p2 + (int32_t)g * g2);
+    const uint32_t c = (tile * 64 + (threadIdx.x & 63)) * N;
+    if (c >= L) return;
+    if (c + N <= L) {
+        const rt_u32x4 x = load_raw<T, LM>(lp, c, 1);
+        rt_u32x4 y = x;
+        if constexpr (OP != kOpCopy) y = load_raw<T, RM>(rp, c, 1);
+        Vec16<T> xv = __builtin_bit_cast(Vec16<T>, x);
+        bin_apply_vec<OP, T>(xv, __builtin_bit_cast(Vec16<T>, y));
+        rt_st16u_nt<T>(dp + c, __builtin_bit_cast(rt_u32x4, xv));
+    } else {
+        for (uint32_t k = c; k < L; ++k) dp[k] = bin_apply<OP, T>(lp[LM == M_VEC ? k : 0], rp[RM == M_VEC ? k : 0]);
+    }
+}
+
+template <class T, int OP>
+void launch_rows4(int lm, int rm, dim3 grid, hipStream_t s, const T* l, const T* r, T* d, const Rows4Args& a) {
+    if (lm == M_VEC && rm == M_VEC) hipLaunchKernelGGL((bin_rows4_kernel<T, OP, M_VEC, M_VEC>), grid, dim3(256), 0, s, l, r, d, a);
+    else if (lm == M_VEC) hipLaunchKernelGGL((bin_rows4_kernel<T, OP, M_VEC, M_BCAST>), grid, dim3(256), 0, s, l, r, d, a);
+    else if (rm == M_VEC) hipLaunchKernelGGL((bin_rows4_kernel<T, OP, M_BCAST, M_VEC>), grid, dim3(256), 0, s, l, r, d, a);
+    else hipLaunchKernelGGL((bin_rows4_kernel<T, OP, M_BCAST, M_BCAST>), grid, dim3(256), 0, s, l, r, d, a);
 }
 
 // ---- generic ------------------------------------------------------------------------------------------------------------
@@ -283,10 +327,12 @@ __global__ __launch_bounds__(kRBlock) void bin_flat_kernel(const T* l, const T* 
 // (bias add): a lane owns one 16-byte vector of dst, reads the streamed input at the same position and the row at position
 // v mod (L / N) -- the shape of the plain copy kernel plus one cached load.
 template <class T, int OP, bool ROW_IS_LEFT>
-__global__ __launch_bounds__(kRBlock) void bin_flat_row_kernel(const T* __restrict__ flat, const T* __restrict__ row, T* __restrict__ d, uint32_t nvec,
-                                                               uint32_t row_vecs, FastDiv32 row_div) {
-    const uint32_t v = blockIdx.x * kRBlock + threadIdx.x;
-    if (v >= nvec) return;
+__global__ __launch_bounds__(kCBlock2) void bin_flat_row_kernel(const T* flat, const T* __restrict__ row, T* d, uint32_t nvec, uint32_t row_vecs,
+                                                                FastDiv32 row_div, TileMap m) {
+    // `flat` and `d` may be the same buffer (in-place form): every lane reads its vector before it writes it
+    size_t vi;
+    if (!rt_tile_index(m, blockIdx.x, kCBlock2, threadIdx.x, nvec, &vi)) return;
+    const uint32_t v = (uint32_t)vi;
     Vec16<T> x = rt_ld16_nt(reinterpret_cast<const Vec16<T>*>(flat) + v);
     Vec16<T> y;
     if (row_vecs == 0) {                                          // the "row" is a single element (tensor op one-element tensor)
@@ -322,27 +368,27 @@ __global__ __launch_bounds__(kBlock) void bin_generic64_kernel(const T* l, const
 
 // ---- host: kernel choice ----------------------------------------------------------------------------------------------
 template <class T, int OP, int LM, int RM>
-void launch_rows_g(bool batched, dim3 grid, hipStream_t s, const T* l, const T* r, T* d, const RowArgs& a) {
+void launch_rows_g(bool batched, dim3 grid, unsigned bs, hipStream_t s, const T* l, const T* r, T* d, const RowArgs& a) {
     // the batched long-loop form is only ever chosen when one input is gathered element-wise
     if constexpr (LM == M_ELEM || RM == M_ELEM) {
-        if (batched) { hipLaunchKernelGGL((bin_rows_kernel<T, OP, LM, RM, 4>), grid, dim3(kRBlock), 0, s, l, r, d, a); return; }
+        if (batched) { hipLaunchKernelGGL((bin_rows_kernel<T, OP, LM, RM, 4>), grid, dim3(bs), 0, s, l, r, d, a); return; }
     }
-    hipLaunchKernelGGL((bin_rows_kernel<T, OP, LM, RM, 1>), grid, dim3(kRBlock), 0, s, l, r, d, a);
+    hipLaunchKernelGGL((bin_rows_kernel<T, OP, LM, RM, 1>), grid, dim3(bs), 0, s, l, r, d, a);
 }
 template <class T, int OP, int LM>
-void launch_rows_r(int rm, bool batched, dim3 grid, hipStream_t s, const T* l, const T* r, T* d, const RowArgs& a) {
+void launch_rows_r(int rm, bool batched, dim3 grid, unsigned bs, hipStream_t s, const T* l, const T* r, T* d, const RowArgs& a) {
     switch (rm) {
-        case M_VEC: launch_rows_g<T, OP, LM, M_VEC>(batched, grid, s, l, r, d, a); break;
-        case M_BCAST: launch_rows_g<T, OP, LM, M_BCAST>(batched, grid, s, l, r, d, a); break;
-        default: launch_rows_g<T, OP, LM, M_ELEM>(batched, grid, s, l, r, d, a); break;
+        case M_VEC: launch_rows_g<T, OP, LM, M_VEC>(batched, grid, bs, s, l, r, d, a); break;
+        case M_BCAST: launch_rows_g<T, OP, LM, M_BCAST>(batched, grid, bs, s, l, r, d, a); break;
+        default: launch_rows_g<T, OP, LM, M_ELEM>(batched, grid, bs, s, l, r, d, a); break;
     }
 }
 template <class T, int OP>
-void launch_rows(int lm, int rm, bool batched, dim3 grid, hipStream_t s, const T* l, const T* r, T* d, const RowArgs& a) {
+void launch_rows(int lm, int rm, bool batched, dim3 grid, unsigned bs, hipStream_t s, const T* l, const T* r, T* d, const RowArgs& a) {
     switch (lm) {
-        case M_VEC: launch_rows_r<T, OP, M_VEC>(rm, batched, grid, s, l, r, d, a); break;
-        case M_BCAST: launch_rows_r<T, OP, M_BCAST>(rm, batched, grid, s, l, r, d, a); break;
-        default: launch_rows_r<T, OP, M_ELEM>(rm, batched, grid, s, l, r, d, a); break;
+        case M_VEC: launch_rows_r<T, OP, M_VEC>(rm, batched, grid, bs, s, l, r, d, a); break;
+        case M_BCAST: launch_rows_r<T, OP, M_BCAST>(rm, batched, grid, bs, s, l, r, d, a); break;
+        default: launch_rows_r<T, OP, M_ELEM>(rm, batched, grid, bs, s, l, r, d, a); break;
     }
 }
 
@@ -370,12 +416,13 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
             size_t head = ((128 - (reinterpret_cast<uintptr_t>(dp) & 127)) & 127) / sizeof(T);
             if (head > n) head = n;
             size_t nvec = (n - head) / N, tail = n - head - nvec * N;
-            size_t blocks = (nvec + (size_t)kRBlock - 1) / (size_t)kRBlock;
+            const TileMap m = rt_make_tilemap(dp + head, nvec, kCBlock2);
+            size_t blocks = rt_tilemap_blocks(m, nvec, kCBlock2);
             if (blocks < 1) blocks = 1;                            // fewer elements than a vector: edges only
             if (blocks > 0x7fffffffull) return rt_fail(RT_E_INVALID, "broadcast: %zu elements is too long for one launch", n);
-            hipLaunchKernelGGL((bin_contig_kernel<T, OP>), dim3((unsigned)blocks), dim3(kRBlock), 0, s,
+            hipLaunchKernelGGL((bin_contig_kernel<T, OP>), dim3((unsigned)blocks), dim3(kCBlock2), 0, s,
                                reinterpret_cast<const Vec16<T>*>(lp + head), reinterpret_cast<const Vec16<T>*>(rp + head),
-                               reinterpret_cast<Vec16<T>*>(dp + head), nvec, (uint32_t)head, (uint32_t)tail);
+                               reinterpret_cast<Vec16<T>*>(dp + head), nvec, (uint32_t)head, (uint32_t)tail, m);
             RT_HIP(hipGetLastError());
             return RT_OK;
         }
@@ -426,9 +473,10 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
                 if (!(is_row || is_scalar) || !row_major_run(o) || (reinterpret_cast<uintptr_t>(fo) & 15)) continue;
                 if (!is_scalar && (reinterpret_cast<uintptr_t>(ro) & 15)) continue;
                 const uint32_t nvec = (uint32_t)(count / N), row_vecs = is_scalar ? 0u : (uint32_t)(dsc.shape[rank - 1] / N);
-                dim3 grid((nvec + kRBlock - 1) / kRBlock), blk(kRBlock);
-                if (p == 0) hipLaunchKernelGGL((bin_flat_row_kernel<T, OP, true>), grid, blk, 0, s, fo, ro, d + dsc.offset[2], nvec, row_vecs, make_fastdiv(row_vecs ? row_vecs : 1u));
-                else hipLaunchKernelGGL((bin_flat_row_kernel<T, OP, false>), grid, blk, 0, s, fo, ro, d + dsc.offset[2], nvec, row_vecs, make_fastdiv(row_vecs ? row_vecs : 1u));
+                const TileMap m = rt_make_tilemap(d + dsc.offset[2], nvec, kCBlock2);
+                dim3 grid((unsigned)rt_tilemap_blocks(m, nvec, kCBlock2)), blk(kCBlock2);
+                if (p == 0) hipLaunchKernelGGL((bin_flat_row_kernel<T, OP, true>), grid, blk, 0, s, fo, ro, d + dsc.offset[2], nvec, row_vecs, make_fastdiv(row_vecs ? row_vecs : 1u), m);
+                else hipLaunchKernelGGL((bin_flat_row_kernel<T, OP, false>), grid, blk, 0, s, fo, ro, d + dsc.offset[2], nvec, row_vecs, make_fastdiv(row_vecs ? row_vecs : 1u), m);
                 RT_HIP(hipGetLastError());
                 return RT_OK;
             }
@@ -515,6 +563,34 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
         uint32_t vecs = (uint32_t)((a.L + N - 1) / N);
         uint32_t tpr = 1;
         while (tpr < vecs && tpr < (uint32_t)kRBlock) tpr <<= 1;
+        // the lean form: rows of 1 KiB and more, no gathered input, at most two outer dims (of at most 65535 each), rows not shifted,
+        // every offset inside an operand below 2^31
+        if (steps == 2 && vecs >= 64 && a.G >= 4 && lead == 0 && rank <= 4 && lm != M_ELEM && rm != M_ELEM) {
+            bool fits = true;
+            for (int o = 0; o < 3; ++o) {
+                uint64_t reach = 0;
+                for (int k = 0; k < rank; ++k) reach += (uint64_t)(dsc.shape[k] - 1) * (uint64_t)(dsc.stride[o][k] < 0 ? -dsc.stride[o][k] : dsc.stride[o][k]);
+                fits = fits && reach < (1ull << 31);
+            }
+            const uint64_t n0 = rank >= 3 ? (uint64_t)dsc.shape[rank - 3] : 1ull, n1 = rank >= 4 ? (uint64_t)dsc.shape[rank - 4] : 1ull;
+            Rows4Args q;
+            memset(&q, 0, sizeof(q));
+            q.L = (uint32_t)dsc.shape[rank - 1];
+            q.G = a.G;
+            q.tiles = (vecs + 63) / 64;
+            q.tiles_div = make_fastdiv(q.tiles);
+            const uint64_t gx = (uint64_t)q.tiles * ((a.G + 3) / 4);
+            if (fits && n0 <= 65535 && n1 <= 65535 && gx < (1ull << 31)) {
+                for (int o = 0; o < 3; ++o) {
+                    q.gs[o] = (int32_t)dsc.stride[o][rank - 2];
+                    q.o0s[o] = rank >= 3 ? (int32_t)dsc.stride[o][rank - 3] : 0;
+                    q.o1s[o] = rank >= 4 ? (int32_t)dsc.stride[o][rank - 4] : 0;
+                }
+                launch_rows4<T, OP>(lm, rm, dim3((unsigned)gx, (unsigned)n0, (unsigned)n1), s, l + dsc.offset[0], r + dsc.offset[1], d + dsc.offset[2], q);
+                RT_HIP(hipGetLastError());
+                return RT_OK;
+            }
+        }
         a.tpr = tpr;
         a.tiles = (vecs + tpr - 1) / tpr;
         const uint32_t gy = kRBlock / tpr;
@@ -528,7 +604,7 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
         const uint64_t blocks = outer * a.nchunks * a.tiles;
         if (blocks < (1ull << 31)) {
             // the operand pointers address column 0 of the moved origin (never dereferenced below column `lead`)
-            launch_rows<T, OP>(lm, rm, steps > 2, dim3((unsigned)blocks), s, l + dsc.offset[0] - (int64_t)lead * a.istride[0],
+            launch_rows<T, OP>(lm, rm, steps > 2, dim3((unsigned)blocks), kRBlock, s, l + dsc.offset[0] - (int64_t)lead * a.istride[0],
                                r + dsc.offset[1] - (int64_t)lead * a.istride[1], d + dsc.offset[2] - (int64_t)lead, a);
             RT_HIP(hipGetLastError());
             return RT_OK;

@@ -63,19 +63,9 @@ __global__ __launch_bounds__(kTBlock) void bin_tile_kernel(const T* xt, const T*
     b = q;
     q = fd_div(b, a.nchunks_div);
     const uint32_t chunk = b - q * a.nchunks;
-    uint32_t rem = q;
-    int64_t offx = 0, offo = 0, offd = 0;
-#pragma unroll
-    for (int k = RT_MAX_RANK - 1; k >= 0; --k) {
-        if (k < a.nouter) {
-            uint32_t qq = fd_div(rem, a.odiv[k]);
-            uint32_t c = rem - qq * a.oshape[k];
-            offx += (int64_t)c * a.ostride[0][k];
-            offo += (int64_t)c * a.ostride[1][k];
-            offd += (int64_t)c * a.ostride[2][k];
-            rem = qq;
-        }
-    }
+    int64_t off3[3];
+    rt_outer_offsets<3>(q, a.nouter, a.oshape, a.odiv, a.ostride, off3);
+    const int64_t offx = off3[0], offo = off3[1], offd = off3[2];
     xt += offx;
     xo += offo;
     T* dp = d + offd;
@@ -120,23 +110,24 @@ __global__ __launch_bounds__(kTBlock) void bin_tile_kernel(const T* xt, const T*
                 constexpr int GPI = kTBlock / VT;              // groups of P inner-dim positions covered per iteration
                 constexpr int IT = TL / (GPI * P);
                 const uint32_t tq = threadIdx.x % VT, lg = threadIdx.x / VT;
-                const uint32_t t0 = k0 + tq * N;
+                // K is a multiple of N on this path; tile rows past the end of dim t hold a repeat of its last vector and are never stored
+                const uint32_t t0 = min(k0 + tq * N, a.K - N);
                 const bool fwd = a.tstride[0] > 0;
                 const T* src = xg + (fwd ? (int64_t)t0 : -(int64_t)(t0 + N - 1));
                 rt_u32x4 grp[IT][P];
+                // one branch on the launch-wide non-temporal hint around all loads, so that they are in flight together
+                auto load_all = [&](auto nt_c) {
 #pragma unroll
-                for (int i = 0; i < IT; ++i) {
+                    for (int i = 0; i < IT; ++i) {
 #pragma unroll
-                    for (int p = 0; p < P; ++p) {
-                        const uint32_t col = min(l0 + (lg + i * GPI) * P + p, a.L - 1);
-                        if (t0 < a.K) {                        // K is a multiple of N on this path
+                        for (int p = 0; p < P; ++p) {
+                            const uint32_t col = min(l0 + (lg + i * GPI) * P + p, a.L - 1);
                             const rt_u32x4* q4 = reinterpret_cast<const rt_u32x4*>(src + (int64_t)col * a.istride[0]);
-                            grp[i][p] = rt_ld16_dyn(q4, a.nt_xt != 0);
-                        } else {
-                            grp[i][p] = rt_u32x4{0, 0, 0, 0};
+                            if constexpr (decltype(nt_c)::value) grp[i][p] = rt_ld16_nt(q4); else grp[i][p] = rt_ld16(q4);
                         }
                     }
-                }
+                };
+                if (a.nt_xt) load_all(std::true_type{}); else load_all(std::false_type{});
 #pragma unroll
                 for (int i = 0; i < IT; ++i) {
                     const uint32_t colw = (lg + i * GPI) * P;
@@ -167,21 +158,21 @@ __global__ __launch_bounds__(kTBlock) void bin_tile_kernel(const T* xt, const T*
                 constexpr int LPI = kTBlock / VT;              // inner-dim positions covered per iteration
                 constexpr int IT = TL / LPI;
                 const uint32_t tq = threadIdx.x % VT, ls = threadIdx.x / VT;
-                const uint32_t t0 = k0 + tq * N;
+                // K is a multiple of N on this path; tile rows past the end of dim t hold a repeat of its last vector and are never stored
+                const uint32_t t0 = min(k0 + tq * N, a.K - N);
                 const bool fwd = a.tstride[0] > 0;
                 // lowest address of the vector: element t0 when dim t ascends in memory, element t0+N-1 when it descends
                 const T* src = xg + (fwd ? (int64_t)t0 : -(int64_t)(t0 + N - 1));
                 Vec16<T> grp[IT];
+                auto load_all = [&](auto nt_c) {
 #pragma unroll
-                for (int i = 0; i < IT; ++i) {
-                    const uint32_t col = min(l0 + ls + i * LPI, a.L - 1);
-                    if (t0 < a.K) {                            // K is a multiple of N on this path
+                    for (int i = 0; i < IT; ++i) {
+                        const uint32_t col = min(l0 + ls + i * LPI, a.L - 1);
                         const Vec16<T>* p = reinterpret_cast<const Vec16<T>*>(src + (int64_t)col * a.istride[0]);
-                        grp[i] = rt_ld16_dyn(p, a.nt_xt != 0);
-                    } else {
-                        grp[i] = Vec16<T>{};
+                        if constexpr (decltype(nt_c)::value) grp[i] = rt_ld16_nt(p); else grp[i] = rt_ld16(p);
                     }
-                }
+                };
+                if (a.nt_xt) load_all(std::true_type{}); else load_all(std::false_type{});
 #pragma unroll
                 for (int i = 0; i < IT; ++i) {
 #pragma unroll
@@ -242,6 +233,130 @@ __global__ __launch_bounds__(kTBlock) void bin_tile_kernel(const T* xt, const T*
     }
 }
 
+
+// ---- staged kernel: 4- and 8-byte elements, vector gather -------------------------------------------------------------------------
+// The same job as bin_tile_kernel in the shape that measured fastest for 4-byte elements on MI355X: 512 lanes, a tile of 16 rows
+// (along dim t) by 64 vectors (1 KiB) of dst's inner dim, two stores per lane and no loop over other dims -- a dim along which the
+// transposed input does not move is just one more outer dim, so blocks that run together write one compact window of dst and the
+// transposed input's tile is re-read from cache for every index of that dim.  (Keeping the tile for several indices of such a dim
+// makes every lane store to places megabytes apart: config 3b, x (16,1,512,1024) permuted + reversed plus y (1,64,1,1024): 0.90 of
+// peak with one index per block, 0.82 with two, 0.73 with four, 0.76 for the row kernel that gathers x element-wise and keeps it
+// in registers for 16 indices.)  The gather reads N vectors of N elements along dim t, transposes the N x N block in registers and
+// writes N whole vectors to LDS.
+constexpr int kSVecs = 64;                    // tile columns in 16-byte vectors (one wave writes one row piece)
+// Tile rows (along dim t), two per wave.  WIDE = 32 rows of 4-byte elements, 1024 lanes: a whole 128-byte line of the transposed
+// input per inner-dim position, for an input that is streamed from memory once (16384^2 f32: a + b.transpose() 0.74 -> 0.79 of
+// peak, transposing copy 0.68 -> 0.76 against 16 rows).  Otherwise 16 rows, 512 lanes: an input that is re-read from cache for
+// every index of a dim along which it does not move (config 3b: 0.89 with 16 rows, 0.87 with 32).
+template <class T, bool WIDE> struct StageGeom {
+    static constexpr int kRows = (WIDE && sizeof(T) == 4) ? 32 : 16;
+    static constexpr int kWaves = kRows / 2;
+    static constexpr int kBlock = kWaves * RT_WAVE;
+};
+
+// At most two outer dims besides dim t and the inner dim; everything a wave needs from the kernel arguments is fetched in one batch.
+struct StageArgs {
+    uint32_t L, K, ltiles;
+    FastDiv32 ltiles_div;
+    // strides by role (0 = the transposed input, 1 = the other input, 2 = dst) along dim t, the inner dim and the two outer dims;
+    // every offset inside an operand fits 32 bits (checked on the host)
+    int32_t ts[3], is[3], o0s[3], o1s[3];
+    uint32_t x_is_left, nt_xt;
+};
+
+// grid: x = inner-dim tile + ltiles * (tile along t), y = index along the inner outer dim, z = index along the outer one
+template <class T, int OP, int OM, bool WIDE>
+__global__ __launch_bounds__((StageGeom<T, WIDE>::kBlock)) void bin_stage_kernel(const T* xt, const T* xo, T* d, StageArgs a) {
+    constexpr int N = 16 / sizeof(T);
+    constexpr int kSRows = StageGeom<T, WIDE>::kRows, kSWaves = StageGeom<T, WIDE>::kWaves, kSBlock = StageGeom<T, WIDE>::kBlock;
+    constexpr int TK = kSRows, TL = kSVecs * N, KQ = TK / N, NU = kSVecs * KQ, RPL = TK / kSWaves;
+    static_assert(TK % N == 0 && TK % kSWaves == 0, "tile shape");
+    __shared__ alignas(16) T tile[TK][TL + N];
+    uint32_t L = a.L, K = a.K, ltiles = a.ltiles, x_left = a.x_is_left, nt_xt = a.nt_xt, lm = a.ltiles_div.mul, lsh = a.ltiles_div.shift;
+    int32_t ts0 = a.ts[0], ts1 = a.ts[1], ts2 = a.ts[2], is0 = a.is[0], is1 = a.is[1];
+    int32_t p0 = a.o0s[0], p1 = a.o0s[1], p2 = a.o0s[2], q0 = a.o1s[0], q1 = a.o1s[1], q2 = a.o1s[2];
+    RT_PIN(L); RT_PIN(K); RT_PIN(ltiles); RT_PIN(x_left); RT_PIN(nt_xt); RT_PIN(lm); RT_PIN(lsh);
+    RT_PIN(ts0); RT_PIN(ts1); RT_PIN(ts2); RT_PIN(is0); RT_PIN(is1);
+    RT_PIN(p0); RT_PIN(p1); RT_PIN(p2); RT_PIN(q0); RT_PIN(q1); RT_PIN(q2);
+    RT_TOUCH(xt); RT_TOUCH(xo); RT_TOUCH(d);
+    const uint32_t ktile = (uint32_t)(((uint64_t)__umulhi(blockIdx.x, lm) + blockIdx.x) >> lsh);
+    const uint32_t ltile = blockIdx.x - ktile * ltiles;
+    const int32_t i0 = (int32_t)blockIdx.y, i1 = (int32_t)blockIdx.z;
+    xt += i1 * q0 + i0 * p0;
+    xo += i1 * q1 + i0 * p1;
+    T* dp = d + (i1 * q2 + i0 * p2);
+    const uint32_t k0 = ktile * TK, l0 = ltile * TL;
+    const uint32_t lane = threadIdx.x & (RT_WAVE - 1);
+    const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x / RT_WAVE));
+    const uint32_t c = l0 + lane * N;
+    const bool full_vec = c + N <= L;
+    // rows of the other input, issued before the gather so that both are in flight together
+    Vec16<T> ov[RPL] = {};
+    if constexpr (OP != kOpCopy) {
+        if (full_vec) {
+#pragma unroll
+            for (int i = 0; i < RPL; ++i) {
+                const uint32_t k = min(k0 + wv * RPL + i, K - 1);
+                ov[i] = load_vec<T, OM>(xo + (int32_t)k * ts1, c, is1);
+            }
+        }
+    }
+    // (the non-temporal hint is a launch-wide fact: one branch around the whole gather, not one per load, so that all loads of a
+    // lane are in flight together)
+    auto gather = [&](auto nt_c) {
+        constexpr bool NTG = decltype(nt_c)::value;
+        const bool fwd = ts0 > 0;
+#pragma unroll
+        for (int u0 = 0; u0 < NU; u0 += kSBlock) {
+            const uint32_t v = u0 + threadIdx.x;
+            if (NU % kSBlock == 0 || v < (uint32_t)NU) {
+                const uint32_t lq = v / KQ, tq = v % KQ;
+                const uint32_t t0 = min(k0 + tq * N, K - N);        // K % N == 0 here; rows past the end of dim t are never stored
+                // lowest address of a vector: element t0 when dim t ascends in memory, element t0 + N - 1 when it descends
+                const T* src = xt + (fwd ? (int64_t)t0 : -(int64_t)(t0 + N - 1));
+                Vec16<T> g[N];
+#pragma unroll
+                for (int j = 0; j < N; ++j) {
+                    const uint32_t col = min(l0 + lq * N + j, L - 1);
+                    const Vec16<T>* gp = reinterpret_cast<const Vec16<T>*>(src + (int32_t)col * is0);
+                    if constexpr (NTG) g[j] = rt_ld16_nt(gp); else g[j] = rt_ld16(gp);
+                }
+#pragma unroll
+                for (int e = 0; e < N; ++e) {
+                    Vec16<T> w;
+#pragma unroll
+                    for (int j = 0; j < N; ++j) w.e[j] = g[j].e[e];
+                    *reinterpret_cast<Vec16<T>*>(&tile[tq * N + (fwd ? e : N - 1 - e)][lq * N]) = w;
+                }
+            }
+        }
+    };
+    if (nt_xt) gather(std::true_type{}); else gather(std::false_type{});
+    __syncthreads();
+    if (c >= L) return;
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) {
+        const uint32_t kk = wv * RPL + i;
+        if (k0 + kk >= K) continue;
+        T* drow = dp + (int32_t)(k0 + kk) * ts2;
+        if (full_vec) {
+            const Vec16<T> xv = *reinterpret_cast<const Vec16<T>*>(&tile[kk][lane * N]);
+            Vec16<T> out;
+            if (x_left) { out = xv; bin_apply_vec<OP, T>(out, ov[i]); }
+            else { out = ov[i]; bin_apply_vec<OP, T>(out, xv); }
+            rt_st16u_nt<T>(drow + c, __builtin_bit_cast(rt_u32x4, out));
+        } else {
+            // ragged end of a row: element accesses
+            for (uint32_t cc = c; cc < L; ++cc) {
+                T xe = tile[kk][cc - l0];
+                T oe = xe;
+                if constexpr (OP != kOpCopy) oe = (xo + (int32_t)(k0 + kk) * ts1)[(int32_t)cc * is1];
+                drow[cc] = x_left ? bin_apply<OP, T>(xe, oe) : bin_apply<OP, T>(oe, xe);
+            }
+        }
+    }
+}
+
 }  // namespace
 
 namespace rtb {
@@ -270,13 +385,78 @@ bool tile_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* l, const 
             if (dsc.stride[o][k] == 0 && dsc.shape[k] >= 8) return true;
         return false;
     };
-    if ((tl >= 0) == (tr >= 0) || hoistable(tl >= 0 ? 0 : 1)) return false;
+    if ((tl >= 0) == (tr >= 0)) return false;
     const int xt = tl >= 0 ? 0 : 1, o = 1 - xt, tdim = tl >= 0 ? tl : tr;
     int om;
     {
         int64_t is = dsc.stride[o][rank - 1];
         om = is == 0 ? (int)M_BCAST : (is == 1 ? (int)M_VEC : (int)M_ELEM);
     }
+    // 4- and 8-byte elements whose transposed input can be read with aligned 16-byte vectors along dim t: the staged kernel, also
+    // when that input does not move along some dim
+    if constexpr (sizeof(T) == 4 || sizeof(T) == 8) {
+        const T* xbase = (xt == 0 ? l : r) + dsc.offset[xt];
+        const int64_t ts = dsc.stride[xt][tdim];
+        const T* first = ts > 0 ? xbase : xbase - (N - 1);
+        bool ok = (reinterpret_cast<uintptr_t>(first) & 15) == 0 && dsc.shape[tdim] % N == 0;
+        bool xstream = true;
+        for (int k = 0; k < rank; ++k) {
+            if (k != tdim) ok = ok && mult_of(dsc.stride[xt][k], N);
+            xstream = xstream && dsc.stride[xt][k] != 0;
+        }
+        for (int q = 0; q < 3 && ok; ++q) {                       // 32-bit offsets inside every operand
+            uint64_t reach = 0;
+            for (int k = 0; k < rank; ++k) reach += (uint64_t)(dsc.shape[k] - 1) * (uint64_t)(dsc.stride[q][k] < 0 ? -dsc.stride[q][k] : dsc.stride[q][k]);
+            ok = reach < (1ull << 31);
+        }
+        if (ok && rank <= 4) {
+            StageArgs a;
+            memset(&a, 0, sizeof(a));
+            a.L = (uint32_t)dsc.shape[rank - 1];
+            a.K = (uint32_t)dsc.shape[tdim];
+            const int role[3] = {xt, o, 2};
+            a.x_is_left = xt == 0 ? 1u : 0u;
+            a.nt_xt = xstream ? 1u : 0u;
+            int od[2], nod = 0;                                    // the outer dims, innermost first
+            for (int k = rank - 2; k >= 0; --k)
+                if (k != tdim) od[nod++] = k;
+            const uint64_t n0 = nod >= 1 ? (uint64_t)dsc.shape[od[0]] : 1ull, n1 = nod >= 2 ? (uint64_t)dsc.shape[od[1]] : 1ull;
+            for (int q = 0; q < 3; ++q) {
+                a.ts[q] = (int32_t)dsc.stride[role[q]][tdim];
+                a.is[q] = (int32_t)dsc.stride[role[q]][rank - 1];
+                a.o0s[q] = nod >= 1 ? (int32_t)dsc.stride[role[q]][od[0]] : 0;
+                a.o1s[q] = nod >= 2 ? (int32_t)dsc.stride[role[q]][od[1]] : 0;
+            }
+            const bool wide = xstream && sizeof(T) == 4;
+            const uint32_t kSRows = wide ? 32u : 16u, kSBlock = kSRows / 2 * RT_WAVE;
+            const uint32_t ktiles = (a.K + kSRows - 1) / kSRows;
+            a.ltiles = (a.L + kSVecs * (uint32_t)N - 1) / (kSVecs * (uint32_t)N);
+            a.ltiles_div = make_fastdiv(a.ltiles);
+            const uint64_t gx = (uint64_t)ktiles * a.ltiles;
+            if (gx < (1ull << 31) && n0 <= 65535 && n1 <= 65535) {
+                const T* xp = (xt == 0 ? l : r) + dsc.offset[xt];
+                const T* op = (xt == 0 ? r : l) + dsc.offset[o];
+                T* dp = d + dsc.offset[2];
+                dim3 grid((unsigned)gx, (unsigned)n0, (unsigned)n1), blk(kSBlock);
+                auto go = [&](auto wide_c) {
+                    constexpr bool W = decltype(wide_c)::value;
+                    if constexpr (OP == kOpCopy) {
+                        hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_BCAST, W>), grid, blk, 0, ctx->stream, xp, op, dp, a);
+                    } else {
+                        if (om == M_VEC) hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_VEC, W>), grid, blk, 0, ctx->stream, xp, op, dp, a);
+                        else if (om == M_BCAST) hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_BCAST, W>), grid, blk, 0, ctx->stream, xp, op, dp, a);
+                        else hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_ELEM, W>), grid, blk, 0, ctx->stream, xp, op, dp, a);
+                    }
+                };
+                if constexpr (sizeof(T) == 4) { if (wide) go(std::true_type{}); else go(std::false_type{}); }
+                else go(std::false_type{});
+                hipError_t e = hipGetLastError();
+                *status = e == hipSuccess ? RT_OK : rt_hip_fail(e, "broadcast (staged tile kernel) launch");
+                return true;
+            }
+        }
+    }
+    if (hoistable(xt)) return false;
     TileArgs a;
     memset(&a, 0, sizeof(a));
     a.L = (uint32_t)dsc.shape[rank - 1];
@@ -378,18 +558,9 @@ __global__ __launch_bounds__(kTBlock) void planar_copy_kernel(const T* __restric
     uint32_t b = blockIdx.x;
     uint32_t q = fd_div(b, a.ntiles_div);
     const uint32_t tl = b - q * a.ntiles;
-    uint32_t rem = q;
-    int64_t offs = 0, offd = 0;
-#pragma unroll
-    for (int k = RT_MAX_RANK - 1; k >= 0; --k) {
-        if (k < a.nouter) {
-            uint32_t qq = fd_div(rem, a.odiv[k]);
-            uint32_t c = rem - qq * a.oshape[k];
-            offs += (int64_t)c * a.ostride[0][k];
-            offd += (int64_t)c * a.ostride[1][k];
-            rem = qq;
-        }
-    }
+    int64_t off2[2];
+    rt_outer_offsets<2>(q, a.nouter, a.oshape, a.odiv, a.ostride, off2);
+    const int64_t offs = off2[0], offd = off2[1];
     const uint32_t n0 = tl * a.B;
     const uint32_t nb = min(a.B, a.M - n0);
     const uint32_t ne = nb * a.C;

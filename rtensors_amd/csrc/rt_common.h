@@ -5,6 +5,7 @@
 #include <stdint.h>
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <map>
@@ -193,6 +194,55 @@ __device__ __forceinline__ uint32_t rt_negmask_4x8(uint32_t a) {
 }
 struct rt_words4 { uint32_t w[4]; };
 
+// ---- tiled traversal of a contiguous run ------------------------------------------------------------------------------------------
+// The streaming kernels give lane i of the grid the i-th 16-byte vector of a run.  Walking the run in that order, a block of 256
+// lanes owns one whole 4 KiB page.  Measured on MI355X, the same kernels are 4-6 % faster when a block instead owns the same
+// 1 KiB quarter of four neighbouring pages (and the next block the next quarter of those pages): 1 GiB f32, in-place op 0.82 ->
+// 0.87 of the 8 TB/s peak, copy 0.81 -> 0.87, c = a + b 0.82 -> 0.86, and a fill with 512-lane blocks owning 1 KiB pieces of
+// pages 64 KiB apart 0.84 -> 0.89.  Blocks are dealt to the eight XCDs in turn, so in this order every XCD keeps to its own slice
+// of each page instead of all eight sweeping the same address bits together.  The map is a permutation of the vector indices inside
+// windows of `rows` pieces at a pitch of `stride` bytes; the vectors before the first 4 KiB boundary and after the last whole window
+// keep their plain order.
+struct TileMap {
+    uint64_t lead;                  // vectors before the first window (plain order)
+    uint64_t bulk;                  // vectors inside whole windows
+    uint32_t pad;                   // idle lanes at the front of the grid, so that windows start on block boundaries
+    uint32_t lp, lr, lc;            // log2 of: vectors per piece, pieces (rows) per block column, pieces per row of the window
+};
+static inline TileMap rt_make_tilemap(const void* body, size_t nvec, uint32_t nthreads, uint32_t piece_bytes = 1024, uint32_t rows = 4,
+                                      uint32_t stride_bytes = 4096) {
+    TileMap m;
+    const uintptr_t addr = reinterpret_cast<uintptr_t>(body);
+    size_t lead = ((4096 - (addr & 4095)) & 4095) / 16;
+    if (lead > nvec) lead = nvec;
+    const size_t window = (size_t)rows * stride_bytes / 16;
+    m.lead = lead;
+    m.bulk = (nvec - lead) / window * window;
+    m.pad = (uint32_t)((nthreads - lead % nthreads) % nthreads);
+    m.lp = (uint32_t)__builtin_ctz(piece_bytes / 16);
+    m.lr = (uint32_t)__builtin_ctz(rows);
+    m.lc = (uint32_t)__builtin_ctz(stride_bytes / piece_bytes);
+    return m;
+}
+static inline size_t rt_tilemap_blocks(const TileMap& m, size_t nvec, uint32_t nthreads) { return (nvec + m.pad + nthreads - 1) / nthreads; }
+// The vector that lane `tid` of block `block` owns; false when the lane has none.
+__device__ __forceinline__ bool rt_tile_index(const TileMap& m, uint32_t block, uint32_t nthreads, uint32_t tid, size_t nvec, size_t* out) {
+    const int64_t i = (int64_t)block * nthreads + tid - (int64_t)m.pad;
+    if (i < 0 || (size_t)i >= nvec) return false;
+    size_t j = (size_t)i - m.lead;                      // wraps to a huge value for i < lead
+    if (j < m.bulk) {
+        const size_t within = j & (((size_t)1 << m.lp) - 1);
+        size_t t = j >> m.lp;
+        const size_t r = t & (((size_t)1 << m.lr) - 1);
+        t >>= m.lr;
+        const size_t c = t & (((size_t)1 << m.lc) - 1);
+        const size_t w = t >> m.lc;
+        j = ((((w << m.lr) + r) << (m.lc + m.lp)) + (c << m.lp)) + within;
+    }
+    *out = m.lead + j;
+    return true;
+}
+
 // Division of a 32-bit numerator by a runtime-constant divisor via multiply-high (round-up method); exact for
 // every n < 2^31 and 1 <= d < 2^31.
 struct FastDiv32 {
@@ -201,7 +251,7 @@ struct FastDiv32 {
 static inline FastDiv32 make_fastdiv(uint32_t d) {
     FastDiv32 f;
     f.d = d;
-    if (d == 1) { f.mul = 0; f.shift = 0; return f; }
+    if (d == 1) { f.mul = 1; f.shift = 0; return f; }             // (umulhi(n, 1) + n) >> 0 == n: no special case on the device
     uint32_t l = 32 - __builtin_clz(d - 1);                       // ceil(log2 d)
     uint64_t m = (((uint64_t)1 << 32) * (((uint64_t)1 << l) - d)) / d + 1;
     f.mul = (uint32_t)m;
@@ -209,7 +259,45 @@ static inline FastDiv32 make_fastdiv(uint32_t d) {
     return f;
 }
 __device__ __forceinline__ uint32_t fd_div(uint32_t n, const FastDiv32& f) {
-    if (f.d == 1) return n;
     uint32_t t = __umulhi(n, f.mul);
     return (uint32_t)(((uint64_t)t + n) >> f.shift);
+}
+
+// Keeps a wave-uniform value that came from the kernel arguments in a scalar register from this point on.  Kernel arguments are
+// fetched with scalar loads where they are first used; a kernel that uses them one after another behind branches waits for scalar
+// memory once per use.  Pinning everything a short-lived wave needs at the top of the kernel makes all those loads one batch with
+// one wait.  (A wave of the one-vector-per-lane kernels has about a microsecond to live if the chip is to stay at full bandwidth.)
+#define RT_PIN(x) asm volatile("" : "+s"(x))
+// The same for pointers: as an input only, so that the compiler still knows they point to global memory (a pointer that comes out
+// of an asm statement is accessed with the slower flat instructions).
+#define RT_TOUCH(x) asm volatile("" : : "s"(x))
+
+// blockIdx remainder -> element offsets of NOPS operands over the outer dims of a launch (outermost first, the entries from
+// `nouter` on hold shape 1).  Branch-free over a fixed number of dims: written as a loop that tests `k < nouter`, every dim costs
+// a chain of dependent scalar loads of the kernel arguments (load the shape, wait, branch, load the divisor, wait, ...), some thirty
+// waits before a wave issues its first global load.  Launches with at most two outer dims, nearly all of them, take the short form.
+template <int NOPS>
+__device__ __forceinline__ void rt_outer_offsets(uint32_t rem, int nouter, const uint32_t (&oshape)[RT_MAX_RANK], const FastDiv32 (&odiv)[RT_MAX_RANK],
+                                                 const int64_t (&ostride)[NOPS][RT_MAX_RANK], int64_t (&off)[NOPS]) {
+#pragma unroll
+    for (int o = 0; o < NOPS; ++o) off[o] = 0;
+    if (nouter <= 2) {
+#pragma unroll
+        for (int k = 1; k >= 0; --k) {
+            const uint32_t q = fd_div(rem, odiv[k]);
+            const uint32_t c = rem - q * oshape[k];
+#pragma unroll
+            for (int o = 0; o < NOPS; ++o) off[o] += (int64_t)c * ostride[o][k];
+            rem = q;
+        }
+    } else {
+#pragma unroll
+        for (int k = RT_MAX_RANK - 1; k >= 0; --k) {
+            const uint32_t q = fd_div(rem, odiv[k]);
+            const uint32_t c = rem - q * oshape[k];
+#pragma unroll
+            for (int o = 0; o < NOPS; ++o) off[o] += (int64_t)c * ostride[o][k];
+            rem = q;
+        }
+    }
 }

@@ -227,8 +227,7 @@ constexpr int kEU = 4;          // element-per-lane kernels: elements in flight 
 // on MI355X this shape (with non-temporal accesses for read-modify-write, plain stores for write-only) was the
 // fastest of the block-size / unroll / grid-stride variants tried, ~6.7 TB/s in place and ~6.8 TB/s for fill.
 template <class T, class F>
-__global__ __launch_bounds__(256) void ew_contig_kernel(Vec16<T>* __restrict__ p, size_t nvec, uint32_t head, uint32_t tail, F f) {
-    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+__global__ __launch_bounds__(512) void ew_contig_kernel(Vec16<T>* __restrict__ p, size_t nvec, uint32_t head, uint32_t tail, TileMap m, F f) {
     // The `head` elements before and the `tail` elements after the 16-byte aligned body (fewer than a vector each) are taken by
     // lanes of the first and the last block: launches of their own cost a run that starts off a 16-byte boundary 9 % (1 GiB f32
     // `+= 1`: 0.363 ms with three launches against 0.331 ms aligned).
@@ -244,12 +243,12 @@ __global__ __launch_bounds__(256) void ew_contig_kernel(Vec16<T>* __restrict__ p
         if constexpr (F::kReads) x = *e;
         *e = f(x);
     }
-    if (i >= nvec) return;
+    size_t i;
+    if (!rt_tile_index(m, blockIdx.x, blockDim.x, threadIdx.x, nvec, &i)) return;
     Vec16<T> v;
     if constexpr (F::kReads) v = rt_ld16_nt(p + i);
     apply_vec(v, f);
-    if constexpr (F::kReads) rt_st16_nt(p + i, v);
-    else p[i] = v;
+    rt_st16_nt(p + i, v);
 }
 
 // Edges of a contiguous run that do not fill a 16-byte vector, and 1-D strided views: one element per lane.
@@ -323,7 +322,7 @@ struct RowsArgs {
     int nouter;
     uint32_t oshape[RT_MAX_RANK];
     FastDiv32 odiv[RT_MAX_RANK];
-    int64_t ostride[RT_MAX_RANK];
+    int64_t ostride[1][RT_MAX_RANK];
     int64_t gstride;
 };
 
@@ -339,16 +338,9 @@ __global__ __launch_bounds__(kCBlock) void ew_rows_kernel(T* __restrict__ p, Row
     b = q;
     q = fd_div(b, a.nchunks_div);
     const uint32_t chunk = b - q * a.nchunks;
-    uint32_t rem = q;
-    int64_t off = 0;
-#pragma unroll
-    for (int k = RT_MAX_RANK - 1; k >= 0; --k) {
-        if (k < a.nouter) {
-            uint32_t qq = fd_div(rem, a.odiv[k]);
-            off += (int64_t)(rem - qq * a.oshape[k]) * a.ostride[k];
-            rem = qq;
-        }
-    }
+    int64_t off1[1];
+    rt_outer_offsets<1>(q, a.nouter, a.oshape, a.odiv, a.ostride, off1);
+    const int64_t off = off1[0];
     const uint32_t tx = threadIdx.x & (a.tpr - 1), ty = threadIdx.x / a.tpr, gy = kCBlock / a.tpr;
     const uint32_t c = (tile * a.tpr + tx) * N;
     if (c >= a.L) return;
@@ -427,12 +419,15 @@ int32_t launch_contig(rt_ctx* ctx, T* p, size_t n, F f) {
     if (head > n) head = n;
     size_t nvec = (n - head) / N;
     size_t tail = n - head - nvec * N;
-    const size_t bs = F::kReads ? (size_t)kCBlock : (size_t)256;          // pure stores: 256 lanes measured best
-    size_t blocks = (nvec + bs - 1) / bs;
+    // read-modify-write: 256 lanes, a block owns a 1 KiB quarter of four neighbouring pages; pure stores: 512 lanes, 1 KiB pieces of
+    // pages 64 KiB apart (see TileMap)
+    const uint32_t bs = F::kReads ? 256u : 512u;
+    const TileMap m = F::kReads ? rt_make_tilemap(p + head, nvec, bs) : rt_make_tilemap(p + head, nvec, bs, 1024, 16, 65536);
+    size_t blocks = rt_tilemap_blocks(m, nvec, bs);
     if (blocks < 1) blocks = 1;                                           // a run shorter than a vector: edges only
     if (blocks > 0x7fffffffull) return rt_fail(RT_E_INVALID, "contiguous run of %zu elements is too long for one launch", n);
-    hipLaunchKernelGGL((ew_contig_kernel<T, F>), dim3((unsigned)blocks), dim3((unsigned)bs), 0, ctx->stream,
-                       reinterpret_cast<Vec16<T>*>(p + head), nvec, (uint32_t)head, (uint32_t)tail, f);
+    hipLaunchKernelGGL((ew_contig_kernel<T, F>), dim3((unsigned)blocks), dim3(bs), 0, ctx->stream,
+                       reinterpret_cast<Vec16<T>*>(p + head), nvec, (uint32_t)head, (uint32_t)tail, m, f);
     RT_HIP(hipGetLastError());
     return RT_OK;
 }
@@ -440,14 +435,14 @@ int32_t launch_contig(rt_ctx* ctx, T* p, size_t n, F f) {
 // Out of place: dst[i] = f(src[i]) for a contiguous run; what `tensor.op()` needs instead of clone + in-place op, at half the
 // traffic (2 * N * sizeof(T) instead of 4 * N * sizeof(T)).
 template <class T, class F>
-__global__ __launch_bounds__(kCBlock) void ew_contig_out_kernel(const T* __restrict__ s, T* __restrict__ d, size_t nvec, uint32_t head, uint32_t tail, F f) {
+__global__ __launch_bounds__(256) void ew_contig_out_kernel(const T* __restrict__ s, T* __restrict__ d, size_t nvec, uint32_t head, uint32_t tail, TileMap m, F f) {
     constexpr size_t N = 16 / sizeof(T);
-    const size_t i = (size_t)blockIdx.x * kCBlock + threadIdx.x;
     // s and d point at the vector body, which starts on a 128-byte line of d; the `head` elements before it and the `tail`
     // elements after it go to lanes of the first and the last block
     if (blockIdx.x == 0 && threadIdx.x < head) { const int64_t e = (int64_t)threadIdx.x - (int64_t)head; d[e] = f(s[e]); }
     if (blockIdx.x == gridDim.x - 1 && threadIdx.x < tail) { const size_t e = nvec * N + threadIdx.x; d[e] = f(s[e]); }
-    if (i >= nvec) return;
+    size_t i;
+    if (!rt_tile_index(m, blockIdx.x, 256, threadIdx.x, nvec, &i)) return;
     Vec16<T> v = __builtin_bit_cast(Vec16<T>, rt_ld16u<T, true>(s + i * N));          // the source may be in any phase
     apply_vec(v, f);
     rt_st16_nt(reinterpret_cast<Vec16<T>*>(d) + i, v);
@@ -461,11 +456,12 @@ int32_t launch_contig_out(rt_ctx* ctx, const T* s, T* d, size_t n, F f) {
     size_t head = ((kBodyAlign - (addr & (kBodyAlign - 1))) & (kBodyAlign - 1)) / sizeof(T);
     if (head > n) head = n;
     const size_t nvec = (n - head) / N, tail = n - head - nvec * N;
-    size_t blocks = (nvec + kCBlock - 1) / kCBlock;
+    const TileMap m = rt_make_tilemap(d + head, nvec, 256);
+    size_t blocks = rt_tilemap_blocks(m, nvec, 256);
     if (blocks < 1) blocks = 1;
     if (blocks > 0x7fffffffull) return rt_fail(RT_E_INVALID, "contiguous run of %zu elements is too long for one launch", n);
-    hipLaunchKernelGGL((ew_contig_out_kernel<T, F>), dim3((unsigned)blocks), dim3(kCBlock), 0, ctx->stream, s + head, d + head, nvec, (uint32_t)head,
-                       (uint32_t)tail, f);
+    hipLaunchKernelGGL((ew_contig_out_kernel<T, F>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, s + head, d + head, nvec, (uint32_t)head,
+                       (uint32_t)tail, m, f);
     RT_HIP(hipGetLastError());
     return RT_OK;
 }
@@ -514,7 +510,7 @@ int32_t launch_view(rt_ctx* ctx, T* base, const NdDesc& d, uint64_t count, F f) 
         for (int k = 0; k < gdim; ++k) {
             r.oshape[r.nouter] = (uint32_t)d.shape[k];
             r.odiv[r.nouter] = make_fastdiv((uint32_t)d.shape[k]);
-            r.ostride[r.nouter] = d.stride[0][k];
+            r.ostride[0][r.nouter] = d.stride[0][k];
             if ((d.stride[0][k] * (int64_t)sizeof(T)) % 128 != 0) whole_lines = false;
             outer *= (uint64_t)d.shape[k];
             r.nouter++;

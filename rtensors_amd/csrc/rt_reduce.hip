@@ -159,6 +159,9 @@ __device__ __forceinline__ void fold_run(Acc<OP, T>& a, const T* __restrict__ p,
         Vec16<T> v[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) v[u] = rt_ld16_nt(pv + i + (uint64_t)u * nthreads);
+        // nothing may move across this point: left alone, the scheduler puts the first add (and with it a wait for the first
+        // load) in front of the other three loads, and every trip then costs two memory latencies instead of one
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int u = 0; u < U; ++u) {
 #pragma unroll
@@ -274,6 +277,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(const T* __restrict
             VecW v[U];
 #pragma unroll
             for (int u = 0; u < U; ++u) v[u] = load(p + (k + (uint64_t)u * kWaves) * inner);
+            __builtin_amdgcn_sched_barrier(0);                    // all loads of a trip before the first add (see fold_run)
 #pragma unroll
             for (int u = 0; u < U; ++u) {
 #pragma unroll
