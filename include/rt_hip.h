@@ -37,7 +37,7 @@ typedef enum rt_status {
     RT_E_HIP = 4,          /* HIP runtime failure; see rt_last_error() */
     RT_E_OOM = 5,          /* device allocation failed */
     RT_E_RANK = 6,         /* more than RT_MAX_RANK dims remain after collapsing */
-    RT_E_ARITH = 7,        /* integer division by a zero scalar / mean over an empty integer axis (reference panics) */
+    RT_E_ARITH = 7,        /* integer division by zero or MIN / -1, mean over an empty integer axis (the reference panics) */
     RT_E_WRONG_DIMS = 8,   /* TensorError::WrongDims: reduction source is not contiguous (backend/mod.rs:386-390) */
     RT_E_SIZE_MISMATCH = 9 /* TensorError::SizeMismatch (backend/cpu.rs:151-161) */
 } rt_status;
@@ -153,7 +153,11 @@ int32_t rt_scalar_nd(rt_ctx* ctx, int32_t dtype, int32_t op, void* buf, uint64_t
 /* ---- N-d broadcast (Backend::broadcast, backend/mod.rs:296-309; Cpu backend/cpu.rs:292-352) --------------------
  * dst[c] = left[c] (op) right[c] for every coordinate c of `shape`.  The three operands share `shape`
  * (expansion is expressed as stride 0, ops/broadcast/mod.rs:13-55); strides may be negative.  dst may be the
- * same buffer as left with the same layout (in-place `a op= b`). */
+ * same buffer as left with the same layout (in-place `a op= b`).
+ * Integer division: a zero divisor or MIN / -1 inside the tensors (a panic in the reference, ops/base.rs:27-37) cannot be seen
+ * before the kernel has run; the kernel stores 0 / MIN for such elements and sets a fault word of the context, and the next
+ * call that waits for the stream (rt_sync, rt_read, rt_dump, rt_equal) returns RT_E_ARITH once and clears it.  The same holds for
+ * rt_scalar_* division of a signed tensor by -1.  A zero scalar divisor is refused at once. */
 int32_t rt_broadcast(rt_ctx* ctx, int32_t dtype, int32_t op, int32_t rank, const uint64_t* shape,
                      const void* left, uint64_t left_len, uint64_t left_offset, const int64_t* left_strides,
                      const void* right, uint64_t right_len, uint64_t right_offset, const int64_t* right_strides,

@@ -25,14 +25,14 @@ namespace {
 constexpr int kCBlock2 = 256;
 template <class T, int OP>
 __global__ __launch_bounds__(kCBlock2) void bin_contig_kernel(const Vec16<T>* l, const Vec16<T>* r, Vec16<T>* d, size_t nvec, uint32_t head,
-                                                              uint32_t tail, TileMap m) {
+                                                              uint32_t tail, TileMap m, int32_t* fault) {
     // the `head` elements before and the `tail` elements after the aligned body (fewer than a vector each; all three operands
     // share the phase) are taken by lanes of the first and the last block instead of launches of their own
     auto edge = [&](int64_t e) {
         const T x = *(reinterpret_cast<const T*>(l) + e);
         T y = x;
         if constexpr (OP != kOpCopy) y = *(reinterpret_cast<const T*>(r) + e);
-        *(reinterpret_cast<T*>(d) + e) = bin_apply<OP, T>(x, y);
+        *(reinterpret_cast<T*>(d) + e) = bin_apply<OP, T>(x, y, fault);
     };
     if (blockIdx.x == 0 && threadIdx.x < head) edge((int64_t)threadIdx.x - (int64_t)head);
     if (blockIdx.x == gridDim.x - 1 && threadIdx.x < tail) edge((int64_t)(nvec * (16 / sizeof(T))) + (int64_t)threadIdx.x);
@@ -41,7 +41,7 @@ __global__ __launch_bounds__(kCBlock2) void bin_contig_kernel(const Vec16<T>* l,
     Vec16<T> a = rt_ld16_nt(l + i);
     Vec16<T> b;
     if constexpr (OP != kOpCopy) b = rt_ld16_nt(r + i); else b = a;
-    bin_apply_vec<OP, T>(a, b);
+    bin_apply_vec<OP, T>(a, b, fault);
     rt_st16_nt(d + i, a);
 }
 
@@ -64,7 +64,7 @@ struct RowArgs {
 };
 
 template <class T, int OP, int LM, int RM, int GU>
-__global__ __launch_bounds__(256) void bin_rows_kernel(const T* l, const T* r, T* d, RowArgs a) {
+__global__ __launch_bounds__(256) void bin_rows_kernel(const T* l, const T* r, T* d, RowArgs a, int32_t* fault) {
     constexpr int N = 16 / sizeof(T);
     // blockIdx -> (outer index, chunk of the loop dim, column tile); all uniform, computed on the scalar unit
     uint32_t b = blockIdx.x;
@@ -93,7 +93,7 @@ __global__ __launch_bounds__(256) void bin_rows_kernel(const T* l, const T* r, T
         auto ldr = [&](int64_t off) { return load_raw<T, RM>(r + off, c, a.istride[1]); };
         auto combine_store = [&](Raw x, Raw y, uint32_t g) {
             Vec16<T> xv = __builtin_bit_cast(Vec16<T>, x);
-            bin_apply_vec<OP, T>(xv, __builtin_bit_cast(Vec16<T>, y));
+            bin_apply_vec<OP, T>(xv, __builtin_bit_cast(Vec16<T>, y), fault);
             rt_st16u_nt<T>(d + od + (int64_t)g * a.gstride[2] + c, __builtin_bit_cast(rt_u32x4, xv));
         };
         Raw lh = {}, rh = {};                                   // operands that do not move along the loop dim
@@ -145,7 +145,7 @@ __global__ __launch_bounds__(256) void bin_rows_kernel(const T* l, const T* r, T
             const T* rp = r + orr + (int64_t)g * a.gstride[1];
             T* dp = d + od + (int64_t)g * a.gstride[2];
             for (uint32_t k = max(c, a.lead); k < min(c + (uint32_t)N, a.L); ++k)
-                dp[k] = bin_apply<OP, T>(lp[(int64_t)k * a.istride[0]], rp[(int64_t)k * a.istride[1]]);
+                dp[k] = bin_apply<OP, T>(lp[(int64_t)k * a.istride[0]], rp[(int64_t)k * a.istride[1]], fault);
         }
     }
 }
@@ -166,7 +166,7 @@ struct Rows4Args {
 // grid: x = column tile + tiles * (chunk of four rows), y = index along the inner outer dim, z = index along the outer one.  Every
 // offset inside an operand fits 32 bits (checked on the host).
 template <class T, int OP, int LM, int RM>
-__global__ __launch_bounds__(256) void bin_rows4_kernel(const T* l, const T* r, T* d, Rows4Args a) {
+__global__ __launch_bounds__(256) void bin_rows4_kernel(const T* l, const T* r, T* d, Rows4Args a, int32_t* fault) {
     constexpr int N = 16 / sizeof(T);
     uint32_t L = a.L, G = a.G, tiles = a.tiles, tm = a.tiles_div.mul, ts = a.tiles_div.shift;
     int32_t g0 = a.gs[0], g1 = a.gs[1], g2 = a.gs[2], p0 = a.o0s[0], p1 = a.o0s[1], p2 = a.o0s[2], q0 = a.o1s[0], q1 = a.o1s[1], q2 = a.o1s[2];
@@ -188,19 +188,19 @@ __global__ __launch_bounds__(256) void bin_rows4_kernel(const T* l, const T* r, 
         rt_u32x4 y = x;
         if constexpr (OP != kOpCopy) y = load_raw<T, RM>(rp, c, 1);
         Vec16<T> xv = __builtin_bit_cast(Vec16<T>, x);
-        bin_apply_vec<OP, T>(xv, __builtin_bit_cast(Vec16<T>, y));
+        bin_apply_vec<OP, T>(xv, __builtin_bit_cast(Vec16<T>, y), fault);
         rt_st16u_nt<T>(dp + c, __builtin_bit_cast(rt_u32x4, xv));
     } else {
-        for (uint32_t k = c; k < L; ++k) dp[k] = bin_apply<OP, T>(lp[LM == M_VEC ? k : 0], rp[RM == M_VEC ? k : 0]);
+        for (uint32_t k = c; k < L; ++k) dp[k] = bin_apply<OP, T>(lp[LM == M_VEC ? k : 0], rp[RM == M_VEC ? k : 0], fault);
     }
 }
 
 template <class T, int OP>
-void launch_rows4(int lm, int rm, dim3 grid, hipStream_t s, const T* l, const T* r, T* d, const Rows4Args& a) {
-    if (lm == M_VEC && rm == M_VEC) hipLaunchKernelGGL((bin_rows4_kernel<T, OP, M_VEC, M_VEC>), grid, dim3(256), 0, s, l, r, d, a);
-    else if (lm == M_VEC) hipLaunchKernelGGL((bin_rows4_kernel<T, OP, M_VEC, M_BCAST>), grid, dim3(256), 0, s, l, r, d, a);
-    else if (rm == M_VEC) hipLaunchKernelGGL((bin_rows4_kernel<T, OP, M_BCAST, M_VEC>), grid, dim3(256), 0, s, l, r, d, a);
-    else hipLaunchKernelGGL((bin_rows4_kernel<T, OP, M_BCAST, M_BCAST>), grid, dim3(256), 0, s, l, r, d, a);
+void launch_rows4(int lm, int rm, dim3 grid, hipStream_t s, const T* l, const T* r, T* d, const Rows4Args& a, int32_t* fault) {
+    if (lm == M_VEC && rm == M_VEC) hipLaunchKernelGGL((bin_rows4_kernel<T, OP, M_VEC, M_VEC>), grid, dim3(256), 0, s, l, r, d, a, fault);
+    else if (lm == M_VEC) hipLaunchKernelGGL((bin_rows4_kernel<T, OP, M_VEC, M_BCAST>), grid, dim3(256), 0, s, l, r, d, a, fault);
+    else if (rm == M_VEC) hipLaunchKernelGGL((bin_rows4_kernel<T, OP, M_BCAST, M_VEC>), grid, dim3(256), 0, s, l, r, d, a, fault);
+    else hipLaunchKernelGGL((bin_rows4_kernel<T, OP, M_BCAST, M_BCAST>), grid, dim3(256), 0, s, l, r, d, a, fault);
 }
 
 // ---- generic ------------------------------------------------------------------------------------------------------------
@@ -214,7 +214,7 @@ struct GenArgs {
 constexpr int kGU = 4;          // elements in flight per lane in the generic kernel
 
 template <class T, int OP>
-__global__ __launch_bounds__(kBlock) void bin_generic_kernel(const T* l, const T* r, T* d, GenArgs a, uint32_t first, uint32_t n) {
+__global__ __launch_bounds__(kBlock) void bin_generic_kernel(const T* l, const T* r, T* d, GenArgs a, uint32_t first, uint32_t n, int32_t* fault) {
     // a block owns kGU * kBlock consecutive elements per trip, lane t the elements t, t + kBlock, ...; all loads are issued
     // before the first store
     constexpr uint32_t span = kGU * kBlock, step = kBlock;
@@ -243,7 +243,7 @@ __global__ __launch_bounds__(kBlock) void bin_generic_kernel(const T* l, const T
         }
 #pragma unroll
         for (int u = 0; u < kGU; ++u)
-            if (i + u * step < n) d[od[u]] = bin_apply<OP, T>(x[u], y[u]);
+            if (i + u * step < n) d[od[u]] = bin_apply<OP, T>(x[u], y[u], fault);
     }
 }
 
@@ -286,7 +286,7 @@ __device__ __forceinline__ Vec16<T> load_row_vec(const T* __restrict__ row, uint
 }
 
 template <class T, int OP, int LMODE, int RMODE>
-__global__ __launch_bounds__(kRBlock) void bin_flat_kernel(const T* l, const T* r, T* d, GenArgs a, uint32_t nvec) {
+__global__ __launch_bounds__(kRBlock) void bin_flat_kernel(const T* l, const T* r, T* d, GenArgs a, uint32_t nvec, int32_t* fault) {
     constexpr int N = 16 / sizeof(T);
     constexpr bool LE = LMODE == F_ELEM, RE = RMODE == F_ELEM && OP != kOpCopy;
     const uint32_t v = blockIdx.x * kRBlock + threadIdx.x;
@@ -319,7 +319,7 @@ __global__ __launch_bounds__(kRBlock) void bin_flat_kernel(const T* l, const T* 
         }
     }
     if constexpr (OP == kOpCopy) y = x;
-    bin_apply_vec<OP, T>(x, y);
+    bin_apply_vec<OP, T>(x, y, fault);
     rt_st16_nt(reinterpret_cast<Vec16<T>*>(d) + v, x);
 }
 
@@ -328,7 +328,7 @@ __global__ __launch_bounds__(kRBlock) void bin_flat_kernel(const T* l, const T* 
 // v mod (L / N) -- the shape of the plain copy kernel plus one cached load.
 template <class T, int OP, bool ROW_IS_LEFT>
 __global__ __launch_bounds__(kCBlock2) void bin_flat_row_kernel(const T* flat, const T* __restrict__ row, T* d, uint32_t nvec, uint32_t row_vecs,
-                                                                FastDiv32 row_div, TileMap m) {
+                                                                FastDiv32 row_div, TileMap m, int32_t* fault) {
     // `flat` and `d` may be the same buffer (in-place form): every lane reads its vector before it writes it
     size_t vi;
     if (!rt_tile_index(m, blockIdx.x, kCBlock2, threadIdx.x, nvec, &vi)) return;
@@ -343,12 +343,12 @@ __global__ __launch_bounds__(kCBlock2) void bin_flat_row_kernel(const T* flat, c
         const uint32_t c = v - fd_div(v, row_div) * row_vecs;
         y = rt_ld16(reinterpret_cast<const Vec16<T>*>(row) + c);
     }
-    if constexpr (ROW_IS_LEFT) { bin_apply_vec<OP, T>(y, x); rt_st16_nt(reinterpret_cast<Vec16<T>*>(d) + v, y); }
-    else { bin_apply_vec<OP, T>(x, y); rt_st16_nt(reinterpret_cast<Vec16<T>*>(d) + v, x); }
+    if constexpr (ROW_IS_LEFT) { bin_apply_vec<OP, T>(y, x, fault); rt_st16_nt(reinterpret_cast<Vec16<T>*>(d) + v, y); }
+    else { bin_apply_vec<OP, T>(x, y, fault); rt_st16_nt(reinterpret_cast<Vec16<T>*>(d) + v, x); }
 }
 
 template <class T, int OP>
-__global__ __launch_bounds__(kBlock) void bin_generic64_kernel(const T* l, const T* r, T* d, NdDesc a, uint64_t n) {
+__global__ __launch_bounds__(kBlock) void bin_generic64_kernel(const T* l, const T* r, T* d, NdDesc a, uint64_t n, int32_t* fault) {
     uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
     const uint64_t step = (uint64_t)gridDim.x * kBlock;
     for (; i < n; i += step) {
@@ -362,33 +362,65 @@ __global__ __launch_bounds__(kBlock) void bin_generic64_kernel(const T* l, const
             od += c * a.stride[2][k];
             rem = q;
         }
-        d[od] = bin_apply<OP, T>(l[ol], r[orr]);
+        d[od] = bin_apply<OP, T>(l[ol], r[orr], fault);
     }
+}
+
+// Layouts that keep more than RT_MAX_RANK dims after collapsing (the reference accepts rank <= 128): the descriptor is read from
+// device memory, one element per lane, 64-bit index arithmetic.  Correct for every layout; nothing here is tuned.
+template <class T, int OP>
+__global__ __launch_bounds__(kBlock) void bin_big_kernel(const T* l, const T* r, T* d, const int64_t* __restrict__ w, int rank, uint64_t n, int32_t* fault) {
+    uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    const uint64_t step = (uint64_t)gridDim.x * kBlock;
+    for (; i < n; i += step) {
+        uint64_t rem = i;
+        int64_t ol = 0, orr = 0, od = 0;
+        for (int k = rank - 1; k >= 0; --k) {
+            const uint64_t sh = (uint64_t)w[k];
+            const uint64_t q = rem / sh;
+            const int64_t c = (int64_t)(rem - q * sh);
+            ol += c * w[rank + k];
+            orr += c * w[2 * rank + k];
+            od += c * w[3 * rank + k];
+            rem = q;
+        }
+        d[od] = bin_apply<OP, T>(l[ol], r[orr], fault);
+    }
+}
+
+template <class T, int OP>
+int32_t broadcast_big(rt_ctx* ctx, const BigDesc& b, uint64_t count, const void* lv, const void* rv, void* dv) {
+    const size_t blocks = (size_t)((count + kBlock - 1) / kBlock);
+    const size_t cap = (size_t)ctx->num_cus * 64;
+    hipLaunchKernelGGL((bin_big_kernel<T, OP>), dim3((unsigned)(blocks < cap ? blocks : cap)), dim3(kBlock), 0, ctx->stream,
+                       (const T*)lv + b.offset[0], (const T*)rv + b.offset[1], (T*)dv + b.offset[2], b.words, b.rank, count, fault_of<T, OP>(ctx));
+    RT_HIP(hipGetLastError());
+    return RT_OK;
 }
 
 // ---- host: kernel choice ----------------------------------------------------------------------------------------------
 template <class T, int OP, int LM, int RM>
-void launch_rows_g(bool batched, dim3 grid, unsigned bs, hipStream_t s, const T* l, const T* r, T* d, const RowArgs& a) {
+void launch_rows_g(bool batched, dim3 grid, unsigned bs, hipStream_t s, const T* l, const T* r, T* d, const RowArgs& a, int32_t* fault) {
     // the batched long-loop form is only ever chosen when one input is gathered element-wise
     if constexpr (LM == M_ELEM || RM == M_ELEM) {
-        if (batched) { hipLaunchKernelGGL((bin_rows_kernel<T, OP, LM, RM, 4>), grid, dim3(bs), 0, s, l, r, d, a); return; }
+        if (batched) { hipLaunchKernelGGL((bin_rows_kernel<T, OP, LM, RM, 4>), grid, dim3(bs), 0, s, l, r, d, a, fault); return; }
     }
-    hipLaunchKernelGGL((bin_rows_kernel<T, OP, LM, RM, 1>), grid, dim3(bs), 0, s, l, r, d, a);
+    hipLaunchKernelGGL((bin_rows_kernel<T, OP, LM, RM, 1>), grid, dim3(bs), 0, s, l, r, d, a, fault);
 }
 template <class T, int OP, int LM>
-void launch_rows_r(int rm, bool batched, dim3 grid, unsigned bs, hipStream_t s, const T* l, const T* r, T* d, const RowArgs& a) {
+void launch_rows_r(int rm, bool batched, dim3 grid, unsigned bs, hipStream_t s, const T* l, const T* r, T* d, const RowArgs& a, int32_t* fault) {
     switch (rm) {
-        case M_VEC: launch_rows_g<T, OP, LM, M_VEC>(batched, grid, bs, s, l, r, d, a); break;
-        case M_BCAST: launch_rows_g<T, OP, LM, M_BCAST>(batched, grid, bs, s, l, r, d, a); break;
-        default: launch_rows_g<T, OP, LM, M_ELEM>(batched, grid, bs, s, l, r, d, a); break;
+        case M_VEC: launch_rows_g<T, OP, LM, M_VEC>(batched, grid, bs, s, l, r, d, a, fault); break;
+        case M_BCAST: launch_rows_g<T, OP, LM, M_BCAST>(batched, grid, bs, s, l, r, d, a, fault); break;
+        default: launch_rows_g<T, OP, LM, M_ELEM>(batched, grid, bs, s, l, r, d, a, fault); break;
     }
 }
 template <class T, int OP>
-void launch_rows(int lm, int rm, bool batched, dim3 grid, unsigned bs, hipStream_t s, const T* l, const T* r, T* d, const RowArgs& a) {
+void launch_rows(int lm, int rm, bool batched, dim3 grid, unsigned bs, hipStream_t s, const T* l, const T* r, T* d, const RowArgs& a, int32_t* fault) {
     switch (lm) {
-        case M_VEC: launch_rows_r<T, OP, M_VEC>(rm, batched, grid, bs, s, l, r, d, a); break;
-        case M_BCAST: launch_rows_r<T, OP, M_BCAST>(rm, batched, grid, bs, s, l, r, d, a); break;
-        default: launch_rows_r<T, OP, M_ELEM>(rm, batched, grid, bs, s, l, r, d, a); break;
+        case M_VEC: launch_rows_r<T, OP, M_VEC>(rm, batched, grid, bs, s, l, r, d, a, fault); break;
+        case M_BCAST: launch_rows_r<T, OP, M_BCAST>(rm, batched, grid, bs, s, l, r, d, a, fault); break;
+        default: launch_rows_r<T, OP, M_ELEM>(rm, batched, grid, bs, s, l, r, d, a, fault); break;
     }
 }
 
@@ -422,7 +454,7 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
             if (blocks > 0x7fffffffull) return rt_fail(RT_E_INVALID, "broadcast: %zu elements is too long for one launch", n);
             hipLaunchKernelGGL((bin_contig_kernel<T, OP>), dim3((unsigned)blocks), dim3(kCBlock2), 0, s,
                                reinterpret_cast<const Vec16<T>*>(lp + head), reinterpret_cast<const Vec16<T>*>(rp + head),
-                               reinterpret_cast<Vec16<T>*>(dp + head), nvec, (uint32_t)head, (uint32_t)tail, m);
+                               reinterpret_cast<Vec16<T>*>(dp + head), nvec, (uint32_t)head, (uint32_t)tail, m, fault_of<T, OP>(ctx));
             RT_HIP(hipGetLastError());
             return RT_OK;
         }
@@ -475,8 +507,8 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
                 const uint32_t nvec = (uint32_t)(count / N), row_vecs = is_scalar ? 0u : (uint32_t)(dsc.shape[rank - 1] / N);
                 const TileMap m = rt_make_tilemap(d + dsc.offset[2], nvec, kCBlock2);
                 dim3 grid((unsigned)rt_tilemap_blocks(m, nvec, kCBlock2)), blk(kCBlock2);
-                if (p == 0) hipLaunchKernelGGL((bin_flat_row_kernel<T, OP, true>), grid, blk, 0, s, fo, ro, d + dsc.offset[2], nvec, row_vecs, make_fastdiv(row_vecs ? row_vecs : 1u), m);
-                else hipLaunchKernelGGL((bin_flat_row_kernel<T, OP, false>), grid, blk, 0, s, fo, ro, d + dsc.offset[2], nvec, row_vecs, make_fastdiv(row_vecs ? row_vecs : 1u), m);
+                if (p == 0) hipLaunchKernelGGL((bin_flat_row_kernel<T, OP, true>), grid, blk, 0, s, fo, ro, d + dsc.offset[2], nvec, row_vecs, make_fastdiv(row_vecs ? row_vecs : 1u), m, fault_of<T, OP>(ctx));
+                else hipLaunchKernelGGL((bin_flat_row_kernel<T, OP, false>), grid, blk, 0, s, fo, ro, d + dsc.offset[2], nvec, row_vecs, make_fastdiv(row_vecs ? row_vecs : 1u), m, fault_of<T, OP>(ctx));
                 RT_HIP(hipGetLastError());
                 return RT_OK;
             }
@@ -586,7 +618,7 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
                     q.o0s[o] = rank >= 3 ? (int32_t)dsc.stride[o][rank - 3] : 0;
                     q.o1s[o] = rank >= 4 ? (int32_t)dsc.stride[o][rank - 4] : 0;
                 }
-                launch_rows4<T, OP>(lm, rm, dim3((unsigned)gx, (unsigned)n0, (unsigned)n1), s, l + dsc.offset[0], r + dsc.offset[1], d + dsc.offset[2], q);
+                launch_rows4<T, OP>(lm, rm, dim3((unsigned)gx, (unsigned)n0, (unsigned)n1), s, l + dsc.offset[0], r + dsc.offset[1], d + dsc.offset[2], q, fault_of<T, OP>(ctx));
                 RT_HIP(hipGetLastError());
                 return RT_OK;
             }
@@ -605,7 +637,7 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
         if (blocks < (1ull << 31)) {
             // the operand pointers address column 0 of the moved origin (never dereferenced below column `lead`)
             launch_rows<T, OP>(lm, rm, steps > 2, dim3((unsigned)blocks), kRBlock, s, l + dsc.offset[0] - (int64_t)lead * a.istride[0],
-                               r + dsc.offset[1] - (int64_t)lead * a.istride[1], d + dsc.offset[2] - (int64_t)lead, a);
+                               r + dsc.offset[1] - (int64_t)lead * a.istride[1], d + dsc.offset[2] - (int64_t)lead, a, fault_of<T, OP>(ctx));
             RT_HIP(hipGetLastError());
             return RT_OK;
         }
@@ -638,35 +670,69 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
             };
             const bool lrow = !lv && rv && row_like(0), rrow = lv && !rv && OP != kOpCopy && row_like(1);
             dim3 grid((nvec + kRBlock - 1) / kRBlock), blk(kRBlock);
-            if (lrow) hipLaunchKernelGGL((bin_flat_kernel<T, OP, F_ROW, F_VEC>), grid, blk, 0, s, lp, rp, dp, g, nvec);
-            else if (rrow) hipLaunchKernelGGL((bin_flat_kernel<T, OP, F_VEC, F_ROW>), grid, blk, 0, s, lp, rp, dp, g, nvec);
-            else if (lv && rv) hipLaunchKernelGGL((bin_flat_kernel<T, OP, F_VEC, F_VEC>), grid, blk, 0, s, lp, rp, dp, g, nvec);
-            else if (lv) hipLaunchKernelGGL((bin_flat_kernel<T, OP, F_VEC, F_ELEM>), grid, blk, 0, s, lp, rp, dp, g, nvec);
-            else if (rv) hipLaunchKernelGGL((bin_flat_kernel<T, OP, F_ELEM, F_VEC>), grid, blk, 0, s, lp, rp, dp, g, nvec);
-            else hipLaunchKernelGGL((bin_flat_kernel<T, OP, F_ELEM, F_ELEM>), grid, blk, 0, s, lp, rp, dp, g, nvec);
+            if (lrow) hipLaunchKernelGGL((bin_flat_kernel<T, OP, F_ROW, F_VEC>), grid, blk, 0, s, lp, rp, dp, g, nvec, fault_of<T, OP>(ctx));
+            else if (rrow) hipLaunchKernelGGL((bin_flat_kernel<T, OP, F_VEC, F_ROW>), grid, blk, 0, s, lp, rp, dp, g, nvec, fault_of<T, OP>(ctx));
+            else if (lv && rv) hipLaunchKernelGGL((bin_flat_kernel<T, OP, F_VEC, F_VEC>), grid, blk, 0, s, lp, rp, dp, g, nvec, fault_of<T, OP>(ctx));
+            else if (lv) hipLaunchKernelGGL((bin_flat_kernel<T, OP, F_VEC, F_ELEM>), grid, blk, 0, s, lp, rp, dp, g, nvec, fault_of<T, OP>(ctx));
+            else if (rv) hipLaunchKernelGGL((bin_flat_kernel<T, OP, F_ELEM, F_VEC>), grid, blk, 0, s, lp, rp, dp, g, nvec, fault_of<T, OP>(ctx));
+            else hipLaunchKernelGGL((bin_flat_kernel<T, OP, F_ELEM, F_ELEM>), grid, blk, 0, s, lp, rp, dp, g, nvec, fault_of<T, OP>(ctx));
             first = nvec * (uint32_t)N;                          // the last count % N elements go to the element kernel
         }
         if (first < count) {
             size_t blocks = ((size_t)(count - first) + kGU * kBlock - 1) / (kGU * kBlock);
-            hipLaunchKernelGGL((bin_generic_kernel<T, OP>), dim3((unsigned)blocks), dim3(kBlock), 0, s, lp, rp, dp, g, first, (uint32_t)count);
+            hipLaunchKernelGGL((bin_generic_kernel<T, OP>), dim3((unsigned)blocks), dim3(kBlock), 0, s, lp, rp, dp, g, first, (uint32_t)count, fault_of<T, OP>(ctx));
         }
     } else {
         size_t cap = (size_t)ctx->num_cus * 64;
         hipLaunchKernelGGL((bin_generic64_kernel<T, OP>), dim3((unsigned)cap), dim3(kBlock), 0, s,
-                           l + dsc.offset[0], r + dsc.offset[1], d + dsc.offset[2], dsc, count);
+                           l + dsc.offset[0], r + dsc.offset[1], d + dsc.offset[2], dsc, count, fault_of<T, OP>(ctx));
     }
     RT_HIP(hipGetLastError());
     return RT_OK;
 }
 
-template <class T>
-int32_t broadcast_ops(rt_ctx* ctx, int op, const NdDesc& d, uint64_t count, const void* l, const void* r, void* dst) {
-    switch (op) {
-        case RT_ADD: return broadcast_typed<T, RT_ADD>(ctx, d, count, l, r, dst);
-        case RT_SUB: return broadcast_typed<T, RT_SUB>(ctx, d, count, l, r, dst);
-        case RT_MUL: return broadcast_typed<T, RT_MUL>(ctx, d, count, l, r, dst);
+template <class T> struct type_tag { typedef T type; };
+
+// Calls fn(type_tag<T>, integral_constant<OP>) for the element carrier and op of a broadcast; + - * on two's-complement integers
+// do not depend on signedness, so they run on the unsigned type of the same width (one instantiation per width).
+template <class Fn>
+int32_t with_type_op(int dtype, int op, Fn&& fn) {
+    if (op == RT_DIV) {
+        typedef std::integral_constant<int, RT_DIV> D;
+        switch (dtype) {
+            case RT_U8: return fn(type_tag<uint8_t>{}, D{});
+            case RT_I8: return fn(type_tag<int8_t>{}, D{});
+            case RT_U16: return fn(type_tag<uint16_t>{}, D{});
+            case RT_I16: return fn(type_tag<int16_t>{}, D{});
+            case RT_U32: return fn(type_tag<uint32_t>{}, D{});
+            case RT_I32: return fn(type_tag<int32_t>{}, D{});
+            case RT_U64: return fn(type_tag<uint64_t>{}, D{});
+            case RT_I64: return fn(type_tag<int64_t>{}, D{});
+            case RT_F32: return fn(type_tag<float>{}, D{});
+            case RT_F64: return fn(type_tag<double>{}, D{});
+            case RT_BOOL: return rt_fail(RT_E_ARITH, "broadcast: division is not implemented for boolean in the reference (todo!())");
+        }
+        return rt_fail(RT_E_DTYPE, "broadcast: 128-bit integer division is not built for the device");
     }
-    return rt_fail(RT_E_INVALID, "broadcast: unknown op code %d", op);
+    auto ops = [&](auto t) -> int32_t {
+        switch (op) {
+            case RT_ADD: return fn(t, std::integral_constant<int, RT_ADD>{});
+            case RT_SUB: return fn(t, std::integral_constant<int, RT_SUB>{});
+            case RT_MUL: return fn(t, std::integral_constant<int, RT_MUL>{});
+        }
+        return rt_fail(RT_E_INVALID, "broadcast: unknown op code %d", op);
+    };
+    switch (dtype) {
+        case RT_U8: case RT_I8: return ops(type_tag<uint8_t>{});
+        case RT_U16: case RT_I16: return ops(type_tag<uint16_t>{});
+        case RT_U32: case RT_I32: return ops(type_tag<uint32_t>{});
+        case RT_U64: case RT_I64: return ops(type_tag<uint64_t>{});
+        case RT_F32: return ops(type_tag<float>{});
+        case RT_F64: return ops(type_tag<double>{});
+        case RT_BOOL: return ops(type_tag<boolean_t>{});
+        case RT_U128: case RT_I128: return ops(type_tag<u128_t>{});
+    }
+    return rt_fail(RT_E_DTYPE, "broadcast: unknown dtype code %d", dtype);
 }
 
 }  // namespace
@@ -694,10 +760,21 @@ extern "C" int32_t rt_gather(rt_ctx* ctx, int32_t dtype, const void* src, uint64
     NdDesc d;
     const int64_t* sp[3] = {sst, sst, dstr};
     const uint64_t offs[3] = {offset * words, offset * words, 0};
-    RT_TRY(rt_collapse(3, r2, shp, sp, offs, /*reorder=*/true, /*key=*/2, &d));
-    for (int k = 0; k < RT_MAX_RANK; ++k) d.stride[1][k] = 0;           // right operand: one element, never advanced
-    CtxGuard g(ctx);
     const uint64_t n = count * words;
+    const int32_t cst = rt_collapse(3, r2, shp, sp, offs, /*reorder=*/true, /*key=*/2, &d);
+    CtxGuard g(ctx);
+    if (cst == RT_E_RANK) {
+        BigDesc b;
+        RT_TRY(rt_collapse_big(ctx, 3, r2, shp, sp, offs, /*reorder=*/true, /*key=*/2, &b));
+        switch (es) {
+            case 1: return broadcast_big<uint8_t, kOpCopy>(ctx, b, n, src, src, dst);
+            case 2: return broadcast_big<uint16_t, kOpCopy>(ctx, b, n, src, src, dst);
+            case 4: return broadcast_big<uint32_t, kOpCopy>(ctx, b, n, src, src, dst);
+            default: return broadcast_big<uint64_t, kOpCopy>(ctx, b, n, src, src, dst);
+        }
+    }
+    RT_TRY(cst);
+    for (int k = 0; k < RT_MAX_RANK; ++k) d.stride[1][k] = 0;           // right operand: one element, never advanced
     switch (es) {
         case 1: return broadcast_typed<uint8_t, kOpCopy>(ctx, d, n, src, src, dst);
         case 2: return broadcast_typed<uint16_t, kOpCopy>(ctx, d, n, src, src, dst);
@@ -726,34 +803,17 @@ extern "C" int32_t rt_broadcast(rt_ctx* ctx, int32_t dtype, int32_t op, int32_t 
     NdDesc d;
     const int64_t* sp[3] = {left_strides, right_strides, dst_strides};
     const uint64_t offs[3] = {left_offset, right_offset, dst_offset};
-    RT_TRY(rt_collapse(3, rank, shape, sp, offs, /*reorder=*/true, /*key=*/2, &d));
+    const int32_t cst = rt_collapse(3, rank, shape, sp, offs, /*reorder=*/true, /*key=*/2, &d);
     CtxGuard g(ctx);
-    if (op == RT_DIV) {
-        switch (dtype) {
-            case RT_U8: return broadcast_typed<uint8_t, RT_DIV>(ctx, d, count, left, right, dst);
-            case RT_I8: return broadcast_typed<int8_t, RT_DIV>(ctx, d, count, left, right, dst);
-            case RT_U16: return broadcast_typed<uint16_t, RT_DIV>(ctx, d, count, left, right, dst);
-            case RT_I16: return broadcast_typed<int16_t, RT_DIV>(ctx, d, count, left, right, dst);
-            case RT_U32: return broadcast_typed<uint32_t, RT_DIV>(ctx, d, count, left, right, dst);
-            case RT_I32: return broadcast_typed<int32_t, RT_DIV>(ctx, d, count, left, right, dst);
-            case RT_U64: return broadcast_typed<uint64_t, RT_DIV>(ctx, d, count, left, right, dst);
-            case RT_I64: return broadcast_typed<int64_t, RT_DIV>(ctx, d, count, left, right, dst);
-            case RT_F32: return broadcast_typed<float, RT_DIV>(ctx, d, count, left, right, dst);
-            case RT_F64: return broadcast_typed<double, RT_DIV>(ctx, d, count, left, right, dst);
-            case RT_BOOL: return rt_fail(RT_E_ARITH, "broadcast: division is not implemented for boolean in the reference (todo!())");
-        }
-        return rt_fail(RT_E_DTYPE, "broadcast: 128-bit integer division is not built for the device");
+    if (cst == RT_E_RANK) {
+        BigDesc b;
+        RT_TRY(rt_collapse_big(ctx, 3, rank, shape, sp, offs, /*reorder=*/true, /*key=*/2, &b));
+        return with_type_op(dtype, op, [&](auto t, auto opc) -> int32_t {
+            return broadcast_big<typename decltype(t)::type, decltype(opc)::value>(ctx, b, count, left, right, dst);
+        });
     }
-    // + - * on two's-complement integers do not depend on signedness: one instantiation per width
-    switch (dtype) {
-        case RT_U8: case RT_I8: return broadcast_ops<uint8_t>(ctx, op, d, count, left, right, dst);
-        case RT_U16: case RT_I16: return broadcast_ops<uint16_t>(ctx, op, d, count, left, right, dst);
-        case RT_U32: case RT_I32: return broadcast_ops<uint32_t>(ctx, op, d, count, left, right, dst);
-        case RT_U64: case RT_I64: return broadcast_ops<uint64_t>(ctx, op, d, count, left, right, dst);
-        case RT_F32: return broadcast_ops<float>(ctx, op, d, count, left, right, dst);
-        case RT_F64: return broadcast_ops<double>(ctx, op, d, count, left, right, dst);
-        case RT_BOOL: return broadcast_ops<boolean_t>(ctx, op, d, count, left, right, dst);
-        case RT_U128: case RT_I128: return broadcast_ops<u128_t>(ctx, op, d, count, left, right, dst);
-    }
-    return rt_fail(RT_E_DTYPE, "broadcast: unknown dtype code %d", dtype);
+    RT_TRY(cst);
+    return with_type_op(dtype, op, [&](auto t, auto opc) -> int32_t {
+        return broadcast_typed<typename decltype(t)::type, decltype(opc)::value>(ctx, d, count, left, right, dst);
+    });
 }

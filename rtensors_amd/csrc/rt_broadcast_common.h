@@ -4,6 +4,7 @@
 
 #include "rt_common.h"
 
+#include <limits>
 #include <type_traits>
 
 namespace rtb {
@@ -20,7 +21,11 @@ template <class T> struct carrier<T, typename std::enable_if<std::is_integral<T>
 // ops/base.rs:27-37 on T; integers wrap (release build), integer division truncates toward zero
 constexpr int kOpCopy = 4;      // internal: dst = left (strided gather); right is ignored
 
-template <int OP, class T> __device__ __forceinline__ T bin_apply(T a, T b) {
+// `fault`: where integer division reports what the reference answers with a panic (ops/base.rs:27-37: `/` on a zero divisor, and
+// MIN / -1, which overflows): the lane stores 1 there -- a plain store, every lane that meets a fault writes the same value -- and
+// the host turns a set word into RT_E_ARITH at the next call that waits for the stream.  The element itself becomes 0 (MIN for
+// MIN / -1).
+template <int OP, class T> __device__ __forceinline__ T bin_apply(T a, T b, int32_t* fault = nullptr) {
     if constexpr (OP == kOpCopy) {
         return a;
     } else if constexpr (is_flt<T>::value) {
@@ -38,10 +43,15 @@ template <int OP, class T> __device__ __forceinline__ T bin_apply(T a, T b) {
         else if constexpr (OP == RT_SUB) return (T)(W)((W)a - (W)b);
         else if constexpr (OP == RT_MUL) return (T)(W)((W)a * (W)b);
         else {
-            // the reference panics on b == 0 and MIN / -1; the device yields 0 and MIN there and raises no error
-            if (b == 0) return (T)0;
+            if (b == 0) {
+                if (fault) *fault = 1;
+                return (T)0;
+            }
             if constexpr (std::is_signed<T>::value) {
-                if (b == (T)-1) return (T)(W)((W)0 - (W)a);
+                if (b == (T)-1) {
+                    if (a == std::numeric_limits<T>::min() && fault) *fault = 1;
+                    return (T)(W)((W)0 - (W)a);
+                }
             }
             return (T)(a / b);
         }
@@ -51,7 +61,7 @@ template <int OP, class T> __device__ __forceinline__ T bin_apply(T a, T b) {
 template <class T> struct alignas(16) Vec16 { T e[16 / sizeof(T)]; };
 
 // x = x OP y on a whole vector.  1-byte add / subtract (and every bool op) run on four elements per 32-bit word.
-template <int OP, class T> __device__ __forceinline__ void bin_apply_vec(Vec16<T>& x, const Vec16<T>& y) {
+template <int OP, class T> __device__ __forceinline__ void bin_apply_vec(Vec16<T>& x, const Vec16<T>& y, int32_t* fault = nullptr) {
     if constexpr (sizeof(T) == 1 && (OP == RT_ADD || OP == RT_SUB || (OP == RT_MUL && is_bool<T>::value))) {
         rt_words4 a = __builtin_bit_cast(rt_words4, x);
         const rt_words4 b = __builtin_bit_cast(rt_words4, y);
@@ -63,7 +73,18 @@ template <int OP, class T> __device__ __forceinline__ void bin_apply_vec(Vec16<T
         x = __builtin_bit_cast(Vec16<T>, a);
     } else {
 #pragma unroll
-        for (int j = 0; j < (int)(16 / sizeof(T)); ++j) x.e[j] = bin_apply<OP, T>(x.e[j], y.e[j]);
+        for (int j = 0; j < (int)(16 / sizeof(T)); ++j) x.e[j] = bin_apply<OP, T>(x.e[j], y.e[j], fault);
+    }
+}
+
+// The fault word of the context for a launch that can raise an integer-division fault (and a note for the host to look at it at
+// the next synchronising call); null for every other launch.
+template <class T, int OP> static inline int32_t* fault_of(rt_ctx* ctx) {
+    if constexpr (OP == RT_DIV && std::is_integral<T>::value) {
+        ctx->fault_pending = true;
+        return ctx->fault_dev;
+    } else {
+        return nullptr;
     }
 }
 

@@ -48,7 +48,7 @@ struct TileArgs {
 // xt / xo: the transposed and the other input.  OM = access mode of the other input along the inner dim; VG = the transposed
 // input can be read with aligned 16-byte loads along dim t (else element loads).
 template <class T, int OP, int OM, bool VG>
-__global__ __launch_bounds__(kTBlock) void bin_tile_kernel(const T* xt, const T* xo, T* d, TileArgs a) {
+__global__ __launch_bounds__(kTBlock) void bin_tile_kernel(const T* xt, const T* xo, T* d, TileArgs a, int32_t* fault) {
     constexpr int N = 16 / sizeof(T);
     constexpr int LPR = TileGeom<T>::LPR, RPI = TileGeom<T>::RPI, TK = TileGeom<T>::TK, TL = TileGeom<T>::TL;
     __shared__ alignas(16) T tile[TK][TL + N];
@@ -210,8 +210,8 @@ __global__ __launch_bounds__(kTBlock) void bin_tile_kernel(const T* xt, const T*
                 if (k0 + kk < a.K) {
                     const Vec16<T> xv = *reinterpret_cast<const Vec16<T>*>(&tile[kk][(lane % LPR) * N]);
                     Vec16<T> out;
-                    if (x_left) { out = xv; bin_apply_vec<OP, T>(out, ov[i]); }
-                    else { out = ov[i]; bin_apply_vec<OP, T>(out, xv); }
+                    if (x_left) { out = xv; bin_apply_vec<OP, T>(out, ov[i], fault); }
+                    else { out = ov[i]; bin_apply_vec<OP, T>(out, xv, fault); }
                     rt_st16u_nt<T>(drow + (int64_t)(k0 + kk) * a.tstride[2] + c, __builtin_bit_cast(rt_u32x4, out));
                 }
             }
@@ -225,7 +225,7 @@ __global__ __launch_bounds__(kTBlock) void bin_tile_kernel(const T* xt, const T*
                         T xe = tile[kk][cc - l0];
                         T oe = xe;
                         if constexpr (OP != kOpCopy) oe = (orow + (int64_t)(k0 + kk) * a.tstride[1])[(int64_t)cc * a.istride[1]];
-                        drow[(int64_t)(k0 + kk) * a.tstride[2] + cc] = x_left ? bin_apply<OP, T>(xe, oe) : bin_apply<OP, T>(oe, xe);
+                        drow[(int64_t)(k0 + kk) * a.tstride[2] + cc] = x_left ? bin_apply<OP, T>(xe, oe, fault) : bin_apply<OP, T>(oe, xe, fault);
                     }
                 }
             }
@@ -266,7 +266,7 @@ struct StageArgs {
 
 // grid: x = inner-dim tile + ltiles * (tile along t), y = index along the inner outer dim, z = index along the outer one
 template <class T, int OP, int OM, bool WIDE>
-__global__ __launch_bounds__((StageGeom<T, WIDE>::kBlock)) void bin_stage_kernel(const T* xt, const T* xo, T* d, StageArgs a) {
+__global__ __launch_bounds__((StageGeom<T, WIDE>::kBlock)) void bin_stage_kernel(const T* xt, const T* xo, T* d, StageArgs a, int32_t* fault) {
     constexpr int N = 16 / sizeof(T);
     constexpr int kSRows = StageGeom<T, WIDE>::kRows, kSWaves = StageGeom<T, WIDE>::kWaves, kSBlock = StageGeom<T, WIDE>::kBlock;
     constexpr int TK = kSRows, TL = kSVecs * N, KQ = TK / N, NU = kSVecs * KQ, RPL = TK / kSWaves;
@@ -342,8 +342,8 @@ __global__ __launch_bounds__((StageGeom<T, WIDE>::kBlock)) void bin_stage_kernel
         if (full_vec) {
             const Vec16<T> xv = *reinterpret_cast<const Vec16<T>*>(&tile[kk][lane * N]);
             Vec16<T> out;
-            if (x_left) { out = xv; bin_apply_vec<OP, T>(out, ov[i]); }
-            else { out = ov[i]; bin_apply_vec<OP, T>(out, xv); }
+            if (x_left) { out = xv; bin_apply_vec<OP, T>(out, ov[i], fault); }
+            else { out = ov[i]; bin_apply_vec<OP, T>(out, xv, fault); }
             rt_st16u_nt<T>(drow + c, __builtin_bit_cast(rt_u32x4, out));
         } else {
             // ragged end of a row: element accesses
@@ -351,7 +351,7 @@ __global__ __launch_bounds__((StageGeom<T, WIDE>::kBlock)) void bin_stage_kernel
                 T xe = tile[kk][cc - l0];
                 T oe = xe;
                 if constexpr (OP != kOpCopy) oe = (xo + (int32_t)(k0 + kk) * ts1)[(int32_t)cc * is1];
-                drow[cc] = x_left ? bin_apply<OP, T>(xe, oe) : bin_apply<OP, T>(oe, xe);
+                drow[cc] = x_left ? bin_apply<OP, T>(xe, oe, fault) : bin_apply<OP, T>(oe, xe, fault);
             }
         }
     }
@@ -441,11 +441,11 @@ bool tile_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* l, const 
                 auto go = [&](auto wide_c) {
                     constexpr bool W = decltype(wide_c)::value;
                     if constexpr (OP == kOpCopy) {
-                        hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_BCAST, W>), grid, blk, 0, ctx->stream, xp, op, dp, a);
+                        hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_BCAST, W>), grid, blk, 0, ctx->stream, xp, op, dp, a, fault_of<T, OP>(ctx));
                     } else {
-                        if (om == M_VEC) hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_VEC, W>), grid, blk, 0, ctx->stream, xp, op, dp, a);
-                        else if (om == M_BCAST) hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_BCAST, W>), grid, blk, 0, ctx->stream, xp, op, dp, a);
-                        else hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_ELEM, W>), grid, blk, 0, ctx->stream, xp, op, dp, a);
+                        if (om == M_VEC) hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_VEC, W>), grid, blk, 0, ctx->stream, xp, op, dp, a, fault_of<T, OP>(ctx));
+                        else if (om == M_BCAST) hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_BCAST, W>), grid, blk, 0, ctx->stream, xp, op, dp, a, fault_of<T, OP>(ctx));
+                        else hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_ELEM, W>), grid, blk, 0, ctx->stream, xp, op, dp, a, fault_of<T, OP>(ctx));
                     }
                 };
                 if constexpr (sizeof(T) == 4) { if (wide) go(std::true_type{}); else go(std::false_type{}); }
@@ -516,8 +516,8 @@ bool tile_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* l, const 
     T* dp = d + dsc.offset[2];
     hipStream_t s = ctx->stream;
     dim3 grid((unsigned)blocks), blk(kTBlock);
-#define RT_TILE(OM) do { if (vec_gather) hipLaunchKernelGGL((bin_tile_kernel<T, OP, OM, true>), grid, blk, 0, s, xp, op, dp, a); \
-                         else hipLaunchKernelGGL((bin_tile_kernel<T, OP, OM, false>), grid, blk, 0, s, xp, op, dp, a); } while (0)
+#define RT_TILE(OM) do { if (vec_gather) hipLaunchKernelGGL((bin_tile_kernel<T, OP, OM, true>), grid, blk, 0, s, xp, op, dp, a, fault_of<T, OP>(ctx)); \
+                         else hipLaunchKernelGGL((bin_tile_kernel<T, OP, OM, false>), grid, blk, 0, s, xp, op, dp, a, fault_of<T, OP>(ctx)); } while (0)
     if constexpr (OP == kOpCopy) {
         RT_TILE(M_BCAST);                        // the copy op has no second input
     } else {

@@ -57,6 +57,10 @@ struct rt_ctx {
     int (*blas_destroy)(void*) = nullptr;
     // device flag written by the equality kernel and read back by rt_equal
     int32_t* flag_dev = nullptr;
+    // device word set by integer-division kernels that met a zero divisor or MIN / -1 (the reference panics there); looked at by
+    // the next call that waits for the stream, and only when such a kernel was launched since the last look
+    int32_t* fault_dev = nullptr;
+    bool fault_pending = false;
     int num_cus = 256;
 };
 
@@ -70,6 +74,9 @@ int32_t rt_ctx_enter(rt_ctx* ctx);                                   // validate
 int32_t rt_alloc_bytes(rt_ctx* ctx, size_t bytes, void** out);       // caller holds ctx->mu
 int32_t rt_free_locked(rt_ctx* ctx, void* p);
 int32_t rt_scratch(rt_ctx* ctx, size_t bytes, void** out);           // caller holds ctx->mu
+// After the stream has been waited for: RT_E_ARITH if an integer division launched since the last look met a fault, and the fault
+// word is cleared.  Caller holds ctx->mu.
+int32_t rt_take_fault(rt_ctx* ctx);
 
 // Validation shared by the reduce and argmax entry points.  *run == false after RT_OK: there are no outputs, launch nothing.
 int32_t rt_check_reduce_flat(uint64_t src_len, const void* src, const void* dst, uint64_t dst_len, uint64_t start, uint64_t len);
@@ -110,6 +117,16 @@ struct NdDesc {
 // and sorted by that operand's stride, largest first, which maximises merging and makes its accesses ascend.
 int32_t rt_collapse(int nops, int rank, const uint64_t* shape, const int64_t* const* strides, const uint64_t* offsets,
                     bool reorder, int key, NdDesc* out);
+
+// A collapsed layout of any rank with its descriptor in device memory: words[0 .. rank) = shape, words[(o + 1) * rank + i] = stride
+// of operand o along dim i (dim 0 outermost).  Used when more than RT_MAX_RANK dims remain after collapsing.
+struct BigDesc {
+    int rank;
+    const int64_t* words;           // device pointer (the context's scratch buffer; valid until the next call that uses scratch)
+    int64_t offset[3];
+};
+int32_t rt_collapse_big(rt_ctx* ctx, int nops, int rank, const uint64_t* shape, const int64_t* const* strides, const uint64_t* offsets,
+                        bool reorder, int key, BigDesc* out);
 
 // ---- device helpers ------------------------------------------------------------------------------------------------
 #define RT_WAVE 64

@@ -176,6 +176,7 @@ template <int OP, class T> struct ScalarF {
     static constexpr bool kReads = true;
     static constexpr bool kPacked = sizeof(T) == 1 && (OP == RT_S_ADD || OP == RT_S_SUB || (OP == RT_S_MUL && is_bool<T>::value));
     T v;
+    int32_t* fault;                     // division of a signed integer by -1 only: set to 1 when an element is MIN (the reference panics)
     __device__ __forceinline__ uint32_t packed(uint32_t w) const {
         uint8_t b;
         __builtin_memcpy(&b, &v, 1);
@@ -187,7 +188,12 @@ template <int OP, class T> struct ScalarF {
         if constexpr (OP == RT_S_ADD) return w_add<T>(x, v);                                      // cpu.rs:678-696
         else if constexpr (OP == RT_S_SUB) return w_sub<T>(x, v);
         else if constexpr (OP == RT_S_MUL) return w_mul<T>(x, v);
-        else if constexpr (OP == RT_S_DIV) return w_div<T>(x, v);
+        else if constexpr (OP == RT_S_DIV) {
+            if constexpr (is_sint<T>::value && sizeof(T) <= 8) {
+                if (fault && x == std::numeric_limits<T>::min()) *fault = 1;                       // MIN / -1 overflows
+            }
+            return w_div<T>(x, v);
+        }
         else if constexpr (OP == RT_S_LEAKY_RELU) return gt0(x) ? x : w_mul<T>(x, v);             // cpu.rs:708-715
         else if constexpr (OP == RT_S_LOG) return m_log(x) / m_log(v);                            // f32::log(base)
         else if constexpr (OP == RT_S_LOG1P) return m_log1p(x) / m_log(v);                        // core/value.rs vlog1p
@@ -403,6 +409,28 @@ __global__ __launch_bounds__(kBlock) void ew_nd64_kernel(T* __restrict__ p, NdDe
     }
 }
 
+// Views that keep more than RT_MAX_RANK dims after collapsing (the reference accepts rank <= 128, core/primitives.rs:377-383):
+// shape and strides are read from device memory (words[0 .. rank) = shape, words[rank .. 2 rank) = strides).
+template <class T, class F>
+__global__ __launch_bounds__(kBlock) void ew_big_kernel(T* __restrict__ p, const int64_t* __restrict__ w, int rank, uint64_t n, F f) {
+    uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    const uint64_t step = (uint64_t)gridDim.x * kBlock;
+    for (; i < n; i += step) {
+        uint64_t rem = i;
+        int64_t off = 0;
+        for (int k = rank - 1; k >= 0; --k) {
+            const uint64_t sh = (uint64_t)w[k];
+            const uint64_t q = rem / sh;
+            off += (int64_t)(rem - q * sh) * w[rank + k];
+            rem = q;
+        }
+        T* q = p + off;
+        T x = zero_of<T>();
+        if constexpr (F::kReads) x = *q;
+        *q = f(x);
+    }
+}
+
 // ---- launch logic ---------------------------------------------------------------------------------------------------
 constexpr uintptr_t kBodyAlign = 128;        // at most 127 one-byte elements before the body: fewer than the lanes of a block
 static inline unsigned capped_grid(size_t blocks, size_t cap) { return (unsigned)(blocks < 1 ? 1 : (blocks > cap ? cap : blocks)); }
@@ -573,8 +601,21 @@ int32_t run_view(rt_ctx* ctx, const char* what, const ViewArg& va, F f) {
     NdDesc d;
     const int64_t* sp[1] = {va.strides};
     // out of place the element order matters (dst is row-major): no reordering of dims
-    RT_TRY(rt_collapse(1, va.rank, va.shape, sp, &offset, /*reorder=*/va.dst == nullptr, 0, &d));
+    const int32_t cst = rt_collapse(1, va.rank, va.shape, sp, &offset, /*reorder=*/va.dst == nullptr, 0, &d);
     CtxGuard g(ctx);
+    if (cst == RT_E_RANK && !va.dst) {
+        // more than RT_MAX_RANK dims remain: descriptor in device memory, rank-generic kernel
+        BigDesc b;
+        RT_TRY(rt_collapse_big(ctx, 1, va.rank, va.shape, sp, &offset, /*reorder=*/true, 0, &b));
+        const size_t blocks = (size_t)((count + kBlock - 1) / kBlock);
+        hipLaunchKernelGGL((ew_big_kernel<T, F>), dim3(capped_grid(blocks, (size_t)ctx->num_cus * 64)), dim3(kBlock), 0, ctx->stream,
+                           (T*)va.buf + b.offset[0], b.words, b.rank, count, f);
+        RT_HIP(hipGetLastError());
+        return RT_OK;
+    }
+    if (cst == RT_E_RANK)
+        return rt_fail(RT_E_WRONG_DIMS, "%s: the out-of-place form takes a forward contiguous run (gather other views first)", what);
+    RT_TRY(cst);
     if (!va.dst) return launch_view<T, F>(ctx, (T*)va.buf, d, count, f);
     if (va.dst == va.buf) return rt_fail(RT_E_INVALID, "%s: the out-of-place form needs a destination other than the source", what);
     if (!(d.rank == 0 || (d.rank == 1 && d.stride[0][0] == 1)))
@@ -660,7 +701,15 @@ int32_t unary_any(rt_ctx* ctx, int32_t dtype, int32_t op, const ViewArg& va) {
 
 template <class T, int OP>
 int32_t scalar_go(rt_ctx* ctx, const ViewArg& va, const void* value) {
-    return run_view<T, ScalarF<OP, T>>(ctx, "scalar", va, ScalarF<OP, T>{load_scalar<T>(value)});
+    int32_t* fault = nullptr;
+    if constexpr (OP == RT_S_DIV && is_sint<T>::value && sizeof(T) <= 8) {
+        if (load_scalar<T>(value) == (T)-1) {                 // x / -1 overflows for x == MIN: the kernel reports it
+            fault = ctx->fault_dev;
+            CtxGuard g(ctx);
+            ctx->fault_pending = true;
+        }
+    }
+    return run_view<T, ScalarF<OP, T>>(ctx, "scalar", va, ScalarF<OP, T>{load_scalar<T>(value), fault});
 }
 
 template <class T>

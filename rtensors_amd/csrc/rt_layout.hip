@@ -39,12 +39,15 @@ int32_t rt_check_extent(const char* what, uint64_t offset, int rank, const uint6
     return RT_OK;
 }
 
-int32_t rt_collapse(int nops, int rank, const uint64_t* shape, const int64_t* const* strides, const uint64_t* offsets,
-                    bool reorder, int key, NdDesc* out) {
-    struct Dim { int64_t n; int64_t s[3]; };
+namespace {
+struct Dim { int64_t n; int64_t s[3]; };
+
+// size-1 dims dropped, dims optionally flipped / sorted by operand `key`, adjacent dims merged where every operand allows it
+void collapse_dims(int nops, int rank, const uint64_t* shape, const int64_t* const* strides, const uint64_t* offsets, bool reorder, int key,
+                   std::vector<Dim>* merged_out, int64_t (&off)[3]) {
     std::vector<Dim> dims;
     dims.reserve((size_t)rank);
-    int64_t off[3] = {0, 0, 0};
+    off[0] = off[1] = off[2] = 0;
     for (int o = 0; o < nops; ++o) off[o] = (int64_t)offsets[o];
     for (int i = 0; i < rank; ++i) {
         if (shape[i] == 1) continue;                        // size-1 dims never move an address
@@ -62,7 +65,8 @@ int32_t rt_collapse(int nops, int rank, const uint64_t* shape, const int64_t* co
         std::stable_sort(dims.begin(), dims.end(), [key](const Dim& a, const Dim& b) { return a.s[key] > b.s[key]; });
     }
     // merge dim i+1 into dim i when, for every operand, stepping dim i once equals stepping dim i+1 shape[i+1] times
-    std::vector<Dim> merged;
+    std::vector<Dim>& merged = *merged_out;
+    merged.clear();
     for (const Dim& d : dims) {
         if (!merged.empty()) {
             Dim& p = merged.back();
@@ -76,13 +80,46 @@ int32_t rt_collapse(int nops, int rank, const uint64_t* shape, const int64_t* co
         }
         merged.push_back(d);
     }
+}
+}  // namespace
+
+int32_t rt_collapse(int nops, int rank, const uint64_t* shape, const int64_t* const* strides, const uint64_t* offsets,
+                    bool reorder, int key, NdDesc* out) {
+    std::vector<Dim> merged;
+    int64_t off[3];
+    collapse_dims(nops, rank, shape, strides, offsets, reorder, key, &merged, off);
     if ((int)merged.size() > RT_MAX_RANK)
-        return rt_fail(RT_E_RANK, "layout needs %d dims after collapsing; at most %d are supported", (int)merged.size(), RT_MAX_RANK);
+        return rt_fail(RT_E_RANK, "layout needs %d dims after collapsing; the kernel-argument descriptor holds %d", (int)merged.size(), RT_MAX_RANK);
     out->rank = (int)merged.size();
     for (int i = 0; i < RT_MAX_RANK; ++i) {
         out->shape[i] = i < out->rank ? merged[(size_t)i].n : 1;
         for (int o = 0; o < 3; ++o) out->stride[o][i] = i < out->rank ? merged[(size_t)i].s[o] : 0;
     }
+    for (int o = 0; o < 3; ++o) out->offset[o] = off[o];
+    return RT_OK;
+}
+
+// The same for layouts that keep more than RT_MAX_RANK dims (the reference accepts rank <= 128, core/primitives.rs:377-383): the
+// descriptor goes to device memory (the context's scratch buffer) as int64 words [shape[rank], stride0[rank], stride1[rank],
+// stride2[rank]] and a rank-generic kernel reads it from there.  Caller holds ctx->mu.
+int32_t rt_collapse_big(rt_ctx* ctx, int nops, int rank, const uint64_t* shape, const int64_t* const* strides, const uint64_t* offsets,
+                        bool reorder, int key, BigDesc* out) {
+    std::vector<Dim> merged;
+    int64_t off[3];
+    collapse_dims(nops, rank, shape, strides, offsets, reorder, key, &merged, off);
+    const int r = (int)merged.size();
+    std::vector<int64_t> words((size_t)r * 4);
+    for (int i = 0; i < r; ++i) {
+        words[(size_t)i] = merged[(size_t)i].n;
+        for (int o = 0; o < 3; ++o) words[(size_t)(o + 1) * r + i] = merged[(size_t)i].s[o];
+    }
+    void* dev = nullptr;
+    RT_TRY(rt_scratch(ctx, words.size() * sizeof(int64_t) + 8, &dev));
+    // a pageable source is staged by the runtime before the call returns; the copy is ordered on the stream like the kernels
+    RT_HIP(hipMemcpyAsync(dev, words.data(), words.size() * sizeof(int64_t), hipMemcpyHostToDevice, ctx->stream));
+    RT_HIP(hipStreamSynchronize(ctx->stream));
+    out->rank = r;
+    out->words = (const int64_t*)dev;
     for (int o = 0; o < 3; ++o) out->offset[o] = off[o];
     return RT_OK;
 }

@@ -257,7 +257,7 @@ extern "C" int32_t rt_equal(rt_ctx* ctx, int32_t dtype, const void* a, uint64_t 
     RT_HIP(hipMemcpyAsync(&host, ctx->flag_dev, sizeof(host), hipMemcpyDeviceToHost, ctx->stream));
     RT_HIP(hipStreamSynchronize(ctx->stream));
     *out_equal = host;
-    return RT_OK;
+    return rt_take_fault(ctx);
 }
 
 extern "C" int32_t rt_convert(rt_ctx* ctx, int32_t src_dtype, const void* src, uint64_t src_len, int32_t dst_dtype, void* dst, uint64_t dst_len) {

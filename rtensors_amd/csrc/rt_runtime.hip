@@ -74,6 +74,9 @@ extern "C" int32_t rt_ctx_create(int32_t device, rt_ctx** out) {
     if (hipGetDeviceProperties(&prop, device) == hipSuccess && prop.multiProcessorCount > 0) c->num_cus = prop.multiProcessorCount;
     e = hipMalloc((void**)&c->flag_dev, 256);
     if (e != hipSuccess) { (void)hipStreamDestroy(c->stream); delete c; return rt_hip_fail(e, "hipMalloc(flag)"); }
+    e = hipMemset(c->flag_dev, 0, 256);
+    if (e != hipSuccess) { (void)hipFree(c->flag_dev); (void)hipStreamDestroy(c->stream); delete c; return rt_hip_fail(e, "hipMemset(flag)"); }
+    c->fault_dev = c->flag_dev + 16;                         // its own 64-byte piece of the block
     *out = c;
     return RT_OK;
 }
@@ -98,10 +101,26 @@ extern "C" int32_t rt_ctx_destroy(rt_ctx* ctx) {
     return RT_OK;
 }
 
+__global__ void rt_clear_word_kernel(int32_t* p) { *p = 0; }
+
+int32_t rt_take_fault(rt_ctx* ctx) {
+    if (!ctx->fault_pending) return RT_OK;
+    ctx->fault_pending = false;
+    int32_t host = 0;
+    RT_HIP(hipMemcpyAsync(&host, ctx->fault_dev, sizeof(host), hipMemcpyDeviceToHost, ctx->stream));
+    RT_HIP(hipStreamSynchronize(ctx->stream));
+    if (!host) return RT_OK;
+    hipLaunchKernelGGL(rt_clear_word_kernel, dim3(1), dim3(1), 0, ctx->stream, ctx->fault_dev);
+    RT_HIP(hipGetLastError());
+    return rt_fail(RT_E_ARITH, "an integer division enqueued earlier met a zero divisor or MIN / -1 (the reference panics there); "
+                               "the elements concerned hold 0 / MIN");
+}
+
 extern "C" int32_t rt_sync(rt_ctx* ctx) {
     RT_TRY(rt_ctx_enter(ctx));
     RT_HIP(hipStreamSynchronize(ctx->stream));
-    return RT_OK;
+    CtxGuard g(ctx);
+    return rt_take_fault(ctx);
 }
 
 // ---- caching allocator ---------------------------------------------------------------------------------------------
@@ -438,7 +457,7 @@ extern "C" int32_t rt_read(rt_ctx* ctx, int32_t dtype, const void* buf, uint64_t
     CtxGuard g(ctx);
     RT_HIP(hipMemcpyAsync(out_value, (const char*)buf + offset * es, es, hipMemcpyDeviceToHost, ctx->stream));
     RT_HIP(hipStreamSynchronize(ctx->stream));
-    return RT_OK;
+    return rt_take_fault(ctx);
 }
 
 struct Cell16 { uint32_t w[4]; };
@@ -487,7 +506,8 @@ extern "C" int32_t rt_dump(rt_ctx* ctx, int32_t dtype, const void* src, uint64_t
     if (!bytes) return RT_OK;
     if (!src || !host_dst) return rt_fail(RT_E_INVALID, "rt_dump: null pointer");
     CtxGuard g(ctx);
-    return download(ctx, host_dst, src, bytes);
+    RT_TRY(download(ctx, host_dst, src, bytes));
+    return rt_take_fault(ctx);
 }
 
 // ---- events / stats -----------------------------------------------------------------------------------------------

@@ -445,6 +445,7 @@ def test_reference_vectors_on_gpu(hip, case):
 @pytest.mark.parametrize("dtype", ALL_DTYPES)
 @pytest.mark.parametrize("op", ["add", "sub", "mul", "div"])
 def test_broadcast_random_vs_oracle(hip, dtype, op):
+    from rtensors_amd import hip as H
     rng = np.random.default_rng(zlib.crc32((dtype + op).encode()))
     if dtype == "bool" and op == "div":
         pytest.skip("boolean division is todo!() in the reference")
@@ -459,22 +460,107 @@ def test_broadcast_random_vs_oracle(hip, dtype, op):
         if rng.random() < 0.3:
             sb = sb[int(rng.integers(0, rank)):]
         va, vb = rand_values(dtype, int(np.prod(sa)), rng), rand_values(dtype, int(np.prod(sb)), rng)
-        if op == "div" and vb.dtype.kind != "f":
-            vb[vb == 0] = 1
+        if op == "div" and vb.dtype.kind != "f" and trial % 3 != 0:
+            vb[vb == 0] = 1                                                # every third trial keeps its zero divisors
+        if op == "div" and vb.dtype.kind == "i" and trial % 6 == 3 and va.size and vb.size:
+            va[rng.integers(0, va.size)] = np.iinfo(va.dtype).min          # MIN / -1 overflows
+            vb[rng.integers(0, vb.size)] = -1
         oa, ob = OTensor.from_buf(dtype, va, sa), OTensor.from_buf(dtype, vb, sb)
         ga, gb = G(hip, dtype, va, sa), G(hip, dtype, vb, sb)
         ova, ovb = random_view(oa, rng), random_view(ob, rng)
+        fault = False
         try:
             with np.errstate(all="ignore"):
                 want = {"add": ova.__add__, "sub": ova.__sub__, "mul": ova.__mul__, "div": ova.__truediv__}[op](ovb)
         except OErr as e:
-            if e.kind != "BroadcastError":
-                continue                                                   # MIN / -1 and the like: the reference panics
-            continue
+            if e.kind == "BroadcastError":
+                continue
+            assert e.kind == "ArithmeticPanic" and op == "div", e.kind
+            fault = True                                                   # zero divisor or MIN / -1: the reference panics
         gva, gvb = replay(ova, ga), replay(ovb, gb)
         got = {"add": gva.__add__, "sub": gva.__sub__, "mul": gva.__mul__, "div": gva.__truediv__}[op](gvb)
+        if fault:
+            # the kernel has run; the fault comes back from the next call that waits for the stream, once
+            with pytest.raises(H.TensorError) as e:
+                got.dump()
+            assert e.value.kind == "ArithmeticError", (trial, dtype, ova.meta, ovb.meta)
+            hip.sync()
+            continue
         assert got.meta.shape == want.meta.shape
         assert got.dump().tobytes() == want.buf.tobytes(), (trial, dtype, op, ova.meta, ovb.meta)
+    hip.sync()                                                             # no fault may be left behind
+
+
+@pytest.mark.parametrize("dtype", ["i8", "u8", "i16", "u16", "i32", "u32", "i64", "u64"])
+def test_integer_division_faults(hip, dtype):
+    """A zero divisor or MIN / -1 inside a tensor: the reference panics (ops/base.rs:27-37), the oracle answers ArithmeticPanic, and the
+    backend returns RT_E_ARITH from the next call that waits for the stream -- once -- for every kernel shape of the broadcast
+    family; without a fault nothing is reported."""
+    from rtensors_amd import hip as H
+    rng = np.random.default_rng(zlib.crc32(dtype.encode()) + 99)
+    npd = cpu.NP_DTYPE[cpu.DTYPE_BY_NAME[dtype]]
+    signed = npd.kind == "i"
+    # (shape of a, shape of b, view of b): contiguous, bias row, column, row kernel, transposed operand, strided generic
+    layouts = [([4096], [4096], None), ([64, 256], [256], None), ([64, 256], [64, 1], None), ([8, 16, 1024], [16, 1], None),
+               ([128, 256], [256, 128], "T"), ([33, 70], [33, 70], "step2"), ([3, 5, 7], [1], None)]
+    for sa, sb, how in layouts:
+        for kind in ("zero", "min_neg1", "clean"):
+            if kind == "min_neg1" and not signed:
+                continue
+            va = rng.integers(1, 100, size=int(np.prod(sa))).astype(npd)
+            vb = rng.integers(1, 10, size=int(np.prod(sb))).astype(npd)
+            ia, ib = int(rng.integers(0, va.size)), int(rng.integers(0, vb.size))
+            if kind == "zero":
+                vb[ib] = 0
+            elif kind == "min_neg1":
+                va[:] = np.iinfo(npd).min                                  # wherever the -1 lands, it meets MIN
+                vb[ib] = -1
+            oa, ob = OTensor.from_buf(dtype, va, sa), OTensor.from_buf(dtype, vb, sb)
+            ga, gb = G(hip, dtype, va, sa), G(hip, dtype, vb, sb)
+            if how == "T":
+                ob, gb = ob.transpose(), gb.transpose()
+            elif how == "step2":
+                oa, ga = oa.slice(1, Slice(None, None, 2)), ga.slice(1, Slice(None, None, 2))
+                ob, gb = ob.slice(1, Slice(None, None, 2)), gb.slice(1, Slice(None, None, 2))
+                if kind != "clean" and (ib % 70) % 2 == 1:
+                    continue                                               # the planted element is not in the view
+            try:
+                want = oa / ob
+                faulted = False
+            except OErr as e:
+                assert e.kind == "ArithmeticPanic"
+                faulted = True
+            assert faulted == (kind != "clean"), (dtype, sa, sb, how, kind)
+            got = ga / gb                                                  # enqueued; nothing is known yet
+            if faulted:
+                with pytest.raises(H.TensorError) as e:
+                    hip.sync()
+                assert e.value.kind == "ArithmeticError" and e.value.status == 7
+                hip.sync()                                                 # reported once, then clear
+                out = got.dump()                                           # the other elements are still the quotients
+                if kind == "zero" and how is None and sa == sb:
+                    ref = np.where(vb == 0, 0, va // np.where(vb == 0, 1, vb)).astype(npd)
+                    assert out.tobytes() == ref.tobytes()
+            else:
+                hip.sync()
+                assert got.dump().tobytes() == want.buf.tobytes(), (dtype, sa, sb, how)
+    # tensor / scalar: a zero scalar is refused at once; -1 faults only if MIN is present
+    v = rng.integers(1, 100, size=1000).astype(npd)
+    g = G(hip, dtype, v, [1000])
+    with pytest.raises(H.TensorError) as e:
+        g /= 0
+    assert e.value.kind == "ArithmeticError"
+    if signed:
+        g /= -1
+        hip.sync()
+        assert g.dump().tobytes() == (-v).astype(npd).tobytes()
+        v[17] = np.iinfo(npd).min
+        g = G(hip, dtype, v, [1000])
+        g /= -1
+        with pytest.raises(H.TensorError) as e:
+            g.dump()
+        assert e.value.kind == "ArithmeticError"
+        hip.sync()
 
 
 @pytest.mark.parametrize("dtype", ["u8", "i8", "i16", "f32", "f64", "bool"])
@@ -902,14 +988,37 @@ def test_rank_limits(hip):
     g = hip.alloc_from_slice(H.F32, x)
     hip.unary_nd("relu", g, 0, shape, strides)
     assert np.array_equal(hip.dump(g), np.maximum(x, 0))
-    # 10 dims of a (3^10)-buffer, every dim sliced with step 2: nothing merges, more than 8 dims remain -> refused, not launched
+    # 10 dims of a (3^10)-buffer, every dim sliced with step 2 (some of them backwards): nothing merges, more than 8 dims remain
+    # after collapsing; the reference takes any rank up to 128 (core/primitives.rs:377-383, backend/cpu.rs:292-352)
+    rng = np.random.default_rng(77)
     n = 3
-    full = [n] * 10
-    st = [n ** (9 - i) * 2 for i in range(10)]
-    big = hip.alloc(H.F32, n ** 10 * 2)
-    with pytest.raises(H.TensorError) as e:
-        hip.unary_nd("relu", big, 0, [2] * 10, st)
-    assert e.value.kind == "UnsupportedOperation"
+    for dtype in ("f32", "i32", "u8", "f64"):
+        vals = rand_values(dtype, n ** 10, rng)
+        o = OTensor.from_buf(dtype, vals.copy(), [n] * 10)
+        g = G(hip, dtype, vals, [n] * 10)
+        ov, gv = o.view(), g.view()
+        for d in range(10):
+            sl = Slice(None, None, -2) if d in (2, 7) else Slice(None, None, 2)
+            ov, gv = ov.slice(d, sl), gv.slice(d, sl)
+        assert ov.meta.shape == [2] * 10
+        # in-place unary, scalar, fill through the view
+        ov.unary_inplace("relu"); gv.unary_inplace("relu")
+        assert g.dump().tobytes() == o.buf.tobytes(), dtype
+        ov += 3; gv += 3
+        assert g.dump().tobytes() == o.buf.tobytes(), dtype
+        # broadcast against a (2, 1, 2) operand and an owned() gather
+        vb = rand_values(dtype, 4, rng)
+        ob, gb = OTensor.from_buf(dtype, vb, [2, 1, 2]), G(hip, dtype, vb, [2, 1, 2])
+        with np.errstate(all="ignore"):
+            want, got = ov + ob, gv + gb
+        assert got.meta.shape == want.meta.shape
+        assert got.dump().tobytes() == want.buf.tobytes(), dtype
+        with np.errstate(all="ignore"):
+            ov *= ob; gv *= gb
+        assert g.dump().tobytes() == o.buf.tobytes(), dtype
+        assert gv.owned().dump().tobytes() == ov.owned().buf.tobytes(), dtype
+        ov.fill(7); gv.fill(7)
+        assert g.dump().tobytes() == o.buf.tobytes(), dtype
     # rank 0 and empty views
     one = hip.alloc_from_slice(H.F32, np.array([-3.0], np.float32))
     hip.unary_nd("neg", one, 0, [], [])
