@@ -1204,6 +1204,35 @@ def test_statistic_reductions_shapes(hip, dtype):
         _check_stat(hip, dtype, 30000, R, 1, rng, offset=8)
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f64"])
+def test_logsumexp_results_near_zero(hip, dtype):
+    """Runs whose logsumexp is close to 0 (R values around -ln R, and mixed-sign pairs): the result is the sum of two terms of
+    opposite sign, max + log(sum exp(x - max)), so its error is relative to the larger of |result| and |largest element|, not to
+    |result| -- the bound the C header states.  (f32 uses the hardware exponential: |error| is about 5e-8 here, which a bound
+    relative to a result of 1e-4 would not admit.)"""
+    code = cpu.DTYPE_BY_NAME[dtype]
+    npd = cpu.NP_DTYPE[code]
+    rng = np.random.default_rng(zlib.crc32(dtype.encode()) + 11)
+    rel = 1e-5 if dtype == "f32" else 1e-12
+    for outer, R, inner in [(20000, 2, 1), (20000, 3, 1), (4000, 10, 1), (300, 1000, 1), (1, 2, 5000), (7, 64, 33), (1, 5000, 3)]:
+        n = outer * R * inner
+        for centre in (-np.log(R), 0.0):
+            x = (centre + rng.normal(size=n) * (1e-3 if centre else 1.0)).astype(npd)
+            if centre == 0.0:
+                x[::2] = -np.abs(x[::2])                                   # mixed signs
+            src = hip.alloc_from_slice(code, x)
+            dst = hip.alloc(code, outer * inner)
+            shape, strides = [outer, R, inner], [R * inner, inner, 1]
+            hip.apply_reduce_contiguous_nd((src, (0, shape, strides)), dst, 1, "logsumexp")
+            got = hip.dump(dst).astype(np.float64)
+            xs = x.astype(np.float64).reshape(outer, R, inner)
+            want = np.logaddexp.reduce(xs, axis=1).reshape(-1)
+            scale = np.maximum(np.abs(want), np.abs(xs).max(axis=1).reshape(-1))
+            assert (np.abs(got - want) <= rel * scale).all(), (dtype, outer, R, inner, centre, np.abs(got - want).max())
+            if centre:
+                assert np.abs(want).max() < 0.05                          # these results really are near zero
+
+
 @pytest.mark.parametrize("dtype", ["f32", "f64", "i32", "u8", "i64", "i16"])
 def test_argmax_argmin_shapes(hip, dtype):
     rng = np.random.default_rng(zlib.crc32(dtype.encode()))
