@@ -445,14 +445,18 @@ def host_layer_runs(iters=10):
     x = T.Tensor.from_buf(be, "f32", rng.standard_normal(rows * cols, dtype=np.float32), [rows, cols])
     target = T.Tensor.from_buf(be, "f32", rng.random(rows * cols, dtype=np.float32) * 2 - 1, [rows, cols])
     bias = T.Tensor.from_buf(be, "f32", rng.standard_normal(cols, dtype=np.float32) * 0.1, [cols])
-    for _ in range(2):
-        T.train_step(x, bias, target, 0.01)
-    be.sync()
-    t0 = time.perf_counter()
-    for _ in range(iters):
-        T.train_step(x, bias, target, 0.01)
-    be.sync()
-    out["c5_train_step_ms"] = round((time.perf_counter() - t0) / iters * 1e3, 4)
+    # the step in three fused passes (rt_fused_*: 7 x 1 GiB of traffic) and on the tape, one backend call per arithmetic step (about 22 x)
+    for name, fn in (("c5_train_step_ms", lambda: T.train_step_fused(x, bias, target, 0.01)), ("c5_train_step_tape_ms", lambda: T.train_step(x, bias, target, 0.01))):
+        for _ in range(2):
+            fn()
+        be.sync()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            fn()
+        be.sync()
+        out[name] = round((time.perf_counter() - t0) / iters * 1e3, 4)
+    out["c5_train_step_bytes"] = 7 * rows * cols * 4
+    out["c5_train_step_GBps"] = round(out["c5_train_step_bytes"] / (out["c5_train_step_ms"] * 1e-3) / 1e9, 1)
     return out
 
 

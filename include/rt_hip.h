@@ -225,6 +225,24 @@ int32_t rt_unary_to(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, uin
 int32_t rt_scalar_to(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, uint64_t src_len, const void* value,
                      uint64_t start, uint64_t len, void* dst, uint64_t dst_len);
 
+/* ---- fused passes of the broadcast / reduce training step ------------------------------------------------------------------
+ * No single counterpart in the trait: the reference's engine issues y = relu(x + bias), loss = mean_l1_loss(y, target)
+ * (ops/broadcast/l1.rs:49-84) and its backward (grad/backwards.rs:148-161, 229-239, 516-538) as one backend call per arithmetic
+ * step, with a full-size temporary between each two.  These three optional entry points run the same IEEE operations per element,
+ * in the same order, in one pass each; every element-wise result is bit for bit what the separate calls give, the two sums are tree
+ * sums within the tolerance of rt_reduce_*.  f32 / f64, row-major contiguous operands from element 0 of 16-byte aligned buffers,
+ * cols (resp. n) a whole number of 16-byte vectors -- anything else is RT_E_INVALID and the caller issues the separate ops.
+ *   rt_fused_bias_relu          y[i, j] = relu(x[i, j] + bias[j])
+ *   rt_fused_l1_forward         gmap[k] = sign(y[k] - target[k]) / N,  loss[0] = (sum_k |y[k] - target[k]|) / N,  N = (T)(f32)n
+ *   rt_fused_l1_relu_backward   dbias[j] = sum_i (y[i, j] > 0 ? 1 : 0) * (gmap[i, j] * upstream[0])   (upstream: one device element,
+ *                               the loss-seeded root of grad/mod.rs:442-447 or a one) */
+int32_t rt_fused_bias_relu(rt_ctx* ctx, int32_t dtype, const void* x, uint64_t x_len, const void* bias, uint64_t bias_len,
+                           void* y, uint64_t y_len, uint64_t rows, uint64_t cols);
+int32_t rt_fused_l1_forward(rt_ctx* ctx, int32_t dtype, const void* y, uint64_t y_len, const void* target, uint64_t target_len,
+                            void* gmap, uint64_t gmap_len, void* loss, uint64_t loss_len, uint64_t n);
+int32_t rt_fused_l1_relu_backward(rt_ctx* ctx, int32_t dtype, const void* gmap, uint64_t gmap_len, const void* y, uint64_t y_len,
+                                  const void* upstream, uint64_t upstream_len, void* dbias, uint64_t dbias_len, uint64_t rows, uint64_t cols);
+
 /* ---- matmul ------------------------------------------------------------------------------------------------------
  * BackendMatMul::matmul (backend/mod.rs:474-485; Cpu backend/cpu.rs:725-951), argument list of protocol Op::Matmul
  * (backend/remote/protocol.rs:269-277): dst[b] = lhs[b] (m x k) * rhs[b] (k x n) for every batch, dst row-major and

@@ -27,7 +27,7 @@ FLAGS = [
 ]
 
 LIBS = {
-    "librt_hip.so": ["rt_runtime.hip", "rt_layout.hip", "rt_elementwise.hip", "rt_broadcast.hip", "rt_broadcast_tile.hip", "rt_reduce.hip", "rt_reduce_stat.hip", "rt_misc.hip", "rt_matmul.hip"],
+    "librt_hip.so": ["rt_runtime.hip", "rt_layout.hip", "rt_elementwise.hip", "rt_broadcast.hip", "rt_broadcast_tile.hip", "rt_reduce.hip", "rt_reduce_stat.hip", "rt_misc.hip", "rt_matmul.hip", "rt_fused.hip"],
     "librt_datagen.so": ["rt_datagen.hip"],
 }
 HEADERS = [os.path.join(CSRC, "rt_common.h"), os.path.join(CSRC, "rt_broadcast_common.h"), os.path.join(HERE, "..", "include", "rt_hip.h")]

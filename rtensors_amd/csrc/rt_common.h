@@ -82,6 +82,8 @@ int32_t rt_take_fault(rt_ctx* ctx);
 int32_t rt_check_reduce_flat(uint64_t src_len, const void* src, const void* dst, uint64_t dst_len, uint64_t start, uint64_t len);
 int32_t rt_check_reduce_nd(uint64_t src_len, const void* src, uint64_t offset, int32_t rank, const uint64_t* shape, const int64_t* strides,
                            const void* dst, uint64_t dst_len, int32_t dim, uint64_t* outer, uint64_t* inner, bool* run);
+int32_t rt_reduce_rows(rt_ctx* ctx, int dtype, int op, const void* src, void* out, uint64_t rows, uint64_t R);     // caller holds ctx->mu
+int32_t rt_reduce_cols(rt_ctx* ctx, int dtype, int op, const void* src, void* out, uint64_t R, uint64_t inner);
 // variance / stdev / logsumexp / norms (out: T*) and argmax / argmin (out: uint64_t*) of src viewed as (outer, R, inner); caller
 // holds ctx->mu
 int32_t rt_reduce_stat(rt_ctx* ctx, int dtype, int op, const void* src, void* out, uint64_t outer, uint64_t R, uint64_t inner);

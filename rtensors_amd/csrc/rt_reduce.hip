@@ -881,6 +881,15 @@ static int32_t reduce_dispatch(rt_ctx* ctx, int dtype, int op, const void* src, 
     return reduce_any(ctx, dtype, op, src, out, outer, R, inner);
 }
 
+// For other translation units (the fused training-step passes): fold `rows` contiguous rows of R elements, or the R rows of an
+// (R, inner) matrix; caller holds ctx->mu.
+int32_t rt_reduce_rows(rt_ctx* ctx, int dtype, int op, const void* src, void* out, uint64_t rows, uint64_t R) {
+    return reduce_dispatch(ctx, dtype, op, src, out, rows, R, 1);
+}
+int32_t rt_reduce_cols(rt_ctx* ctx, int dtype, int op, const void* src, void* out, uint64_t R, uint64_t inner) {
+    return reduce_dispatch(ctx, dtype, op, src, out, 1, R, inner);
+}
+
 extern "C" int32_t rt_reduce_flat(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, uint64_t src_len, void* dst, uint64_t dst_len,
                                   uint64_t start, uint64_t len) {
     RT_TRY(rt_ctx_enter(ctx));

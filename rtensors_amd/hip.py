@@ -261,6 +261,17 @@ class Hip:
         _check(lib.rt_matmul(self._ctx, dst.dtype, lb.ptr, lb.len, loff, len(lshape), _u64s(lshape), _i64s(lstr), CONTIGUITY[lc],
                              rb.ptr, rb.len, roff, len(rshape), _u64s(rshape), _i64s(rstr), CONTIGUITY[rc], dst.ptr, dst.len, b, m, k, n))
 
+    # ---- fused passes of the training step (no counterpart in the trait) --------------------------------------------------------------
+    def fused_bias_relu(self, x: HipBuf, bias: HipBuf, y: HipBuf, rows: int, cols: int):
+        _check(lib.rt_fused_bias_relu(self._ctx, x.dtype, x.ptr, x.len, bias.ptr, bias.len, y.ptr, y.len, rows, cols))
+
+    def fused_l1_forward(self, y: HipBuf, target: HipBuf, gmap: HipBuf, loss: HipBuf, n: int):
+        _check(lib.rt_fused_l1_forward(self._ctx, y.dtype, y.ptr, y.len, target.ptr, target.len, gmap.ptr, gmap.len, loss.ptr, loss.len, n))
+
+    def fused_l1_relu_backward(self, gmap: HipBuf, y: HipBuf, upstream: HipBuf, dbias: HipBuf, rows: int, cols: int):
+        _check(lib.rt_fused_l1_relu_backward(self._ctx, y.dtype, gmap.ptr, gmap.len, y.ptr, y.len, upstream.ptr, upstream.len, dbias.ptr, dbias.len,
+                                             rows, cols))
+
     # ---- timing -----------------------------------------------------------------------------------------------------------
     def event(self):
         e = C.c_void_p()

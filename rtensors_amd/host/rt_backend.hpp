@@ -272,6 +272,19 @@ class Hip {
                         b, m, k, n));
     }
 
+    // ---- fused passes of y = relu(x + bias), mean_l1_loss(y, t) and their backward (no counterpart in the trait; every element-wise
+    // result is bit for bit what the separate calls give) -----------------------------------------------------------------------
+    void fused_bias_relu(const HipBuf& x, const HipBuf& bias, HipBuf& y, uint64_t rows, uint64_t cols) const {
+        check(rt_fused_bias_relu(raw(), y.dtype(), x.ptr(), x.len(), bias.ptr(), bias.len(), y.ptr(), y.len(), rows, cols));
+    }
+    void fused_l1_forward(const HipBuf& y, const HipBuf& target, HipBuf& gmap, HipBuf& loss, uint64_t n) const {
+        check(rt_fused_l1_forward(raw(), y.dtype(), y.ptr(), y.len(), target.ptr(), target.len(), gmap.ptr(), gmap.len(), loss.ptr(), loss.len(), n));
+    }
+    void fused_l1_relu_backward(const HipBuf& gmap, const HipBuf& y, const HipBuf& upstream, HipBuf& dbias, uint64_t rows, uint64_t cols) const {
+        check(rt_fused_l1_relu_backward(raw(), y.dtype(), gmap.ptr(), gmap.len(), y.ptr(), y.len(), upstream.ptr(), upstream.len(), dbias.ptr(), dbias.len(),
+                                        rows, cols));
+    }
+
     // row-major copy of a view (what TensorView::owned needs, core/tensor.rs:299-325) in one launch
     void gather(const HipBuf& src, const MetaTensor& m, HipBuf& dst) const {
         check(rt_gather(raw(), src.dtype(), src.ptr(), src.len(), m.offset, (int32_t)m.rank(), m.shape.data(), m.strides.data(), dst.ptr(), dst.len()));

@@ -316,6 +316,14 @@ def train_step(x: Tensor, bias: Tensor, target: Tensor, lr: float, mode: str = "
     return Tensor(pl, x.backend), Tensor(pg, x.backend)
 
 
+def train_step_fused(x: Tensor, bias: Tensor, target: Tensor, lr: float, seed_with_loss: bool = True):
+    """The same step through the three fused passes (rt_fused_*).  Returns (loss, d_bias, used_fused); operands the fused form does
+    not take (views, dtypes other than f32 / f64, rows that are not whole 16-byte vectors) go through the tape and used_fused is False."""
+    pl, pg, used = C.c_void_p(), C.c_void_p(), C.c_int(0)
+    _ck(_h.rth_train_step_fused(x._p, bias._p, target._p, C.c_double(lr), 1 if seed_with_loss else 0, C.byref(pl), C.byref(pg), C.byref(used)))
+    return Tensor(pl, x.backend), Tensor(pg, x.backend), bool(used.value)
+
+
 def linear_step(x: Tensor, w: Tensor, target: Tensor, lr: float, seed_with_loss: bool = True):
     """y = x @ w; loss = mean_l1_loss(y, target); backward; SGD(lr) on w in place.  Returns (loss, d_w)."""
     pl, pg = C.c_void_p(), C.c_void_p()

@@ -250,6 +250,87 @@ def test_train_step_matches_oracle(T, be, dtype, mode, seed_with_loss):
 
 @pytest.mark.parametrize("dtype", ["f32", "f64"])
 @pytest.mark.parametrize("seed_with_loss", [True, False])
+def test_fused_train_step_matches_oracle(T, be, dtype, seed_with_loss):
+    """The three fused passes against the oracle's literal sequence: y and the L1 gradient map bit for bit (through the C ABI), the
+    loss and d(bias) within the reduction tolerance, the updated bias as the tape leaves it; and the host layer's fused step against
+    its own tape."""
+    from rtensors_amd import datagen, hip as H
+    npd = cpu.NP_DTYPE[cpu.DTYPE_BY_NAME[dtype]]
+    tol = 1e-5 if dtype == "f32" else 1e-12
+    for n, d in ((384, 96), (1000, 260), (7, 4), (5, 6), (4100, 4096)):
+        x = datagen.normal(npd, n * d, 4, 0)
+        bias = datagen.normal(npd, d, 4, 1, 0.1)
+        target = datagen.uniform(npd, n * d, 4, 2)
+        x[::97] = 0; bias[::5] = 0; target[::89] = 0                     # ties: pre == 0, y == t
+        ox, ob, ot = OTensor.from_buf(dtype, x, [n, d]), OTensor.from_buf(dtype, bias, [d]), OTensor.from_buf(dtype, target, [n, d])
+        # element-wise pieces of the literal sequence, op by op, on the oracle
+        oy = (ox + ob).unary("relu")
+        odiff = oy - ot
+        ogmap = odiff.unary("sign") / float(np.float32(n * d))
+        absdiff = np.abs(odiff.buf.astype(np.float64))
+        fits = d % (4 if dtype == "f32" else 2) == 0
+        # the same through the C ABI
+        hip = H.Hip.new(0) if fits else None
+        if not fits:
+            terms = None
+        if fits:
+            code = H.DTYPE_BY_NAME[dtype]
+            hx, hb, ht = hip.alloc_from_slice(code, x), hip.alloc_from_slice(code, bias), hip.alloc_from_slice(code, target)
+            hy, hg, hl, hd = hip.alloc(code, n * d), hip.alloc(code, n * d), hip.alloc(code, 1), hip.alloc(code, d)
+            hip.fused_bias_relu(hx, hb, hy, n, d)
+            hip.fused_l1_forward(hy, ht, hg, hl, n * d)
+            assert hip.dump(hy).tobytes() == oy.buf.tobytes(), (dtype, n, d, "y")
+            assert hip.dump(hg).tobytes() == ogmap.buf.tobytes(), (dtype, n, d, "gmap")
+            loss = hip.dump(hl)[0]
+            assert abs(float(loss) - absdiff.sum() / float(np.float32(n * d))) <= tol * absdiff.sum() / (n * d) + 1e-300
+            up = hl if seed_with_loss else hip.alloc_from_slice(code, np.ones(1, npd))
+            hip.fused_l1_relu_backward(hg, hy, up, hd, n, d)
+            upv = loss if seed_with_loss else npd.type(1)
+            terms = ((oy.buf > 0).astype(npd) * (ogmap.buf * upv).astype(npd)).astype(npd).reshape(n, d).astype(np.float64)
+            assert np.all(np.abs(hip.dump(hd).astype(np.float64) - terms.sum(axis=0)) <= tol * np.abs(terms).sum(axis=0) + 1e-300), (dtype, n, d)
+            hip.close()
+        # host layer: fused step against the tape and the oracle's step
+        gx, gt = T.Tensor.from_buf(be, dtype, x, [n, d]), T.Tensor.from_buf(be, dtype, target, [n, d])
+        gb1, gb2 = T.Tensor.from_buf(be, dtype, bias, [d]), T.Tensor.from_buf(be, dtype, bias, [d])
+        floss, fgrad, used = T.train_step_fused(gx, gb1, gt, 0.01, seed_with_loss)
+        tloss, tgrad = T.train_step(gx, gb2, gt, 0.01, "sum", seed_with_loss)
+        assert used == fits
+        assert abs(float(floss.to_numpy()) - absdiff.sum() / float(np.float32(n * d))) <= tol * absdiff.sum() / (n * d) + 1e-300
+        assert fgrad.shape == [d]
+        if terms is None:
+            upv = npd.type(floss.to_numpy()) if seed_with_loss else npd.type(1)
+            terms = ((oy.buf > 0).astype(npd) * (ogmap.buf * upv).astype(npd)).astype(npd).reshape(n, d).astype(np.float64)
+        gtol = 2 * tol * np.abs(terms).sum(axis=0) + 1e-300
+        assert np.all(np.abs(fgrad.to_numpy().astype(np.float64) - tgrad.to_numpy().astype(np.float64)) <= gtol)
+        assert np.max(np.abs(gb1.to_numpy().astype(np.float64) - gb2.to_numpy().astype(np.float64))) <= 0.01 * gtol.max() + np.finfo(npd).eps
+        if n * d <= 300000:
+            # the oracle's whole step (its loss is a sequential f32 sum, which is itself only good to about 1e-7 * n: small shapes only)
+            oloss, ograd = oracle_train_step(ox, ob, ot, 0.01, "sum", seed_with_loss)
+            assert abs(float(floss.to_numpy()) - float(oloss.buf[0])) <= tol * absdiff.sum() / (n * d) + 1e-300
+            assert ograd.meta.shape == [d]
+            assert np.all(np.abs(fgrad.to_numpy().astype(np.float64) - ograd.buf.astype(np.float64)) <= gtol)
+            assert np.max(np.abs(gb1.to_numpy().astype(np.float64) - ob.buf.astype(np.float64))) <= 0.01 * gtol.max() + np.finfo(npd).eps
+
+
+def test_fused_passes_refuse_what_they_do_not_take(be):
+    from rtensors_amd import hip as H
+    hip = H.Hip.new(0)
+    a, b, c = hip.alloc(H.F32, 4 * 6), hip.alloc(H.F32, 6), hip.alloc(H.F32, 4 * 6)
+    with pytest.raises(H.TensorError) as e:
+        hip.fused_bias_relu(a, b, c, 4, 6)                                # rows of 6 f32 are not whole vectors
+    assert e.value.status == 1
+    with pytest.raises(H.TensorError) as e:
+        hip.fused_bias_relu(a, b, c, 5, 8)                                # more than the buffers hold
+    assert e.value.kind == "IdxOutOfBounds"
+    i = hip.alloc(H.I32, 16)
+    with pytest.raises(H.TensorError) as e:
+        hip.fused_bias_relu(i, i, i, 2, 8)
+    assert e.value.kind == "UnsupportedOperation"
+    hip.close()
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64"])
+@pytest.mark.parametrize("seed_with_loss", [True, False])
 def test_linear_step_matches_oracle(T, be, dtype, seed_with_loss):
     """y = x @ w, mean L1 loss, backward through the MatMul node (d(w) = x^T @ upstream), SGD on w."""
     from rtensors_amd import datagen
@@ -421,7 +502,10 @@ def test_config5_full_size_step(be, T):
     bias = datagen.normal(np.float32, d, 4, 1, 0.1)
     target = datagen.uniform(np.float32, n * d, 4, 2)
     gx, gb, gt = T.Tensor.from_buf(be, "f32", x, [n, d]), T.Tensor.from_buf(be, "f32", bias, [d]), T.Tensor.from_buf(be, "f32", target, [n, d])
+    gb_fused = T.Tensor.from_buf(be, "f32", bias, [d])
     gloss, ggrad = T.train_step(gx, gb, gt, 0.01, "sum", True)
+    floss, fgrad, used = T.train_step_fused(gx, gb_fused, gt, 0.01, True)
+    assert used
     pre = x.reshape(n, d) + bias
     y = np.maximum(pre, 0)
     diff = y - target.reshape(n, d)
@@ -438,3 +522,9 @@ def test_config5_full_size_step(be, T):
     new_bias = gb.to_numpy()
     want_bias = bias - (ggrad.to_numpy() * np.float32(0.01)).astype(np.float32)
     assert new_bias.tobytes() == want_bias.astype(np.float32).tobytes()
+    # the fused passes: the same loss and gradient within the same bounds, the same update rule
+    assert abs(float(floss.to_numpy()) - loss) <= 1e-5 * loss
+    up_f = (gm * np.float32(float(floss.to_numpy()))).astype(np.float32) * (pre > 0)
+    assert np.all(np.abs(fgrad.to_numpy().astype(np.float64) - up_f.astype(np.float64).sum(axis=0)) <= 1e-5 * np.abs(up_f.astype(np.float64)).sum(axis=0) + 1e-30)
+    want_fused = bias - (fgrad.to_numpy() * np.float32(0.01)).astype(np.float32)
+    assert gb_fused.to_numpy().tobytes() == want_fused.astype(np.float32).tobytes()
