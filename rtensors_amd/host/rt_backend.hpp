@@ -4,6 +4,7 @@
 // layer builds with a plain host compiler, the way a Rust FFI binding would.
 #pragma once
 
+#include <cmath>
 #include <limits>
 #include <cstring>
 #include <memory>
@@ -34,14 +35,29 @@ struct Scalar {
     alignas(16) unsigned char bytes[16] = {0};
     template <class T> static Scalar of(T v) { Scalar s; s.dtype = dtype_of<T>::value; std::memcpy(s.bytes, &v, sizeof(T)); return s; }
     template <class T> T as() const { T v; std::memcpy(&v, bytes, sizeof(T)); return v; }
+    // double -> integer with the meaning of Rust's `as` (core/value.rs:268-312 uses it for every conversion): NaN is 0, values
+    // beyond the type's range saturate, the rest truncate toward zero.  A plain C++ cast is undefined for the first two.
+    template <class T> static T int_from_double(double x) {
+        if (x != x) return (T)0;
+        constexpr bool is_signed = (T)-1 < (T)0;
+        constexpr int bits = (int)(8 * sizeof(T)) - (is_signed ? 1 : 0);
+        const double hi = std::ldexp(1.0, bits);                        // first value above the range, exact in double
+        // through u128 so that no signed shift overflows: the conversion back to T is modular
+        const T max_v = is_signed ? (T)(((u128)1 << (bits & 127)) - 1) : (T)~(T)0;
+        const T min_v = is_signed ? (T)((u128)1 << (bits & 127)) : (T)0;
+        if (x >= hi) return max_v;
+        if (is_signed ? x < -hi : x <= -1.0) return min_v;
+        if (!is_signed && x < 0.0) return (T)0;                         // (-1, 0) truncates to 0
+        return (T)x;
+    }
     // numeric literal -> element of `dtype` (what `T::from` does for the scalar operand of `tensor + 3`)
     static Scalar from_double(int dtype, double x) {
         switch (dtype) {
-            case RT_U8: return of<uint8_t>((uint8_t)x);  case RT_I8: return of<int8_t>((int8_t)x);
-            case RT_U16: return of<uint16_t>((uint16_t)x); case RT_I16: return of<int16_t>((int16_t)x);
-            case RT_U32: return of<uint32_t>((uint32_t)x); case RT_I32: return of<int32_t>((int32_t)x);
-            case RT_U64: return of<uint64_t>((uint64_t)x); case RT_I64: return of<int64_t>((int64_t)x);
-            case RT_U128: return of<u128>((u128)x); case RT_I128: return of<i128>((i128)x);
+            case RT_U8: return of<uint8_t>(int_from_double<uint8_t>(x));    case RT_I8: return of<int8_t>(int_from_double<int8_t>(x));
+            case RT_U16: return of<uint16_t>(int_from_double<uint16_t>(x)); case RT_I16: return of<int16_t>(int_from_double<int16_t>(x));
+            case RT_U32: return of<uint32_t>(int_from_double<uint32_t>(x)); case RT_I32: return of<int32_t>(int_from_double<int32_t>(x));
+            case RT_U64: return of<uint64_t>(int_from_double<uint64_t>(x)); case RT_I64: return of<int64_t>(int_from_double<int64_t>(x));
+            case RT_U128: return of<u128>(int_from_double<u128>(x));        case RT_I128: return of<i128>(int_from_double<i128>(x));
             case RT_F32: return of<float>((float)x); case RT_F64: return of<double>(x);
             case RT_BOOL: return of<boolean>(boolean{(uint8_t)(x != 0)});
         }
