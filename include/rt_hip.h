@@ -111,7 +111,8 @@ int32_t rt_alloc_from_slice(rt_ctx* ctx, int32_t dtype, const void* host_src, ui
 int32_t rt_free(rt_ctx* ctx, void* buf);
 /* Backend::copy_from_slice: lengths must match (RT_E_SIZE_MISMATCH otherwise). */
 int32_t rt_copy_from_slice(rt_ctx* ctx, int32_t dtype, void* dst, uint64_t dst_len, const void* host_src, uint64_t src_len);
-/* Backend::copy_range_within: device-to-device copy of `len` elements. */
+/* Backend::copy_range_within: device-to-device copy of `len` elements.  A range copied onto itself is a no-op; ranges of one buffer
+ * that overlap otherwise are refused with RT_E_INVALID (the trait's `&mut dst` / `&src` pair cannot express them either). */
 int32_t rt_copy_range_within(rt_ctx* ctx, int32_t dtype, void* dst, uint64_t dst_len, const void* src, uint64_t src_len,
                              uint64_t dst_offset, uint64_t src_offset, uint64_t len);
 /* Backend::read / Backend::write: one element; synchronises first. */
@@ -153,7 +154,8 @@ int32_t rt_scalar_nd(rt_ctx* ctx, int32_t dtype, int32_t op, void* buf, uint64_t
 /* ---- N-d broadcast (Backend::broadcast, backend/mod.rs:296-309; Cpu backend/cpu.rs:292-352) --------------------
  * dst[c] = left[c] (op) right[c] for every coordinate c of `shape`.  The three operands share `shape`
  * (expansion is expressed as stride 0, ops/broadcast/mod.rs:13-55); strides may be negative.  dst may be the
- * same buffer as left with the same layout (in-place `a op= b`).
+ * very same view as an input (same buffer, offset and strides: the in-place `a op= b`).  A destination whose address range meets
+ * an input's in any other way is refused with RT_E_INVALID: block order would decide the result.
  * Integer division: a zero divisor or MIN / -1 inside the tensors (a panic in the reference, ops/base.rs:27-37) cannot be seen
  * before the kernel has run; the kernel stores 0 / MIN for such elements and sets a fault word of the context, and the next
  * call that waits for the stream (rt_sync, rt_read, rt_dump, rt_equal) returns RT_E_ARITH once and clears it.  The same holds for

@@ -748,6 +748,8 @@ extern "C" int32_t rt_gather(rt_ctx* ctx, int32_t dtype, const void* src, uint64
     if (count > dst_len) return rt_fail(RT_E_OUT_OF_BOUNDS, "gather: %llu elements into a buffer of %llu", (unsigned long long)count, (unsigned long long)dst_len);
     if (count == 0) return RT_OK;
     if (!src || !dst) return rt_fail(RT_E_INVALID, "gather: null buffer");
+    if (rt_spans_meet(rt_view_span(src, es, offset, rank, shape, strides), rt_run_span(dst, es, 0, count)))
+        return rt_fail(RT_E_INVALID, "gather: the destination overlaps the source view");
     // 128-bit elements move as pairs of 64-bit words: one more unit-stride dim of size 2
     const int words = es == 16 ? 2 : 1;
     uint64_t shp[RT_MAX_INPUT_RANK + 1];
@@ -800,6 +802,16 @@ extern "C" int32_t rt_broadcast(rt_ctx* ctx, int32_t dtype, int32_t op, int32_t 
         if (shape[i] > 1 && dst_strides[i] == 0)
             return rt_fail(RT_E_INVALID, "broadcast: destination has stride 0 along dim %d of size %llu (it would be written more than once)",
                            i, (unsigned long long)shape[i]);
+    {
+        const int es = rt_elem_size(dtype);
+        const ByteSpan ds = rt_view_span(dst, es, dst_offset, rank, shape, dst_strides);
+        if (rt_spans_meet(ds, rt_view_span(left, es, left_offset, rank, shape, left_strides)) &&
+            !rt_same_view(left, left_offset, left_strides, dst, dst_offset, dst_strides, rank, shape))
+            return rt_fail(RT_E_INVALID, "broadcast: the destination overlaps the left operand without being the same view");
+        if (rt_spans_meet(ds, rt_view_span(right, es, right_offset, rank, shape, right_strides)) &&
+            !rt_same_view(right, right_offset, right_strides, dst, dst_offset, dst_strides, rank, shape))
+            return rt_fail(RT_E_INVALID, "broadcast: the destination overlaps the right operand without being the same view");
+    }
     NdDesc d;
     const int64_t* sp[3] = {left_strides, right_strides, dst_strides};
     const uint64_t offs[3] = {left_offset, right_offset, dst_offset};

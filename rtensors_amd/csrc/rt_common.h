@@ -105,6 +105,19 @@ static inline int rt_elem_size(int dtype) {
 int32_t rt_check_extent(const char* what, uint64_t offset, int rank, const uint64_t* shape, const int64_t* strides,
                         uint64_t len, uint64_t* count);
 
+// Byte range [lo, hi) that a non-empty, already validated view touches in its buffer.
+struct ByteSpan { uintptr_t lo, hi; };
+ByteSpan rt_view_span(const void* base, int elem_size, uint64_t offset, int rank, const uint64_t* shape, const int64_t* strides);
+inline ByteSpan rt_run_span(const void* base, int elem_size, uint64_t start, uint64_t len) {
+    const uintptr_t lo = reinterpret_cast<uintptr_t>(base) + (uintptr_t)start * (uintptr_t)elem_size;
+    return ByteSpan{lo, lo + (uintptr_t)len * (uintptr_t)elem_size};
+}
+inline bool rt_spans_meet(ByteSpan a, ByteSpan b) { return a.lo < b.hi && b.lo < a.hi; }
+// The one aliasing an output may have with an input: the very same elements in the same order (what the in-place operators
+// pass).  Every lane then reads its elements before it writes them.  Any other overlap makes the result depend on block order.
+bool rt_same_view(const void* a, uint64_t a_offset, const int64_t* a_strides, const void* b, uint64_t b_offset, const int64_t* b_strides,
+                  int rank, const uint64_t* shape);
+
 // A view over up to three operands sharing one shape, after removal of size-1 dims and merging of adjacent dims
 // that are mergeable in every operand.  Dim 0 is outermost.
 struct NdDesc {

@@ -620,6 +620,8 @@ int32_t run_view(rt_ctx* ctx, const char* what, const ViewArg& va, F f) {
     if (va.dst == va.buf) return rt_fail(RT_E_INVALID, "%s: the out-of-place form needs a destination other than the source", what);
     if (!(d.rank == 0 || (d.rank == 1 && d.stride[0][0] == 1)))
         return rt_fail(RT_E_WRONG_DIMS, "%s: the out-of-place form takes a forward contiguous run (gather other views first)", what);
+    if (rt_spans_meet(rt_run_span(va.buf, (int)sizeof(T), (uint64_t)d.offset[0], count), rt_run_span(va.dst, (int)sizeof(T), 0, count)))
+        return rt_fail(RT_E_INVALID, "%s: the destination overlaps the source run", what);
     return launch_contig_out<T, F>(ctx, (const T*)va.buf + d.offset[0], (T*)va.dst, (size_t)count, f);
 }
 

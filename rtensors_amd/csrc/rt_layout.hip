@@ -39,6 +39,24 @@ int32_t rt_check_extent(const char* what, uint64_t offset, int rank, const uint6
     return RT_OK;
 }
 
+ByteSpan rt_view_span(const void* base, int elem_size, uint64_t offset, int rank, const uint64_t* shape, const int64_t* strides) {
+    __int128 lo = (__int128)offset, hi = (__int128)offset;
+    for (int i = 0; i < rank; ++i) {
+        __int128 span = ((__int128)shape[i] - 1) * (__int128)strides[i];
+        if (span < 0) lo += span; else hi += span;
+    }
+    const uintptr_t b = reinterpret_cast<uintptr_t>(base);
+    return ByteSpan{b + (uintptr_t)lo * (uintptr_t)elem_size, b + ((uintptr_t)hi + 1) * (uintptr_t)elem_size};
+}
+
+bool rt_same_view(const void* a, uint64_t a_offset, const int64_t* a_strides, const void* b, uint64_t b_offset, const int64_t* b_strides,
+                  int rank, const uint64_t* shape) {
+    if (a != b || a_offset != b_offset) return false;
+    for (int i = 0; i < rank; ++i)
+        if (shape[i] > 1 && a_strides[i] != b_strides[i]) return false;
+    return true;
+}
+
 namespace {
 struct Dim { int64_t n; int64_t s[3]; };
 

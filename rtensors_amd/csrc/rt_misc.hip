@@ -268,6 +268,8 @@ extern "C" int32_t rt_convert(rt_ctx* ctx, int32_t src_dtype, const void* src, u
                        (unsigned long long)dst_len);
     if (src_len == 0) return RT_OK;
     if (!src || !dst) return rt_fail(RT_E_INVALID, "convert: null buffer");
+    if (rt_spans_meet(rt_run_span(src, rt_elem_size(src_dtype), 0, src_len), rt_run_span(dst, rt_elem_size(dst_dtype), 0, dst_len)))
+        return rt_fail(RT_E_INVALID, "convert: the destination overlaps the source");
     CtxGuard g(ctx);
     return convert_any(ctx, src_dtype, src, dst_dtype, dst, (size_t)src_len);
 }

@@ -443,6 +443,11 @@ extern "C" int32_t rt_copy_range_within(rt_ctx* ctx, int32_t dtype, void* dst, u
                        (unsigned long long)src_offset, (unsigned long long)len);
     if (!len) return RT_OK;
     if (!dst || !src) return rt_fail(RT_E_INVALID, "copy_range_within: null pointer");
+    {
+        const ByteSpan a = rt_run_span(dst, es, dst_offset, len), b = rt_run_span(src, es, src_offset, len);
+        if (a.lo == b.lo) return RT_OK;                       // a range onto itself
+        if (rt_spans_meet(a, b)) return rt_fail(RT_E_INVALID, "copy_range_within: the two ranges overlap");
+    }
     CtxGuard g(ctx);
     return device_copy(ctx, (char*)dst + dst_offset * es, (const char*)src + src_offset * es, (size_t)len * es);
 }

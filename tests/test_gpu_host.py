@@ -447,12 +447,32 @@ def test_config3_both_variants_agree_and_match_formula(be, T):
     z2 = hb.alloc_uninit(H.F32, B * J * K * L)
     hb.broadcast((gbase, (mv.meta.offset, shape, [K * L, 0, -1, K])), (gy, (0, shape, [0, L, 0, 1])), (z2, (0, shape, zs)), "add")
     assert z1 == z2                                                   # device-side equality over all 2^29 elements
+    # each result on its own against the formula: whole (b, j) slabs of K rows -- 12 slabs = 6144 rows per variant, drawn
+    # separately for the two, every b and both ends of j among them -- and 64 single rows anywhere
     rng = np.random.default_rng(0)
-    for _ in range(64):
-        b, j, k = int(rng.integers(0, B)), int(rng.integers(0, J)), int(rng.integers(0, K))
+    slab = hb.alloc_uninit(H.F32, K * L)
+    for name, z in (("contiguous x", z1), ("permuted x", z2)):
+        pairs = {(0, 0), (B - 1, J - 1), (0, J - 1), (B - 1, 0)}
+        while len(pairs) < 12:
+            pairs.add((int(rng.integers(0, B)), int(rng.integers(0, J))))
+        for b, j in sorted(pairs):
+            hb.copy_range_within(slab, z, 0, (b * J + j) * K * L, K * L)
+            assert hb.dump(slab).tobytes() == (x[b] + y[j][None, :]).tobytes(), (name, b, j)
         row = hb.alloc_uninit(H.F32, L)
-        hb.copy_range_within(row, z1, 0, ((b * J + j) * K + k) * L, L)
-        assert hb.dump(row).tobytes() == (x[b, k] + y[j]).tobytes()
+        for _ in range(64):
+            b, j, k = int(rng.integers(0, B)), int(rng.integers(0, J)), int(rng.integers(0, K))
+            hb.copy_range_within(row, z, 0, ((b * J + j) * K + k) * L, L)
+            assert hb.dump(row).tobytes() == (x[b, k] + y[j]).tobytes(), (name, b, j, k)
+    # a checksum over everything: sum over (j, k) of z[b, j, k, :] = J * sum_k x[b, k, :] + K * sum_j y[j, :], evaluated by the
+    # device's own axis reductions on the 2 GiB result and compared with float64 on the host within the reduction tolerance
+    for z in (z1, z2):
+        part = hb.alloc(H.F32, B * J * L)
+        hb.apply_reduce_contiguous_nd((z, (0, [B * J, K, L], [K * L, L, 1])), part, 1, "sum")
+        tot = hb.alloc(H.F32, B * L)
+        hb.apply_reduce_contiguous_nd((part, (0, [B, J, L], [J * L, L, 1])), tot, 1, "sum")
+        want = J * x.astype(np.float64).sum(axis=1) + K * y.astype(np.float64).sum(axis=0)[None, :]
+        bound = 2e-5 * (J * np.abs(x.astype(np.float64)).sum(axis=1) + K * np.abs(y.astype(np.float64)).sum(axis=0)[None, :])
+        assert np.all(np.abs(hb.dump(tot).reshape(B, L).astype(np.float64) - want) <= bound)
     hb.sync()
 
 

@@ -714,6 +714,52 @@ def test_bad_descriptors_are_refused_not_launched(hip):
     assert not hip.dump(g).any()
 
 
+def test_overlapping_source_and_destination_are_refused(hip):
+    """An output may be the very same view as an input (the in-place operators); any other overlap of the address ranges would
+    let block order decide the result and is refused before a launch.  The trait's `&mut dst` / `&src` pairs
+    (backend/mod.rs:228, 303-309) cannot express such calls in the reference either."""
+    from rtensors_amd import hip as H
+    base = np.arange(64, dtype=np.float32)
+    g = hip.alloc_from_slice(H.F32, base)
+    other = hip.alloc_from_slice(H.F32, np.ones(64, np.float32))
+    row = (0, [32], [1])
+    # the same view on both sides: in place, fine -- for the left and for the right operand
+    hip.broadcast((g, row), (other, row), (g, row), "add")
+    hip.broadcast((other, row), (g, row), (g, row), "mul")
+    assert np.array_equal(hip.dump(g)[:32], base[:32] + 1) and np.array_equal(hip.dump(g)[32:], base[32:])
+    for bad in [(1, [32], [1]), (31, [32], [-1]), (0, [16], [2])]:
+        shape = bad[1]
+        dst = (0, shape, [1])
+        for left, right in (((g, bad), (other, dst)), ((other, dst), (g, bad))):
+            with pytest.raises(H.TensorError) as e:
+                hip.broadcast(left, right, (g, dst), "add")
+            assert e.value.kind == "InvalidArgument" and "overlaps" in str(e.value), bad
+    # disjoint halves of one buffer are fine
+    hip.broadcast((g, (32, [32], [1])), (other, row), (g, row), "add")
+    assert np.array_equal(hip.dump(g)[:32], base[32:] + 1)
+    # copy_range_within: onto itself is a no-op, a shifted overlap is refused, disjoint ranges are copied
+    hip.copy_range_within(g, g, 4, 4, 20)
+    with pytest.raises(H.TensorError) as e:
+        hip.copy_range_within(g, g, 4, 0, 20)
+    assert e.value.kind == "InvalidArgument"
+    hip.copy_range_within(g, g, 0, 40, 8)
+    assert np.array_equal(hip.dump(g)[:8], base[40:48])
+    # out-of-place unary / scalar, gather and convert into a range of their own source
+    def window(byte_offset, length, dtype):           # a range inside g, not owned: backend None keeps it from being freed
+        return H.HipBuf(None, g.ptr + byte_offset, length, dtype)
+    sub = window(32, 32, H.F32)
+    with pytest.raises(H.TensorError):
+        hip.unary_to("relu", g, 0, 16, sub)
+    with pytest.raises(H.TensorError):
+        hip.scalar_to("add", g, 1.0, 0, 16, sub)
+    with pytest.raises(H.TensorError):
+        hip.gather(g, (0, [4, 4], [1, 4]), sub)
+    with pytest.raises(H.TensorError):
+        hip.convert(window(0, 32, H.F32), window(64, 32, H.I32))
+    hip.unary_to("relu", g, 0, 8, sub)                # source elements 0..8, destination elements 8..16: disjoint
+    assert np.array_equal(hip.dump(g)[8:16], hip.dump(g)[:8])
+
+
 def test_gather_views(hip):
     rng = np.random.default_rng(6)
     for dtype in ("f32", "u8", "i64", "i16"):
