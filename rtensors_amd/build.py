@@ -24,6 +24,8 @@ ARCH = os.environ.get("RT_HIP_ARCH", "gfx950")
 FLAGS = [
     "-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17", "-ffp-contract=off", "-fno-fast-math",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wno-unused-function",
+    # the device code of each object is stored zstd-compressed and unpacked by the HIP runtime when the library is loaded
+    "--offload-compress",
 ]
 
 LIBS = {
