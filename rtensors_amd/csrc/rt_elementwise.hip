@@ -655,9 +655,24 @@ int32_t fill_any(rt_ctx* ctx, int32_t dtype, void* buf, uint64_t buf_len, const 
     RT_TRY(rt_ctx_enter(ctx));
     if (!value) return rt_fail(RT_E_INVALID, "fill: null value");
     const ViewArg va{buf, buf_len, offset, rank, shape, strides, nullptr, 0};
-    RT_FOR_DTYPE(dtype, return (run_view<T, FillF<T>>(ctx, "fill", va, FillF<T>{load_scalar<T>(value)})));
+    // a fill moves bits: one instantiation per element width serves every dtype of that width
+    switch (rt_elem_size(dtype)) {
+        case 1: return run_view<uint8_t, FillF<uint8_t>>(ctx, "fill", va, FillF<uint8_t>{load_scalar<uint8_t>(value)});
+        case 2: return run_view<uint16_t, FillF<uint16_t>>(ctx, "fill", va, FillF<uint16_t>{load_scalar<uint16_t>(value)});
+        case 4: return run_view<uint32_t, FillF<uint32_t>>(ctx, "fill", va, FillF<uint32_t>{load_scalar<uint32_t>(value)});
+        case 8: return run_view<uint64_t, FillF<uint64_t>>(ctx, "fill", va, FillF<uint64_t>{load_scalar<uint64_t>(value)});
+        case 16: return run_view<u128_t, FillF<u128_t>>(ctx, "fill", va, FillF<u128_t>{load_scalar<u128_t>(value)});
+    }
     return no_dtype("fill", dtype);
 }
+
+// Wrapping add / subtract / multiply give the same bits for a signed integer and the unsigned one of its width.
+template <class T> struct unsigned_twin { typedef T type; };
+template <> struct unsigned_twin<int8_t> { typedef uint8_t type; };
+template <> struct unsigned_twin<int16_t> { typedef uint16_t type; };
+template <> struct unsigned_twin<int32_t> { typedef uint32_t type; };
+template <> struct unsigned_twin<int64_t> { typedef uint64_t type; };
+template <> struct unsigned_twin<i128_t> { typedef u128_t type; };
 
 template <class T, int OP>
 int32_t unary_go(rt_ctx* ctx, const ViewArg& va) {
@@ -717,9 +732,9 @@ int32_t scalar_go(rt_ctx* ctx, const ViewArg& va, const void* value) {
 template <class T>
 int32_t scalar_typed(rt_ctx* ctx, int op, const ViewArg& va, const void* value) {
     switch (op) {
-        case RT_S_ADD: return scalar_go<T, RT_S_ADD>(ctx, va, value);
-        case RT_S_SUB: return scalar_go<T, RT_S_SUB>(ctx, va, value);
-        case RT_S_MUL: return scalar_go<T, RT_S_MUL>(ctx, va, value);
+        case RT_S_ADD: return scalar_go<typename unsigned_twin<T>::type, RT_S_ADD>(ctx, va, value);
+        case RT_S_SUB: return scalar_go<typename unsigned_twin<T>::type, RT_S_SUB>(ctx, va, value);
+        case RT_S_MUL: return scalar_go<typename unsigned_twin<T>::type, RT_S_MUL>(ctx, va, value);
         case RT_S_LEAKY_RELU: return scalar_go<T, RT_S_LEAKY_RELU>(ctx, va, value);
         case RT_S_LEAKY_GRAD: return scalar_go<T, RT_S_LEAKY_GRAD>(ctx, va, value);
         case RT_S_DIV:

@@ -794,11 +794,19 @@ int32_t reduce_typed(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t
     return cols_launch<OP, T, 1>(ctx, src, out, outer, R, inner, R, true);
 }
 
+// Wrapping sums and products have the same bits for a signed integer and the unsigned one of its width: one instantiation serves both.
+template <class T> struct wrap_twin { typedef T type; };
+template <> struct wrap_twin<int8_t> { typedef uint8_t type; };
+template <> struct wrap_twin<int16_t> { typedef uint16_t type; };
+template <> struct wrap_twin<int32_t> { typedef uint32_t type; };
+template <> struct wrap_twin<int64_t> { typedef uint64_t type; };
+
 template <class T>
 int32_t reduce_ops(rt_ctx* ctx, int op, const void* src, void* out, uint64_t outer, uint64_t R, uint64_t inner) {
+    typedef typename wrap_twin<T>::type W;
     switch (op) {
-        case RT_R_SUM: return reduce_typed<RT_R_SUM, T>(ctx, (const T*)src, (T*)out, outer, R, inner);
-        case RT_R_PROD: return reduce_typed<RT_R_PROD, T>(ctx, (const T*)src, (T*)out, outer, R, inner);
+        case RT_R_SUM: return reduce_typed<RT_R_SUM, W>(ctx, (const W*)src, (W*)out, outer, R, inner);
+        case RT_R_PROD: return reduce_typed<RT_R_PROD, W>(ctx, (const W*)src, (W*)out, outer, R, inner);
         case RT_R_MAX: return reduce_typed<RT_R_MAX, T>(ctx, (const T*)src, (T*)out, outer, R, inner);
         case RT_R_MIN: return reduce_typed<RT_R_MIN, T>(ctx, (const T*)src, (T*)out, outer, R, inner);
         case RT_R_MEAN: return reduce_typed<RT_R_MEAN, T>(ctx, (const T*)src, (T*)out, outer, R, inner);
