@@ -401,23 +401,29 @@ def preheat(hip, fns, seconds):
         hip.sync()
 
 
-def time_kernel(hip, fn, iters, warmup, settle=0.0):
-    """Duration in ms (mean, median, min) of `fn`'s launch, HIP events on the backend's own stream.  `settle`: seconds of the same
-    launch, untimed, before the warm-up.  A kernel with another power profile than its predecessor (LDS traffic, more lanes)
-    starts at full speed, is held back for some tens of milliseconds while the board's power management finds its level, and then
-    recovers: the staged config-3b add 0.30 ms -> up to 0.42 ms -> 0.305 ms over its first hundred launches.  The steady level is
-    what a run of the same kernel sees."""
+def time_kernel(hip, fn, iters, warmup, settle=0.0, block=10):
+    """Average duration in ms of one launch of `fn`: (mean over all launches, median and min over blocks of `block` launches),
+    HIP events on the backend's own stream.  An event is recorded every `block` launches, not after every launch: an event
+    between two launches costs the stream about 5 us (the next kernel waits until the marker has been processed), which a
+    caller that just issues kernels never pays and which the rocprofv3 kernel trace of the same launches does not contain.
+    `settle`: seconds of the same launch, untimed, before the warm-up.  A kernel with another power profile than its
+    predecessor (LDS traffic, more lanes) starts at full speed, is held back for some tens of milliseconds while the board's
+    power management finds its level, and then recovers: the staged config-3b add 0.30 ms -> up to 0.42 ms -> 0.305 ms over its
+    first hundred launches.  The steady level is what a run of the same kernel sees."""
     if settle > 0:
         preheat(hip, [fn], settle)
     for _ in range(warmup):
         fn()
-    evs = [hip.event() for _ in range(iters + 1)]
+    block = max(1, min(block, iters))
+    nblocks = max(1, iters // block)
+    evs = [hip.event() for _ in range(nblocks + 1)]
     hip.record(evs[0])
-    for i in range(iters):
-        fn()
-        hip.record(evs[i + 1])
+    for b in range(nblocks):
+        for _ in range(block):
+            fn()
+        hip.record(evs[b + 1])
     hip.sync()
-    times = [hip.elapsed_ms(evs[i], evs[i + 1]) for i in range(iters)]
+    times = [hip.elapsed_ms(evs[b], evs[b + 1]) / block for b in range(nblocks)]
     return float(np.mean(times)), float(np.median(times)), float(np.min(times))
 
 
@@ -575,9 +581,24 @@ def main():
     for _ in range(args.warmup):
         add_fn(); sum_fn()
     K = args.steps
-    evs = [hip.event() for _ in range(2 * K + 1)]
+    # the timed region: K steps issued as a caller would issue them, one event before and one after, barrier on both sides
+    e0, e1 = hip.event(), hip.event()
     hip.sync()
     t0 = time.perf_counter()
+    hip.record(e0)
+    for i in range(K):
+        add_fn()
+        sum_fn()
+    hip.record(e1)
+    hip.sync()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / K
+    step_ms_events = hip.elapsed_ms(e0, e1) / K
+    step_bytes = add_bytes + sum_bytes
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    # the same K steps once more with an event after every kernel, to split the step between its two kernels.  Every event
+    # holds the stream up for about 5 us, so these figures are upper bounds of the kernels' durations inside the step.
+    evs = [hip.event() for _ in range(2 * K + 1)]
     hip.record(evs[0])
     for i in range(K):
         add_fn()
@@ -585,22 +606,20 @@ def main():
         sum_fn()
         hip.record(evs[2 * i + 2])
     hip.sync()
-    wall = time.perf_counter() - t0
     add_all = [hip.elapsed_ms(evs[2 * i], evs[2 * i + 1]) for i in range(K)]
     sum_all = [hip.elapsed_ms(evs[2 * i + 1], evs[2 * i + 2]) for i in range(K)]
-    add_ms, sum_ms = float(np.mean(add_all)), float(np.mean(sum_all))
-    add_med, sum_med = float(np.median(add_all)), float(np.median(sum_all))
-    ms_per_step = wall * 1e3 / K
-    step_bytes = add_bytes + sum_bytes
-    value = step_bytes / (ms_per_step * 1e-3) / 1e9
-    # the same add kernel launched back to back (what `rocprofv3 -- python3 bench.py --kernel c3a_add` sees)
-    sa_mean, sa_med, _ = time_kernel(hip, add_fn, 50, 10, settle=0.1)
+    in_step = {"add_ms": round(float(np.mean(add_all)), 4), "add_ms_median": round(float(np.median(add_all)), 4),
+               "sum_ms": round(float(np.mean(sum_all)), 4), "sum_ms_median": round(float(np.median(sum_all)), 4),
+               "note": "same K steps repeated with an event after every kernel; each event adds about 5 us to the launch before it"}
+    # each kernel on its own, launched back to back (what `rocprofv3 --kernel-trace -- python3 bench.py --kernel c3a_add` times)
+    add_ms, add_med, _ = time_kernel(hip, add_fn, 100, 10, settle=0.1)
+    sum_ms, sum_med, _ = time_kernel(hip, sum_fn, 100, 10, settle=0.1)
 
     detail = {}
     if not args.no_detail:
         for name in DETAIL:
             fn, nbytes, nelem = getattr(w, name)()
-            mean, med, mn = time_kernel(hip, fn, 50, 10, settle=0.0 if nbytes < (1 << 28) else 0.1)
+            mean, med, mn = time_kernel(hip, fn, 60, 10, settle=0.0 if nbytes < (1 << 28) else 0.1)
             detail[name] = {"ms": round(mean, 4), "ms_median": round(med, 4), "GBps": round(nbytes / (mean * 1e-3) / 1e9, 1),
                             "frac": round(nbytes / (mean * 1e-3) / PEAK_HBM, 4), "Gelem_s": round(nelem / (mean * 1e-3) / 1e9, 2)}
     w.drop()
@@ -618,14 +637,15 @@ def main():
                    "bytes_per_step": step_bytes, "pct_of_peak": round(100 * value * 1e9 / PEAK_HBM, 2)},
         # frac / achieved / kernel_ms: the add kernel inside the timed alternating add / sum loop (mean over the K steps, HIP events);
         # frac_median: the same by the median; standalone: the same kernel launched back to back, outside the loop
+        "step_ms_by_events": round(step_ms_events, 4),
         "roofline": {"bound": "hbm", "kernel": "bin_rows4_kernel<float, add, vec, vec> (config 3 broadcast add)",
                      "achieved": round(add_bytes / (add_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM / 1e9, "unit": "GB/s",
                      "frac": round(add_bytes / (add_ms * 1e-3) / PEAK_HBM, 4), "traffic": profiled_traffic(),
                      "traffic_source": "profiles/" + os.path.basename(TRAFFIC_PROFILE) + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measured by this run)",
+                     "measured": "average over 100 launches back to back, HIP events on the backend stream every 10 launches",
                      "kernel_ms": round(add_ms, 4), "kernel_ms_median": round(add_med, 4),
                      "frac_median": round(add_bytes / (add_med * 1e-3) / PEAK_HBM, 4),
-                     "standalone": {"kernel_ms": round(sa_mean, 4), "kernel_ms_median": round(sa_med, 4),
-                                    "frac": round(add_bytes / (sa_mean * 1e-3) / PEAK_HBM, 4)},
+                     "in_step": in_step,
                      "axis_sum": {"kernel": "reduce_rows_block_kernel<sum, float>", "achieved": round(sum_bytes / (sum_ms * 1e-3) / 1e9, 1),
                                   "frac": round(sum_bytes / (sum_ms * 1e-3) / PEAK_HBM, 4), "kernel_ms": round(sum_ms, 4),
                                   "kernel_ms_median": round(sum_med, 4)}},

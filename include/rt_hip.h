@@ -91,7 +91,9 @@ typedef enum rt_reduce_op {
 #define RT_MAX_INPUT_RANK 128 /* the reference's own cap on rank (core/primitives.rs:377-383) */
 
 /* ---- context ------------------------------------------------------------------------------------------------
- * Replaces the lazily built per-device singleton + default stream of backend/cuda.rs:38-51, 143-185. */
+ * Replaces the lazily built per-device singleton + default stream of backend/cuda.rs:38-51, 143-185.
+ * device >= 0 names the device; device == -1 takes the environment variable RT_HIP_DEVICE (a device index; 0 when it is unset).
+ * A malformed or out-of-range value is RT_E_INVALID. */
 int32_t rt_ctx_create(int32_t device, rt_ctx** out);
 int32_t rt_ctx_destroy(rt_ctx* ctx);
 int32_t rt_sync(rt_ctx* ctx);                       /* Cuda::sync, backend/cuda.rs:164-185 */

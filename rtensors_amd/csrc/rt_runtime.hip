@@ -64,6 +64,15 @@ extern "C" int32_t rt_ctx_create(int32_t device, rt_ctx** out) {
     *out = nullptr;
     int n = 0;
     RT_HIP(hipGetDeviceCount(&n));
+    if (device == -1) {
+        device = 0;
+        if (const char* e = getenv("RT_HIP_DEVICE")) {
+            char* end = nullptr;
+            const long v = strtol(e, &end, 10);
+            if (end == e || *end != '\0' || v < 0 || v > 1 << 20) return rt_fail(RT_E_INVALID, "rt_ctx_create: RT_HIP_DEVICE='%s' is not a device index", e);
+            device = (int32_t)v;
+        }
+    }
     if (device < 0 || device >= n) return rt_fail(RT_E_INVALID, "rt_ctx_create: device %d of %d", device, n);
     RT_HIP(hipSetDevice(device));
     rt_ctx* c = new rt_ctx();

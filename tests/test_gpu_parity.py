@@ -714,6 +714,24 @@ def test_bad_descriptors_are_refused_not_launched(hip):
     assert not hip.dump(g).any()
 
 
+def test_device_from_environment(hip, monkeypatch):
+    """device -1 asks rt_ctx_create to take the device index from RT_HIP_DEVICE (0 when unset)."""
+    from rtensors_amd import hip as H
+    monkeypatch.delenv("RT_HIP_DEVICE", raising=False)
+    H.Hip(-1).close()
+    monkeypatch.setenv("RT_HIP_DEVICE", "0")
+    h = H.Hip(-1)
+    b = h.alloc_from_slice(H.I32, np.arange(5, dtype=np.int32))
+    assert h.dump(b).tolist() == [0, 1, 2, 3, 4]
+    del b
+    h.close()
+    for bad in ("banana", "-2", "3x", "4096"):
+        monkeypatch.setenv("RT_HIP_DEVICE", bad)
+        with pytest.raises(H.TensorError) as e:
+            H.Hip(-1)
+        assert e.value.kind == "InvalidArgument", bad
+
+
 def test_overlapping_source_and_destination_are_refused(hip):
     """An output may be the very same view as an input (the in-place operators); any other overlap of the address ranges would
     let block order decide the result and is refused before a launch.  The trait's `&mut dst` / `&src` pairs
