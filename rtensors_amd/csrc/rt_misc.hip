@@ -11,16 +11,17 @@ constexpr int kBlock = 256;
 __global__ void set_flag_kernel(int32_t* flag, int32_t v) { *flag = v; }
 
 template <class T> struct alignas(16) Vec16 { T e[16 / sizeof(T)]; };
-constexpr int kVBlock = 128;    // vector kernels: one 16-byte vector (or one group of vectors) per lane
+constexpr int kVBlock = 256;    // vector kernels: one 16-byte vector (or one group of vectors) per lane, tiled traversal (see TileMap)
 
 // `==` per element: NaN != NaN, -0.0 == 0.0 (what Box<[T]> == Box<[T]> gives; the reference's device version is
 // K/kernels/utils/buffer_equal.cu:7-39).  All lanes that see a mismatch store the same value.  Both buffers are read
 // exactly once: one 16-byte vector per lane, non-temporal loads.
 template <class T>
-__global__ __launch_bounds__(kVBlock) void equal_vec_kernel(const Vec16<T>* __restrict__ a, const Vec16<T>* __restrict__ b, size_t nvec, int32_t* flag) {
+__global__ __launch_bounds__(kVBlock) void equal_vec_kernel(const Vec16<T>* __restrict__ a, const Vec16<T>* __restrict__ b, size_t nvec, int32_t* flag,
+                                                            TileMap m) {
     constexpr int N = 16 / sizeof(T);
-    const size_t i = (size_t)blockIdx.x * kVBlock + threadIdx.x;
-    if (i >= nvec) return;
+    size_t i;
+    if (!rt_tile_index(m, blockIdx.x, kVBlock, threadIdx.x, nvec, &i)) return;
     const Vec16<T> x = rt_ld16_nt(a + i), y = rt_ld16_nt(b + i);
     bool bad = false;
 #pragma unroll
@@ -42,10 +43,11 @@ int32_t equal_typed(rt_ctx* ctx, const void* a, const void* b, size_t n) {
     const bool aligned = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15) == 0;
     const size_t nvec = aligned ? n / N : 0;
     if (nvec) {
-        const size_t blocks = (nvec + kVBlock - 1) / kVBlock;
+        const TileMap m = rt_make_tilemap(a, nvec, kVBlock);
+        const size_t blocks = rt_tilemap_blocks(m, nvec, kVBlock);
         if (blocks > 0x7fffffffull) return rt_fail(RT_E_INVALID, "rt_equal: %zu elements is too long for one launch", n);
         hipLaunchKernelGGL((equal_vec_kernel<T>), dim3((unsigned)blocks), dim3(kVBlock), 0, ctx->stream, (const Vec16<T>*)a, (const Vec16<T>*)b, nvec,
-                           ctx->flag_dev);
+                           ctx->flag_dev, m);
     }
     const size_t rest = n - nvec * N;
     if (rest) {
@@ -158,12 +160,12 @@ template <class P> __device__ __forceinline__ void pack_st_nt(P* p, const P& v) 
 // (Giving each lane 16 bytes of the narrower type and several vectors of the wider one leaves every wide access
 // half-coalesced: f32 -> f64 measured 4.0 TB/s that way against 4.8 TB/s for one element per lane.)
 template <class S, class D>
-__global__ __launch_bounds__(kVBlock) void convert_vec_kernel(const S* __restrict__ s, D* __restrict__ d, size_t ngroups) {
+__global__ __launch_bounds__(kVBlock) void convert_vec_kernel(const S* __restrict__ s, D* __restrict__ d, size_t ngroups, TileMap m) {
     constexpr int E = 16 / (sizeof(S) > sizeof(D) ? sizeof(S) : sizeof(D));
     struct alignas(E * sizeof(S)) SP { S e[E]; };
     struct alignas(E * sizeof(D)) DP { D e[E]; };
-    const size_t i = (size_t)blockIdx.x * kVBlock + threadIdx.x;
-    if (i >= ngroups) return;
+    size_t i;
+    if (!rt_tile_index(m, blockIdx.x, kVBlock, threadIdx.x, ngroups, &i)) return;
     const SP in = pack_ld_nt(reinterpret_cast<const SP*>(s) + i);
     DP out;
 #pragma unroll
@@ -177,9 +179,11 @@ int32_t convert_go(rt_ctx* ctx, const void* s, void* d, size_t n) {
     const bool aligned = ((reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) & 15) == 0;
     const size_t ngroups = aligned ? n / E : 0;
     if (ngroups) {
-        const size_t blocks = (ngroups + kVBlock - 1) / kVBlock;
+        // the map walks the wider type's 16-byte vectors; the narrower side follows in proportionally smaller pieces
+        const TileMap m = rt_make_tilemap(sizeof(S) >= sizeof(D) ? s : (const void*)d, ngroups, kVBlock);
+        const size_t blocks = rt_tilemap_blocks(m, ngroups, kVBlock);
         if (blocks > 0x7fffffffull) return rt_fail(RT_E_INVALID, "convert: %zu elements is too long for one launch", n);
-        hipLaunchKernelGGL((convert_vec_kernel<S, D>), dim3((unsigned)blocks), dim3(kVBlock), 0, ctx->stream, (const S*)s, (D*)d, ngroups);
+        hipLaunchKernelGGL((convert_vec_kernel<S, D>), dim3((unsigned)blocks), dim3(kVBlock), 0, ctx->stream, (const S*)s, (D*)d, ngroups, m);
     }
     const size_t rest = n - ngroups * E;
     if (rest) {

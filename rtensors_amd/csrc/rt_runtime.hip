@@ -351,11 +351,13 @@ int32_t upload(rt_ctx* ctx, void* dev_dst, const void* host_src, size_t bytes) {
 // for hipMemcpyAsync(DeviceToDevice).  s and d point at the vector body, which starts on a 128-byte line of d; the source may be
 // in any phase (16-byte loads at byte alignment).  The `head` bytes before the body and the `tail` bytes after it go to lanes of
 // the first and the last block.
-__global__ __launch_bounds__(128) void rt_copy_vec_kernel(const uint8_t* __restrict__ s, uint8_t* __restrict__ d, size_t nvec, uint32_t head, uint32_t tail) {
-    const size_t i = (size_t)blockIdx.x * 128 + threadIdx.x;
+__global__ __launch_bounds__(256) void rt_copy_vec_kernel(const uint8_t* __restrict__ s, uint8_t* __restrict__ d, size_t nvec, uint32_t head, uint32_t tail,
+                                                          TileMap m) {
     if (blockIdx.x == 0 && threadIdx.x < head) { const int64_t e = (int64_t)threadIdx.x - (int64_t)head; d[e] = s[e]; }
     if (blockIdx.x == gridDim.x - 1 && threadIdx.x < tail) { const size_t e = nvec * 16 + threadIdx.x; d[e] = s[e]; }
-    if (i < nvec) __builtin_nontemporal_store(rt_ld16u<uint8_t, true>(s + i * 16), reinterpret_cast<rt_u32x4*>(d) + i);
+    size_t i;
+    if (!rt_tile_index(m, blockIdx.x, 256, threadIdx.x, nvec, &i)) return;          // a block owns a quarter of four pages (see TileMap)
+    __builtin_nontemporal_store(rt_ld16u<uint8_t, true>(s + i * 16), reinterpret_cast<rt_u32x4*>(d) + i);
 }
 
 static int32_t device_copy(rt_ctx* ctx, void* dst, const void* src, size_t bytes) {      // caller holds ctx->mu
@@ -364,14 +366,15 @@ static int32_t device_copy(rt_ctx* ctx, void* dst, const void* src, size_t bytes
     size_t head = (128 - (da & 127)) & 127;
     if (head > bytes) head = bytes;
     const size_t nvec = (bytes - head) / 16, tail = bytes - head - nvec * 16;
-    size_t blocks = (nvec + 127) / 128;
+    const TileMap m = rt_make_tilemap((const uint8_t*)dst + head, nvec, 256);
+    size_t blocks = rt_tilemap_blocks(m, nvec, 256);
     if (blocks < 1) blocks = 1;
     if (blocks > 0x7fffffffull) {
         RT_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx->stream));
         return RT_OK;
     }
-    hipLaunchKernelGGL(rt_copy_vec_kernel, dim3((unsigned)blocks), dim3(128), 0, ctx->stream, (const uint8_t*)src + head, (uint8_t*)dst + head, nvec,
-                       (uint32_t)head, (uint32_t)tail);
+    hipLaunchKernelGGL(rt_copy_vec_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (const uint8_t*)src + head, (uint8_t*)dst + head, nvec,
+                       (uint32_t)head, (uint32_t)tail, m);
     RT_HIP(hipGetLastError());
     return RT_OK;
 }
