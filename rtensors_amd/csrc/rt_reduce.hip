@@ -234,10 +234,9 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_lane_kernel(const T* __res
 // src viewed as (outer, R, inner).  VW = elements per lane along `inner` (16 bytes worth when rows are aligned, else 1).
 // blockIdx.x -> (o, seg, tile); lane tx covers columns (tile*64 + tx)*VW .., wave ty takes k = begin+ty, +kWaves, ...
 // out index: ((seg * outer) + o) * inner + column   (seg = 0, splits = 1 when this is the only stage)
-template <int OP, class T, int VW>
+template <int OP, class T, int VW, int U = 4>
 __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(const T* __restrict__ src, T* __restrict__ out, uint64_t R, uint64_t inner, uint64_t outer,
                                                              uint32_t tiles, uint32_t splits, uint64_t seglen, uint64_t count, int last) {
-    constexpr int U = 4;
     struct alignas(sizeof(T) * VW) VecW { T e[VW]; };
     uint64_t b = blockIdx.x;
     const uint32_t tile = (uint32_t)(b % tiles);
@@ -677,6 +676,7 @@ int32_t cols_launch(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t 
     const uint64_t tiles = (inner + per_tile - 1) / per_tile;
     // Two blocks of four waves per CU, each streaming a long run of rows, measured best on MI355X for every row pitch from
     // 1 KiB to 256 KiB (1 GiB f32 sum over axis 0: 6.4-6.8 TB/s, against 5.6-6.6 TB/s with eight blocks per CU).
+    // (Loads in flight per lane: 8 against 4 gained 0.5-1 % on the 1 GiB axis-0 sums; 3 or 4 blocks per CU were level or slower.)
     const uint64_t want = (uint64_t)ctx->num_cus * 2;
     uint32_t splits = 1;
     if (allow_split && outer * tiles < want) {
@@ -689,7 +689,7 @@ int32_t cols_launch(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t 
     }
     uint64_t seglen = (R + splits - 1) / splits;
     if (splits > 1) {
-        seglen = (seglen + 4 * kWaves - 1) / (4 * kWaves) * (4 * kWaves);
+        seglen = (seglen + 8 * kWaves - 1) / (8 * kWaves) * (8 * kWaves);
         splits = (uint32_t)((R + seglen - 1) / seglen);
     }
     const uint64_t blocks = outer * splits * tiles;
@@ -703,7 +703,7 @@ int32_t cols_launch(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t 
     void* scratch = nullptr;
     RT_TRY(rt_scratch(ctx, (size_t)(splits * outer * inner) * sizeof(T), &scratch));
     T* part = (T*)scratch;
-    hipLaunchKernelGGL((reduce_cols_kernel<OP, T, VW>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, part, R, inner, outer,
+    hipLaunchKernelGGL((reduce_cols_kernel<OP, T, VW, 8>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, part, R, inner, outer,
                        (uint32_t)tiles, splits, seglen, count, 0);
     RT_HIP(hipGetLastError());
     // second stage: partials are (splits, outer*inner): a column reduce with R = splits
