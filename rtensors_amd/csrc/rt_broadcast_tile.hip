@@ -265,7 +265,8 @@ struct StageArgs {
 };
 
 // grid: x = inner-dim tile + ltiles * (tile along t), y = index along the inner outer dim, z = index along the outer one
-template <class T, int OP, int OM, bool WIDE>
+// FULL: K and L are whole numbers of tiles, so no index is clamped and no row or vector is tested against an edge.
+template <class T, int OP, int OM, bool WIDE, bool FULL>
 __global__ __launch_bounds__((StageGeom<T, WIDE>::kBlock)) void bin_stage_kernel(const T* xt, const T* xo, T* d, StageArgs a, int32_t* fault) {
     constexpr int N = 16 / sizeof(T);
     constexpr int kSRows = StageGeom<T, WIDE>::kRows, kSWaves = StageGeom<T, WIDE>::kWaves, kSBlock = StageGeom<T, WIDE>::kBlock;
@@ -289,14 +290,14 @@ __global__ __launch_bounds__((StageGeom<T, WIDE>::kBlock)) void bin_stage_kernel
     const uint32_t lane = threadIdx.x & (RT_WAVE - 1);
     const uint32_t wv = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x / RT_WAVE));
     const uint32_t c = l0 + lane * N;
-    const bool full_vec = c + N <= L;
+    const bool full_vec = FULL || c + N <= L;
     // rows of the other input, issued before the gather so that both are in flight together
     Vec16<T> ov[RPL] = {};
     if constexpr (OP != kOpCopy) {
         if (full_vec) {
 #pragma unroll
             for (int i = 0; i < RPL; ++i) {
-                const uint32_t k = min(k0 + wv * RPL + i, K - 1);
+                const uint32_t k = FULL ? k0 + wv * RPL + i : min(k0 + wv * RPL + i, K - 1);
                 ov[i] = load_vec<T, OM>(xo + (int32_t)k * ts1, c, is1);
             }
         }
@@ -311,13 +312,13 @@ __global__ __launch_bounds__((StageGeom<T, WIDE>::kBlock)) void bin_stage_kernel
             const uint32_t v = u0 + threadIdx.x;
             if (NU % kSBlock == 0 || v < (uint32_t)NU) {
                 const uint32_t lq = v / KQ, tq = v % KQ;
-                const uint32_t t0 = min(k0 + tq * N, K - N);        // K % N == 0 here; rows past the end of dim t are never stored
+                const uint32_t t0 = FULL ? k0 + tq * N : min(k0 + tq * N, K - N);   // K % N == 0 here; rows past the end of dim t are never stored
                 // lowest address of a vector: element t0 when dim t ascends in memory, element t0 + N - 1 when it descends
                 const T* src = xt + (fwd ? (int64_t)t0 : -(int64_t)(t0 + N - 1));
                 Vec16<T> g[N];
 #pragma unroll
                 for (int j = 0; j < N; ++j) {
-                    const uint32_t col = min(l0 + lq * N + j, L - 1);
+                    const uint32_t col = FULL ? l0 + lq * N + j : min(l0 + lq * N + j, L - 1);
                     const Vec16<T>* gp = reinterpret_cast<const Vec16<T>*>(src + (int32_t)col * is0);
                     if constexpr (NTG) g[j] = rt_ld16_nt(gp); else g[j] = rt_ld16(gp);
                 }
@@ -333,11 +334,11 @@ __global__ __launch_bounds__((StageGeom<T, WIDE>::kBlock)) void bin_stage_kernel
     };
     if (nt_xt) gather(std::true_type{}); else gather(std::false_type{});
     __syncthreads();
-    if (c >= L) return;
+    if (!FULL && c >= L) return;
 #pragma unroll
     for (int i = 0; i < RPL; ++i) {
         const uint32_t kk = wv * RPL + i;
-        if (k0 + kk >= K) continue;
+        if (!FULL && k0 + kk >= K) continue;
         T* drow = dp + (int32_t)(k0 + kk) * ts2;
         if (full_vec) {
             const Vec16<T> xv = *reinterpret_cast<const Vec16<T>*>(&tile[kk][lane * N]);
@@ -438,18 +439,20 @@ bool tile_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* l, const 
                 const T* op = (xt == 0 ? r : l) + dsc.offset[o];
                 T* dp = d + dsc.offset[2];
                 dim3 grid((unsigned)gx, (unsigned)n0, (unsigned)n1), blk(kSBlock);
-                auto go = [&](auto wide_c) {
-                    constexpr bool W = decltype(wide_c)::value;
+                const bool full = a.K % kSRows == 0 && a.L % (kSVecs * (uint32_t)N) == 0;
+                auto go = [&](auto wide_c, auto full_c) {
+                    constexpr bool W = decltype(wide_c)::value, F = decltype(full_c)::value;
                     if constexpr (OP == kOpCopy) {
-                        hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_BCAST, W>), grid, blk, 0, ctx->stream, xp, op, dp, a, fault_of<T, OP>(ctx));
+                        hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_BCAST, W, F>), grid, blk, 0, ctx->stream, xp, op, dp, a, fault_of<T, OP>(ctx));
                     } else {
-                        if (om == M_VEC) hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_VEC, W>), grid, blk, 0, ctx->stream, xp, op, dp, a, fault_of<T, OP>(ctx));
-                        else if (om == M_BCAST) hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_BCAST, W>), grid, blk, 0, ctx->stream, xp, op, dp, a, fault_of<T, OP>(ctx));
-                        else hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_ELEM, W>), grid, blk, 0, ctx->stream, xp, op, dp, a, fault_of<T, OP>(ctx));
+                        if (om == M_VEC) hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_VEC, W, F>), grid, blk, 0, ctx->stream, xp, op, dp, a, fault_of<T, OP>(ctx));
+                        else if (om == M_BCAST) hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_BCAST, W, F>), grid, blk, 0, ctx->stream, xp, op, dp, a, fault_of<T, OP>(ctx));
+                        else hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_ELEM, W, F>), grid, blk, 0, ctx->stream, xp, op, dp, a, fault_of<T, OP>(ctx));
                     }
                 };
-                if constexpr (sizeof(T) == 4) { if (wide) go(std::true_type{}); else go(std::false_type{}); }
-                else go(std::false_type{});
+                auto go_w = [&](auto wide_c) { if (full) go(wide_c, std::true_type{}); else go(wide_c, std::false_type{}); };
+                if constexpr (sizeof(T) == 4) { if (wide) go_w(std::true_type{}); else go_w(std::false_type{}); }
+                else go_w(std::false_type{});
                 hipError_t e = hipGetLastError();
                 *status = e == hipSuccess ? RT_OK : rt_hip_fail(e, "broadcast (staged tile kernel) launch");
                 return true;
