@@ -239,7 +239,8 @@ int32_t rt_scalar_to(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, ui
  *   rt_fused_bias_relu          y[i, j] = relu(x[i, j] + bias[j])
  *   rt_fused_l1_forward         gmap[k] = sign(y[k] - target[k]) / N,  loss[0] = (sum_k |y[k] - target[k]|) / N,  N = (T)(f32)n
  *   rt_fused_l1_relu_backward   dbias[j] = sum_i (y[i, j] > 0 ? 1 : 0) * (gmap[i, j] * upstream[0])   (upstream: one device element,
- *                               the loss-seeded root of grad/mod.rs:442-447 or a one) */
+ *                               the loss-seeded root of grad/mod.rs:442-447 or a one)
+ * y may be x itself and gmap may be y or target itself (in place); an output that overlaps an input in any other way is RT_E_INVALID. */
 int32_t rt_fused_bias_relu(rt_ctx* ctx, int32_t dtype, const void* x, uint64_t x_len, const void* bias, uint64_t bias_len,
                            void* y, uint64_t y_len, uint64_t rows, uint64_t cols);
 int32_t rt_fused_l1_forward(rt_ctx* ctx, int32_t dtype, const void* y, uint64_t y_len, const void* target, uint64_t target_len,

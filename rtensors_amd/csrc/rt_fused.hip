@@ -140,6 +140,12 @@ int32_t check_float(const char* what, int dtype) {
     return RT_OK;
 }
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+// An output may be the very same run as an input of its own length (every lane reads its vector before it writes it); any other
+// overlap would let block order decide the result.
+bool bad_overlap(const void* out, uint64_t out_n, const void* in, uint64_t in_n, int es) {
+    if (out == in && out_n == in_n) return false;
+    return rt_spans_meet(rt_run_span(out, es, 0, out_n), rt_run_span(in, es, 0, in_n));
+}
 
 template <class T>
 int32_t bias_relu_typed(rt_ctx* ctx, const void* x, const void* bias, void* y, uint64_t rows, uint64_t cols) {
@@ -218,6 +224,11 @@ extern "C" int32_t rt_fused_bias_relu(rt_ctx* ctx, int32_t dtype, const void* x,
     if (!x || !bias || !y) return rt_fail(RT_E_INVALID, "fused bias relu: null buffer");
     if (cols % N || !aligned16(x) || !aligned16(bias) || !aligned16(y))
         return rt_fail(RT_E_INVALID, "fused bias relu: needs 16-byte aligned operands and whole vectors per row (issue the separate ops instead)");
+    {
+        const int es = rt_elem_size(dtype);
+        if (bad_overlap(y, rows * cols, x, rows * cols, es) || rt_spans_meet(rt_run_span(y, es, 0, rows * cols), rt_run_span(bias, es, 0, cols)))
+            return rt_fail(RT_E_INVALID, "fused bias relu: the output overlaps an input");
+    }
     CtxGuard g(ctx);
     return dtype == RT_F32 ? bias_relu_typed<float>(ctx, x, bias, y, rows, cols) : bias_relu_typed<double>(ctx, x, bias, y, rows, cols);
 }
@@ -232,6 +243,13 @@ extern "C" int32_t rt_fused_l1_forward(rt_ctx* ctx, int32_t dtype, const void* y
     if (!y || !target || !gmap || !loss) return rt_fail(RT_E_INVALID, "fused l1 forward: null buffer");
     if (n % N || !aligned16(y) || !aligned16(target) || !aligned16(gmap))
         return rt_fail(RT_E_INVALID, "fused l1 forward: needs 16-byte aligned operands and a whole number of vectors (issue the separate ops instead)");
+    {
+        const int es = rt_elem_size(dtype);
+        const ByteSpan ls = rt_run_span(loss, es, 0, 1);
+        if (bad_overlap(gmap, n, y, n, es) || bad_overlap(gmap, n, target, n, es) || rt_spans_meet(ls, rt_run_span(y, es, 0, n)) ||
+            rt_spans_meet(ls, rt_run_span(target, es, 0, n)) || rt_spans_meet(ls, rt_run_span(gmap, es, 0, n)))
+            return rt_fail(RT_E_INVALID, "fused l1 forward: an output overlaps an input or the other output");
+    }
     CtxGuard g(ctx);
     return dtype == RT_F32 ? l1_forward_typed<float>(ctx, dtype, y, target, gmap, loss, n) : l1_forward_typed<double>(ctx, dtype, y, target, gmap, loss, n);
 }
@@ -247,6 +265,13 @@ extern "C" int32_t rt_fused_l1_relu_backward(rt_ctx* ctx, int32_t dtype, const v
     if (!gmap || !y || !upstream || !dbias) return rt_fail(RT_E_INVALID, "fused backward: null buffer");
     if (cols % N || !aligned16(gmap) || !aligned16(y) || !aligned16(dbias))
         return rt_fail(RT_E_INVALID, "fused backward: needs 16-byte aligned operands and whole vectors per row (issue the separate ops instead)");
+    {
+        const int es = rt_elem_size(dtype);
+        const ByteSpan ds = rt_run_span(dbias, es, 0, cols);
+        if (rt_spans_meet(ds, rt_run_span(gmap, es, 0, rows * cols)) || rt_spans_meet(ds, rt_run_span(y, es, 0, rows * cols)) ||
+            rt_spans_meet(ds, rt_run_span(upstream, es, 0, 1)))
+            return rt_fail(RT_E_INVALID, "fused backward: the output overlaps an input");
+    }
     CtxGuard g(ctx);
     return dtype == RT_F32 ? backward_typed<float>(ctx, dtype, gmap, y, upstream, dbias, rows, cols)
                            : backward_typed<double>(ctx, dtype, gmap, y, upstream, dbias, rows, cols);

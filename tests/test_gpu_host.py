@@ -326,6 +326,20 @@ def test_fused_passes_refuse_what_they_do_not_take(be):
     with pytest.raises(H.TensorError) as e:
         hip.fused_bias_relu(i, i, i, 2, 8)
     assert e.value.kind == "UnsupportedOperation"
+    # outputs that overlap an input: in place on the very same run is fine, anything else is refused
+    x = hip.alloc_from_slice(H.F32, np.arange(-16, 16, dtype=np.float32))
+    bias = hip.alloc_from_slice(H.F32, np.ones(8, np.float32))
+    hip.fused_bias_relu(x, bias, x, 4, 8)
+    assert np.array_equal(hip.dump(x), np.maximum(np.arange(-16, 16, dtype=np.float32) + 1, 0))
+    shifted = H.HipBuf(None, x.ptr + 16, 24, H.F32)                        # a window into x, not owned
+    with pytest.raises(H.TensorError) as e:
+        hip.fused_bias_relu(x, bias, shifted, 2, 8)
+    assert e.value.status == 1 and "overlaps" in str(e.value)
+    loss = hip.alloc(H.F32, 1)
+    with pytest.raises(H.TensorError):
+        hip.fused_l1_forward(x, c, shifted, loss, 24)
+    with pytest.raises(H.TensorError):
+        hip.fused_l1_relu_backward(x, x, loss, H.HipBuf(None, x.ptr, 8, H.F32), 4, 8)
     hip.close()
 
 
