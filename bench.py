@@ -382,11 +382,20 @@ class Workloads:
         self.hip.fused_l1_forward(y, t, g, loss, n * d)
         return (lambda: self.hip.fused_l1_relu_backward(g, y, loss, db, n, d)), (2 * n * d + d) * 4 + 4, n * d
 
+    def c5_fused2_forward(self):
+        n, d, x, t, bias, y, g, loss, db = self._c5_fused_bufs()
+        return (lambda: self.hip.fused_bias_relu_l1(x, bias, t, y, loss, n, d)), (3 * n * d + d) * 4 + 4, n * d
+
+    def c5_fused2_backward(self):
+        n, d, x, t, bias, y, g, loss, db = self._c5_fused_bufs()
+        self.hip.fused_bias_relu_l1(x, bias, t, y, loss, n, d)
+        return (lambda: self.hip.fused_l1_relu_backward_t(y, t, loss, db, n, d)), (2 * n * d + d) * 4 + 4, n * d
+
 
 HEADLINE = ["c3a_add", "c4_sum1"]
 DETAIL = ["copy", "fill", "c1_add", "c1_sum1", "c2_mul", "c2_add", "c2_relu", "c2_sub", "c2_f64_mul", "c2_f64_add", "c2_i32_mul", "c2_i32_add",
           "c3a_add", "c3b_add", "c4_sum1", "c4_mean1", "c4_max1", "c4_sum0", "c4_sum_all", "c4_i32_sum1", "c4_i32_max1", "c4_i32_min0",
-          "c4_var1", "c4_std0", "c4_lse1", "c4_argmax1", "c5_bias_add", "c5_colsum", "c5_fused_bias_relu", "c5_fused_l1_forward", "c5_fused_backward",
+          "c4_var1", "c4_std0", "c4_lse1", "c4_argmax1", "c5_bias_add", "c5_colsum", "c5_fused_bias_relu", "c5_fused_l1_forward", "c5_fused_backward", "c5_fused2_forward", "c5_fused2_backward",
           "view_relu", "tr_add", "tr_copy"]
 KIND = {"copy": "elementwise", "fill": "elementwise"}
 
@@ -494,8 +503,11 @@ def host_layer_runs(iters=10):
     x = T.Tensor.from_buf(be, "f32", rng.standard_normal(rows * cols, dtype=np.float32), [rows, cols])
     target = T.Tensor.from_buf(be, "f32", rng.random(rows * cols, dtype=np.float32) * 2 - 1, [rows, cols])
     bias = T.Tensor.from_buf(be, "f32", rng.standard_normal(cols, dtype=np.float32) * 0.1, [cols])
-    # the step in three fused passes (rt_fused_*: 7 x 1 GiB of traffic) and on the tape, one backend call per arithmetic step (about 22 x)
-    for name, fn in (("c5_train_step_ms", lambda: T.train_step_fused(x, bias, target, 0.01)), ("c5_train_step_tape_ms", lambda: T.train_step(x, bias, target, 0.01))):
+    # the step in two fused passes (rt_fused_bias_relu_l1 + rt_fused_l1_relu_backward_t: 5 x 1 GiB of traffic), in three (the gradient map
+    # stored: 7 x) and on the tape, one backend call per arithmetic step (about 22 x)
+    for name, fn in (("c5_train_step_ms", lambda: T.train_step_fused(x, bias, target, 0.01)),
+                     ("c5_train_step_3pass_ms", lambda: T.train_step_fused(x, bias, target, 0.01, True, 3)),
+                     ("c5_train_step_tape_ms", lambda: T.train_step(x, bias, target, 0.01))):
         for _ in range(2):
             fn()
         be.sync()
@@ -504,7 +516,7 @@ def host_layer_runs(iters=10):
             fn()
         be.sync()
         out[name] = round((time.perf_counter() - t0) / iters * 1e3, 4)
-    out["c5_train_step_bytes"] = 7 * rows * cols * 4
+    out["c5_train_step_bytes"] = 5 * rows * cols * 4
     out["c5_train_step_GBps"] = round(out["c5_train_step_bytes"] / (out["c5_train_step_ms"] * 1e-3) / 1e9, 1)
     return out
 

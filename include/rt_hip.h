@@ -247,6 +247,16 @@ int32_t rt_fused_l1_forward(rt_ctx* ctx, int32_t dtype, const void* y, uint64_t 
                             void* gmap, uint64_t gmap_len, void* loss, uint64_t loss_len, uint64_t n);
 int32_t rt_fused_l1_relu_backward(rt_ctx* ctx, int32_t dtype, const void* gmap, uint64_t gmap_len, const void* y, uint64_t y_len,
                                   const void* upstream, uint64_t upstream_len, void* dbias, uint64_t dbias_len, uint64_t rows, uint64_t cols);
+/* The same step without the gradient map, which is a temporary of the tape and not a result (5 instead of 7 passes over a tensor):
+ *   rt_fused_bias_relu_l1         y[i, j] = relu(x[i, j] + bias[j]),  loss[0] = (sum |y - target|) / N      (reads x, target; writes y)
+ *   rt_fused_l1_relu_backward_t   dbias[j] = sum_i (y[i, j] > 0 ? 1 : 0) * ((sign(y[i, j] - target[i, j]) / N) * upstream[0])
+ * with N = (T)(f32)(rows * cols).  Per element these are the operations of the three-pass form in the same order, so y and every
+ * summand are bit for bit the same; same operand requirements; y may be x itself. */
+int32_t rt_fused_bias_relu_l1(rt_ctx* ctx, int32_t dtype, const void* x, uint64_t x_len, const void* bias, uint64_t bias_len,
+                              const void* target, uint64_t target_len, void* y, uint64_t y_len, void* loss, uint64_t loss_len,
+                              uint64_t rows, uint64_t cols);
+int32_t rt_fused_l1_relu_backward_t(rt_ctx* ctx, int32_t dtype, const void* y, uint64_t y_len, const void* target, uint64_t target_len,
+                                    const void* upstream, uint64_t upstream_len, void* dbias, uint64_t dbias_len, uint64_t rows, uint64_t cols);
 
 /* ---- matmul ------------------------------------------------------------------------------------------------------
  * BackendMatMul::matmul (backend/mod.rs:474-485; Cpu backend/cpu.rs:725-951), argument list of protocol Op::Matmul

@@ -573,6 +573,25 @@ impl Hip {
         })
     }
 
+    /// `y = relu(x + bias)` and `loss[0] = mean |y - target|` in one pass; with `fused_l1_relu_backward_t` the whole step
+    /// without a stored gradient map.
+    pub fn fused_bias_relu_l1<T: WeightValue>(&self, x: &HipBuf<T>, bias: &HipBuf<T>, target: &HipBuf<T>, y: &mut HipBuf<T>,
+        loss: &mut HipBuf<T>, rows: usize, cols: usize) -> Result<(), TensorError> {
+        check(unsafe {
+            ffi::rt_fused_bias_relu_l1(self.raw(), dt::<T>(), x.ptr, x.len as u64, bias.ptr, bias.len as u64, target.ptr,
+                target.len as u64, y.ptr, y.len as u64, loss.ptr, loss.len as u64, rows as u64, cols as u64)
+        })
+    }
+
+    /// `dbias[c] = sum over r of (y[r, c] > 0) * ((sign(y[r, c] - target[r, c]) / (rows * cols)) * upstream[0])`.
+    pub fn fused_l1_relu_backward_t<T: WeightValue>(&self, y: &HipBuf<T>, target: &HipBuf<T>, upstream: &HipBuf<T>,
+        dbias: &mut HipBuf<T>, rows: usize, cols: usize) -> Result<(), TensorError> {
+        check(unsafe {
+            ffi::rt_fused_l1_relu_backward_t(self.raw(), dt::<T>(), y.ptr, y.len as u64, target.ptr, target.len as u64,
+                upstream.ptr, upstream.len as u64, dbias.ptr, dbias.len as u64, rows as u64, cols as u64)
+        })
+    }
+
     /// One pass for a value-returning unary op on a contiguous operand (`alloc` + this, instead of `owned()` + the
     /// in-place op, which is two passes: ops/unary/mod.rs:114-126).
     pub fn unary_to<T: TensorValue>(&self, op: i32, src: &HipBuf<T>, start: usize, len: usize, dst: &mut HipBuf<T>)

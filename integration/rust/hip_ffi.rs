@@ -154,6 +154,12 @@ extern "C" {
     pub fn rt_fused_l1_relu_backward(ctx: *mut rt_ctx, dtype: i32, gmap: *const c_void, gmap_len: u64, y: *const c_void,
                                      y_len: u64, upstream: *const c_void, upstream_len: u64, dbias: *mut c_void,
                                      dbias_len: u64, rows: u64, cols: u64) -> i32;
+    pub fn rt_fused_bias_relu_l1(ctx: *mut rt_ctx, dtype: i32, x: *const c_void, x_len: u64, bias: *const c_void, bias_len: u64,
+                                 target: *const c_void, target_len: u64, y: *mut c_void, y_len: u64, loss: *mut c_void, loss_len: u64,
+                                 rows: u64, cols: u64) -> i32;
+    pub fn rt_fused_l1_relu_backward_t(ctx: *mut rt_ctx, dtype: i32, y: *const c_void, y_len: u64, target: *const c_void,
+                                       target_len: u64, upstream: *const c_void, upstream_len: u64, dbias: *mut c_void,
+                                       dbias_len: u64, rows: u64, cols: u64) -> i32;
     pub fn rt_matmul(ctx: *mut rt_ctx, dtype: i32, lhs: *const c_void, lhs_len: u64, lhs_offset: u64, lhs_rank: i32,
                      lhs_shape: *const u64, lhs_strides: *const i64, lhs_contiguity: i32, rhs: *const c_void, rhs_len: u64,
                      rhs_offset: u64, rhs_rank: i32, rhs_shape: *const u64, rhs_strides: *const i64, rhs_contiguity: i32,

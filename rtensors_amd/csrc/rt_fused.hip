@@ -5,6 +5,9 @@
 //   rt_fused_bias_relu          y = relu(x + bias)                                           reads x, writes y            (2 N s)
 //   rt_fused_l1_forward         gmap = sign(y - t) / N,  loss = sum |y - t| / N              reads y, t, writes gmap      (3 N s)
 //   rt_fused_l1_relu_backward   dbias[j] = sum_i [y_ij > 0] * (gmap_ij * up)                 reads gmap, y                (2 N s)
+// and, without ever storing the gradient map (it is a temporary of the tape, not a result), in two:
+//   rt_fused_bias_relu_l1       y = relu(x + bias),  loss = sum |y - t| / N                  reads x, t, writes y         (3 N s)
+//   rt_fused_l1_relu_backward_t dbias[j] = sum_i [y_ij > 0] * ((sign(y_ij - t_ij) / N) * up) reads y, t                   (2 N s)
 // Every element-wise result (y, gmap, and the products that are summed) is bit for bit what the separate ops give; the two sums are
 // tree sums, held to the same tolerance as the reductions (1e-5 / 1e-12 of sum |x|).  f32 and f64 (the autograd engine is bounded on
 // WeightValue, core/value.rs:61).  The ReLU gradient map is not stored: [pre > 0] == [relu(pre) > 0].
@@ -73,13 +76,50 @@ __global__ __launch_bounds__(kFBlock) void fused_l1_forward_kernel(const T* __re
 
 template <class T> __global__ void fused_divide_kernel(T* p, T count) { *p = *p / count; }
 
+// ---- y = relu(x + bias) and the partial sums of |y - t| in one pass ----------------------------------------------------------------------
+template <class T>
+__global__ __launch_bounds__(kFBlock) void fused_bias_relu_l1_kernel(const T* __restrict__ x, const T* __restrict__ bias, const T* __restrict__ t,
+                                                                     T* __restrict__ y, T* __restrict__ part, uint32_t nvec, uint32_t row_vecs,
+                                                                     FastDiv32 row_div, TileMap m) {
+    constexpr int N = 16 / sizeof(T);
+    __shared__ T sv[kFWaves];
+    size_t vi;
+    T acc = (T)0;
+    if (rt_tile_index(m, blockIdx.x, kFBlock, threadIdx.x, nvec, &vi)) {
+        const uint32_t v = (uint32_t)vi;
+        Vec16<T> a = rt_ld16_nt(reinterpret_cast<const Vec16<T>*>(x) + v);
+        const Vec16<T> tt = rt_ld16_nt(reinterpret_cast<const Vec16<T>*>(t) + v);
+        const uint32_t c = v - fd_div(v, row_div) * row_vecs;
+        const Vec16<T> b = rt_ld16(reinterpret_cast<const Vec16<T>*>(bias) + c);
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            a.e[j] = relu_of<T>(a.e[j] + b.e[j]);
+            acc = acc + abs_of(a.e[j] - tt.e[j]);
+        }
+        rt_st16_nt(reinterpret_cast<Vec16<T>*>(y) + v, a);
+    }
+#pragma unroll
+    for (int d = RT_WAVE / 2; d >= 1; d >>= 1) acc = acc + __shfl_down(acc, d, RT_WAVE);
+    const int lane = threadIdx.x & (RT_WAVE - 1), w = threadIdx.x / RT_WAVE;
+    if (lane == 0) sv[w] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        T s = sv[0];
+#pragma unroll
+        for (int k = 1; k < kFWaves; ++k) s = s + sv[k];
+        part[blockIdx.x] = s;
+    }
+}
+
 // ---- dbias[j] = sum_i [y_ij > 0] * (gmap_ij * up) ------------------------------------------------------------------------------------
 // The shape of the column reduction: lanes along the columns (one 16-byte vector each), the four waves of a block take interleaved
 // rows, four rows in flight per wave, LDS combine; the rows are split over `splits` blocks per column tile and a second launch (the
 // ordinary column sum) folds the partials.  out index: seg * cols + column.
-template <class T>
+// FROM_TARGET: `gmap` holds the target instead, and the gradient map's element sign(y - t) / count is formed in registers.
+template <class T, bool FROM_TARGET>
 __global__ __launch_bounds__(kFBlock) void fused_backward_cols_kernel(const T* __restrict__ gmap, const T* __restrict__ y, const T* __restrict__ up,
-                                                                      T* __restrict__ out, uint64_t rows, uint64_t cols, uint32_t tiles, uint64_t seglen) {
+                                                                      T* __restrict__ out, uint64_t rows, uint64_t cols, uint32_t tiles, uint64_t seglen,
+                                                                      T count) {
     constexpr int N = 16 / sizeof(T);
     constexpr int U = 4;
     const uint32_t tile = blockIdx.x % tiles, seg = blockIdx.x / tiles;
@@ -96,7 +136,9 @@ __global__ __launch_bounds__(kFBlock) void fused_backward_cols_kernel(const T* _
     auto fold = [&](const Vec16<T>& g, const Vec16<T>& a) {
 #pragma unroll
         for (int j = 0; j < N; ++j) {
-            const T g1 = g.e[j] * u;                               // backwards_l1: grad_map * upstream
+            T gm = g.e[j];
+            if constexpr (FROM_TARGET) gm = sign_of<T>(a.e[j] - g.e[j]) / count;   // l1.rs:29-36, 58-60: sign(lhs - target) / N
+            const T g1 = gm * u;                                   // backwards_l1: grad_map * upstream
             const T g2 = (a.e[j] > (T)0 ? (T)1 : (T)0) * g1;       // backwards_relu: relu map * upstream
             acc[j] = acc[j] + g2;
         }
@@ -182,7 +224,31 @@ int32_t l1_forward_typed(rt_ctx* ctx, int dtype, const void* y, const void* t, v
 }
 
 template <class T>
-int32_t backward_typed(rt_ctx* ctx, int dtype, const void* gmap, const void* y, const void* up, void* dbias, uint64_t rows, uint64_t cols) {
+int32_t bias_relu_l1_typed(rt_ctx* ctx, int dtype, const void* x, const void* bias, const void* t, void* y, void* loss, uint64_t rows, uint64_t cols) {
+    constexpr uint64_t N = 16 / sizeof(T);
+    const uint64_t n = rows * cols;
+    const uint32_t nvec = (uint32_t)(n / N), row_vecs = (uint32_t)(cols / N);
+    const TileMap m = rt_make_tilemap(y, nvec, kFBlock);
+    const size_t blocks = rt_tilemap_blocks(m, nvec, kFBlock);
+    void* part = nullptr;
+    RT_TRY(rt_alloc_bytes(ctx, blocks * sizeof(T), &part));
+    const T count = (T)(float)n;
+    hipLaunchKernelGGL((fused_bias_relu_l1_kernel<T>), dim3((unsigned)blocks), dim3(kFBlock), 0, ctx->stream, (const T*)x, (const T*)bias, (const T*)t, (T*)y,
+                       (T*)part, nvec, row_vecs, make_fastdiv(row_vecs), m);
+    hipError_t e = hipGetLastError();
+    int32_t st = e == hipSuccess ? RT_OK : rt_hip_fail(e, "fused bias relu l1 launch");
+    if (st == RT_OK) st = rt_reduce_rows(ctx, dtype, RT_R_SUM, part, loss, 1, blocks);
+    if (st == RT_OK) {
+        hipLaunchKernelGGL((fused_divide_kernel<T>), dim3(1), dim3(1), 0, ctx->stream, (T*)loss, count);
+        e = hipGetLastError();
+        if (e != hipSuccess) st = rt_hip_fail(e, "fused bias relu l1 launch");
+    }
+    (void)rt_free_locked(ctx, part);
+    return st;
+}
+
+template <class T>
+int32_t backward_typed(rt_ctx* ctx, int dtype, const void* gmap, const void* y, const void* up, void* dbias, uint64_t rows, uint64_t cols, bool from_target) {
     constexpr uint64_t N = 16 / sizeof(T);
     const uint64_t tiles = (cols / N + RT_WAVE - 1) / RT_WAVE;
     const uint64_t want = (uint64_t)ctx->num_cus * 2;              // two resident blocks per CU, as the column reduction
@@ -199,8 +265,13 @@ int32_t backward_typed(rt_ctx* ctx, int dtype, const void* gmap, const void* y, 
     if (tiles * splits >= (1ull << 31)) return rt_fail(RT_E_INVALID, "fused backward: too many blocks for one launch");
     void* part = dbias;
     if (splits > 1) RT_TRY(rt_alloc_bytes(ctx, (size_t)(splits * cols) * sizeof(T), &part));
-    hipLaunchKernelGGL((fused_backward_cols_kernel<T>), dim3((unsigned)(tiles * splits)), dim3(kFBlock), 0, ctx->stream, (const T*)gmap, (const T*)y, (const T*)up,
-                       (T*)part, rows, cols, (uint32_t)tiles, seglen);
+    const T count = (T)(float)(rows * cols);                       // WeightValue::from_usize goes through f32 (core/value.rs:54-56)
+    if (from_target)
+        hipLaunchKernelGGL((fused_backward_cols_kernel<T, true>), dim3((unsigned)(tiles * splits)), dim3(kFBlock), 0, ctx->stream, (const T*)gmap, (const T*)y,
+                           (const T*)up, (T*)part, rows, cols, (uint32_t)tiles, seglen, count);
+    else
+        hipLaunchKernelGGL((fused_backward_cols_kernel<T, false>), dim3((unsigned)(tiles * splits)), dim3(kFBlock), 0, ctx->stream, (const T*)gmap, (const T*)y,
+                           (const T*)up, (T*)part, rows, cols, (uint32_t)tiles, seglen, count);
     hipError_t e = hipGetLastError();
     int32_t st = e == hipSuccess ? RT_OK : rt_hip_fail(e, "fused backward launch");
     if (splits > 1) {
@@ -273,6 +344,55 @@ extern "C" int32_t rt_fused_l1_relu_backward(rt_ctx* ctx, int32_t dtype, const v
             return rt_fail(RT_E_INVALID, "fused backward: the output overlaps an input");
     }
     CtxGuard g(ctx);
-    return dtype == RT_F32 ? backward_typed<float>(ctx, dtype, gmap, y, upstream, dbias, rows, cols)
-                           : backward_typed<double>(ctx, dtype, gmap, y, upstream, dbias, rows, cols);
+    return dtype == RT_F32 ? backward_typed<float>(ctx, dtype, gmap, y, upstream, dbias, rows, cols, false)
+                           : backward_typed<double>(ctx, dtype, gmap, y, upstream, dbias, rows, cols, false);
+}
+
+extern "C" int32_t rt_fused_bias_relu_l1(rt_ctx* ctx, int32_t dtype, const void* x, uint64_t x_len, const void* bias, uint64_t bias_len, const void* target,
+                                         uint64_t target_len, void* y, uint64_t y_len, void* loss, uint64_t loss_len, uint64_t rows, uint64_t cols) {
+    RT_TRY(rt_ctx_enter(ctx));
+    RT_TRY(check_float("fused bias relu l1", dtype));
+    const uint64_t N = 16 / (uint64_t)rt_elem_size(dtype);
+    if (cols == 0 || rows == 0 || rows > (uint64_t)INT64_MAX / cols || rows * cols / N >= (1ull << 31))
+        return rt_fail(RT_E_INVALID, "fused bias relu l1: %llu x %llu is empty or too long for one launch", (unsigned long long)rows, (unsigned long long)cols);
+    const uint64_t n = rows * cols;
+    if (n > x_len || n > y_len || n > target_len || cols > bias_len || loss_len < 1)
+        return rt_fail(RT_E_OUT_OF_BOUNDS, "fused bias relu l1: operands shorter than rows * cols");
+    if (!x || !bias || !target || !y || !loss) return rt_fail(RT_E_INVALID, "fused bias relu l1: null buffer");
+    if (cols % N || !aligned16(x) || !aligned16(bias) || !aligned16(target) || !aligned16(y))
+        return rt_fail(RT_E_INVALID, "fused bias relu l1: needs 16-byte aligned operands and whole vectors per row (issue the separate ops instead)");
+    {
+        const int es = rt_elem_size(dtype);
+        const ByteSpan ys = rt_run_span(y, es, 0, n), ls = rt_run_span(loss, es, 0, 1);
+        if (bad_overlap(y, n, x, n, es) || rt_spans_meet(ys, rt_run_span(target, es, 0, n)) || rt_spans_meet(ys, rt_run_span(bias, es, 0, cols)) ||
+            rt_spans_meet(ls, ys) || rt_spans_meet(ls, rt_run_span(x, es, 0, n)) || rt_spans_meet(ls, rt_run_span(target, es, 0, n)) ||
+            rt_spans_meet(ls, rt_run_span(bias, es, 0, cols)))
+            return rt_fail(RT_E_INVALID, "fused bias relu l1: an output overlaps an input or the other output");
+    }
+    CtxGuard g(ctx);
+    return dtype == RT_F32 ? bias_relu_l1_typed<float>(ctx, dtype, x, bias, target, y, loss, rows, cols)
+                           : bias_relu_l1_typed<double>(ctx, dtype, x, bias, target, y, loss, rows, cols);
+}
+
+extern "C" int32_t rt_fused_l1_relu_backward_t(rt_ctx* ctx, int32_t dtype, const void* y, uint64_t y_len, const void* target, uint64_t target_len,
+                                               const void* upstream, uint64_t upstream_len, void* dbias, uint64_t dbias_len, uint64_t rows, uint64_t cols) {
+    RT_TRY(rt_ctx_enter(ctx));
+    RT_TRY(check_float("fused backward", dtype));
+    const uint64_t N = 16 / (uint64_t)rt_elem_size(dtype);
+    if (cols == 0 || rows == 0) return rt_fail(RT_E_INVALID, "fused backward: empty operand");
+    if (rows > (uint64_t)INT64_MAX / cols || rows * cols > target_len || rows * cols > y_len || cols > dbias_len || upstream_len < 1)
+        return rt_fail(RT_E_OUT_OF_BOUNDS, "fused backward: operands shorter than rows * cols");
+    if (!target || !y || !upstream || !dbias) return rt_fail(RT_E_INVALID, "fused backward: null buffer");
+    if (cols % N || !aligned16(target) || !aligned16(y) || !aligned16(dbias))
+        return rt_fail(RT_E_INVALID, "fused backward: needs 16-byte aligned operands and whole vectors per row (issue the separate ops instead)");
+    {
+        const int es = rt_elem_size(dtype);
+        const ByteSpan ds = rt_run_span(dbias, es, 0, cols);
+        if (rt_spans_meet(ds, rt_run_span(target, es, 0, rows * cols)) || rt_spans_meet(ds, rt_run_span(y, es, 0, rows * cols)) ||
+            rt_spans_meet(ds, rt_run_span(upstream, es, 0, 1)))
+            return rt_fail(RT_E_INVALID, "fused backward: the output overlaps an input");
+    }
+    CtxGuard g(ctx);
+    return dtype == RT_F32 ? backward_typed<float>(ctx, dtype, target, y, upstream, dbias, rows, cols, true)
+                           : backward_typed<double>(ctx, dtype, target, y, upstream, dbias, rows, cols, true);
 }

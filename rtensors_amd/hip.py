@@ -272,6 +272,14 @@ class Hip:
         _check(lib.rt_fused_l1_relu_backward(self._ctx, y.dtype, gmap.ptr, gmap.len, y.ptr, y.len, upstream.ptr, upstream.len, dbias.ptr, dbias.len,
                                              rows, cols))
 
+    def fused_bias_relu_l1(self, x: HipBuf, bias: HipBuf, target: HipBuf, y: HipBuf, loss: HipBuf, rows: int, cols: int):
+        _check(lib.rt_fused_bias_relu_l1(self._ctx, x.dtype, x.ptr, x.len, bias.ptr, bias.len, target.ptr, target.len, y.ptr, y.len, loss.ptr, loss.len,
+                                         rows, cols))
+
+    def fused_l1_relu_backward_t(self, y: HipBuf, target: HipBuf, upstream: HipBuf, dbias: HipBuf, rows: int, cols: int):
+        _check(lib.rt_fused_l1_relu_backward_t(self._ctx, y.dtype, y.ptr, y.len, target.ptr, target.len, upstream.ptr, upstream.len, dbias.ptr, dbias.len,
+                                               rows, cols))
+
     # ---- timing -----------------------------------------------------------------------------------------------------------
     def event(self):
         e = C.c_void_p()

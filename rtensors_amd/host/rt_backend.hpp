@@ -301,6 +301,16 @@ class Hip {
                                         rows, cols));
     }
 
+    // the same step without a stored gradient map
+    void fused_bias_relu_l1(const HipBuf& x, const HipBuf& bias, const HipBuf& target, HipBuf& y, HipBuf& loss, uint64_t rows, uint64_t cols) const {
+        check(rt_fused_bias_relu_l1(raw(), y.dtype(), x.ptr(), x.len(), bias.ptr(), bias.len(), target.ptr(), target.len(), y.ptr(), y.len(), loss.ptr(),
+                                    loss.len(), rows, cols));
+    }
+    void fused_l1_relu_backward_t(const HipBuf& y, const HipBuf& target, const HipBuf& upstream, HipBuf& dbias, uint64_t rows, uint64_t cols) const {
+        check(rt_fused_l1_relu_backward_t(raw(), y.dtype(), y.ptr(), y.len(), target.ptr(), target.len(), upstream.ptr(), upstream.len(), dbias.ptr(),
+                                          dbias.len(), rows, cols));
+    }
+
     // row-major copy of a view (what TensorView::owned needs, core/tensor.rs:299-325) in one launch
     void gather(const HipBuf& src, const MetaTensor& m, HipBuf& dst) const {
         check(rt_gather(raw(), src.dtype(), src.ptr(), src.len(), m.offset, (int32_t)m.rank(), m.shape.data(), m.strides.data(), dst.ptr(), dst.len()));

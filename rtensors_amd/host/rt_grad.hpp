@@ -258,21 +258,29 @@ inline bool fused_step_applies(const Tensor& x, const Tensor& bias, const Tensor
     auto whole = [](const Tensor& t) { return t.offset() == 0 && t.is_contiguous() && t.strides().back() == 1 && t.size() == t.buf()->len(); };
     return whole(x) && whole(bias) && whole(target);
 }
-inline FusedStep fused_bias_relu_l1_step(const Tensor& x, const Tensor& bias, const Tensor& target, bool seed_with_loss) {
+// passes == 3: y, then the loss and the stored gradient map, then d(bias) from the map (7 passes over a tensor).  passes == 2 (default):
+// y and the loss together, then d(bias) from y and the target with the map's elements formed in registers (5 passes).  The map is a
+// temporary of the tape (ops/broadcast/l1.rs:58-60), not a result; every value that is summed is the same bits either way.
+inline FusedStep fused_bias_relu_l1_step(const Tensor& x, const Tensor& bias, const Tensor& target, bool seed_with_loss, int passes = 2) {
     const Hip& be = x.backend();
     const int dt = x.dtype();
     const uint64_t rows = x.shape()[0], cols = x.shape()[1], n = rows * cols;
     FusedStep out;
-    Buf y = be.alloc_uninit(dt, n);
-    be.fused_bias_relu(*x.buf(), *bias.buf(), *y, rows, cols);
-    Buf gmap = be.alloc_uninit(dt, n), loss = be.alloc_uninit(dt, 1);
-    be.fused_l1_forward(*y, *target.buf(), *gmap, *loss, n);
+    Buf y = be.alloc_uninit(dt, n), loss = be.alloc_uninit(dt, 1), gmap;
+    if (passes == 3) {
+        be.fused_bias_relu(*x.buf(), *bias.buf(), *y, rows, cols);
+        gmap = be.alloc_uninit(dt, n);
+        be.fused_l1_forward(*y, *target.buf(), *gmap, *loss, n);
+    } else {
+        be.fused_bias_relu_l1(*x.buf(), *bias.buf(), *target.buf(), *y, *loss, rows, cols);
+    }
     out.y = Tensor(be, y, MetaTensor::row_major(x.shape()));
     out.loss = Tensor(be, loss, MetaTensor::row_major(Shape{}));
     // grad/mod.rs:442-447 seeds the root with the loss tensor itself
     Tensor seed = seed_with_loss ? out.loss : Tensor::ones(be, dt, Shape{});
     Buf dbias = be.alloc_uninit(dt, cols);
-    be.fused_l1_relu_backward(*gmap, *y, *seed.buf(), *dbias, rows, cols);
+    if (passes == 3) be.fused_l1_relu_backward(*gmap, *y, *seed.buf(), *dbias, rows, cols);
+    else be.fused_l1_relu_backward_t(*y, *target.buf(), *seed.buf(), *dbias, rows, cols);
     out.dbias = Tensor(be, dbias, MetaTensor::row_major(Shape{cols}));
     return out;
 }

@@ -176,16 +176,16 @@ int rth_train_step(void* x, void* bias, void* target, double lr, int mode, int s
     });
 }
 
-// The same step through the three fused passes (seed_with_loss as above; the broadcast gradient is the sum).  Returns 1 through
+// The same step through the fused passes, two or three of them (seed_with_loss as above; the broadcast gradient is the sum).  Returns 1 through
 // *out_used when the operands fit the fused form, else runs the tape and returns 0 there.
-int rth_train_step_fused(void* x, void* bias, void* target, double lr, int seed_with_loss, void** out_loss, void** out_grad, int* out_used) {
+int rth_train_step_fused(void* x, void* bias, void* target, double lr, int seed_with_loss, int passes, void** out_loss, void** out_grad, int* out_used) {
     if (!grad::fused_step_applies(*(Tensor*)x, *(Tensor*)bias, *(Tensor*)target)) {
         *out_used = 0;
         return rth_train_step(x, bias, target, lr, 0, seed_with_loss, out_loss, out_grad);
     }
     *out_used = 1;
     return guarded([&] {
-        grad::FusedStep st = grad::fused_bias_relu_l1_step(*(Tensor*)x, *(Tensor*)bias, *(Tensor*)target, seed_with_loss != 0);
+        grad::FusedStep st = grad::fused_bias_relu_l1_step(*(Tensor*)x, *(Tensor*)bias, *(Tensor*)target, seed_with_loss != 0, passes == 3 ? 3 : 2);
         *out_grad = new Tensor(st.dbias);
         *out_loss = new Tensor(st.loss);
         // SGD::step (grad/optim.rs:28-50): update = grad * lr, rounded to T, then an in-place broadcast sub through a mutable view

@@ -316,11 +316,12 @@ def train_step(x: Tensor, bias: Tensor, target: Tensor, lr: float, mode: str = "
     return Tensor(pl, x.backend), Tensor(pg, x.backend)
 
 
-def train_step_fused(x: Tensor, bias: Tensor, target: Tensor, lr: float, seed_with_loss: bool = True):
-    """The same step through the three fused passes (rt_fused_*).  Returns (loss, d_bias, used_fused); operands the fused form does
+def train_step_fused(x: Tensor, bias: Tensor, target: Tensor, lr: float, seed_with_loss: bool = True, passes: int = 2):
+    """The same step through the fused passes (rt_fused_*): passes=2 forms the L1 gradient map in registers, passes=3 stores it as
+    the tape does.  Returns (loss, d_bias, used_fused); operands the fused form does
     not take (views, dtypes other than f32 / f64, rows that are not whole 16-byte vectors) go through the tape and used_fused is False."""
     pl, pg, used = C.c_void_p(), C.c_void_p(), C.c_int(0)
-    _ck(_h.rth_train_step_fused(x._p, bias._p, target._p, C.c_double(lr), 1 if seed_with_loss else 0, C.byref(pl), C.byref(pg), C.byref(used)))
+    _ck(_h.rth_train_step_fused(x._p, bias._p, target._p, C.c_double(lr), 1 if seed_with_loss else 0, int(passes), C.byref(pl), C.byref(pg), C.byref(used)))
     return Tensor(pl, x.backend), Tensor(pg, x.backend), bool(used.value)
 
 

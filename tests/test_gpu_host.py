@@ -288,12 +288,27 @@ def test_fused_train_step_matches_oracle(T, be, dtype, seed_with_loss):
             upv = loss if seed_with_loss else npd.type(1)
             terms = ((oy.buf > 0).astype(npd) * (ogmap.buf * upv).astype(npd)).astype(npd).reshape(n, d).astype(np.float64)
             assert np.all(np.abs(hip.dump(hd).astype(np.float64) - terms.sum(axis=0)) <= tol * np.abs(terms).sum(axis=0) + 1e-300), (dtype, n, d)
+            # the two-pass form: the same y bit for bit, the same loss and d(bias) within the tolerance of a sum, no gradient map stored
+            hy2, hl2, hd2 = hip.alloc(code, n * d), hip.alloc(code, 1), hip.alloc(code, d)
+            hip.fused_bias_relu_l1(hx, hb, ht, hy2, hl2, n, d)
+            assert hip.dump(hy2).tobytes() == oy.buf.tobytes(), (dtype, n, d, "y, two passes")
+            loss2 = hip.dump(hl2)[0]
+            assert abs(float(loss2) - absdiff.sum() / float(np.float32(n * d))) <= tol * absdiff.sum() / (n * d) + 1e-300
+            up2 = hl2 if seed_with_loss else up
+            hip.fused_l1_relu_backward_t(hy2, ht, up2, hd2, n, d)
+            upv2 = loss2 if seed_with_loss else npd.type(1)
+            terms2 = ((oy.buf > 0).astype(npd) * (ogmap.buf * upv2).astype(npd)).astype(npd).reshape(n, d).astype(np.float64)
+            assert np.all(np.abs(hip.dump(hd2).astype(np.float64) - terms2.sum(axis=0)) <= tol * np.abs(terms2).sum(axis=0) + 1e-300), (dtype, n, d)
             hip.close()
         # host layer: fused step against the tape and the oracle's step
         gx, gt = T.Tensor.from_buf(be, dtype, x, [n, d]), T.Tensor.from_buf(be, dtype, target, [n, d])
-        gb1, gb2 = T.Tensor.from_buf(be, dtype, bias, [d]), T.Tensor.from_buf(be, dtype, bias, [d])
-        floss, fgrad, used = T.train_step_fused(gx, gb1, gt, 0.01, seed_with_loss)
+        gb3, gb2 = T.Tensor.from_buf(be, dtype, bias, [d]), T.Tensor.from_buf(be, dtype, bias, [d])
         tloss, tgrad = T.train_step(gx, gb2, gt, 0.01, "sum", seed_with_loss)
+        floss3, fgrad3, used3 = T.train_step_fused(gx, gb3, gt, 0.01, seed_with_loss, passes=3)
+        gb1 = T.Tensor.from_buf(be, dtype, bias, [d])
+        floss, fgrad, used = T.train_step_fused(gx, gb1, gt, 0.01, seed_with_loss)          # two passes (the default)
+        assert used3 == fits
+        assert abs(float(floss3.to_numpy()) - float(floss.to_numpy())) <= 2 * tol * absdiff.sum() / (n * d) + 1e-300
         assert used == fits
         assert abs(float(floss.to_numpy()) - absdiff.sum() / float(np.float32(n * d))) <= tol * absdiff.sum() / (n * d) + 1e-300
         assert fgrad.shape == [d]
@@ -302,7 +317,9 @@ def test_fused_train_step_matches_oracle(T, be, dtype, seed_with_loss):
             terms = ((oy.buf > 0).astype(npd) * (ogmap.buf * upv).astype(npd)).astype(npd).reshape(n, d).astype(np.float64)
         gtol = 2 * tol * np.abs(terms).sum(axis=0) + 1e-300
         assert np.all(np.abs(fgrad.to_numpy().astype(np.float64) - tgrad.to_numpy().astype(np.float64)) <= gtol)
+        assert np.all(np.abs(fgrad3.to_numpy().astype(np.float64) - tgrad.to_numpy().astype(np.float64)) <= gtol)
         assert np.max(np.abs(gb1.to_numpy().astype(np.float64) - gb2.to_numpy().astype(np.float64))) <= 0.01 * gtol.max() + np.finfo(npd).eps
+        assert np.max(np.abs(gb3.to_numpy().astype(np.float64) - gb2.to_numpy().astype(np.float64))) <= 0.01 * gtol.max() + np.finfo(npd).eps
         if n * d <= 300000:
             # the oracle's whole step (its loss is a sequential f32 sum, which is itself only good to about 1e-7 * n: small shapes only)
             oloss, ograd = oracle_train_step(ox, ob, ot, 0.01, "sum", seed_with_loss)
@@ -540,6 +557,9 @@ def test_config5_full_size_step(be, T):
     gloss, ggrad = T.train_step(gx, gb, gt, 0.01, "sum", True)
     floss, fgrad, used = T.train_step_fused(gx, gb_fused, gt, 0.01, True)
     assert used
+    gb_fused3 = T.Tensor.from_buf(be, "f32", bias, [d])
+    floss3, fgrad3, used3 = T.train_step_fused(gx, gb_fused3, gt, 0.01, True, passes=3)
+    assert used3
     pre = x.reshape(n, d) + bias
     y = np.maximum(pre, 0)
     diff = y - target.reshape(n, d)
@@ -562,3 +582,8 @@ def test_config5_full_size_step(be, T):
     assert np.all(np.abs(fgrad.to_numpy().astype(np.float64) - up_f.astype(np.float64).sum(axis=0)) <= 1e-5 * np.abs(up_f.astype(np.float64)).sum(axis=0) + 1e-30)
     want_fused = bias - (fgrad.to_numpy() * np.float32(0.01)).astype(np.float32)
     assert gb_fused.to_numpy().tobytes() == want_fused.astype(np.float32).tobytes()
+    assert abs(float(floss3.to_numpy()) - loss) <= 1e-5 * loss
+    up_3 = (gm * np.float32(float(floss3.to_numpy()))).astype(np.float32) * (pre > 0)
+    assert np.all(np.abs(fgrad3.to_numpy().astype(np.float64) - up_3.astype(np.float64).sum(axis=0)) <= 1e-5 * np.abs(up_3.astype(np.float64)).sum(axis=0) + 1e-30)
+    want_fused3 = bias - (fgrad3.to_numpy() * np.float32(0.01)).astype(np.float32)
+    assert gb_fused3.to_numpy().tobytes() == want_fused3.astype(np.float32).tobytes()
