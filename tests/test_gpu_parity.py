@@ -648,6 +648,55 @@ def _tol(dtype, x):
     return {"f32": 1e-5, "f64": 1e-12}[dtype] * float(np.abs(x.astype(np.float64)).sum())
 
 
+@pytest.mark.parametrize("dtype", ["f32", "u8", "i16", "f64"])
+def test_broadcast_long_rows(hip, dtype):
+    """Rows of 64 or more 16-byte vectors with every pairing of row-wise and repeated operands (the one-vector-per-lane row kernel):
+    ragged row ends, rows cut out of longer rows at odd offsets, one to three outer dims, reversed and stepped outer dims, an operand
+    that does not move along an outer dim, in-place accumulation."""
+    rng = np.random.default_rng(43)
+    per_vec = 16 // np.dtype(cpu.NP_DTYPE[cpu.DTYPE_BY_NAME[dtype]]).itemsize
+    L = 66 * per_vec + 3
+    def cut(t, cuts):
+        for dim, sl in cuts:
+            t = t.slice(dim, sl)
+        return t
+    cases = [
+        # (shape of a, cuts of a, shape of b, cuts of b)
+        ([7, L], [], [7, L], []),
+        ([7, L], [], [L], []),
+        ([7, 1], [], [7, L], []),
+        ([9, L + 9], [(1, Slice(4, 4 + L, 1))], [L], []),
+        ([5, 6, L], [(1, Slice(None, None, -1))], [6, L], []),
+        ([5, 6, L], [(0, Slice(0, None, 2))], [3, 6, 1], []),
+        ([2, 5, 4, L], [(2, Slice(None, None, -1)), (3, Slice(1, L, 1))], [5, 1, L - 1], []),
+        ([2, 1, 4, L], [], [1, 5, 1, L], []),
+        ([4, 64 * per_vec], [], [4, 1], []),
+        ([6, 128 * per_vec], [(1, Slice(0, 64 * per_vec, 1))], [6, 128 * per_vec], [(1, Slice(64 * per_vec, None, 1))]),
+    ]
+    for trial, (sa, ca, sb, cb) in enumerate(cases):
+        va, vb = rand_values(dtype, int(np.prod(sa)), rng), rand_values(dtype, int(np.prod(sb)), rng)
+        for op in ("add", "mul", "sub"):
+            oa, ob = OTensor.from_buf(dtype, va, sa), OTensor.from_buf(dtype, vb, sb)
+            ga, gb = G(hip, dtype, va, sa), G(hip, dtype, vb, sb)
+            ova, ovb, gva, gvb = cut(oa, ca), cut(ob, cb), cut(ga, ca), cut(gb, cb)
+            with np.errstate(all="ignore"):
+                want = {"add": ova.__add__, "sub": ova.__sub__, "mul": ova.__mul__}[op](ovb)
+                got = {"add": gva.__add__, "sub": gva.__sub__, "mul": gva.__mul__}[op](gvb)
+                assert got.meta.shape == want.meta.shape
+                assert got.dump().tobytes() == want.buf.tobytes(), (trial, dtype, op, "a op b")
+                want2 = {"add": ovb.__add__, "sub": ovb.__sub__, "mul": ovb.__mul__}[op](ova)
+                got2 = {"add": gvb.__add__, "sub": gvb.__sub__, "mul": gvb.__mul__}[op](gva)
+                assert got2.dump().tobytes() == want2.buf.tobytes(), (trial, dtype, op, "b op a")
+                if want.meta.shape == ova.meta.shape and all(st != 0 for st in ova.meta.strides):
+                    if op == "add":
+                        ova += ovb; gva += gvb
+                    elif op == "sub":
+                        ova -= ovb; gva -= gvb
+                    else:
+                        ova *= ovb; gva *= gvb
+                    assert ga.dump().tobytes() == oa.buf.tobytes(), (trial, dtype, op, "in place")
+
+
 @pytest.mark.parametrize("dtype", ["f32", "f64", "i32", "i64", "u8", "i16", "u32"])
 @pytest.mark.parametrize("op", ["sum", "prod", "max", "min", "mean"])
 def test_reduce_random_vs_oracle(hip, dtype, op):
@@ -830,7 +879,8 @@ def test_gather_transposed_views(hip, dtype):
     """Row-major copy (`owned()` / `contiguous()`) of permuted, reversed and stepped views large enough for the
     LDS-transpose copy kernel, with ragged tile edges."""
     rng = np.random.default_rng(17)
-    for shape in [(64, 257), (3, 40, 70), (2, 5, 33, 130), (4, 17, 1030), (100, 36), (2, 3, 16, 16), (7, 300, 9), (48, 2100), (2, 32, 1040), (160, 520)]:
+    for shape in [(64, 257), (3, 40, 70), (2, 5, 33, 130), (4, 17, 1030), (100, 36), (2, 3, 16, 16), (7, 300, 9), (48, 2100), (2, 32, 1040), (160, 520),
+                  (512, 64), (2, 768, 32), (1024, 256)]:                     # whole numbers of tiles once transposed
         r = len(shape)
         vals = rand_values(dtype, int(np.prod(shape)), rng)
         o, g = OTensor.from_buf(dtype, vals, list(shape)), G(hip, dtype, vals, list(shape))
@@ -980,7 +1030,9 @@ def test_broadcast_with_transposed_operand(hip, dtype):
     """One input is a permuted (and possibly reversed / strided) view whose unit-stride dim is not the output's inner dim:
     the LDS-transpose tile kernel.  Ragged tile edges, both operand positions, broadcast and in-place forms."""
     rng = np.random.default_rng(zlib.crc32(dtype.encode()))
-    shapes = [(3, 40, 70), (2, 5, 33, 130), (64, 257), (1, 100, 36), (4, 17, 1030), (2, 3, 16, 16), (48, 2100), (2, 32, 1040), (160, 520)]
+    # the last two shapes are whole numbers of tiles for every element size (the kernel's form without edge tests)
+    shapes = [(3, 40, 70), (2, 5, 33, 130), (64, 257), (1, 100, 36), (4, 17, 1030), (2, 3, 16, 16), (48, 2100), (2, 32, 1040), (160, 520),
+              (64, 512), (2, 3, 32, 768)]
     for shape in shapes:
         r = len(shape)
         perm = list(range(r)); perm[-1], perm[-2] = perm[-2], perm[-1]
