@@ -214,6 +214,14 @@ __global__ void rt_zero_kernel(uint4* p, size_t nvec) {
     const size_t step = (size_t)gridDim.x * blockDim.x;
     for (; i < nvec; i += step) p[i] = make_uint4(0, 0, 0, 0);
 }
+// The zero fill of Backend::alloc for large blocks: one vector per lane in the write-only tiled order (512-lane blocks own 1 KiB
+// pieces of 16 pages 64 KiB apart, see TileMap), non-temporal stores.  1 GiB: 0.279 ms with the grid-stride kernel above, 0.15 ms so.
+__global__ __launch_bounds__(512) void rt_zero_tiled_kernel(rt_u32x4* p, size_t nvec, TileMap m) {
+    size_t i;
+    if (!rt_tile_index(m, blockIdx.x, 512, threadIdx.x, nvec, &i)) return;
+    const rt_u32x4 z = {0u, 0u, 0u, 0u};
+    __builtin_nontemporal_store(z, p + i);
+}
 
 // ---- host <-> device transfers ----------------------------------------------------------------------------------------
 // A copy between device memory and ordinary (pageable) host memory goes through a ring of pinned staging buffers: the DMA
@@ -398,9 +406,15 @@ static int32_t alloc_impl(rt_ctx* ctx, int32_t dtype, uint64_t len, void** out, 
     if (zero && bytes) {
         // whole size class is zeroed (capacity is a multiple of 512 B), by a fill kernel rather than a memset node
         size_t nvec = size_class(bytes) / 16;
-        size_t blocks = (nvec + 255) / 256;
-        if (blocks > (size_t)ctx->num_cus * 16) blocks = (size_t)ctx->num_cus * 16;
-        hipLaunchKernelGGL(rt_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (uint4*)*out, nvec);
+        const TileMap m = rt_make_tilemap(*out, nvec, 512, 1024, 16, 65536);
+        const size_t tiled_blocks = rt_tilemap_blocks(m, nvec, 512);
+        if (nvec >= (1u << 16) && tiled_blocks <= 0x7fffffffull) {
+            hipLaunchKernelGGL(rt_zero_tiled_kernel, dim3((unsigned)tiled_blocks), dim3(512), 0, ctx->stream, (rt_u32x4*)*out, nvec, m);
+        } else {
+            size_t blocks = (nvec + 255) / 256;
+            if (blocks > (size_t)ctx->num_cus * 16) blocks = (size_t)ctx->num_cus * 16;
+            hipLaunchKernelGGL(rt_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (uint4*)*out, nvec);
+        }
         RT_HIP(hipGetLastError());
     }
     return RT_OK;
