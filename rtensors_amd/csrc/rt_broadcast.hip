@@ -433,6 +433,11 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
     hipStream_t s = ctx->stream;
     const int rank = dsc.rank;
 
+    // 2^31 elements or more in an N-d layout (a 2 GiB u8 broadcast): slices along the outermost dim, each through the kernels below
+    // (the element-per-lane 64-bit kernel that would otherwise take it runs at 3 % of their speed)
+    if (count >= (1ull << 31) && rank >= 2)
+        return rt_for_slices_below_2g(dsc, count, [&](const NdDesc& sub, uint64_t n) { return broadcast_typed<T, OP>(ctx, sub, n, lv, rv, dv); });
+
     // (1) one unit-stride run in all three operands
     // (for the gather op the right operand is a placeholder that is never read: treat it as a twin of the left one)
     const bool r_unit = (OP == kOpCopy) || rank == 0 || dsc.stride[1][0] == 1;

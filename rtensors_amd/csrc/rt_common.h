@@ -118,6 +118,12 @@ inline bool rt_spans_meet(ByteSpan a, ByteSpan b) { return a.lo < b.hi && b.lo <
 bool rt_same_view(const void* a, uint64_t a_offset, const int64_t* a_strides, const void* b, uint64_t b_offset, const int64_t* b_strides,
                   int rank, const uint64_t* shape);
 
+// Launches whose index arithmetic is 32-bit take fewer than 2^31 elements.  A larger N-d descriptor is cut along its outermost dim into
+// slices below that bound (`fn(sub, count_of_sub)` is called for each, in order); when one index of that dim alone is too large the
+// dim is dropped and every index becomes a descriptor of its own, to be cut further by the callee.  Returns the first non-zero status.
+struct NdDesc;
+template <class Fn> int32_t rt_for_slices_below_2g(const NdDesc& d, uint64_t count, Fn fn);
+
 // A view over up to three operands sharing one shape, after removal of size-1 dims and merging of adjacent dims
 // that are mergeable in every operand.  Dim 0 is outermost.
 struct NdDesc {
@@ -126,6 +132,29 @@ struct NdDesc {
     int64_t stride[3][RT_MAX_RANK];
     int64_t offset[3];
 };
+
+template <class Fn> int32_t rt_for_slices_below_2g(const NdDesc& d, uint64_t count, Fn fn) {
+    const uint64_t n0 = (uint64_t)d.shape[0], per = count / n0;
+    const bool drop = per >= (1ull << 31);                        // one index alone is too large: a descriptor per index, dim 0 removed
+    const uint64_t step = drop ? 1 : ((1ull << 31) - 1) / per;
+    for (uint64_t i0 = 0; i0 < n0; i0 += step) {
+        const uint64_t take = n0 - i0 < step ? n0 - i0 : step;
+        NdDesc sub = d;
+        for (int o = 0; o < 3; ++o) sub.offset[o] += (int64_t)i0 * d.stride[o][0];
+        if (take == 1) {
+            for (int k = 1; k < d.rank; ++k) {
+                sub.shape[k - 1] = d.shape[k];
+                for (int o = 0; o < 3; ++o) sub.stride[o][k - 1] = d.stride[o][k];
+            }
+            sub.rank = d.rank - 1;
+        } else {
+            sub.shape[0] = (int64_t)take;
+        }
+        const int32_t st = fn(sub, take * per);
+        if (st != 0) return st;
+    }
+    return 0;
+}
 
 // Collapses `nops` operands (1..3).  When `reorder` is set (allowed whenever the visiting order of elements is
 // irrelevant, i.e. for every elementwise op), dims are first flipped so operand `key`'s strides are non-negative

@@ -548,6 +548,8 @@ int32_t launch_view(rt_ctx* ctx, T* base, const NdDesc& d, uint64_t count, F f) 
         RT_HIP(hipGetLastError());
         return RT_OK;
     }
+    if (count >= (1ull << 31) && d.rank >= 2)                     // slices along the outermost dim, each through the 32-bit kernels below
+        return rt_for_slices_below_2g(d, count, [&](const NdDesc& sub, uint64_t n) { return launch_view<T, F>(ctx, base, sub, n, f); });
     if (count >= (1ull << 31)) {
         size_t blocks = (size_t)((count + kBlock - 1) / kBlock);
         hipLaunchKernelGGL((ew_nd64_kernel<T, F>), dim3(capped_grid(blocks, (size_t)ctx->num_cus * 64)), dim3(kBlock), 0, ctx->stream,

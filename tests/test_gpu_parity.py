@@ -1223,6 +1223,22 @@ def test_more_than_2_31_elements(hip):
     hip.apply_argmax_contiguous_nd((d, (0, [rows, cols], [cols, 1])), idx, 1, "argmax")
     got = hip.dump(idx)
     assert int(got[p_max // cols]) == p_max % cols and int(got.sum()) == p_max % cols
+    # an N-d broadcast and an N-d in-place op over 2^31+ elements: issued as slices along the outer dim (2047 rows, then 2), each
+    # through the 32-bit kernels; rows on both sides of the cut and at both ends are held to numpy
+    del a, idx
+    yv = (np.arange(cols) % 5).astype(np.uint8)
+    y = hip.alloc_from_slice(H.U8, yv)
+    z = hip.alloc_uninit(H.U8, n)
+    full = (0, [rows, cols], [cols, 1])
+    hip.broadcast((d, full), (y, (0, [rows, cols], [0, 1])), (z, full), "add")
+    hip.scalar_nd("add", z, 1, 0, [rows, cols - 1], [cols, 1])          # every row but its last column
+    row_x, row_z = hip.alloc_uninit(H.U8, cols), hip.alloc_uninit(H.U8, cols)
+    for r in (0, 1, 2046, 2047, 2048, rows - 1, p_max // cols):
+        hip.copy_range_within(row_x, d, 0, r * cols, cols)
+        hip.copy_range_within(row_z, z, 0, r * cols, cols)
+        want = hip.dump(row_x) + yv
+        want[:-1] += 1
+        assert np.array_equal(hip.dump(row_z), want), r
     hip.sync()
 
 
