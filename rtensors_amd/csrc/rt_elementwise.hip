@@ -389,7 +389,7 @@ __global__ __launch_bounds__(kCBlock) void ew_rows_kernel(T* __restrict__ p, Row
     }
 }
 
-// Lean form of the row kernel for rows of at least 64 vectors and at most two outer dims besides the row dim: a 256-lane block owns
+// Lean form of the row kernel for rows of at least 128 vectors and at most two outer dims besides the row dim: a 256-lane block owns
 // the same 1 KiB piece of four consecutive rows, one wave per row, one vector per lane; the outer dims are grid dims y / z, every
 // kernel argument is fetched in one batch and all offsets fit 32 bits (checked on the host).  A wave's whole life is one load,
 // the op and one store.  relu in place on the left half of a 16384 x 16384 f32 matrix: 0.79 -> 0.85 of peak.
@@ -399,7 +399,11 @@ struct Rows4Args {
     int32_t gs, o0s, o1s;           // strides along the row dim and the two outer dims (inner one first)
 };
 
-template <class T, class F, bool NT>
+// Vectors sit on the 16-byte grid of memory whatever the phase of the row: the lane's column is shifted back by the row's phase, the
+// up to N - 1 elements before the first whole vector and after the last one are handled one by one.  (Vectors at element alignment
+// cost `m[:, 1:]` of a 65536 x 4096 f32 matrix 0.72 of peak with cached and 0.63 with non-temporal accesses; 0.83 so, all accesses
+// non-temporal.  A fill of all but three columns of that matrix: 0.51 -> 0.76.)
+template <class T, class F>
 __global__ __launch_bounds__(256) void ew_rows4_kernel(T* p, Rows4Args a, F f) {
     constexpr int N = 16 / sizeof(T);
     uint32_t L = a.L, G = a.G, tiles = a.tiles, tm = a.tiles_div.mul, ts = a.tiles_div.shift;
@@ -411,21 +415,27 @@ __global__ __launch_bounds__(256) void ew_rows4_kernel(T* p, Rows4Args a, F f) {
     const uint32_t g = chunk * 4 + (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     if (g >= G) return;
     T* rowp = p + ((int32_t)blockIdx.z * o1 + (int32_t)blockIdx.y * o0 + (int32_t)g * gs);
-    const uint32_t c = (tile * 64 + (threadIdx.x & 63)) * N;
-    if (c >= L) return;
-    if (c + N <= L) {
-        rt_u32x4 w = {};
-        if constexpr (F::kReads) w = rt_ld16u<T, NT>(rowp + c);
-        Vec16<T> e = __builtin_bit_cast(Vec16<T>, w);
+    const uint32_t phase = (uint32_t)((reinterpret_cast<uintptr_t>(rowp) / sizeof(T)) & (uintptr_t)(N - 1));
+    const int32_t c = (int32_t)((tile * 64 + (threadIdx.x & 63)) * N) - (int32_t)phase;
+    if (c >= (int32_t)L) return;
+    if (c >= 0 && (uint32_t)c + N <= L) {
+        Vec16<T>* vp = reinterpret_cast<Vec16<T>*>(rowp + c);
+        Vec16<T> e = {};
+        if constexpr (F::kReads) e = rt_ld16_nt(vp);
         apply_vec(e, f);
-        w = __builtin_bit_cast(rt_u32x4, e);
-        if constexpr (F::kReads && NT) rt_st16u_nt<T>(rowp + c, w); else rt_st16u<T>(rowp + c, w);
+        rt_st16_nt(vp, e);
     } else {
-        for (uint32_t k = c; k < L; ++k) {
-            T x = zero_of<T>();
-            if constexpr (F::kReads) x = rowp[k];
-            rowp[k] = f(x);
+        // the ragged ends of a row: all loads, then all stores
+        const uint32_t k0 = c < 0 ? 0u : (uint32_t)c, k1 = min((uint32_t)(c + N), L);
+        T x[N];
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            x[j] = zero_of<T>();
+            if constexpr (F::kReads) { if (k0 + j < k1) x[j] = rowp[k0 + j]; }
         }
+#pragma unroll
+        for (int j = 0; j < N; ++j)
+            if (k0 + j < k1) rowp[k0 + j] = f(x[j]);
     }
 }
 
@@ -587,13 +597,26 @@ int32_t launch_view(rt_ctx* ctx, T* base, const NdDesc& d, uint64_t count, F f) 
         }
         for (int k = r.nouter; k < RT_MAX_RANK; ++k) { r.oshape[k] = 1; r.odiv[k] = make_fastdiv(1); }
         const uint32_t vecs = (uint32_t)((r.L + N - 1) / N);
-        if (vecs >= 64 && r.G >= 4 && d.rank <= 4) {
+        // (rows of one tile, 64 ... 127 vectors, measured level or a little faster on the general kernel below)
+        if (vecs >= 128 && r.G >= 4 && d.rank <= 4) {
             uint64_t reach = 0;
             for (int k = 0; k < d.rank; ++k) reach += (uint64_t)(d.shape[k] - 1) * (uint64_t)(d.stride[0][k] < 0 ? -d.stride[0][k] : d.stride[0][k]);
             const uint64_t n0 = d.rank >= 3 ? (uint64_t)d.shape[d.rank - 3] : 1ull, n1 = d.rank >= 4 ? (uint64_t)d.shape[d.rank - 4] : 1ull;
             Rows4Args q;
             q.L = r.L; q.G = r.G;
-            q.tiles = (vecs + 63) / 64;
+            // room for the largest phase a row can have: the base's own when every row starts a whole number of vectors from it
+            uint32_t max_phase = (uint32_t)((reinterpret_cast<uintptr_t>(p) / sizeof(T)) & (uintptr_t)(N - 1));
+            for (int k = 0; k < d.rank - 1; ++k)
+                if (d.stride[0][k] % N != 0) max_phase = (uint32_t)N - 1;
+            q.tiles = (uint32_t)(((r.L + max_phase + N - 1) / N + 63) / 64);
+            // Rows with ragged ends that are read and written: an odd number of tiles per row.  Blocks go to the eight XCDs in turn, so
+            // with an even count the first tile of every row -- whose first lane handles the row's ragged start element by element, the
+            // longest-lived wave of the row -- keeps landing on the same few XCDs, and the last tile on others.  One more (empty) tile
+            // makes the assignment drift: relu on m[:, 1:] of 65536 x 4096 f32 0.70 -> 0.84 of peak, of 8192 x 32768 0.82 -> 0.85, of
+            // 262144 x 1024 0.66 -> 0.76, of 524288 x 512 0.70 -> 0.76.  Rotating the tile index instead was slower for long rows, and fills (no loads, nothing
+            // long-lived) lose 10 % either way and keep the exact count.
+            const bool ragged = max_phase != 0 || r.L % N != 0;
+            if (F::kReads && ragged && q.tiles % 2 == 0) q.tiles += 1;
             q.tiles_div = make_fastdiv(q.tiles);
             const uint64_t gx = (uint64_t)q.tiles * ((r.G + 3) / 4);
             if (reach < (1ull << 31) && n0 <= 65535 && n1 <= 65535 && gx < (1ull << 31)) {
@@ -601,8 +624,7 @@ int32_t launch_view(rt_ctx* ctx, T* base, const NdDesc& d, uint64_t count, F f) 
                 q.o0s = d.rank >= 3 ? (int32_t)d.stride[0][d.rank - 3] : 0;
                 q.o1s = d.rank >= 4 ? (int32_t)d.stride[0][d.rank - 4] : 0;
                 const dim3 grid((unsigned)gx, (unsigned)n0, (unsigned)n1);
-                if (whole_lines) hipLaunchKernelGGL((ew_rows4_kernel<T, F, true>), grid, dim3(256), 0, ctx->stream, p, q, f);
-                else hipLaunchKernelGGL((ew_rows4_kernel<T, F, false>), grid, dim3(256), 0, ctx->stream, p, q, f);
+                hipLaunchKernelGGL((ew_rows4_kernel<T, F>), grid, dim3(256), 0, ctx->stream, p, q, f);
                 RT_HIP(hipGetLastError());
                 return RT_OK;
             }

@@ -424,15 +424,18 @@ def test_inplace_ops_on_long_row_views(hip, dtype):
     untouched."""
     rng = np.random.default_rng(41)
     per_vec = 16 // np.dtype(cpu.NP_DTYPE[cpu.DTYPE_BY_NAME[dtype]]).itemsize
-    L0 = 70 * per_vec + 3
+    L0 = 135 * per_vec + 3
     for trial, (shape, cuts) in enumerate([
+        ([9, 70 * per_vec + 3], [(1, Slice(1, 70 * per_vec, 1))]),
         ([9, L0], [(1, Slice(1, L0 - 2, 1))]),
-        ([9, L0 + 13], [(1, Slice(5, 5 + 64 * per_vec, 1)), (0, Slice(None, None, -1))]),
+        ([9, L0 + 13], [(1, Slice(5, 5 + 128 * per_vec, 1)), (0, Slice(None, None, -1))]),
+        ([9, L0 + 13], [(1, Slice(3, 3 + 128 * per_vec + 2, 1))]),
         ([3, 6, L0], [(2, Slice(2, None, 1)), (1, Slice(0, None, 2))]),
         ([2, 3, 5, L0], [(3, Slice(0, L0 - 1, 1)), (1, Slice(None, None, -1)), (2, Slice(1, 5, 1))]),
-        ([5, 4, 2 * L0], [(2, Slice(L0 // 2, L0 // 2 + 65 * per_vec + 1, 1)), (0, Slice(1, 4, 1))]),
+        ([5, 4, 2 * L0], [(2, Slice(L0 // 2, L0 // 2 + 129 * per_vec + 1, 1)), (0, Slice(1, 4, 1))]),
         ([4, 128 * per_vec], [(0, Slice(0, 4, 1))]),
         ([6, 256 * per_vec], [(1, Slice(0, 128 * per_vec, 1))]),
+        ([6, 256 * per_vec], [(1, Slice(1, 255 * per_vec, 1))]),
     ]):
         vals = rand_values(dtype, int(np.prod(shape)), rng)
         for which in range(4):
