@@ -675,6 +675,11 @@ def test_broadcast_long_rows(hip, dtype):
         ([2, 1, 4, L], [], [1, 5, 1, L], []),
         ([4, 64 * per_vec], [], [4, 1], []),
         ([6, 128 * per_vec], [(1, Slice(0, 64 * per_vec, 1))], [6, 128 * per_vec], [(1, Slice(64 * per_vec, None, 1))]),
+        # dst rows off the 16-byte grid (the in-place leg writes through the view of a): every phase, ragged at both ends
+        ([6, L + 5], [(1, Slice(1, 1 + L, 1))], [L], []),
+        ([6, L + 5], [(1, Slice(2, 2 + L, 1))], [6, 1], []),
+        ([3, 5, L + 4], [(2, Slice(3, 3 + L, 1)), (1, Slice(None, None, -1))], [5, L], []),
+        ([8, 130 * per_vec + 1], [(1, Slice(1, None, 1))], [8, 130 * per_vec + 1], [(1, Slice(0, 130 * per_vec, 1))]),
     ]
     for trial, (sa, ca, sb, cb) in enumerate(cases):
         va, vb = rand_values(dtype, int(np.prod(sa)), rng), rand_values(dtype, int(np.prod(sb)), rng)
