@@ -165,7 +165,9 @@ struct Rows4Args {
 
 // grid: x = column tile + tiles * (chunk of four rows), y = index along the inner outer dim, z = index along the outer one.  Every
 // offset inside an operand fits 32 bits (checked on the host).
-template <class T, int OP, int LM, int RM>
+// NTM: bit 0 / 1 = the left / right input is a row-wise operand that is read exactly once (no stride-0 dim): non-temporal loads.  A
+// compile-time choice: two loads that differ only in the hint are merged by the compiler, and the hint is lost.
+template <class T, int OP, int LM, int RM, int NTM>
 __global__ __launch_bounds__(256) void bin_rows4_kernel(const T* l, const T* r, T* d, Rows4Args a, int32_t* fault) {
     constexpr int N = 16 / sizeof(T);
     uint32_t L = a.L, G = a.G, tiles = a.tiles, tm = a.tiles_div.mul, ts = a.tiles_div.shift;
@@ -186,9 +188,11 @@ __global__ __launch_bounds__(256) void bin_rows4_kernel(const T* l, const T* r, 
     const int32_t c = (int32_t)((tile * 64 + (threadIdx.x & 63)) * N) - (int32_t)phase;
     if (c >= (int32_t)L) return;
     if (c >= 0 && (uint32_t)c + N <= L) {
-        const rt_u32x4 x = load_raw<T, LM>(lp, (uint32_t)c, 1);
-        rt_u32x4 y = x;
-        if constexpr (OP != kOpCopy) y = load_raw<T, RM>(rp, (uint32_t)c, 1);
+        rt_u32x4 x, y;
+        if constexpr (LM == M_VEC && (NTM & 1)) x = rt_ld16u<T, true>(lp + c); else x = load_raw<T, LM>(lp, (uint32_t)c, 1);
+        if constexpr (OP == kOpCopy) y = x;
+        else if constexpr (RM == M_VEC && (NTM & 2)) y = rt_ld16u<T, true>(rp + c);
+        else y = load_raw<T, RM>(rp, (uint32_t)c, 1);
         Vec16<T> xv = __builtin_bit_cast(Vec16<T>, x);
         bin_apply_vec<OP, T>(xv, __builtin_bit_cast(Vec16<T>, y), fault);
         rt_st16_nt(reinterpret_cast<Vec16<T>*>(dp + c), xv);
@@ -209,11 +213,19 @@ __global__ __launch_bounds__(256) void bin_rows4_kernel(const T* l, const T* r, 
 }
 
 template <class T, int OP>
-void launch_rows4(int lm, int rm, dim3 grid, hipStream_t s, const T* l, const T* r, T* d, const Rows4Args& a, int32_t* fault) {
-    if (lm == M_VEC && rm == M_VEC) hipLaunchKernelGGL((bin_rows4_kernel<T, OP, M_VEC, M_VEC>), grid, dim3(256), 0, s, l, r, d, a, fault);
-    else if (lm == M_VEC) hipLaunchKernelGGL((bin_rows4_kernel<T, OP, M_VEC, M_BCAST>), grid, dim3(256), 0, s, l, r, d, a, fault);
-    else if (rm == M_VEC) hipLaunchKernelGGL((bin_rows4_kernel<T, OP, M_BCAST, M_VEC>), grid, dim3(256), 0, s, l, r, d, a, fault);
-    else hipLaunchKernelGGL((bin_rows4_kernel<T, OP, M_BCAST, M_BCAST>), grid, dim3(256), 0, s, l, r, d, a, fault);
+void launch_rows4(int lm, int rm, int ntm, dim3 grid, hipStream_t s, const T* l, const T* r, T* d, const Rows4Args& a, int32_t* fault) {
+    const bool nl = lm == M_VEC && (ntm & 1), nr = rm == M_VEC && (ntm & 2);
+#define RT_R4(LMV, RMV, NT) hipLaunchKernelGGL((bin_rows4_kernel<T, OP, LMV, RMV, NT>), grid, dim3(256), 0, s, l, r, d, a, fault)
+    if (lm == M_VEC && rm == M_VEC) {
+        if (nl && nr) RT_R4(M_VEC, M_VEC, 3); else if (nl) RT_R4(M_VEC, M_VEC, 1); else if (nr) RT_R4(M_VEC, M_VEC, 2); else RT_R4(M_VEC, M_VEC, 0);
+    } else if (lm == M_VEC) {
+        if (nl) RT_R4(M_VEC, M_BCAST, 1); else RT_R4(M_VEC, M_BCAST, 0);
+    } else if (rm == M_VEC) {
+        if (nr) RT_R4(M_BCAST, M_VEC, 2); else RT_R4(M_BCAST, M_VEC, 0);
+    } else {
+        RT_R4(M_BCAST, M_BCAST, 0);
+    }
+#undef RT_R4
 }
 
 // ---- generic ------------------------------------------------------------------------------------------------------------
@@ -644,7 +656,15 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
                     q.o0s[o] = rank >= 3 ? (int32_t)dsc.stride[o][rank - 3] : 0;
                     q.o1s[o] = rank >= 4 ? (int32_t)dsc.stride[o][rank - 4] : 0;
                 }
-                launch_rows4<T, OP>(lm, rm, dim3((unsigned)gx, (unsigned)n0, (unsigned)n1), s, l + dsc.offset[0], r + dsc.offset[1], d + dsc.offset[2], q, fault_of<T, OP>(ctx));
+                // inputs that are read exactly once (no stride-0 dim) are loaded with the non-temporal hint: a left half += (R, 1) on
+                // 65536 x 8192 f32 0.78 -> 0.82 of peak, w = a + b on half-width views 0.78 -> 0.85, z += x over 2 GiB 0.74 -> 0.79
+                int ntm = 0;
+                for (int o = 0; o < 2; ++o) {
+                    bool once = true;
+                    for (int k = 0; k < rank; ++k) once = once && dsc.stride[o][k] != 0;
+                    if (once) ntm |= 1 << o;
+                }
+                launch_rows4<T, OP>(lm, rm, ntm, dim3((unsigned)gx, (unsigned)n0, (unsigned)n1), s, l + dsc.offset[0], r + dsc.offset[1], d + dsc.offset[2], q, fault_of<T, OP>(ctx));
                 RT_HIP(hipGetLastError());
                 return RT_OK;
             }

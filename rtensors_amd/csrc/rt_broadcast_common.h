@@ -100,9 +100,9 @@ template <class T, int MODE>
 __device__ __forceinline__ rt_u32x4 load_raw(const T* __restrict__ rowp, uint32_t c, int64_t istride) {
     constexpr int N = 16 / sizeof(T);
     if constexpr (MODE == M_VEC) {
-        // Unit stride along the row; the row may start at any element.  Plain (cached) loads also for operands that are read only
-        // once: a non-temporal hint chosen at run time measured no gain on them (a column-sliced 1 GiB operand plus a row, the
-        // transposed add) and its second code path cost the config-3 add 4 %.
+        // Unit stride along the row; the row may start at any element.  Plain (cached) loads: right for operands that are re-read
+        // (broadcast along some dim).  Kernels that know an operand is read once load it with rt_ld16u<T, true> themselves -- the
+        // choice has to be made at compile time, because two loads that differ only in the hint are merged and the hint is lost.
         return rt_ld16u<T, false>(rowp + c);
     } else {
         Vec16<T> v;

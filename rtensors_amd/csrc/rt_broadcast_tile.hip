@@ -266,7 +266,8 @@ struct StageArgs {
 
 // grid: x = inner-dim tile + ltiles * (tile along t), y = index along the inner outer dim, z = index along the outer one
 // FULL: K and L are whole numbers of tiles, so no index is clamped and no row or vector is tested against an edge.
-template <class T, int OP, int OM, bool WIDE, bool FULL>
+// NTO: the other input is a row-wise operand that is read exactly once: non-temporal loads (a compile-time choice, see load_raw).
+template <class T, int OP, int OM, bool WIDE, bool FULL, bool NTO>
 __global__ __launch_bounds__((StageGeom<T, WIDE>::kBlock)) void bin_stage_kernel(const T* xt, const T* xo, T* d, StageArgs a, int32_t* fault) {
     constexpr int N = 16 / sizeof(T);
     constexpr int kSRows = StageGeom<T, WIDE>::kRows, kSWaves = StageGeom<T, WIDE>::kWaves, kSBlock = StageGeom<T, WIDE>::kBlock;
@@ -298,7 +299,8 @@ __global__ __launch_bounds__((StageGeom<T, WIDE>::kBlock)) void bin_stage_kernel
 #pragma unroll
             for (int i = 0; i < RPL; ++i) {
                 const uint32_t k = FULL ? k0 + wv * RPL + i : min(k0 + wv * RPL + i, K - 1);
-                ov[i] = load_vec<T, OM>(xo + (int32_t)k * ts1, c, is1);
+                if constexpr (OM == M_VEC && NTO) ov[i] = __builtin_bit_cast(Vec16<T>, rt_ld16u<T, true>(xo + (int32_t)k * ts1 + c));
+                else ov[i] = load_vec<T, OM>(xo + (int32_t)k * ts1, c, is1);
             }
         }
     }
@@ -440,14 +442,17 @@ bool tile_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* l, const 
                 T* dp = d + dsc.offset[2];
                 dim3 grid((unsigned)gx, (unsigned)n0, (unsigned)n1), blk(kSBlock);
                 const bool full = a.K % kSRows == 0 && a.L % (kSVecs * (uint32_t)N) == 0;
+                bool other_once = om == M_VEC;
+                for (int k = 0; k < rank; ++k) other_once = other_once && dsc.stride[o][k] != 0;
                 auto go = [&](auto wide_c, auto full_c) {
                     constexpr bool W = decltype(wide_c)::value, F = decltype(full_c)::value;
                     if constexpr (OP == kOpCopy) {
-                        hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_BCAST, W, F>), grid, blk, 0, ctx->stream, xp, op, dp, a, fault_of<T, OP>(ctx));
+                        hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_BCAST, W, F, false>), grid, blk, 0, ctx->stream, xp, op, dp, a, fault_of<T, OP>(ctx));
                     } else {
-                        if (om == M_VEC) hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_VEC, W, F>), grid, blk, 0, ctx->stream, xp, op, dp, a, fault_of<T, OP>(ctx));
-                        else if (om == M_BCAST) hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_BCAST, W, F>), grid, blk, 0, ctx->stream, xp, op, dp, a, fault_of<T, OP>(ctx));
-                        else hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_ELEM, W, F>), grid, blk, 0, ctx->stream, xp, op, dp, a, fault_of<T, OP>(ctx));
+                        if (om == M_VEC && other_once) hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_VEC, W, F, true>), grid, blk, 0, ctx->stream, xp, op, dp, a, fault_of<T, OP>(ctx));
+                        else if (om == M_VEC) hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_VEC, W, F, false>), grid, blk, 0, ctx->stream, xp, op, dp, a, fault_of<T, OP>(ctx));
+                        else if (om == M_BCAST) hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_BCAST, W, F, false>), grid, blk, 0, ctx->stream, xp, op, dp, a, fault_of<T, OP>(ctx));
+                        else hipLaunchKernelGGL((bin_stage_kernel<T, OP, M_ELEM, W, F, false>), grid, blk, 0, ctx->stream, xp, op, dp, a, fault_of<T, OP>(ctx));
                     }
                 };
                 auto go_w = [&](auto wide_c) { if (full) go(wide_c, std::true_type{}); else go(wide_c, std::false_type{}); };
