@@ -396,8 +396,10 @@ bool tile_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* l, const 
         om = is == 0 ? (int)M_BCAST : (is == 1 ? (int)M_VEC : (int)M_ELEM);
     }
     // 4- and 8-byte elements whose transposed input can be read with aligned 16-byte vectors along dim t: the staged kernel, also
-    // when that input does not move along some dim
-    if constexpr (sizeof(T) == 4 || sizeof(T) == 8) {
+    // when that input does not move along some dim.  2-byte elements only in that last case, where the input is re-read from cache
+    // (config 3b at i16: 0.62 -> 0.74 of peak); when it is streamed once the tile kernel below is faster for them (16384^2 i16
+    // a + b.transpose(): 0.68 against 0.54), as it is for 1-byte elements in both cases.
+    if constexpr (sizeof(T) >= 2) {
         const T* xbase = (xt == 0 ? l : r) + dsc.offset[xt];
         const int64_t ts = dsc.stride[xt][tdim];
         const T* first = ts > 0 ? xbase : xbase - (N - 1);
@@ -407,6 +409,7 @@ bool tile_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* l, const 
             if (k != tdim) ok = ok && mult_of(dsc.stride[xt][k], N);
             xstream = xstream && dsc.stride[xt][k] != 0;
         }
+        if (sizeof(T) == 2 && xstream) ok = false;
         for (int q = 0; q < 3 && ok; ++q) {                       // 32-bit offsets inside every operand
             uint64_t reach = 0;
             for (int k = 0; k < rank; ++k) reach += (uint64_t)(dsc.shape[k] - 1) * (uint64_t)(dsc.stride[q][k] < 0 ? -dsc.stride[q][k] : dsc.stride[q][k]);
@@ -514,6 +517,7 @@ bool tile_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* l, const 
             if (k != tdim) ok = ok && mult_of(dsc.stride[xt][k], N);
             xstream = xstream && dsc.stride[xt][k] != 0;
         }
+        if (sizeof(T) == 2 && xstream) ok = false;
         vec_gather = ok;
         a.nt_xt = xstream ? 1u : 0u;
     }

@@ -1064,6 +1064,13 @@ def test_broadcast_with_transposed_operand(hip, dtype):
                 g1, g2 = getattr(gxv, f)(gy), getattr(gy, f)(gxv)
                 assert g1.dump().tobytes() == w1.buf.tobytes(), (dtype, shape, variant, op, "x op y")
                 assert g2.dump().tobytes() == w2.buf.tobytes(), (dtype, shape, variant, op, "y op x")
+            if r <= 3 and variant < 2:                         # the transposed operand itself repeats along a new leading dim
+                s3 = [9] + list(oxv.meta.shape)
+                v3 = rand_values(dtype, int(np.prod(s3)), rng)
+                o3, g3 = OTensor.from_buf(dtype, v3, s3), G(hip, dtype, v3, s3)
+                with np.errstate(all="ignore"):
+                    w3 = o3 - oxv
+                assert (g3 - gxv).dump().tobytes() == w3.buf.tobytes(), (dtype, shape, variant, "repeated transposed operand")
             if sy == list(oxv.meta.shape):                     # in place: y (contiguous) += transposed x
                 oy += oxv; gy += gxv
                 assert gy.dump().tobytes() == oy.buf.tobytes(), (dtype, shape, variant, "inplace")
