@@ -183,10 +183,11 @@ __global__ __launch_bounds__(256) void bin_rows4_kernel(const T* l, const T* r, 
     const T* lp = l + (i1 * q0 + i0 * p0 + (int32_t)g * g0);
     const T* rp = r + (i1 * q1 + i0 * p1 + (int32_t)g * g1);
     T* dp = d + (i1 * q2 + i0 * p2 + (int32_t)g * g2);
-    // the lane's vector sits on the 16-byte grid of dst's memory whatever the phase of the row; the inputs follow at element alignment
-    const uint32_t phase = (uint32_t)((reinterpret_cast<uintptr_t>(dp) / sizeof(T)) & (uintptr_t)(N - 1));
+    // a wave's vectors sit on the 128-byte line grid of dst's memory whatever the start of the row (see rt_row_tiling); the inputs
+    // follow at element alignment
+    const uint32_t phase = (uint32_t)((reinterpret_cast<uintptr_t>(dp) / sizeof(T)) & (uintptr_t)(128 / sizeof(T) - 1));
     const int32_t c = (int32_t)((tile * 64 + (threadIdx.x & 63)) * N) - (int32_t)phase;
-    if (c >= (int32_t)L) return;
+    if (c >= (int32_t)L || c + (int32_t)N <= 0) return;
     if (c >= 0 && (uint32_t)c + N <= L) {
         rt_u32x4 x, y;
         if constexpr (LM == M_VEC && (NTM & 1)) x = rt_ld16u<T, true>(lp + c); else x = load_raw<T, LM>(lp, (uint32_t)c, 1);
@@ -640,14 +641,11 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
             memset(&q, 0, sizeof(q));
             q.L = (uint32_t)dsc.shape[rank - 1];
             q.G = a.G;
-            // room for the largest phase a dst row can have: the base's own when every row starts a whole number of vectors from it
-            uint32_t max_phase = (uint32_t)((reinterpret_cast<uintptr_t>(d + dsc.offset[2]) / sizeof(T)) & (uintptr_t)(N - 1));
-            for (int k = 0; k < rank - 1; ++k)
-                if (dsc.stride[2][k] % N != 0) max_phase = (uint32_t)N - 1;
-            q.tiles = (uint32_t)(((q.L + max_phase + N - 1) / N + 63) / 64);
+            const RowTiling rt = rt_row_tiling(reinterpret_cast<uintptr_t>(d + dsc.offset[2]) / sizeof(T), dsc.stride[2], rank - 1, q.L, (uint32_t)sizeof(T));
+            q.tiles = rt.tiles;
             // rows with ragged ends: an odd number of tiles, so that the long-lived waves at the ends of the rows do not keep landing
             // on the same XCDs (see the in-place row kernel): m[:, 1:] += row on 65536 x 4096 f32 0.58 -> 0.8 of peak
-            if ((max_phase != 0 || q.L % N != 0) && q.tiles >= 2 && q.tiles % 2 == 0) q.tiles += 1;
+            if (rt.ragged && q.tiles >= 2 && q.tiles % 2 == 0) q.tiles += 1;
             q.tiles_div = make_fastdiv(q.tiles);
             const uint64_t gx = (uint64_t)q.tiles * ((a.G + 3) / 4);
             if (fits && n0 <= 65535 && n1 <= 65535 && gx < (1ull << 31)) {

@@ -118,6 +118,27 @@ inline bool rt_spans_meet(ByteSpan a, ByteSpan b) { return a.lo < b.hi && b.lo <
 bool rt_same_view(const void* a, uint64_t a_offset, const int64_t* a_strides, const void* b, uint64_t b_offset, const int64_t* b_strides,
                   int rank, const uint64_t* shape);
 
+// The one-wave-per-row kernels (ew_rows4_kernel, bin_rows4_kernel) put a wave's 64 vectors on the 128-byte line grid of memory: the
+// lane's column is moved back by the row's phase, the distance in elements from the line boundary at or below the row's first element,
+// so that a wave writes eight whole lines whatever the row's start.  Tiles of 64 vectors a row needs for the largest phase its rows can
+// have, and whether rows have ends that do not fill a 16-byte vector.  `first` = address of the view's first element in elements;
+// `strides` = the strides of the dims outside the row.
+struct RowTiling { uint32_t tiles; bool ragged; };
+inline RowTiling rt_row_tiling(uint64_t first, const int64_t* strides, int nstrides, uint32_t L, uint32_t esize) {
+    const uint32_t N = 16 / esize, LN = 128 / esize;
+    bool line_uniform = true, vec_uniform = true;
+    for (int k = 0; k < nstrides; ++k) {
+        if (strides[k] % (int64_t)LN != 0) line_uniform = false;
+        if (strides[k] % (int64_t)N != 0) vec_uniform = false;
+    }
+    const uint32_t vphase = (uint32_t)(first % N);
+    const uint32_t max_phase = line_uniform ? (uint32_t)(first % LN) : (vec_uniform ? LN - N + vphase : LN - 1);
+    RowTiling t;
+    t.tiles = (uint32_t)((((uint64_t)L + max_phase + N - 1) / N + 63) / 64);
+    t.ragged = !vec_uniform || vphase != 0 || (vphase + L) % N != 0;
+    return t;
+}
+
 // Launches whose index arithmetic is 32-bit take fewer than 2^31 elements.  A larger N-d descriptor is cut along its outermost dim into
 // slices below that bound (`fn(sub, count_of_sub)` is called for each, in order); when one index of that dim alone is too large the
 // dim is dropped and every index becomes a descriptor of its own, to be cut further by the callee.  Returns the first non-zero status.

@@ -399,10 +399,13 @@ struct Rows4Args {
     int32_t gs, o0s, o1s;           // strides along the row dim and the two outer dims (inner one first)
 };
 
-// Vectors sit on the 16-byte grid of memory whatever the phase of the row: the lane's column is shifted back by the row's phase, the
-// up to N - 1 elements before the first whole vector and after the last one are handled one by one.  (Vectors at element alignment
+// A wave's 64 vectors sit on the 128-byte line grid of memory whatever the start of the row: the lane's column is shifted back by the
+// row's phase (its distance from the line boundary below it, see rt_row_tiling), lanes wholly before the row do nothing, and the up
+// to N - 1 elements before the first whole vector and after the last one are handled one by one.  (Vectors at element alignment
 // cost `m[:, 1:]` of a 65536 x 4096 f32 matrix 0.72 of peak with cached and 0.63 with non-temporal accesses; 0.83 so, all accesses
-// non-temporal.  A fill of all but three columns of that matrix: 0.51 -> 0.76.)
+// non-temporal.  A fill of all but three columns of that matrix: 0.51 -> 0.76.  On the 16-byte grid only, a wave of a row that
+// starts 16 or 32 bytes into a line shares its first and last line with its neighbours: relu on m[:, 4:C-4] of that matrix 0.70
+// against 0.85 on the line grid, on m[:, 1:] of 65536 x 4095, where every row has its own phase, 0.65 against 0.81.)
 template <class T, class F>
 __global__ __launch_bounds__(256) void ew_rows4_kernel(T* p, Rows4Args a, F f) {
     constexpr int N = 16 / sizeof(T);
@@ -415,9 +418,9 @@ __global__ __launch_bounds__(256) void ew_rows4_kernel(T* p, Rows4Args a, F f) {
     const uint32_t g = chunk * 4 + (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     if (g >= G) return;
     T* rowp = p + ((int32_t)blockIdx.z * o1 + (int32_t)blockIdx.y * o0 + (int32_t)g * gs);
-    const uint32_t phase = (uint32_t)((reinterpret_cast<uintptr_t>(rowp) / sizeof(T)) & (uintptr_t)(N - 1));
+    const uint32_t phase = (uint32_t)((reinterpret_cast<uintptr_t>(rowp) / sizeof(T)) & (uintptr_t)(128 / sizeof(T) - 1));
     const int32_t c = (int32_t)((tile * 64 + (threadIdx.x & 63)) * N) - (int32_t)phase;
-    if (c >= (int32_t)L) return;
+    if (c >= (int32_t)L || c + (int32_t)N <= 0) return;
     if (c >= 0 && (uint32_t)c + N <= L) {
         Vec16<T>* vp = reinterpret_cast<Vec16<T>*>(rowp + c);
         Vec16<T> e = {};
@@ -604,18 +607,15 @@ int32_t launch_view(rt_ctx* ctx, T* base, const NdDesc& d, uint64_t count, F f) 
             const uint64_t n0 = d.rank >= 3 ? (uint64_t)d.shape[d.rank - 3] : 1ull, n1 = d.rank >= 4 ? (uint64_t)d.shape[d.rank - 4] : 1ull;
             Rows4Args q;
             q.L = r.L; q.G = r.G;
-            // room for the largest phase a row can have: the base's own when every row starts a whole number of vectors from it
-            uint32_t max_phase = (uint32_t)((reinterpret_cast<uintptr_t>(p) / sizeof(T)) & (uintptr_t)(N - 1));
-            for (int k = 0; k < d.rank - 1; ++k)
-                if (d.stride[0][k] % N != 0) max_phase = (uint32_t)N - 1;
-            q.tiles = (uint32_t)(((r.L + max_phase + N - 1) / N + 63) / 64);
+            const RowTiling rt = rt_row_tiling(reinterpret_cast<uintptr_t>(p) / sizeof(T), d.stride[0], d.rank - 1, r.L, (uint32_t)sizeof(T));
+            q.tiles = rt.tiles;
             // Rows with ragged ends that are read and written: an odd number of tiles per row.  Blocks go to the eight XCDs in turn, so
             // with an even count the first tile of every row -- whose first lane handles the row's ragged start element by element, the
             // longest-lived wave of the row -- keeps landing on the same few XCDs, and the last tile on others.  One more (empty) tile
             // makes the assignment drift: relu on m[:, 1:] of 65536 x 4096 f32 0.70 -> 0.84 of peak, of 8192 x 32768 0.82 -> 0.85, of
             // 262144 x 1024 0.66 -> 0.76, of 524288 x 512 0.70 -> 0.76.  Rotating the tile index instead was slower for long rows, and fills (no loads, nothing
             // long-lived) lose 10 % either way and keep the exact count.
-            const bool ragged = max_phase != 0 || r.L % N != 0;
+            const bool ragged = rt.ragged;
             if (F::kReads && ragged && q.tiles % 2 == 0) q.tiles += 1;
             q.tiles_div = make_fastdiv(q.tiles);
             const uint64_t gx = (uint64_t)q.tiles * ((r.G + 3) / 4);
