@@ -600,14 +600,17 @@ int32_t launch_view(rt_ctx* ctx, T* base, const NdDesc& d, uint64_t count, F f) 
         }
         for (int k = r.nouter; k < RT_MAX_RANK; ++k) { r.oshape[k] = 1; r.odiv[k] = make_fastdiv(1); }
         const uint32_t vecs = (uint32_t)((r.L + N - 1) / N);
-        // (rows of one tile, 64 ... 127 vectors, measured level or a little faster on the general kernel below)
-        if (vecs >= 128 && r.G >= 4 && d.rank <= 4) {
+        // The lean kernel takes rows of 128 vectors and more; shorter ones, down to 32 vectors, when they are whole vectors and fill
+        // their tiles to 85 % (rows of one partly filled or ragged tile measured faster on the general kernel below: relu on m[:, 1:]
+        // of 2^20 x 256 f32 0.71 against 0.68, on m[:, :128] 0.74 against 0.68; but on m[:, 16:C-16] of 2^19 x 512 0.64 against 0.81)
+        const RowTiling rt = rt_row_tiling(reinterpret_cast<uintptr_t>(p) / sizeof(T), d.stride[0], d.rank - 1, r.L, (uint32_t)sizeof(T));
+        const bool lean = vecs >= 128 || (vecs >= 32 && !rt.ragged && (uint64_t)vecs * 100 >= (uint64_t)rt.tiles * 64 * 85);
+        if (lean && r.G >= 4 && d.rank <= 4) {
             uint64_t reach = 0;
             for (int k = 0; k < d.rank; ++k) reach += (uint64_t)(d.shape[k] - 1) * (uint64_t)(d.stride[0][k] < 0 ? -d.stride[0][k] : d.stride[0][k]);
             const uint64_t n0 = d.rank >= 3 ? (uint64_t)d.shape[d.rank - 3] : 1ull, n1 = d.rank >= 4 ? (uint64_t)d.shape[d.rank - 4] : 1ull;
             Rows4Args q;
             q.L = r.L; q.G = r.G;
-            const RowTiling rt = rt_row_tiling(reinterpret_cast<uintptr_t>(p) / sizeof(T), d.stride[0], d.rank - 1, r.L, (uint32_t)sizeof(T));
             q.tiles = rt.tiles;
             // Rows with ragged ends that are read and written: an odd number of tiles per row.  Blocks go to the eight XCDs in turn, so
             // with an even count the first tile of every row -- whose first lane handles the row's ragged start element by element, the
