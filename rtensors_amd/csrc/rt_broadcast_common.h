@@ -53,7 +53,8 @@ template <int OP, class T> __device__ __forceinline__ T bin_apply(T a, T b, int3
                     return (T)(W)((W)0 - (W)a);
                 }
             }
-            return (T)(a / b);
+            if constexpr (sizeof(T) <= 2) return rt_div_narrow<T>(a, b);
+            else return (T)(a / b);
         }
     }
 }
@@ -71,6 +72,21 @@ template <int OP, class T> __device__ __forceinline__ void bin_apply_vec(Vec16<T
             else a.w[j] = OP == RT_ADD ? rt_add_4x8(a.w[j], b.w[j]) : rt_sub_4x8(a.w[j], b.w[j]);
         }
         x = __builtin_bit_cast(Vec16<T>, a);
+    } else if constexpr (OP == RT_DIV && std::is_integral<T>::value && sizeof(T) == 2) {
+        // 16-bit division without a branch per element, so that the eight quotients of a vector are computed side by side: a zero
+        // divisor is replaced by 1 and its result selected afterwards, the fault word is written once per vector.  (Measured on the
+        // config-3 shapes: i16 0.37 -> 0.48 of peak against a branch per element, u16 level; 1-byte and 32-bit elements lose.)
+        bool bad = false;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const T a = x.e[j], b = y.e[j];
+            const bool zero = b == (T)0;
+            const int32_t q = rt_div_narrow_wide<T>(a, zero ? (T)1 : b);
+            bad |= zero;
+            if constexpr (std::is_signed<T>::value) bad |= q > (int32_t)std::numeric_limits<T>::max();      // MIN / -1
+            x.e[j] = zero ? (T)0 : (T)q;
+        }
+        if (bad && fault) *fault = 1;
     } else {
 #pragma unroll
         for (int j = 0; j < (int)(16 / sizeof(T)); ++j) x.e[j] = bin_apply<OP, T>(x.e[j], y.e[j], fault);

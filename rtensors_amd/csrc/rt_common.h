@@ -3,6 +3,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 #include <stdarg.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -258,6 +259,23 @@ template <class V> __device__ __forceinline__ V rt_ld16_dyn(const V* p, bool nt)
     }
     return rt_ld16(p);
 }
+
+// Truncating division of integers of at most 16 bits through the float unit (the compiler's 32-bit integer expansion is about three
+// times as long).  With |a|, |b| < 2^16 the value (|a| + 0.5) / |b| lies at least 0.5 / |b| away from every integer, while
+// (|a| + 0.5) * rcp(|b|) is off by less than 0.02 / |b| (the reciprocal to one ulp, the product to half an ulp, of a value below
+// 2^16 / |b|): truncating it gives the exact quotient.  Signed operands keep their signs through the float arithmetic (the half is
+// given the dividend's sign, the conversion truncates toward zero).  b != 0.  Returns the quotient before narrowing: MIN / -1 is the
+// one pair whose quotient does not fit T.
+template <class T> __device__ __forceinline__ int32_t rt_div_narrow_wide(T a, T b) {
+    static_assert(sizeof(T) <= 2, "operands below 2^16 in magnitude");
+    if constexpr (std::is_signed<T>::value) {
+        const float fa = (float)(int32_t)a;
+        return (int32_t)((fa + __builtin_copysignf(0.5f, fa)) * __builtin_amdgcn_rcpf((float)(int32_t)b));
+    } else {
+        return (int32_t)(uint32_t)(((float)(uint32_t)a + 0.5f) * __builtin_amdgcn_rcpf((float)(uint32_t)b));
+    }
+}
+template <class T> __device__ __forceinline__ T rt_div_narrow(T a, T b) { return (T)rt_div_narrow_wide<T>(a, b); }
 
 // Four 1-byte integers packed in a 32-bit word, wrapping add / subtract of every byte at once: the low seven bits are
 // combined with the top bits masked so that no carry or borrow crosses a byte, then the top bits are restored by xor.

@@ -53,10 +53,12 @@ template <class T> __device__ __forceinline__ T w_div(T a, T b) {
     else if constexpr (is_sint<T>::value) {
         if (b == 0) return 0;
         if (b == (T)-1) return w_sub<T>((T)0, a);
-        return (T)(a / b);
+        if constexpr (sizeof(T) <= 2) return rt_div_narrow<T>(a, b);
+        else return (T)(a / b);
     } else {
         if (b == 0) return 0;
-        return (T)(a / b);
+        if constexpr (sizeof(T) <= 2) return rt_div_narrow<T>(a, b);
+        else return (T)(a / b);
     }
 }
 template <class T> __device__ __forceinline__ bool gt0(T x) {

@@ -601,6 +601,45 @@ def test_integer_division_faults(hip, dtype):
         hip.sync()
 
 
+@pytest.mark.parametrize("dtype", ["i16", "u16"])
+def test_16_bit_division_every_dividend_and_every_divisor(hip, dtype):
+    """Integers of at most 16 bits are divided through the float unit (reciprocal, multiply, truncate).  Every dividend against a
+    set of divisors, and every divisor against a set of dividends, must equal the truncating quotient; so must the scalar form.
+    (All 2^32 pairs were checked once when the kernel was written; 8-bit types have every pair in test_one_byte_types_every_pair.)"""
+    npd = cpu.NP_DTYPE[cpu.DTYPE_BY_NAME[dtype]]
+    info = np.iinfo(npd)
+    allv = np.arange(info.min, info.max + 1, dtype=np.int64)
+    picks = [1, 2, 3, 5, 7, 10, 11, 13, 127, 128, 129, 181, 182, 255, 256, 257, 1000, 4681, 21845, 32766, 32767, info.max, info.max - 1]
+    if info.min < 0:
+        picks += [-p for p in picks] + [info.min, info.min + 1]
+    else:
+        picks += [32768, 32769, 43691, 65534]
+    picks = np.array(sorted(set(picks)), dtype=np.int64)
+
+    def trunc_div(a, b):
+        return ((np.abs(a) // np.abs(b)) * np.sign(a) * np.sign(b)).astype(npd)
+    divisors = picks[(picks != 0) & (picks != -1)]
+    for av, bv in ((allv, divisors), (picks, allv[(allv != 0) & (allv != -1)])):
+        a, b = hip.alloc_from_slice(cpu.DTYPE_BY_NAME[dtype], av.astype(npd)), hip.alloc_from_slice(cpu.DTYPE_BY_NAME[dtype], bv.astype(npd))
+        R, C = av.size, bv.size
+        out = hip.alloc_uninit(cpu.DTYPE_BY_NAME[dtype], R * C)
+        hip.broadcast((a, (0, [R, C], [1, 0])), (b, (0, [R, C], [0, 1])), (out, (0, [R, C], [C, 1])), "div")
+        got = hip.dump(out).reshape(R, C)
+        want = trunc_div(av[:, None], bv[None, :])
+        assert got.tobytes() == want.tobytes(), [(int(av[i]), int(bv[j]), int(got[i, j]), int(want[i, j])) for i, j in np.argwhere(got != want)[:3]]
+    keep = allv[allv != info.min] if info.min < 0 else allv
+    if info.min < 0:                                       # a divisor of -1 inside a tensor: every dividend but MIN (which faults)
+        code = cpu.DTYPE_BY_NAME[dtype]
+        a, b = hip.alloc_from_slice(code, keep.astype(npd)), hip.alloc_from_slice(code, np.full(keep.size, -1, dtype=npd))
+        out = hip.alloc_uninit(code, keep.size)
+        hip.broadcast((a, (0, [keep.size], [1])), (b, (0, [keep.size], [1])), (out, (0, [keep.size], [1])), "div")
+        assert hip.dump(out).tobytes() == (-keep).astype(npd).tobytes()
+    for d in divisors[::3]:
+        g = G(hip, dtype, keep.astype(npd), [keep.size])
+        g /= int(d)
+        assert g.dump().tobytes() == trunc_div(keep, np.int64(d)).tobytes(), int(d)
+
+
 @pytest.mark.parametrize("dtype", ["u8", "i8", "i16", "f32", "f64", "bool"])
 def test_broadcast_repeated_row_any_length(hip, dtype):
     """(rows, L) op (L,) for row lengths that are not a whole number of 16-byte vectors, so that vectors of the output straddle the
