@@ -927,13 +927,17 @@ def test_gather_transposed_views(hip, dtype):
     LDS-transpose copy kernel, with ragged tile edges."""
     rng = np.random.default_rng(17)
     for shape in [(64, 257), (3, 40, 70), (2, 5, 33, 130), (4, 17, 1030), (100, 36), (2, 3, 16, 16), (7, 300, 9), (48, 2100), (2, 32, 1040), (160, 520),
-                  (512, 64), (2, 768, 32), (1024, 256)]:                     # whole numbers of tiles once transposed
+                  (512, 64), (2, 768, 32), (1024, 256),                      # whole numbers of tiles once transposed
+                  (6, 300, 64), (3, 5, 272, 48)]:                            # for the rotations below
         r = len(shape)
         vals = rand_values(dtype, int(np.prod(shape)), rng)
         o, g = OTensor.from_buf(dtype, vals, list(shape)), G(hip, dtype, vals, list(shape))
         perms = [list(range(r - 2)) + [r - 1, r - 2]]
         if r >= 3:
             perms.append([r - 1] + list(range(1, r - 1)) + [0])
+            perms.append([r - 1] + list(range(r - 1)))                       # the unit-stride dim becomes the outermost
+        if r >= 4:
+            perms.append([0, r - 1] + list(range(1, r - 1)))                 # ... or lands between the outer dims
         for perm in perms:
             for variant in range(3):
                 ov, gv = o.permute(perm), g.permute(perm)
@@ -1103,6 +1107,15 @@ def test_broadcast_with_transposed_operand(hip, dtype):
                 g1, g2 = getattr(gxv, f)(gy), getattr(gy, f)(gxv)
                 assert g1.dump().tobytes() == w1.buf.tobytes(), (dtype, shape, variant, op, "x op y")
                 assert g2.dump().tobytes() == w2.buf.tobytes(), (dtype, shape, variant, op, "y op x")
+            if variant < 2:                                    # both operands transposed alike (a.transpose() - b.transpose()), and unlike
+                vz = rand_values(dtype, int(np.prod(shape)), rng)
+                oz, gz = OTensor.from_buf(dtype, vz, base_shape).permute(perm), G(hip, dtype, vz, base_shape).permute(perm)
+                ozr, gzr = oz.slice(r - 2, Slice(None, None, -1)), gz.slice(r - 2, Slice(None, None, -1))
+                for (o2, g2, what) in ((oz, gz, "forward"), (ozr, gzr, "reversed")):
+                    with np.errstate(all="ignore"):
+                        w4, w5 = oxv - o2, o2 * oxv
+                    assert (gxv - g2).dump().tobytes() == w4.buf.tobytes(), (dtype, shape, variant, "both transposed, second " + what)
+                    assert (g2 * gxv).dump().tobytes() == w5.buf.tobytes(), (dtype, shape, variant, "both transposed, second " + what)
             if r <= 3 and variant < 2:                         # the transposed operand itself repeats along a new leading dim
                 s3 = [9] + list(oxv.meta.shape)
                 v3 = rand_values(dtype, int(np.prod(s3)), rng)
