@@ -161,6 +161,9 @@ struct Rows4Args {
     uint32_t L, G, tiles;
     FastDiv32 tiles_div;
     int32_t gs[3], o0s[3], o1s[3];       // strides of left, right, dst along the loop dim and the two outer dims (inner one first)
+    // block order for a long repeated row (see the kernel): 0, or tiles per group (a power of two) * chunks of four rows per band
+    uint32_t group, tg_shift, band_blocks, band_chunks;
+    FastDiv32 group_div, band_div;
 };
 
 // grid: x = column tile + tiles * (chunk of four rows), y = index along the inner outer dim, z = index along the outer one.  Every
@@ -170,13 +173,28 @@ struct Rows4Args {
 template <class T, int OP, int LM, int RM, int NTM>
 __global__ __launch_bounds__(256) void bin_rows4_kernel(const T* l, const T* r, T* d, Rows4Args a, int32_t* fault) {
     constexpr int N = 16 / sizeof(T);
-    uint32_t L = a.L, G = a.G, tiles = a.tiles, tm = a.tiles_div.mul, ts = a.tiles_div.shift;
+    uint32_t L = a.L, G = a.G, tiles = a.tiles, tm = a.tiles_div.mul, ts = a.tiles_div.shift, group = a.group, gm = a.group_div.mul, gsh = a.group_div.shift;
     int32_t g0 = a.gs[0], g1 = a.gs[1], g2 = a.gs[2], p0 = a.o0s[0], p1 = a.o0s[1], p2 = a.o0s[2], q0 = a.o1s[0], q1 = a.o1s[1], q2 = a.o1s[2];
-    RT_PIN(L); RT_PIN(G); RT_PIN(tiles); RT_PIN(tm); RT_PIN(ts);
+    RT_PIN(L); RT_PIN(G); RT_PIN(tiles); RT_PIN(tm); RT_PIN(ts); RT_PIN(group); RT_PIN(gm); RT_PIN(gsh);
     RT_PIN(g0); RT_PIN(g1); RT_PIN(g2); RT_PIN(p0); RT_PIN(p1); RT_PIN(p2); RT_PIN(q0); RT_PIN(q1); RT_PIN(q2);
     RT_TOUCH(l); RT_TOUCH(r); RT_TOUCH(d);
-    const uint32_t chunk = (uint32_t)(((uint64_t)__umulhi(blockIdx.x, tm) + blockIdx.x) >> ts);
-    const uint32_t tile = blockIdx.x - chunk * tiles;
+    uint32_t chunk, tile;
+    if (group == 0) {
+        chunk = (uint32_t)(((uint64_t)__umulhi(blockIdx.x, tm) + blockIdx.x) >> ts);
+        tile = blockIdx.x - chunk * tiles;
+    } else {
+        // A row of several MiB that repeats along the loop dim.  The rows are taken in bands of `band_chunks` chunks of four rows;
+        // inside a band, a group of tiles of every chunk before the next group of tiles, so that a piece of the repeated row is used
+        // by all rows of the band while it is in cache.  In plain order the row is streamed from memory once per chunk of four rows.
+        const uint32_t bm = a.band_div.mul, bsh = a.band_div.shift, bb = a.band_blocks, bc = a.band_chunks, tgs = a.tg_shift;
+        const uint32_t band = (uint32_t)(((uint64_t)__umulhi(blockIdx.x, bm) + blockIdx.x) >> bsh);
+        const uint32_t inb = blockIdx.x - band * bb;
+        const uint32_t th = (uint32_t)(((uint64_t)__umulhi(inb, gm) + inb) >> gsh);
+        const uint32_t rem = inb - th * group;
+        chunk = band * bc + (rem >> tgs);
+        tile = (th << tgs) + (rem & ((1u << tgs) - 1));
+        if (tile >= tiles) return;
+    }
     const int32_t i0 = (int32_t)blockIdx.y, i1 = (int32_t)blockIdx.z;
     const uint32_t g = chunk * 4 + (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     if (g >= G) return;
@@ -650,7 +668,32 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
             // on the same XCDs (see the in-place row kernel): m[:, 1:] += row on 65536 x 4096 f32 0.58 -> 0.8 of peak
             if (rt.ragged && q.tiles >= 2 && q.tiles % 2 == 0) q.tiles += 1;
             q.tiles_div = make_fastdiv(q.tiles);
-            const uint64_t gx = (uint64_t)q.tiles * ((a.G + 3) / 4);
+            const uint32_t chunks = (a.G + 3) / 4;
+            uint64_t gx = (uint64_t)q.tiles * chunks;
+            // A row-wise input of more than 4 MiB per row that does not move along the loop dim: bands of 32 rows, groups of 32 tiles
+            // (f32 (64, 2^21) + (1, 2^21): 0.73 -> 0.80 of peak, (16, 2^24) + (1, 2^24): 0.72 -> 0.74).  Shorter rows stay in cache from
+            // one chunk of rows to the next in plain order and lose with any banding: 1.5 MiB rows 0.81 -> 0.76, 4 MiB rows level.
+            bool long_repeated_row = false;
+            for (int o = 0; o < 2; ++o)
+                if ((o == 0 ? lm : rm) == M_VEC && dsc.stride[o][rank - 2] == 0 && (uint64_t)q.L * sizeof(T) > (4u << 20)) long_repeated_row = true;
+            q.group = 0;
+            q.group_div = make_fastdiv(1);
+            q.band_div = make_fastdiv(1);
+            if (long_repeated_row && chunks >= 2) {
+                q.band_chunks = chunks < 8u ? chunks : 8u;
+                q.tg_shift = 5;
+                q.group = q.band_chunks << q.tg_shift;
+                q.group_div = make_fastdiv(q.group);
+                const uint64_t per_band = (uint64_t)((q.tiles + (1u << q.tg_shift) - 1) >> q.tg_shift) * q.group;
+                const uint64_t bands = (chunks + q.band_chunks - 1) / q.band_chunks;
+                if (per_band < (1ull << 31)) {
+                    q.band_blocks = (uint32_t)per_band;
+                    q.band_div = make_fastdiv(q.band_blocks);
+                    gx = per_band * bands;
+                } else {
+                    q.group = 0;
+                }
+            }
             if (fits && n0 <= 65535 && n1 <= 65535 && gx < (1ull << 31)) {
                 for (int o = 0; o < 3; ++o) {
                     q.gs[o] = (int32_t)dsc.stride[o][rank - 2];

@@ -686,6 +686,32 @@ def test_broadcast_inplace_random(hip, dtype):
         assert ga.dump().tobytes() == oa.buf.tobytes(), (trial, ov.meta, sb)
 
 
+@pytest.mark.parametrize("dtype", ["f32", "i16"])
+def test_broadcast_row_of_several_mib_repeated(hip, dtype):
+    """A row-wise operand of more than 4 MiB per row that repeats along the rows: the row kernel walks bands of rows and groups of
+    tiles instead of whole rows (ragged row length, a number of rows that is not a whole number of bands, an outer dim, both operand
+    positions, in place).  Checked against numpy: one IEEE / wrapping operation per element."""
+    rng = np.random.default_rng(77)
+    code = cpu.DTYPE_BY_NAME[dtype]
+    npd = cpu.NP_DTYPE[code]
+    L = (4 << 20) // np.dtype(npd).itemsize + 4099
+    for rows_shape in ([37], [2, 9]):
+        shape = rows_shape + [L]
+        n = int(np.prod(shape))
+        va, vb = rand_values(dtype, n, rng), rand_values(dtype, L, rng)
+        a, b = hip.alloc_from_slice(code, va), hip.alloc_from_slice(code, vb)
+        out = hip.alloc_uninit(code, n)
+        st = [int(np.prod(shape[i + 1:])) for i in range(len(shape))]
+        A, B, O = (a, (0, shape, st)), (b, (0, shape, [0] * len(rows_shape) + [1])), (out, (0, shape, st))
+        with np.errstate(all="ignore"):
+            hip.broadcast(A, B, O, "sub")
+            assert hip.dump(out).tobytes() == (va.reshape(shape) - vb).astype(npd).tobytes(), (dtype, shape, "a - row")
+            hip.broadcast(B, A, O, "sub")
+            assert hip.dump(out).tobytes() == (vb - va.reshape(shape)).astype(npd).tobytes(), (dtype, shape, "row - a")
+            hip.broadcast(A, B, A, "add")
+            assert hip.dump(a).tobytes() == (va.reshape(shape) + vb).astype(npd).tobytes(), (dtype, shape, "a += row")
+
+
 def _tol(dtype, x):
     return {"f32": 1e-5, "f64": 1e-12}[dtype] * float(np.abs(x.astype(np.float64)).sum())
 
