@@ -81,7 +81,14 @@ __device__ __forceinline__ float m_expm1(float x) { return expm1f(x); }
 __device__ __forceinline__ double m_expm1(double x) { return expm1(x); }
 __device__ __forceinline__ float m_log(float x) { return logf(x); }
 __device__ __forceinline__ double m_log(double x) { return log(x); }
-__device__ __forceinline__ float m_log1p(float x) { return log1pf(x); }
+// ln(1 + x) in f32 from the plain logarithm (Kahan): with u = fl(1 + x), ln(u) * x / (u - 1) cancels the rounding of u, a few ulp over
+// the whole range and about twice as fast as the library routine, which left the 1 GiB pass ALU-bound at 0.47 of the memory rate.
+__device__ __forceinline__ float m_log1p(float x) {
+    const float u = 1.0f + x;
+    if (u == 1.0f) return x;                                   // |x| below half an ulp of 1 (keeps -0.0)
+    if (u == __builtin_inff()) return u;
+    return logf(u) * (x / (u - 1.0f));
+}
 __device__ __forceinline__ double m_log1p(double x) { return log1p(x); }
 __device__ __forceinline__ float m_sqrt(float x) { return sqrtf(x); }
 __device__ __forceinline__ double m_sqrt(double x) { return sqrt(x); }
