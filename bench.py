@@ -557,9 +557,10 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--preheat", type=float, default=0.25,
+    ap.add_argument("--preheat", type=float, default=1.5,
                     help="seconds of untimed GPU work during set-up, before the warm-up steps: right after process start the "
-                         "device runs below its steady clocks (the same kernel measures 0.40 ms cold and 0.31 ms after ~50 ms of work)")
+                         "device runs below its steady clocks (the same kernel measures 0.40 ms cold and 0.31 ms after ~50 ms of work; "
+                         "on some machines the axis sum was still 4 %% slower a quarter of a second in than a few seconds later)")
     ap.add_argument("--kernel", type=str, default=None, help="run only this kernel (see DETAIL) --steps times")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-detail", action="store_true")
