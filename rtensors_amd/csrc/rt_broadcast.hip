@@ -160,14 +160,16 @@ __global__ __launch_bounds__(256) void bin_rows_kernel(const T* l, const T* r, T
 struct Rows4Args {
     uint32_t L, G, tiles;
     FastDiv32 tiles_div;
-    int32_t gs[3], o0s[3], o1s[3];       // strides of left, right, dst along the loop dim and the two outer dims (inner one first)
+    int32_t gs[3], o0s[3], o1s[3], o2s[3];   // strides of left, right, dst along the loop dim and the three outer dims (inner one first)
+    FastDiv32 n1_div;                    // grid z = index along the second outer dim + its extent n1 * index along the third
+    uint32_t n1;
     // block order for a long repeated row (see the kernel): 0, or tiles per group (a power of two) * chunks of four rows per band
     uint32_t group, tg_shift, band_blocks, band_chunks;
     FastDiv32 group_div, band_div;
 };
 
-// grid: x = column tile + tiles * (chunk of four rows), y = index along the inner outer dim, z = index along the outer one.  Every
-// offset inside an operand fits 32 bits (checked on the host).
+// grid: x = column tile + tiles * (chunk of four rows), y = index along the inner outer dim, z = the indices along the next two outer
+// dims folded into one.  Every offset inside an operand fits 32 bits (checked on the host).
 // NTM: bit 0 / 1 = the left / right input is a row-wise operand that is read exactly once (no stride-0 dim): non-temporal loads.  A
 // compile-time choice: two loads that differ only in the hint are merged by the compiler, and the hint is lost.
 template <class T, int OP, int LM, int RM, int NTM>
@@ -175,6 +177,9 @@ __global__ __launch_bounds__(256) void bin_rows4_kernel(const T* l, const T* r, 
     constexpr int N = 16 / sizeof(T);
     uint32_t L = a.L, G = a.G, tiles = a.tiles, tm = a.tiles_div.mul, ts = a.tiles_div.shift, group = a.group, gm = a.group_div.mul, gsh = a.group_div.shift;
     int32_t g0 = a.gs[0], g1 = a.gs[1], g2 = a.gs[2], p0 = a.o0s[0], p1 = a.o0s[1], p2 = a.o0s[2], q0 = a.o1s[0], q1 = a.o1s[1], q2 = a.o1s[2];
+    int32_t r0 = a.o2s[0], r1 = a.o2s[1], r2 = a.o2s[2];
+    uint32_t n1 = a.n1, nm = a.n1_div.mul, nsh = a.n1_div.shift;
+    RT_PIN(r0); RT_PIN(r1); RT_PIN(r2); RT_PIN(n1); RT_PIN(nm); RT_PIN(nsh);
     RT_PIN(L); RT_PIN(G); RT_PIN(tiles); RT_PIN(tm); RT_PIN(ts); RT_PIN(group); RT_PIN(gm); RT_PIN(gsh);
     RT_PIN(g0); RT_PIN(g1); RT_PIN(g2); RT_PIN(p0); RT_PIN(p1); RT_PIN(p2); RT_PIN(q0); RT_PIN(q1); RT_PIN(q2);
     RT_TOUCH(l); RT_TOUCH(r); RT_TOUCH(d);
@@ -195,12 +200,13 @@ __global__ __launch_bounds__(256) void bin_rows4_kernel(const T* l, const T* r, 
         tile = (th << tgs) + (rem & ((1u << tgs) - 1));
         if (tile >= tiles) return;
     }
-    const int32_t i0 = (int32_t)blockIdx.y, i1 = (int32_t)blockIdx.z;
+    const uint32_t zi2 = (uint32_t)(((uint64_t)__umulhi(blockIdx.z, nm) + blockIdx.z) >> nsh);
+    const int32_t i0 = (int32_t)blockIdx.y, i1 = (int32_t)(blockIdx.z - zi2 * n1), i2 = (int32_t)zi2;
     const uint32_t g = chunk * 4 + (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     if (g >= G) return;
-    const T* lp = l + (i1 * q0 + i0 * p0 + (int32_t)g * g0);
-    const T* rp = r + (i1 * q1 + i0 * p1 + (int32_t)g * g1);
-    T* dp = d + (i1 * q2 + i0 * p2 + (int32_t)g * g2);
+    const T* lp = l + (i2 * r0 + i1 * q0 + i0 * p0 + (int32_t)g * g0);
+    const T* rp = r + (i2 * r1 + i1 * q1 + i0 * p1 + (int32_t)g * g1);
+    T* dp = d + (i2 * r2 + i1 * q2 + i0 * p2 + (int32_t)g * g2);
     // a wave's vectors sit on the 128-byte line grid of dst's memory whatever the start of the row (see rt_row_tiling); the inputs
     // follow at element alignment
     const uint32_t phase = (uint32_t)((reinterpret_cast<uintptr_t>(dp) / sizeof(T)) & (uintptr_t)(128 / sizeof(T) - 1));
@@ -651,7 +657,7 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
         // (m[:, 16:C-16] += row on 2^20 x 256 f32: 0.61 -> 0.73 of peak; rows of one half-filled or ragged tile are faster below)
         const RowTiling rt = rt_row_tiling(reinterpret_cast<uintptr_t>(d + dsc.offset[2]) / sizeof(T), dsc.stride[2], rank - 1, (uint32_t)dsc.shape[rank - 1], (uint32_t)sizeof(T));
         const bool lean = true_vecs >= 64 || (true_vecs >= 32 && !rt.ragged && (uint64_t)true_vecs * 100 >= (uint64_t)rt.tiles * 64 * 85);
-        if (steps == 2 && lean && a.G >= 4 && rank <= 4 && lm != M_ELEM && rm != M_ELEM) {
+        if (steps == 2 && lean && a.G >= 4 && rank <= 5 && lm != M_ELEM && rm != M_ELEM) {
             bool fits = true;
             for (int o = 0; o < 3; ++o) {
                 uint64_t reach = 0;
@@ -659,6 +665,7 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
                 fits = fits && reach < (1ull << 31);
             }
             const uint64_t n0 = rank >= 3 ? (uint64_t)dsc.shape[rank - 3] : 1ull, n1 = rank >= 4 ? (uint64_t)dsc.shape[rank - 4] : 1ull;
+            const uint64_t n2 = rank >= 5 ? (uint64_t)dsc.shape[rank - 5] : 1ull;
             Rows4Args q;
             memset(&q, 0, sizeof(q));
             q.L = (uint32_t)dsc.shape[rank - 1];
@@ -694,8 +701,11 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
                     q.group = 0;
                 }
             }
-            if (fits && n0 <= 65535 && n1 <= 65535 && gx < (1ull << 31)) {
+            if (fits && n0 <= 65535 && n1 * n2 <= 65535 && gx < (1ull << 31)) {
+                q.n1 = (uint32_t)n1;
+                q.n1_div = make_fastdiv(q.n1);
                 for (int o = 0; o < 3; ++o) {
+                    q.o2s[o] = rank >= 5 ? (int32_t)dsc.stride[o][rank - 5] : 0;
                     q.gs[o] = (int32_t)dsc.stride[o][rank - 2];
                     q.o0s[o] = rank >= 3 ? (int32_t)dsc.stride[o][rank - 3] : 0;
                     q.o1s[o] = rank >= 4 ? (int32_t)dsc.stride[o][rank - 4] : 0;
@@ -708,7 +718,7 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
                     for (int k = 0; k < rank; ++k) once = once && dsc.stride[o][k] != 0;
                     if (once) ntm |= 1 << o;
                 }
-                launch_rows4<T, OP>(lm, rm, ntm, dim3((unsigned)gx, (unsigned)n0, (unsigned)n1), s, l + dsc.offset[0], r + dsc.offset[1], d + dsc.offset[2], q, fault_of<T, OP>(ctx));
+                launch_rows4<T, OP>(lm, rm, ntm, dim3((unsigned)gx, (unsigned)n0, (unsigned)(n1 * n2)), s, l + dsc.offset[0], r + dsc.offset[1], d + dsc.offset[2], q, fault_of<T, OP>(ctx));
                 RT_HIP(hipGetLastError());
                 return RT_OK;
             }

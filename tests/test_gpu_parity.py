@@ -745,6 +745,10 @@ def test_broadcast_long_rows(hip, dtype):
         ([6, L + 5], [(1, Slice(2, 2 + L, 1))], [6, 1], []),
         ([3, 5, L + 4], [(2, Slice(3, 3 + L, 1)), (1, Slice(None, None, -1))], [5, L], []),
         ([8, 130 * per_vec + 1], [(1, Slice(1, None, 1))], [8, 130 * per_vec + 1], [(1, Slice(0, 130 * per_vec, 1))]),
+        # five dims that do not merge (the third outer dim is folded into the grid's z)
+        ([2, 3, 2, 5, L], [], [1, 3, 1, 5, 1], []),
+        ([2, 3, 2, 5, L], [(3, Slice(None, None, -1)), (1, Slice(0, None, 2))], [2, 1, 2, 1, L], []),
+        ([3, 1, 2, 1, 64 * per_vec], [], [1, 4, 1, 5, 1], []),
     ]
     for trial, (sa, ca, sb, cb) in enumerate(cases):
         va, vb = rand_values(dtype, int(np.prod(sa)), rng), rand_values(dtype, int(np.prod(sb)), rng)
