@@ -54,6 +54,7 @@ template <int OP, class T> __device__ __forceinline__ T bin_apply(T a, T b, int3
                 }
             }
             if constexpr (sizeof(T) <= 2) return rt_div_narrow<T>(a, b);
+            else if constexpr (sizeof(T) == 4) return rt_div32<T>(a, b);
             else return (T)(a / b);
         }
     }
@@ -85,6 +86,24 @@ template <int OP, class T> __device__ __forceinline__ void bin_apply_vec(Vec16<T
             bad |= zero;
             if constexpr (std::is_signed<T>::value) bad |= q > (int32_t)std::numeric_limits<T>::max();      // MIN / -1
             x.e[j] = zero ? (T)0 : (T)q;
+        }
+        if (bad && fault) *fault = 1;
+    } else if constexpr (OP == RT_DIV && std::is_integral<T>::value && sizeof(T) == 4) {
+        // 32-bit division, likewise without a branch per element
+        bool bad = false;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const T a = x.e[j], b = y.e[j];
+            const bool zero = b == (T)0;
+            const double q = rt_div32_real<T>(a, zero ? (T)1 : b);
+            bad |= zero;
+            if constexpr (std::is_signed<T>::value) {
+                const bool ovf = q >= 2147483648.0;                                                        // MIN / -1
+                bad |= ovf;
+                x.e[j] = zero ? (T)0 : (ovf ? std::numeric_limits<T>::min() : (T)(int32_t)q);
+            } else {
+                x.e[j] = zero ? (T)0 : (T)(uint32_t)q;
+            }
         }
         if (bad && fault) *fault = 1;
     } else {

@@ -277,6 +277,23 @@ template <class T> __device__ __forceinline__ int32_t rt_div_narrow_wide(T a, T 
 }
 template <class T> __device__ __forceinline__ T rt_div_narrow(T a, T b) { return (T)rt_div_narrow_wide<T>(a, b); }
 
+// Truncating division of 32-bit integers through the f64 unit.  r = 1 / b after one Newton step on the hardware reciprocal is good
+// to better than 2^-40; (|a| + 0.5) / |b| lies at least 0.5 / |b| away from every integer and (|a| + 0.5) * r is off by less than
+// 2^32 / |b| * 2^-40, so truncation gives the exact quotient.  b != 0; rt_div32_real returns the biased quotient before truncation (MIN / -1: 2^31 + 0.5, which does not fit).
+template <class T> __device__ __forceinline__ double rt_div32_real(T a, T b) {
+    static_assert(sizeof(T) == 4, "32-bit operands");
+    const double fb = (double)b;
+    double r = __builtin_amdgcn_rcp(fb);
+    r = __builtin_fma(__builtin_fma(-fb, r, 1.0), r, r);
+    const double fa = (double)a;
+    if constexpr (std::is_signed<T>::value) return (fa + __builtin_copysign(0.5, fa)) * r;
+    else return (fa + 0.5) * r;
+}
+template <class T> __device__ __forceinline__ T rt_div32(T a, T b) {
+    if constexpr (std::is_signed<T>::value) return (T)(int32_t)rt_div32_real<T>(a, b);
+    else return (T)(uint32_t)rt_div32_real<T>(a, b);
+}
+
 // Four 1-byte integers packed in a 32-bit word, wrapping add / subtract of every byte at once: the low seven bits are
 // combined with the top bits masked so that no carry or borrow crosses a byte, then the top bits are restored by xor.
 // Per-byte code (sub-dword selects and re-packing) costs about twice the vector instructions per 16-byte vector, enough

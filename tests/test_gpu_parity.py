@@ -640,6 +640,42 @@ def test_16_bit_division_every_dividend_and_every_divisor(hip, dtype):
         assert g.dump().tobytes() == trunc_div(keep, np.int64(d)).tobytes(), int(d)
 
 
+@pytest.mark.parametrize("dtype", ["i32", "u32"])
+def test_32_bit_division_edge_pairs_and_multiples(hip, dtype):
+    """32-bit integers are divided through the f64 unit (reciprocal, one Newton step, multiply, truncate).  What a rounding error
+    would break: dividends at and next to multiples of the divisor, quotients near the type's limits, powers of two and their
+    neighbours -- all pairs of an edge set, and a million structured pairs, against integer arithmetic."""
+    npd = cpu.NP_DTYPE[cpu.DTYPE_BY_NAME[dtype]]
+    code = cpu.DTYPE_BY_NAME[dtype]
+    info = np.iinfo(npd)
+    rng = np.random.default_rng(3232)
+    E = {0, 1, 2, 3, 5, 7, 10, info.max, info.max - 1, info.max // 2, info.max // 2 + 1, info.max // 3, 46340, 46341, 65535, 65536, 65537}
+    for k in range(1, 33):
+        E |= {(1 << k) - 1, 1 << k, (1 << k) + 1}
+    if info.min < 0:
+        E |= {-e for e in E} | {info.min, info.min + 1}
+    E = np.array(sorted(e for e in E if info.min <= e <= info.max), dtype=np.int64)
+    A, B = [m.ravel() for m in np.meshgrid(E, E, indexing="ij")]
+    m = 1 << 20
+    b2 = (rng.integers(0, 1 << 62, size=m, dtype=np.int64) >> (62 - rng.integers(1, 32, size=m))) + 1
+    q2 = (rng.random(m) * np.maximum(info.max // b2, 1)).astype(np.int64)
+    a2 = q2 * b2 + rng.integers(-1, 2, size=m)
+    if info.min < 0:
+        a2 *= rng.choice([-1, 1], size=m); b2 *= rng.choice([-1, 1], size=m)
+    a, b = np.concatenate([A, a2]), np.concatenate([B, b2])
+    keep = (b != 0) & (a >= info.min) & (a <= info.max) & ~((a == info.min) & (b == -1))
+    a, b = a[keep], b[keep]
+    want = ((np.abs(a) // np.abs(b)) * np.sign(a) * np.sign(b)).astype(npd)
+    ga, gb = hip.alloc_from_slice(code, a.astype(npd)), hip.alloc_from_slice(code, b.astype(npd))
+    out = hip.alloc_uninit(code, a.size)
+    hip.broadcast((ga, (0, [a.size], [1])), (gb, (0, [a.size], [1])), (out, (0, [a.size], [1])), "div")     # vector path
+    got = hip.dump(out)
+    assert got.tobytes() == want.tobytes(), [(int(a[i]), int(b[i]), int(got[i]), int(want[i])) for i in np.nonzero(got != want)[0][:3]]
+    n2 = a.size // 2
+    hip.broadcast((ga, (0, [n2], [2])), (gb, (0, [n2], [2])), (out, (0, [n2], [2])), "div")                 # element path
+    assert hip.dump(out)[:2 * n2:2].tobytes() == want[:2 * n2:2].tobytes()
+
+
 @pytest.mark.parametrize("dtype", ["u8", "i8", "i16", "f32", "f64", "bool"])
 def test_broadcast_repeated_row_any_length(hip, dtype):
     """(rows, L) op (L,) for row lengths that are not a whole number of 16-byte vectors, so that vectors of the output straddle the
