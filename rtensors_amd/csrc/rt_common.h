@@ -200,6 +200,7 @@ int32_t rt_collapse_big(rt_ctx* ctx, int nops, int rank, const uint64_t* shape, 
 // A dynamic-LDS size that lets four 256-lane blocks share a CU's 160 KiB of LDS (each block also holds a few hundred bytes of
 // static LDS).  Passed as the launch's dynamic LDS by long streaming reductions to cap their occupancy; the memory is not used.
 constexpr size_t kRtFourBlocksLds = 40000;
+constexpr size_t kRtThreeBlocksLds = 54000;      // likewise, three resident blocks
 
 // 16-byte global accesses.  The non-temporal forms mark data that is touched once (streamed operands, outputs):
 // measured on MI355X they lift a read-modify-write pass from ~5.5 to ~6.7 TB/s and a read-only pass from ~5.5 to

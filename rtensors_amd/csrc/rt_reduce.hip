@@ -142,10 +142,9 @@ template <class T> struct alignas(16) Vec16 { T e[16 / sizeof(T)]; };
 
 // fold elements [begin, end) of the contiguous run `p`, lanes `tid` of `nthreads` cooperating; positions are
 // reported relative to `p`
-template <int OP, class T>
+template <int OP, class T, int U = 4>
 __device__ __forceinline__ void fold_run(Acc<OP, T>& a, const T* __restrict__ p, uint64_t begin, uint64_t end, uint32_t tid, uint32_t nthreads) {
     constexpr uint32_t N = 16 / sizeof(T);
-    constexpr int U = 4;
     if (begin >= end) return;
     // elements before the first 16-byte boundary
     uint64_t head = ((16 - (reinterpret_cast<uintptr_t>(p + begin) & 15)) & 15) / sizeof(T);
@@ -189,7 +188,7 @@ __device__ __forceinline__ void fold_run(Acc<OP, T>& a, const T* __restrict__ p,
 
 // ---- rows -------------------------------------------------------------------------------------------------------------
 // grid.x = rows * splits.  Block b folds segment (b % splits) of row (b / splits); out[b] (stage 1 of 2) or out[row].
-template <int OP, class T>
+template <int OP, class T, int U = 4>
 __global__ __launch_bounds__(kBlock) void reduce_rows_block_kernel(const T* __restrict__ src, T* __restrict__ out, uint64_t R, uint32_t splits,
                                                                    uint64_t seglen, uint64_t count, int last) {
     const uint64_t row = blockIdx.x / splits;
@@ -199,7 +198,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_block_kernel(const T* __re
     if (end > R) end = R;
     Acc<OP, T> a;
     a.init();
-    fold_run<OP, T>(a, src + row * R, begin, end, threadIdx.x, kBlock);
+    fold_run<OP, T, U>(a, src + row * R, begin, end, threadIdx.x, kBlock);
     block_reduce<OP, T>(a);
     if (threadIdx.x == 0) out[blockIdx.x] = last ? finalize<OP, T>(a.v, count) : a.v;
 }
@@ -645,7 +644,15 @@ int32_t rows_stage(rt_ctx* ctx, const T* src, T* out, uint64_t rows, uint64_t R,
     }
     if (rows * splits >= (1ull << 31)) return rt_fail(RT_E_INVALID, "reduce: too many rows for one launch");
     if (splits == 1) {
-        hipLaunchKernelGGL((reduce_rows_block_kernel<OP, T>), dim3((unsigned)rows), dim3(kBlock), kRtFourBlocksLds, s, src, out, R, 1u, R, count, 1);
+        // Rows of 80 ... 256 KiB: eight loads in flight per lane (a trip of the block covers 32 KiB) and three resident blocks per CU
+        // instead of four loads and four blocks -- fewer, fatter streams.  1 GiB, rows of 32768 f32: sum 0.867 -> 0.895 of peak, max
+        // 0.858 -> 0.877; f64 rows of 10000 ... 32768: 0.87 -> 0.89-0.90.  Shorter rows do not fill such trips (rows of 10000 f32:
+        // 0.90 -> 0.77), longer ones lose 1-2 %.
+        const uint64_t row_bytes = R * sizeof(T);
+        if (row_bytes >= 80 * 1024 && row_bytes <= 256 * 1024)
+            hipLaunchKernelGGL((reduce_rows_block_kernel<OP, T, 8>), dim3((unsigned)rows), dim3(kBlock), kRtThreeBlocksLds, s, src, out, R, 1u, R, count, 1);
+        else
+            hipLaunchKernelGGL((reduce_rows_block_kernel<OP, T>), dim3((unsigned)rows), dim3(kBlock), kRtFourBlocksLds, s, src, out, R, 1u, R, count, 1);
         RT_HIP(hipGetLastError());
         return RT_OK;
     }
