@@ -640,6 +640,9 @@ int32_t rows_stage(rt_ctx* ctx, const T* src, T* out, uint64_t rows, uint64_t R,
         uint64_t by_need = (want + rows - 1) / rows;
         uint64_t sp = by_need < by_size ? by_need : by_size;
         if (sp > 4096) sp = 4096;
+        // enough data for `want` segments of 128 KiB: segments of that size, which stream fastest (see below); at most 65536 partials
+        const uint64_t by_fat = (R * sizeof(T) + (128u << 10) - 1) / (128u << 10);
+        if (by_fat > sp && rows * by_fat >= want) sp = rows * by_fat <= 65536 ? by_fat : 65536 / rows;
         if (sp > 1) splits = (uint32_t)sp;
     }
     if (rows * splits >= (1ull << 31)) return rt_fail(RT_E_INVALID, "reduce: too many rows for one launch");
@@ -663,7 +666,10 @@ int32_t rows_stage(rt_ctx* ctx, const T* src, T* out, uint64_t rows, uint64_t R,
     void* scratch = nullptr;
     RT_TRY(rt_scratch(ctx, (size_t)(rows * splits) * sizeof(T), &scratch));
     T* part = (T*)scratch;
-    hipLaunchKernelGGL((reduce_rows_block_kernel<OP, T>), dim3((unsigned)(rows * splits)), dim3(kBlock), kRtFourBlocksLds, s, src, part, R, splits, seglen, count, 0);
+    if (seglen * sizeof(T) >= 80 * 1024 && seglen * sizeof(T) <= 256 * 1024)
+        hipLaunchKernelGGL((reduce_rows_block_kernel<OP, T, 8>), dim3((unsigned)(rows * splits)), dim3(kBlock), kRtThreeBlocksLds, s, src, part, R, splits, seglen, count, 0);
+    else
+        hipLaunchKernelGGL((reduce_rows_block_kernel<OP, T>), dim3((unsigned)(rows * splits)), dim3(kBlock), kRtFourBlocksLds, s, src, part, R, splits, seglen, count, 0);
     RT_HIP(hipGetLastError());
     // second stage: each row of `splits` partials -> one output (mean divides by the original count)
     if (splits < 64) {
