@@ -840,6 +840,31 @@ def test_reduce_random_vs_oracle(hip, dtype, op):
                 assert a.tobytes() == b.tobytes(), (dtype, op, shape, axis)
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f64", "i32"])
+def test_reduce_rows_of_80_to_256_kib_unsplit(hip, dtype):
+    """Rows of 80 ... 256 KiB, enough of them that no row is split: the block-per-row kernel with eight loads in flight per lane.
+    Row lengths that leave 1 ... 7 vectors and a few elements for the last trip, and a contiguous offset view."""
+    rng = np.random.default_rng(zlib.crc32(dtype.encode()) + 80)
+    es = np.dtype(cpu.NP_DTYPE[cpu.DTYPE_BY_NAME[dtype]]).itemsize
+    rows = 2100
+    for R in (81920 // es + 3, 98304 // es + 16 * 256 // es * 3 + 1, 131072 // es):
+        x = rand_values(dtype, rows * R + 5, rng, -100, 100)
+        for offset in (0, 5):
+            o = OTensor.from_buf(dtype, x, [rows * R + 5]).slice(0, Slice(offset, offset + rows * R, 1))
+            g = G(hip, dtype, x, [rows * R + 5]).slice(0, Slice(offset, offset + rows * R, 1))
+            o = OTensor(o.dtype, o.buf, MetaTensor([rows, R], [R, 1], offset), is_view=True)
+            g = type(g)(g.backend, g.buf, MetaTensor([rows, R], [R, 1], offset), is_view=True)
+            for op in ("sum", "max", "min"):
+                want, got = o.reduce(op, 1), g.reduce(op, 1)
+                a, b = got.dump(), want.buf
+                if x.dtype.kind == "f" and op == "sum":
+                    xs = np.abs(x[offset:offset + rows * R].astype(np.float64)).reshape(rows, R).sum(axis=1)
+                    tol = (1e-5 if dtype == "f32" else 1e-12) * xs + 1e-30
+                    assert (np.abs(a.astype(np.float64) - b.astype(np.float64)).reshape(-1) <= tol).all(), (dtype, op, R, offset)
+                else:
+                    assert a.tobytes() == b.tobytes(), (dtype, op, R, offset)
+
+
 def test_reduce_corner_values(hip):
     nan, inf = np.nan, np.inf
     lowest, highest = np.finfo(np.float32).min, np.finfo(np.float32).max
