@@ -1527,6 +1527,9 @@ def test_statistic_reductions_shapes(hip, dtype):
     for R in (2, 4, 8, 16):                                       # aligned starts reach the kernel without staging
         _check_stat(hip, dtype, 30000, R, 1, rng, offset=0)
         _check_stat(hip, dtype, 30000, R, 1, rng, offset=8)
+    # unsplit rows of 80 ... 256 KiB: eight loads in flight per lane for the variance and norm states
+    es = 4 if dtype == "f32" else 8
+    _check_stat(hip, dtype, 2100, 81920 // es + 3, 1, rng, offset=3)
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f64"])
