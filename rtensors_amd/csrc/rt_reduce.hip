@@ -687,16 +687,23 @@ int32_t cols_launch(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t 
     hipStream_t s = ctx->stream;
     const uint64_t per_tile = (uint64_t)RT_WAVE * VW;
     const uint64_t tiles = (inner + per_tile - 1) / per_tile;
-    // Two blocks of four waves per CU, each streaming a long run of rows, measured best on MI355X for every row pitch from
-    // 1 KiB to 256 KiB (1 GiB f32 sum over axis 0: 6.4-6.8 TB/s, against 5.6-6.6 TB/s with eight blocks per CU).
-    // (Loads in flight per lane: 8 against 4 gained 0.5-1 % on the 1 GiB axis-0 sums; 3 or 4 blocks per CU were level or slower.)
-    const uint64_t want = (uint64_t)ctx->num_cus * 2;
+    // One block of four waves per CU, eight loads in flight per lane, each block streaming a long run of rows: the segments are cut so
+    // that the blocks do not outnumber the CUs (1 GiB f32 sums over axis 0, against two blocks per CU: 8192 x 32768 0.857 -> 0.893 of
+    // peak, 26844 x 10000 0.66 -> 0.82, 13422 x 20000 0.74 -> 0.88, 65536 x 4096 0.82 -> 0.83; eight blocks per CU: 0.70-0.83).
+    // When that would leave more than a quarter of the CUs without a block (150 column tiles: 0.60 for a max), two blocks per CU as
+    // before.  Outputs that already give every CU a block are not split.
+    const uint64_t cus = (uint64_t)ctx->num_cus;
     uint32_t splits = 1;
-    if (allow_split && outer * tiles < want) {
+    if (allow_split && outer * tiles < cus) {
         const uint64_t min_seg = 64;                          // k values per block
-        uint64_t by_size = R / min_seg;
-        uint64_t by_need = (want + outer * tiles - 1) / (outer * tiles);
-        uint64_t sp = by_need < by_size ? by_need : by_size;
+        const uint64_t by_size = R / min_seg;
+        uint64_t sp = cus / (outer * tiles);
+        if (sp > by_size) sp = by_size;
+        if (sp < 1) sp = 1;
+        if (outer * tiles * sp * 4 < cus * 3) {
+            const uint64_t by_need = (2 * cus + outer * tiles - 1) / (outer * tiles);
+            sp = by_need < by_size ? by_need : by_size;
+        }
         if (sp > 1024) sp = 1024;
         if (sp > 1) splits = (uint32_t)sp;
     }
@@ -708,8 +715,13 @@ int32_t cols_launch(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t 
     const uint64_t blocks = outer * splits * tiles;
     if (blocks >= (1ull << 31) || tiles >= (1ull << 31)) return rt_fail(RT_E_INVALID, "reduce: too many outputs for one launch");
     if (splits == 1) {
-        hipLaunchKernelGGL((reduce_cols_kernel<OP, T, VW>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, out, R, inner, outer,
-                           (uint32_t)tiles, 1u, seglen, count, 1);
+        // (eight loads in flight per lane from 256 rows on; a short axis would spend its time in the one-row-at-a-time remainder)
+        if (R >= 256)
+            hipLaunchKernelGGL((reduce_cols_kernel<OP, T, VW, 8>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, out, R, inner, outer,
+                               (uint32_t)tiles, 1u, seglen, count, 1);
+        else
+            hipLaunchKernelGGL((reduce_cols_kernel<OP, T, VW>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, out, R, inner, outer,
+                               (uint32_t)tiles, 1u, seglen, count, 1);
         RT_HIP(hipGetLastError());
         return RT_OK;
     }
