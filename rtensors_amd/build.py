@@ -32,7 +32,8 @@ LIBS = {
     "librt_hip.so": ["rt_runtime.hip", "rt_layout.hip", "rt_elementwise.hip", "rt_broadcast.hip", "rt_broadcast_tile.hip", "rt_reduce.hip", "rt_reduce_stat.hip", "rt_misc.hip", "rt_matmul.hip", "rt_fused.hip"],
     "librt_datagen.so": ["rt_datagen.hip"],
 }
-HEADERS = [os.path.join(CSRC, "rt_common.h"), os.path.join(CSRC, "rt_broadcast_common.h"), os.path.join(HERE, "..", "include", "rt_hip.h")]
+HEADERS = [os.path.join(CSRC, "rt_common.h"), os.path.join(CSRC, "rt_broadcast_common.h"), os.path.join(CSRC, "rt_div128.h"),
+           os.path.join(HERE, "..", "include", "rt_hip.h")]
 
 
 def _stale(target: str, deps) -> bool:
@@ -90,7 +91,7 @@ def _build_host(force: bool) -> None:
     host = os.path.join(HERE, "host")
     src = os.path.join(host, "rt_host_capi.cpp")
     out = os.path.join(LIB, "librt_host.so")
-    deps = [src] + [os.path.join(host, h) for h in ("rt_meta.hpp", "rt_backend.hpp", "rt_tensor.hpp", "rt_grad.hpp")] + HEADERS[2:]
+    deps = [src] + [os.path.join(host, h) for h in ("rt_meta.hpp", "rt_backend.hpp", "rt_tensor.hpp", "rt_grad.hpp")] + HEADERS[3:]
     if force or _stale(out, deps + [os.path.join(LIB, "librt_hip.so")]):
         cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra", "-o", out, src, "-L" + LIB, "-lrt_hip", "-Wl,-rpath,$ORIGIN"]
         r = subprocess.run(cmd, capture_output=True, text=True)

@@ -810,9 +810,11 @@ int32_t with_type_op(int dtype, int op, Fn&& fn) {
             case RT_I64: return fn(type_tag<int64_t>{}, D{});
             case RT_F32: return fn(type_tag<float>{}, D{});
             case RT_F64: return fn(type_tag<double>{}, D{});
+            case RT_U128: return fn(type_tag<u128_t>{}, D{});
+            case RT_I128: return fn(type_tag<i128_t>{}, D{});
             case RT_BOOL: return rt_fail(RT_E_ARITH, "broadcast: division is not implemented for boolean in the reference (todo!())");
         }
-        return rt_fail(RT_E_DTYPE, "broadcast: 128-bit integer division is not built for the device");
+        return rt_fail(RT_E_DTYPE, "broadcast: unknown dtype code %d", dtype);
     }
     auto ops = [&](auto t) -> int32_t {
         switch (op) {

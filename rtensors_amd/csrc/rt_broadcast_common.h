@@ -3,6 +3,7 @@
 #pragma once
 
 #include "rt_common.h"
+#include "rt_div128.h"
 
 #include <limits>
 #include <type_traits>
@@ -14,7 +15,10 @@ template <class T> struct is_flt : std::integral_constant<bool, std::is_same<T, 
 template <class T> struct is_bool : std::is_same<T, boolean_t> {};
 
 typedef unsigned __int128 u128_t;
+typedef __int128 i128_t;              // only division tells the two 128-bit types apart; + - * run on u128_t
+template <class T> struct is_int128 : std::integral_constant<bool, std::is_same<T, u128_t>::value || std::is_same<T, i128_t>::value> {};
 template <class T, class E = void> struct carrier { typedef T type; };
+template <> struct carrier<i128_t, void> { typedef u128_t type; };
 template <class T> struct carrier<T, typename std::enable_if<std::is_integral<T>::value && sizeof(T) <= 4>::type> { typedef uint32_t type; };
 template <class T> struct carrier<T, typename std::enable_if<std::is_integral<T>::value && sizeof(T) == 8>::type> { typedef uint64_t type; };
 
@@ -42,7 +46,19 @@ template <int OP, class T> __device__ __forceinline__ T bin_apply(T a, T b, int3
         if constexpr (OP == RT_ADD) return (T)(W)((W)a + (W)b);
         else if constexpr (OP == RT_SUB) return (T)(W)((W)a - (W)b);
         else if constexpr (OP == RT_MUL) return (T)(W)((W)a * (W)b);
-        else {
+        else if constexpr (is_int128<T>::value) {
+            // hand-written long division (rt_div128.h); MIN / -1 wraps to MIN there
+            if (b == 0) {
+                if (fault) *fault = 1;
+                return (T)0;
+            }
+            if constexpr (std::is_same<T, i128_t>::value) {
+                if (b == (T)-1 && a == (T)((u128_t)1 << 127) && fault) *fault = 1;
+                return rt_idiv128(a, b);
+            } else {
+                return rt_udiv128(a, b);
+            }
+        } else {
             if (b == 0) {
                 if (fault) *fault = 1;
                 return (T)0;
@@ -115,7 +131,7 @@ template <int OP, class T> __device__ __forceinline__ void bin_apply_vec(Vec16<T
 // The fault word of the context for a launch that can raise an integer-division fault (and a note for the host to look at it at
 // the next synchronising call); null for every other launch.
 template <class T, int OP> static inline int32_t* fault_of(rt_ctx* ctx) {
-    if constexpr (OP == RT_DIV && std::is_integral<T>::value) {
+    if constexpr (OP == RT_DIV && (std::is_integral<T>::value || is_int128<T>::value)) {
         ctx->fault_pending = true;
         return ctx->fault_dev;
     } else {

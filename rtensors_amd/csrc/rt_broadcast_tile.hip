@@ -727,7 +727,7 @@ RT_TILE_INST_ASM(uint8_t) RT_TILE_INST_ASM(uint16_t) RT_TILE_INST_ASM(uint32_t) 
 RT_TILE_INST_ASM(float) RT_TILE_INST_ASM(double) RT_TILE_INST_ASM(boolean_t) RT_TILE_INST_ASM(u128_t)
 RT_TILE_INST(uint8_t, RT_DIV) RT_TILE_INST(int8_t, RT_DIV) RT_TILE_INST(uint16_t, RT_DIV) RT_TILE_INST(int16_t, RT_DIV)
 RT_TILE_INST(uint32_t, RT_DIV) RT_TILE_INST(int32_t, RT_DIV) RT_TILE_INST(uint64_t, RT_DIV) RT_TILE_INST(int64_t, RT_DIV)
-RT_TILE_INST(float, RT_DIV) RT_TILE_INST(double, RT_DIV)
+RT_TILE_INST(float, RT_DIV) RT_TILE_INST(double, RT_DIV) RT_TILE_INST(u128_t, RT_DIV) RT_TILE_INST(i128_t, RT_DIV)
 RT_TILE_INST(uint8_t, kOpCopy) RT_TILE_INST(uint16_t, kOpCopy) RT_TILE_INST(uint32_t, kOpCopy) RT_TILE_INST(uint64_t, kOpCopy)
 
 }  // namespace rtb

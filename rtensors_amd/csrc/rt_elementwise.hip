@@ -7,6 +7,7 @@
 // wavefront touching 1 KiB of consecutive addresses, in many small blocks.  Algorithmic traffic is 2*N*sizeof(T) for
 // read-modify-write ops and N*sizeof(T) for fill.
 #include "rt_common.h"
+#include "rt_div128.h"
 
 #include <type_traits>
 
@@ -17,7 +18,7 @@ struct boolean_t { uint8_t v; };      // core/value.rs:650-765: + is OR, - is XO
 
 template <class T> struct is_flt : std::integral_constant<bool, std::is_same<T, float>::value || std::is_same<T, double>::value> {};
 template <class T> struct is_bool : std::is_same<T, boolean_t> {};
-typedef unsigned __int128 u128_t;      // core/value.rs: u128 / i128 (no division on the device: there is no 128-bit divide routine)
+typedef unsigned __int128 u128_t;      // core/value.rs: u128 / i128 (division by hand, rt_div128.h)
 typedef __int128 i128_t;
 template <class T> struct is_sint : std::integral_constant<bool, (std::is_integral<T>::value && std::is_signed<T>::value) || std::is_same<T, i128_t>::value> {};
 template <class T> struct is_uint : std::integral_constant<bool, (std::is_integral<T>::value && std::is_unsigned<T>::value) || std::is_same<T, u128_t>::value> {};
@@ -49,8 +50,11 @@ template <class T> __device__ __forceinline__ T w_mul(T a, T b) {
 template <class T> __device__ __forceinline__ T w_div(T a, T b) {
     if constexpr (is_flt<T>::value) return a / b;
     else if constexpr (is_bool<T>::value) return boolean_t{0};
-    else if constexpr (sizeof(T) == 16) return (T)0;                      // refused on the host
-    else if constexpr (is_sint<T>::value) {
+    else if constexpr (sizeof(T) == 16) {
+        if (b == 0) return 0;
+        if constexpr (is_sint<T>::value) return rt_idiv128(a, b);         // MIN / -1 wraps to MIN
+        else return rt_udiv128(a, b);
+    } else if constexpr (is_sint<T>::value) {
         if (b == 0) return 0;
         if (b == (T)-1) return w_sub<T>((T)0, a);
         if constexpr (sizeof(T) <= 2) return rt_div_narrow<T>(a, b);
@@ -68,6 +72,10 @@ template <class T> __device__ __forceinline__ bool gt0(T x) {
 template <class T> __device__ __forceinline__ T zero_of() {
     if constexpr (is_bool<T>::value) return boolean_t{0};
     else return (T)0;
+}
+template <class T> __device__ __forceinline__ T min_of() {                // signed integers
+    typedef typename carrier<T>::type W;
+    return (T)((W)1 << (sizeof(T) * 8 - 1));
 }
 template <class T> __device__ __forceinline__ T one_of() {
     if constexpr (is_bool<T>::value) return boolean_t{1};
@@ -198,8 +206,8 @@ template <int OP, class T> struct ScalarF {
         else if constexpr (OP == RT_S_SUB) return w_sub<T>(x, v);
         else if constexpr (OP == RT_S_MUL) return w_mul<T>(x, v);
         else if constexpr (OP == RT_S_DIV) {
-            if constexpr (is_sint<T>::value && sizeof(T) <= 8) {
-                if (fault && x == std::numeric_limits<T>::min()) *fault = 1;                       // MIN / -1 overflows
+            if constexpr (is_sint<T>::value) {
+                if (fault && x == min_of<T>()) *fault = 1;                                         // MIN / -1 overflows
             }
             return w_div<T>(x, v);
         }
@@ -815,7 +823,7 @@ int32_t unary_any(rt_ctx* ctx, int32_t dtype, int32_t op, const ViewArg& va) {
 template <class T, int OP>
 int32_t scalar_go(rt_ctx* ctx, const ViewArg& va, const void* value) {
     int32_t* fault = nullptr;
-    if constexpr (OP == RT_S_DIV && is_sint<T>::value && sizeof(T) <= 8) {
+    if constexpr (OP == RT_S_DIV && is_sint<T>::value) {
         if (load_scalar<T>(value) == (T)-1) {                 // x / -1 overflows for x == MIN: the kernel reports it
             fault = ctx->fault_dev;
             CtxGuard g(ctx);
@@ -836,8 +844,6 @@ int32_t scalar_typed(rt_ctx* ctx, int op, const ViewArg& va, const void* value) 
         case RT_S_DIV:
             if constexpr (is_bool<T>::value) {
                 return rt_fail(RT_E_ARITH, "scalar div: division is not implemented for boolean in the reference (todo!())");
-            } else if constexpr (sizeof(T) == 16) {
-                return rt_fail(RT_E_DTYPE, "scalar div: 128-bit integer division is not built for the device");
             } else {
                 if constexpr (!is_flt<T>::value) {
                     if (load_scalar<T>(value) == (T)0) return rt_fail(RT_E_ARITH, "scalar div: integer division by zero (the reference panics)");

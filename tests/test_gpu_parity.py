@@ -1220,7 +1220,7 @@ def test_broadcast_with_transposed_operand(hip, dtype):
 
 
 def test_128bit_integers(hip):
-    """u128 / i128: fill, + - * (tensor and scalar), relu / abs / neg, leaky_relu, gather, equality; division is refused."""
+    """u128 / i128: fill, + - * / (tensor and scalar), relu / abs / neg, leaky_relu, gather, equality (division in depth: test_gpu_int128.py)."""
     from rtensors_amd import hip as H
     rng = np.random.default_rng(128)
     vals_a = [int(rng.integers(-2 ** 62, 2 ** 62)) * int(rng.integers(1, 2 ** 62)) for _ in range(600)]
@@ -1246,9 +1246,8 @@ def test_128bit_integers(hip):
         o2.slice(1, Slice(None, None, 2)).fill(5); g2.slice(1, Slice(None, None, 2)).fill(5)
         assert g2.dump().tobytes() == o2.buf.tobytes()
         assert g2.buf == hip.copy(g2.buf) and not (g2.buf == ga.buf)
-        with pytest.raises(H.TensorError) as e:
-            ga / gb
-        assert e.value.kind == "UnsupportedOperation"
+        ones = cpu.from_ints(code, [v or 1 for v in vals_b])
+        assert (ga / G(hip, name, ones, [20, 30])).dump().tobytes() == (oa / OTensor.from_buf(name, ones, [20, 30])).buf.tobytes()
 
 
 def test_allocation_failure_is_an_error_not_an_abort(hip):
