@@ -201,6 +201,27 @@ class Workloads:
             return (lambda: self.hip.fill_contiguous(c, one, 0, n)), n * es, n
         raise KeyError(which)
 
+    def _c2_fused(self, dtype_name):
+        """c = relu(a * 3 + b) - 1 as one rt_fused_chain launch: two reads and one write."""
+        H = self.H
+        if dtype_name == "f32":
+            dt, n, es = H.F32, 1 << 28, 4
+            a = self._gen("c2a", dt, n, "normal", 1, 0); b = self._gen("c2b", dt, n, "normal", 1, 1)
+        elif dtype_name == "f64":
+            dt, n, es = H.F64, 1 << 27, 8
+            a = self._gen("c2a64", dt, n, "normal", 1, 0); b = self._gen("c2b64", dt, n, "normal", 1, 1)
+        else:
+            dt, n, es = H.I32, 1 << 28, 4
+            a = self._gen("c2ai", dt, n, "int", 1, 0, -(1 << 20), 1 << 20); b = self._gen("c2bi", dt, n, "int", 1, 1, -(1 << 20), 1 << 20)
+        c = self._out("c2c" + dtype_name, dt, n)
+        three, one = (3, 1) if dtype_name == "i32" else (3.0, 1.0)
+        steps = [("scalar", "mul", three), ("binary", "add", 1), ("unary", "relu"), ("scalar", "sub", one)]
+        return (lambda: self.hip.fused_chain([(a, 0), (b, 0)], steps, c, n)), 3 * n * es, n
+
+    def c2_fused(self): return self._c2_fused("f32")
+    def c2_fused_f64(self): return self._c2_fused("f64")
+    def c2_fused_i32(self): return self._c2_fused("i32")
+
     def c2_mul(self): return self._c2("mul")
     def c2_add(self): return self._c2("add")
     def c2_relu(self): return self._c2("relu")
@@ -394,6 +415,7 @@ class Workloads:
 
 HEADLINE = ["c3a_add", "c4_sum1"]
 DETAIL = ["copy", "fill", "c1_add", "c1_sum1", "c2_mul", "c2_add", "c2_relu", "c2_sub", "c2_f64_mul", "c2_f64_add", "c2_i32_mul", "c2_i32_add",
+          "c2_fused", "c2_fused_f64", "c2_fused_i32",
           "c3a_add", "c3b_add", "c4_sum1", "c4_mean1", "c4_max1", "c4_sum0", "c4_sum_all", "c4_i32_sum1", "c4_i32_max1", "c4_i32_min0",
           "c4_var1", "c4_std0", "c4_lse1", "c4_argmax1", "c5_bias_add", "c5_colsum", "c5_fused_bias_relu", "c5_fused_l1_forward", "c5_fused_backward", "c5_fused2_forward", "c5_fused2_backward",
           "view_relu", "tr_add", "tr_copy"]

@@ -258,6 +258,37 @@ int32_t rt_fused_bias_relu_l1(rt_ctx* ctx, int32_t dtype, const void* x, uint64_
 int32_t rt_fused_l1_relu_backward_t(rt_ctx* ctx, int32_t dtype, const void* y, uint64_t y_len, const void* target, uint64_t target_len,
                                     const void* upstream, uint64_t upstream_len, void* dbias, uint64_t dbias_len, uint64_t rows, uint64_t cols);
 
+/* ---- fused elementwise chain ------------------------------------------------------------------------------------------------
+ * No single counterpart in the trait: the reference issues an expression such as `c = relu(a * 3.0 + b); c -= 1.0` as one backend
+ * call per operator, each a pass over the whole tensor, with a clone before every value-returning scalar / unary op
+ * (ops/scalar/add.rs:84-113, ops/unary/mod.rs:114-126).  This entry point runs a program of up to RT_CHAIN_MAX_STEPS such steps in
+ * registers, reading each input once and writing the result once:
+ *     acc = inputs[0][input_starts[0] + i];  for every step: acc = step(acc);  dst[dst_start + i] = acc        (i < len)
+ *   RT_CHAIN_UNARY       acc = op(acc)                       op: rt_unary_op
+ *   RT_CHAIN_SCALAR      acc = acc op value                  op: rt_scalar_op, value: one element of dtype
+ *   RT_CHAIN_BINARY      acc = acc op inputs[operand][..]    op: rt_binary_op
+ *   RT_CHAIN_BINARY_REV  acc = inputs[operand][..] op acc
+ * Each step is the same IEEE / wrapping operation as the separate call, in the same order (no contraction), so the result is bit for
+ * bit that of the sequence.  All operands are forward contiguous runs of `len` elements (gather other views first), in any alignment.
+ * dst may be the very run of one of the inputs (in place); any other overlap is RT_E_INVALID.  Available: f32 / f64 and the 8..64-bit
+ * integers; unary relu abs step (+ neg abs_grad for signed and float; + sqrt floor ceil round trunc rsqrt reciprocal square cube sign
+ * exp sigmoid silu tanh for float), scalar add sub mul leaky_relu leaky_grad (+ div for float), binary add sub mul (+ div for float).
+ * Anything else is RT_E_DTYPE and the caller issues the separate ops (integer division reports its faults per launch; the other float
+ * ops are ALU-bound on their own). */
+#define RT_CHAIN_MAX_STEPS 8
+#define RT_CHAIN_MAX_INPUTS 4
+typedef enum rt_chain_kind { RT_CHAIN_UNARY = 0, RT_CHAIN_SCALAR = 1, RT_CHAIN_BINARY = 2, RT_CHAIN_BINARY_REV = 3 } rt_chain_kind;
+typedef struct rt_chain_step {
+    int32_t kind;        /* rt_chain_kind */
+    int32_t op;          /* rt_unary_op / rt_scalar_op / rt_binary_op according to kind */
+    int32_t operand;     /* binary kinds: index into inputs[] of the other side */
+    int32_t reserved;    /* 0 */
+    uint8_t value[8];    /* scalar kind: the element, in the dtype's own representation */
+} rt_chain_step;
+int32_t rt_fused_chain(rt_ctx* ctx, int32_t dtype, int32_t n_inputs, const void* const* inputs, const uint64_t* input_lens,
+                       const uint64_t* input_starts, uint64_t len, int32_t n_steps, const rt_chain_step* steps,
+                       void* dst, uint64_t dst_len, uint64_t dst_start);
+
 /* ---- matmul ------------------------------------------------------------------------------------------------------
  * BackendMatMul::matmul (backend/mod.rs:474-485; Cpu backend/cpu.rs:725-951), argument list of protocol Op::Matmul
  * (backend/remote/protocol.rs:269-277): dst[b] = lhs[b] (m x k) * rhs[b] (k x n) for every batch, dst row-major and
@@ -287,7 +318,7 @@ int32_t rt_event_create(rt_ctx* ctx, rt_event** out);
 int32_t rt_event_record(rt_ctx* ctx, rt_event* ev);              /* on the context's stream */
 int32_t rt_event_elapsed_ms(rt_ctx* ctx, rt_event* start, rt_event* stop, float* out_ms);   /* waits for `stop` */
 int32_t rt_event_destroy(rt_ctx* ctx, rt_event* ev);
-/* bytes currently handed out, bytes cached in free lists, number of hipMalloc calls so far */
+/* bytes currently handed out, bytes cached in free lists, number of hipMalloc calls so far (blocks and growth of the scratch buffer) */
 int32_t rt_mem_stats(rt_ctx* ctx, uint64_t* in_use, uint64_t* cached, uint64_t* device_allocs);
 int32_t rt_mem_trim(rt_ctx* ctx);                                /* hipFree everything in the free lists */
 

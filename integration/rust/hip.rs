@@ -592,6 +592,41 @@ impl Hip {
         })
     }
 
+    /// A program of up to `RT_CHAIN_MAX_STEPS` elementwise steps in one pass: `dst[dst_start + i] = steps(inputs[0][start0 + i])`,
+    /// each input read once, the result written once.  The reference issues `relu(a * 3.0 + b) - 1.0` as four kernels and two
+    /// clones (ops/scalar/add.rs:84-113, ops/unary/mod.rs:114-126); every step here is the same operation on `T` in the same
+    /// order, so the result is bit for bit the same.  Build steps with `ChainStep::{unary, scalar, binary, binary_rev}`.
+    /// `RT_E_DTYPE` (-> `UnsupportedOperation`) names a step that is not available in a chain: issue the separate ops then.
+    pub fn fused_chain<T: TensorValue>(&self, inputs: &[(&HipBuf<T>, usize)], steps: &[ChainStep], len: usize,
+        dst: &mut HipBuf<T>, dst_start: usize) -> Result<(), TensorError> {
+        let ptrs: Vec<*const c_void> = inputs.iter().map(|(b, _)| b.ptr as *const c_void).collect();
+        let lens: Vec<u64> = inputs.iter().map(|(b, _)| b.len as u64).collect();
+        let starts: Vec<u64> = inputs.iter().map(|(_, s)| *s as u64).collect();
+        let raw: Vec<ffi::rt_chain_step> = steps.iter().map(|s| s.0).collect();
+        check(unsafe {
+            ffi::rt_fused_chain(self.raw(), dt::<T>(), ptrs.len() as i32, ptrs.as_ptr(), lens.as_ptr(), starts.as_ptr(),
+                len as u64, raw.len() as i32, raw.as_ptr(), dst.ptr, dst.len as u64, dst_start as u64)
+        })
+    }
+
+    /// As `fused_chain`, in place on `inputs[which]`'s own run (the one aliasing the entry point allows).
+    pub fn fused_chain_inplace<T: TensorValue>(&self, target: &mut HipBuf<T>, start: usize, others: &[(&HipBuf<T>, usize)],
+        steps: &[ChainStep], len: usize) -> Result<(), TensorError> {
+        let mut ptrs: Vec<*const c_void> = vec![target.ptr as *const c_void];
+        let mut lens: Vec<u64> = vec![target.len as u64];
+        let mut starts: Vec<u64> = vec![start as u64];
+        for (b, s) in others {
+            ptrs.push(b.ptr as *const c_void);
+            lens.push(b.len as u64);
+            starts.push(*s as u64);
+        }
+        let raw: Vec<ffi::rt_chain_step> = steps.iter().map(|s| s.0).collect();
+        check(unsafe {
+            ffi::rt_fused_chain(self.raw(), dt::<T>(), ptrs.len() as i32, ptrs.as_ptr(), lens.as_ptr(), starts.as_ptr(),
+                len as u64, raw.len() as i32, raw.as_ptr(), target.ptr, target.len as u64, start as u64)
+        })
+    }
+
     /// One pass for a value-returning unary op on a contiguous operand (`alloc` + this, instead of `owned()` + the
     /// in-place op, which is two passes: ops/unary/mod.rs:114-126).
     pub fn unary_to<T: TensorValue>(&self, op: i32, src: &HipBuf<T>, start: usize, len: usize, dst: &mut HipBuf<T>)
@@ -619,5 +654,31 @@ impl Hip {
                 meta.shape.as_slice().as_ptr() as *const u64, meta.strides.as_slice().as_ptr() as *const i64, dst.ptr,
                 dst.len as u64)
         })
+    }
+}
+
+/// One step of `Hip::fused_chain`.
+#[derive(Clone, Copy, Debug)]
+pub struct ChainStep(ffi::rt_chain_step);
+
+impl ChainStep {
+    /// `acc = op(acc)`, `op` one of `ffi::RT_U_*`.
+    pub fn unary(op: i32) -> Self {
+        ChainStep(ffi::rt_chain_step { kind: ffi::RT_CHAIN_UNARY, op, ..Default::default() })
+    }
+    /// `acc = acc op value`, `op` one of `ffi::RT_S_*`; the value travels in `T`'s own representation.
+    pub fn scalar<T: TensorValue>(op: i32, value: T) -> Self {
+        let mut raw = [0u8; 8];
+        let n = std::mem::size_of::<T>().min(8);
+        unsafe { std::ptr::copy_nonoverlapping(&value as *const T as *const u8, raw.as_mut_ptr(), n) };
+        ChainStep(ffi::rt_chain_step { kind: ffi::RT_CHAIN_SCALAR, op, value: raw, ..Default::default() })
+    }
+    /// `acc = acc op inputs[operand]`, `op` a `BinaryOpType` code (ops/base.rs:7-12).
+    pub fn binary(op: BinaryOpType, operand: usize) -> Self {
+        ChainStep(ffi::rt_chain_step { kind: ffi::RT_CHAIN_BINARY, op: op as i32, operand: operand as i32, ..Default::default() })
+    }
+    /// `acc = inputs[operand] op acc`.
+    pub fn binary_rev(op: BinaryOpType, operand: usize) -> Self {
+        ChainStep(ffi::rt_chain_step { kind: ffi::RT_CHAIN_BINARY_REV, op: op as i32, operand: operand as i32, ..Default::default() })
     }
 }

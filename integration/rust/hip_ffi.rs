@@ -16,6 +16,25 @@ pub struct rt_event {
     _private: [u8; 0],
 }
 
+/// One step of a fused elementwise chain (`rt_chain_step`): 24 bytes, same field order as the header.
+#[repr(C)]
+#[derive(Clone, Copy, Debug, Default)]
+pub struct rt_chain_step {
+    pub kind: i32,
+    pub op: i32,
+    pub operand: i32,
+    pub reserved: i32,
+    pub value: [u8; 8],
+}
+
+// rt_chain_kind and the limits of a chain
+pub const RT_CHAIN_UNARY: i32 = 0;
+pub const RT_CHAIN_SCALAR: i32 = 1;
+pub const RT_CHAIN_BINARY: i32 = 2;
+pub const RT_CHAIN_BINARY_REV: i32 = 3;
+pub const RT_CHAIN_MAX_STEPS: i32 = 8;
+pub const RT_CHAIN_MAX_INPUTS: i32 = 4;
+
 // rt_status
 pub const RT_OK: i32 = 0;
 pub const RT_E_INVALID: i32 = 1;
@@ -160,6 +179,9 @@ extern "C" {
     pub fn rt_fused_l1_relu_backward_t(ctx: *mut rt_ctx, dtype: i32, y: *const c_void, y_len: u64, target: *const c_void,
                                        target_len: u64, upstream: *const c_void, upstream_len: u64, dbias: *mut c_void,
                                        dbias_len: u64, rows: u64, cols: u64) -> i32;
+    pub fn rt_fused_chain(ctx: *mut rt_ctx, dtype: i32, n_inputs: i32, inputs: *const *const c_void, input_lens: *const u64,
+                          input_starts: *const u64, len: u64, n_steps: i32, steps: *const rt_chain_step, dst: *mut c_void,
+                          dst_len: u64, dst_start: u64) -> i32;
     pub fn rt_matmul(ctx: *mut rt_ctx, dtype: i32, lhs: *const c_void, lhs_len: u64, lhs_offset: u64, lhs_rank: i32,
                      lhs_shape: *const u64, lhs_strides: *const i64, lhs_contiguity: i32, rhs: *const c_void, rhs_len: u64,
                      rhs_offset: u64, rhs_rank: i32, rhs_shape: *const u64, rhs_strides: *const i64, rhs_contiguity: i32,

@@ -18,12 +18,19 @@ SYMBOLS = [
     "rt_unary_contiguous", "rt_unary_1d_strided", "rt_unary_nd",
     "rt_scalar_contiguous", "rt_scalar_1d_strided", "rt_scalar_nd", "rt_unary_to", "rt_scalar_to",
     "rt_broadcast", "rt_reduce_flat", "rt_reduce_nd", "rt_reduce_nd_static", "rt_argmax_flat", "rt_argmax_nd", "rt_gather", "rt_matmul", "rt_fused_bias_relu", "rt_fused_l1_forward", "rt_fused_l1_relu_backward",
-    "rt_fused_bias_relu_l1", "rt_fused_l1_relu_backward_t",
+    "rt_fused_bias_relu_l1", "rt_fused_l1_relu_backward_t", "rt_fused_chain",
     "rt_event_create", "rt_event_record", "rt_event_elapsed_ms", "rt_event_destroy", "rt_mem_stats", "rt_mem_trim",
 ]
 
 u64, i64, i32, vp = C.c_uint64, C.c_int64, C.c_int32, C.c_void_p
 u64p, i64p, i32p, vpp = C.POINTER(C.c_uint64), C.POINTER(C.c_int64), C.POINTER(C.c_int32), C.POINTER(C.c_void_p)
+
+
+
+class ChainStep(C.Structure):
+    """rt_chain_step of include/rt_hip.h"""
+    _fields_ = [("kind", C.c_int32), ("op", C.c_int32), ("operand", C.c_int32), ("reserved", C.c_int32), ("value", C.c_uint8 * 8)]
+
 
 _SIGS = {
     "rt_ctx_create": [i32, vpp], "rt_ctx_destroy": [vp], "rt_sync": [vp], "rt_dtype_size": [i32], "rt_device_count": [i32p],
@@ -52,6 +59,7 @@ _SIGS = {
     "rt_fused_l1_relu_backward": [vp, i32, vp, u64, vp, u64, vp, u64, vp, u64, u64, u64],
     "rt_fused_bias_relu_l1": [vp, i32, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, u64, u64],
     "rt_fused_l1_relu_backward_t": [vp, i32, vp, u64, vp, u64, vp, u64, vp, u64, u64, u64],
+    "rt_fused_chain": [vp, i32, i32, vpp, u64p, u64p, u64, i32, C.POINTER(ChainStep), vp, u64, u64],
     "rt_event_create": [vp, vpp], "rt_event_record": [vp, vp], "rt_event_elapsed_ms": [vp, vp, vp, C.POINTER(C.c_float)],
     "rt_event_destroy": [vp, vp], "rt_mem_stats": [vp, u64p, u64p, u64p], "rt_mem_trim": [vp],
 }

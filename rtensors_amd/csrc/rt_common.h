@@ -50,6 +50,7 @@ struct rt_ctx {
     void* fixed_scratch = nullptr;
     size_t fixed_scratch_bytes = 0;
     bool fixed_only = false;
+    void* static_scratch = nullptr;                // this device's copy of the library's built-in workspace (rt_static_scratch_init)
     // pinned staging ring for large host<->device transfers (allocated by the first one), one event per slot
     void* stage[4] = {nullptr, nullptr, nullptr, nullptr};
     hipEvent_t stage_ev[4] = {nullptr, nullptr, nullptr, nullptr};
@@ -74,7 +75,9 @@ struct CtxGuard {
 int32_t rt_ctx_enter(rt_ctx* ctx);                                   // validates ctx and makes its device current
 int32_t rt_alloc_bytes(rt_ctx* ctx, size_t bytes, void** out);       // caller holds ctx->mu
 int32_t rt_free_locked(rt_ctx* ctx, void* p);
-int32_t rt_scratch(rt_ctx* ctx, size_t bytes, void** out);           // caller holds ctx->mu
+int32_t rt_scratch(rt_ctx* ctx, size_t bytes, void** out);           // caller holds ctx->mu; growth counts as a device allocation
+// Device address of the built-in workspace of rt_reduce_nd_static on `device`, which must be current (looked up once per device).
+int32_t rt_static_scratch_init(int device, void** out);
 // After the stream has been waited for: RT_E_ARITH if an integer division launched since the last look met a fault, and the fault
 // word is cleared.  Caller holds ctx->mu.
 int32_t rt_take_fault(rt_ctx* ctx);

@@ -869,6 +869,189 @@ int32_t scalar_any(rt_ctx* ctx, int32_t dtype, int32_t op, const ViewArg& va, co
     return no_dtype("scalar", dtype);
 }
 
+
+// ---- fused chain -------------------------------------------------------------------------------------------------------------------
+// A short program of elementwise steps applied in registers: acc = in[0][i]; acc = step_k(acc) for every step; dst[i] = acc.  Every
+// input is read once and the result written once, whatever the number of steps; each step is the same IEEE / wrapping operation as
+// the separate kernel (UnaryF / ScalarF / w_add ...), applied in the same order, so the result is bit for bit that of the sequence of
+// backend calls.  The op codes are wave-uniform kernel arguments: the step loop is a handful of scalar branches per vector.
+constexpr int kChainUnary = 0, kChainScalar = 1, kChainBinary = 2, kChainBinaryRev = 3;
+
+struct ChainProg {
+    int32_t nsteps, ninputs;
+    int32_t code[RT_CHAIN_MAX_STEPS];            // kind << 8 | op
+    int32_t operand[RT_CHAIN_MAX_STEPS];
+    uint64_t value[RT_CHAIN_MAX_STEPS];          // scalar steps: the element's bits (T is at most 8 bytes here)
+};
+template <class T> struct ChainPtrs { const T* p[RT_CHAIN_MAX_INPUTS]; };
+
+template <class T> __device__ __forceinline__ T chain_value(uint64_t bits) {
+    T v;
+    __builtin_memcpy(&v, &bits, sizeof(T));
+    return v;
+}
+
+#define RT_CH(K, OP) ((K) << 8 | (OP))
+// one step over N elements held in registers; `y` is the other side of a binary step
+template <class T, int N>
+__device__ __forceinline__ void chain_apply(T (&a)[N], const T (&y)[N], int code, uint64_t bits) {
+    const T v = chain_value<T>(bits);
+#define RT_CH_U(OP) case RT_CH(kChainUnary, OP): { _Pragma("unroll") for (int j = 0; j < N; ++j) a[j] = UnaryF<OP, T>{}(a[j]); } break
+#define RT_CH_S(OP) case RT_CH(kChainScalar, OP): { const ScalarF<OP, T> f{v, nullptr}; _Pragma("unroll") for (int j = 0; j < N; ++j) a[j] = f(a[j]); } break
+    switch (code) {
+        RT_CH_U(RT_U_RELU); RT_CH_U(RT_U_ABS); RT_CH_U(RT_U_STEP);
+        RT_CH_S(RT_S_ADD); RT_CH_S(RT_S_SUB); RT_CH_S(RT_S_MUL); RT_CH_S(RT_S_LEAKY_RELU); RT_CH_S(RT_S_LEAKY_GRAD);
+        case RT_CH(kChainBinary, RT_ADD): { _Pragma("unroll") for (int j = 0; j < N; ++j) a[j] = w_add<T>(a[j], y[j]); } break;
+        case RT_CH(kChainBinary, RT_SUB): { _Pragma("unroll") for (int j = 0; j < N; ++j) a[j] = w_sub<T>(a[j], y[j]); } break;
+        case RT_CH(kChainBinary, RT_MUL): { _Pragma("unroll") for (int j = 0; j < N; ++j) a[j] = w_mul<T>(a[j], y[j]); } break;
+        case RT_CH(kChainBinaryRev, RT_ADD): { _Pragma("unroll") for (int j = 0; j < N; ++j) a[j] = w_add<T>(y[j], a[j]); } break;
+        case RT_CH(kChainBinaryRev, RT_SUB): { _Pragma("unroll") for (int j = 0; j < N; ++j) a[j] = w_sub<T>(y[j], a[j]); } break;
+        case RT_CH(kChainBinaryRev, RT_MUL): { _Pragma("unroll") for (int j = 0; j < N; ++j) a[j] = w_mul<T>(y[j], a[j]); } break;
+        default:
+            if constexpr (is_sint<T>::value || is_flt<T>::value) {
+                switch (code) {
+                    RT_CH_U(RT_U_NEG); RT_CH_U(RT_U_ABS_GRAD);
+                    default: break;
+                }
+            }
+            if constexpr (is_flt<T>::value) {
+                switch (code) {
+                    RT_CH_U(RT_U_SQRT); RT_CH_U(RT_U_FLOOR); RT_CH_U(RT_U_CEIL); RT_CH_U(RT_U_ROUND); RT_CH_U(RT_U_TRUNC); RT_CH_U(RT_U_RSQRT);
+                    RT_CH_U(RT_U_RECIPROCAL); RT_CH_U(RT_U_SQUARE); RT_CH_U(RT_U_CUBE); RT_CH_U(RT_U_SIGN);
+                    RT_CH_U(RT_U_EXP); RT_CH_U(RT_U_SIGMOID); RT_CH_U(RT_U_SILU); RT_CH_U(RT_U_TANH);
+                    RT_CH_S(RT_S_DIV);
+                    case RT_CH(kChainBinary, RT_DIV): { _Pragma("unroll") for (int j = 0; j < N; ++j) a[j] = a[j] / y[j]; } break;
+                    case RT_CH(kChainBinaryRev, RT_DIV): { _Pragma("unroll") for (int j = 0; j < N; ++j) a[j] = y[j] / a[j]; } break;
+                    default: break;
+                }
+            }
+            break;
+    }
+#undef RT_CH_U
+#undef RT_CH_S
+}
+
+// the whole program over N elements; fetch(k, y) unpacks the elements of input k
+template <class T, int N, class Fetch>
+__device__ __forceinline__ void chain_run(T (&acc)[N], const ChainProg& prog, Fetch fetch) {
+#pragma unroll 1
+    for (int s = 0; s < prog.nsteps; ++s) {
+        const int code = prog.code[s];
+        T y[N];
+        fetch(prog.operand[s], y);
+        chain_apply<T, N>(acc, y, code, prog.value[s]);
+    }
+}
+
+// dst and every input point at the vector body, which starts on a 128-byte line of dst; the inputs may be in any phase.  The `head`
+// elements before the body and the `tail` elements after it go to lanes of the first and the last block.
+template <class T>
+__global__ __launch_bounds__(256) void chain_kernel(ChainPtrs<T> in, T* __restrict__ d, size_t nvec, uint32_t head, uint32_t tail, TileMap m, ChainProg prog) {
+    constexpr int N = 16 / sizeof(T);
+    const bool at_head = blockIdx.x == 0 && threadIdx.x < head, at_tail = blockIdx.x == gridDim.x - 1 && threadIdx.x < tail;
+    if (at_head || at_tail) {
+        // one element per lane: before the body (negative index) or after it
+        auto one = [&](int64_t e) {
+            T x[RT_CHAIN_MAX_INPUTS], acc[1];
+#pragma unroll
+            for (int k = 0; k < RT_CHAIN_MAX_INPUTS; ++k) x[k] = k < prog.ninputs ? in.p[k][e] : zero_of<T>();
+            acc[0] = x[0];
+            chain_run<T, 1>(acc, prog, [&](int k, T (&y)[1]) { y[0] = k == 0 ? x[0] : (k == 1 ? x[1] : (k == 2 ? x[2] : x[3])); });
+            d[e] = acc[0];
+        };
+        if (at_head) one((int64_t)threadIdx.x - (int64_t)head);
+        if (at_tail) one((int64_t)(nvec * N + threadIdx.x));
+    }
+    size_t i;
+    if (!rt_tile_index(m, blockIdx.x, 256, threadIdx.x, nvec, &i)) return;
+    // every input's load is issued before the first use; the vectors stay packed (four 32-bit words) until a step needs their elements
+    rt_u32x4 w[RT_CHAIN_MAX_INPUTS];
+#pragma unroll
+    for (int k = 0; k < RT_CHAIN_MAX_INPUTS; ++k) {
+        w[k] = rt_u32x4{0, 0, 0, 0};
+        if (k < prog.ninputs) w[k] = rt_ld16u<T, true>(in.p[k] + i * N);
+    }
+    T acc[N];
+    {
+        const Vec16<T> v = __builtin_bit_cast(Vec16<T>, w[0]);
+#pragma unroll
+        for (int j = 0; j < N; ++j) acc[j] = v.e[j];
+    }
+    chain_run<T, N>(acc, prog, [&](int k, T (&y)[N]) {
+        const rt_u32x4 ws = k == 0 ? w[0] : (k == 1 ? w[1] : (k == 2 ? w[2] : w[3]));
+        const Vec16<T> v = __builtin_bit_cast(Vec16<T>, ws);
+#pragma unroll
+        for (int j = 0; j < N; ++j) y[j] = v.e[j];
+    });
+    Vec16<T> out;
+#pragma unroll
+    for (int j = 0; j < N; ++j) out.e[j] = acc[j];
+    rt_st16_nt(reinterpret_cast<Vec16<T>*>(d) + i, out);
+}
+
+// Is (kind, op) a step the chain kernel has for T?  The dtype rules are those of rt_unary_* / rt_scalar_* / rt_broadcast; left out are
+// the ops that are ALU-bound on their own (logarithms, trigonometric and hyperbolic inverses ...), integer division (its faults are
+// reported per launch) and the 1-byte bool and 16-byte integer types.
+template <class T> bool chain_has(int kind, int op) {
+    constexpr bool F = is_flt<T>::value, S = is_sint<T>::value;
+    if (kind == kChainUnary) {
+        switch (op) {
+            case RT_U_RELU: case RT_U_ABS: case RT_U_STEP: return true;
+            case RT_U_NEG: case RT_U_ABS_GRAD: return F || S;
+            case RT_U_SQRT: case RT_U_FLOOR: case RT_U_CEIL: case RT_U_ROUND: case RT_U_TRUNC: case RT_U_RSQRT: case RT_U_RECIPROCAL:
+            case RT_U_SQUARE: case RT_U_CUBE: case RT_U_SIGN: case RT_U_EXP: case RT_U_SIGMOID: case RT_U_SILU: case RT_U_TANH: return F;
+        }
+        return false;
+    }
+    if (kind == kChainScalar) {
+        switch (op) {
+            case RT_S_ADD: case RT_S_SUB: case RT_S_MUL: case RT_S_LEAKY_RELU: case RT_S_LEAKY_GRAD: return true;
+            case RT_S_DIV: return F;
+        }
+        return false;
+    }
+    if (kind == kChainBinary || kind == kChainBinaryRev) return op == RT_ADD || op == RT_SUB || op == RT_MUL || (op == RT_DIV && F);
+    return false;
+}
+
+template <class T>
+int32_t chain_typed(rt_ctx* ctx, int n_inputs, const void* const* inputs, const uint64_t* starts, uint64_t len, int n_steps, const rt_chain_step* steps,
+                    void* dst, uint64_t dst_start) {
+    constexpr size_t N = 16 / sizeof(T);
+    ChainProg prog;
+    memset(&prog, 0, sizeof(prog));
+    prog.nsteps = n_steps;
+    prog.ninputs = n_inputs;
+    for (int s = 0; s < n_steps; ++s) {
+        const rt_chain_step& st = steps[s];
+        if (!chain_has<T>(st.kind, st.op))
+            return rt_fail(RT_E_DTYPE, "fused chain: step %d (kind %d, op %d) is not available for this dtype in a chain (issue the separate ops instead)", s, st.kind, st.op);
+        const bool bin = st.kind == kChainBinary || st.kind == kChainBinaryRev;
+        if (bin && (st.operand < 0 || st.operand >= n_inputs)) return rt_fail(RT_E_INVALID, "fused chain: step %d names input %d of %d", s, st.operand, n_inputs);
+        prog.code[s] = RT_CH(st.kind, st.op);
+        prog.operand[s] = bin ? st.operand : 0;
+        memcpy(&prog.value[s], st.value, sizeof(T));
+    }
+    T* d = (T*)dst + dst_start;
+    ChainPtrs<T> in;
+    const uintptr_t addr = reinterpret_cast<uintptr_t>(d);
+    size_t head = ((kBodyAlign - (addr & (kBodyAlign - 1))) & (kBodyAlign - 1)) / sizeof(T);
+    if (head > len) head = (size_t)len;
+    const size_t nvec = ((size_t)len - head) / N, tail = (size_t)len - head - nvec * N;
+    for (int k = 0; k < RT_CHAIN_MAX_INPUTS; ++k) in.p[k] = k < n_inputs ? (const T*)inputs[k] + starts[k] + head : nullptr;
+    const TileMap m = rt_make_tilemap(d + head, nvec, 256);
+    size_t blocks = rt_tilemap_blocks(m, nvec, 256);
+    if (blocks < 1) blocks = 1;
+    if (blocks > 0x7fffffffull) return rt_fail(RT_E_INVALID, "fused chain: a run of %llu elements is too long for one launch", (unsigned long long)len);
+    // the edge arguments are compared with the lane index inside the kernel: they must be below the block size
+    if (head >= 256 || tail >= 256 || head + nvec * N + tail != len) return rt_fail(RT_E_INVALID, "fused chain: inconsistent launch geometry");
+    CtxGuard g(ctx);
+    hipLaunchKernelGGL((chain_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, in, d + head, nvec, (uint32_t)head, (uint32_t)tail, m, prog);
+    RT_HIP(hipGetLastError());
+    return RT_OK;
+}
+#undef RT_CH
+
 }  // namespace
 
 // ---- C ABI ------------------------------------------------------------------------------------------------------------
@@ -926,4 +1109,37 @@ extern "C" int32_t rt_scalar_to(rt_ctx* ctx, int32_t dtype, int32_t op, const vo
     const int64_t one = 1;
     if (!dst && len) return rt_fail(RT_E_INVALID, "scalar: null destination");
     return scalar_any(ctx, dtype, op, ViewArg{const_cast<void*>(src), src_len, start, 1, &len, &one, dst, dst_len}, value);
+}
+
+// Fused chain: dst[dst_start + i] = step_{n-1}(... step_0(inputs[0][starts[0] + i]) ...) for i < len.
+extern "C" int32_t rt_fused_chain(rt_ctx* ctx, int32_t dtype, int32_t n_inputs, const void* const* inputs, const uint64_t* input_lens,
+                                  const uint64_t* input_starts, uint64_t len, int32_t n_steps, const rt_chain_step* steps, void* dst, uint64_t dst_len,
+                                  uint64_t dst_start) {
+    RT_TRY(rt_ctx_enter(ctx));
+    const int es = rt_elem_size(dtype);
+    if (!es) return no_dtype("fused chain", dtype);
+    if (n_inputs < 1 || n_inputs > RT_CHAIN_MAX_INPUTS) return rt_fail(RT_E_INVALID, "fused chain: %d inputs (1..%d)", n_inputs, RT_CHAIN_MAX_INPUTS);
+    if (n_steps < 1 || n_steps > RT_CHAIN_MAX_STEPS) return rt_fail(RT_E_INVALID, "fused chain: %d steps (1..%d)", n_steps, RT_CHAIN_MAX_STEPS);
+    if (!inputs || !input_lens || !input_starts || !steps) return rt_fail(RT_E_INVALID, "fused chain: null argument");
+    if (dst_start > dst_len || len > dst_len - dst_start)
+        return rt_fail(RT_E_OUT_OF_BOUNDS, "fused chain: %llu results from element %llu of a buffer of %llu", (unsigned long long)len, (unsigned long long)dst_start,
+                       (unsigned long long)dst_len);
+    for (int k = 0; k < n_inputs; ++k)
+        if (input_starts[k] > input_lens[k] || len > input_lens[k] - input_starts[k])
+            return rt_fail(RT_E_OUT_OF_BOUNDS, "fused chain: input %d is shorter than start + len", k);
+    if (dtype == RT_BOOL || es == 16) return rt_fail(RT_E_DTYPE, "fused chain: bool and 128-bit integers are not built (issue the separate ops instead)");
+    if (len == 0) return RT_OK;
+    if (!dst) return rt_fail(RT_E_INVALID, "fused chain: null destination");
+    const ByteSpan ds = rt_run_span(dst, es, dst_start, len);
+    for (int k = 0; k < n_inputs; ++k) {
+        if (!inputs[k]) return rt_fail(RT_E_INVALID, "fused chain: null input %d", k);
+        // the destination may be the very run of an input (every lane reads its elements before it writes them), nothing else
+        const bool same = inputs[k] == dst && input_starts[k] == dst_start;
+        if (!same && rt_spans_meet(ds, rt_run_span(inputs[k], es, input_starts[k], len)))
+            return rt_fail(RT_E_INVALID, "fused chain: the destination overlaps input %d without being the same run", k);
+    }
+    RT_FOR_DTYPE(dtype, {
+        if constexpr (!is_bool<T>::value && sizeof(T) <= 8) return chain_typed<T>(ctx, n_inputs, inputs, input_starts, len, n_steps, steps, dst, dst_start);
+    });
+    return no_dtype("fused chain", dtype);
 }

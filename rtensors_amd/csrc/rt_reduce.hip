@@ -950,7 +950,8 @@ extern "C" int32_t rt_reduce_nd(rt_ctx* ctx, int32_t dtype, int32_t op, const vo
 // rt_reduce_nd with the partial results of a split reduction in a workspace that is part of the library's device image instead of
 // device memory allocated on demand, for callers that cannot allocate (HIP graph capture, serving loops, harnesses that forbid
 // hipMalloc).  `scratch` below is a host-side stand-in for the device array, not a device address: the address on each device
-// is fetched once with hipGetSymbolAddress, with that device current, and only that pointer is ever handed to a kernel.
+// is fetched with hipGetSymbolAddress, with that device current, when the first context on that device is created, and only that
+// pointer is ever handed to a kernel.  The entry point itself makes no runtime query.
 // Nothing in the workspace has to start at zero: every partial that the second stage reads was written by the first stage of the
 // same call.  All calls on one device share the workspace, so calls that overlap on one device (two contexts, two streams) race.
 constexpr size_t kStaticScratchBytes = RT_STATIC_SCRATCH_BYTES;
@@ -959,28 +960,31 @@ constexpr int kMaxDevices = 64;
 static std::mutex g_static_mu;
 static void* g_static_ptr[kMaxDevices] = {};
 
+int32_t rt_static_scratch_init(int device, void** out) {
+    *out = nullptr;
+    if (device < 0 || device >= kMaxDevices) return RT_OK;          // such a context has no workspace; the entry point refuses it
+    std::lock_guard<std::mutex> lk(g_static_mu);
+    if (!g_static_ptr[device]) {
+        void* p = nullptr;
+        RT_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));          // this device's copy of the array (the device is current)
+        g_static_ptr[device] = p;
+    }
+    *out = g_static_ptr[device];
+    return RT_OK;
+}
+
 extern "C" int32_t rt_reduce_nd_static(rt_ctx* ctx, int32_t dtype, int32_t op, const void* src, uint64_t src_len, uint64_t offset, int32_t rank,
                                        const uint64_t* shape, const int64_t* strides, void* dst, uint64_t dst_len, int32_t dim) {
     RT_TRY(rt_ctx_enter(ctx));
     int es = rt_elem_size(dtype);
     if (!es) return rt_fail(RT_E_DTYPE, "reduce: unknown dtype code %d", dtype);
-    if (ctx->device < 0 || ctx->device >= kMaxDevices) return rt_fail(RT_E_INVALID, "reduce: device index %d is beyond the %d this entry point keeps a workspace for", ctx->device, kMaxDevices);
+    if (!ctx->static_scratch) return rt_fail(RT_E_INVALID, "reduce: device index %d is beyond the %d this entry point keeps a workspace for", ctx->device, kMaxDevices);
     uint64_t outer = 0, inner = 0;
     bool run = false;
     RT_TRY(rt_check_reduce_nd(src_len, src, offset, rank, shape, strides, dst, dst_len, dim, &outer, &inner, &run));
     if (!run) return RT_OK;
-    void* ws = nullptr;
-    {
-        std::lock_guard<std::mutex> lk(g_static_mu);
-        if (!g_static_ptr[ctx->device]) {
-            void* p = nullptr;
-            RT_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));      // this device's copy of the array (the device is current)
-            g_static_ptr[ctx->device] = p;
-        }
-        ws = g_static_ptr[ctx->device];
-    }
     CtxGuard g(ctx);
-    ctx->fixed_scratch = ws;
+    ctx->fixed_scratch = ctx->static_scratch;
     ctx->fixed_scratch_bytes = kStaticScratchBytes;
     ctx->fixed_only = true;
     const int32_t st = reduce_dispatch(ctx, dtype, op, (const char*)src + offset * es, dst, outer, shape[dim], inner);

@@ -86,6 +86,10 @@ extern "C" int32_t rt_ctx_create(int32_t device, rt_ctx** out) {
     e = hipMemset(c->flag_dev, 0, 256);
     if (e != hipSuccess) { (void)hipFree(c->flag_dev); (void)hipStreamDestroy(c->stream); delete c; return rt_hip_fail(e, "hipMemset(flag)"); }
     c->fault_dev = c->flag_dev + 16;                         // its own 64-byte piece of the block
+    // the device address of the library's built-in workspace, looked up here so that the entry point that allocates nothing makes no
+    // runtime query of its own (a symbol lookup is not safe under stream capture)
+    const int32_t ws = rt_static_scratch_init(device, &c->static_scratch);
+    if (ws != RT_OK) { (void)hipFree(c->flag_dev); (void)hipStreamDestroy(c->stream); delete c; return ws; }
     *out = c;
     return RT_OK;
 }
@@ -204,6 +208,7 @@ int32_t rt_scratch(rt_ctx* ctx, size_t bytes, void** out) {
         size_t cap = size_class(bytes < (1u << 20) ? (1u << 20) : bytes);
         RT_HIP(hipMalloc(&ctx->scratch, cap));
         ctx->scratch_bytes = cap;
+        ctx->device_allocs += 1;
     }
     *out = ctx->scratch;
     return RT_OK;

@@ -280,6 +280,27 @@ class Hip:
         _check(lib.rt_fused_l1_relu_backward_t(self._ctx, y.dtype, y.ptr, y.len, target.ptr, target.len, upstream.ptr, upstream.len, dbias.ptr, dbias.len,
                                                rows, cols))
 
+    def fused_chain(self, inputs, steps, dst: HipBuf, length: int, dst_start: int = 0):
+        """rt_fused_chain: `inputs` = [(buffer, start), ...]; `steps` = [("unary", op), ("scalar", op, value), ("binary", op, k),
+        ("binary_rev", op, k)] with k an index into `inputs`; dst[dst_start + i] = steps(inputs[0][start0 + i]) for i < length."""
+        dtype = dst.dtype
+        n = len(inputs)
+        ptrs = (C.c_void_p * max(n, 1))(*[b.ptr for b, _ in inputs])
+        lens = _u64s([b.len for b, _ in inputs])
+        starts = _u64s([st for _, st in inputs])
+        arr = (_ffi.ChainStep * max(len(steps), 1))()
+        for i, st in enumerate(steps):
+            kind = {"unary": 0, "scalar": 1, "binary": 2, "binary_rev": 3}[st[0]]
+            arr[i].kind = kind
+            arr[i].op = (UNARY, SCALAR, BINARY, BINARY)[kind][st[1]]
+            if kind == 1:
+                raw = _value(dtype, st[2]).tobytes()
+                for j, byte in enumerate(raw[:8]):
+                    arr[i].value[j] = byte
+            elif kind >= 2:
+                arr[i].operand = st[2]
+        _check(lib.rt_fused_chain(self._ctx, dtype, n, ptrs, lens, starts, length, len(steps), arr, dst.ptr, dst.len, dst_start))
+
     # ---- timing -----------------------------------------------------------------------------------------------------------
     def event(self):
         e = C.c_void_p()

@@ -27,6 +27,8 @@ C_TO_RUST = {
     "const uint64_t*": "*const u64",
     "uint64_t*": "*mut u64",
     "const int64_t*": "*const i64",
+    "const void*const*": "*const *const c_void",
+    "const rt_chain_step*": "*const rt_chain_step",
     "int32_t*": "*mut i32",
     "float*": "*mut f32",
     "const char*": "*const c_char",
@@ -91,6 +93,34 @@ def test_arguments_agree(name):
     for (pname, ctype), (_, rtype) in zip(c_params, r_params):
         assert ctype in C_TO_RUST, f"{name}({pname}): C type {ctype!r} has no Rust mapping in this test"
         assert C_TO_RUST[ctype] == rtype, f"{name}({pname}): {ctype} declared as {rtype}"
+
+
+def test_chain_step_struct_agrees():
+    """rt_chain_step crosses the boundary by pointer: same fields, order and machine types on both sides (24 bytes, no padding)."""
+    text = strip_c_comments(HEADER.read_text())
+    m = re.search(r"typedef\s+struct\s+rt_chain_step\s*\{(.*?)\}\s*rt_chain_step\s*;", text, flags=re.S)
+    c_fields = []
+    for decl in m.group(1).split(";"):
+        decl = " ".join(decl.split())
+        if not decl:
+            continue
+        fm = re.match(r"(\w+) (\w+)(?:\[(\d+)\])?$", decl)
+        c_fields.append((fm.group(2), fm.group(1), fm.group(3)))
+    rust = re.sub(r"//[^\n]*", " ", FFI.read_text())
+    rm = re.search(r"#\[repr\(C\)\]\s*(?:#\[derive\([^)]*\)\]\s*)?pub struct rt_chain_step\s*\{(.*?)\}", rust, flags=re.S)
+    r_fields = []
+    for decl in rm.group(1).split(","):
+        decl = " ".join(decl.split())
+        if decl:
+            name, ty = decl.replace("pub ", "").split(":")
+            r_fields.append((name.strip(), ty.strip()))
+    assert [f[0] for f in c_fields] == [f[0] for f in r_fields]
+    size = 0
+    for (name, ctype, count), (_, rtype) in zip(c_fields, r_fields):
+        want = {"int32_t": "i32", "uint8_t": "u8"}[ctype]
+        assert rtype == (f"[{want}; {count}]" if count else want), (name, rtype)
+        size += {"int32_t": 4, "uint8_t": 1}[ctype] * int(count or 1)
+    assert size == 24
 
 
 def header_constants():

@@ -32,6 +32,25 @@ def _both(hip, H, src, shape, dim, op, out_dtype=None):
     return hip.dump(a), hip.dump(b)
 
 
+def test_static_call_leaves_the_scratch_buffer_alone():
+    """On a fresh context a split reduction through rt_reduce_nd grows the context's scratch buffer (one device allocation, which the
+    allocator's counter sees); the same reduction through rt_reduce_nd_static, issued first, must not."""
+    from rtensors_amd import hip as H
+    be = H.Hip.new(0)
+    n = 1 << 22
+    src = be.alloc_from_slice(H.F32, np.ones(n, dtype=np.float32))
+    a, b = be.alloc(H.F32, 1), be.alloc(H.F32, 1)
+    be.sync()
+    before = be.mem_stats()["device_allocs"]
+    be.apply_reduce_contiguous_nd_static((src, (0, [n], [1])), b, 0, "sum")
+    assert be.mem_stats()["device_allocs"] == before, "the static entry point grew the context's scratch buffer"
+    be.apply_reduce_contiguous_nd((src, (0, [n], [1])), a, 0, "sum")
+    assert be.mem_stats()["device_allocs"] == before + 1, "the scratch growth of rt_reduce_nd is not counted: the check above proves nothing"
+    assert be.dump(a)[0] == be.dump(b)[0] == float(n)
+    del src, a, b
+    be.close()
+
+
 @pytest.mark.parametrize("dtype", ["f32", "i32", "f64"])
 def test_static_workspace_reduction_matches_rt_reduce_nd(hip, dtype):
     from rtensors_amd import hip as H
