@@ -91,7 +91,7 @@ def _build_host(force: bool) -> None:
     host = os.path.join(HERE, "host")
     src = os.path.join(host, "rt_host_capi.cpp")
     out = os.path.join(LIB, "librt_host.so")
-    deps = [src] + [os.path.join(host, h) for h in ("rt_meta.hpp", "rt_backend.hpp", "rt_tensor.hpp", "rt_grad.hpp")] + HEADERS[3:]
+    deps = [src] + [os.path.join(host, h) for h in ("rt_meta.hpp", "rt_backend.hpp", "rt_tensor.hpp", "rt_expr.hpp", "rt_grad.hpp")] + HEADERS[3:]
     if force or _stale(out, deps + [os.path.join(LIB, "librt_hip.so")]):
         cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra", "-o", out, src, "-L" + LIB, "-lrt_hip", "-Wl,-rpath,$ORIGIN"]
         r = subprocess.run(cmd, capture_output=True, text=True)

@@ -4,6 +4,7 @@
 #include <cstring>
 #include <string>
 
+#include "rt_expr.hpp"
 #include "rt_grad.hpp"
 
 using namespace rt;
@@ -150,6 +151,28 @@ int rth_set(void* a, int n, const uint64_t* idx, double v) {
 int rth_to_host(void* a, void* dst) { return guarded([&] { ((Tensor*)a)->to_host(dst); }); }
 int rth_dump_buffer(void* a, void* dst) { return guarded([&] { ((Tensor*)a)->dump_buffer(dst); }); }
 int rth_equals(void* a, void* b, int* out) { return guarded([&] { *out = ((Tensor*)a)->equals(*(Tensor*)b) ? 1 : 0; }); }
+
+// ---- expressions -----------------------------------------------------------------------------------------------------------
+// An elementwise expression starting at `first`: step k is (kinds[k], ops[k]) with values[k] for a scalar step and operands[k] (a tensor
+// handle) for a binary one; kinds are rt_chain_kind.  Evaluated through rt::Expr: fused launches where the operands allow, the ordinary
+// operators elsewhere.  *out_fused receives the number of fused launches.
+int rth_expr_eval(void* first, int nsteps, const int* kinds, const int* ops, const double* values, void* const* operands, void** out, int* out_fused) {
+    return guarded([&] {
+        Expr e(*(Tensor*)first);
+        for (int k = 0; k < nsteps; ++k) {
+            switch (kinds[k]) {
+                case RT_CHAIN_UNARY: e = e.unary(ops[k]); break;
+                case RT_CHAIN_SCALAR: e = e.scalar(ops[k], values[k]); break;
+                case RT_CHAIN_BINARY: e = e.binary((BinaryOpType)ops[k], *(Tensor*)operands[k]); break;
+                case RT_CHAIN_BINARY_REV: e = e.binary_rev((BinaryOpType)ops[k], *(Tensor*)operands[k]); break;
+                default: throw TensorError(ErrorKind::UnsupportedOperation, "unknown step kind");
+            }
+        }
+        int fused = 0;
+        *out = new Tensor(e.eval(&fused));
+        if (out_fused) *out_fused = fused;
+    });
+}
 
 // ---- the training step of the autograd configuration -----------------------------------------------------------------------
 // y = relu(x + bias); loss = mean_l1_loss(y, target); backward; SGD(lr) on bias (updated in place).

@@ -308,6 +308,51 @@ class Tensor:
         return bool(r.value)
 
 
+class Expr:
+    """A pending elementwise expression (rt::Expr of the host layer): the operators are recorded, `eval()` issues them as fused
+    passes where the operands allow (every operand read once, the result written once) and as the ordinary operators elsewhere.
+    `lazy(a) * 3.0 + b` ... `.relu()` ... `- 1.0` ... `.eval()`; `fused_launches` holds the number of fused launches of the last eval."""
+
+    def __init__(self, first: Tensor, steps=()):
+        self.first, self.steps, self.fused_launches = first, list(steps), None
+
+    def _with(self, step): return Expr(self.first, self.steps + [step])
+
+    def _bin(self, o, op, rev=False):
+        if isinstance(o, Tensor):
+            return self._with((3 if rev else 2, BINARY[op], 0.0, o))
+        if rev:
+            raise TypeError("scalar op expression is not an operator of the reference")
+        return self._with((1, SCALAR[op], float(o), None))
+
+    def __add__(self, o): return self._bin(o, "add")
+    def __sub__(self, o): return self._bin(o, "sub")
+    def __mul__(self, o): return self._bin(o, "mul")
+    def __truediv__(self, o): return self._bin(o, "div")
+    def rsub(self, t: Tensor): return self._bin(t, "sub", True)
+    def rdiv(self, t: Tensor): return self._bin(t, "div", True)
+    def unary(self, op): return self._with((0, UNARY[op], 0.0, None))
+    def scalar(self, op, v): return self._with((1, SCALAR[op], float(v), None))
+    def relu(self): return self.unary("relu")
+    def abs(self): return self.unary("abs")
+    def __neg__(self): return self.unary("neg")
+
+    def eval(self) -> Tensor:
+        n = len(self.steps)
+        kinds = (C.c_int * max(n, 1))(*[s[0] for s in self.steps])
+        ops = (C.c_int * max(n, 1))(*[s[1] for s in self.steps])
+        vals = (C.c_double * max(n, 1))(*[s[2] for s in self.steps])
+        opnds = (C.c_void_p * max(n, 1))(*[s[3]._p if s[3] is not None else None for s in self.steps])
+        p, fused = C.c_void_p(), C.c_int(0)
+        _ck(_h.rth_expr_eval(self.first._p, n, kinds, ops, vals, opnds, C.byref(p), C.byref(fused)))
+        self.fused_launches = fused.value
+        return Tensor(p, self.first.backend)
+
+
+def lazy(t: Tensor) -> Expr:
+    return Expr(t)
+
+
 def train_step(x: Tensor, bias: Tensor, target: Tensor, lr: float, mode: str = "sum", seed_with_loss: bool = True):
     """y = relu(x + bias); loss = mean_l1_loss(y, target); backward; SGD(lr) on bias in place.  Returns (loss, d_bias).
     mode 'sum' sums the upstream gradient over the broadcast dim; 'reference_literal' reproduces grad/backwards.rs:527."""

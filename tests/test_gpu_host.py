@@ -90,6 +90,64 @@ def test_random_programs_match_oracle(T, be):
             assert got.max().to_numpy().tobytes() == want.max().to_numpy().tobytes()
 
 
+def test_expressions_fuse_and_match_the_eager_operators(T, be):
+    """`lazy(a) * 3 + b ...`: the recorded expression must give, bit for bit, what the same operators give when each runs as its own
+    backend call (the oracle's OTensor), whether it is issued as fused launches (same-shape forward runs) or falls back to the
+    operators (broadcast operands, stepped views, steps a chain does not have)."""
+    rng = np.random.default_rng(77)
+    for trial in range(48):
+        dtype = ["f32", "f64", "i32", "i64", "u8", "i16"][trial % 6]
+        flt = dtype[0] == "f"
+        shape = [int(rng.integers(1, 20)) for _ in range(int(rng.integers(1, 4)))]
+        n = int(np.prod(shape))
+        mode = trial % 4                # 0, 1: same-shape operands; 2: b needs broadcasting; 3: a is a stepped view
+        sb = shape if mode != 2 else ([1] * (len(shape) - 1) + [shape[-1]])
+        va, vb, vc = rand_values(dtype, n, rng), rand_values(dtype, int(np.prod(sb)), rng), rand_values(dtype, n, rng)
+        if dtype == "u8":
+            va, vb, vc = np.abs(va).astype(np.uint8), np.abs(vb).astype(np.uint8), np.abs(vc).astype(np.uint8)
+        oa, ob, oc = OTensor.from_buf(dtype, va, shape), OTensor.from_buf(dtype, vb, sb), OTensor.from_buf(dtype, vc, shape)
+        ga, gb, gc = T.Tensor.from_buf(be, dtype, va, shape), T.Tensor.from_buf(be, dtype, vb, sb), T.Tensor.from_buf(be, dtype, vc, shape)
+        if mode == 3 and shape[0] > 1:
+            oa, ga = oa.slice(0, OSlice(None, None, 2)), ga.slice(0, T.Slice(None, None, 2))
+            oc, gc = oc.slice(0, OSlice(None, None, 2)), gc.slice(0, T.Slice(None, None, 2))
+            if mode != 2:
+                ob, gb = ob.slice(0, OSlice(None, None, 2)), gb.slice(0, T.Slice(None, None, 2))
+        # ((a * 3 + b).relu() - 1) * c - a, then |.|, then (floats) sqrt -- nine or ten steps: more than one launch when fused
+        want = ((((oa * 3) + ob).unary("relu") - 1) * oc - oa).unary("abs")
+        e = ((((T.lazy(ga) * 3) + gb).relu() - 1) * gc - ga).abs()
+        want = want * 2 + oc
+        e = e * 2 + gc
+        want = (want - ob) if mode != 2 else want
+        e = (e - gb) if mode != 2 else e
+        if flt:
+            want = want.unary("abs").unary("sqrt").unary("ln")           # `ln` is not available in a chain: the operator runs it
+            e = e.abs().unary("sqrt").unary("ln")
+        with np.errstate(all="ignore"):
+            got = e.eval()
+        assert got.shape == want.meta.shape
+        g, w = got.to_numpy().reshape(-1), want.to_numpy().reshape(-1)
+        if flt:
+            ok = np.isclose(g.astype(np.float64), w.astype(np.float64), rtol=1e-5, atol=1e-5, equal_nan=True)       # through ln: the reference's 1e-5
+            assert ok.all(), (trial, dtype, mode)
+            # the exact part, without the logarithm, bit for bit
+            e2 = (((((T.lazy(ga) * 3) + gb).relu() - 1) * gc - ga).abs() * 2 + gc)
+            w2 = (((((oa * 3) + ob).unary("relu") - 1) * oc - oa).unary("abs") * 2 + oc)
+            assert e2.eval().to_numpy().tobytes() == w2.to_numpy().tobytes(), (trial, dtype, mode)
+            fused = e2.fused_launches
+        else:
+            assert g.tobytes() == w.tobytes(), (trial, dtype, mode)
+            fused = e.fused_launches
+        if mode in (0, 1):
+            assert fused >= 1, (trial, dtype, "same-shape forward runs must take the fused path")
+        if mode == 3 and shape[0] > 2 and len(shape) > 1:
+            assert e.fused_launches is not None
+    # an expression without steps is a copy; a single unfusable step is just the operator
+    a = T.Tensor.from_buf(be, "f32", np.arange(6, dtype=np.float32), [2, 3])
+    assert T.lazy(a).eval().to_numpy().tobytes() == a.to_numpy().tobytes()
+    ev = T.lazy(a).unary("sin")
+    assert np.allclose(ev.eval().to_numpy(), np.sin(np.arange(6, dtype=np.float32)).reshape(2, 3), rtol=1e-5, atol=1e-6) and ev.fused_launches == 0
+
+
 def test_reduce_of_noncontiguous_and_reversed_views(T, be):
     x = np.arange(24, dtype=np.float64) * 0.5 - 3
     o, g = OTensor.from_buf("f64", x, [2, 3, 4]), T.Tensor.from_buf(be, "f64", x, [2, 3, 4])
@@ -452,6 +510,21 @@ def test_config2_chain_full_size(be, T):
             assert got.tobytes() == want.tobytes(), (dtype, start)
         del da, db, t, u, c
         hb.sync()
+    # the same expression through the host layer's lazy form: one fused launch, the same bits as the operators one by one
+    rng = np.random.default_rng(2)
+    n = (1 << 24) + 3
+    for dtype in ("f32", "f64", "i32"):
+        va, vb = rand_values(dtype, n, rng), rand_values(dtype, n, rng)
+        a, b = T.Tensor.from_buf(be, dtype, va, [n]), T.Tensor.from_buf(be, dtype, vb, [n])
+        eager = ((a * 3.0) + b).relu()
+        eager -= 1.0
+        e = ((T.lazy(a) * 3.0) + b).relu() - 1.0
+        fusedv = e.eval()
+        assert e.fused_launches == 1
+        assert fusedv.equals(eager)
+        npd = va.dtype
+        want = (np.maximum((va * npd.type(3)).astype(npd) + vb, 0).astype(npd) - npd.type(1)).astype(npd)
+        assert fusedv.to_numpy().tobytes() == want.tobytes()
 
 
 def test_config3_both_variants_agree_and_match_formula(be, T):
