@@ -15,6 +15,25 @@ def _m(meta: MetaTensor):
     return (meta.offset, list(meta.shape), list(meta.strides))
 
 
+# How the in-place unary / scalar / fill ops of a GTensor reach the backend:
+#   "nd"         the whole (offset, shape, strides) through the `_nd` entry point (what the binding's dispatching methods do: the
+#                library canonicalises the layout with signed strides)
+#   "three_way"  the dispatch of the trait's default methods (backend/mod.rs:15-94): `_contiguous(offset, size)` when the view is
+#                contiguous by the reference's |stride| rule (core/meta.rs:526-541), `_1d_strided(offset, stride, len)` when exactly one
+#                dim is longer than 1, else `_nd` -- the three entry points as the reference's own code would call them
+DISPATCH = "nd"
+
+
+def _three_way(meta: MetaTensor):
+    if meta.is_contiguous():
+        return "contiguous", (meta.offset, meta.size())
+    dims = meta.non_singleton_dims()
+    if len(dims) == 1:
+        _, size, stride = dims[0]
+        return "1d_strided", (meta.offset, stride, size)
+    return "nd", _m(meta)
+
+
 class GTensor:
     def __init__(self, backend, buf, meta: MetaTensor, is_view=False):
         self.backend, self.buf, self.meta, self.is_view = backend, buf, meta, is_view
@@ -109,6 +128,10 @@ class GTensor:
         return self
 
     def _scalar_assign(self, v, op):
+        if DISPATCH == "three_way":
+            entry, args = _three_way(self.meta)
+            getattr(self.backend, f"scalar_{entry}")(op, self.buf, v, *args)
+            return self
         self.backend.scalar_apply(op, self.buf, v, _m(self.meta))
         return self
 
@@ -127,16 +150,25 @@ class GTensor:
     def __itruediv__(self, o): return self._d(o, "div", True)
 
     def unary_inplace(self, op):
+        if DISPATCH == "three_way":
+            entry, args = _three_way(self.meta)
+            getattr(self.backend, f"unary_{entry}")(op, self.buf, *args)
+            self.last_path = entry
+            return self
         self.backend.apply_unary(op, self.buf, _m(self.meta))
         return self
 
     def unary(self, op): return self.owned().unary_inplace(op)
 
     def scalar_op_inplace(self, op, v):
-        self.backend.scalar_apply(op, self.buf, v, _m(self.meta))
-        return self
+        return self._scalar_assign(v, op)
 
-    def fill(self, v): self.backend.fill(self.buf, v, _m(self.meta))
+    def fill(self, v):
+        if DISPATCH == "three_way":
+            entry, args = _three_way(self.meta)
+            getattr(self.backend, f"fill_{entry}")(self.buf, v, *args)
+            return
+        self.backend.fill(self.buf, v, _m(self.meta))
 
     def matmul(self, other):
         """ops/linalg/matmul.rs:5-139 over the C ABI's rt_matmul."""

@@ -470,12 +470,20 @@ def test_reversed_view_is_walked_backwards_not_out_of_bounds(hip):
 CASES = golden_dsl.load("reference_vectors.json") + golden_dsl.load("reference_scalar_vectors.json") + golden_dsl.load("reference_view_vectors.json") + golden_dsl.load("reference_operand_vectors.json") + golden_dsl.load("reference_matmul_vectors.json")
 
 
+@pytest.mark.parametrize("dispatch", ["nd", "three_way"])
 @pytest.mark.parametrize("case", CASES, ids=lambda c: c["name"])
-def test_reference_vectors_on_gpu(hip, case):
+def test_reference_vectors_on_gpu(hip, case, dispatch, monkeypatch):
+    """The reference's own known answers.  `nd`: every in-place op goes down as (offset, shape, strides); `three_way`: through the
+    `_contiguous` / `_1d_strided` / `_nd` entry point that the trait's default dispatch (backend/mod.rs:15-94) would pick."""
+    import copy
+    import gpu_tensor
     from gpu_tensor import GTensor
+    monkeypatch.setattr(gpu_tensor, "DISPATCH", dispatch)
+    case = copy.deepcopy(case)
     env, err = golden_dsl.run_case(case, lambda dt, v, s: GTensor.from_buf(hip, dt, v, s), Slice, OErr)
-    for exp in case["expect"]:
-        exp.pop("path", None)
+    if dispatch == "nd":
+        for exp in case["expect"]:
+            exp.pop("path", None)             # which of the three loops ran is only defined for the three-way dispatch
     golden_dsl.check_case(case, env, err, lambda t: t.to_numpy(), lambda t, idx: t.get(idx),
                           lambda t: (t.meta.shape, t.meta.strides, t.meta.offset, t.meta.is_contiguous()))
 
