@@ -322,6 +322,21 @@ int32_t rt_event_destroy(rt_ctx* ctx, rt_event* ev);
 int32_t rt_mem_stats(rt_ctx* ctx, uint64_t* in_use, uint64_t* cached, uint64_t* device_allocs);
 int32_t rt_mem_trim(rt_ctx* ctx);                                /* hipFree everything in the free lists */
 
+/* ---- the host-side checks on their own (no counterpart in the reference's trait; they restate its remote server's validators,
+ * backend/remote/server.rs:241-295) -------------------------------------------------------------------------------------------------
+ * What every entry point does to a view before it launches anything, callable without a context or a device, so that the validation
+ * can be exercised (and fuzzed under a sanitizer) on a machine without a GPU.
+ *   rt_debug_check_view     the extent check (lowest and highest addressed element inside [0, len), 128-bit arithmetic) and, for a
+ *                           non-empty view, the canonical layout a kernel would get: size-1 dims dropped, dims flipped to non-negative
+ *                           strides, sorted by stride, adjacent dims merged.  out_shape / out_strides hold RT_MAX_RANK entries;
+ *                           RT_E_RANK when more dims remain.  *out_count = number of elements (0 for an empty view).
+ *   rt_debug_check_overlap  two views of one buffer with a common shape: *out_meet = their address ranges intersect, *out_same = they
+ *                           are the very same view (the one aliasing an output may have with an input). */
+int32_t rt_debug_check_view(uint64_t offset, int32_t rank, const uint64_t* shape, const int64_t* strides, uint64_t len,
+                            uint64_t* out_count, int32_t* out_rank, int64_t* out_shape, int64_t* out_strides, int64_t* out_offset);
+int32_t rt_debug_check_overlap(int32_t elem_size, int32_t rank, const uint64_t* shape, uint64_t a_offset, const int64_t* a_strides,
+                               uint64_t b_offset, const int64_t* b_strides, uint64_t len, int32_t* out_meet, int32_t* out_same);
+
 #ifdef __cplusplus
 }
 #endif

@@ -188,6 +188,10 @@ extern "C" {
                      dst: *mut c_void, dst_len: u64, b: u64, m: u64, k: u64, n: u64) -> i32;
     pub fn rt_gather(ctx: *mut rt_ctx, dtype: i32, src: *const c_void, src_len: u64, offset: u64, rank: i32,
                      shape: *const u64, strides: *const i64, dst: *mut c_void, dst_len: u64) -> i32;
+    pub fn rt_debug_check_view(offset: u64, rank: i32, shape: *const u64, strides: *const i64, len: u64, out_count: *mut u64,
+                               out_rank: *mut i32, out_shape: *mut i64, out_strides: *mut i64, out_offset: *mut i64) -> i32;
+    pub fn rt_debug_check_overlap(elem_size: i32, rank: i32, shape: *const u64, a_offset: u64, a_strides: *const i64,
+                                  b_offset: u64, b_strides: *const i64, len: u64, out_meet: *mut i32, out_same: *mut i32) -> i32;
     pub fn rt_event_create(ctx: *mut rt_ctx, out: *mut *mut rt_event) -> i32;
     pub fn rt_event_record(ctx: *mut rt_ctx, ev: *mut rt_event) -> i32;
     pub fn rt_event_elapsed_ms(ctx: *mut rt_ctx, start: *mut rt_event, stop: *mut rt_event, out_ms: *mut f32) -> i32;

@@ -300,3 +300,38 @@ def contiguity_type(meta: MetaTensor) -> str:
     if batch.rank() > 1 and not batch.is_flat():
         return "none"
     return inner
+
+
+def view_bounds(offset: int, shape: Sequence[int], strides: Sequence[int]) -> Tuple[int, int]:
+    """Lowest and highest buffer index a non-empty view addresses (exact integers)."""
+    lo = hi = offset
+    for d, s in zip(shape, strides):
+        span = (d - 1) * s
+        if span < 0:
+            lo += span
+        else:
+            hi += span
+    return lo, hi
+
+
+def check_extent(offset: int, shape: Sequence[int], strides: Sequence[int], length: int) -> Tuple[str, int]:
+    """`check_extent` of the reference's remote server (backend/remote/server.rs:241-275): ("ok", element count), ("invalid", 0) for a
+    malformed descriptor, ("out_of_bounds", 0) when an addressed element lies outside [0, length).  The element count is folded left
+    to right with `checked_mul` over usize, so an overflow met before a zero dim is an error.  Two rules are tighter than the
+    reference's: a buffer length or a non-empty view's element count beyond i64::MAX is refused (device kernels index with signed
+    64-bit integers)."""
+    if len(shape) != len(strides) or length > (1 << 63) - 1:
+        return "invalid", 0
+    n = 1
+    for d in shape:
+        n *= d
+        if n > (1 << 64) - 1:
+            return "invalid", 0
+    if any(d == 0 for d in shape):
+        return ("out_of_bounds", 0) if offset > length else ("ok", 0)
+    if n > (1 << 63) - 1:
+        return "invalid", 0
+    lo, hi = view_bounds(offset, shape, strides)
+    if lo < 0 or hi >= length:
+        return "out_of_bounds", 0
+    return "ok", n

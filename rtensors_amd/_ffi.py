@@ -18,7 +18,8 @@ SYMBOLS = [
     "rt_unary_contiguous", "rt_unary_1d_strided", "rt_unary_nd",
     "rt_scalar_contiguous", "rt_scalar_1d_strided", "rt_scalar_nd", "rt_unary_to", "rt_scalar_to",
     "rt_broadcast", "rt_reduce_flat", "rt_reduce_nd", "rt_reduce_nd_static", "rt_argmax_flat", "rt_argmax_nd", "rt_gather", "rt_matmul", "rt_fused_bias_relu", "rt_fused_l1_forward", "rt_fused_l1_relu_backward",
-    "rt_fused_bias_relu_l1", "rt_fused_l1_relu_backward_t", "rt_fused_chain",
+    "rt_fused_bias_relu_l1", "rt_fused_l1_relu_backward_t", "rt_fused_chain", "rt_debug_check_view", "rt_debug_check_overlap",
+    "rt_debug_check_view", "rt_debug_check_overlap",
     "rt_event_create", "rt_event_record", "rt_event_elapsed_ms", "rt_event_destroy", "rt_mem_stats", "rt_mem_trim",
 ]
 
@@ -60,6 +61,8 @@ _SIGS = {
     "rt_fused_bias_relu_l1": [vp, i32, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, u64, u64],
     "rt_fused_l1_relu_backward_t": [vp, i32, vp, u64, vp, u64, vp, u64, vp, u64, u64, u64],
     "rt_fused_chain": [vp, i32, i32, vpp, u64p, u64p, u64, i32, C.POINTER(ChainStep), vp, u64, u64],
+    "rt_debug_check_view": [u64, i32, u64p, i64p, u64, u64p, i32p, i64p, i64p, i64p],
+    "rt_debug_check_overlap": [i32, i32, u64p, u64, i64p, u64, i64p, u64, i32p, i32p],
     "rt_event_create": [vp, vpp], "rt_event_record": [vp, vp], "rt_event_elapsed_ms": [vp, vp, vp, C.POINTER(C.c_float)],
     "rt_event_destroy": [vp, vp], "rt_mem_stats": [vp, u64p, u64p, u64p], "rt_mem_trim": [vp],
 }

@@ -507,6 +507,7 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
             size_t blocks = rt_tilemap_blocks(m, nvec, kCBlock2);
             if (blocks < 1) blocks = 1;                            // fewer elements than a vector: edges only
             if (blocks > 0x7fffffffull) return rt_fail(RT_E_INVALID, "broadcast: %zu elements is too long for one launch", n);
+            RT_TRY(rt_check_edges("broadcast", head, nvec, (size_t)N, tail, n, kCBlock2));
             hipLaunchKernelGGL((bin_contig_kernel<T, OP>), dim3((unsigned)blocks), dim3(kCBlock2), 0, s,
                                reinterpret_cast<const Vec16<T>*>(lp + head), reinterpret_cast<const Vec16<T>*>(rp + head),
                                reinterpret_cast<Vec16<T>*>(dp + head), nvec, (uint32_t)head, (uint32_t)tail, m, fault_of<T, OP>(ctx));

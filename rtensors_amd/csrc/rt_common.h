@@ -103,6 +103,16 @@ static inline int rt_elem_size(int dtype) {
     return 0;
 }
 
+// The contiguous kernels hand the `head` elements before their 16-byte vector body and the `tail` elements after it to lanes of the
+// first and the last block, which compare those counts with the lane index.  A count of a block size or more, or pieces that do not
+// add up to the run, would make lanes store past the run: checked on the host before every such launch.
+inline int32_t rt_check_edges(const char* what, size_t head, size_t nvec, size_t per_vec, size_t tail, size_t n, unsigned block) {
+    if (head >= block || tail >= block || tail >= per_vec || nvec > (SIZE_MAX - head - tail) / per_vec || head + nvec * per_vec + tail != n)
+        return rt_fail(RT_E_INVALID, "%s: launch geometry does not cover the run (head %zu, %zu vectors of %zu, tail %zu, run %zu, block %u)", what, head, nvec,
+                       per_vec, tail, n, block);
+    return RT_OK;
+}
+
 // ---- descriptor validation and canonicalisation (host) -----------------------------------------------------------
 // check_extent of the reference's remote server (backend/remote/server.rs:241-270): lowest and highest addressed
 // element must lie inside [0, len).  Returns the element count through *count (0 when any dim is 0).

@@ -524,6 +524,7 @@ int32_t launch_contig(rt_ctx* ctx, T* p, size_t n, F f) {
     size_t blocks = rt_tilemap_blocks(m, nvec, bs);
     if (blocks < 1) blocks = 1;                                           // a run shorter than a vector: edges only
     if (blocks > 0x7fffffffull) return rt_fail(RT_E_INVALID, "contiguous run of %zu elements is too long for one launch", n);
+    RT_TRY(rt_check_edges("elementwise", head, nvec, N, tail, n, bs));
     hipLaunchKernelGGL((ew_contig_kernel<T, F>), dim3((unsigned)blocks), dim3(bs), 0, ctx->stream,
                        reinterpret_cast<Vec16<T>*>(p + head), nvec, (uint32_t)head, (uint32_t)tail, m, f);
     RT_HIP(hipGetLastError());
@@ -558,6 +559,7 @@ int32_t launch_contig_out(rt_ctx* ctx, const T* s, T* d, size_t n, F f) {
     size_t blocks = rt_tilemap_blocks(m, nvec, 256);
     if (blocks < 1) blocks = 1;
     if (blocks > 0x7fffffffull) return rt_fail(RT_E_INVALID, "contiguous run of %zu elements is too long for one launch", n);
+    RT_TRY(rt_check_edges("elementwise", head, nvec, N, tail, n, 256));
     hipLaunchKernelGGL((ew_contig_out_kernel<T, F>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, s + head, d + head, nvec, (uint32_t)head,
                        (uint32_t)tail, m, f);
     RT_HIP(hipGetLastError());
@@ -1043,8 +1045,7 @@ int32_t chain_typed(rt_ctx* ctx, int n_inputs, const void* const* inputs, const 
     size_t blocks = rt_tilemap_blocks(m, nvec, 256);
     if (blocks < 1) blocks = 1;
     if (blocks > 0x7fffffffull) return rt_fail(RT_E_INVALID, "fused chain: a run of %llu elements is too long for one launch", (unsigned long long)len);
-    // the edge arguments are compared with the lane index inside the kernel: they must be below the block size
-    if (head >= 256 || tail >= 256 || head + nvec * N + tail != len) return rt_fail(RT_E_INVALID, "fused chain: inconsistent launch geometry");
+    RT_TRY(rt_check_edges("fused chain", head, nvec, N, tail, (size_t)len, 256));
     CtxGuard g(ctx);
     hipLaunchKernelGGL((chain_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, in, d + head, nvec, (uint32_t)head, (uint32_t)tail, m, prog);
     RT_HIP(hipGetLastError());

@@ -10,15 +10,17 @@ int32_t rt_check_extent(const char* what, uint64_t offset, int rank, const uint6
                         uint64_t len, uint64_t* count) {
     if (rank < 0 || rank > RT_MAX_INPUT_RANK) return rt_fail(RT_E_INVALID, "%s: rank %d outside 0..%d", what, rank, RT_MAX_INPUT_RANK);
     if (rank > 0 && (!shape || !strides)) return rt_fail(RT_E_INVALID, "%s: null shape/strides", what);
+    // every address of a view that passes lies in [0, len): with len within int64 the signed 64-bit arithmetic of the canonicalisation
+    // and of the kernels cannot overflow
+    if (len > (uint64_t)INT64_MAX) return rt_fail(RT_E_INVALID, "%s: a buffer of %llu elements is beyond signed 64-bit indexing", what, (unsigned long long)len);
+    // element count as the reference folds it (checked_mul over usize, left to right: a product that overflows before a zero dim is
+    // met is refused, backend/remote/server.rs:246-248, 272-275)
     unsigned __int128 n = 1;
     bool empty = false;
     for (int i = 0; i < rank; ++i) {
         if (shape[i] == 0) empty = true;
         n *= shape[i];
-        if (n > (unsigned __int128)INT64_MAX) {
-            // keep multiplying only to detect zeros; an overflowing non-empty shape is refused below
-            n = (unsigned __int128)INT64_MAX + 1;
-        }
+        if (n > (unsigned __int128)UINT64_MAX) return rt_fail(RT_E_INVALID, "%s: shape has too many elements", what);
     }
     if (empty) {
         if (offset > len) return rt_fail(RT_E_OUT_OF_BOUNDS, "%s: offset %llu is past the end of a buffer with %llu elements", what,
@@ -26,6 +28,7 @@ int32_t rt_check_extent(const char* what, uint64_t offset, int rank, const uint6
         if (count) *count = 0;
         return RT_OK;
     }
+    // kernels index with signed 64-bit arithmetic
     if (n > (unsigned __int128)INT64_MAX) return rt_fail(RT_E_INVALID, "%s: shape has too many elements", what);
     __int128 lo = (__int128)offset, hi = (__int128)offset;
     for (int i = 0; i < rank; ++i) {
@@ -139,5 +142,43 @@ int32_t rt_collapse_big(rt_ctx* ctx, int nops, int rank, const uint64_t* shape, 
     out->rank = r;
     out->words = (const int64_t*)dev;
     for (int o = 0; o < 3; ++o) out->offset[o] = off[o];
+    return RT_OK;
+}
+
+// ---- the host-side checks on their own (no context, no device) ---------------------------------------------------------------------
+extern "C" int32_t rt_debug_check_view(uint64_t offset, int32_t rank, const uint64_t* shape, const int64_t* strides, uint64_t len, uint64_t* out_count,
+                                       int32_t* out_rank, int64_t* out_shape, int64_t* out_strides, int64_t* out_offset) {
+    uint64_t count = 0;
+    RT_TRY(rt_check_extent("view", offset, rank, shape, strides, len, &count));
+    if (out_count) *out_count = count;
+    if (out_rank) *out_rank = 0;
+    if (count == 0) return RT_OK;
+    NdDesc d;
+    const int64_t* sp[1] = {strides};
+    RT_TRY(rt_collapse(1, rank, shape, sp, &offset, /*reorder=*/true, 0, &d));
+    if (out_rank) *out_rank = d.rank;
+    for (int i = 0; i < d.rank; ++i) {
+        if (out_shape) out_shape[i] = d.shape[i];
+        if (out_strides) out_strides[i] = d.stride[0][i];
+    }
+    if (out_offset) *out_offset = d.offset[0];
+    return RT_OK;
+}
+
+extern "C" int32_t rt_debug_check_overlap(int32_t elem_size, int32_t rank, const uint64_t* shape, uint64_t a_offset, const int64_t* a_strides, uint64_t b_offset,
+                                          const int64_t* b_strides, uint64_t len, int32_t* out_meet, int32_t* out_same) {
+    if (elem_size < 1 || elem_size > 16) return rt_fail(RT_E_INVALID, "element size %d", elem_size);
+    uint64_t ca = 0, cb = 0;
+    RT_TRY(rt_check_extent("view a", a_offset, rank, shape, a_strides, len, &ca));
+    RT_TRY(rt_check_extent("view b", b_offset, rank, shape, b_strides, len, &cb));
+    int meet = 0, same = 0;
+    if (ca != 0) {
+        // any base address will do: both views live in one buffer
+        const void* base = reinterpret_cast<const void*>((uintptr_t)1 << 40);
+        meet = rt_spans_meet(rt_view_span(base, elem_size, a_offset, rank, shape, a_strides), rt_view_span(base, elem_size, b_offset, rank, shape, b_strides)) ? 1 : 0;
+        same = rt_same_view(base, a_offset, a_strides, base, b_offset, b_strides, rank, shape) ? 1 : 0;
+    }
+    if (out_meet) *out_meet = meet;
+    if (out_same) *out_same = same;
     return RT_OK;
 }

@@ -386,6 +386,7 @@ static int32_t device_copy(rt_ctx* ctx, void* dst, const void* src, size_t bytes
         RT_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx->stream));
         return RT_OK;
     }
+    RT_TRY(rt_check_edges("copy", head, nvec, 16, tail, bytes, 256));
     hipLaunchKernelGGL(rt_copy_vec_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (const uint8_t*)src + head, (uint8_t*)dst + head, nvec,
                        (uint32_t)head, (uint32_t)tail, m);
     RT_HIP(hipGetLastError());

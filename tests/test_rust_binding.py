@@ -30,6 +30,7 @@ C_TO_RUST = {
     "const void*const*": "*const *const c_void",
     "const rt_chain_step*": "*const rt_chain_step",
     "int32_t*": "*mut i32",
+    "int64_t*": "*mut i64",
     "float*": "*mut f32",
     "const char*": "*const c_char",
     "int32_t": "i32",
