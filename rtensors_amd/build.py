@@ -19,21 +19,32 @@ OBJ = os.path.join(HERE, "_build")
 LIB = os.path.join(HERE, "lib")
 ARCH = os.environ.get("RT_HIP_ARCH", "gfx950")
 
-# -ffp-contract=off / no fast-math: float results must be the plain IEEE operations the reference's Cpu backend does.
-# -packed-fp32-ops is switched off on purpose (scalar v_add/v_mul/v_fma f32 only).
-FLAGS = [
-    "-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17", "-ffp-contract=off", "-fno-fast-math",
-    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wno-unused-function",
-    # the device code of each object is stored zstd-compressed and unpacked by the HIP runtime when the library is loaded
-    "--offload-compress",
-]
 
+
+def read_build_flags(path: str = os.path.join(CSRC, "build_flags.txt"), arch: str = ARCH) -> dict:
+    """The sections of csrc/build_flags.txt (compile flags, sources, headers, link flags): the one description of the build that
+    this builder and the Rust-side build script (integration/rust/build_hip.rs) both read."""
+    out, cur = {}, None
+    for ln in open(path):
+        ln = ln.strip()
+        if not ln or ln.startswith("#"):
+            continue
+        if ln.startswith("[") and ln.endswith("]"):
+            cur = ln[1:-1]
+            out[cur] = []
+        else:
+            out[cur].append(ln.replace("{arch}", arch))
+    return out
+
+
+_B = read_build_flags()
+FLAGS = _B["compile"]
+LINK = _B["link"]
 LIBS = {
-    "librt_hip.so": ["rt_runtime.hip", "rt_layout.hip", "rt_elementwise.hip", "rt_broadcast.hip", "rt_broadcast_tile.hip", "rt_reduce.hip", "rt_reduce_stat.hip", "rt_misc.hip", "rt_matmul.hip", "rt_fused.hip"],
-    "librt_datagen.so": ["rt_datagen.hip"],
+    "librt_hip.so": _B["sources"],
+    "librt_datagen.so": ["rt_datagen.hip"],          # synthetic-data generator of the benchmark and the tests, not part of the backend
 }
-HEADERS = [os.path.join(CSRC, "rt_common.h"), os.path.join(CSRC, "rt_broadcast_common.h"), os.path.join(CSRC, "rt_div128.h"),
-           os.path.join(HERE, "..", "include", "rt_hip.h")]
+HEADERS = [os.path.normpath(os.path.join(CSRC, h)) for h in _B["headers"]]
 
 
 def _stale(target: str, deps) -> bool:
@@ -76,7 +87,8 @@ def build(force: bool = False, jobs: int = 8) -> None:
         out = os.path.join(LIB, lib)
         deps = [objs[s] for s in ss]
         if force or _stale(out, deps):
-            r = subprocess.run(["hipcc", f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", out] + deps + ["-ldl", "-lpthread"], capture_output=True, text=True)
+            r = subprocess.run(["hipcc"] + [f for f in LINK if not f.startswith("-l")] + ["-o", out] + deps + [f for f in LINK if f.startswith("-l")],
+                               capture_output=True, text=True)
             if r.returncode != 0:
                 raise RuntimeError(f"link of {lib} failed:\n{_filter(r.stdout + r.stderr)}")
             print(f"[build] linked {lib}", file=sys.stderr)
@@ -91,7 +103,7 @@ def _build_host(force: bool) -> None:
     host = os.path.join(HERE, "host")
     src = os.path.join(host, "rt_host_capi.cpp")
     out = os.path.join(LIB, "librt_host.so")
-    deps = [src] + [os.path.join(host, h) for h in ("rt_meta.hpp", "rt_backend.hpp", "rt_tensor.hpp", "rt_expr.hpp", "rt_grad.hpp")] + HEADERS[3:]
+    deps = [src] + [os.path.join(host, h) for h in ("rt_meta.hpp", "rt_backend.hpp", "rt_tensor.hpp", "rt_expr.hpp", "rt_grad.hpp")] + [h for h in HEADERS if h.endswith('rt_hip.h')]
     if force or _stale(out, deps + [os.path.join(LIB, "librt_hip.so")]):
         cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra", "-o", out, src, "-L" + LIB, "-lrt_hip", "-Wl,-rpath,$ORIGIN"]
         r = subprocess.run(cmd, capture_output=True, text=True)

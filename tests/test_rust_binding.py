@@ -164,33 +164,79 @@ def test_constants_agree():
         assert not missing, missing
 
 
-UNARY = ["neg", "relu", "sigmoid", "silu", "tanh", "abs", "sqrt", "ln", "expm1", "ln1p", "floor", "ceil", "round", "trunc",
-         "sin", "cos", "tan", "asin", "acos", "atan", "sinh", "cosh", "asinh", "acosh", "atanh", "rsqrt", "reciprocal",
-         "square", "cube", "exp", "sign"]
-SCALAR = ["add", "sub", "mul", "div", "log", "log1p", "leaky_relu", "elu"]
-PLAIN = ["device_type", "alloc_from_slice", "alloc", "copy_from_slice", "copy_range_within", "read", "write", "len", "copy",
-         "dump", "convert", "new", "fill_nd", "fill_1d_strided", "fill_contiguous", "broadcast", "apply_reduce_contiguous_flat",
-         "apply_reduce_contiguous_nd", "apply_argmax_contiguous_flat", "apply_argmax_contiguous_nd", "apply_conv_2d"]
+def _trait_golden():
+    import json
+    return json.loads((ROOT / "tests" / "golden" / "reference_trait_signatures.json").read_text())
 
 
-def test_every_trait_method_is_implemented():
+def _impl_methods(header_regex):
+    import rust_sig
+    text = rust_sig.expand(rust_sig.strip_comments(HIP.read_text()))
+    return {m["name"]: m for m in rust_sig.functions(rust_sig.block_of(text, header_regex))}
+
+
+def test_every_trait_method_is_implemented_with_the_trait_s_signature():
+    """`impl Backend for Hip` against the reference's trait, signature by signature (tests/golden/reference_trait_signatures.json, written
+    from backend/mod.rs:216-485 with its two macros expanded; hip.rs's own `hip_unary!` / `hip_scalar!` are expanded the same way): every
+    method the trait leaves without a body is implemented, nothing is implemented that the trait does not have, and each method's
+    generics, argument names, argument types, return type and `where` clause equal the trait's token for token."""
+    golden = _trait_golden()
+    impl = _impl_methods(r"impl\s+Backend\s+for\s+Hip\s*\{")
+    trait = {m["name"]: m for m in golden["Backend"]}
+    assert len(trait) == 181                                  # 25 plain methods + (31 unary + 8 scalar ops) x 4
+    missing = [n for n, m in trait.items() if not m["has_body"] and n not in impl]
+    assert not missing, missing
+    extra = [n for n in impl if n not in trait]
+    assert not extra, extra
+    for name, got in impl.items():
+        want = trait[name]
+        for field in ("generics", "args", "ret", "where"):
+            w, g = want[field], got[field]
+            if field == "ret" and w == "Self":
+                assert g in ("Self", "Hip"), (name, g)
+                continue
+            if field == "args":
+                g = [[a.lstrip("_") or a, t] for a, t in g]      # an unused argument may carry a leading underscore
+            assert g == w, f"{name}: {field} is `{g}`, the trait has `{w}`"
+        assert got["has_body"], name
+    # the dispatching methods are overridden on purpose (signed-stride canonicalisation in the library instead of the |stride| test)
+    for name in ["fill"] + [n for n in trait if n.startswith("apply_") and trait[n]["has_body"] and n not in ("apply_reduce", "apply_argmax")] + \
+            [n for n in trait if n.startswith("scalar_apply_") and trait[n]["has_body"]]:
+        assert name in impl, f"{name}: the trait's default dispatch would be used"
+    mm = _impl_methods(r"impl\s*<\s*T\s*:\s*TensorValue\s*>\s*BackendMatMul\s*<\s*T\s*>\s*for\s+Hip\s*\{")
+    want = golden["BackendMatMul"][0]
+    got = mm["matmul"]
+    for field in ("generics", "args", "ret", "where"):
+        assert got[field] == want[field], ("matmul", field, got[field], want[field])
     text = HIP.read_text()
-    body = text[text.index("impl Backend for Hip"):text.index("impl<T: TensorValue> BackendMatMul<T> for Hip")]
-    for name in PLAIN:
-        assert re.search(rf"\bfn {name}\b", body), name
-    # the two macros produce the four methods of each op; each op is invoked once with the header's code of the same name
-    for macro, prefix in (("hip_unary", "apply_"), ("hip_scalar", "scalar_apply_")):
-        mdef = text[text.index(f"macro_rules! {macro}"):]
-        mdef = mdef[:mdef.index("\n}\n")]
-        for suffix in ("", "_nd", "_1d_strided", "_contiguous"):
-            want = f"[<{prefix} $name {suffix}>]" if suffix else f"[<{prefix} $name>]"
-            assert want in mdef, (macro, suffix)
-    for name in UNARY:
-        assert re.search(rf"hip_unary! \{{{name}, ffi::RT_U_{name.upper()}[,}}]", body), name
-    for name in SCALAR:
-        assert re.search(rf"hip_scalar! \{{{name}, ffi::RT_S_{name.upper()}[,}}]", body), name
-    assert "fn matmul" in text[text.index("BackendMatMul<T> for Hip"):]
     assert "todo!" not in text.replace("never `todo!()`", "") and "unimplemented!" not in text
+
+
+def test_signature_parser_on_known_text():
+    """The parser itself, on a trait written out here: macro expansion, tuple arguments, `where` clauses, default bodies."""
+    import rust_sig
+    src = """
+    macro_rules! cabal { ($name:ident $( where $($extra:tt)+ )?) => { paste! {
+        fn [<apply_ $name>]<T: TensorValue>(&self, buf: &mut Self::Buf<T>, meta: &MetaTensor) -> Result<(), TensorError>
+        $( where $($extra)+ )? { body!(self, [<apply_ $name _nd>]) }
+        fn [<apply_ $name _nd>]<T: TensorValue>(&self, buf: &mut Self::Buf<T>, shape: &[usize]) -> Result<(), TensorError> $( where $($extra)+ )? ;
+    } }; }
+    pub trait B: Send { type Buf<T: V>: Send;
+        fn device_type() -> crate::core::primitives::DeviceType; // a comment with fn fake() in it
+        fn bc<T: V>(&self, left: (*const Self::Buf<T>, &MetaTensor), op: Op) -> Result<(), E>;
+        cabal!{neg where T: std::ops::Neg<Output = T>}
+        cabal!{relu}
+        fn with_body(&self) -> usize { if x { 1 } else { 2 } }
+    }"""
+    fns = rust_sig.functions(rust_sig.block_of(rust_sig.expand(rust_sig.strip_comments(src)), r"pub\s+trait\s+B\s*:[^{]*\{"))
+    by = {f["name"]: f for f in fns}
+    assert list(by) == ["device_type", "bc", "apply_neg", "apply_neg_nd", "apply_relu", "apply_relu_nd", "with_body"]
+    assert by["device_type"]["ret"] == "DeviceType" and not by["device_type"]["has_body"]
+    assert by["bc"]["args"] == [["& self", ""], ["left", "( * const Self :: Buf < T > , & MetaTensor )"], ["op", "Op"]]
+    assert by["apply_neg"]["where"] == "T : Neg < Output = T >" and by["apply_neg"]["has_body"]
+    assert by["apply_neg_nd"]["where"] == "T : Neg < Output = T >" and not by["apply_neg_nd"]["has_body"]
+    assert by["apply_relu"]["where"] == "" and by["apply_relu_nd"]["args"][2] == ["shape", "& [ usize ]"]
+    assert by["with_body"]["has_body"] and by["with_body"]["ret"] == "usize"
 
 
 def test_binding_calls_only_declared_functions():
@@ -201,3 +247,26 @@ def test_binding_calls_only_declared_functions():
     for name in ("rt_broadcast", "rt_reduce_nd", "rt_reduce_flat", "rt_argmax_nd", "rt_argmax_flat", "rt_unary_nd",
                  "rt_scalar_nd", "rt_fill_nd", "rt_convert", "rt_equal", "rt_matmul", "rt_copy_range_within"):
         assert name in used, name
+
+
+def test_build_description_is_shared_by_both_builders():
+    """csrc/build_flags.txt is the one description of how librt_hip.so is built: the Python builder uses exactly its entries, the
+    Rust-side build block (integration/rust/build_hip.rs) reads the same sections, every listed file exists and every .hip source of
+    the library is listed."""
+    import os
+    from rtensors_amd import build as B
+    csrc = ROOT / "rtensors_amd" / "csrc"
+    b = B.read_build_flags(str(csrc / "build_flags.txt"), "gfx950")
+    assert set(b) == {"compile", "sources", "headers", "link"}
+    assert B.FLAGS == B.read_build_flags()["compile"] and B.LIBS["librt_hip.so"] == b["sources"] and B.LINK == B.read_build_flags()["link"]
+    for f in b["sources"] + b["headers"]:
+        assert (csrc / f).exists(), f
+    on_disk = sorted(p.name for p in csrc.glob("*.hip") if p.name != "rt_datagen.hip")
+    assert sorted(b["sources"]) == on_disk
+    assert sorted(h for h in b["headers"] if "/" not in h) == sorted(p.name for p in csrc.glob("*.h"))
+    for flag in ("-ffp-contract=off", "-fno-fast-math", "--offload-arch=gfx950", "-packed-fp32-ops"):
+        assert flag in b["compile"], flag
+    rs = (ROOT / "integration" / "rust" / "build_hip.rs").read_text()
+    for needle in ("build_flags.txt", "HIPCC_PATH", "RT_HIP_ARCH", "RT_HIP_LIB_DIR", 'b["compile"]', 'b["sources"]', 'b["headers"]', 'b["link"]', "{arch}",
+                   "cargo:rustc-link-lib=dylib=rt_hip", "cargo:rerun-if-changed"):
+        assert needle in rs, needle
