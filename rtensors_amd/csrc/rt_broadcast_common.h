@@ -71,7 +71,7 @@ template <int OP, class T> __device__ __forceinline__ T bin_apply(T a, T b, int3
             }
             if constexpr (sizeof(T) <= 2) return rt_div_narrow<T>(a, b);
             else if constexpr (sizeof(T) == 4) return rt_div32<T>(a, b);
-            else return (T)(a / b);
+            else return rt_div64<T>(a, b);
         }
     }
 }

@@ -8,6 +8,7 @@
 // read-modify-write ops and N*sizeof(T) for fill.
 #include "rt_common.h"
 #include "rt_div128.h"
+#include "rt_math64.h"
 
 #include <type_traits>
 
@@ -58,10 +59,12 @@ template <class T> __device__ __forceinline__ T w_div(T a, T b) {
         if (b == 0) return 0;
         if (b == (T)-1) return w_sub<T>((T)0, a);
         if constexpr (sizeof(T) <= 2) return rt_div_narrow<T>(a, b);
+        else if constexpr (sizeof(T) == 8) return rt_div64<T>(a, b);
         else return (T)(a / b);
     } else {
         if (b == 0) return 0;
         if constexpr (sizeof(T) <= 2) return rt_div_narrow<T>(a, b);
+        else if constexpr (sizeof(T) == 8) return rt_div64<T>(a, b);
         else return (T)(a / b);
     }
 }
@@ -88,7 +91,7 @@ __device__ __forceinline__ double m_exp(double x) { return exp(x); }
 __device__ __forceinline__ float m_expm1(float x) { return expm1f(x); }
 __device__ __forceinline__ double m_expm1(double x) { return expm1(x); }
 __device__ __forceinline__ float m_log(float x) { return logf(x); }
-__device__ __forceinline__ double m_log(double x) { return log(x); }
+__device__ __forceinline__ double m_log(double x) { return rt_log_f64(x); }      // by hand: the library routine is ALU-bound (rt_math64.h)
 // ln(1 + x) in f32 from the plain logarithm (Kahan): with u = fl(1 + x), ln(u) * x / (u - 1) cancels the rounding of u, a few ulp over
 // the whole range and about twice as fast as the library routine, which left the 1 GiB pass ALU-bound at 0.47 of the memory rate.
 __device__ __forceinline__ float m_log1p(float x) {
@@ -97,7 +100,7 @@ __device__ __forceinline__ float m_log1p(float x) {
     if (u == __builtin_inff()) return u;
     return logf(u) * (x / (u - 1.0f));
 }
-__device__ __forceinline__ double m_log1p(double x) { return log1p(x); }
+__device__ __forceinline__ double m_log1p(double x) { return rt_log1p_f64(x); }
 __device__ __forceinline__ float m_sqrt(float x) { return sqrtf(x); }
 __device__ __forceinline__ double m_sqrt(double x) { return sqrt(x); }
 __device__ __forceinline__ float m_sin(float x) { return sinf(x); }
