@@ -153,6 +153,19 @@ inline RowTiling rt_row_tiling(uint64_t first, const int64_t* strides, int nstri
     return t;
 }
 
+// LDS pitch, in elements, of the rows that the short-row reductions stage in a tile.  Lanes (or lane groups) walk different rows, so
+// two rows whose starts are a multiple of 32 words apart meet in one bank.  The row length itself is the pitch -- the tile is then a
+// plain copy of the run, written with 16-byte stores -- when that puts at most two rows on a bank (R words with gcd(R, 32) <= 2:
+// rows of 10 f32 staged this way instead of element by element: logsumexp 0.65 -> see the measured table), and always for 1- and
+// 2-byte elements; other lengths are padded to an odd pitch.
+inline uint32_t rt_tile_pitch(uint32_t R, uint32_t esize) {
+    if (esize < 4) return R;
+    const uint64_t words = (uint64_t)R * (esize / 4);
+    uint64_t g = words, h = 32;
+    while (h) { const uint64_t t = g % h; g = h; h = t; }
+    return g <= 2 ? R : (R | 1u);
+}
+
 // Launches whose index arithmetic is 32-bit take fewer than 2^31 elements.  A larger N-d descriptor is cut along its outermost dim into
 // slices below that bound (`fn(sub, count_of_sub)` is called for each, in order); when one index of that dim alone is too large the
 // dim is dropped and every index becomes a descriptor of its own, to be cut further by the callee.  Returns the first non-zero status.

@@ -126,10 +126,49 @@ __device__ __forceinline__ double m_trunc(double x) { return trunc(x); }
 __device__ __forceinline__ float m_abs(float x) { return fabsf(x); }
 __device__ __forceinline__ double m_abs(double x) { return fabs(x); }
 
+// a / ln(base).  ln(base) is one value for the whole launch.  f32: the plain division.  f64: the general division sequence is some 25
+// instructions per element, so the quotient is formed from the refined reciprocal with one correction step (the correctly rounded
+// quotient in all but rare cases, within one ulp always); a base whose logarithm is zero, infinite, NaN or beyond 2^+-500 keeps the
+// general division, which alone gets those right.
+__device__ __forceinline__ float over_log_base(float a, float base) { return a / m_log(base); }
+__device__ __forceinline__ double over_log_base(double a, double base) {
+    const double d = m_log(base);
+    const double ad = fabs(d);
+    if (!(ad > 0x1p-500 && ad < 0x1p500)) return a / d;        // wave-uniform: d does not depend on the element
+    const double r = rt_rcp_f64(d);
+    const double q = a * r;
+    const double q2 = __builtin_fma(__builtin_fma(-d, q, a), r, q);
+    return __builtin_isfinite(q) ? q2 : q;                      // a = +-inf: q is the answer, the correction would make it NaN
+}
+
 // ---- functors ---------------------------------------------------------------------------------------------------
 // A functor over 1-byte elements may offer `packed`: the same op on four elements in one 32-bit word (rt_common.h).
+// kVectors: 16-byte vectors a lane of the contiguous kernels handles.  One for the ops that are a few instructions per element: the
+// wave is gone as soon as its load has come back and been stored.  Four for the ops whose arithmetic takes as long as the memory
+// round trip itself (f64 transcendental functions, division-heavy maps): a wave that computes for a microsecond holds its slot
+// without having anything in flight, and with one vector per lane the chip runs out of slots before it runs out of bandwidth (f64 ln
+// stayed at 0.70 of peak although its ~60 instructions per element are well inside the ALU budget); with all four loads issued first,
+// the arithmetic of one vector runs under the latency of the next ones (f64 ln 0.70 -> 0.75, atan 0.70 -> 0.77, sinh 0.70 -> 0.78).
+template <int OP, class T> constexpr int unary_vectors() {
+    if (std::is_same<T, double>::value) {
+        switch (OP) {
+            case RT_U_SIGMOID: case RT_U_SILU: case RT_U_TANH: case RT_U_LN: case RT_U_LN1P: case RT_U_SIN: case RT_U_COS: case RT_U_TAN:
+            case RT_U_ASIN: case RT_U_ACOS: case RT_U_ATAN: case RT_U_SINH: case RT_U_COSH: case RT_U_ASINH: case RT_U_ACOSH: case RT_U_ATANH: return 4;
+            default: return 1;                      // measured: exp, expm1, rsqrt and every f32 op lose 3 .. 8 % with four
+        }
+    }
+    return 1;
+}
+template <int OP, class T> constexpr int scalar_vectors() {
+    if (std::is_same<T, double>::value && (OP == RT_S_LOG || OP == RT_S_LOG1P)) return 4;
+    if (std::is_same<T, float>::value && OP == RT_S_LOG1P) return 4;
+    if (OP == RT_S_DIV && !std::is_same<T, float>::value && !std::is_same<T, double>::value && !std::is_same<T, boolean_t>::value) return 4;
+    return 1;
+}
+
 template <int OP, class T> struct UnaryF {
     static constexpr bool kReads = true;
+    static constexpr int kVectors = unary_vectors<OP, T>();
     static constexpr bool kPacked = sizeof(T) == 1 && (OP == RT_U_RELU || OP == RT_U_NEG || OP == RT_U_ABS);
     __device__ __forceinline__ uint32_t packed(uint32_t w) const {
         if constexpr (!is_sint<T>::value) {
@@ -194,6 +233,7 @@ template <int OP, class T> struct UnaryF {
 
 template <int OP, class T> struct ScalarF {
     static constexpr bool kReads = true;
+    static constexpr int kVectors = scalar_vectors<OP, T>();
     static constexpr bool kPacked = sizeof(T) == 1 && (OP == RT_S_ADD || OP == RT_S_SUB || (OP == RT_S_MUL && is_bool<T>::value));
     T v;
     int32_t* fault;                     // division of a signed integer by -1 only: set to 1 when an element is MIN (the reference panics)
@@ -215,8 +255,8 @@ template <int OP, class T> struct ScalarF {
             return w_div<T>(x, v);
         }
         else if constexpr (OP == RT_S_LEAKY_RELU) return gt0(x) ? x : w_mul<T>(x, v);             // cpu.rs:708-715
-        else if constexpr (OP == RT_S_LOG) return m_log(x) / m_log(v);                            // f32::log(base)
-        else if constexpr (OP == RT_S_LOG1P) return m_log1p(x) / m_log(v);                        // core/value.rs vlog1p
+        else if constexpr (OP == RT_S_LOG) return over_log_base(m_log(x), v);                     // f32::log(base) = ln(x) / ln(base)
+        else if constexpr (OP == RT_S_LOG1P) return over_log_base(m_log1p(x), v);                 // core/value.rs vlog1p
         else if constexpr (OP == RT_S_ELU) return x >= (T)0 ? x : v * m_expm1(x);                 // cpu.rs:717-724
         else if constexpr (OP == RT_S_LEAKY_GRAD) return gt0(x) ? one_of<T>() : v;                // ops/scalar/mod.rs:149-166
         else return x;
@@ -225,6 +265,7 @@ template <int OP, class T> struct ScalarF {
 
 template <class T> struct FillF {
     static constexpr bool kReads = false;
+    static constexpr int kVectors = 1;
     static constexpr bool kPacked = false;
     T v;
     __device__ __forceinline__ T operator()(T) const { return v; }
@@ -269,12 +310,32 @@ __global__ __launch_bounds__(512) void ew_contig_kernel(Vec16<T>* __restrict__ p
         if constexpr (F::kReads) x = *e;
         *e = f(x);
     }
-    size_t i;
-    if (!rt_tile_index(m, blockIdx.x, blockDim.x, threadIdx.x, nvec, &i)) return;
-    Vec16<T> v;
-    if constexpr (F::kReads) v = rt_ld16_nt(p + i);
-    apply_vec(v, f);
-    rt_st16_nt(p + i, v);
+    // a block stands for kVectors consecutive blocks of the one-vector-per-lane traversal; every load is issued before the first use
+    constexpr int U = F::kVectors;
+    if constexpr (U == 1) {
+        size_t i1;
+        if (!rt_tile_index(m, blockIdx.x, blockDim.x, threadIdx.x, nvec, &i1)) return;
+        Vec16<T> v1;
+        if constexpr (F::kReads) v1 = rt_ld16_nt(p + i1);
+        apply_vec(v1, f);
+        rt_st16_nt(p + i1, v1);
+        return;
+    }
+    size_t i[U];
+    bool has[U];
+    Vec16<T> v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        has[u] = rt_tile_index(m, blockIdx.x * U + u, blockDim.x, threadIdx.x, nvec, &i[u]);
+        if constexpr (F::kReads) { if (has[u]) v[u] = rt_ld16_nt(p + i[u]); }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        if (has[u]) {
+            apply_vec(v[u], f);
+            rt_st16_nt(p + i[u], v[u]);
+        }
+    }
 }
 
 // Edges of a contiguous run that do not fill a 16-byte vector, and 1-D strided views: one element per lane.
@@ -524,7 +585,7 @@ int32_t launch_contig(rt_ctx* ctx, T* p, size_t n, F f) {
     // pages 64 KiB apart (see TileMap)
     const uint32_t bs = F::kReads ? 256u : 512u;
     const TileMap m = F::kReads ? rt_make_tilemap(p + head, nvec, bs) : rt_make_tilemap(p + head, nvec, bs, 1024, 16, 65536);
-    size_t blocks = rt_tilemap_blocks(m, nvec, bs);
+    size_t blocks = (rt_tilemap_blocks(m, nvec, bs) + F::kVectors - 1) / F::kVectors;
     if (blocks < 1) blocks = 1;                                           // a run shorter than a vector: edges only
     if (blocks > 0x7fffffffull) return rt_fail(RT_E_INVALID, "contiguous run of %zu elements is too long for one launch", n);
     RT_TRY(rt_check_edges("elementwise", head, nvec, N, tail, n, bs));
@@ -543,11 +604,31 @@ __global__ __launch_bounds__(256) void ew_contig_out_kernel(const T* __restrict_
     // elements after it go to lanes of the first and the last block
     if (blockIdx.x == 0 && threadIdx.x < head) { const int64_t e = (int64_t)threadIdx.x - (int64_t)head; d[e] = f(s[e]); }
     if (blockIdx.x == gridDim.x - 1 && threadIdx.x < tail) { const size_t e = nvec * N + threadIdx.x; d[e] = f(s[e]); }
-    size_t i;
-    if (!rt_tile_index(m, blockIdx.x, 256, threadIdx.x, nvec, &i)) return;
-    Vec16<T> v = __builtin_bit_cast(Vec16<T>, rt_ld16u<T, true>(s + i * N));          // the source may be in any phase
-    apply_vec(v, f);
-    rt_st16_nt(reinterpret_cast<Vec16<T>*>(d) + i, v);
+    constexpr int U = F::kVectors;
+    if constexpr (U == 1) {
+        size_t i1;
+        if (!rt_tile_index(m, blockIdx.x, 256, threadIdx.x, nvec, &i1)) return;
+        Vec16<T> v1 = __builtin_bit_cast(Vec16<T>, rt_ld16u<T, true>(s + i1 * N));        // the source may be in any phase
+        apply_vec(v1, f);
+        rt_st16_nt(reinterpret_cast<Vec16<T>*>(d) + i1, v1);
+        return;
+    }
+    size_t i[U];
+    bool has[U];
+    rt_u32x4 w[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        has[u] = rt_tile_index(m, blockIdx.x * U + u, 256, threadIdx.x, nvec, &i[u]);
+        if (has[u]) w[u] = rt_ld16u<T, true>(s + i[u] * N);                              // the source may be in any phase
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        if (has[u]) {
+            Vec16<T> v = __builtin_bit_cast(Vec16<T>, w[u]);
+            apply_vec(v, f);
+            rt_st16_nt(reinterpret_cast<Vec16<T>*>(d) + i[u], v);
+        }
+    }
 }
 
 template <class T, class F>
@@ -559,7 +640,7 @@ int32_t launch_contig_out(rt_ctx* ctx, const T* s, T* d, size_t n, F f) {
     if (head > n) head = n;
     const size_t nvec = (n - head) / N, tail = n - head - nvec * N;
     const TileMap m = rt_make_tilemap(d + head, nvec, 256);
-    size_t blocks = rt_tilemap_blocks(m, nvec, 256);
+    size_t blocks = (rt_tilemap_blocks(m, nvec, 256) + F::kVectors - 1) / F::kVectors;
     if (blocks < 1) blocks = 1;
     if (blocks > 0x7fffffffull) return rt_fail(RT_E_INVALID, "contiguous run of %zu elements is too long for one launch", n);
     RT_TRY(rt_check_edges("elementwise", head, nvec, N, tail, n, 256));

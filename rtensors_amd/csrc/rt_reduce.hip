@@ -332,12 +332,14 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_tile_kernel(const T* __res
     const uint32_t nrows = (uint32_t)(a.rows - row0 < a.rpb ? a.rows - row0 : a.rpb);
     const uint32_t ne = nrows * a.R;
     const T* p = src + row0 * a.R;
-    // 1- and 2-byte elements: the run is copied as it lies, with 16-byte LDS stores (an element-wise scatter would issue 8 or 16
-    // sub-word stores per vector: u8 rows of 100 ran at 1.9 TB/s); `mis` keeps the 16-byte phase of the global address
-    constexpr bool kVerbatim = sizeof(T) < 4;
-    const uint32_t mis = kVerbatim ? (uint32_t)((reinterpret_cast<uintptr_t>(p) & 15) / sizeof(T)) : 0u;
+    // pitch == R: the run is copied as it lies, with 16-byte LDS stores; `mis` keeps the 16-byte phase of the global address.  Always
+    // for 1- and 2-byte elements (an element-wise scatter would issue 8 or 16 sub-word stores per vector: u8 rows of 100 ran at
+    // 1.9 TB/s), and for wider elements whenever rows at that pitch meet at most two to a bank (see tile_pitch); otherwise rows go
+    // to a padded pitch element by element, an index division per element.
+    const bool verbatim = a.pitch == a.R;
+    const uint32_t mis = verbatim ? (uint32_t)((reinterpret_cast<uintptr_t>(p) & 15) / sizeof(T)) : 0u;
     auto put = [&](uint32_t e, T v) {
-        if constexpr (kVerbatim) {
+        if (verbatim) {
             tile[mis + e] = v;
         } else {
             const uint32_t r = fd_div(e, a.r_div);
@@ -358,7 +360,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_tile_kernel(const T* __res
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             if (v0 + u * kBlock < nvec) {
-                if constexpr (kVerbatim) {
+                if (verbatim) {
                     *reinterpret_cast<Vec16<T>*>(&tile[mis + head + (v0 + u * kBlock) * N]) = x[u];
                 } else {
 #pragma unroll
@@ -601,8 +603,8 @@ int32_t rows_stage(rt_ctx* ctx, const T* src, T* out, uint64_t rows, uint64_t R,
         RowsTileArgs a;
         a.rows = rows;
         a.R = (uint32_t)R;
-        a.pitch = sizeof(T) < 4 ? a.R : (a.R | 1u);
-        a.rpb = (uint32_t)(kRowsTileBytes / sizeof(T) - (sizeof(T) < 4 ? 16 / sizeof(T) : 0)) / a.pitch;
+        a.pitch = rt_tile_pitch(a.R, (uint32_t)sizeof(T));
+        a.rpb = (uint32_t)(kRowsTileBytes / sizeof(T) - (a.pitch == a.R ? 16 / sizeof(T) : 0)) / a.pitch;
         a.r_div = make_fastdiv(a.R);
         uint32_t t = 1;                                           // lanes per row: fill the block, at most one wave, at most R
         while (t < 64 && (uint64_t)t * 2 * a.rpb <= (uint64_t)kBlock && t * 2 <= a.R) t <<= 1;

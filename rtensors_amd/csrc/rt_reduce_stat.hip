@@ -114,6 +114,16 @@ template <class T> struct LseState {
         m = top;
     }
     __device__ __forceinline__ T result(int) const { return s == (T)0 ? m : m + m_log(s); }
+    // a whole row by one lane: the maximum first, then one exponential per element (the running form above pays one more per block
+    // of four for rescaling the sum: 14 instead of 10 on rows of 10)
+    __device__ __forceinline__ void fold_row(const T* row, uint32_t R) {
+        T top = row[0];
+        for (uint32_t k = 1; k < R; ++k) top = m_max(top, row[k]);
+        T acc = (T)0;
+        for (uint32_t k = 0; k < R; ++k) acc = acc + term(row[k], top);
+        m = top;
+        s = acc;
+    }
 };
 
 template <class T, bool SQ> struct NormState {
@@ -281,12 +291,14 @@ __global__ __launch_bounds__(kBlock) void st_rows_tile_kernel(const T* __restric
     const uint32_t nrows = (uint32_t)(a.rows - row0 < a.rpb ? a.rows - row0 : a.rpb);
     const uint32_t ne = nrows * a.R;
     const T* p = src + row0 * a.R;
-    // 1- and 2-byte elements: the run is copied as it lies, with 16-byte LDS stores (an element-wise scatter would issue 8 or 16
-    // sub-word stores per vector: u8 rows of 100 ran at 1.9 TB/s); `mis` keeps the 16-byte phase of the global address
-    constexpr bool kVerbatim = sizeof(T) < 4;
-    const uint32_t mis = kVerbatim ? (uint32_t)((reinterpret_cast<uintptr_t>(p) & 15) / sizeof(T)) : 0u;
+    // pitch == R: the run is copied as it lies, with 16-byte LDS stores; `mis` keeps the 16-byte phase of the global address.  Always
+    // for 1- and 2-byte elements (an element-wise scatter would issue 8 or 16 sub-word stores per vector: u8 rows of 100 ran at
+    // 1.9 TB/s), and for wider elements whenever rows at that pitch meet at most two to a bank (see tile_pitch); otherwise rows go
+    // to a padded pitch element by element, an index division per element.
+    const bool verbatim = a.pitch == a.R;
+    const uint32_t mis = verbatim ? (uint32_t)((reinterpret_cast<uintptr_t>(p) & 15) / sizeof(T)) : 0u;
     auto put = [&](uint32_t e, T v) {
-        if constexpr (kVerbatim) {
+        if (verbatim) {
             tile[mis + e] = v;
         } else {
             const uint32_t r = fd_div(e, a.r_div);
@@ -298,7 +310,7 @@ __global__ __launch_bounds__(kBlock) void st_rows_tile_kernel(const T* __restric
     if (threadIdx.x < head) put(threadIdx.x, p[threadIdx.x]);
     const uint32_t nvec = (ne - head) / N;
     const Vec16<T>* pv = reinterpret_cast<const Vec16<T>*>(p + head);
-    constexpr int U = 4;
+    constexpr int U = 8;                                           // the whole 32 KiB tile in flight at once: 8 vectors per lane
     for (uint32_t v0 = threadIdx.x; v0 < nvec; v0 += U * kBlock) {
         Vec16<T> x[U];
 #pragma unroll
@@ -307,7 +319,7 @@ __global__ __launch_bounds__(kBlock) void st_rows_tile_kernel(const T* __restric
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             if (v0 + u * kBlock < nvec) {
-                if constexpr (kVerbatim) {
+                if (verbatim) {
                     *reinterpret_cast<Vec16<T>*>(&tile[mis + head + (v0 + u * kBlock) * N]) = x[u];
                 } else {
 #pragma unroll
@@ -327,6 +339,9 @@ __global__ __launch_bounds__(kBlock) void st_rows_tile_kernel(const T* __restric
         if (r < nrows) {
             const T* row = tile + mis + r * a.pitch;              // pitch == R in the verbatim layout
             uint32_t k = j;
+            if constexpr (std::is_same<S, LseState<T>>::value) {
+                if (a.G == 1) { acc.fold_row(row, a.R); k = a.R; }
+            }
             for (; k + 3 * a.G < a.R; k += 4 * a.G) {
                 T x[4];
 #pragma unroll
@@ -604,8 +619,8 @@ int32_t rows_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t rows
         TileArgs a;
         a.rows = rows;
         a.R = (uint32_t)R;
-        a.pitch = sizeof(T) < 4 ? a.R : (a.R | 1u);
-        a.rpb = (uint32_t)(kTileBytes / sizeof(T) - (sizeof(T) < 4 ? 16 / sizeof(T) : 0)) / a.pitch;
+        a.pitch = rt_tile_pitch(a.R, (uint32_t)sizeof(T));
+        a.rpb = (uint32_t)(kTileBytes / sizeof(T) - (a.pitch == a.R ? 16 / sizeof(T) : 0)) / a.pitch;
         a.r_div = make_fastdiv(a.R);
         uint32_t g = 1;                                           // lanes per row: fill the block, at most one wave, at most R
         while (g < 64 && (uint64_t)g * 2 * a.rpb <= (uint64_t)kBlock && g * 2 <= a.R) g <<= 1;
