@@ -39,6 +39,22 @@ def profiled_traffic():
     return None
 
 
+def profiled_duration_us(path=TRAFFIC_PROFILE, kernel="bin_rows4_kernel"):
+    """Average duration of the kernel's timed launches in the committed rocprofv3 kernel trace (the `timed avg us` column of the
+    summary): the figure of the machine the profile was taken on, to set beside this run's own."""
+    try:
+        for ln in open(path):
+            if kernel in ln and "blocks" not in ln.split(kernel)[0][-8:] and "FETCH_SIZE" not in ln:
+                parts = ln.split()
+                try:
+                    return float(parts[-1])
+                except ValueError:
+                    continue
+    except OSError:
+        pass
+    return None
+
+
 def row_major(shape):
     st = [1] * len(shape)
     for i in range(len(shape) - 2, -1, -1):
@@ -318,6 +334,43 @@ class Workloads:
         a = self._gen("c2a", H.F32, 1 << 28, "normal", 1, 0)
         d = self._out("cvt32", H.I32, 1 << 28)
         return (lambda: self.hip.convert(a, d)), (1 << 28) * 8, 1 << 28
+
+    # ---- ALU-heavy maps: the f64 logarithm (hand-written) and integer division on the config-3 shapes ---------------------------------------
+    def _f64_unary(self, op):
+        H = self.H
+        n = 1 << 27
+        a = self._gen("c2a64", H.F64, n, "uniform", 1, 0)
+        z = self._out("c2cf64", H.F64, n)
+        return (lambda: self.hip.unary_to(op, a, 0, n, z)), 2 * n * 8, n
+
+    def f64_ln(self): return self._f64_unary("ln")
+    def f64_ln1p(self): return self._f64_unary("ln1p")
+    def f64_atan(self): return self._f64_unary("atan")
+
+    def _c3_div(self, dtype_name):
+        """x / y on the config-3 shapes (x (16,1,512,L) / y (1,64,1,L) -> (16,64,512,L), L = 4 KiB of elements per row), values 1 .. 100."""
+        H = self.H
+        dt = H.DTYPE_BY_NAME[dtype_name]
+        es = H.NP_DTYPE[dt].itemsize
+        B, J, K, L = 16, 64, 512, 4096 // es
+        def ints(name, n, stream):
+            key = (name,)
+            if key not in self._cache:
+                f = self.hip.alloc_uninit(H.I32, n)
+                self.dg.fill_device(f, "int", 2, stream, 1, 100)
+                b = self.hip.alloc_uninit(dt, n)
+                self.hip.convert(f, b)
+                self._cache[key] = b
+            return self._cache[key]
+        x, y = ints("c3dx" + dtype_name, B * K * L, 0), ints("c3dy" + dtype_name, J * L, 1)
+        z = self._out("c3dz" + dtype_name, dt, B * J * K * L)
+        shape = [B, J, K, L]
+        return (lambda: self.hip.broadcast((x, (0, shape, [K * L, 0, L, 1])), (y, (0, shape, [0, L, 0, 1])), (z, (0, shape, row_major(shape))), "div")), \
+            (x.len + y.len + z.len) * es, z.len
+
+    def c3_div_i64(self): return self._c3_div("i64")
+    def c3_div_i32(self): return self._c3_div("i32")
+    def c3_div_u8(self): return self._c3_div("u8")
 
     # ---- matmul (behind the same trait; MFMA-bound, not part of the headline) ---------------------------------------------------------
     def _mm(self, dtype_name, n):
@@ -684,20 +737,31 @@ def main():
         "config": {"workload": "config 3 strided broadcast add x(16,1,512,1024)+y(1,64,1,1024)->(16,64,512,1024) f32 (2 GiB out), "
                                "then config 4 sum over the last axis of (8192,32768) f32 (1 GiB in)",
                    "bytes_per_step": step_bytes, "pct_of_peak": round(100 * value * 1e9 / PEAK_HBM, 2)},
-        # frac / achieved / kernel_ms: the add kernel inside the timed alternating add / sum loop (mean over the K steps, HIP events);
-        # frac_median: the same by the median; standalone: the same kernel launched back to back, outside the loop
         "step_ms_by_events": round(step_ms_events, 4),
+        # achieved / frac / kernel_ms: the add kernel inside the alternating add / sum steps (mean over K steps, HIP events on the
+        # backend stream, one after every kernel; each event holds the stream for about 5 us, so the figure is a lower bound of the
+        # kernel's own rate).  standalone: the same kernel launched back to back, outside the steps.  profile: the kernel's average
+        # duration in the committed rocprofv3 trace (another machine, another day) and the fraction that duration implies.
         "roofline": {"bound": "hbm", "kernel": "bin_rows4_kernel<float, add, vec, vec> (config 3 broadcast add)",
-                     "achieved": round(add_bytes / (add_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM / 1e9, "unit": "GB/s",
-                     "frac": round(add_bytes / (add_ms * 1e-3) / PEAK_HBM, 4), "traffic": profiled_traffic(),
+                     "achieved": round(add_bytes / (in_step["add_ms"] * 1e-3) / 1e9, 1), "peak": PEAK_HBM / 1e9, "unit": "GB/s",
+                     "frac": round(add_bytes / (in_step["add_ms"] * 1e-3) / PEAK_HBM, 4), "traffic": profiled_traffic(),
                      "traffic_source": "profiles/" + os.path.basename(TRAFFIC_PROFILE) + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measured by this run)",
-                     "measured": "average over 100 launches back to back, HIP events on the backend stream every 10 launches",
-                     "kernel_ms": round(add_ms, 4), "kernel_ms_median": round(add_med, 4),
-                     "frac_median": round(add_bytes / (add_med * 1e-3) / PEAK_HBM, 4),
-                     "in_step": in_step,
-                     "axis_sum": {"kernel": "reduce_rows_block_kernel<sum, float>", "achieved": round(sum_bytes / (sum_ms * 1e-3) / 1e9, 1),
-                                  "frac": round(sum_bytes / (sum_ms * 1e-3) / PEAK_HBM, 4), "kernel_ms": round(sum_ms, 4),
-                                  "kernel_ms_median": round(sum_med, 4)}},
+                     "measured": "inside the add / sum steps: K steps with a HIP event after every kernel (each event costs the stream about 5 us)",
+                     "kernel_ms": in_step["add_ms"], "kernel_ms_median": in_step["add_ms_median"],
+                     "frac_median": round(add_bytes / (in_step["add_ms_median"] * 1e-3) / PEAK_HBM, 4),
+                     "standalone": {"kernel_ms": round(add_ms, 4), "kernel_ms_median": round(add_med, 4),
+                                    "achieved": round(add_bytes / (add_ms * 1e-3) / 1e9, 1), "frac": round(add_bytes / (add_ms * 1e-3) / PEAK_HBM, 4),
+                                    "measured": "100 launches back to back, a HIP event every 10 launches"},
+                     "profile": (lambda us: {"timed_avg_us": us, "frac_profile": round(add_bytes / (us * 1e-6) / PEAK_HBM, 4) if us else None,
+                                             "source": "profiles/" + os.path.basename(TRAFFIC_PROFILE) + " (rocprofv3 --kernel-trace of `bench.py --kernel c3a_add`, the machine that took the profile)"})(profiled_duration_us()),
+                     "axis_sum": {"kernel": "reduce_rows_block_kernel<sum, float>", "achieved": round(sum_bytes / (in_step["sum_ms"] * 1e-3) / 1e9, 1),
+                                  "frac": round(sum_bytes / (in_step["sum_ms"] * 1e-3) / PEAK_HBM, 4), "kernel_ms": in_step["sum_ms"],
+                                  "kernel_ms_median": in_step["sum_ms_median"],
+                                  "standalone": {"kernel_ms": round(sum_ms, 4), "kernel_ms_median": round(sum_med, 4),
+                                                 "frac": round(sum_bytes / (sum_ms * 1e-3) / PEAK_HBM, 4)},
+                                  "profile": (lambda us: {"timed_avg_us": us, "frac_profile": round(sum_bytes / (us * 1e-6) / PEAK_HBM, 4) if us else None,
+                                                          "source": "profiles/reduce_rows_block_kernel_config4_sum_last_axis.txt"})(
+                                      profiled_duration_us(os.path.join(ROOT, "profiles", "reduce_rows_block_kernel_config4_sum_last_axis.txt"), "reduce_rows_block_kernel"))}},
         "detail": detail,
     }
     if not args.no_cpu:

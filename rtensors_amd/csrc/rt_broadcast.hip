@@ -26,6 +26,11 @@ constexpr int kCBlock2 = 256;
 template <class T, int OP>
 __global__ __launch_bounds__(kCBlock2) void bin_contig_kernel(const Vec16<T>* l, const Vec16<T>* r, Vec16<T>* d, size_t nvec, uint32_t head,
                                                               uint32_t tail, TileMap m, int32_t* fault) {
+    __shared__ int32_t div8[uses_div8<T, OP>::value ? 256 : 1];
+    if constexpr (uses_div8<T, OP>::value) {
+        div8_table_init<T>(div8);
+        __syncthreads();
+    }
     // the `head` elements before and the `tail` elements after the aligned body (fewer than a vector each; all three operands
     // share the phase) are taken by lanes of the first and the last block instead of launches of their own
     auto edge = [&](int64_t e) {
@@ -41,7 +46,7 @@ __global__ __launch_bounds__(kCBlock2) void bin_contig_kernel(const Vec16<T>* l,
     Vec16<T> a = rt_ld16_nt(l + i);
     Vec16<T> b;
     if constexpr (OP != kOpCopy) b = rt_ld16_nt(r + i); else b = a;
-    bin_apply_vec<OP, T>(a, b, fault);
+    bin_apply_vec_t<OP, T>(a, b, fault, div8);
     rt_st16_nt(d + i, a);
 }
 
@@ -175,6 +180,11 @@ struct Rows4Args {
 template <class T, int OP, int LM, int RM, int NTM>
 __global__ __launch_bounds__(256) void bin_rows4_kernel(const T* l, const T* r, T* d, Rows4Args a, int32_t* fault) {
     constexpr int N = 16 / sizeof(T);
+    __shared__ int32_t div8[uses_div8<T, OP>::value ? 256 : 1];
+    if constexpr (uses_div8<T, OP>::value) {                       // before any lane leaves: every lane fills one entry
+        div8_table_init<T>(div8);
+        __syncthreads();
+    }
     uint32_t L = a.L, G = a.G, tiles = a.tiles, tm = a.tiles_div.mul, ts = a.tiles_div.shift, group = a.group, gm = a.group_div.mul, gsh = a.group_div.shift;
     int32_t g0 = a.gs[0], g1 = a.gs[1], g2 = a.gs[2], p0 = a.o0s[0], p1 = a.o0s[1], p2 = a.o0s[2], q0 = a.o1s[0], q1 = a.o1s[1], q2 = a.o1s[2];
     int32_t r0 = a.o2s[0], r1 = a.o2s[1], r2 = a.o2s[2];
@@ -219,7 +229,7 @@ __global__ __launch_bounds__(256) void bin_rows4_kernel(const T* l, const T* r, 
         else if constexpr (RM == M_VEC && (NTM & 2)) y = rt_ld16u<T, true>(rp + c);
         else y = load_raw<T, RM>(rp, (uint32_t)c, 1);
         Vec16<T> xv = __builtin_bit_cast(Vec16<T>, x);
-        bin_apply_vec<OP, T>(xv, __builtin_bit_cast(Vec16<T>, y), fault);
+        bin_apply_vec_t<OP, T>(xv, __builtin_bit_cast(Vec16<T>, y), fault, div8);
         rt_st16_nt(reinterpret_cast<Vec16<T>*>(dp + c), xv);
     } else {
         // the ragged ends of a row: all loads, then all stores

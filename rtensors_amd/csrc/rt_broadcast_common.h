@@ -128,6 +128,61 @@ template <int OP, class T> __device__ __forceinline__ void bin_apply_vec(Vec16<T
     }
 }
 
+// ---- division of 1-byte integers through a table of multipliers ---------------------------------------------------------------------
+// For 0 <= a < 256 and 1 <= b < 256 the quotient a / b equals (a * M[b]) >> 16 with M[b] = 65536 / b + 1: the product overshoots
+// a / b by a * (M[b] - 65536 / b) / 65536 < 256 / 65536, less than the 1 / b that separates a / b from the next integer.  Signed
+// bytes use the same multipliers with the divisor's sign on them: p = a * Ms[b] has the sign of the quotient and a magnitude that is
+// never a whole multiple of 65536 unless it is 0, so the truncating quotient is (p >> 16) + (p < 0) (all 256 x 255 pairs of either
+// type checked against integer arithmetic).  The 256 multipliers live in LDS, one computed per lane when the block starts; per
+// element that is a lookup, a 24-bit multiply and a shift, against two conversions, a quarter-rate reciprocal, a multiply and a
+// conversion back on the float path -- which stays for the kernels without the table.  M[0] = 0: the quotient of a zero divisor is 0.
+template <class T, int OP> struct uses_div8 : std::integral_constant<bool, OP == RT_DIV && sizeof(T) == 1 && std::is_integral<T>::value> {};
+
+template <class T> __device__ __forceinline__ void div8_table_init(int32_t* tbl) {          // 256 lanes; caller synchronises
+    const uint32_t byte = threadIdx.x & 255u;
+    const int32_t v = std::is_signed<T>::value ? (int32_t)(int8_t)byte : (int32_t)byte;
+    const int32_t mag = v < 0 ? -v : v;
+    // floor of the correctly rounded f32 quotient: exact, the true quotient is at least 1 / 255 away from the next integer
+    const int32_t m = mag ? (int32_t)(65536.0f / (float)mag) + 1 : 0;
+    tbl[byte] = v < 0 ? -m : m;
+}
+
+template <class T> __device__ __forceinline__ void div8_vec(Vec16<T>& x, const Vec16<T>& y, const int32_t* tbl, int32_t* fault) {
+    rt_words4 a = __builtin_bit_cast(rt_words4, x);
+    const rt_words4 b = __builtin_bit_cast(rt_words4, y);
+    bool bad = false;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        const uint32_t bw = b.w[w];
+        bad |= ((bw - 0x01010101u) & ~bw & 0x80808080u) != 0;                         // a zero byte among the four divisors
+        uint32_t out = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int32_t m = tbl[(bw >> (8 * k)) & 0xffu];
+            if constexpr (std::is_signed<T>::value) {
+                const int32_t av = (int32_t)(int8_t)(a.w[w] >> (8 * k));
+                const int32_t p = av * m;
+                const int32_t q = (p >> 16) + (int32_t)((uint32_t)p >> 31);
+                bad |= q == 128;                                                          // MIN / -1
+                out |= ((uint32_t)q & 0xffu) << (8 * k);
+            } else {
+                const uint32_t av = (a.w[w] >> (8 * k)) & 0xffu;
+                out |= ((av * (uint32_t)m) >> 16) << (8 * k);
+            }
+        }
+        a.w[w] = out;
+    }
+    if (bad && fault) *fault = 1;
+    x = __builtin_bit_cast(Vec16<T>, a);
+}
+
+// x = x OP y on a whole vector, for the kernels that hold the 1-byte division table (`tbl`: 256 words of LDS, filled by
+// div8_table_init, when uses_div8<T, OP>; ignored otherwise)
+template <int OP, class T> __device__ __forceinline__ void bin_apply_vec_t(Vec16<T>& x, const Vec16<T>& y, int32_t* fault, const int32_t* tbl) {
+    if constexpr (uses_div8<T, OP>::value) div8_vec<T>(x, y, tbl, fault);
+    else bin_apply_vec<OP, T>(x, y, fault);
+}
+
 // The fault word of the context for a launch that can raise an integer-division fault (and a note for the host to look at it at
 // the next synchronising call); null for every other launch.
 template <class T, int OP> static inline int32_t* fault_of(rt_ctx* ctx) {

@@ -609,6 +609,70 @@ def test_integer_division_faults(hip, dtype):
         hip.sync()
 
 
+@pytest.mark.parametrize("dtype", ["i8", "u8"])
+def test_8_bit_division_every_pair(hip, dtype):
+    """1-byte integers are divided through a table of multipliers in LDS (contiguous and long-row kernels) or through the float unit
+    (every other kernel).  Every (dividend, divisor) pair through each: the contiguous kernel, the row kernel with the divisors as a
+    repeated row, the element kernel (stepped views) and the scalar form; zero divisors and MIN / -1 give 0 / MIN and raise the fault."""
+    from rtensors_amd import hip as H
+    code = cpu.DTYPE_BY_NAME[dtype]
+    npd = cpu.NP_DTYPE[code]
+    info = np.iinfo(npd)
+    vals = np.arange(256, dtype=np.uint8).view(npd).astype(np.int64)                   # every value of the type, in byte order
+
+    def trunc_div(a, b):
+        return ((np.abs(a) // np.abs(b)) * np.sign(a) * np.sign(b)).astype(npd)
+    a = np.repeat(vals, 256); b = np.tile(vals, 256)
+    clean = (b != 0) & ~((a == info.min) & (b == -1))
+    bc = np.where(clean, b, 1)
+    want = trunc_div(a, bc)
+    n = a.size
+    ga, gb = hip.alloc_from_slice(code, a.astype(npd)), hip.alloc_from_slice(code, bc.astype(npd))
+    out = hip.alloc(code, n)
+    flat = (0, [n], [1])
+    hip.broadcast((ga, flat), (gb, flat), (out, flat), "div")                         # contiguous kernel
+    hip.sync()
+    assert hip.dump(out).tobytes() == want.tobytes()
+    half = (0, [n // 2], [2])
+    out2 = hip.alloc(code, n)
+    hip.broadcast((ga, half), (gb, half), (out2, half), "div")                        # element kernel
+    assert hip.dump(out2)[::2].tobytes() == want[::2].tobytes()
+    # rows of 1024 divisors (every value four times) under 64 rows of dividends arranged so that every pair occurs
+    cols = np.arange(1024)
+    rows = np.arange(64)
+    a2 = vals[(rows[:, None] * 4 + cols[None, :] // 256) % 256]
+    b2 = vals[cols % 256]
+    b2c = np.where(b2 == 0, 1, b2)
+    keep = ~((a2 == info.min) & (b2c[None, :] == -1))
+    a2c = np.where(keep, a2, 0)
+    gra, grb = hip.alloc_from_slice(code, a2c.astype(npd).reshape(-1)), hip.alloc_from_slice(code, b2c.astype(npd))
+    out3 = hip.alloc(code, 64 * 1024)
+    shape = [64, 1024]
+    hip.broadcast((gra, (0, shape, [1024, 1])), (grb, (0, shape, [0, 1])), (out3, (0, shape, [1024, 1])), "div")     # long-row kernel
+    hip.sync()
+    assert hip.dump(out3).tobytes() == trunc_div(a2c, b2c[None, :]).reshape(-1).tobytes()
+    pairs = set(zip(a2c.reshape(-1).tolist(), np.broadcast_to(b2c[None, :], a2c.shape).reshape(-1).tolist()))
+    assert len(pairs) >= 256 * 255 - 2
+    # the faults: the same operands with their zero divisors (and MIN / -1) left in
+    gb0 = hip.alloc_from_slice(code, b.astype(npd))
+    hip.broadcast((ga, flat), (gb0, flat), (out, flat), "div")
+    with pytest.raises(H.TensorError) as e:
+        hip.sync()
+    assert e.value.kind == "ArithmeticError"
+    got = hip.dump(out)
+    ref = np.where(b == 0, 0, trunc_div(a, np.where(b == 0, 1, b)).astype(np.int64)).astype(npd)         # MIN / -1 wraps to MIN
+    assert got.tobytes() == ref.tobytes()
+    grb0 = hip.alloc_from_slice(code, b2.astype(npd))
+    hip.broadcast((gra, (0, shape, [1024, 1])), (grb0, (0, shape, [0, 1])), (out3, (0, shape, [1024, 1])), "div")
+    with pytest.raises(H.TensorError):
+        hip.sync()
+    hip.sync()
+    for d in [int(v) for v in vals if v not in (0, -1)][::5]:
+        g = G(hip, dtype, vals.astype(npd), [256])
+        g /= d
+        assert g.dump().tobytes() == trunc_div(vals, np.int64(d)).tobytes(), d
+
+
 @pytest.mark.parametrize("dtype", ["i16", "u16"])
 def test_16_bit_division_every_dividend_and_every_divisor(hip, dtype):
     """Integers of at most 16 bits are divided through the float unit (reciprocal, multiply, truncate).  Every dividend against a
