@@ -749,6 +749,7 @@ def main():
                      "measured": "inside the add / sum steps: K steps with a HIP event after every kernel (each event costs the stream about 5 us)",
                      "kernel_ms": in_step["add_ms"], "kernel_ms_median": in_step["add_ms_median"],
                      "frac_median": round(add_bytes / (in_step["add_ms_median"] * 1e-3) / PEAK_HBM, 4),
+                     "in_step": in_step,
                      "standalone": {"kernel_ms": round(add_ms, 4), "kernel_ms_median": round(add_med, 4),
                                     "achieved": round(add_bytes / (add_ms * 1e-3) / 1e9, 1), "frac": round(add_bytes / (add_ms * 1e-3) / PEAK_HBM, 4),
                                     "measured": "100 launches back to back, a HIP event every 10 launches"},
