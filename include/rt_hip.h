@@ -139,6 +139,11 @@ int32_t rt_fill_nd(rt_ctx* ctx, int32_t dtype, void* buf, uint64_t buf_len, cons
                    uint64_t offset, int32_t rank, const uint64_t* shape, const int64_t* strides);
 
 /* ---- in-place unary ops (Backend::apply_<op>_{contiguous,1d_strided,nd}, backend/mod.rs:96-141, 311-355) ------ */
+/* The exact ops (neg, relu, abs, sqrt, reciprocal, square, cube, sign, the four roundings) give the bits of the reference's Cpu
+ * backend.  The transcendental ops are within the reference's own test tolerance of 1e-5 but not bit-identical to the platform
+ * libm it calls; where the backend computes by its own routine the bound is: f64 ln within 1 ulp of the exact value, f64 ln1p
+ * within 3 ulp, f32 ln1p within 3.5 ulp; f64 asinh / acosh / atanh and the log(base) / log1p(base) scalar ops build on that
+ * logarithm. */
 int32_t rt_unary_contiguous(rt_ctx* ctx, int32_t dtype, int32_t op, void* buf, uint64_t buf_len, uint64_t start, uint64_t len);
 int32_t rt_unary_1d_strided(rt_ctx* ctx, int32_t dtype, int32_t op, void* buf, uint64_t buf_len,
                             uint64_t offset, int64_t stride, uint64_t len);
