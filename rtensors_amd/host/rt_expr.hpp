@@ -94,6 +94,7 @@ class Expr {
         if (dtype == RT_BOOL || dtype == RT_U128 || dtype == RT_I128) return false;
         std::vector<const Tensor*> ins{&cur};
         std::vector<rt_chain_step> prog;
+        std::vector<size_t> ins_after;                        // inputs in use after each step: they are appended in order of first use
         size_t k = s;
         for (; k < steps_.size() && prog.size() < RT_CHAIN_MAX_STEPS; ++k) {
             const Step& st = steps_[k];
@@ -120,10 +121,13 @@ class Expr {
                 std::memcpy(cs.value, st.value.bytes, 8);
             }
             prog.push_back(cs);
+            ins_after.push_back(ins.size());
         }
+        if (prog.empty()) return false;
+        // the first launch of an expression writes a fresh tensor; later ones overwrite the temporary in place
+        Tensor dst = owned ? cur : cur.like_row_major();
         while (!prog.empty()) {
-            // the first launch of an expression writes a fresh tensor; later ones overwrite the temporary in place
-            Tensor dst = owned ? cur : cur.like_row_major();
+            ins.resize(ins_after[prog.size() - 1]);           // an input that only dropped steps name is not read
             std::vector<const void*> ptrs;
             std::vector<uint64_t> lens, starts;
             for (const Tensor* t : ins) { ptrs.push_back(t->buf()->ptr()); lens.push_back(t->buf()->len()); starts.push_back(t->offset()); }

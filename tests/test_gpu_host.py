@@ -146,6 +146,12 @@ def test_expressions_fuse_and_match_the_eager_operators(T, be):
     assert T.lazy(a).eval().to_numpy().tobytes() == a.to_numpy().tobytes()
     ev = T.lazy(a).unary("sin")
     assert np.allclose(ev.eval().to_numpy(), np.sin(np.arange(6, dtype=np.float32)).reshape(2, 3), rtol=1e-5, atol=1e-6) and ev.fused_launches == 0
+    # an operand that is first named after a step the chain does not have: the steps before the logarithm are one launch (which must
+    # not read b), the logarithm is the operator, the addition is a launch of its own
+    b = T.Tensor.from_buf(be, "f32", np.arange(6, dtype=np.float32) * 0.25, [2, 3])
+    ev = (T.lazy(a) + 1).unary("ln") + b
+    want = np.log(np.arange(6, dtype=np.float32) + 1) + np.arange(6, dtype=np.float32) * 0.25
+    assert np.allclose(ev.eval().to_numpy().reshape(-1), want, rtol=1e-5, atol=1e-6) and ev.fused_launches == 2
 
 
 def test_reduce_of_noncontiguous_and_reversed_views(T, be):
