@@ -126,19 +126,35 @@ __device__ __forceinline__ double m_trunc(double x) { return trunc(x); }
 __device__ __forceinline__ float m_abs(float x) { return fabsf(x); }
 __device__ __forceinline__ double m_abs(double x) { return fabs(x); }
 
-// a / ln(base).  ln(base) is one value for the whole launch.  f32: the plain division.  f64: the general division sequence is some 25
-// instructions per element, so the quotient is formed from the refined reciprocal with one correction step (the correctly rounded
-// quotient in all but rare cases, within one ulp always); a base whose logarithm is zero, infinite, NaN or beyond 2^+-500 keeps the
-// general division, which alone gets those right.
+// a / ln(base).  ln(base) is one value for the whole launch.  f32: the plain division.  f64: the host computes ln(base) and its
+// reciprocal once (LogBase64) and every element takes three operations (the correctly rounded quotient in all but rare cases, within one
+// ulp always) instead of the general division sequence's twenty and a logarithm of the base per lane; a base whose logarithm is zero,
+// infinite, NaN or beyond 2^+-500 keeps the general division, which alone gets those right.
 __device__ __forceinline__ float over_log_base(float a, float base) { return a / m_log(base); }
-__device__ __forceinline__ double over_log_base(double a, double base) {
-    const double d = m_log(base);
-    const double ad = fabs(d);
-    if (!(ad > 0x1p-500 && ad < 0x1p500)) return a / d;        // wave-uniform: d does not depend on the element
-    const double r = rt_rcp_f64(d);
-    const double q = a * r;
-    const double q2 = __builtin_fma(__builtin_fma(-d, q, a), r, q);
-    return __builtin_isfinite(q) ? q2 : q;                      // a = +-inf: q is the answer, the correction would make it NaN
+struct LogBase64 {
+    double d = 0.0, r = 0.0;                                    // ln(base); its reciprocal, or 0 for "divide"
+    static LogBase64 of(double base) {
+        LogBase64 b;
+        b.d = rt_log_f64(base);
+        const double ad = __builtin_fabs(b.d);
+        b.r = (ad > 0x1p-500 && ad < 0x1p500) ? rt_rcp_f64(b.d) : 0.0;
+        return b;
+    }
+};
+__device__ __forceinline__ double over_log_base(double a, const LogBase64& b) {
+    if (b.r == 0.0) return a / b.d;                             // wave-uniform
+    const double q = rt_quot_by_rcp_f64(a, b.d, b.r);
+    return __builtin_isfinite(a) ? q : a * b.r;                 // a = +-inf: the product is the answer, the correction would make it NaN
+}
+
+// (1 + x) / (1 - x) of atanh.  f64: inside the domain, |x| < 1, the divisor lies in [2^-53, 2] and the dividend in [2^-53, 2], where the
+// reciprocal-based quotient (within an ulp) takes a third of the general division sequence; everything else (x = +-1, beyond the domain,
+// infinite, NaN) keeps the plain division, which alone gets those right.
+__device__ __forceinline__ float atanh_ratio(float x) { return (1.0f + x) / (1.0f - x); }
+__device__ __forceinline__ double atanh_ratio(double x) {
+    const double a = 1.0 + x, d = 1.0 - x;
+    if (__builtin_fabs(x) < 1.0) return rt_quot_f64(a, d);
+    return a / d;
 }
 
 // ---- functors ---------------------------------------------------------------------------------------------------
@@ -218,7 +234,7 @@ template <int OP, class T> struct UnaryF {
             else if constexpr (OP == RT_U_COSH) { T a = m_exp(x), b = m_exp(-x); return (a + b) / (one + one); }   // cpu.rs:492-497
             else if constexpr (OP == RT_U_ASINH) { T sq = x * x; return m_log(x + m_sqrt(sq + one)); }              // cpu.rs:499-505
             else if constexpr (OP == RT_U_ACOSH) { T sq = x * x; return m_log(x + m_sqrt(sq - one)); }              // cpu.rs:507-513
-            else if constexpr (OP == RT_U_ATANH) { T two = one + one; return m_log((one + x) / (one - x)) / two; }  // cpu.rs:515-521
+            else if constexpr (OP == RT_U_ATANH) { T two = one + one; return m_log(atanh_ratio(x)) / two; }  // cpu.rs:515-521
             else if constexpr (OP == RT_U_RSQRT) return one / m_sqrt(x);                          // cpu.rs:523-526
             else if constexpr (OP == RT_U_RECIPROCAL) return one / x;                             // cpu.rs:528-531
             else if constexpr (OP == RT_U_SQUARE) return x * x;                                   // cpu.rs:533-536
@@ -237,6 +253,7 @@ template <int OP, class T> struct ScalarF {
     T v;
     int32_t* fault;                     // division of a signed integer by -1 only: set to 1 when an element is MIN (the reference panics)
     int32_t magic = 0;                  // division of 1-byte integers: sign(v) * (65536 / |v| + 1), see div8_magic
+    LogBase64 base = {};                // f64 log / log1p: ln(v) and its reciprocal, from the host
     __device__ __forceinline__ uint32_t packed(uint32_t w) const {
         uint8_t b;
         __builtin_memcpy(&b, &v, 1);
@@ -263,8 +280,13 @@ template <int OP, class T> struct ScalarF {
             }
         }
         else if constexpr (OP == RT_S_LEAKY_RELU) return gt0(x) ? x : w_mul<T>(x, v);             // cpu.rs:708-715
-        else if constexpr (OP == RT_S_LOG) return over_log_base(m_log(x), v);                     // f32::log(base) = ln(x) / ln(base)
-        else if constexpr (OP == RT_S_LOG1P) return over_log_base(m_log1p(x), v);                 // core/value.rs vlog1p
+        else if constexpr (OP == RT_S_LOG) {                                                      // f32::log(base) = ln(x) / ln(base)
+            if constexpr (std::is_same<T, double>::value) return over_log_base(m_log(x), base);
+            else return over_log_base(m_log(x), v);
+        } else if constexpr (OP == RT_S_LOG1P) {                                                  // core/value.rs vlog1p
+            if constexpr (std::is_same<T, double>::value) return over_log_base(m_log1p(x), base);
+            else return over_log_base(m_log1p(x), v);
+        }
         else if constexpr (OP == RT_S_ELU) return x >= (T)0 ? x : v * m_expm1(x);                 // cpu.rs:717-724
         else if constexpr (OP == RT_S_LEAKY_GRAD) return gt0(x) ? one_of<T>() : v;                // ops/scalar/mod.rs:149-166
         else return x;
@@ -935,6 +957,7 @@ int32_t scalar_go(rt_ctx* ctx, const ViewArg& va, const void* value) {
     }
     ScalarF<OP, T> f{load_scalar<T>(value), fault};
     if constexpr (OP == RT_S_DIV && sizeof(T) == 1 && is_int<T>::value) f.magic = div8_magic((int32_t)load_scalar<T>(value));
+    if constexpr ((OP == RT_S_LOG || OP == RT_S_LOG1P) && std::is_same<T, double>::value) f.base = LogBase64::of(load_scalar<T>(value));
     return run_view<T, ScalarF<OP, T>>(ctx, "scalar", va, f);
 }
 

@@ -1,5 +1,5 @@
 """Error bounds of the logarithms the device computes with routines of its own instead of the library's (ocml): f64 ln (hand-written,
-rtensors_amd/csrc/rt_math64.h) within 1 ulp and f64 ln1p within 3 ulp of the exact value (80-bit reference), f32 ln1p (Kahan's formula over
+rtensors_amd/csrc/rt_math64.h) and f64 ln1p within 1 ulp of the exact value (80-bit reference), f32 ln1p (Kahan's formula over
 the f32 logarithm) within 3.5 ulp of the f64 result.  The reference's Cpu backend calls Rust's f64::ln / ln_1p (platform libm, under
 1 ulp) and its tests hold these ops to 1e-5, so bit parity is unpinned here; what a caller can rely on is the bound asserted below.
 The ops built on the logarithm (log_b, log1p_b, asinh, acosh, atanh) are held to the oracle at the reference's 1e-5 elsewhere."""
@@ -49,17 +49,19 @@ def test_f64_ln_within_one_ulp(hip):
     assert sp[0] == -np.inf and sp[1] == -np.inf and np.isnan(sp[2]) and np.isnan(sp[3]) and sp[4] == np.inf and np.isnan(sp[5]) and sp[6] == 0.0
 
 
-def test_f64_ln1p_within_three_ulp(hip):
+def test_f64_ln1p_within_one_ulp(hip):
     if np.finfo(np.longdouble).nmant < 63:
         pytest.skip("no 80-bit long double on this machine")
     rng = np.random.default_rng(2)
     mag = 10.0 ** rng.uniform(-300, 300, size=400_000)
     x = np.concatenate([mag, -mag[mag < 1], rng.uniform(-1, 1, size=300_000), -1 + 10.0 ** rng.uniform(-16, 0, size=50_000),
+                        rng.uniform(0.40, 0.43, size=100_000), rng.uniform(-0.30, -0.28, size=100_000),          # where the routine changes form
+                        10.0 ** rng.uniform(-17, -14, size=100_000), -(10.0 ** rng.uniform(-17, -14, size=100_000)),  # 1 + x rounds to 1 or next to it
                         np.array([1e-16, -1e-16, 2.0 ** -53, 2.0 ** -52, 1.0, np.finfo(np.float64).max, 5e-324, -5e-324])])
     x = x[x > -1]
     got = device_unary(hip, "f64", "ln1p", x)
     err = ulp_error(got, np.log1p(x.astype(np.longdouble)), np.float64)
-    assert err.max() < 3.0, (float(err.max()), float(x[err.argmax()]))
+    assert err.max() < 1.0, (float(err.max()), float(x[err.argmax()]))
     with np.errstate(all="ignore"):
         sp = device_unary(hip, "f64", "ln1p", np.array([0.0, -0.0, -1.0, -2.0, np.inf, np.nan]))
     assert sp[0] == 0.0 and np.signbit(sp[1]) and sp[2] == -np.inf and np.isnan(sp[3]) and sp[4] == np.inf and np.isnan(sp[5])
