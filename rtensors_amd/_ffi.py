@@ -19,7 +19,6 @@ SYMBOLS = [
     "rt_scalar_contiguous", "rt_scalar_1d_strided", "rt_scalar_nd", "rt_unary_to", "rt_scalar_to",
     "rt_broadcast", "rt_reduce_flat", "rt_reduce_nd", "rt_reduce_nd_static", "rt_argmax_flat", "rt_argmax_nd", "rt_gather", "rt_matmul", "rt_fused_bias_relu", "rt_fused_l1_forward", "rt_fused_l1_relu_backward",
     "rt_fused_bias_relu_l1", "rt_fused_l1_relu_backward_t", "rt_fused_chain", "rt_debug_check_view", "rt_debug_check_overlap",
-    "rt_debug_check_view", "rt_debug_check_overlap",
     "rt_event_create", "rt_event_record", "rt_event_elapsed_ms", "rt_event_destroy", "rt_mem_stats", "rt_mem_trim",
 ]
 

@@ -389,8 +389,9 @@ static inline TileMap rt_make_tilemap(const void* body, size_t nvec, uint32_t nt
     return m;
 }
 static inline size_t rt_tilemap_blocks(const TileMap& m, size_t nvec, uint32_t nthreads) { return (nvec + m.pad + nthreads - 1) / nthreads; }
-// The vector that lane `tid` of block `block` owns; false when the lane has none.
-__device__ __forceinline__ bool rt_tile_index(const TileMap& m, uint32_t block, uint32_t nthreads, uint32_t tid, size_t nvec, size_t* out) {
+// The vector that lane `tid` of block `block` owns; false when the lane has none.  Lane by lane, from the lane's own position: the form
+// of the kernels that do a few instructions per element (every lane starts its load after one short chain of vector arithmetic).
+__host__ __device__ __forceinline__ bool rt_tile_index(const TileMap& m, uint32_t block, uint32_t nthreads, uint32_t tid, size_t nvec, size_t* out) {
     const int64_t i = (int64_t)block * nthreads + tid - (int64_t)m.pad;
     if (i < 0 || (size_t)i >= nvec) return false;
     size_t j = (size_t)i - m.lead;                      // wraps to a huge value for i < lead
@@ -405,6 +406,29 @@ __device__ __forceinline__ bool rt_tile_index(const TileMap& m, uint32_t block, 
     }
     *out = m.lead + j;
     return true;
+}
+// The same answer with the block's share of the arithmetic kept apart from the lane's.  Windows start on block boundaries (`pad`), so a
+// block that lies inside the windows owns whole pieces of one piece column: window, column and first row are the same for all of its
+// lanes -- 64-bit arithmetic on the block index, which the compiler keeps on the scalar unit -- and a lane adds its row and its place
+// in the piece, two 32-bit operations, instead of walking the whole decomposition in 64-bit vector arithmetic (17 vector instructions
+// per vector, a tenth of the vector work of the heavier maps).  Blocks that hold the vectors before the first window or after the
+// last one take the lane-by-lane form.  For the kernels whose arithmetic shows: measured on 1 GiB maps, f32 tanh 0.76 -> 0.81 of the
+// memory rate, f32 log1p_b 0.71 -> 0.78, f64 asinh 0.70 -> 0.74; the cheap maps lose 2 % with it (the scalar chain delays a wave's first
+// load) and keep the lane form.
+__host__ __device__ __forceinline__ bool rt_tile_index_block(const TileMap& m, uint32_t block, uint32_t nthreads, uint32_t tid, size_t nvec, size_t* out) {
+    const int64_t jb = (int64_t)block * nthreads - (int64_t)m.pad - (int64_t)m.lead;      // position of lane 0 counted from the first window
+    const uint32_t pieces = nthreads >> m.lp;                                            // pieces a block owns: consecutive rows of one column
+    if (jb >= 0 && (uint64_t)jb + nthreads <= m.bulk && pieces <= (1u << m.lr) && (pieces << m.lp) == nthreads) {
+        const uint64_t tb = (uint64_t)jb >> m.lp;                                        // a multiple of `pieces`
+        const uint64_t r0 = tb & (((uint64_t)1 << m.lr) - 1);
+        const uint64_t c = (tb >> m.lr) & (((uint64_t)1 << m.lc) - 1);
+        const uint64_t w = tb >> (m.lr + m.lc);
+        const uint64_t base = m.lead + ((((w << m.lr) + r0) << (m.lc + m.lp)) + (c << m.lp));
+        const uint32_t lane = ((tid >> m.lp) << (m.lc + m.lp)) + (tid & ((1u << m.lp) - 1));
+        *out = base + lane;
+        return true;
+    }
+    return rt_tile_index(m, block, nthreads, tid, nvec, out);
 }
 
 // Division of a 32-bit numerator by a runtime-constant divisor via multiply-high (round-up method); exact for

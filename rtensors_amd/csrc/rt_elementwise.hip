@@ -104,15 +104,16 @@ __device__ __forceinline__ double m_log1p(double x) { return rt_log1p_f64(x); }
 __device__ __forceinline__ float m_sqrt(float x) { return sqrtf(x); }
 __device__ __forceinline__ double m_sqrt(double x) { return sqrt(x); }
 __device__ __forceinline__ float m_sin(float x) { return sinf(x); }
-__device__ __forceinline__ double m_sin(double x) { return sin(x); }
+// f64 sine, cosine, tangent: by hand below 2^30 (rt_math64.h), the library routine with its full-range reduction beyond, for infinities and NaN
+__device__ __forceinline__ double m_sin(double x) { return rt_trig_in_range(x) ? rt_sin_f64(x) : sin(x); }
 __device__ __forceinline__ float m_cos(float x) { return cosf(x); }
-__device__ __forceinline__ double m_cos(double x) { return cos(x); }
+__device__ __forceinline__ double m_cos(double x) { return rt_trig_in_range(x) ? rt_cos_f64(x) : cos(x); }
 __device__ __forceinline__ float m_tan(float x) { return tanf(x); }
-__device__ __forceinline__ double m_tan(double x) { return tan(x); }
+__device__ __forceinline__ double m_tan(double x) { return rt_trig_in_range(x) ? rt_tan_f64(x) : tan(x); }
 __device__ __forceinline__ float m_asin(float x) { return asinf(x); }
-__device__ __forceinline__ double m_asin(double x) { return asin(x); }
+__device__ __forceinline__ double m_asin(double x) { return rt_asin_f64(x); }      // by hand, as the logarithm (rt_math64.h)
 __device__ __forceinline__ float m_acos(float x) { return acosf(x); }
-__device__ __forceinline__ double m_acos(double x) { return acos(x); }
+__device__ __forceinline__ double m_acos(double x) { return rt_acos_f64(x); }
 __device__ __forceinline__ float m_atan(float x) { return atanf(x); }
 __device__ __forceinline__ double m_atan(double x) { return atan(x); }
 __device__ __forceinline__ float m_floor(float x) { return floorf(x); }
@@ -143,8 +144,11 @@ struct LogBase64 {
 };
 __device__ __forceinline__ double over_log_base(double a, const LogBase64& b) {
     if (b.r == 0.0) return a / b.d;                             // wave-uniform
-    const double q = rt_quot_by_rcp_f64(a, b.d, b.r);
-    return __builtin_isfinite(a) ? q : a * b.r;                 // a = +-inf: the product is the answer, the correction would make it NaN
+    // a = +-inf: the product is the answer, and its residual inf - inf is NaN; the minimum of a NaN and a number is the number, the
+    // correction term stays finite and leaves the infinite product as it is
+    const double q = a * b.r;
+    const double e = __builtin_fmin(__builtin_fma(-b.d, q, a), 0x1p1023);
+    return __builtin_fma(e, b.r, q);
 }
 
 // (1 + x) / (1 - x) of atanh.  f64: inside the domain, |x| < 1, the divisor lies in [2^-53, 2] and the dividend in [2^-53, 2], where the
@@ -157,6 +161,26 @@ __device__ __forceinline__ double atanh_ratio(double x) {
     return a / d;
 }
 
+// 1 / (1 + e) of sigmoid and silu, e = exp(-x) >= 0, and (a - b) / (a + b) of tanh, a = exp(x), b = exp(-x).  f64: the divisor is at
+// least 1, so away from the overflowing end the refined reciprocal (within an ulp) replaces the general division sequence, which is a
+// third of these kernels' arithmetic; the overflowing end, infinities and NaN keep the division (sigmoid(-inf) = 0, tanh(+-inf) = NaN as
+// the reference's formula has it).
+__device__ __forceinline__ float recip_1p(float e) { return 1.0f / (1.0f + e); }
+__device__ __forceinline__ double recip_1p(double e) {
+    const double d = 1.0 + e;
+    if (e < 0x1p1000) return rt_rcp_f64(d);
+    return 1.0 / d;
+}
+__device__ __forceinline__ float tanh_ratio(float x, float a, float b) { return (a - b) / (a + b); }
+__device__ __forceinline__ double tanh_ratio(double x, double a, double b) {
+    if (__builtin_fabs(x) < 690.0) return rt_quot_f64(a - b, a + b);        // a + b < 2^996
+    return (a - b) / (a + b);
+}
+// sqrt(x^2 + 1) of asinh: the argument is at least 1, so the scaling and the zero / denormal handling of the general square root fall
+// away (within an ulp).
+__device__ __forceinline__ float sqrt_ge1(float a) { return sqrtf(a); }
+__device__ __forceinline__ double sqrt_ge1(double a) { return rt_sqrt_ge1_f64(a); }
+
 // ---- functors ---------------------------------------------------------------------------------------------------
 // A functor over 1-byte elements may offer `packed`: the same op on four elements in one 32-bit word (rt_common.h).
 // kVectors: 16-byte vectors a lane of the contiguous kernels handles.  One for the ops that are a few instructions per element: the
@@ -168,12 +192,28 @@ __device__ __forceinline__ double atanh_ratio(double x) {
 template <int OP, class T> constexpr int unary_vectors() {
     if (std::is_same<T, double>::value) {
         switch (OP) {
-            case RT_U_SIGMOID: case RT_U_SILU: case RT_U_TANH: case RT_U_LN: case RT_U_LN1P: case RT_U_SIN: case RT_U_COS: case RT_U_TAN:
+            case RT_U_SIGMOID: case RT_U_SILU: return 2;      // measured: 0.82 of peak with two, 0.78 with one or four
+            case RT_U_TANH: case RT_U_LN: case RT_U_LN1P: case RT_U_SIN: case RT_U_COS: case RT_U_TAN:
             case RT_U_ASIN: case RT_U_ACOS: case RT_U_ATAN: case RT_U_SINH: case RT_U_COSH: case RT_U_ASINH: case RT_U_ACOSH: case RT_U_ATANH: return 4;
             default: return 1;                      // measured: exp, expm1, rsqrt and every f32 op lose 3 .. 8 % with four
         }
     }
     return 1;
+}
+// kHeavy: the op's arithmetic is a sizeable part of its time; its contiguous kernels take the block-wise form of the traversal's index
+// arithmetic (rt_tile_index_block), which the cheap ops lose 2 % with.
+template <int OP, class T> constexpr bool unary_heavy() {
+    if (!(std::is_same<T, double>::value || std::is_same<T, float>::value)) return false;
+    switch (OP) {
+        case RT_U_SIGMOID: case RT_U_SILU: case RT_U_TANH: case RT_U_LN: case RT_U_EXPM1: case RT_U_LN1P: case RT_U_SIN: case RT_U_COS: case RT_U_TAN:
+        case RT_U_ASIN: case RT_U_ACOS: case RT_U_ATAN: case RT_U_SINH: case RT_U_COSH: case RT_U_ASINH: case RT_U_ACOSH: case RT_U_ATANH:
+            return true;                            // exp alone measured 1 .. 2 % better with the lane form
+        default: return false;
+    }
+}
+template <int OP, class T> constexpr bool scalar_heavy() {
+    if (std::is_same<T, double>::value || std::is_same<T, float>::value) return OP == RT_S_LOG || OP == RT_S_LOG1P || OP == RT_S_ELU;
+    return OP == RT_S_DIV && !is_bool<T>::value;
 }
 template <int OP, class T> constexpr int scalar_vectors() {
     if (std::is_same<T, double>::value && (OP == RT_S_LOG || OP == RT_S_LOG1P)) return 4;
@@ -184,6 +224,7 @@ template <int OP, class T> constexpr int scalar_vectors() {
 template <int OP, class T> struct UnaryF {
     static constexpr bool kReads = true;
     static constexpr int kVectors = unary_vectors<OP, T>();
+    static constexpr bool kHeavy = unary_heavy<OP, T>();
     static constexpr bool kPacked = sizeof(T) == 1 && (OP == RT_U_RELU || OP == RT_U_NEG || OP == RT_U_ABS);
     __device__ __forceinline__ uint32_t packed(uint32_t w) const {
         if constexpr (!is_sint<T>::value) {
@@ -213,9 +254,9 @@ template <int OP, class T> struct UnaryF {
             else return w_sub<T>(zero_of<T>(), x);
         } else {
             const T one = (T)1;
-            if constexpr (OP == RT_U_SIGMOID) return one / (one + m_exp(-x));                     // cpu.rs:661-667
-            else if constexpr (OP == RT_U_SILU) return x * (one / (one + m_exp(-x)));             // cpu.rs:669-675
-            else if constexpr (OP == RT_U_TANH) { T a = m_exp(x), b = m_exp(-x); return (a - b) / (a + b); }   // cpu.rs:624-629
+            if constexpr (OP == RT_U_SIGMOID) return recip_1p(m_exp(-x));                         // cpu.rs:661-667
+            else if constexpr (OP == RT_U_SILU) return x * recip_1p(m_exp(-x));                   // cpu.rs:669-675
+            else if constexpr (OP == RT_U_TANH) { T a = m_exp(x), b = m_exp(-x); return tanh_ratio(x, a, b); }   // cpu.rs:624-629
             else if constexpr (OP == RT_U_SQRT) return m_sqrt(x);
             else if constexpr (OP == RT_U_LN) return m_log(x);
             else if constexpr (OP == RT_U_EXPM1) return m_expm1(x);
@@ -232,7 +273,7 @@ template <int OP, class T> struct UnaryF {
             else if constexpr (OP == RT_U_ATAN) return m_atan(x);
             else if constexpr (OP == RT_U_SINH) { T a = m_exp(x), b = m_exp(-x); return (a - b) / (one + one); }   // cpu.rs:485-490
             else if constexpr (OP == RT_U_COSH) { T a = m_exp(x), b = m_exp(-x); return (a + b) / (one + one); }   // cpu.rs:492-497
-            else if constexpr (OP == RT_U_ASINH) { T sq = x * x; return m_log(x + m_sqrt(sq + one)); }              // cpu.rs:499-505
+            else if constexpr (OP == RT_U_ASINH) { T sq = x * x; return m_log(x + sqrt_ge1(sq + one)); }            // cpu.rs:499-505
             else if constexpr (OP == RT_U_ACOSH) { T sq = x * x; return m_log(x + m_sqrt(sq - one)); }              // cpu.rs:507-513
             else if constexpr (OP == RT_U_ATANH) { T two = one + one; return m_log(atanh_ratio(x)) / two; }  // cpu.rs:515-521
             else if constexpr (OP == RT_U_RSQRT) return one / m_sqrt(x);                          // cpu.rs:523-526
@@ -249,6 +290,7 @@ template <int OP, class T> struct UnaryF {
 template <int OP, class T> struct ScalarF {
     static constexpr bool kReads = true;
     static constexpr int kVectors = scalar_vectors<OP, T>();
+    static constexpr bool kHeavy = scalar_heavy<OP, T>();
     static constexpr bool kPacked = sizeof(T) == 1 && (OP == RT_S_ADD || OP == RT_S_SUB || (OP == RT_S_MUL && is_bool<T>::value));
     T v;
     int32_t* fault;                     // division of a signed integer by -1 only: set to 1 when an element is MIN (the reference panics)
@@ -305,6 +347,7 @@ inline int32_t div8_magic(int32_t v) {
 template <class T> struct FillF {
     static constexpr bool kReads = false;
     static constexpr int kVectors = 1;
+    static constexpr bool kHeavy = false;
     static constexpr bool kPacked = false;
     T v;
     __device__ __forceinline__ T operator()(T) const { return v; }
@@ -328,6 +371,11 @@ template <class T, class F> __device__ __forceinline__ void apply_vec(Vec16<T>& 
 constexpr int kBlock = 256;     // element-per-lane kernels
 constexpr int kCBlock = 128;    // contiguous kernel: one 16-byte vector per lane, 128 lanes per block
 constexpr int kEU = 4;          // element-per-lane kernels: elements in flight per lane
+
+template <class F> __device__ __forceinline__ bool ew_tile_index(const TileMap& m, uint32_t block, uint32_t nthreads, uint32_t tid, size_t nvec, size_t* out) {
+    if constexpr (F::kHeavy) return rt_tile_index_block(m, block, nthreads, tid, nvec, out);
+    else return rt_tile_index(m, block, nthreads, tid, nvec, out);
+}
 
 // Body: `nvec` 16-byte vectors starting at the 16-byte aligned address `p`.  One vector per lane and small blocks:
 // on MI355X this shape (with non-temporal accesses for read-modify-write, plain stores for write-only) was the
@@ -353,7 +401,7 @@ __global__ __launch_bounds__(512) void ew_contig_kernel(Vec16<T>* __restrict__ p
     constexpr int U = F::kVectors;
     if constexpr (U == 1) {
         size_t i1;
-        if (!rt_tile_index(m, blockIdx.x, blockDim.x, threadIdx.x, nvec, &i1)) return;
+        if (!ew_tile_index<F>(m, blockIdx.x, blockDim.x, threadIdx.x, nvec, &i1)) return;
         Vec16<T> v1;
         if constexpr (F::kReads) v1 = rt_ld16_nt(p + i1);
         apply_vec(v1, f);
@@ -365,7 +413,7 @@ __global__ __launch_bounds__(512) void ew_contig_kernel(Vec16<T>* __restrict__ p
     Vec16<T> v[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-        has[u] = rt_tile_index(m, blockIdx.x * U + u, blockDim.x, threadIdx.x, nvec, &i[u]);
+        has[u] = ew_tile_index<F>(m, blockIdx.x * U + u, blockDim.x, threadIdx.x, nvec, &i[u]);
         if constexpr (F::kReads) { if (has[u]) v[u] = rt_ld16_nt(p + i[u]); }
     }
 #pragma unroll
@@ -646,7 +694,7 @@ __global__ __launch_bounds__(256) void ew_contig_out_kernel(const T* __restrict_
     constexpr int U = F::kVectors;
     if constexpr (U == 1) {
         size_t i1;
-        if (!rt_tile_index(m, blockIdx.x, 256, threadIdx.x, nvec, &i1)) return;
+        if (!ew_tile_index<F>(m, blockIdx.x, 256, threadIdx.x, nvec, &i1)) return;
         Vec16<T> v1 = __builtin_bit_cast(Vec16<T>, rt_ld16u<T, true>(s + i1 * N));        // the source may be in any phase
         apply_vec(v1, f);
         rt_st16_nt(reinterpret_cast<Vec16<T>*>(d) + i1, v1);
@@ -657,7 +705,7 @@ __global__ __launch_bounds__(256) void ew_contig_out_kernel(const T* __restrict_
     rt_u32x4 w[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-        has[u] = rt_tile_index(m, blockIdx.x * U + u, 256, threadIdx.x, nvec, &i[u]);
+        has[u] = ew_tile_index<F>(m, blockIdx.x * U + u, 256, threadIdx.x, nvec, &i[u]);
         if (has[u]) w[u] = rt_ld16u<T, true>(s + i[u] * N);                              // the source may be in any phase
     }
 #pragma unroll

@@ -10,3 +10,27 @@ extern "C" void log_many(size_t n, const double* x, double* y) {
 extern "C" void log1p_many(size_t n, const double* x, double* y) {
     for (size_t i = 0; i < n; ++i) y[i] = rt_log1p_f64(x[i]);
 }
+extern "C" void asin_many(size_t n, const double* x, double* y) {
+    for (size_t i = 0; i < n; ++i) y[i] = rt_asin_f64(x[i]);
+}
+extern "C" void acos_many(size_t n, const double* x, double* y) {
+    for (size_t i = 0; i < n; ++i) y[i] = rt_acos_f64(x[i]);
+}
+extern "C" void sqrt_ge1_many(size_t n, const double* x, double* y) {
+    for (size_t i = 0; i < n; ++i) y[i] = rt_sqrt_ge1_f64(x[i]);
+}
+extern "C" void rcp_many(size_t n, const double* x, double* y) {
+    for (size_t i = 0; i < n; ++i) y[i] = rt_rcp_f64(x[i]);
+}
+extern "C" void quot_many(size_t n, const double* a, const double* d, double* y) {
+    for (size_t i = 0; i < n; ++i) y[i] = rt_quot_f64(a[i], d[i]);
+}
+extern "C" void sin_many(size_t n, const double* x, double* y) {
+    for (size_t i = 0; i < n; ++i) y[i] = rt_sin_f64(x[i]);
+}
+extern "C" void cos_many(size_t n, const double* x, double* y) {
+    for (size_t i = 0; i < n; ++i) y[i] = rt_cos_f64(x[i]);
+}
+extern "C" void tan_many(size_t n, const double* x, double* y) {
+    for (size_t i = 0; i < n; ++i) y[i] = rt_tan_f64(x[i]);
+}

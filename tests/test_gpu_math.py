@@ -1,6 +1,7 @@
-"""Error bounds of the logarithms the device computes with routines of its own instead of the library's (ocml): f64 ln (hand-written,
-rtensors_amd/csrc/rt_math64.h) and f64 ln1p within 1 ulp of the exact value (80-bit reference), f32 ln1p (Kahan's formula over
-the f32 logarithm) within 3.5 ulp of the f64 result.  The reference's Cpu backend calls Rust's f64::ln / ln_1p (platform libm, under
+"""Error bounds of the functions the device computes with routines of its own instead of the library's (ocml): f64 ln (hand-written,
+rtensors_amd/csrc/rt_math64.h) and f64 ln1p within 1 ulp of the exact value (80-bit reference), f64 asin within 2 and acos within 1.5
+ulp, f64 sin / cos within 2 and tan within 3 ulp below 2^30 (the library routine beyond), f32 ln1p (Kahan's formula over the f32
+logarithm) within 3.5 ulp of the f64 result.  The reference's Cpu backend calls Rust's f64::ln / ln_1p (platform libm, under
 1 ulp) and its tests hold these ops to 1e-5, so bit parity is unpinned here; what a caller can rely on is the bound asserted below.
 The ops built on the logarithm (log_b, log1p_b, asinh, acosh, atanh) are held to the oracle at the reference's 1e-5 elsewhere."""
 import numpy as np
@@ -82,3 +83,90 @@ def test_f32_ln1p_within_three_and_a_half_ulp(hip):
     with np.errstate(all="ignore"):
         sp = device_unary(hip, "f32", "ln1p", np.array([0.0, -0.0, -1.0, -2.0, np.inf, np.nan], dtype=np.float32))
     assert sp[0] == 0.0 and np.signbit(sp[1]) and sp[2] == -np.inf and np.isnan(sp[3]) and sp[4] == np.inf and np.isnan(sp[5])
+
+
+def test_f64_asin_acos_bounds(hip):
+    if np.finfo(np.longdouble).nmant < 63:
+        pytest.skip("no 80-bit long double on this machine")
+    rng = np.random.default_rng(4)
+    x = np.concatenate([rng.uniform(-1, 1, 600_000), 1 - 10.0 ** rng.uniform(-16, 0, 100_000), -1 + 10.0 ** rng.uniform(-16, 0, 100_000),
+                        10.0 ** rng.uniform(-300, 0, 100_000), -(10.0 ** rng.uniform(-300, 0, 100_000)), rng.uniform(0.49, 0.51, 50_000),
+                        rng.uniform(-0.51, -0.49, 50_000), np.array([0.5, -0.5, 0.975, 5e-324])])
+    x = x[np.abs(x) < 1]
+    xl = x.astype(np.longdouble)
+    err = ulp_error(device_unary(hip, "f64", "asin", x), np.arcsin(xl), np.float64)
+    assert err.max() < 2.0, ("asin", float(err.max()), float(x[err.argmax()]))
+    err = ulp_error(device_unary(hip, "f64", "acos", x), np.arccos(xl), np.float64)
+    assert err.max() < 1.5, ("acos", float(err.max()), float(x[err.argmax()]))
+    sp = np.array([0.0, -0.0, 1.0, -1.0, 1.5, -1.5, np.nan, np.inf, -np.inf, 5e-324, -5e-324, np.nextafter(1.0, 2)])
+    with np.errstate(all="ignore"):
+        a, b = device_unary(hip, "f64", "asin", sp), device_unary(hip, "f64", "acos", sp)
+        assert np.array_equal(a, np.arcsin(sp), equal_nan=True) and np.signbit(a[1]) and not np.signbit(a[0])
+        assert np.array_equal(b, np.arccos(sp), equal_nan=True)
+
+
+def test_f64_sin_cos_tan_bounds(hip):
+    if np.finfo(np.longdouble).nmant < 63:
+        pytest.skip("no 80-bit long double on this machine")
+    rng = np.random.default_rng(8)
+    k = rng.integers(-2 ** 20, 2 ** 20, 200_000)
+    near = (k * (np.pi / 2)) * (1 + rng.standard_normal(k.size) * 10.0 ** rng.integers(-16, -3, k.size))      # next to multiples of pi/2
+    # below 2^30 (the hand-written path) and beyond it up to the largest finite value (the library routine's reduction), in one buffer:
+    # waves that hold both kinds take both branches
+    x = np.concatenate([rng.uniform(-10, 10, 400_000), rng.uniform(-1e6, 1e6, 200_000), 10.0 ** rng.uniform(-300, 9, 200_000),
+                        -(10.0 ** rng.uniform(-300, 9, 200_000)), near, rng.uniform(-2.0 ** 30, 2.0 ** 30, 200_000),
+                        10.0 ** rng.uniform(9, 308, 100_000), -(10.0 ** rng.uniform(9, 308, 100_000)),
+                        np.array([np.pi / 4, -np.pi / 4, np.pi / 2, np.pi, 2.0 ** 30 - 1, 2.0 ** 30, np.finfo(np.float64).max, 5e-324])])
+    rng.shuffle(x)
+    xl = x.astype(np.longdouble)
+    small = np.abs(x) < 2.0 ** 30
+    for op, exact, bound in (("sin", np.sin(xl), 2.0), ("cos", np.cos(xl), 2.0), ("tan", np.tan(xl), 3.0)):
+        got = device_unary(hip, "f64", op, x)
+        err = ulp_error(got, exact, np.float64)
+        assert err[small].max() < bound, (op, float(err[small].max()), float(x[small][err[small].argmax()]))
+        # beyond 2^30 numpy's 80-bit routine reduces with a 64-bit pi and is itself inexact: the device's library routine is only held to
+        # the range of the function there
+        assert np.isfinite(got[~small]).all() and (op == "tan" or (np.abs(got[~small]) <= 1).all())
+    sp = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 5e-324, -5e-324])
+    with np.errstate(all="ignore"):
+        for op, ref in (("sin", np.sin), ("cos", np.cos), ("tan", np.tan)):
+            got = device_unary(hip, "f64", op, sp)
+            assert np.array_equal(got, ref(sp), equal_nan=True), (op, got)
+            if op != "cos":
+                assert np.signbit(got[1]) and not np.signbit(got[0])
+
+
+def test_f64_sigmoid_tanh_asinh_atanh_close_to_the_formulas(hip):
+    """The ops whose division or square root comes from the reciprocal estimates: within a few ulp of the reference's own formula
+    evaluated in 80-bit arithmetic, over the range where the formula is well conditioned, and the formula's own answers at its ends."""
+    if np.finfo(np.longdouble).nmant < 63:
+        pytest.skip("no 80-bit long double on this machine")
+    rng = np.random.default_rng(9)
+    x = np.concatenate([rng.uniform(-30, 30, 400_000), rng.uniform(-700, 700, 100_000), 10.0 ** rng.uniform(-300, 2, 100_000)])
+    xl = x.astype(np.longdouble)
+    one = np.longdouble(1)
+    with np.errstate(all="ignore"):
+        cases = (("sigmoid", one / (one + np.exp(-xl)), 4.0), ("silu", xl / (one + np.exp(-xl)), 4.0))
+        for op, exact, bound in cases:
+            err = ulp_error(device_unary(hip, "f64", op, x), exact, np.float64)
+            assert err.max() < bound, (op, float(err.max()), float(x[err.argmax()]))
+    y = x[np.abs(x) > 0.5]; yl = y.astype(np.longdouble)                   # exp(x) - exp(-x) cancels below that: the formula's own loss
+    err = ulp_error(device_unary(hip, "f64", "tanh", y), np.tanh(yl), np.float64)
+    assert err.max() < 6.0, ("tanh", float(err.max()), float(y[err.argmax()]))
+    a = rng.uniform(2, 1e6, 300_000); al = a.astype(np.longdouble)        # asinh's formula cancels for negative and for small arguments
+    err = ulp_error(device_unary(hip, "f64", "asinh", a), np.arcsinh(al), np.float64)
+    assert err.max() < 4.0, ("asinh", float(err.max()), float(a[err.argmax()]))
+    t = np.concatenate([rng.uniform(0.5, 1, 200_000), -rng.uniform(0.5, 1, 200_000), 1 - 10.0 ** rng.uniform(-16, -1, 50_000)])
+    t = t[np.abs(t) < 1]; tl = t.astype(np.longdouble)
+    err = ulp_error(device_unary(hip, "f64", "atanh", t), np.arctanh(tl), np.float64)
+    assert err.max() < 4.0, ("atanh", float(err.max()), float(t[err.argmax()]))
+    sp = np.array([0.0, 1.0, -1.0, 2.0, np.inf, -np.inf, np.nan, 750.0, -750.0, -0.0])
+    with np.errstate(all="ignore"):
+        got = device_unary(hip, "f64", "atanh", sp)
+        assert got[0] == 0 and got[1] == np.inf and got[2] == -np.inf and np.isnan(got[3:7]).all()
+        got = device_unary(hip, "f64", "sigmoid", sp)
+        assert got[0] == 0.5 and got[4] == 1.0 and got[5] == 0.0 and np.isnan(got[6]) and got[7] == 1.0 and got[8] == 0.0
+        got = device_unary(hip, "f64", "tanh", sp)       # the reference's (e^x - e^-x) / (e^x + e^-x) is inf / inf beyond +-710
+        assert got[0] == 0 and np.isnan(got[4:9]).all()
+        got = device_unary(hip, "f64", "asinh", np.array([0.0, np.inf, np.nan, 1e200, 1.0]))
+        assert got[0] == 0 and got[1] == np.inf and np.isnan(got[2]) and got[3] == np.inf and abs(got[4] - np.arcsinh(1.0)) < 1e-15

@@ -1,6 +1,8 @@
-"""The hand-written f64 logarithm of the device code (rtensors_amd/csrc/rt_math64.h), built for the host with g++ and measured against
-numpy's 80-bit long double logarithm: error in units of the last place over the whole range (every binade sampled, the neighbourhood of
-1 where the result cancels, denormals), and the special values of IEEE / Rust's f64::ln and f64::ln_1p."""
+"""The hand-written f64 routines of the device code (rtensors_amd/csrc/rt_math64.h: logarithm, arcsine / arccosine, sine / cosine /
+tangent and the reciprocal, quotient and square-root helpers under them), built for the host with g++ and measured against numpy's
+80-bit long double functions: error in units of the last place over the whole range each routine is used on, and the special values of
+IEEE / Rust's f64 methods.  The host build replaces the hardware's reciprocal and reciprocal-square-root estimates by cruder ones
+(20 bits), so the bounds hold for the device a fortiori; tests/test_gpu_math.py asserts them there as well."""
 import ctypes as C
 import os
 import subprocess
@@ -16,8 +18,9 @@ def lib(tmp_path_factory):
     out = str(tmp_path_factory.mktemp("math64") / "libmath64.so")
     subprocess.check_call(["g++", "-O2", "-ffp-contract=off", "-shared", "-fPIC", "-o", out, os.path.join(HERE, "support", "math64_host.cpp")])
     L = C.CDLL(out)
-    for f in (L.log_many, L.log1p_many):
+    for f in (L.log_many, L.log1p_many, L.asin_many, L.acos_many, L.sin_many, L.cos_many, L.tan_many, L.sqrt_ge1_many, L.rcp_many):
         f.argtypes = [C.c_size_t, C.c_void_p, C.c_void_p]
+    L.quot_many.argtypes = [C.c_size_t, C.c_void_p, C.c_void_p, C.c_void_p]
     return L
 
 
@@ -84,3 +87,71 @@ def test_special_values(lib):
         got = call(lib.log1p_many, np.array([0.0, -0.0, -1.0, -2.0, inf, -inf, nan, 1e-300]))
     assert got[0] == 0.0 and not np.signbit(got[0]) and got[1] == 0.0 and np.signbit(got[1])
     assert got[2] == -inf and np.isnan(got[3]) and got[4] == inf and np.isnan(got[5]) and np.isnan(got[6]) and got[7] == 1e-300
+
+
+def need_long_double():
+    if np.finfo(np.longdouble).nmant < 63:
+        pytest.skip("no 80-bit long double on this machine")
+
+
+def test_asin_acos_within_two_ulp(lib):
+    need_long_double()
+    rng = np.random.default_rng(3)
+    # the whole domain; next to +-1, where the square-root form ends; every magnitude down to the denormals; either side of |x| = 0.5, where
+    # the two forms meet
+    x = np.concatenate([rng.uniform(-1, 1, 1_000_000), 1 - 10.0 ** rng.uniform(-16, 0, 100_000), -1 + 10.0 ** rng.uniform(-16, 0, 100_000),
+                        10.0 ** rng.uniform(-300, 0, 100_000), -(10.0 ** rng.uniform(-300, 0, 100_000)), rng.uniform(0.49, 0.51, 100_000),
+                        rng.uniform(-0.51, -0.49, 100_000), np.array([0.5, -0.5, 1.0, -1.0, 0.975, 5e-324])])
+    x = x[np.abs(x) <= 1]
+    xl = x.astype(np.longdouble)
+    err = ulp_error(call(lib.asin_many, x), np.arcsin(xl))
+    assert err.max() < 2.0, ("asin", float(err.max()), float(x[err.argmax()]))
+    err = ulp_error(call(lib.acos_many, x[x < 1]), np.arccos(xl[x < 1]))                # acos(1) = 0 exactly, checked below
+    assert err.max() < 1.5, ("acos", float(err.max()), float(x[err.argmax()]))
+    sp = np.array([0.0, -0.0, 1.0, -1.0, 1.5, -1.5, np.nan, np.inf, -np.inf, 5e-324, -5e-324, np.nextafter(1.0, 2)])
+    with np.errstate(all="ignore"):
+        a, b = call(lib.asin_many, sp), call(lib.acos_many, sp)
+        assert np.array_equal(a, np.arcsin(sp), equal_nan=True) and np.signbit(a[1]) and not np.signbit(a[0])
+        assert np.array_equal(b, np.arccos(sp), equal_nan=True)
+
+
+def trig_arguments(rng):
+    k = rng.integers(-2 ** 20, 2 ** 20, 200_000)
+    near = (k * (np.pi / 2)) * (1 + rng.standard_normal(k.size) * 10.0 ** rng.integers(-16, -3, k.size))      # next to multiples of pi/2
+    x = np.concatenate([rng.uniform(-10, 10, 600_000), rng.uniform(-1e6, 1e6, 300_000), 10.0 ** rng.uniform(-300, 9, 200_000),
+                        -(10.0 ** rng.uniform(-300, 9, 200_000)), near, rng.uniform(-2.0 ** 30, 2.0 ** 30, 200_000), rng.uniform(-0.8, 0.8, 200_000),
+                        np.array([np.pi / 4, -np.pi / 4, np.pi / 2, np.pi, 3 * np.pi / 4, 2.0 ** 30 - 1, 5e-324])])
+    return x[np.abs(x) < 2.0 ** 30]
+
+
+def test_sin_cos_tan_below_2_30(lib):
+    need_long_double()
+    x = trig_arguments(np.random.default_rng(7))
+    xl = x.astype(np.longdouble)
+    for name, fn, exact, bound in (("sin", lib.sin_many, np.sin(xl), 2.0), ("cos", lib.cos_many, np.cos(xl), 2.0), ("tan", lib.tan_many, np.tan(xl), 3.0)):
+        err = ulp_error(call(fn, x), exact)
+        assert err.max() < bound, (name, float(err.max()), float(x[err.argmax()]))
+    sp = np.array([0.0, -0.0, 5e-324, -5e-324, 1e-300, np.pi / 2, np.pi, -np.pi / 4])
+    for fn, ref in ((lib.sin_many, np.sin), (lib.tan_many, np.tan)):
+        got = call(fn, sp)
+        assert np.array_equal(got, ref(sp)) and np.signbit(got[1]) and not np.signbit(got[0])
+    assert np.array_equal(call(lib.cos_many, sp), np.cos(sp))
+
+
+def test_reciprocal_quotient_and_square_root_helpers(lib):
+    need_long_double()
+    rng = np.random.default_rng(5)
+    a = np.concatenate([1 + rng.random(300_000) * 3, 10.0 ** rng.uniform(0, 307, 300_000), 1 + 10.0 ** rng.uniform(-16, 0, 100_000)])
+    err = ulp_error(call(lib.sqrt_ge1_many, a), np.sqrt(a.astype(np.longdouble)))
+    assert err.max() <= 1.0, float(err.max())
+    got = call(lib.sqrt_ge1_many, np.array([1.0, np.inf, np.nan, 4.0]))
+    assert got[0] == 1.0 and got[1] == np.inf and np.isnan(got[2]) and got[3] == 2.0
+    d = np.concatenate([1 + 10.0 ** rng.uniform(-16, 300, 300_000), rng.uniform(1, 2, 300_000), rng.uniform(-500, 500, 100_000)])
+    err = ulp_error(call(lib.rcp_many, d), 1 / d.astype(np.longdouble))
+    assert err.max() <= 1.0, float(err.max())
+    n, d = rng.uniform(-2, 2, 500_000), rng.uniform(2.0 ** -53, 2, 500_000)
+    n[:1000], d[:1000] = 2.0 - 2.0 ** -52, 2.0 ** -53 * (1 + rng.random(1000))               # the largest quotients atanh forms
+    x = np.ascontiguousarray(n); y = np.ascontiguousarray(d); out = np.empty_like(x)
+    lib.quot_many(x.size, x.ctypes.data, y.ctypes.data, out.ctypes.data)
+    err = ulp_error(out, x.astype(np.longdouble) / y.astype(np.longdouble))
+    assert err.max() <= 1.0, float(err.max())
