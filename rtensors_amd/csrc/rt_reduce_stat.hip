@@ -49,6 +49,7 @@ __device__ __forceinline__ double m_recip(double x) { return 1.0 / x; }
 template <class T> struct MomentState {
     typedef T Out;
     static constexpr int kColsBlocksPerCU = 2;
+    static constexpr int kNarrowBlocksPerCU = 2;   // narrow-column kernel: resident blocks per CU (1 GiB over 3 and 100 columns: 0.85 .. 0.88 of peak with 2, 0.79 .. 0.81 with 4)
     T mean, m2;
     double n;                                                   // a count, exact up to 2^53; as a double it converts to T in one instruction
     __device__ __forceinline__ void init() { mean = (T)0; m2 = (T)0; n = 0.0; }
@@ -84,6 +85,7 @@ template <class T> struct MomentState {
 template <class T> struct LseState {
     typedef T Out;
     static constexpr int kColsBlocksPerCU = 4;                  // one exp per element: more waves per CU to hide it (0.215 -> 0.180 ms on 1 GiB)
+    static constexpr int kNarrowBlocksPerCU = 2;
     T m, s;
     __device__ __forceinline__ void init() { m = -std::numeric_limits<T>::infinity(); s = (T)0; }
     // exp(x - top), with x == top giving 1 also when both are infinite.  The argument is never positive, so for f32 the hardware
@@ -129,6 +131,7 @@ template <class T> struct LseState {
 template <class T, bool SQ> struct NormState {
     typedef T Out;
     static constexpr int kColsBlocksPerCU = 2;
+    static constexpr int kNarrowBlocksPerCU = 2;
     T s;
     __device__ __forceinline__ void init() { s = (T)0; }
     __device__ __forceinline__ void push(T x, uint64_t) { s = s + (SQ ? x * x : m_abs(x)); }
@@ -145,6 +148,7 @@ template <class T, bool SQ> struct NormState {
 template <class T, bool MAX> struct ArgState {
     typedef uint64_t Out;
     static constexpr int kColsBlocksPerCU = 2;
+    static constexpr int kNarrowBlocksPerCU = 3;   // narrow columns: 0.80 with 3 or 4, 0.71 with 2
     T v;
     uint64_t idx;
     __device__ __forceinline__ void init() {
@@ -275,7 +279,10 @@ __global__ __launch_bounds__(kBlock) void st_rows_wave_kernel(const T* __restric
 
 // short rows (1 <= R <= 1024): the block's rows are one contiguous run, copied into LDS with coalesced 16-byte loads (row pitch R | 1
 // keeps lanes that walk different rows on different banks), then groups of G lanes fold one row each.
-constexpr uint32_t kTileBytes = 32768;
+// 24 KiB: six resident blocks per CU.  Measured on 1 GiB of f32 rows against 32 KiB (five blocks): logsumexp over rows of 10
+// 0.69 -> 0.76 of peak, variance 0.71 -> 0.77, sum 0.71 -> 0.76; rows of 100: 0.67 -> 0.73, 0.73 -> 0.79, 0.73 -> 0.81; 16, 20, 22 and
+// 26 KiB lie between, 48 KiB (three blocks) loses 10 %.
+constexpr uint32_t kTileBytes = 24576;
 constexpr uint64_t kTileMaxR = 1024;
 struct TileArgs {
     uint64_t rows;
@@ -728,7 +735,7 @@ int32_t narrow_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t ou
     a.G = 1;
     while (a.G < 64 && (uint64_t)a.G * 2 * inner <= (uint64_t)kBlock && a.G * 2 <= a.L) a.G <<= 1;
     const uint64_t ntiles = (R + a.L - 1) / a.L;
-    const uint64_t want = (uint64_t)ctx->num_cus * 4;
+    const uint64_t want = (uint64_t)ctx->num_cus * S::kNarrowBlocksPerCU;
     uint64_t splits = outer >= want ? 1 : (want + outer - 1) / outer;
     if (splits > ntiles / 8) splits = ntiles / 8;              // at least 8 tiles per block
     if (splits < 1) splits = 1;
