@@ -347,6 +347,17 @@ class Workloads:
     def f64_ln1p(self): return self._f64_unary("ln1p")
     def f64_atan(self): return self._f64_unary("atan")
 
+    def __getattr__(self, name):
+        """`f64_<op>` for every unary op: the out-of-place map over 1 GiB of f64 (f64_tan, f64_asin, f64_tanh ...); `c3_div_<dtype>` for
+        every integer dtype: the division on the config-3 shapes."""
+        if name in ("H", "hip", "dg", "_cache"):
+            raise AttributeError(name)
+        if name.startswith("f64_") and name[4:] in self.H.UNARY:
+            return lambda: self._f64_unary(name[4:])
+        if name.startswith("c3_div_") and name[7:] in ("u8", "i8", "u16", "i16", "u32", "i32", "u64", "i64"):
+            return lambda: self._c3_div(name[7:])
+        raise AttributeError(name)
+
     def _c3_div(self, dtype_name):
         """x / y on the config-3 shapes (x (16,1,512,L) / y (1,64,1,L) -> (16,64,512,L), L = 4 KiB of elements per row), values 1 .. 100."""
         H = self.H
