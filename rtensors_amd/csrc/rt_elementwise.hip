@@ -152,37 +152,42 @@ __device__ __forceinline__ double over_log_base(double a, const LogBase64& b) {
 }
 
 // (1 + x) / (1 - x) of atanh.  f64: inside the domain, |x| < 1, the divisor lies in [2^-53, 2] and the dividend in [2^-53, 2], where the
-// reciprocal-based quotient (within an ulp) takes a third of the general division sequence; everything else (x = +-1, beyond the domain,
-// infinite, NaN) keeps the plain division, which alone gets those right.
+// reciprocal-based quotient (within an ulp) takes a third of the general division sequence.  Everywhere else the logarithm only needs
+// the kind of the quotient -- inf at x = 1, 0 at x = -1, negative beyond the domain, NaN for NaN and for +-inf -- which the dividend
+// times the raw reciprocal estimate has.  Straight-line code: no lane leaves the wave's path.
 __device__ __forceinline__ float atanh_ratio(float x) { return (1.0f + x) / (1.0f - x); }
 __device__ __forceinline__ double atanh_ratio(double x) {
     const double a = 1.0 + x, d = 1.0 - x;
-    if (__builtin_fabs(x) < 1.0) return rt_quot_f64(a, d);
-    return a / d;
+    const double q = rt_quot_f64(a, d);
+    return __builtin_fabs(x) < 1.0 ? q : a * rt_rcp_seed_f64(d);
 }
 
 // 1 / (1 + e) of sigmoid and silu, e = exp(-x) >= 0, and (a - b) / (a + b) of tanh, a = exp(x), b = exp(-x).  f64: the divisor is at
-// least 1, so away from the overflowing end the refined reciprocal (within an ulp) replaces the general division sequence, which is a
-// third of these kernels' arithmetic; the overflowing end, infinities and NaN keep the division (sigmoid(-inf) = 0, tanh(+-inf) = NaN as
-// the reference's formula has it).
+// least 1, so the refined reciprocal (within an ulp) replaces the general division sequence, which is a third of these kernels'
+// arithmetic.  The ends of the range are patched by selects, with what the reference's formulas give there: 1 / (1 + inf) = 0;
+// (a - b) / (a + b) = +-1 exactly from |x| = 690 on (the smaller exponential is lost in the sum) and inf / inf = NaN once exp overflows.
 __device__ __forceinline__ float recip_1p(float e) { return 1.0f / (1.0f + e); }
 __device__ __forceinline__ double recip_1p(double e) {
     const double d = 1.0 + e;
-    if (e < 0x1p1000) return rt_rcp_f64(d);
-    return 1.0 / d;
+    const double r = rt_rcp_f64(d);                              // NaN for d = inf (and for NaN)
+    return d == __builtin_inf() ? 0.0 : r;
 }
 __device__ __forceinline__ float tanh_ratio(float x, float a, float b) { return (a - b) / (a + b); }
 __device__ __forceinline__ double tanh_ratio(double x, double a, double b) {
-    if (__builtin_fabs(x) < 690.0) return rt_quot_f64(a - b, a + b);        // a + b < 2^996
-    return (a - b) / (a + b);
+    const double t = a + b;
+    const double q = rt_quot_f64(a - b, t);
+    const double far = __builtin_copysign(1.0, x) + (t - t);     // t - t: 0 for a finite sum, NaN for inf and NaN
+    return __builtin_fabs(x) < 690.0 ? q : far;
 }
-// exp(-x) next to a = exp(x), for tanh, sinh and cosh.  f64: away from the ends of the range it is 1 / a from the refined reciprocal
-// (within an ulp, as the library's exponential is) at a quarter of a second exponential's instructions; beyond +-690, where a leaves
-// the normal numbers, and for NaN it is the exponential itself.
+// exp(-x) next to a = exp(x), for tanh, sinh and cosh.  f64: 1 / a from the refined reciprocal (within an ulp, as the library's
+// exponential is) at a quarter of a second exponential's instructions.  Where the refinement has no answer -- a = 0 and a = inf, the
+// exponential under- or overflowed -- the raw estimate has the right one (inf, 0).
 __device__ __forceinline__ float exp_neg(float x, float a) { return m_exp(-x); }
 __device__ __forceinline__ double exp_neg(double x, double a) {
-    if (__builtin_fabs(x) < 690.0) return rt_rcp_f64(a);
-    return m_exp(-x);
+    const double seed = rt_rcp_seed_f64(a);
+    double r = __builtin_fma(__builtin_fma(-a, seed, 1.0), seed, seed);
+    r = __builtin_fma(__builtin_fma(-a, r, 1.0), r, r);
+    return r != r ? seed : r;
 }
 // sqrt(x^2 + 1) of asinh: the argument is at least 1, so the scaling and the zero / denormal handling of the general square root fall
 // away (within an ulp).

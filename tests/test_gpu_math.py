@@ -164,6 +164,14 @@ def test_f64_sigmoid_tanh_asinh_atanh_close_to_the_formulas(hip):
     with np.errstate(all="ignore"):
         got = device_unary(hip, "f64", "atanh", sp)
         assert got[0] == 0 and got[1] == np.inf and got[2] == -np.inf and np.isnan(got[3:7]).all()
+        got = device_unary(hip, "f64", "atanh", np.array([1e308, -1e308, 1.5, -1.0000000000000002, np.nextafter(1.0, 0)]))
+        assert np.isnan(got[:4]).all() and abs(got[4] - np.arctanh(np.nextafter(1.0, 0))) < 1e-13
+        got = device_unary(hip, "f64", "tanh", np.array([700.0, -700.0, 709.0, -709.0, 720.0, -720.0, 20.0]))
+        assert got[0] == 1.0 and got[1] == -1.0 and got[2] == 1.0 and got[3] == -1.0 and np.isnan(got[4]) and np.isnan(got[5]) and got[6] == 1.0
+        got = device_unary(hip, "f64", "sinh", np.array([720.0, -720.0, 700.0, -700.0]))
+        assert got[0] == np.inf and got[1] == -np.inf and abs(got[2] / np.sinh(700.0) - 1) < 1e-14 and abs(got[3] / np.sinh(-700.0) - 1) < 1e-14
+        got = device_unary(hip, "f64", "cosh", np.array([720.0, -720.0, -700.0, 0.0]))
+        assert got[0] == np.inf and got[1] == np.inf and abs(got[2] / np.cosh(700.0) - 1) < 1e-14 and got[3] == 1.0
         got = device_unary(hip, "f64", "sigmoid", sp)
         assert got[0] == 0.5 and got[4] == 1.0 and got[5] == 0.0 and np.isnan(got[6]) and got[7] == 1.0 and got[8] == 0.0
         got = device_unary(hip, "f64", "tanh", sp)       # the reference's (e^x - e^-x) / (e^x + e^-x) is inf / inf beyond +-710
