@@ -141,9 +141,11 @@ int32_t rt_fill_nd(rt_ctx* ctx, int32_t dtype, void* buf, uint64_t buf_len, cons
 /* ---- in-place unary ops (Backend::apply_<op>_{contiguous,1d_strided,nd}, backend/mod.rs:96-141, 311-355) ------ */
 /* The exact ops (neg, relu, abs, sqrt, reciprocal, square, cube, sign, the four roundings) give the bits of the reference's Cpu
  * backend.  The transcendental ops are within the reference's own test tolerance of 1e-5 but not bit-identical to the platform
- * libm it calls; where the backend computes by its own routine the bound is: f64 ln within 1 ulp of the exact value, f64 ln1p
- * within 3 ulp, f32 ln1p within 3.5 ulp; f64 asinh / acosh / atanh and the log(base) / log1p(base) scalar ops build on that
- * logarithm. */
+ * libm it calls.  Where the backend computes by its own routine instead of the device library's the bound is, in units of the last
+ * place of the exact value: f64 ln and ln1p 1, f64 asin 2, f64 acos 1.5, f64 tan 3 (arguments below 2^30; the library routine
+ * beyond), f32 ln1p 3.5.  f64 sigmoid, silu, tanh, sinh, cosh, asinh, acosh, atanh and the log(base) / log1p(base) scalar ops are
+ * the reference's formulas over these routines and the library's exponential, with quotients and square roots that are within an
+ * ulp instead of correctly rounded; at the ends of their ranges (overflow, +-1, +-inf, NaN) they return what the formulas return. */
 int32_t rt_unary_contiguous(rt_ctx* ctx, int32_t dtype, int32_t op, void* buf, uint64_t buf_len, uint64_t start, uint64_t len);
 int32_t rt_unary_1d_strided(rt_ctx* ctx, int32_t dtype, int32_t op, void* buf, uint64_t buf_len,
                             uint64_t offset, int64_t stride, uint64_t len);

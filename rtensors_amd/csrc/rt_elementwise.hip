@@ -104,11 +104,11 @@ __device__ __forceinline__ double m_log1p(double x) { return rt_log1p_f64(x); }
 __device__ __forceinline__ float m_sqrt(float x) { return sqrtf(x); }
 __device__ __forceinline__ double m_sqrt(double x) { return sqrt(x); }
 __device__ __forceinline__ float m_sin(float x) { return sinf(x); }
-// f64 sine, cosine, tangent: by hand below 2^30 (rt_math64.h), the library routine with its full-range reduction beyond, for infinities and NaN
-__device__ __forceinline__ double m_sin(double x) { return rt_trig_in_range(x) ? rt_sin_f64(x) : sin(x); }
+__device__ __forceinline__ double m_sin(double x) { return sin(x); }
 __device__ __forceinline__ float m_cos(float x) { return cosf(x); }
-__device__ __forceinline__ double m_cos(double x) { return rt_trig_in_range(x) ? rt_cos_f64(x) : cos(x); }
+__device__ __forceinline__ double m_cos(double x) { return cos(x); }
 __device__ __forceinline__ float m_tan(float x) { return tanf(x); }
+// f64 tangent: by hand below 2^30 (rt_math64.h), the library routine with its full-range reduction beyond, for infinities and NaN
 __device__ __forceinline__ double m_tan(double x) { return rt_trig_in_range(x) ? rt_tan_f64(x) : tan(x); }
 __device__ __forceinline__ float m_asin(float x) { return asinf(x); }
 __device__ __forceinline__ double m_asin(double x) { return rt_asin_f64(x); }      // by hand, as the logarithm (rt_math64.h)

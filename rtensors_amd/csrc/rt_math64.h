@@ -236,14 +236,15 @@ RT_M64 double rt_acos_f64(double x) {
     return big ? (x < 0.0 ? neg : pos) : mid;
 }
 
-// ---- f64 sine, cosine, tangent ---------------------------------------------------------------------------------------------------------
+// ---- f64 tangent ---------------------------------------------------------------------------------------------------------------------
 // For |x| < 2^30: n = nearest integer to x * 2/pi, r = x - n * pi/2 with pi/2 as the sum of three doubles -- the first product is
 // subtracted exactly by the fused multiply-add (every bit of x - n * P1 lies between 2^-52 and 1), the other two bring the remainder
 // to full precision even where x is within 2^-60 of a multiple of pi/2 -- then the classical kernels on |r| <= pi/4 (Sun's fdlibm
-// k_sin.c / k_cos.c: odd and even minimax polynomials of degree 13 and 14), and for the tangent their quotient, sin / cos in even
-// quadrants and -cos / sin in odd ones, from the reciprocal estimate.  Straight-line code, about 45 operations for the tangent against
-// the library routine's 90, which leaves a 1 GiB pass ALU-bound at 0.62 of the memory rate.  Results within 2 ulp (sine, cosine: 1.5 measured, half an ulp of it
-// from rounding r) and 3 ulp (tangent), measured against 80-bit arithmetic by tests/test_math64_host.py.  Larger arguments, infinities and NaN are not for
+// k_sin.c / k_cos.c: odd and even minimax polynomials of degree 13 and 14), and their quotient, sin / cos in even quadrants and
+// -cos / sin in odd ones, from the reciprocal estimate.  Straight-line code at 20 instructions per element fewer than the library's
+// tangent, which leaves a 1 GiB pass ALU-bound at 0.62 of the memory rate.  (The library's sine and cosine are as short as these
+// kernels and more accurate: they stay.)  The tangent is within 3 ulp, measured against 80-bit arithmetic by
+// tests/test_math64_host.py; sine and cosine of the kernels themselves within 1.5.  Larger arguments, infinities and NaN are not for
 // this code (rt_trig_in_range says so): the caller sends them to the library routine, whose reduction handles the whole range.
 RT_M64 bool rt_trig_in_range(double x) { return __builtin_fabs(x) < 0x1p30; }
 
@@ -268,32 +269,6 @@ RT_M64 void rt_sincos_kernel(double r, double* s_out, double* c_out) {
     const double pc = z * __builtin_fma(z, __builtin_fma(z, __builtin_fma(z, __builtin_fma(z, __builtin_fma(z, C6, C5), C4), C3), C2), C1);
     const double hz = 0.5 * z, w = 1.0 - hz;
     *c_out = w + (((1.0 - w) - hz) + z * pc);
-}
-
-// +v or -v by bit 1 of the quadrant (quadrants 2 and 3 of the sine, 1 and 2 of the cosine after the shift by one)
-RT_M64 double rt_flip_sign(double v, int flip) {
-    uint64_t b;
-    memcpy(&b, &v, 8);
-    b ^= (uint64_t)(uint32_t)(flip & 2) << 62;
-    memcpy(&v, &b, 8);
-    return v;
-}
-
-RT_M64 double rt_sin_f64(double x) {
-    int n;
-    const double r = rt_pio2_reduce(x, &n);
-    double s, c;
-    rt_sincos_kernel(r, &s, &c);
-    const double v = rt_flip_sign((n & 1) ? c : s, n);
-    return x == 0.0 ? x : v;                                                    // keeps -0.0
-}
-
-RT_M64 double rt_cos_f64(double x) {
-    int n;
-    const double r = rt_pio2_reduce(x, &n);
-    double s, c;
-    rt_sincos_kernel(r, &s, &c);
-    return rt_flip_sign((n & 1) ? s : c, n + 1);
 }
 
 RT_M64 double rt_tan_f64(double x) {

@@ -25,11 +25,13 @@ extern "C" void rcp_many(size_t n, const double* x, double* y) {
 extern "C" void quot_many(size_t n, const double* a, const double* d, double* y) {
     for (size_t i = 0; i < n; ++i) y[i] = rt_quot_f64(a[i], d[i]);
 }
-extern "C" void sin_many(size_t n, const double* x, double* y) {
-    for (size_t i = 0; i < n; ++i) y[i] = rt_sin_f64(x[i]);
-}
-extern "C" void cos_many(size_t n, const double* x, double* y) {
-    for (size_t i = 0; i < n; ++i) y[i] = rt_cos_f64(x[i]);
+// sine and cosine of the reduced argument as the tangent's kernels form them (the quadrant is not applied)
+extern "C" void sincos_kernel_many(size_t n, const double* x, double* s, double* c) {
+    for (size_t i = 0; i < n; ++i) {
+        int q;
+        const double r = rt_pio2_reduce(x[i], &q);
+        rt_sincos_kernel(r, &s[i], &c[i]);
+    }
 }
 extern "C" void tan_many(size_t n, const double* x, double* y) {
     for (size_t i = 0; i < n; ++i) y[i] = rt_tan_f64(x[i]);

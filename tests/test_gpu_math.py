@@ -1,6 +1,6 @@
 """Error bounds of the functions the device computes with routines of its own instead of the library's (ocml): f64 ln (hand-written,
 rtensors_amd/csrc/rt_math64.h) and f64 ln1p within 1 ulp of the exact value (80-bit reference), f64 asin within 2 and acos within 1.5
-ulp, f64 sin / cos within 2 and tan within 3 ulp below 2^30 (the library routine beyond), f32 ln1p (Kahan's formula over the f32
+ulp, f64 tan within 3 ulp below 2^30 (the library routine beyond; sin and cos are the library's and are held to 2 ulp alongside), f32 ln1p (Kahan's formula over the f32
 logarithm) within 3.5 ulp of the f64 result.  The reference's Cpu backend calls Rust's f64::ln / ln_1p (platform libm, under
 1 ulp) and its tests hold these ops to 1e-5, so bit parity is unpinned here; what a caller can rely on is the bound asserted below.
 The ops built on the logarithm (log_b, log1p_b, asinh, acosh, atanh) are held to the oracle at the reference's 1e-5 elsewhere."""

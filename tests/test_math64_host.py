@@ -18,9 +18,10 @@ def lib(tmp_path_factory):
     out = str(tmp_path_factory.mktemp("math64") / "libmath64.so")
     subprocess.check_call(["g++", "-O2", "-ffp-contract=off", "-shared", "-fPIC", "-o", out, os.path.join(HERE, "support", "math64_host.cpp")])
     L = C.CDLL(out)
-    for f in (L.log_many, L.log1p_many, L.asin_many, L.acos_many, L.sin_many, L.cos_many, L.tan_many, L.sqrt_ge1_many, L.rcp_many):
+    for f in (L.log_many, L.log1p_many, L.asin_many, L.acos_many, L.tan_many, L.sqrt_ge1_many, L.rcp_many):
         f.argtypes = [C.c_size_t, C.c_void_p, C.c_void_p]
     L.quot_many.argtypes = [C.c_size_t, C.c_void_p, C.c_void_p, C.c_void_p]
+    L.sincos_kernel_many.argtypes = [C.c_size_t, C.c_void_p, C.c_void_p, C.c_void_p]
     return L
 
 
@@ -124,18 +125,21 @@ def trig_arguments(rng):
     return x[np.abs(x) < 2.0 ** 30]
 
 
-def test_sin_cos_tan_below_2_30(lib):
+def test_tan_below_2_30(lib):
     need_long_double()
     x = trig_arguments(np.random.default_rng(7))
     xl = x.astype(np.longdouble)
-    for name, fn, exact, bound in (("sin", lib.sin_many, np.sin(xl), 2.0), ("cos", lib.cos_many, np.cos(xl), 2.0), ("tan", lib.tan_many, np.tan(xl), 3.0)):
-        err = ulp_error(call(fn, x), exact)
-        assert err.max() < bound, (name, float(err.max()), float(x[err.argmax()]))
+    err = ulp_error(call(lib.tan_many, x), np.tan(xl))
+    assert err.max() < 3.0, ("tan", float(err.max()), float(x[err.argmax()]))
     sp = np.array([0.0, -0.0, 5e-324, -5e-324, 1e-300, np.pi / 2, np.pi, -np.pi / 4])
-    for fn, ref in ((lib.sin_many, np.sin), (lib.tan_many, np.tan)):
-        got = call(fn, sp)
-        assert np.array_equal(got, ref(sp)) and np.signbit(got[1]) and not np.signbit(got[0])
-    assert np.array_equal(call(lib.cos_many, sp), np.cos(sp))
+    got = call(lib.tan_many, sp)
+    assert np.array_equal(got, np.tan(sp)) and np.signbit(got[1]) and not np.signbit(got[0])
+    # the two kernels under it, on arguments within a quarter turn of 0 (no quadrant): sine and cosine within 1.5 ulp
+    y = np.ascontiguousarray(np.concatenate([np.random.default_rng(8).uniform(-np.pi / 4, np.pi / 4, 500_000), 10.0 ** np.random.default_rng(9).uniform(-300, -1, 100_000)]))
+    s_out, c_out = np.empty_like(y), np.empty_like(y)
+    lib.sincos_kernel_many(y.size, y.ctypes.data, s_out.ctypes.data, c_out.ctypes.data)
+    yl = y.astype(np.longdouble)
+    assert ulp_error(s_out, np.sin(yl)).max() < 1.5 and ulp_error(c_out, np.cos(yl)).max() < 1.5
 
 
 def test_reciprocal_quotient_and_square_root_helpers(lib):
