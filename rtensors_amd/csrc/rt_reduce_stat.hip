@@ -317,7 +317,7 @@ __global__ __launch_bounds__(kBlock) void st_rows_tile_kernel(const T* __restric
     if (threadIdx.x < head) put(threadIdx.x, p[threadIdx.x]);
     const uint32_t nvec = (ne - head) / N;
     const Vec16<T>* pv = reinterpret_cast<const Vec16<T>*>(p + head);
-    constexpr int U = 8;                                           // the whole 32 KiB tile in flight at once: 8 vectors per lane
+    constexpr int U = 8;                                           // the whole tile in flight at once (six vectors per lane at 24 KiB)
     for (uint32_t v0 = threadIdx.x; v0 < nvec; v0 += U * kBlock) {
         Vec16<T> x[U];
 #pragma unroll
