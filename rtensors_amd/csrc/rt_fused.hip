@@ -248,8 +248,12 @@ int32_t bias_relu_l1_typed(rt_ctx* ctx, int dtype, const void* x, const void* bi
 }
 
 template <class T>
-int32_t backward_typed(rt_ctx* ctx, int dtype, const void* gmap, const void* y, const void* up, void* dbias, uint64_t rows, uint64_t cols, bool from_target) {
+int32_t backward_typed(rt_ctx* ctx, int dtype, const void* gmap, const void* y, const void* up, void* dbias, uint64_t rows_all, uint64_t cols_out, bool from_target) {
     constexpr uint64_t N = 16 / sizeof(T);
+    // Short rows are regrouped as in the column reduction (rt_reduce.hip, cols_launch): g consecutive rows are read as one row of
+    // g * cols columns, and the g partial sums per column join the partials of the split in the column sum that follows.
+    const uint64_t g = rt_cols_regroup(rows_all, cols_out * sizeof(T));
+    const uint64_t rows = rows_all / g, cols = cols_out * g;
     const uint64_t tiles = (cols / N + RT_WAVE - 1) / RT_WAVE;
     const uint64_t want = (uint64_t)ctx->num_cus * 2;              // two resident blocks per CU, as the column reduction
     uint64_t splits = 1;
@@ -264,7 +268,8 @@ int32_t backward_typed(rt_ctx* ctx, int dtype, const void* gmap, const void* y, 
     splits = (rows + seglen - 1) / seglen;
     if (tiles * splits >= (1ull << 31)) return rt_fail(RT_E_INVALID, "fused backward: too many blocks for one launch");
     void* part = dbias;
-    if (splits > 1) RT_TRY(rt_alloc_bytes(ctx, (size_t)(splits * cols) * sizeof(T), &part));
+    const bool staged = splits > 1 || g > 1;
+    if (staged) RT_TRY(rt_alloc_bytes(ctx, (size_t)(splits * cols) * sizeof(T), &part));
     const T count = (T)(float)(rows * cols);                       // WeightValue::from_usize goes through f32 (core/value.rs:54-56)
     if (from_target)
         hipLaunchKernelGGL((fused_backward_cols_kernel<T, true>), dim3((unsigned)(tiles * splits)), dim3(kFBlock), 0, ctx->stream, (const T*)gmap, (const T*)y,
@@ -274,8 +279,8 @@ int32_t backward_typed(rt_ctx* ctx, int dtype, const void* gmap, const void* y, 
                            (const T*)up, (T*)part, rows, cols, (uint32_t)tiles, seglen, count);
     hipError_t e = hipGetLastError();
     int32_t st = e == hipSuccess ? RT_OK : rt_hip_fail(e, "fused backward launch");
-    if (splits > 1) {
-        if (st == RT_OK) st = rt_reduce_cols(ctx, dtype, RT_R_SUM, part, dbias, splits, cols);
+    if (staged) {
+        if (st == RT_OK) st = rt_reduce_cols(ctx, dtype, RT_R_SUM, part, dbias, splits * g, cols_out);
         (void)rt_free_locked(ctx, part);
     }
     return st;

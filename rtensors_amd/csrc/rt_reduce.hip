@@ -688,9 +688,14 @@ int32_t rows_stage(rt_ctx* ctx, const T* src, T* out, uint64_t rows, uint64_t R,
 }
 
 template <int OP, class T, int VW>
-int32_t cols_launch(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t R, uint64_t inner, uint64_t count, bool allow_split) {
+int32_t cols_launch(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t R_all, uint64_t inner_out, uint64_t count, bool allow_split) {
     hipStream_t s = ctx->stream;
     const uint64_t per_tile = (uint64_t)RT_WAVE * VW;
+    // Short rows are regrouped (rt_cols_regroup): g consecutive rows of `inner_out` columns are read as one row of g * inner_out
+    // columns, and the g partial results per column join the partials of the split in the second stage.  Not for the float max / min
+    // (their tie-breaking follows row positions) and only for one outer index.
+    const uint64_t g = (allow_split && outer == 1 && !Acc<OP, T>::kTrack && inner_out % VW == 0) ? rt_cols_regroup(R_all, inner_out * sizeof(T)) : 1;
+    const uint64_t R = R_all / g, inner = inner_out * g;
     const uint64_t tiles = (inner + per_tile - 1) / per_tile;
     // One block of four waves per CU, eight loads in flight per lane, each block streaming a long run of rows: the segments are cut so
     // that the blocks do not outnumber the CUs (1 GiB f32 sums over axis 0, against two blocks per CU: 8192 x 32768 0.857 -> 0.893 of
@@ -719,7 +724,7 @@ int32_t cols_launch(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t 
     }
     const uint64_t blocks = outer * splits * tiles;
     if (blocks >= (1ull << 31) || tiles >= (1ull << 31)) return rt_fail(RT_E_INVALID, "reduce: too many outputs for one launch");
-    if (splits == 1) {
+    if (splits == 1 && g == 1) {
         // (eight loads in flight per lane from 256 rows on; a short axis would spend its time in the one-row-at-a-time remainder)
         if (R >= 256)
             hipLaunchKernelGGL((reduce_cols_kernel<OP, T, VW, 8>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, out, R, inner, outer,
@@ -736,13 +741,13 @@ int32_t cols_launch(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t 
     hipLaunchKernelGGL((reduce_cols_kernel<OP, T, VW, 8>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, part, R, inner, outer,
                        (uint32_t)tiles, splits, seglen, count, 0);
     RT_HIP(hipGetLastError());
-    // second stage: partials are (splits, outer*inner): a column reduce with R = splits
-    const uint64_t inner2 = outer * inner;
-    if (merge_few_outputs<OP, T>(ctx, part, out, inner2, splits, count)) { RT_HIP(hipGetLastError()); return RT_OK; }
+    // second stage: partials are (splits, outer * inner) -- with regrouped rows (splits * g, inner_out): a column reduce with R = splits * g
+    const uint64_t inner2 = outer * inner_out, R2 = (uint64_t)splits * g;
+    if (merge_few_outputs<OP, T>(ctx, part, out, inner2, (uint32_t)R2, count)) { RT_HIP(hipGetLastError()); return RT_OK; }
     const uint64_t tiles2 = (inner2 + per_tile - 1) / per_tile;
     if (tiles2 >= (1ull << 31)) return rt_fail(RT_E_INVALID, "reduce: too many outputs for one launch");
-    hipLaunchKernelGGL((reduce_cols_kernel<OP, T, VW>), dim3((unsigned)tiles2), dim3(kBlock), 0, s, part, out, (uint64_t)splits, inner2, (uint64_t)1,
-                       (uint32_t)tiles2, 1u, (uint64_t)splits, count, 1);
+    hipLaunchKernelGGL((reduce_cols_kernel<OP, T, VW>), dim3((unsigned)tiles2), dim3(kBlock), 0, s, part, out, R2, inner2, (uint64_t)1,
+                       (uint32_t)tiles2, 1u, R2, count, 1);
     RT_HIP(hipGetLastError());
     return RT_OK;
 }

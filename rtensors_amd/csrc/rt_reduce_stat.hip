@@ -48,7 +48,10 @@ __device__ __forceinline__ double m_recip(double x) { return 1.0 / x; }
 
 template <class T> struct MomentState {
     typedef T Out;
-    static constexpr int kColsBlocksPerCU = 2;
+    // column kernel: resident blocks per CU and loads in flight per lane.  1 GiB f32 over axis 0: 0.90 of peak with one fat block and
+    // eight loads (the plain column sum's shape), 0.86 with two blocks and four loads, 0.80 with four blocks
+    static constexpr int kColsBlocksPerCU = 1;
+    static constexpr int kColsLoads = 8;
     static constexpr int kNarrowBlocksPerCU = 2;   // narrow-column kernel: resident blocks per CU (1 GiB over 3 and 100 columns: 0.85 .. 0.88 of peak with 2, 0.79 .. 0.81 with 4)
     T mean, m2;
     double n;                                                   // a count, exact up to 2^53; as a double it converts to T in one instruction
@@ -84,7 +87,9 @@ template <class T> struct MomentState {
 
 template <class T> struct LseState {
     typedef T Out;
-    static constexpr int kColsBlocksPerCU = 4;                  // one exp per element: more waves per CU to hide it (0.215 -> 0.180 ms on 1 GiB)
+    // one exp per element: two blocks of four loads (0.87 of peak; one fat block 0.78, four blocks 0.82)
+    static constexpr int kColsBlocksPerCU = 2;
+    static constexpr int kColsLoads = 4;
     static constexpr int kNarrowBlocksPerCU = 2;
     T m, s;
     __device__ __forceinline__ void init() { m = -std::numeric_limits<T>::infinity(); s = (T)0; }
@@ -130,7 +135,8 @@ template <class T> struct LseState {
 
 template <class T, bool SQ> struct NormState {
     typedef T Out;
-    static constexpr int kColsBlocksPerCU = 2;
+    static constexpr int kColsBlocksPerCU = 1;                  // as MomentState
+    static constexpr int kColsLoads = 8;
     static constexpr int kNarrowBlocksPerCU = 2;
     T s;
     __device__ __forceinline__ void init() { s = (T)0; }
@@ -147,7 +153,8 @@ template <class T, bool SQ> struct NormState {
 
 template <class T, bool MAX> struct ArgState {
     typedef uint64_t Out;
-    static constexpr int kColsBlocksPerCU = 2;
+    static constexpr int kColsBlocksPerCU = 2;                  // 0.85 of peak; one fat block 0.76, four blocks 0.80
+    static constexpr int kColsLoads = 4;
     static constexpr int kNarrowBlocksPerCU = 3;   // narrow columns: 0.80 with 3 or 4, 0.71 with 2
     T v;
     uint64_t idx;
@@ -389,10 +396,9 @@ __global__ __launch_bounds__(kBlock) void st_rows_pow2_kernel(const T* __restric
 // ---- cols -------------------------------------------------------------------------------------------------------------
 // src viewed as (outer, R, inner).  blockIdx.x -> (o, seg, tile); lane tx covers columns (tile * 64 + tx) * VW ..; wave ty takes
 // k = begin + ty, + kWaves, ...  Results go to out[o * inner + col], partial states to part[(seg * outer + o) * inner + col].
-template <class S, class T, int VW>
+template <class S, class T, int VW, int U = 4>
 __global__ __launch_bounds__(kBlock) void st_cols_kernel(const T* __restrict__ src, typename S::Out* __restrict__ out, S* __restrict__ part, uint64_t R,
                                                          uint64_t inner, uint64_t outer, uint32_t tiles, uint32_t splits, uint64_t seglen, int flags) {
-    constexpr int U = 4;
     struct alignas(sizeof(T) * VW) VecW { T e[VW]; };
     uint64_t b = blockIdx.x;
     const uint32_t tile = (uint32_t)(b % tiles);
@@ -682,12 +688,19 @@ int32_t rows_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t rows
     return RT_OK;
 }
 
+template <class S> struct is_arg_state : std::false_type {};
+template <class T, bool MAX> struct is_arg_state<ArgState<T, MAX>> : std::true_type {};
+
 template <class S, class T, int VW>
-int32_t cols_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t outer, uint64_t R, uint64_t inner, int flags) {
+int32_t cols_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t outer, uint64_t R_all, uint64_t inner_out, int flags) {
     hipStream_t s = ctx->stream;
     const uint64_t per_tile = (uint64_t)RT_WAVE * VW;
+    // Short rows are regrouped as in the plain column reduction (rt_cols_regroup): g consecutive rows are read as one, and the g
+    // partial states per column join those of the split in the merge.  Not for the index states (their positions are row numbers).
+    const uint64_t g = (outer == 1 && !is_arg_state<S>::value && inner_out % VW == 0) ? rt_cols_regroup(R_all, inner_out * sizeof(T)) : 1;
+    const uint64_t R = R_all / g, inner = inner_out * g;
     const uint64_t tiles = (inner + per_tile - 1) / per_tile;
-    const uint64_t want = (uint64_t)ctx->num_cus * S::kColsBlocksPerCU;       // resident blocks per CU (2 measured best for the cheap states)
+    const uint64_t want = (uint64_t)ctx->num_cus * S::kColsBlocksPerCU;
     uint32_t splits = 1;
     if (outer * tiles < want) {
         const uint64_t min_seg = 64;
@@ -698,21 +711,22 @@ int32_t cols_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t oute
     }
     uint64_t seglen = (R + splits - 1) / splits;
     if (splits > 1) {
-        seglen = (seglen + 4 * kWaves - 1) / (4 * kWaves) * (4 * kWaves);
+        seglen = (seglen + 8 * kWaves - 1) / (8 * kWaves) * (8 * kWaves);
         splits = (uint32_t)((R + seglen - 1) / seglen);
     }
     const uint64_t blocks = outer * splits * tiles;
     if (blocks >= (1ull << 31) || tiles >= (1ull << 31)) return too_many();
     S* part = nullptr;
-    if (splits > 1) {
+    const bool staged = splits > 1 || g > 1;
+    if (staged) {
         void* scratch = nullptr;
         RT_TRY(rt_scratch(ctx, (size_t)(splits * outer * inner) * sizeof(S), &scratch));
         part = (S*)scratch;
     }
-    hipLaunchKernelGGL((st_cols_kernel<S, T, VW>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, out, part, R, inner, outer, (uint32_t)tiles, splits, seglen,
-                       flags);
+    hipLaunchKernelGGL((st_cols_kernel<S, T, VW, S::kColsLoads>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, out, part, R, inner, outer, (uint32_t)tiles,
+                       splits, seglen, flags);
     RT_HIP(hipGetLastError());
-    if (splits > 1) RT_TRY(merge_cols<S>(ctx, part, out, outer * inner, splits, flags));
+    if (staged) RT_TRY(merge_cols<S>(ctx, part, out, outer * inner_out, (uint32_t)(splits * g), flags));
     return RT_OK;
 }
 
