@@ -808,7 +808,9 @@ int32_t reduce_typed(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t
     // Which kernel: measured on MI355X over 1 GiB of f32 (sum), TB/s -- rows of 8 / 32 / 100 / 256 elements 4.8 / 5.2 / 5.4 / 5.7;
     // columns with inner 3 / 17 / 100 5.0 / 5.0 / 4.8; (65536, 64, 64) 6.4; (2^20, 4, 64) 5.4.  One lane or one wave per short row
     // gave 0.3-2.3, lanes along a narrow inner 0.2-1.2.
-    if (R <= 32 && inner <= 1024) {                                             // short reduced axis: a lane per output vector
+    // short reduced axis: a lane per output vector.  Also for slabs of at most 8 KiB with up to 256 rows, which leave a block of the
+    // narrow-column kernel too little to do ((262144, 64, 16) f32: 0.35 -> 0.61 of peak; from 16 KiB on the narrow kernel wins)
+    if ((R <= 32 || (R <= 256 && R * inner * sizeof(T) <= 8192)) && inner <= 1024) {
         const bool v = inner % N == 0;                                          // rows may start at any element
         const uint64_t ivecs = v ? inner / N : inner;
         if (ivecs < (1ull << 31) && outer * ivecs < (1ull << 31)) {
