@@ -177,6 +177,9 @@ template <class T, bool MAX> struct ArgState {
 };
 
 // a state moved between lanes as 32-bit words
+template <class S> struct is_arg_state : std::false_type {};
+template <class T, bool MAX> struct is_arg_state<ArgState<T, MAX>> : std::true_type {};
+
 template <class S> __device__ __forceinline__ S shfl_down_state(const S& s, int d) {
     static_assert(sizeof(S) % 4 == 0, "state is a whole number of words");
     constexpr int W = sizeof(S) / 4;
@@ -695,7 +698,14 @@ int32_t rows_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t rows
         if (kCheap && R * sizeof(T) >= 80 * 1024 && R * sizeof(T) <= 256 * 1024)
             hipLaunchKernelGGL((st_rows_block_kernel<S, T, 8>), dim3((unsigned)rows), dim3(kBlock), kRtThreeBlocksLds, s, src, out, (S*)nullptr, R, 1u, R, flags);
         else
-            hipLaunchKernelGGL((st_rows_block_kernel<S, T>), dim3((unsigned)rows), dim3(kBlock), kRtFourBlocksLds, s, src, out, (S*)nullptr, R, 1u, R, flags);
+        {
+            // The cap of four resident blocks per CU (fewer, fatter streams) pays from rows of 32 KiB on -- 48 KiB for the index
+            // states.  Below that a block is done after one trip and its fold of the states, which is long against the trip, needs the
+            // other blocks' loads to hide behind: rows of 16 KiB ran at 0.62 - 0.70 of peak with the cap and run at 0.84 - 0.87 without.
+            const size_t cap_from = is_arg_state<S>::value ? 48 * 1024 : 32 * 1024;
+            const size_t lds = R * sizeof(T) >= cap_from ? kRtFourBlocksLds : 0;
+            hipLaunchKernelGGL((st_rows_block_kernel<S, T>), dim3((unsigned)rows), dim3(kBlock), lds, s, src, out, (S*)nullptr, R, 1u, R, flags);
+        }
         RT_HIP(hipGetLastError());
         return RT_OK;
     }
@@ -720,9 +730,6 @@ int32_t rows_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t rows
     RT_HIP(hipGetLastError());
     return RT_OK;
 }
-
-template <class S> struct is_arg_state : std::false_type {};
-template <class T, bool MAX> struct is_arg_state<ArgState<T, MAX>> : std::true_type {};
 
 template <class S, class T, int VW>
 int32_t cols_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t outer, uint64_t R_all, uint64_t inner_out, int flags) {
