@@ -15,8 +15,10 @@
 //   fences write back and invalidate whole L2s, about 0.7 us per block, which doubled the 1 GiB full sum to 0.35 ms.
 //
 // Exactness: integer sum/prod wrap, so any association gives the sequential result; max/min are order independent
-// except for the sign of a zero result (-0.0 == 0.0, the sequential loop keeps the first), which is kept by
-// carrying the position of the current extremum.  Float sum/prod/mean are tree results.
+// except for the sign of a zero result (-0.0 == 0.0, the sequential loop keeps the first).  Where lanes fold interleaved
+// positions, the float max / min therefore run in two forms: a quick one that also notes whether a -0.0 was among the
+// elements (a zero result without one is +0.0), and, only when a zero result did meet a -0.0, the same fold again with the
+// position of the current extremum carried along.  Float sum/prod/mean are tree results.
 #include "rt_common.h"
 
 #include <type_traits>
@@ -36,21 +38,32 @@ template <class T> __device__ __host__ constexpr T highest_of() { return std::nu
 constexpr int kBlock = 256;
 constexpr int kWaves = kBlock / RT_WAVE;
 
-// Accumulator state.  `pos` is only carried for float max/min (see the header comment).
-template <int OP, class T> struct Acc {
-    static constexpr bool kTrack = is_flt<T>::value && (OP == RT_R_MAX || OP == RT_R_MIN);
+template <class T> __device__ __forceinline__ T shfl_down_t(T v, int d) { return __shfl_down(v, d, RT_WAVE); }
+template <> __device__ __forceinline__ uint8_t shfl_down_t<uint8_t>(uint8_t v, int d) { return (uint8_t)__shfl_down((int)v, d, RT_WAVE); }
+template <> __device__ __forceinline__ int8_t shfl_down_t<int8_t>(int8_t v, int d) { return (int8_t)__shfl_down((int)v, d, RT_WAVE); }
+template <> __device__ __forceinline__ uint16_t shfl_down_t<uint16_t>(uint16_t v, int d) { return (uint16_t)__shfl_down((int)v, d, RT_WAVE); }
+template <> __device__ __forceinline__ int16_t shfl_down_t<int16_t>(int16_t v, int d) { return (int16_t)__shfl_down((int)v, d, RT_WAVE); }
+template <> __device__ __forceinline__ uint32_t shfl_down_t<uint32_t>(uint32_t v, int d) { return (uint32_t)__shfl_down((int)v, d, RT_WAVE); }
+template <> __device__ __forceinline__ uint64_t shfl_down_t<uint64_t>(uint64_t v, int d) { return (uint64_t)__shfl_down((unsigned long long)v, d, RT_WAVE); }
+template <> __device__ __forceinline__ int64_t shfl_down_t<int64_t>(int64_t v, int d) { return (int64_t)__shfl_down((long long)v, d, RT_WAVE); }
+
+// Accumulator state.  TRACK: the position of the current extremum is carried, so that partial folds over interleaved positions
+// merge to the sequential result (float max / min only, see the header comment); without it a merge keeps its own value on ties,
+// which is the sequential result when everything in `o` comes after everything folded so far.
+template <int OP, class T, bool TRACK, class P = uint64_t> struct AccT {
+    static constexpr bool kTrack = TRACK;
     T v;
-    uint64_t pos;
+    P pos;                  // P = uint32_t where a kernel's positions are known to fit (half the registers and shuffles)
 
     __device__ __forceinline__ void init() {
         if constexpr (OP == RT_R_SUM || OP == RT_R_MEAN) v = (T)0;
         else if constexpr (OP == RT_R_PROD) v = (T)1;
         else if constexpr (OP == RT_R_MAX) v = lowest_of<T>();
         else v = highest_of<T>();
-        pos = ~0ull;
+        pos = (P)~(P)0;
     }
     // fold one element that comes after everything folded so far (ascending position)
-    __device__ __forceinline__ void push(T x, uint64_t p) {
+    __device__ __forceinline__ void push(T x, P p) {
         if constexpr (OP == RT_R_SUM || OP == RT_R_MEAN) {
             if constexpr (is_flt<T>::value) v = v + x;
             else { typedef typename carrier<T>::type W; v = (T)(W)((W)v + (W)x); }
@@ -63,8 +76,8 @@ template <int OP, class T> struct Acc {
             if (x < v) { v = x; if constexpr (kTrack) pos = p; }
         }
     }
-    // merge another partial state (any relative order)
-    __device__ __forceinline__ void merge(const Acc& o) {
+    // merge another partial state (any relative order when positions are tracked)
+    __device__ __forceinline__ void merge(const AccT& o) {
         if constexpr (OP == RT_R_SUM || OP == RT_R_MEAN) {
             if constexpr (is_flt<T>::value) v = v + o.v;
             else { typedef typename carrier<T>::type W; v = (T)(W)((W)v + (W)o.v); }
@@ -79,6 +92,62 @@ template <int OP, class T> struct Acc {
             else { if (o.v < v) v = o.v; }
         }
     }
+    __device__ __forceinline__ AccT shfl_down(int d) const {
+        AccT o;
+        o.v = shfl_down_t<T>(v, d);
+        if constexpr (kTrack) o.pos = shfl_down_t<P>(pos, d); else o.pos = 0;
+        return o;
+    }
+    __device__ __forceinline__ bool settled() const { return true; }
+    __device__ __forceinline__ T value() const { return v; }
+    // what a state carries besides its value, for the kernels that pass states through LDS as separate arrays
+    static constexpr bool kExtra = TRACK;
+    typedef P extra_t;
+    __device__ __forceinline__ extra_t extra() const { return pos; }
+    __device__ __forceinline__ static AccT make(T v, extra_t e) { AccT a; a.v = v; a.pos = e; return a; }
+};
+template <int OP, class T> struct needs_order : std::integral_constant<bool, is_flt<T>::value && (OP == RT_R_MAX || OP == RT_R_MIN)> {};
+// the accumulator for folds over interleaved positions / for folds whose merges go in ascending order of position
+template <int OP, class T> using Acc = AccT<OP, T, needs_order<OP, T>::value>;
+template <int OP, class T> using AccOrd = AccT<OP, T, false>;
+
+// The quick form of the float max / min over interleaved positions: no positions, but the signed minimum `m` of the elements' upper
+// 32 bits, which is INT_MIN exactly when a -0.0 was folded (for f64 also for a negative denormal below 2^-1042: a rare false
+// alarm).  A zero result with no -0.0 among the elements is +0.0 whatever the order; a zero result that met one is `unsettled`, and
+// the caller folds again with AccT<OP, T, true>.
+template <class T> __device__ __forceinline__ int32_t upper_bits(T x) {
+    if constexpr (sizeof(T) == 4) return __builtin_bit_cast(int32_t, x);
+    else return (int32_t)(__builtin_bit_cast(uint64_t, x) >> 32);
+}
+template <int OP, class T> struct AccQuick {
+    static constexpr bool kTrack = false;
+    T v;
+    int32_t m;
+    __device__ __forceinline__ void init() {
+        v = OP == RT_R_MAX ? lowest_of<T>() : highest_of<T>();
+        m = 0;
+    }
+    __device__ __forceinline__ void push(T x, uint64_t) {
+        if constexpr (OP == RT_R_MAX) { if (x > v) v = x; } else { if (x < v) v = x; }
+        const int32_t b = upper_bits<T>(x);
+        m = b < m ? b : m;
+    }
+    __device__ __forceinline__ void merge(const AccQuick& o) {
+        if constexpr (OP == RT_R_MAX) { if (o.v > v) v = o.v; } else { if (o.v < v) v = o.v; }
+        m = o.m < m ? o.m : m;
+    }
+    __device__ __forceinline__ AccQuick shfl_down(int d) const {
+        AccQuick o;
+        o.v = shfl_down_t<T>(v, d);
+        o.m = __shfl_down(m, d, RT_WAVE);
+        return o;
+    }
+    __device__ __forceinline__ bool settled() const { return !(v == (T)0 && m == INT32_MIN); }
+    __device__ __forceinline__ T value() const { return v == (T)0 ? (T)0 : v; }      // a settled zero is +0.0
+    static constexpr bool kExtra = true;
+    typedef int32_t extra_t;
+    __device__ __forceinline__ extra_t extra() const { return m; }
+    __device__ __forceinline__ static AccQuick make(T v, extra_t e) { AccQuick a; a.v = v; a.m = e; return a; }
 };
 
 // WeightValue::from_usize goes through f32 (core/value.rs:54-56); integers saturate like Rust's `as`.
@@ -105,45 +174,43 @@ template <int OP, class T> __device__ __forceinline__ T finalize(T v, uint64_t c
     }
 }
 
-template <class T> __device__ __forceinline__ T shfl_down_t(T v, int d) { return __shfl_down(v, d, RT_WAVE); }
-template <> __device__ __forceinline__ uint8_t shfl_down_t<uint8_t>(uint8_t v, int d) { return (uint8_t)__shfl_down((int)v, d, RT_WAVE); }
-template <> __device__ __forceinline__ int8_t shfl_down_t<int8_t>(int8_t v, int d) { return (int8_t)__shfl_down((int)v, d, RT_WAVE); }
-template <> __device__ __forceinline__ uint16_t shfl_down_t<uint16_t>(uint16_t v, int d) { return (uint16_t)__shfl_down((int)v, d, RT_WAVE); }
-template <> __device__ __forceinline__ int16_t shfl_down_t<int16_t>(int16_t v, int d) { return (int16_t)__shfl_down((int)v, d, RT_WAVE); }
-template <> __device__ __forceinline__ uint64_t shfl_down_t<uint64_t>(uint64_t v, int d) { return (uint64_t)__shfl_down((unsigned long long)v, d, RT_WAVE); }
-template <> __device__ __forceinline__ int64_t shfl_down_t<int64_t>(int64_t v, int d) { return (int64_t)__shfl_down((long long)v, d, RT_WAVE); }
-
 // wave64 tree: after it lane 0 holds the fold of all 64 lanes
-template <int OP, class T> __device__ __forceinline__ void wave_reduce(Acc<OP, T>& a) {
+template <class A> __device__ __forceinline__ void wave_reduce(A& a) {
 #pragma unroll
-    for (int d = RT_WAVE / 2; d >= 1; d >>= 1) {
-        Acc<OP, T> o;
-        o.v = shfl_down_t<T>(a.v, d);
-        if constexpr (Acc<OP, T>::kTrack) o.pos = shfl_down_t<uint64_t>(a.pos, d); else o.pos = 0;
-        a.merge(o);
-    }
+    for (int d = RT_WAVE / 2; d >= 1; d >>= 1) a.merge(a.shfl_down(d));
 }
 
 // block of kBlock lanes: result valid in thread 0
-template <int OP, class T> __device__ __forceinline__ void block_reduce(Acc<OP, T>& a) {
-    __shared__ T sv[kWaves];
-    __shared__ uint64_t sp[kWaves];
-    wave_reduce<OP, T>(a);
+template <class A> __device__ __forceinline__ void block_reduce(A& a) {
+    __shared__ A sa[kWaves];
+    wave_reduce<A>(a);
     const int lane = threadIdx.x & (RT_WAVE - 1), w = threadIdx.x / RT_WAVE;
-    if (lane == 0) { sv[w] = a.v; sp[w] = a.pos; }
+    if (lane == 0) sa[w] = a;
     __syncthreads();
     if (threadIdx.x == 0) {
 #pragma unroll
-        for (int k = 1; k < kWaves; ++k) { Acc<OP, T> o; o.v = sv[k]; o.pos = sp[k]; a.merge(o); }
+        for (int k = 1; k < kWaves; ++k) a.merge(sa[k]);
     }
+}
+
+// the same with the result in every lane (one barrier; a decision taken on the result is then uniform without a second one)
+template <class A> __device__ __forceinline__ void block_reduce_all(A& a) {
+    __shared__ A sa[kWaves];
+    wave_reduce<A>(a);
+    const int lane = threadIdx.x & (RT_WAVE - 1), w = threadIdx.x / RT_WAVE;
+    if (lane == 0) sa[w] = a;
+    __syncthreads();
+    a = sa[0];
+#pragma unroll
+    for (int k = 1; k < kWaves; ++k) a.merge(sa[k]);
 }
 
 template <class T> struct alignas(16) Vec16 { T e[16 / sizeof(T)]; };
 
 // fold elements [begin, end) of the contiguous run `p`, lanes `tid` of `nthreads` cooperating; positions are
 // reported relative to `p`
-template <int OP, class T, int U = 4>
-__device__ __forceinline__ void fold_run(Acc<OP, T>& a, const T* __restrict__ p, uint64_t begin, uint64_t end, uint32_t tid, uint32_t nthreads) {
+template <class A, class T, int U = 4>
+__device__ __forceinline__ void fold_run(A& a, const T* __restrict__ p, uint64_t begin, uint64_t end, uint32_t tid, uint32_t nthreads) {
     constexpr uint32_t N = 16 / sizeof(T);
     if (begin >= end) return;
     // elements before the first 16-byte boundary
@@ -196,10 +263,22 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_block_kernel(const T* __re
     const uint64_t begin = (uint64_t)seg * seglen;
     uint64_t end = begin + seglen;
     if (end > R) end = R;
+    const T* p = src + row * R;
+    if constexpr (Acc<OP, T>::kTrack) {
+        // float max / min: the quick form first; the form with positions only when a zero result met a -0.0
+        AccQuick<OP, T> q;
+        q.init();
+        fold_run<AccQuick<OP, T>, T, U>(q, p, begin, end, threadIdx.x, kBlock);
+        block_reduce_all<AccQuick<OP, T> >(q);
+        if (q.settled()) {
+            if (threadIdx.x == 0) out[blockIdx.x] = last ? finalize<OP, T>(q.value(), count) : q.value();
+            return;
+        }
+    }
     Acc<OP, T> a;
     a.init();
-    fold_run<OP, T, U>(a, src + row * R, begin, end, threadIdx.x, kBlock);
-    block_reduce<OP, T>(a);
+    fold_run<Acc<OP, T>, T, U>(a, p, begin, end, threadIdx.x, kBlock);
+    block_reduce<Acc<OP, T> >(a);
     if (threadIdx.x == 0) out[blockIdx.x] = last ? finalize<OP, T>(a.v, count) : a.v;
 }
 
@@ -209,11 +288,22 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_wave_kernel(const T* __res
                                                                   uint64_t count, int last) {
     const uint64_t row = (uint64_t)blockIdx.x * kWaves + threadIdx.x / RT_WAVE;
     if (row >= rows) return;
+    const uint32_t lane = threadIdx.x & (RT_WAVE - 1);
+    if constexpr (Acc<OP, T>::kTrack) {
+        AccQuick<OP, T> q;
+        q.init();
+        fold_run<AccQuick<OP, T>, T>(q, src + row * R, 0, R, lane, RT_WAVE);
+        wave_reduce<AccQuick<OP, T> >(q);
+        if (__builtin_amdgcn_readfirstlane((int)q.settled())) {             // lane 0 holds the row's result: the same branch for the whole wave
+            if (lane == 0) out[row] = last ? finalize<OP, T>(q.value(), count) : q.value();
+            return;
+        }
+    }
     Acc<OP, T> a;
     a.init();
-    fold_run<OP, T>(a, src + row * R, 0, R, threadIdx.x & (RT_WAVE - 1), RT_WAVE);
-    wave_reduce<OP, T>(a);
-    if ((threadIdx.x & (RT_WAVE - 1)) == 0) out[row] = last ? finalize<OP, T>(a.v, count) : a.v;
+    fold_run<Acc<OP, T>, T>(a, src + row * R, 0, R, lane, RT_WAVE);
+    wave_reduce<Acc<OP, T> >(a);
+    if (lane == 0) out[row] = last ? finalize<OP, T>(a.v, count) : a.v;
 }
 
 // one lane per row (R < 64)
@@ -222,7 +312,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_lane_kernel(const T* __res
                                                                   uint64_t count, int last) {
     const uint64_t row = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
     if (row >= rows) return;
-    Acc<OP, T> a;
+    AccOrd<OP, T> a;                                              // one lane folds its row in order
     a.init();
     const T* p = src + row * R;
     for (uint32_t k = 0; k < R; ++k) a.push(p[k], k);
@@ -233,10 +323,13 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_lane_kernel(const T* __res
 // src viewed as (outer, R, inner).  VW = elements per lane along `inner` (16 bytes worth when rows are aligned, else 1).
 // blockIdx.x -> (o, seg, tile); lane tx covers columns (tile*64 + tx)*VW .., wave ty takes k = begin+ty, +kWaves, ...
 // out index: ((seg * outer) + o) * inner + column   (seg = 0, splits = 1 when this is the only stage)
-template <int OP, class T, int VW, int U = 4>
-__global__ __launch_bounds__(kBlock) void reduce_cols_kernel(const T* __restrict__ src, T* __restrict__ out, uint64_t R, uint64_t inner, uint64_t outer,
-                                                             uint32_t tiles, uint32_t splits, uint64_t seglen, uint64_t count, int last) {
+// One pass of the column kernel with accumulator class A; returns non-zero in a lane that wrote an unsettled result.
+template <class A, int OP, class T, int VW, int U>
+__device__ __forceinline__ int cols_pass(const T* __restrict__ src, T* __restrict__ out, uint64_t R, uint64_t inner, uint64_t outer, uint32_t tiles,
+                                         uint32_t splits, uint64_t seglen, uint64_t count, int last, T (*sv)[RT_WAVE][VW], void* sx_raw) {
     struct alignas(sizeof(T) * VW) VecW { T e[VW]; };
+    typedef typename A::extra_t X;
+    X (*sx)[RT_WAVE][VW] = reinterpret_cast<X (*)[RT_WAVE][VW]>(sx_raw);
     uint64_t b = blockIdx.x;
     const uint32_t tile = (uint32_t)(b % tiles);
     b /= tiles;
@@ -265,7 +358,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(const T* __restrict
     uint64_t end = begin + seglen;
     if (end > R) end = R;
 
-    Acc<OP, T> a[VW];
+    A a[VW];
 #pragma unroll
     for (int j = 0; j < VW; ++j) a[j].init();
     if (active) {
@@ -289,28 +382,44 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(const T* __restrict
         }
     }
     // combine the kWaves interleaved partial folds of each column through LDS
-    __shared__ T sv[kWaves][RT_WAVE][VW];
-    __shared__ uint64_t sp[Acc<OP, T>::kTrack ? kWaves : 1][Acc<OP, T>::kTrack ? RT_WAVE : 1][Acc<OP, T>::kTrack ? VW : 1];
 #pragma unroll
     for (int j = 0; j < VW; ++j) {
         sv[ty][tx][j] = a[j].v;
-        if constexpr (Acc<OP, T>::kTrack) sp[ty][tx][j] = a[j].pos;
+        if constexpr (A::kExtra) sx[ty][tx][j] = a[j].extra();
     }
     __syncthreads();
+    int unsettled = 0;
     if (ty == 0 && active) {
         T* q = out + ((uint64_t)seg * outer + o) * inner + col;
 #pragma unroll
         for (int j = 0; j < VW; ++j) {
 #pragma unroll
             for (int w = 1; w < kWaves; ++w) {
-                Acc<OP, T> x;
-                x.v = sv[w][tx][j];
-                if constexpr (Acc<OP, T>::kTrack) x.pos = sp[w][tx][j]; else x.pos = 0;
-                a[j].merge(x);
+                X e = 0;
+                if constexpr (A::kExtra) e = sx[w][tx][j];
+                a[j].merge(A::make(sv[w][tx][j], e));
             }
-            if ((uint32_t)j >= skip) q[j] = last ? finalize<OP, T>(a[j].v, count) : a[j].v;
+            if ((uint32_t)j >= skip) {
+                unsettled |= !a[j].settled();
+                q[j] = last ? finalize<OP, T>(a[j].value(), count) : a[j].value();
+            }
         }
     }
+    return unsettled;
+}
+
+template <int OP, class T, int VW, int U = 4>
+__global__ __launch_bounds__(kBlock) void reduce_cols_kernel(const T* __restrict__ src, T* __restrict__ out, uint64_t R, uint64_t inner, uint64_t outer,
+                                                             uint32_t tiles, uint32_t splits, uint64_t seglen, uint64_t count, int last) {
+    constexpr bool kTrack = Acc<OP, T>::kTrack;
+    __shared__ T sv[kWaves][RT_WAVE][VW];
+    __shared__ uint64_t sx[kTrack ? kWaves * RT_WAVE * VW : 1];
+    if constexpr (kTrack) {
+        // float max / min: the quick form first; the lanes whose column ended in an unsettled zero have written a provisional value,
+        // and the whole block folds again with positions (every output is then written again by the same lane)
+        if (!__syncthreads_or(cols_pass<AccQuick<OP, T>, OP, T, VW, U>(src, out, R, inner, outer, tiles, splits, seglen, count, last, sv, sx))) return;
+    }
+    cols_pass<Acc<OP, T>, OP, T, VW, U>(src, out, R, inner, outer, tiles, splits, seglen, count, last, sv, sx);
 }
 
 // ---- short rows: 1 <= R <= 1024 ----------------------------------------------------------------------------------------------
@@ -376,17 +485,29 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_tile_kernel(const T* __res
     if (tb + threadIdx.x < ne) put(tb + threadIdx.x, p[tb + threadIdx.x]);
     __syncthreads();
     const uint32_t g = threadIdx.x / a.T, j = threadIdx.x & (a.T - 1), groups = kBlock / a.T;
-    for (uint32_t r = g; r < nrows; r += groups) {
-        Acc<OP, T> acc;
+    // the T lanes of a group take elements j, j + T, ... of their row: interleaved positions
+    auto fold_row = [&](auto& acc, const T* row) {
         acc.init();
-        const T* row = tile + mis + r * a.pitch;                  // pitch == R in the verbatim layout
         for (uint32_t k = j; k < a.R; k += a.T) acc.push(row[k], k);
         for (uint32_t d = a.T / 2; d >= 1; d >>= 1) {
-            Acc<OP, T> o;
-            o.v = shfl_down_t<T>(acc.v, (int)d);
-            if constexpr (Acc<OP, T>::kTrack) o.pos = shfl_down_t<uint64_t>(acc.pos, (int)d); else o.pos = 0;
+            auto o = acc.shfl_down((int)d);
             if (j + d < a.T) acc.merge(o);
         }
+    };
+    for (uint32_t r = g; r < nrows; r += groups) {
+        const T* row = tile + mis + r * a.pitch;                  // pitch == R in the verbatim layout
+        if constexpr (Acc<OP, T>::kTrack) {
+            AccQuick<OP, T> q;
+            fold_row(q, row);
+            // one decision for the wave (its groups share the trip count of this loop up to the last trip, where the lanes of
+            // finished groups are off): any group's unsettled zero sends all of them through the fold with positions
+            if (!__builtin_amdgcn_ballot_w64(j == 0 && !q.settled())) {
+                if (j == 0) out[row0 + r] = finalize<OP, T>(q.value(), count);
+                continue;
+            }
+        }
+        Acc<OP, T> acc;
+        fold_row(acc, row);
         if (j == 0) out[row0 + r] = finalize<OP, T>(acc.v, count);
     }
 }
@@ -408,17 +529,16 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_pow2_kernel(const T* __res
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const uint64_t v = v0 + (uint64_t)u * kBlock;
-        Acc<OP, T> a;
+        // lane j holds elements j*N .. j*N+N-1 of its row, and with the distance doubling from 1 every merge joins a run of lanes
+        // with the run right after it: in ascending order, so the float max / min need no positions here
+        AccOrd<OP, T> a;
         a.init();
         if (v < nvec) {
 #pragma unroll
             for (uint32_t e = 0; e < N; ++e) a.push(x[u].e[e], (uint64_t)j * N + e);
         }
-        for (uint32_t d = VR / 2; d >= 1; d >>= 1) {
-            Acc<OP, T> o;
-            o.v = shfl_down_t<T>(a.v, (int)d);
-            // positions inside a row fit 32 bits here (one shuffle instead of two); "none yet" stays the largest value
-            if constexpr (Acc<OP, T>::kTrack) o.pos = (uint64_t)(uint32_t)__shfl_down((int)(uint32_t)a.pos, (int)d, RT_WAVE); else o.pos = 0;
+        for (uint32_t d = 1; d < VR; d <<= 1) {
+            AccOrd<OP, T> o = a.shfl_down((int)d);
             if (j + d < VR) a.merge(o);
         }
         if (j == 0 && v < nvec) out[v >> vr_shift] = finalize<OP, T>(a.v, count);
@@ -437,20 +557,20 @@ struct ColsNarrowArgs {
     FastDiv32 inner_div;
 };
 
-template <int OP, class T, int VW>
-__global__ __launch_bounds__(kBlock) void reduce_cols_narrow_kernel(const T* __restrict__ src, T* __restrict__ out, ColsNarrowArgs a, uint64_t count,
-                                                                    int last) {
-    constexpr bool kTrack = Acc<OP, T>::kTrack;
+// One pass of the narrow-column kernel with accumulator class A; returns non-zero in a lane that wrote an unsettled result.
+template <class A, int OP, class T, int VW>
+__device__ __forceinline__ int cols_narrow_pass(const T* __restrict__ src, T* __restrict__ out, const ColsNarrowArgs& a, uint64_t count, int last, T* sv,
+                                                void* sx_raw) {
     struct alignas(sizeof(T) * VW) VecW { T e[VW]; };
-    __shared__ T sv[kBlock * VW];
-    __shared__ uint64_t sp[kTrack ? kBlock * VW : 1];
+    typedef typename A::extra_t X;
+    X* sx = reinterpret_cast<X*>(sx_raw);
     const uint64_t o = blockIdx.x / a.splits;
     const uint32_t seg = (uint32_t)(blockIdx.x - o * a.splits);
     const uint32_t t = threadIdx.x;
     const uint32_t S = a.Tn * VW;
     const uint64_t slab = a.R * a.inner;                       // elements of one outer index
     const T* base = src + o * slab;
-    Acc<OP, T> acc[VW];
+    A acc[VW];
     uint32_t krow[VW];
 #pragma unroll
     for (int j = 0; j < VW; ++j) { acc[j].init(); krow[j] = fd_div(t * VW + j, a.inner_div); }
@@ -474,7 +594,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_narrow_kernel(const T* __r
             }
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const uint64_t k0 = (tl + u) * a.L;
+                const uint32_t k0 = (uint32_t)((tl + u - tile_begin) * a.L);       // row inside the segment: below 2^32 (checked on the host)
                 if (full[u]) {
 #pragma unroll
                     for (int j = 0; j < VW; ++j) acc[j].push(x[u].e[j], k0 + krow[j]);
@@ -490,28 +610,42 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_narrow_kernel(const T* __r
 #pragma unroll
     for (int j = 0; j < VW; ++j) {
         sv[t * VW + j] = acc[j].v;
-        if constexpr (kTrack) sp[t * VW + j] = acc[j].pos;
+        if constexpr (A::kExtra) sx[t * VW + j] = acc[j].extra();
     }
     __syncthreads();
     // column c is held by the L values c, c + inner, ...: G lanes per column (a power of two, inner * G <= kBlock) share them
     const uint32_t c = t / a.G, j = t & (a.G - 1);
-    Acc<OP, T> r;
+    A r;
     r.init();
     if (c < a.inner) {
         for (uint32_t q = j; q < a.L; q += a.G) {
-            Acc<OP, T> x;
-            x.v = sv[c + q * a.inner];
-            x.pos = kTrack ? sp[c + q * a.inner] : 0;
-            r.merge(x);
+            X e = 0;
+            if constexpr (A::kExtra) e = sx[c + q * a.inner];
+            r.merge(A::make(sv[c + q * a.inner], e));
         }
     }
     for (uint32_t d = a.G / 2; d >= 1; d >>= 1) {
-        Acc<OP, T> x;
-        x.v = shfl_down_t<T>(r.v, (int)d);
-        if constexpr (kTrack) x.pos = shfl_down_t<uint64_t>(r.pos, (int)d); else x.pos = 0;
+        A x = r.shfl_down((int)d);
         if (j + d < a.G) r.merge(x);
     }
-    if (c < a.inner && j == 0) out[((uint64_t)seg * a.outer + o) * a.inner + c] = last ? finalize<OP, T>(r.v, count) : r.v;
+    if (c < a.inner && j == 0) {
+        out[((uint64_t)seg * a.outer + o) * a.inner + c] = last ? finalize<OP, T>(r.value(), count) : r.value();
+        return !r.settled();
+    }
+    return 0;
+}
+
+template <int OP, class T, int VW>
+__global__ __launch_bounds__(kBlock) void reduce_cols_narrow_kernel(const T* __restrict__ src, T* __restrict__ out, ColsNarrowArgs a, uint64_t count,
+                                                                    int last) {
+    constexpr bool kTrack = Acc<OP, T>::kTrack;
+    __shared__ T sv[kBlock * VW];
+    __shared__ uint32_t sx[kTrack ? kBlock * VW : 1];
+    if constexpr (kTrack) {
+        // float max / min: the quick form first, the fold with positions only when a column's zero result met a -0.0
+        if (!__syncthreads_or(cols_narrow_pass<AccQuick<OP, T>, OP, T, VW>(src, out, a, count, last, sv, sx))) return;
+    }
+    cols_narrow_pass<AccT<OP, T, kTrack, uint32_t>, OP, T, VW>(src, out, a, count, last, sv, sx);
 }
 
 // ---- short reduced axis: R <= 32, any inner -----------------------------------------------------------------------------------
@@ -526,7 +660,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_short_kernel(const T* __re
     const uint32_t o = fd_div((uint32_t)idx, iv_div);           // nvec_out < 2^32 on this path
     const uint32_t iv = (uint32_t)idx - o * inner_vecs;
     const T* p = src + (uint64_t)o * R * inner + (uint64_t)iv * VW;
-    Acc<OP, T> acc[VW];
+    AccOrd<OP, T> acc[VW];                                      // each lane folds its columns in order
 #pragma unroll
     for (int j = 0; j < VW; ++j) acc[j].init();
     constexpr int U = 4;
@@ -565,7 +699,7 @@ __global__ __launch_bounds__(kBlock) void reduce_merge_wave_kernel(const T* __re
     Acc<OP, T> a;
     a.init();
     for (uint32_t k = lane; k < splits; k += RT_WAVE) a.push(part[(uint64_t)k * nout + o], k);       // partials arrive in segment order
-    wave_reduce<OP, T>(a);
+    wave_reduce<Acc<OP, T> >(a);
     if (lane == 0) out[o] = finalize<OP, T>(a.v, count);
 }
 template <int OP, class T>
@@ -586,8 +720,7 @@ int32_t rows_stage(rt_ctx* ctx, const T* src, T* out, uint64_t rows, uint64_t R,
         const uint64_t vr = R / N;
         // (small inputs stay with the staged kernel, where few rows mean one lane per row: a sum in index order, bit for bit the
         // sequential result)
-        // float max / min carry a position through every shuffle step: with 8-byte values that only pays up to 16 lanes per row
-        const uint64_t vr_max = (Acc<OP, T>::kTrack && sizeof(T) == 8) ? 16 : 64;
+        const uint64_t vr_max = 64;
         if (count == R && R % N == 0 && vr >= 1 && vr <= vr_max && (vr & (vr - 1)) == 0 && rows * vr >= 4096) {
             const uint64_t nvec = rows * vr;
             const uint64_t blocks = (nvec + (uint64_t)kBlock * 4 - 1) / ((uint64_t)kBlock * 4);
@@ -626,7 +759,9 @@ int32_t rows_stage(rt_ctx* ctx, const T* src, T* out, uint64_t rows, uint64_t R,
         return RT_OK;
     }
     const uint64_t want = (uint64_t)ctx->num_cus * 8;
-    if (R < 4096 && rows >= want / 2) {
+    // a wave per row up to 16 KiB, a block per row from there on (1 GiB, sum: rows of 8 KiB 0.86 of peak by waves / 0.56 by blocks, rows of
+    // 16 KiB 0.85 / 0.91, of 32 KiB 0.81 / 0.90; the same for 1-, 2-, 4- and 8-byte elements)
+    if (R * sizeof(T) < 16384 && rows >= want / 2) {
         uint64_t blocks = (rows + kWaves - 1) / kWaves;
         if (blocks >= (1ull << 31)) return rt_fail(RT_E_INVALID, "reduce: too many rows for one launch");
         hipLaunchKernelGGL((reduce_rows_wave_kernel<OP, T>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, out, rows, R, count, 1);
@@ -824,7 +959,7 @@ int32_t reduce_typed(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t
             return RT_OK;
         }
     }
-    if (inner < 128 && R >= 64 && outer < (1ull << 20)) return cols_narrow<OP, T>(ctx, src, out, outer, R, inner);
+    if (inner < 128 && R >= 64 && R < (1ull << 32) && outer < (1ull << 20)) return cols_narrow<OP, T>(ctx, src, out, outer, R, inner);
     // one 16-byte vector of columns per lane whatever the alignment of the rows (1 GiB f32 sum over axis 0 with 32767 columns:
     // 0.307 ms with one column per lane, 0.17 ms with unaligned vectors)
     const bool vec = inner >= (uint64_t)N;

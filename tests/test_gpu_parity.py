@@ -1530,6 +1530,47 @@ def test_reduction_shapes_short_rows_narrow_columns_short_axis(hip, dtype):
             _check_reduce(hip, dtype, outer, R, inner, rng, offset=offset)
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f64"])
+def test_float_max_min_keep_the_first_zero_in_every_kernel_shape(hip, dtype):
+    """max over values <= 0 and min over values >= 0 whose zeros come in both signs, in either order, or in one sign only: the
+    result is the first zero of the fiber in index order, as in the sequential loop, whichever kernel folds it (a block, a wave
+    or a group of lanes per row, rows of whole vectors, split rows and the flat form; lanes along wide, narrow and regrouped
+    columns, a lane per output for a short axis).  NaN never wins."""
+    code = cpu.DTYPE_BY_NAME[dtype]
+    npd = np.dtype(cpu.NP_DTYPE[code]).type
+    rng = np.random.default_rng(zlib.crc32(b"zero-sign" + dtype.encode()))
+    shapes = [(4, 100000, 1), (3000, 5000, 1), (1, 1 << 21, 1), (5000, 600, 1), (3000, 2000, 1), (20000, 100, 1), (20000, 10, 1), (40000, 64, 1),
+              (8192, 256, 1), (70, 33, 1), (1, 5000, 512), (8, 300, 1024), (1, 4096, 4096), (2, 3000, 1001), (1, 100000, 3), (4, 5000, 100),
+              (5000, 16, 64), (100, 8, 1000), (1, 70001, 17), (300, 200, 8)]
+    for outer, R, inner in shapes:
+        n = outer * R * inner
+        mag = np.abs(rng.normal(size=n)).astype(npd) + npd(0.5)
+        # per fiber: 0 = no zero, 1 = +0.0 only, 2 = -0.0 only, 3 = both signs; zeros at random places along the fiber
+        kind = rng.integers(0, 4, size=(outer, 1, inner))
+        u = rng.random(size=(outer, R, inner))
+        zero = (u < min(0.5, 3.0 / R)) & (kind > 0)
+        neg = np.where(kind == 3, rng.random(size=(outer, R, inner)) < 0.5, kind == 2)
+        zeros = np.where(neg, npd(-0.0), npd(0.0)).astype(npd)
+        nan = rng.random(size=(outer, R, inner)) < 0.01
+        for op, sign in (("max", -1), ("min", 1)):
+            x = np.where(zero, zeros, (sign * mag).reshape(outer, R, inner)).astype(npd)
+            x[nan & ~zero] = np.nan
+            x = np.ascontiguousarray(x).reshape(-1)
+            m = MetaTensor([outer, R, inner], [R * inner, inner, 1], 0)
+            want = cpu.reduce_nd(code, op, x, m, 1, honour_offset=True)
+            src = hip.alloc_from_slice(code, x)
+            dst = hip.alloc(code, outer * inner)
+            hip.apply_reduce_contiguous_nd((src, (0, [outer, R, inner], [R * inner, inner, 1])), dst, 1, op)
+            got = hip.dump(dst)
+            assert got.tobytes() == want.tobytes(), (dtype, op, outer, R, inner, int(np.flatnonzero(got.view(np.uint8) != want.view(np.uint8))[0]))
+            if outer * inner >= 64:
+                assert np.signbit(want[want == 0]).any() and (~np.signbit(want[want == 0])).any(), "the case is meant to hold zero results of both signs"
+            if inner == 1 and outer == 1:
+                one = hip.alloc(code, 1)
+                hip.apply_reduce_contiguous_flat(src, one, 0, n, op)
+                assert hip.dump(one).tobytes() == want.tobytes(), (dtype, op, "flat", n)
+
+
 def _check_stat(hip, dtype, outer, R, inner, rng, offset=0):
     """Variance / stdev / logsumexp / norms along the middle axis of (outer, R, inner).  The GPU folds in tree order, the oracle in
     index order, so the comparison is by tolerance: within 1e-5 (f32) / 1e-12 (f64), relative, of the oracle run in float64 on the
