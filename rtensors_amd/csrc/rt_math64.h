@@ -280,3 +280,29 @@ RT_M64 double rt_tan_f64(double x) {
     const double q = rt_quot_f64(odd ? -c : s, odd ? s : c);
     return x == 0.0 ? x : q;
 }
+
+// exp(x) for x <= 0 (the terms of a logsumexp, whose arguments are distances below the running maximum): k = nearest integer to
+// x / ln 2, r = x - k ln 2 by two fused multiply-adds with ln 2 as the sum of two doubles (|r| <= 0.347), then
+// exp(r) = 1 + r + r^2 P(r) with P of degree 9, the Chebyshev interpolant of (exp(r) - 1 - r) / r^2 on |r| <= 0.3466 (the polynomial is
+// within 0.15 ulp of exp), scaled by 2^k in one instruction that also forms denormals and the final 0.  No overflow branch, no table:
+// 19 operations where the library's full-range routine takes 38; within 1.5 ulp (1.0 measured against 80-bit arithmetic by
+// tests/test_math64_host.py).  exp(-inf) = 0.  The lower clamp is a maximum, so a NaN argument gives 0, not NaN: the caller looks
+// after NaN itself (the logsumexp state notes NaN elements apart).  Positive arguments are not for this routine.
+RT_M64 double rt_exp_nonpos_f64(double x) {
+    const double xc = __builtin_fmax(x, -750.0);                                // 2^-1082 is already 0
+    const double fn = __builtin_rint(xc * 0x1.71547652b82fep+0);                // 1 / ln 2
+    double r = __builtin_fma(-fn, 0x1.62e42fefa39efp-1, xc);                    // ln 2 = hi + lo + 5.7e-34
+    r = __builtin_fma(-fn, 0x1.abc9e3b39803fp-56, r);
+    double p = 0x1.af38a71a18cb9p-26;
+    p = __builtin_fma(p, r, 0x1.2891834686c7ep-22);
+    p = __builtin_fma(p, r, 0x1.71de0daf7a6ccp-19);
+    p = __builtin_fma(p, r, 0x1.a019b90eefe8ep-16);
+    p = __builtin_fma(p, r, 0x1.a01a01a7c3d59p-13);
+    p = __builtin_fma(p, r, 0x1.6c16c1788b646p-10);
+    p = __builtin_fma(p, r, 0x1.11111111109b4p-7);
+    p = __builtin_fma(p, r, 0x1.5555555553d64p-5);
+    p = __builtin_fma(p, r, 0x1.5555555555556p-3);
+    p = __builtin_fma(p, r, 0x1.0000000000001p-1);
+    const double e = 1.0 + __builtin_fma(r * r, p, r);
+    return __builtin_ldexp(e, (int)fn);
+}

@@ -15,6 +15,7 @@
 //   cols  (inner  > 1): lanes along `inner` with 16-byte loads; a narrow `inner` is streamed as one contiguous run instead
 //   Partial states of split reductions go to the context's scratch buffer and a merge kernel folds them (two launches, no atomics).
 #include "rt_common.h"
+#include "rt_math64.h"
 
 #include <limits>
 #include <type_traits>
@@ -96,13 +97,19 @@ template <class T> struct LseState {
     // exp(x - top), with x == top giving 1 also when both are infinite.  The argument is never positive, so for f32 the hardware
     // exponential (2^(x log2 e), a few ulp for the arguments near 0 that carry the sum) stays inside the 1e-5 of the result; the
     // library routine costs about four times the instructions and made short-row logsumexp compute-bound.
+    // f64: the exponential written for non-positive arguments (rt_math64.h, within 1.5 ulp, half the library routine's instructions),
+    // computed for every lane in straight-line code.  It has no case for x == top: a finite x == top gives exp(0) = 1 exactly, and
+    // under an infinite top the sum does not reach the result (result() returns m = +-inf for s = 0 and for s > 0 alike).  It turns
+    // a NaN argument into 0, so NaN elements are noted apart and make the sum NaN, which every later step keeps.
     static __device__ __forceinline__ T term(T x, T top) {
         if constexpr (std::is_same<T, float>::value) return x == top ? 1.0f : __expf(x - top);
-        else return x == top ? (T)1 : m_exp(x - top);
+        else return rt_exp_nonpos_f64(x - top);
     }
+    static constexpr bool kNoteNan = !std::is_same<T, float>::value;
     __device__ __forceinline__ void push(T x, uint64_t) {
         const T top = m_max(m, x);
         s = s * term(m, top) + term(x, top);
+        if constexpr (kNoteNan) s = x != x ? x : s;
         m = top;
     }
     template <int K> __device__ __forceinline__ void push_block(const T* x, uint64_t, uint64_t) {
@@ -110,8 +117,13 @@ template <class T> struct LseState {
 #pragma unroll
         for (int i = 0; i < K; ++i) top = m_max(top, x[i]);
         T acc = s * term(m, top);
+        bool bad = false;
 #pragma unroll
-        for (int i = 0; i < K; ++i) acc = acc + term(x[i], top);
+        for (int i = 0; i < K; ++i) {
+            acc = acc + term(x[i], top);
+            if constexpr (kNoteNan) bad |= x[i] != x[i];
+        }
+        if constexpr (kNoteNan) acc = bad ? std::numeric_limits<T>::quiet_NaN() : acc;
         s = acc;
         m = top;
     }
@@ -127,7 +139,12 @@ template <class T> struct LseState {
         T top = row[0];
         for (uint32_t k = 1; k < R; ++k) top = m_max(top, row[k]);
         T acc = (T)0;
-        for (uint32_t k = 0; k < R; ++k) acc = acc + term(row[k], top);
+        bool bad = false;
+        for (uint32_t k = 0; k < R; ++k) {
+            acc = acc + term(row[k], top);
+            if constexpr (kNoteNan) bad |= row[k] != row[k];
+        }
+        if constexpr (kNoteNan) acc = bad ? std::numeric_limits<T>::quiet_NaN() : acc;
         m = top;
         s = acc;
     }
@@ -198,6 +215,76 @@ template <class S> __device__ __forceinline__ void group_reduce(S& a, uint32_t w
         S o = shfl_down_state(a, (int)d);
         if (lane_in_group + d < width) a.merge(o);
     }
+}
+
+// ---- sums and maxima over a group of lanes without the LDS crossbar -----------------------------------------------------------------
+// A group is an aligned run of `width` lanes, width a power of two <= 64, all lanes of the wave active.  Inside a row of 16 lanes the
+// data-parallel-primitive lane patterns move the operand as part of an ordinary vector instruction: swap neighbours, swap pairs (after
+// which the four lanes of a quad agree), mirror the halves of 8, mirror the row.  Across rows the four row results are read into scalar
+// registers.  Every lane ends with the group's result.  (The permute instruction these replace goes through the LDS unit, about a
+// hundred cycles a step, six steps per value: variance over rows of 512 f32 spent a sixth of its time there.)
+template <int CTRL> __device__ __forceinline__ float dpp_get(float v) {
+    const int w = __builtin_bit_cast(int, v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(w, w, CTRL, 0xf, 0xf, false));
+}
+template <int CTRL> __device__ __forceinline__ double dpp_get(double v) {
+    const uint64_t w = __builtin_bit_cast(uint64_t, v);
+    const int lo = (int)(uint32_t)w, hi = (int)(uint32_t)(w >> 32);
+    const uint32_t l2 = (uint32_t)__builtin_amdgcn_update_dpp(lo, lo, CTRL, 0xf, 0xf, false);
+    const uint32_t h2 = (uint32_t)__builtin_amdgcn_update_dpp(hi, hi, CTRL, 0xf, 0xf, false);
+    return __builtin_bit_cast(double, (uint64_t)l2 | ((uint64_t)h2 << 32));
+}
+__device__ __forceinline__ float lane_get(float v, int lane) { return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane)); }
+__device__ __forceinline__ double lane_get(double v, int lane) {
+    const uint64_t w = __builtin_bit_cast(uint64_t, v);
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)w, lane), hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(w >> 32), lane);
+    return __builtin_bit_cast(double, (uint64_t)lo | ((uint64_t)hi << 32));
+}
+struct OpSum { template <class T> static __device__ __forceinline__ T f(T a, T b) { return a + b; } };
+struct OpMax { template <class T> static __device__ __forceinline__ T f(T a, T b) { return m_max(a, b); } };
+template <class Op, class T> __device__ __forceinline__ T group_all(T v, uint32_t width) {
+    if (width >= 2) v = Op::f(v, dpp_get<0xB1>(v));              // quad_perm [1, 0, 3, 2]
+    if (width >= 4) v = Op::f(v, dpp_get<0x4E>(v));              // quad_perm [2, 3, 0, 1]
+    if (width >= 8) v = Op::f(v, dpp_get<0x141>(v));             // row_half_mirror
+    if (width >= 16) v = Op::f(v, dpp_get<0x140>(v));            // row_mirror
+    if (width >= 32) {
+        const T lo = Op::f(lane_get(v, 0), lane_get(v, 16)), hi = Op::f(lane_get(v, 32), lane_get(v, 48));
+        if (width >= 64) v = Op::f(lo, hi);
+        else v = (threadIdx.x & 32) ? hi : lo;
+    }
+    return v;
+}
+
+// Norms: one sum.
+template <class T, bool SQ> __device__ __forceinline__ void group_reduce(NormState<T, SQ>& a, uint32_t width, uint32_t) {
+    if (width == 1) return;
+    a.s = group_all<OpSum>(a.s, width);
+}
+// The two states whose merge is expensive (two exponentials; a reciprocal), in phases that need one of those per lane instead of one
+// or two per step.  logsumexp: the group's maximum, every lane's sum rescaled to it once, the sums added.
+template <class T> __device__ __forceinline__ void group_reduce(LseState<T>& a, uint32_t width, uint32_t) {
+    if (width == 1) return;
+    const T top = group_all<OpMax>(a.m, width);
+    a.s = group_all<OpSum>(a.s * LseState<T>::term(a.m, top), width);       // an empty lane (m = -inf, s = 0) contributes 0
+    a.m = top;
+}
+// moments: with d_i = mean_i - c the distances from a common reference (the largest of the lanes' means), the group's mean is c + D,
+// D = sum(n_i d_i) / sum(n_i), and its m2 = sum(m2_i + n_i (d_i - D)^2): sums and one reciprocal.  The distances are differences
+// of nearby values, so nothing is lost to the size of the mean itself.
+template <class T> __device__ __forceinline__ void group_reduce(MomentState<T>& a, uint32_t width, uint32_t) {
+    if (width == 1) return;
+    const T ninf = -std::numeric_limits<T>::infinity();
+    T c = group_all<OpMax>(a.n > 0.0 ? a.mean : ninf, width);
+    c = c == ninf ? (T)0 : c;                                       // no lane holds anything (or nothing but NaN)
+    const T d = a.n > 0.0 ? a.mean - c : (T)0;
+    const T cnt = (T)a.n;                                           // a lane's own count is small enough to be exact in T
+    const double n = group_all<OpSum>(a.n, width);
+    const T w = group_all<OpSum>(cnt * d, width);
+    const T D = n > 0.0 ? w * m_recip((T)n) : (T)0;
+    const T e = d - D;
+    a.m2 = group_all<OpSum>(a.m2 + cnt * (e * e), width);
+    a.mean = c + D;
+    a.n = n;
 }
 
 template <class S> __device__ __forceinline__ void block_reduce(S& a) {
@@ -274,17 +361,18 @@ __global__ __launch_bounds__(kBlock) void st_rows_block_kernel(const T* __restri
     }
 }
 
-// one wave per row
-template <class S, class T>
+// G lanes per row, G = 16, 32 or 64 (a quarter of a wave, half a wave, a wave): the fold over the lanes of a row costs the same per row
+// whatever its length, so rows of 2 ... 4 KiB get 16 lanes (eight vectors per lane) and rows of 4 ... 8 KiB 32
+template <class S, class T, int G>
 __global__ __launch_bounds__(kBlock) void st_rows_wave_kernel(const T* __restrict__ src, typename S::Out* __restrict__ out, uint64_t rows, uint64_t R, int flags) {
-    const uint64_t row = (uint64_t)blockIdx.x * kWaves + threadIdx.x / RT_WAVE;
-    if (row >= rows) return;
-    const uint32_t lane = threadIdx.x & (RT_WAVE - 1);
+    const uint64_t row = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) / G;
+    const uint32_t lane = threadIdx.x & (G - 1);
     S a;
     a.init();
-    fold_run<S, T>(a, src + row * R, 0, R, lane, RT_WAVE);
-    group_reduce(a, RT_WAVE, lane);
-    if (lane == 0) out[row] = a.result(flags);
+    // (a group past the last row folds nothing: the lanes of a wave stay together for the exchange below)
+    if (row < rows) fold_run<S, T>(a, src + row * R, 0, R, lane, G);
+    group_reduce(a, G, lane);
+    if (lane == 0 && row < rows) out[row] = a.result(flags);
 }
 
 // short rows (1 <= R <= 1024): the block's rows are one contiguous run, copied into LDS with coalesced 16-byte loads (row pitch R | 1
@@ -349,6 +437,9 @@ __global__ __launch_bounds__(kBlock) void st_rows_tile_kernel(const T* __restric
     if (tb + threadIdx.x < ne) put(tb + threadIdx.x, p[tb + threadIdx.x]);
     __syncthreads();
     const uint32_t g = threadIdx.x / a.G, j = threadIdx.x & (a.G - 1), groups = kBlock / a.G;
+    // f64 logsumexp reads its rows twice (see below): there the exponentials set the time (rows of 100: 0.49 -> 0.56 of peak); for f32,
+    // whose exponential is one instruction, the second round of LDS reads costs more than the rescaling it saves (rows of 256: 0.70 -> 0.67)
+    constexpr bool kTwoPass = std::is_same<S, LseState<T>>::value && sizeof(T) == 8;
     for (uint32_t r0 = 0; r0 < nrows; r0 += groups) {              // every lane runs every trip: the shuffles below need the whole wave
         const uint32_t r = r0 + g;
         S acc;
@@ -359,15 +450,58 @@ __global__ __launch_bounds__(kBlock) void st_rows_tile_kernel(const T* __restric
             if constexpr (std::is_same<S, LseState<T>>::value) {
                 if (a.G == 1) { acc.fold_row(row, a.R); k = a.R; }
             }
-            for (; k + 3 * a.G < a.R; k += 4 * a.G) {
-                T x[4];
+            if constexpr (!kTwoPass) {
+                for (; k + 3 * a.G < a.R; k += 4 * a.G) {
+                    T x[4];
 #pragma unroll
-                for (int u = 0; u < 4; ++u) x[u] = row[k + u * a.G];
-                acc.template push_block<4>(x, k, a.G);
+                    for (int u = 0; u < 4; ++u) x[u] = row[k + u * a.G];
+                    acc.template push_block<4>(x, k, a.G);
+                }
+                for (; k < a.R; k += a.G) acc.push(row[k], k);
             }
-            for (; k < a.R; k += a.G) acc.push(row[k], k);
         }
-        group_reduce(acc, a.G, j);
+        if constexpr (kTwoPass) {
+            // the row lies in LDS: its maximum first (the lanes' maxima, then the group's by a butterfly), then one exponential per
+            // element and no rescaling of running sums (the running form pays one more per four elements and one per lane at the end)
+            if (a.G > 1) {
+                const T* row = tile + mis + r * a.pitch;
+                T top = -std::numeric_limits<T>::infinity();
+                if (r < nrows) {
+                    uint32_t k = j;
+                    for (; k + 3 * a.G < a.R; k += 4 * a.G) {     // four LDS reads in flight
+                        T x[4];
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) x[u] = row[k + u * a.G];
+                        top = m_max(m_max(top, x[0]), m_max(x[1], m_max(x[2], x[3])));
+                    }
+                    for (; k < a.R; k += a.G) top = m_max(top, row[k]);
+                }
+                for (uint32_t d = a.G / 2; d >= 1; d >>= 1) top = m_max(top, __shfl_xor(top, (int)d, RT_WAVE));
+                T sum = (T)0;
+                bool bad = false;
+                if (r < nrows) {
+                    uint32_t k = j;
+                    for (; k + 3 * a.G < a.R; k += 4 * a.G) {
+                        T x[4];
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) x[u] = row[k + u * a.G];
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) { sum = sum + S::term(x[u], top); bad |= x[u] != x[u]; }
+                    }
+                    for (; k < a.R; k += a.G) {
+                        const T x = row[k];
+                        sum = sum + S::term(x, top);
+                        bad |= x != x;
+                    }
+                }
+                if (S::kNoteNan && bad) sum = std::numeric_limits<T>::quiet_NaN();
+                for (uint32_t d = a.G / 2; d >= 1; d >>= 1) sum = sum + __shfl_xor(sum, (int)d, RT_WAVE);
+                acc.m = top;
+                acc.s = sum;
+            }
+        } else {
+            group_reduce(acc, a.G, j);
+        }
         if (j == 0 && r < nrows) out[row0 + r] = acc.result(flags);
     }
 }
@@ -390,8 +524,31 @@ __global__ __launch_bounds__(kBlock) void st_rows_pow2_kernel(const T* __restric
         const uint64_t v = v0 + (uint64_t)u * kBlock;
         S a;
         a.init();
-        if (v < nvec) a.template push_block<N>(x[u].e, (uint64_t)j * N, 1);
-        group_reduce(a, VR, j);
+        if constexpr (std::is_same<S, LseState<T>>::value) {
+            // the row's maximum before any exponential: N of them per lane and no rescaling
+            T top = -std::numeric_limits<T>::infinity();
+            if (v < nvec) {
+#pragma unroll
+                for (uint32_t e = 0; e < N; ++e) top = m_max(top, x[u].e[e]);
+            }
+            for (uint32_t d = VR / 2; d >= 1; d >>= 1) top = m_max(top, __shfl_xor(top, (int)d, RT_WAVE));
+            T sum = (T)0;
+            bool bad = false;
+            if (v < nvec) {
+#pragma unroll
+                for (uint32_t e = 0; e < N; ++e) {
+                    sum = sum + S::term(x[u].e[e], top);
+                    bad |= x[u].e[e] != x[u].e[e];
+                }
+            }
+            if (S::kNoteNan && bad) sum = std::numeric_limits<T>::quiet_NaN();
+            for (uint32_t d = VR / 2; d >= 1; d >>= 1) sum = sum + __shfl_xor(sum, (int)d, RT_WAVE);
+            a.m = top;
+            a.s = sum;
+        } else {
+            if (v < nvec) a.template push_block<N>(x[u].e, (uint64_t)j * N, 1);
+            group_reduce(a, VR, j);
+        }
         if (j == 0 && v < nvec) out[v >> vr_shift] = a.result(flags);
     }
 }
@@ -667,10 +824,18 @@ int32_t rows_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t rows
         return RT_OK;
     }
     const uint64_t want = (uint64_t)ctx->num_cus * 8;
-    if (R < 4096 && rows >= want / 2) {
-        const uint64_t blocks = (rows + kWaves - 1) / kWaves;
+    if (R * sizeof(T) < 16384 && rows >= want / 2) {             // a block per row from 16 KiB on, as for the plain reductions
+        const uint64_t row_bytes = R * sizeof(T);
+        // 1 GiB, of peak, with 64 / 32 / 16 lanes per row -- f64 variance, rows of 2 KiB: 0.60 / - / 0.85, 3 KiB: 0.73 / - / 0.86; f32 variance,
+        // rows of 2 KiB: 0.78 / - / 0.85, of 4000 B: 0.77 / - / 0.73, of 4 KiB: 0.87 / 0.85 / -; f64 logsumexp, whose exponentials make every
+        // saved step count, rows of 2 KiB: 0.44 / - / 0.75, 4000 B: 0.46 / - / 0.68, 4 KiB: 0.63 / 0.73 / -
+        constexpr bool kDear = std::is_same<S, LseState<double>>::value;
+        const uint32_t g = kDear ? (row_bytes < 4096 ? 16 : (row_bytes < 8192 ? 32 : 64)) : (row_bytes <= 3072 ? 16 : 64);
+        const uint64_t blocks = (rows * g + kBlock - 1) / kBlock;
         if (blocks >= (1ull << 31)) return too_many();
-        hipLaunchKernelGGL((st_rows_wave_kernel<S, T>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, out, rows, R, flags);
+        if (g == 16) hipLaunchKernelGGL((st_rows_wave_kernel<S, T, 16>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, out, rows, R, flags);
+        else if (g == 32) hipLaunchKernelGGL((st_rows_wave_kernel<S, T, 32>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, out, rows, R, flags);
+        else hipLaunchKernelGGL((st_rows_wave_kernel<S, T, 64>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, out, rows, R, flags);
         RT_HIP(hipGetLastError());
         return RT_OK;
     }

@@ -36,3 +36,6 @@ extern "C" void sincos_kernel_many(size_t n, const double* x, double* s, double*
 extern "C" void tan_many(size_t n, const double* x, double* y) {
     for (size_t i = 0; i < n; ++i) y[i] = rt_tan_f64(x[i]);
 }
+extern "C" void exp_nonpos_many(size_t n, const double* x, double* y) {
+    for (size_t i = 0; i < n; ++i) y[i] = rt_exp_nonpos_f64(x[i]);
+}

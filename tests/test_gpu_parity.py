@@ -1683,6 +1683,53 @@ def test_argmax_argmin_shapes(hip, dtype):
         _check_arg(hip, dtype, 30000, R, 1, rng, offset=16)
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f64"])
+def test_logsumexp_special_values_in_every_kernel_shape(hip, dtype):
+    """Fibers that hold NaN, +inf, -inf, nothing but -inf, or values 800 apart (terms that underflow), through every work shape: a NaN
+    anywhere gives NaN, else a +inf gives +inf, a fiber of -inf gives -inf, and the rest agree with the float64 formula."""
+    code = cpu.DTYPE_BY_NAME[dtype]
+    npd = np.dtype(cpu.NP_DTYPE[code]).type
+    rng = np.random.default_rng(zlib.crc32(b"lse-special" + dtype.encode()))
+    shapes = [(4, 100000, 1), (3000, 5000, 1), (1, 1 << 20, 1), (5000, 600, 1), (20000, 100, 1), (20000, 10, 1), (40000, 64, 1), (8192, 256, 1),
+              (40000, 4, 1), (70, 33, 1), (1, 5000, 512), (8, 300, 1024), (1, 4096, 2048), (1, 100000, 3), (4, 5000, 100), (5000, 16, 64), (300, 200, 8)]
+    for outer, R, inner in shapes:
+        x = (rng.normal(size=(outer, R, inner)) * 3).astype(npd)
+        x[rng.random(size=x.shape) < 0.02] -= npd(800.0)
+        kind = rng.integers(0, 6, size=(outer, 1, inner))          # 0, 1: plain; 2: NaN; 3: +inf; 4: -inf among the values; 5: nothing but -inf
+        hit = rng.random(size=x.shape) < min(0.5, 2.0 / R)
+        hit[:, :1, :] |= rng.random(size=(outer, 1, inner)) < 0.5   # often in the first element, where a state starts
+        hit[:, -1:, :] |= rng.random(size=(outer, 1, inner)) < 0.5
+        x = np.where(hit & (kind == 2), npd(np.nan), x)
+        x = np.where(hit & (kind == 3), npd(np.inf), x)
+        x = np.where(hit & (kind == 4), npd(-np.inf), x)
+        x = np.where(np.broadcast_to(kind == 5, x.shape), npd(-np.inf), x).astype(npd)
+        x64 = x.astype(np.float64)
+        with np.errstate(all="ignore"):
+            top = np.nanmax(np.where(np.isnan(x64), -np.inf, x64), axis=1, keepdims=True)
+            safe = np.where(np.isfinite(top), top, 0.0)
+            want = (safe + np.log(np.exp(x64 - safe).sum(axis=1, keepdims=True))).reshape(-1)
+        has_nan = np.isnan(x64).any(axis=1).reshape(-1)
+        has_pinf = (x64 == np.inf).any(axis=1).reshape(-1)
+        all_ninf = (x64 == -np.inf).all(axis=1).reshape(-1)
+        src = hip.alloc_from_slice(code, np.ascontiguousarray(x).reshape(-1))
+        dst = hip.alloc(code, outer * inner)
+        hip.apply_reduce_contiguous_nd((src, (0, [outer, R, inner], [R * inner, inner, 1])), dst, 1, "logsumexp")
+        got = hip.dump(dst).astype(np.float64)
+        case = (dtype, outer, R, inner)
+        assert (np.isnan(got) == has_nan).all(), (case, "NaN", int(np.flatnonzero(np.isnan(got) != has_nan)[0]))
+        assert (got[has_pinf & ~has_nan] == np.inf).all(), (case, "+inf")
+        assert (got[all_ninf] == -np.inf).all(), (case, "-inf")
+        plain = ~has_nan & ~has_pinf & ~all_ninf
+        assert np.isfinite(got[plain]).all(), case
+        tol = (1e-5 if dtype == "f32" else 1e-12) * np.maximum(np.abs(want[plain]), 1.0)
+        assert (np.abs(got[plain] - want[plain]) <= tol).all(), (case, float(np.abs(got[plain] - want[plain]).max()))
+        if inner == 1 and outer == 1:
+            one = hip.alloc(code, 1)
+            hip.apply_reduce_contiguous_flat(src, one, 0, R, "logsumexp")
+            g1 = float(hip.dump(one)[0])
+            assert (np.isnan(g1) and has_nan[0]) or g1 == got[0] or abs(g1 - want[0]) <= 1e-5 * max(abs(want[0]), 1.0), (case, "flat", g1)
+
+
 def test_statistic_reductions_known_answers_and_edges(hip):
     """The reference's Cuda known answers through the C ABI, the flat entry points, and the edge cases the oracle tests pin."""
     import json

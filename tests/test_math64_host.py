@@ -1,5 +1,5 @@
 """The hand-written f64 routines of the device code (rtensors_amd/csrc/rt_math64.h: logarithm, arcsine / arccosine, sine / cosine /
-tangent and the reciprocal, quotient and square-root helpers under them), built for the host with g++ and measured against numpy's
+tangent, the exponential of non-positive arguments, and the reciprocal, quotient and square-root helpers under them), built for the host with g++ and measured against numpy's
 80-bit long double functions: error in units of the last place over the whole range each routine is used on, and the special values of
 IEEE / Rust's f64 methods.  The host build replaces the hardware's reciprocal and reciprocal-square-root estimates by cruder ones
 (20 bits), so the bounds hold for the device a fortiori; tests/test_gpu_math.py asserts them there as well."""
@@ -18,7 +18,7 @@ def lib(tmp_path_factory):
     out = str(tmp_path_factory.mktemp("math64") / "libmath64.so")
     subprocess.check_call(["g++", "-O2", "-ffp-contract=off", "-shared", "-fPIC", "-o", out, os.path.join(HERE, "support", "math64_host.cpp")])
     L = C.CDLL(out)
-    for f in (L.log_many, L.log1p_many, L.asin_many, L.acos_many, L.tan_many, L.sqrt_ge1_many, L.rcp_many):
+    for f in (L.log_many, L.log1p_many, L.asin_many, L.acos_many, L.tan_many, L.sqrt_ge1_many, L.rcp_many, L.exp_nonpos_many):
         f.argtypes = [C.c_size_t, C.c_void_p, C.c_void_p]
     L.quot_many.argtypes = [C.c_size_t, C.c_void_p, C.c_void_p, C.c_void_p]
     L.sincos_kernel_many.argtypes = [C.c_size_t, C.c_void_p, C.c_void_p, C.c_void_p]
@@ -159,3 +159,26 @@ def test_reciprocal_quotient_and_square_root_helpers(lib):
     lib.quot_many(x.size, x.ctypes.data, y.ctypes.data, out.ctypes.data)
     err = ulp_error(out, x.astype(np.longdouble) / y.astype(np.longdouble))
     assert err.max() <= 1.0, float(err.max())
+
+
+def test_exp_of_non_positive_arguments_within_one_and_a_half_ulp(lib):
+    if np.finfo(np.longdouble).nmant < 63:
+        pytest.skip("no 80-bit long double on this machine")
+    rng = np.random.default_rng(9)
+    ln2 = np.log(2.0)
+    k = rng.integers(0, 1080, size=200_000)
+    # the whole range down to where the result is 0, every magnitude near 0, either side of the points where the nearest multiple of
+    # ln 2 changes (|r| largest), results in the denormal range
+    x = -np.concatenate([rng.uniform(0, 760, size=400_000), 10.0 ** rng.uniform(-320, 2.9, size=200_000), (k + 0.5) * ln2 + rng.normal(size=k.size) * 1e-9,
+                         k * ln2 + rng.normal(size=k.size) * 1e-9, rng.uniform(700, 746, size=100_000), np.array([0.0, 5e-324, 1e-16, 1.0, 708.4, 745.13, 745.14, 750.0, 1e300])])
+    x = x[x <= 0]
+    got = call(lib.exp_nonpos_many, x)
+    exact = np.exp(x.astype(np.longdouble))
+    normal = exact >= np.finfo(np.float64).tiny
+    err = ulp_error(got[normal], exact[normal])
+    assert err.max() < 1.5, (float(err.max()), float(x[normal][err.argmax()]))
+    # denormal results: within one unit of the last (denormal) place; and nothing below 2^-1075 comes back non-zero
+    sub = np.abs(got[~normal].astype(np.longdouble) - exact[~normal]) / np.longdouble(5e-324)
+    assert sub.max() <= 1.0, float(sub.max())
+    special = call(lib.exp_nonpos_many, np.array([-np.inf, np.nan, -0.0, -1e308]))
+    assert special[0] == 0.0 and special[1] == 0.0 and special[2] == 1.0 and special[3] == 0.0        # NaN is the caller's business
