@@ -432,15 +432,32 @@ __host__ __device__ __forceinline__ bool rt_tile_index_block(const TileMap& m, u
 }
 
 // Column reductions over short rows: how many consecutive rows to read as one (1 = as they are).  The kernels that reduce over rows
-// with lanes along the columns are fastest when all blocks of the launch sit next to each other on rows of 128 KiB -- a few wide
-// fronts through memory instead of many narrow ones (1 GiB f32 sums over axis 0: 0.82 - 0.86 of peak at 1024 ... 16384 columns,
-// 0.90 at 32768 and beyond, and 0.89 - 0.90 for all of them regrouped).  The largest g that divides the row count, keeps the joined
-// row within 128 KiB and leaves at least 2048 joined rows; the g partial results per column are folded with the partials of the split.
-static inline uint64_t rt_cols_regroup(uint64_t rows, uint64_t row_bytes) {
-    if (row_bytes == 0 || row_bytes > 64 * 1024) return 1;
-    for (uint64_t g = (128 * 1024) / row_bytes; g >= 2; --g)
-        if (rows % g == 0 && rows / g >= 2048) return g;
-    return 1;
+// with lanes along the columns (a wave covers 1 KiB of a row, the rows are split over blocks until the launch has about `want`
+// blocks, one or two per CU) run at 0.72 ... 0.89 of peak on the same 1 GiB depending on how the row length meets that shape; joining g
+// consecutive rows into one changes the row length without changing the result (the g partial results per column are folded with
+// the partials of the split).  Among the g that divide the row count, leave at least 2048 joined rows and keep the joined row
+// within 128 KiB, the one with the best product of what the sweeps showed to matter (f32 sums over axis 0, 1 GiB):
+//   how full the launch is: 1000 columns, g = 20 (79 tiles x 3 segments = 237 blocks) 0.89, g = 24 (94 x 2 = 188) 0.74;
+//   joined rows that are whole 128-byte lines: 500 columns, g = 8 / 16 / 24 0.87 / 0.87 / 0.88, g = 10 / 20 0.80 / 0.82;
+//   how full the last tile of a row is;
+//   longer rows, mildly: 2048 columns, g = 1 / 3 / 10 / 16 0.85 / 0.87 / 0.88 / 0.89 (rows of one tile need no help: 256 columns 0.89).
+static inline uint64_t rt_cols_regroup(uint64_t rows, uint64_t row_bytes, uint64_t want) {
+    if (row_bytes == 0 || row_bytes > 64 * 1024 || want == 0) return 1;
+    uint64_t best = 1;
+    double best_score = 0.0;
+    for (uint64_t g = 1; g * row_bytes <= 128 * 1024; ++g) {
+        if (rows % g != 0 || (g > 1 && rows / g < 2048)) continue;
+        const uint64_t bytes = g * row_bytes, tiles = (bytes + 1023) / 1024;
+        const double lane_fill = (double)bytes / (double)(tiles * 1024);
+        uint64_t blocks = tiles >= want ? tiles : tiles * (want / tiles);
+        if (blocks * 4 < want * 3) blocks = tiles * ((2 * want + tiles - 1) / tiles);      // the split's own rule: twice as many segments
+        const double cu_fill = (double)blocks / (double)(((blocks + want - 1) / want) * want);
+        const double aligned = bytes % 128 == 0 ? 1.0 : 0.92;
+        const double length = tiles == 1 ? 1.0 : (bytes < (16u << 10) ? 0.96 : (bytes < (32u << 10) ? 0.98 : (bytes < (64u << 10) ? 0.99 : (bytes < (128u << 10) ? 0.995 : 1.0))));
+        const double score = lane_fill * cu_fill * aligned * length;
+        if (score > best_score * 1.005) { best_score = score; best = g; }               // a larger g has to earn its extra partials
+    }
+    return best;
 }
 
 // Division of a 32-bit numerator by a runtime-constant divisor via multiply-high (round-up method); exact for

@@ -252,7 +252,7 @@ int32_t backward_typed(rt_ctx* ctx, int dtype, const void* gmap, const void* y, 
     constexpr uint64_t N = 16 / sizeof(T);
     // Short rows are regrouped as in the column reduction (rt_reduce.hip, cols_launch): g consecutive rows are read as one row of
     // g * cols columns, and the g partial sums per column join the partials of the split in the column sum that follows.
-    const uint64_t g = rt_cols_regroup(rows_all, cols_out * sizeof(T));
+    const uint64_t g = rt_cols_regroup(rows_all, cols_out * sizeof(T), (uint64_t)ctx->num_cus * 2);
     const uint64_t rows = rows_all / g, cols = cols_out * g;
     const uint64_t tiles = (cols / N + RT_WAVE - 1) / RT_WAVE;
     const uint64_t want = (uint64_t)ctx->num_cus * 2;              // two resident blocks per CU, as the column reduction

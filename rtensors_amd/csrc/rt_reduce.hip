@@ -702,6 +702,52 @@ __global__ __launch_bounds__(kBlock) void reduce_merge_wave_kernel(const T* __re
     wave_reduce<Acc<OP, T> >(a);
     if (lane == 0) out[o] = finalize<OP, T>(a.v, count);
 }
+// Second stage of a float max / min over regrouped rows (cols_launch): the partials of one column cover interleaved sets of rows,
+// each holding the sequential result of its own set.  Their maximum is the column's; a zero maximum takes the sign that the zero
+// partials share, and where they disagree the column itself is searched for its first zero (the wave walks the rows in order and
+// stops at the first stretch that holds one).  One wave per output.
+template <int OP, class T>
+__global__ __launch_bounds__(kBlock) void reduce_merge_regroup_kernel(const T* __restrict__ part, T* __restrict__ out, const T* __restrict__ src, uint64_t nout,
+                                                                      uint32_t nparts, uint64_t rows) {
+    const uint64_t o = (uint64_t)blockIdx.x * kWaves + threadIdx.x / RT_WAVE;
+    if (o >= nout) return;
+    const uint32_t lane = threadIdx.x & (RT_WAVE - 1);
+    AccOrd<OP, T> a;
+    a.init();
+    bool pz = false, nz = false;
+    for (uint32_t k = lane; k < nparts; k += RT_WAVE) {
+        const T x = part[(uint64_t)k * nout + o];
+        a.push(x, k);
+        if (x == (T)0) { if (upper_bits<T>(x) < 0) nz = true; else pz = true; }
+    }
+    wave_reduce<AccOrd<OP, T> >(a);
+    const bool any_pz = __builtin_amdgcn_ballot_w64(pz) != 0, any_nz = __builtin_amdgcn_ballot_w64(nz) != 0;
+    T v = __shfl(a.v, 0, RT_WAVE);
+    if (v == (T)0) {
+        bool neg = any_nz;
+        if (any_nz && any_pz) {
+            uint64_t first = ~0ull;
+            for (uint64_t base = 0; base < rows; base += (uint64_t)RT_WAVE * 4) {
+#pragma unroll
+                for (int u = 3; u >= 0; --u) {
+                    const uint64_t r = base + (uint64_t)u * RT_WAVE + lane;
+                    if (r < rows && src[r * nout + o] == (T)0) first = r;
+                }
+                if (__builtin_amdgcn_ballot_w64(first != ~0ull)) break;
+            }
+#pragma unroll
+            for (int d = RT_WAVE / 2; d >= 1; d >>= 1) {
+                const uint64_t f2 = shfl_down_t<uint64_t>(first, d);
+                first = f2 < first ? f2 : first;
+            }
+            first = __shfl(first, 0, RT_WAVE);
+            neg = upper_bits<T>(src[first * nout + o]) < 0;
+        }
+        v = neg ? -(T)0 : (T)0;
+    }
+    if (lane == 0) out[o] = v;
+}
+
 template <int OP, class T>
 bool merge_few_outputs(rt_ctx* ctx, const T* part, T* out, uint64_t nout, uint32_t splits, uint64_t count) {
     if (splits < 8 || nout > 16384) return false;
@@ -827,9 +873,9 @@ int32_t cols_launch(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t 
     hipStream_t s = ctx->stream;
     const uint64_t per_tile = (uint64_t)RT_WAVE * VW;
     // Short rows are regrouped (rt_cols_regroup): g consecutive rows of `inner_out` columns are read as one row of g * inner_out
-    // columns, and the g partial results per column join the partials of the split in the second stage.  Not for the float max / min
-    // (their tie-breaking follows row positions) and only for one outer index.
-    const uint64_t g = (allow_split && outer == 1 && !Acc<OP, T>::kTrack && inner_out % VW == 0) ? rt_cols_regroup(R_all, inner_out * sizeof(T)) : 1;
+    // columns, and the g partial results per column join the partials of the split in the second stage (the float max / min, whose
+    // zero results follow row positions, have a second stage of their own for this).  Only for one outer index.
+    const uint64_t g = (allow_split && outer == 1 && inner_out % VW == 0) ? rt_cols_regroup(R_all, inner_out * sizeof(T), (uint64_t)ctx->num_cus) : 1;
     const uint64_t R = R_all / g, inner = inner_out * g;
     const uint64_t tiles = (inner + per_tile - 1) / per_tile;
     // One block of four waves per CU, eight loads in flight per lane, each block streaming a long run of rows: the segments are cut so
@@ -878,6 +924,14 @@ int32_t cols_launch(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t 
     RT_HIP(hipGetLastError());
     // second stage: partials are (splits, outer * inner) -- with regrouped rows (splits * g, inner_out): a column reduce with R = splits * g
     const uint64_t inner2 = outer * inner_out, R2 = (uint64_t)splits * g;
+    if constexpr (Acc<OP, T>::kTrack) {
+        if (g > 1) {
+            hipLaunchKernelGGL((reduce_merge_regroup_kernel<OP, T>), dim3((unsigned)((inner2 + kWaves - 1) / kWaves)), dim3(kBlock), 0, s, part, out, src, inner2,
+                               (uint32_t)R2, R_all);
+            RT_HIP(hipGetLastError());
+            return RT_OK;
+        }
+    }
     if (merge_few_outputs<OP, T>(ctx, part, out, inner2, (uint32_t)R2, count)) { RT_HIP(hipGetLastError()); return RT_OK; }
     const uint64_t tiles2 = (inner2 + per_tile - 1) / per_tile;
     if (tiles2 >= (1ull << 31)) return rt_fail(RT_E_INVALID, "reduce: too many outputs for one launch");

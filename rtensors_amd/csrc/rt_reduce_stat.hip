@@ -476,7 +476,7 @@ __global__ __launch_bounds__(kBlock) void st_rows_tile_kernel(const T* __restric
                     }
                     for (; k < a.R; k += a.G) top = m_max(top, row[k]);
                 }
-                for (uint32_t d = a.G / 2; d >= 1; d >>= 1) top = m_max(top, __shfl_xor(top, (int)d, RT_WAVE));
+                top = group_all<OpMax>(top, a.G);
                 T sum = (T)0;
                 bool bad = false;
                 if (r < nrows) {
@@ -495,7 +495,7 @@ __global__ __launch_bounds__(kBlock) void st_rows_tile_kernel(const T* __restric
                     }
                 }
                 if (S::kNoteNan && bad) sum = std::numeric_limits<T>::quiet_NaN();
-                for (uint32_t d = a.G / 2; d >= 1; d >>= 1) sum = sum + __shfl_xor(sum, (int)d, RT_WAVE);
+                sum = group_all<OpSum>(sum, a.G);
                 acc.m = top;
                 acc.s = sum;
             }
@@ -531,7 +531,7 @@ __global__ __launch_bounds__(kBlock) void st_rows_pow2_kernel(const T* __restric
 #pragma unroll
                 for (uint32_t e = 0; e < N; ++e) top = m_max(top, x[u].e[e]);
             }
-            for (uint32_t d = VR / 2; d >= 1; d >>= 1) top = m_max(top, __shfl_xor(top, (int)d, RT_WAVE));
+            top = group_all<OpMax>(top, VR);
             T sum = (T)0;
             bool bad = false;
             if (v < nvec) {
@@ -542,7 +542,7 @@ __global__ __launch_bounds__(kBlock) void st_rows_pow2_kernel(const T* __restric
                 }
             }
             if (S::kNoteNan && bad) sum = std::numeric_limits<T>::quiet_NaN();
-            for (uint32_t d = VR / 2; d >= 1; d >>= 1) sum = sum + __shfl_xor(sum, (int)d, RT_WAVE);
+            sum = group_all<OpSum>(sum, VR);
             a.m = top;
             a.s = sum;
         } else {
@@ -558,7 +558,8 @@ __global__ __launch_bounds__(kBlock) void st_rows_pow2_kernel(const T* __restric
 // k = begin + ty, + kWaves, ...  Results go to out[o * inner + col], partial states to part[(seg * outer + o) * inner + col].
 template <class S, class T, int VW, int U = 4>
 __global__ __launch_bounds__(kBlock) void st_cols_kernel(const T* __restrict__ src, typename S::Out* __restrict__ out, S* __restrict__ part, uint64_t R,
-                                                         uint64_t inner, uint64_t outer, uint32_t tiles, uint32_t splits, uint64_t seglen, int flags) {
+                                                         uint64_t inner, uint64_t outer, uint32_t tiles, uint32_t splits, uint64_t seglen, int flags,
+                                                         uint32_t regroup, uint64_t inner_out) {
     struct alignas(sizeof(T) * VW) VecW { T e[VW]; };
     uint64_t b = blockIdx.x;
     const uint32_t tile = (uint32_t)(b % tiles);
@@ -625,6 +626,10 @@ __global__ __launch_bounds__(kBlock) void st_cols_kernel(const T* __restrict__ s
 #pragma unroll
             for (int w = 0; w < kWaves - 1; ++w) a[j].merge(sm[w][tx][j]);
             if ((uint32_t)j < skip) continue;
+            if constexpr (is_arg_state<S>::value) {
+                // regrouped rows: column c of the joined row k is column c % inner_out of row k * regroup + c / inner_out
+                if (regroup > 1 && a[j].idx != ~0ull) a[j].idx = a[j].idx * regroup + (col + j) / inner_out;
+            }
             if (part) part[at + j] = a[j];
             else out[at + j] = a[j].result(flags);
         }
@@ -901,16 +906,24 @@ int32_t cols_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t oute
     hipStream_t s = ctx->stream;
     const uint64_t per_tile = (uint64_t)RT_WAVE * VW;
     // Short rows are regrouped as in the plain column reduction (rt_cols_regroup): g consecutive rows are read as one, and the g
-    // partial states per column join those of the split in the merge.  Not for the index states (their positions are row numbers).
-    const uint64_t g = (outer == 1 && !is_arg_state<S>::value && inner_out % VW == 0) ? rt_cols_regroup(R_all, inner_out * sizeof(T)) : 1;
+    // partial states per column join those of the split in the merge (the index states turn their positions back into row numbers).
+    const uint64_t g = (outer == 1 && inner_out % VW == 0) ? rt_cols_regroup(R_all, inner_out * sizeof(T), (uint64_t)ctx->num_cus * S::kColsBlocksPerCU) : 1;
     const uint64_t R = R_all / g, inner = inner_out * g;
     const uint64_t tiles = (inner + per_tile - 1) / per_tile;
     const uint64_t want = (uint64_t)ctx->num_cus * S::kColsBlocksPerCU;
     uint32_t splits = 1;
     if (outer * tiles < want) {
+        // as many segments as keep the blocks within `want` (rounding up put 260 blocks on 256 CUs: the four CUs with two blocks set
+        // the time, 1 GiB f32 variance over axis 0 of 1000 columns 0.62 of peak); when that leaves a quarter of them unused, twice as many
         const uint64_t min_seg = 64;
-        const uint64_t by_size = R / min_seg, by_need = (want + outer * tiles - 1) / (outer * tiles);
-        uint64_t sp = by_need < by_size ? by_need : by_size;
+        const uint64_t by_size = R / min_seg;
+        uint64_t sp = want / (outer * tiles);
+        if (sp > by_size) sp = by_size;
+        if (sp < 1) sp = 1;
+        if (outer * tiles * sp * 4 < want * 3) {
+            const uint64_t by_need = (2 * want + outer * tiles - 1) / (outer * tiles);
+            sp = by_need < by_size ? by_need : by_size;
+        }
         if (sp > 1024) sp = 1024;
         if (sp > 1) splits = (uint32_t)sp;
     }
@@ -929,7 +942,7 @@ int32_t cols_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t oute
         part = (S*)scratch;
     }
     hipLaunchKernelGGL((st_cols_kernel<S, T, VW, S::kColsLoads>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, out, part, R, inner, outer, (uint32_t)tiles,
-                       splits, seglen, flags);
+                       splits, seglen, flags, (uint32_t)g, inner_out);
     RT_HIP(hipGetLastError());
     if (staged) RT_TRY(merge_cols<S>(ctx, part, out, outer * inner_out, (uint32_t)(splits * g), flags));
     return RT_OK;

@@ -1541,7 +1541,7 @@ def test_float_max_min_keep_the_first_zero_in_every_kernel_shape(hip, dtype):
     rng = np.random.default_rng(zlib.crc32(b"zero-sign" + dtype.encode()))
     shapes = [(4, 100000, 1), (3000, 5000, 1), (1, 1 << 21, 1), (5000, 600, 1), (3000, 2000, 1), (20000, 100, 1), (20000, 10, 1), (40000, 64, 1),
               (8192, 256, 1), (70, 33, 1), (1, 5000, 512), (8, 300, 1024), (1, 4096, 4096), (2, 3000, 1001), (1, 100000, 3), (4, 5000, 100),
-              (5000, 16, 64), (100, 8, 1000), (1, 70001, 17), (300, 200, 8)]
+              (5000, 16, 64), (100, 8, 1000), (1, 70001, 17), (300, 200, 8), (1, 70000, 128), (1, 65536, 256), (1, 30000, 1000), (1, 70001, 128)]
     for outer, R, inner in shapes:
         n = outer * R * inner
         mag = np.abs(rng.normal(size=n)).astype(npd) + npd(0.5)
@@ -1628,6 +1628,7 @@ STAT_SHAPES = ([(rows, R, 1) for R in (1, 2, 3, 7, 8, 31, 32, 33, 64, 65, 100, 2
                + [(30000, R, 1) for R in (1, 2, 4, 8, 16, 32, 64)]
                + [(outer, R, inner) for inner in (2, 3, 5, 17, 63, 64, 100, 128) for R, outer in ((64, 3), (1000, 1), (5003, 2), (70001, 1))]
                + [(outer, R, inner) for R in (1, 2, 5, 16, 33) for inner, outer in ((2, 1000), (3, 1), (64, 50), (1028, 2))]
+               + [(1, 65536, 256), (1, 30000, 1000), (1, 8192, 2048)]                  # rows regrouped before the column kernel reads them
                + [(1, 300, 5000), (2, 4000, 260), (1, 70, 2052), (2, 300, 257), (1, 5003, 1001), (3, 100, 129), (1, 2000, 1030), (1, 70, 4099), (2, 40, 131)])
 
 
