@@ -431,13 +431,67 @@ __host__ __device__ __forceinline__ bool rt_tile_index_block(const TileMap& m, u
     return rt_tile_index(m, block, nthreads, tid, nvec, out);
 }
 
+// Column reductions: into how many segments to split the rows of `tiles` column tiles (a tile is what one block covers of a row), when
+// `want` blocks fill the chip (one or two per CU, by the kernel) and a segment should keep at least a few dozen rows (`by_size` = the
+// most segments the row count allows).
+// The plain rule: as many segments as keep the blocks within `want`; when that leaves a quarter of the places unused, twice as many.
+static inline uint32_t rt_cols_splits_plain(uint64_t tiles, uint64_t want, uint64_t by_size) {
+    if (tiles == 0 || tiles >= want) return 1;
+    if (by_size < 1) by_size = 1;
+    uint64_t sp = want / tiles;
+    if (sp > by_size) sp = by_size;
+    if (sp < 1) sp = 1;
+    if (tiles * sp * 4 < want * 3) {
+        const uint64_t by_need = (2 * want + tiles - 1) / tiles;
+        sp = by_need < by_size ? by_need : by_size;
+    }
+    return (uint32_t)(sp > 1024 ? 1024 : sp);
+}
+// Rows of 64 KiB and more (64 tiles; such rows are never regrouped) meet that rule badly: 129 tiles get one segment and half the CUs,
+// 274 tiles 1.07 rounds.  With x = blocks / want, a forced-split sweep (1 GiB f32 sums over axis 0, 98 ... 1024 tiles, 1 ... 16
+// segments, rate relative to the best) reads: up to one round the rate grows as 0.2 + 1.05 x and is at its best from x = 0.77; just
+// past a whole number of rounds it falls off a cliff (x = 1.008: 0.70, 2.016: 0.77, 3.05: 0.84), because the few CUs with one block
+// more finish late, and recovers as the last round fills (1.53: 0.92, 1.84: 0.95, 3.83: 0.95); many rounds cost a little each (smaller
+// segments, more partials).  The split with the best estimate is taken; an unsplit launch spares the second stage, which costs the
+// statistics (`lean` = false: states instead of values, and more arithmetic per element, so that they also gain from every further
+// block up to a full round and take the plain ramp x there) more than the plain reductions.  Against the plain rule, on one machine,
+// of peak -- sum, 129 tiles: 0.70 -> 0.82, 157: 0.80 -> 0.85, 274: 0.66 -> 0.83, 586: 0.78 -> 0.83; variance, 98: 0.75 -> 0.85, 129:
+// 0.68 -> 0.80, 196: 0.75 -> 0.83; f64 sum over 20000 columns 0.81 -> 0.86.
+static inline double rt_cols_launch_rate(uint64_t blocks, uint64_t want, bool lean) {
+    const double x = (double)blocks / (double)want;
+    if (x <= 1.0) {
+        if (!lean) return 0.1 + 0.9 * x;
+        const double r = 0.2 + 1.05 * x;
+        return (r < 1.0 ? r : 1.0) * (0.9 + 0.1 * x);                // among equals the fuller launch
+    }
+    const double k = (double)(blocks / want), fr = x - k;
+    const double time = k + (fr > 0.0 ? 0.35 + 0.6 * fr : 0.0);
+    return 0.95 * x / time * (1.0 - 0.012 * (k - 1.0));
+}
+static inline uint32_t rt_cols_splits_wide(uint64_t tiles, uint64_t want, uint64_t by_size, bool lean) {
+    if (tiles == 0 || want == 0) return 1;
+    if (tiles < 64) return rt_cols_splits_plain(tiles, want, by_size);
+    if (by_size < 1) by_size = 1;
+    uint64_t best = 1;
+    double best_score = 0.0;
+    uint64_t limit = by_size > 1024 ? 1024 : by_size;
+    const uint64_t enough = (8 * want + tiles - 1) / tiles;                      // beyond eight rounds nothing new happens
+    if (limit > enough) limit = enough;
+    for (uint64_t sp = 1; sp <= limit; ++sp) {
+        double score = rt_cols_launch_rate(tiles * sp, want, lean);
+        if (sp > 1) score *= lean ? 0.985 : 0.95;
+        if (score > best_score * 1.002) { best_score = score; best = sp; }
+    }
+    return (uint32_t)best;
+}
+
 // Column reductions over short rows: how many consecutive rows to read as one (1 = as they are).  The kernels that reduce over rows
 // with lanes along the columns (a wave covers 1 KiB of a row, the rows are split over blocks until the launch has about `want`
-// blocks, one or two per CU) run at 0.72 ... 0.89 of peak on the same 1 GiB depending on how the row length meets that shape; joining g
-// consecutive rows into one changes the row length without changing the result (the g partial results per column are folded with
-// the partials of the split).  Among the g that divide the row count, leave at least 2048 joined rows and keep the joined row
-// within 128 KiB, the one with the best product of what the sweeps showed to matter (f32 sums over axis 0, 1 GiB):
-//   how full the launch is: 1000 columns, g = 20 (79 tiles x 3 segments = 237 blocks) 0.89, g = 24 (94 x 2 = 188) 0.74;
+// blocks) run at 0.72 ... 0.89 of peak on the same 1 GiB depending on how the row length meets that shape; joining g consecutive
+// rows into one changes the row length without changing the result (the g partial results per column are folded with the partials
+// of the split).  Among the g that divide the row count, leave at least 2048 joined rows and keep the joined row within 128 KiB, the
+// one with the best product of what the sweeps showed to matter (f32 sums over axis 0, 1 GiB):
+//   how full the launch is under the plain split rule: 1000 columns, g = 20 (79 tiles x 3 segments = 237 blocks) 0.89, g = 24 (94 tiles) 0.74;
 //   joined rows that are whole 128-byte lines: 500 columns, g = 8 / 16 / 24 0.87 / 0.87 / 0.88, g = 10 / 20 0.80 / 0.82;
 //   how full the last tile of a row is;
 //   longer rows, mildly: 2048 columns, g = 1 / 3 / 10 / 16 0.85 / 0.87 / 0.88 / 0.89 (rows of one tile need no help: 256 columns 0.89).
@@ -449,12 +503,11 @@ static inline uint64_t rt_cols_regroup(uint64_t rows, uint64_t row_bytes, uint64
         if (rows % g != 0 || (g > 1 && rows / g < 2048)) continue;
         const uint64_t bytes = g * row_bytes, tiles = (bytes + 1023) / 1024;
         const double lane_fill = (double)bytes / (double)(tiles * 1024);
-        uint64_t blocks = tiles >= want ? tiles : tiles * (want / tiles);
-        if (blocks * 4 < want * 3) blocks = tiles * ((2 * want + tiles - 1) / tiles);      // the split's own rule: twice as many segments
-        const double cu_fill = (double)blocks / (double)(((blocks + want - 1) / want) * want);
+        const uint64_t blocks = tiles * rt_cols_splits_plain(tiles, want, ~0ull);
+        const double launch = (double)blocks / (double)(((blocks + want - 1) / want) * want);
         const double aligned = bytes % 128 == 0 ? 1.0 : 0.92;
         const double length = tiles == 1 ? 1.0 : (bytes < (16u << 10) ? 0.96 : (bytes < (32u << 10) ? 0.98 : (bytes < (64u << 10) ? 0.99 : (bytes < (128u << 10) ? 0.995 : 1.0))));
-        const double score = lane_fill * cu_fill * aligned * length;
+        const double score = lane_fill * launch * aligned * length;
         if (score > best_score * 1.005) { best_score = score; best = g; }               // a larger g has to earn its extra partials
     }
     return best;

@@ -879,25 +879,12 @@ int32_t cols_launch(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t 
     const uint64_t R = R_all / g, inner = inner_out * g;
     const uint64_t tiles = (inner + per_tile - 1) / per_tile;
     // One block of four waves per CU, eight loads in flight per lane, each block streaming a long run of rows: the segments are cut so
-    // that the blocks do not outnumber the CUs (1 GiB f32 sums over axis 0, against two blocks per CU: 8192 x 32768 0.857 -> 0.893 of
-    // peak, 26844 x 10000 0.66 -> 0.82, 13422 x 20000 0.74 -> 0.88, 65536 x 4096 0.82 -> 0.83; eight blocks per CU: 0.70-0.83).
-    // When that would leave more than a quarter of the CUs without a block (150 column tiles: 0.60 for a max), two blocks per CU as
-    // before.  Outputs that already give every CU a block are not split.
+    // that the blocks fill the CUs in whole rounds (1 GiB f32 sums over axis 0, one block per CU against two: 8192 x 32768 0.857 ->
+    // 0.893 of peak, 26844 x 10000 0.66 -> 0.82, 13422 x 20000 0.74 -> 0.88; eight blocks per CU: 0.70-0.83); see rt_cols_splits_plain / _wide.
+    // Outputs that already give every CU a block are not split unless their last round would be far from full.
     const uint64_t cus = (uint64_t)ctx->num_cus;
     uint32_t splits = 1;
-    if (allow_split && outer * tiles < cus) {
-        const uint64_t min_seg = 64;                          // k values per block
-        const uint64_t by_size = R / min_seg;
-        uint64_t sp = cus / (outer * tiles);
-        if (sp > by_size) sp = by_size;
-        if (sp < 1) sp = 1;
-        if (outer * tiles * sp * 4 < cus * 3) {
-            const uint64_t by_need = (2 * cus + outer * tiles - 1) / (outer * tiles);
-            sp = by_need < by_size ? by_need : by_size;
-        }
-        if (sp > 1024) sp = 1024;
-        if (sp > 1) splits = (uint32_t)sp;
-    }
+    if (allow_split) splits = g > 1 ? rt_cols_splits_plain(outer * tiles, cus, R / 64) : rt_cols_splits_wide(outer * tiles, cus, R / 64, true);
     uint64_t seglen = (R + splits - 1) / splits;
     if (splits > 1) {
         seglen = (seglen + 8 * kWaves - 1) / (8 * kWaves) * (8 * kWaves);

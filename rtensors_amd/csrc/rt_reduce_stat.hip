@@ -912,21 +912,9 @@ int32_t cols_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t oute
     const uint64_t tiles = (inner + per_tile - 1) / per_tile;
     const uint64_t want = (uint64_t)ctx->num_cus * S::kColsBlocksPerCU;
     uint32_t splits = 1;
-    if (outer * tiles < want) {
-        // as many segments as keep the blocks within `want` (rounding up put 260 blocks on 256 CUs: the four CUs with two blocks set
-        // the time, 1 GiB f32 variance over axis 0 of 1000 columns 0.62 of peak); when that leaves a quarter of them unused, twice as many
-        const uint64_t min_seg = 64;
-        const uint64_t by_size = R / min_seg;
-        uint64_t sp = want / (outer * tiles);
-        if (sp > by_size) sp = by_size;
-        if (sp < 1) sp = 1;
-        if (outer * tiles * sp * 4 < want * 3) {
-            const uint64_t by_need = (2 * want + outer * tiles - 1) / (outer * tiles);
-            sp = by_need < by_size ? by_need : by_size;
-        }
-        if (sp > 1024) sp = 1024;
-        if (sp > 1) splits = (uint32_t)sp;
-    }
+    // whole rounds of `want` blocks (rounding the need up put 260 blocks on 256 CUs: 1 GiB f32 variance over axis 0 of 1000 columns 0.62 of
+    // peak); wide rows by the estimate of rt_cols_splits_wide, except for the index states, which it did not help (391 tiles: 0.86 -> 0.77)
+    splits = (g > 1 || is_arg_state<S>::value) ? rt_cols_splits_plain(outer * tiles, want, R / 64) : rt_cols_splits_wide(outer * tiles, want, R / 64, false);
     uint64_t seglen = (R + splits - 1) / splits;
     if (splits > 1) {
         seglen = (seglen + 8 * kWaves - 1) / (8 * kWaves) * (8 * kWaves);
