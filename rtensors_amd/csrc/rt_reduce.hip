@@ -430,10 +430,14 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(const T* __restrict
 // 0.69 -> 0.76 of peak, variance 0.71 -> 0.77, sum 0.71 -> 0.76; rows of 100: 0.67 -> 0.73, 0.73 -> 0.79, 0.73 -> 0.81; 16, 20, 22 and
 // 26 KiB lie between, 48 KiB (three blocks) loses 10 %.
 constexpr uint32_t kRowsTileBytes = 24576;
+// The same kernel takes small slabs with a few columns ((outer, R, inner) with inner <= 64 and R * inner elements in at most 8 KiB):
+// a "row" of the tile is then the slab of one outer index, L = R * inner elements, and a group of lanes folds one of its columns,
+// elements c, c + inner, ...  (A lane per output read such slabs from memory with a stride of one slab between lanes: 1 GiB f32
+// summed over the middle axis of (2033601, 33, 2) ran at 0.11 of peak.)
 struct RowsTileArgs {
     uint64_t rows;
-    uint32_t R, pitch, rpb, T;          // row length, LDS pitch, rows per block, lanes per row (power of two <= 64)
-    FastDiv32 r_div;
+    uint32_t R, L, inner, pitch, rpb, T;   // reduced length, elements per row of the tile (R * inner), columns, LDS pitch, rows per block, lanes per output (power of two <= 64)
+    FastDiv32 l_div, inner_div;
 };
 
 template <int OP, class T>
@@ -442,20 +446,20 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_tile_kernel(const T* __res
     __shared__ alignas(16) T tile[kRowsTileBytes / sizeof(T)];
     const uint64_t row0 = (uint64_t)blockIdx.x * a.rpb;
     const uint32_t nrows = (uint32_t)(a.rows - row0 < a.rpb ? a.rows - row0 : a.rpb);
-    const uint32_t ne = nrows * a.R;
-    const T* p = src + row0 * a.R;
-    // pitch == R: the run is copied as it lies, with 16-byte LDS stores; `mis` keeps the 16-byte phase of the global address.  Always
+    const uint32_t ne = nrows * a.L;
+    const T* p = src + row0 * a.L;
+    // pitch == L: the run is copied as it lies, with 16-byte LDS stores; `mis` keeps the 16-byte phase of the global address.  Always
     // for 1- and 2-byte elements (an element-wise scatter would issue 8 or 16 sub-word stores per vector: u8 rows of 100 ran at
     // 1.9 TB/s), and for wider elements whenever rows at that pitch meet at most two to a bank (see tile_pitch); otherwise rows go
     // to a padded pitch element by element, an index division per element.
-    const bool verbatim = a.pitch == a.R;
+    const bool verbatim = a.pitch == a.L;
     const uint32_t mis = verbatim ? (uint32_t)((reinterpret_cast<uintptr_t>(p) & 15) / sizeof(T)) : 0u;
     auto put = [&](uint32_t e, T v) {
         if (verbatim) {
             tile[mis + e] = v;
         } else {
-            const uint32_t r = fd_div(e, a.r_div);
-            tile[r * a.pitch + (e - r * a.R)] = v;
+            const uint32_t r = fd_div(e, a.l_div);
+            tile[r * a.pitch + (e - r * a.L)] = v;
         }
     };
     uint32_t head = (uint32_t)(((16 - (reinterpret_cast<uintptr_t>(p) & 15)) & 15) / sizeof(T));
@@ -485,30 +489,34 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_tile_kernel(const T* __res
     if (tb + threadIdx.x < ne) put(tb + threadIdx.x, p[tb + threadIdx.x]);
     __syncthreads();
     const uint32_t g = threadIdx.x / a.T, j = threadIdx.x & (a.T - 1), groups = kBlock / a.T;
-    // the T lanes of a group take elements j, j + T, ... of their row: interleaved positions
-    auto fold_row = [&](auto& acc, const T* row) {
+    // the T lanes of a group take elements j, j + T, ... of their column: interleaved positions
+    auto fold_row = [&](auto& acc, const T* col) {
         acc.init();
-        for (uint32_t k = j; k < a.R; k += a.T) acc.push(row[k], k);
+        for (uint32_t k = j; k < a.R; k += a.T) acc.push(col[k * a.inner], k);
         for (uint32_t d = a.T / 2; d >= 1; d >>= 1) {
             auto o = acc.shfl_down((int)d);
             if (j + d < a.T) acc.merge(o);
         }
     };
-    for (uint32_t r = g; r < nrows; r += groups) {
-        const T* row = tile + mis + r * a.pitch;                  // pitch == R in the verbatim layout
+    const uint32_t nout = nrows * a.inner;
+    for (uint32_t q = g; q < nout; q += groups) {
+        const uint32_t r = a.inner == 1 ? q : fd_div(q, a.inner_div);
+        const uint32_t c = q - r * a.inner;
+        const T* col = tile + mis + r * a.pitch + c;              // pitch == L in the verbatim layout
+        T* dst = out + (row0 + r) * a.inner + c;
         if constexpr (Acc<OP, T>::kTrack) {
-            AccQuick<OP, T> q;
-            fold_row(q, row);
+            AccQuick<OP, T> qa;
+            fold_row(qa, col);
             // one decision for the wave (its groups share the trip count of this loop up to the last trip, where the lanes of
             // finished groups are off): any group's unsettled zero sends all of them through the fold with positions
-            if (!__builtin_amdgcn_ballot_w64(j == 0 && !q.settled())) {
-                if (j == 0) out[row0 + r] = finalize<OP, T>(q.value(), count);
+            if (!__builtin_amdgcn_ballot_w64(j == 0 && !qa.settled())) {
+                if (j == 0) *dst = finalize<OP, T>(qa.value(), count);
                 continue;
             }
         }
         Acc<OP, T> acc;
-        fold_row(acc, row);
-        if (j == 0) out[row0 + r] = finalize<OP, T>(acc.v, count);
+        fold_row(acc, col);
+        if (j == 0) *dst = finalize<OP, T>(acc.v, count);
     }
 }
 
@@ -659,7 +667,12 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_short_kernel(const T* __re
     if (idx >= nvec_out) return;
     const uint32_t o = fd_div((uint32_t)idx, iv_div);           // nvec_out < 2^32 on this path
     const uint32_t iv = (uint32_t)idx - o * inner_vecs;
-    const T* p = src + (uint64_t)o * R * inner + (uint64_t)iv * VW;
+    // the last vector of a row whose length is not a multiple of VW moves back to the row's last VW columns (VW <= inner here): it
+    // folds `skip` columns of its neighbour a second time and does not write them
+    const uint64_t col0 = (uint64_t)iv * VW;
+    const uint64_t col = inner - col0 < (uint64_t)VW ? inner - VW : col0;
+    const uint32_t skip = (uint32_t)(col0 - col);
+    const T* p = src + (uint64_t)o * R * inner + col;
     AccOrd<OP, T> acc[VW];                                      // each lane folds its columns in order
 #pragma unroll
     for (int j = 0; j < VW; ++j) acc[j].init();
@@ -681,9 +694,10 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_short_kernel(const T* __re
             }
         }
     }
-    T* q = out + (uint64_t)o * inner + (uint64_t)iv * VW;
+    T* q = out + (uint64_t)o * inner + col;
 #pragma unroll
-    for (int j = 0; j < VW; ++j) q[j] = finalize<OP, T>(acc[j].v, count);
+    for (int j = 0; j < VW; ++j)
+        if ((uint32_t)j >= skip) q[j] = finalize<OP, T>(acc[j].v, count);
 }
 
 constexpr uint64_t kRowsTileMaxR = 1024;
@@ -757,6 +771,28 @@ bool merge_few_outputs(rt_ctx* ctx, const T* part, T* out, uint64_t nout, uint32
 }
 
 // ---- host planning ------------------------------------------------------------------------------------------------------
+// the LDS-tiled kernel over `rows` runs of R * inner elements (inner == 1: short rows; else small slabs with a few columns)
+template <int OP, class T>
+int32_t tile_launch(rt_ctx* ctx, const T* src, T* out, uint64_t rows, uint64_t R, uint64_t inner, uint64_t count) {
+    RowsTileArgs a;
+    a.rows = rows;
+    a.R = (uint32_t)R;
+    a.inner = (uint32_t)inner;
+    a.L = (uint32_t)(R * inner);
+    a.pitch = rt_tile_pitch(a.L, (uint32_t)sizeof(T));
+    a.rpb = (uint32_t)(kRowsTileBytes / sizeof(T) - (a.pitch == a.L ? 16 / sizeof(T) : 0)) / a.pitch;
+    a.l_div = make_fastdiv(a.L);
+    a.inner_div = make_fastdiv(a.inner);
+    uint32_t t = 1;                                               // lanes per output: fill the block, at most one wave, at most R
+    while (t < 64 && (uint64_t)t * 2 * a.rpb * inner <= (uint64_t)kBlock && t * 2 <= a.R) t <<= 1;
+    a.T = t;
+    const uint64_t blocks = (rows + a.rpb - 1) / a.rpb;
+    if (blocks >= (1ull << 31)) return rt_fail(RT_E_INVALID, "reduce: too many rows for one launch");
+    hipLaunchKernelGGL((reduce_rows_tile_kernel<OP, T>), dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream, src, out, a, count);
+    RT_HIP(hipGetLastError());
+    return RT_OK;
+}
+
 template <int OP, class T>
 int32_t rows_stage(rt_ctx* ctx, const T* src, T* out, uint64_t rows, uint64_t R, uint64_t count, bool allow_split) {
     hipStream_t s = ctx->stream;
@@ -782,20 +818,7 @@ int32_t rows_stage(rt_ctx* ctx, const T* src, T* out, uint64_t rows, uint64_t R,
     // short rows (not the second stage of a split reduction).  From 2 KiB per row a wave per row is faster (f32 sum, 1 GiB: rows of
     // 512 elements 0.183 ms staged / 0.155 ms direct, 1024: 0.188 / 0.159; below that the staged form wins, 256: 0.185 / 0.222)
     if (R >= 1 && R <= kRowsTileMaxR && R * sizeof(T) < 2048 && count == R) {
-        RowsTileArgs a;
-        a.rows = rows;
-        a.R = (uint32_t)R;
-        a.pitch = rt_tile_pitch(a.R, (uint32_t)sizeof(T));
-        a.rpb = (uint32_t)(kRowsTileBytes / sizeof(T) - (a.pitch == a.R ? 16 / sizeof(T) : 0)) / a.pitch;
-        a.r_div = make_fastdiv(a.R);
-        uint32_t t = 1;                                           // lanes per row: fill the block, at most one wave, at most R
-        while (t < 64 && (uint64_t)t * 2 * a.rpb <= (uint64_t)kBlock && t * 2 <= a.R) t <<= 1;
-        a.T = t;
-        const uint64_t blocks = (rows + a.rpb - 1) / a.rpb;
-        if (blocks >= (1ull << 31)) return rt_fail(RT_E_INVALID, "reduce: too many rows for one launch");
-        hipLaunchKernelGGL((reduce_rows_tile_kernel<OP, T>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, out, a, count);
-        RT_HIP(hipGetLastError());
-        return RT_OK;
+        return tile_launch<OP, T>(ctx, src, out, rows, R, 1, count);
     }
     if (R < 64) {
         uint64_t blocks = (rows + kBlock - 1) / kBlock;
@@ -986,9 +1009,12 @@ int32_t reduce_typed(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t
     // gave 0.3-2.3, lanes along a narrow inner 0.2-1.2.
     // short reduced axis: a lane per output vector.  Also for slabs of at most 8 KiB with up to 256 rows, which leave a block of the
     // narrow-column kernel too little to do ((262144, 64, 16) f32: 0.35 -> 0.61 of peak; from 16 KiB on the narrow kernel wins)
-    if ((R <= 32 || (R <= 256 && R * inner * sizeof(T) <= 8192)) && inner <= 1024) {
-        const bool v = inner % N == 0;                                          // rows may start at any element
-        const uint64_t ivecs = v ? inner / N : inner;
+    // small slabs with a few columns: through LDS (see RowsTileArgs)
+    if (inner <= 64 && R >= 2 && R * inner * sizeof(T) <= 8192 && outer >= 1024) return tile_launch<OP, T>(ctx, src, out, outer, R, inner, R);
+    // an axis of up to four elements is an elementwise pass over `inner` lanes wide: any inner
+    if ((R <= 32 || (R <= 256 && R * inner * sizeof(T) <= 8192)) && (inner <= 1024 || R <= 4)) {
+        const bool v = inner >= (uint64_t)N;                                    // rows may start at any element and have any length
+        const uint64_t ivecs = v ? (inner + N - 1) / N : inner;
         if (ivecs < (1ull << 31) && outer * ivecs < (1ull << 31)) {
             const uint64_t nvec_out = outer * ivecs;
             const uint64_t blocks = (nvec_out + kBlock - 1) / kBlock;

@@ -382,10 +382,12 @@ __global__ __launch_bounds__(kBlock) void st_rows_wave_kernel(const T* __restric
 // 26 KiB lie between, 48 KiB (three blocks) loses 10 %.
 constexpr uint32_t kTileBytes = 24576;
 constexpr uint64_t kTileMaxR = 1024;
+// (also for small slabs with a few columns, as the plain reductions' tiled kernel: a row of the tile is then the slab of one outer
+// index, L = R * inner elements, and a group of lanes folds one of its columns)
 struct TileArgs {
     uint64_t rows;
-    uint32_t R, pitch, rpb, G;
-    FastDiv32 r_div;
+    uint32_t R, L, inner, pitch, rpb, G;
+    FastDiv32 l_div, inner_div;
 };
 
 template <class S, class T>
@@ -394,20 +396,20 @@ __global__ __launch_bounds__(kBlock) void st_rows_tile_kernel(const T* __restric
     __shared__ alignas(16) T tile[kTileBytes / sizeof(T)];
     const uint64_t row0 = (uint64_t)blockIdx.x * a.rpb;
     const uint32_t nrows = (uint32_t)(a.rows - row0 < a.rpb ? a.rows - row0 : a.rpb);
-    const uint32_t ne = nrows * a.R;
-    const T* p = src + row0 * a.R;
+    const uint32_t ne = nrows * a.L;
+    const T* p = src + row0 * a.L;
     // pitch == R: the run is copied as it lies, with 16-byte LDS stores; `mis` keeps the 16-byte phase of the global address.  Always
     // for 1- and 2-byte elements (an element-wise scatter would issue 8 or 16 sub-word stores per vector: u8 rows of 100 ran at
     // 1.9 TB/s), and for wider elements whenever rows at that pitch meet at most two to a bank (see tile_pitch); otherwise rows go
     // to a padded pitch element by element, an index division per element.
-    const bool verbatim = a.pitch == a.R;
+    const bool verbatim = a.pitch == a.L;
     const uint32_t mis = verbatim ? (uint32_t)((reinterpret_cast<uintptr_t>(p) & 15) / sizeof(T)) : 0u;
     auto put = [&](uint32_t e, T v) {
         if (verbatim) {
             tile[mis + e] = v;
         } else {
-            const uint32_t r = fd_div(e, a.r_div);
-            tile[r * a.pitch + (e - r * a.R)] = v;
+            const uint32_t r = fd_div(e, a.l_div);
+            tile[r * a.pitch + (e - r * a.L)] = v;
         }
     };
     uint32_t head = (uint32_t)(((16 - (reinterpret_cast<uintptr_t>(p) & 15)) & 15) / sizeof(T));
@@ -440,56 +442,59 @@ __global__ __launch_bounds__(kBlock) void st_rows_tile_kernel(const T* __restric
     // f64 logsumexp reads its rows twice (see below): there the exponentials set the time (rows of 100: 0.49 -> 0.56 of peak); for f32,
     // whose exponential is one instruction, the second round of LDS reads costs more than the rescaling it saves (rows of 256: 0.70 -> 0.67)
     constexpr bool kTwoPass = std::is_same<S, LseState<T>>::value && sizeof(T) == 8;
-    for (uint32_t r0 = 0; r0 < nrows; r0 += groups) {              // every lane runs every trip: the shuffles below need the whole wave
-        const uint32_t r = r0 + g;
+    const uint32_t nout = nrows * a.inner, in = a.inner;
+    for (uint32_t q0 = 0; q0 < nout; q0 += groups) {                // every lane runs every trip: the exchanges below need the whole wave
+        const uint32_t q = q0 + g;
+        const bool live = q < nout;
+        const uint32_t r = in == 1 ? q : fd_div(q, a.inner_div);
+        const uint32_t c = q - r * in;
+        const T* col = tile + mis + (live ? r * a.pitch + c : 0u);  // pitch == L in the verbatim layout; element k of the column at col[k * in]
         S acc;
         acc.init();
-        if (r < nrows) {
-            const T* row = tile + mis + r * a.pitch;              // pitch == R in the verbatim layout
+        if (live) {
             uint32_t k = j;
             if constexpr (std::is_same<S, LseState<T>>::value) {
-                if (a.G == 1) { acc.fold_row(row, a.R); k = a.R; }
+                if (a.G == 1 && in == 1) { acc.fold_row(col, a.R); k = a.R; }
             }
             if constexpr (!kTwoPass) {
                 for (; k + 3 * a.G < a.R; k += 4 * a.G) {
                     T x[4];
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) x[u] = row[k + u * a.G];
+                    for (int u = 0; u < 4; ++u) x[u] = col[(k + u * a.G) * in];
                     acc.template push_block<4>(x, k, a.G);
                 }
-                for (; k < a.R; k += a.G) acc.push(row[k], k);
+                for (; k < a.R; k += a.G) acc.push(col[k * in], k);
             }
         }
         if constexpr (kTwoPass) {
-            // the row lies in LDS: its maximum first (the lanes' maxima, then the group's by a butterfly), then one exponential per
-            // element and no rescaling of running sums (the running form pays one more per four elements and one per lane at the end)
-            if (a.G > 1) {
-                const T* row = tile + mis + r * a.pitch;
+            // the column lies in LDS: its maximum first (the lanes' maxima, then the group's), then one exponential per element and no
+            // rescaling of running sums (the running form pays one more per four elements and one per lane at the end)
+            if (a.G > 1 || in > 1) {
                 T top = -std::numeric_limits<T>::infinity();
-                if (r < nrows) {
+                if (live) {
                     uint32_t k = j;
                     for (; k + 3 * a.G < a.R; k += 4 * a.G) {     // four LDS reads in flight
                         T x[4];
 #pragma unroll
-                        for (int u = 0; u < 4; ++u) x[u] = row[k + u * a.G];
+                        for (int u = 0; u < 4; ++u) x[u] = col[(k + u * a.G) * in];
                         top = m_max(m_max(top, x[0]), m_max(x[1], m_max(x[2], x[3])));
                     }
-                    for (; k < a.R; k += a.G) top = m_max(top, row[k]);
+                    for (; k < a.R; k += a.G) top = m_max(top, col[k * in]);
                 }
                 top = group_all<OpMax>(top, a.G);
                 T sum = (T)0;
                 bool bad = false;
-                if (r < nrows) {
+                if (live) {
                     uint32_t k = j;
                     for (; k + 3 * a.G < a.R; k += 4 * a.G) {
                         T x[4];
 #pragma unroll
-                        for (int u = 0; u < 4; ++u) x[u] = row[k + u * a.G];
+                        for (int u = 0; u < 4; ++u) x[u] = col[(k + u * a.G) * in];
 #pragma unroll
                         for (int u = 0; u < 4; ++u) { sum = sum + S::term(x[u], top); bad |= x[u] != x[u]; }
                     }
                     for (; k < a.R; k += a.G) {
-                        const T x = row[k];
+                        const T x = col[k * in];
                         sum = sum + S::term(x, top);
                         bad |= x != x;
                     }
@@ -502,7 +507,7 @@ __global__ __launch_bounds__(kBlock) void st_rows_tile_kernel(const T* __restric
         } else {
             group_reduce(acc, a.G, j);
         }
-        if (j == 0 && r < nrows) out[row0 + r] = acc.result(flags);
+        if (j == 0 && live) out[(row0 + r) * in + c] = acc.result(flags);
     }
 }
 
@@ -726,7 +731,12 @@ __global__ __launch_bounds__(kBlock) void st_cols_short_kernel(const T* __restri
     if (idx >= nvec_out) return;
     const uint32_t o = fd_div((uint32_t)idx, iv_div);           // nvec_out < 2^31 on this path
     const uint32_t iv = (uint32_t)idx - o * inner_vecs;
-    const T* p = src + (uint64_t)o * R * inner + (uint64_t)iv * VW;
+    // the last vector of a row whose length is not a multiple of VW moves back to the row's last VW columns (VW <= inner here): it
+    // folds `skip` columns of its neighbour a second time and does not write them
+    const uint64_t col0 = (uint64_t)iv * VW;
+    const uint64_t col = inner - col0 < (uint64_t)VW ? inner - VW : col0;
+    const uint32_t skip = (uint32_t)(col0 - col);
+    const T* p = src + (uint64_t)o * R * inner + col;
     S acc[VW];
 #pragma unroll
     for (int j = 0; j < VW; ++j) acc[j].init();
@@ -754,9 +764,10 @@ __global__ __launch_bounds__(kBlock) void st_cols_short_kernel(const T* __restri
 #pragma unroll
         for (int j = 0; j < VW; ++j) acc[j].push(x.e[j], k);
     }
-    typename S::Out* q = out + (uint64_t)o * inner + (uint64_t)iv * VW;
+    typename S::Out* q = out + (uint64_t)o * inner + col;
 #pragma unroll
-    for (int j = 0; j < VW; ++j) q[j] = acc[j].result(flags);
+    for (int j = 0; j < VW; ++j)
+        if ((uint32_t)j >= skip) q[j] = acc[j].result(flags);
 }
 
 // ---- second stage -------------------------------------------------------------------------------------------------------
@@ -839,6 +850,28 @@ int32_t merge_cols(rt_ctx* ctx, const S* part, typename S::Out* out, uint64_t no
     return RT_OK;
 }
 
+// the LDS-tiled kernel over `rows` runs of R * inner elements (inner == 1: short rows; else small slabs with a few columns)
+template <class S, class T>
+int32_t tile_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t rows, uint64_t R, uint64_t inner, int flags) {
+    TileArgs a;
+    a.rows = rows;
+    a.R = (uint32_t)R;
+    a.inner = (uint32_t)inner;
+    a.L = (uint32_t)(R * inner);
+    a.pitch = rt_tile_pitch(a.L, (uint32_t)sizeof(T));
+    a.rpb = (uint32_t)(kTileBytes / sizeof(T) - (a.pitch == a.L ? 16 / sizeof(T) : 0)) / a.pitch;
+    a.l_div = make_fastdiv(a.L);
+    a.inner_div = make_fastdiv(a.inner);
+    uint32_t g = 1;                                               // lanes per output: fill the block, at most one wave, at most R
+    while (g < 64 && (uint64_t)g * 2 * a.rpb * inner <= (uint64_t)kBlock && g * 2 <= a.R) g <<= 1;
+    a.G = g;
+    const uint64_t blocks = (rows + a.rpb - 1) / a.rpb;
+    if (blocks >= (1ull << 31)) return too_many();
+    hipLaunchKernelGGL((st_rows_tile_kernel<S, T>), dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream, src, out, a, flags);
+    RT_HIP(hipGetLastError());
+    return RT_OK;
+}
+
 template <class S, class T>
 int32_t rows_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t rows, uint64_t R, int flags) {
     hipStream_t s = ctx->stream;
@@ -857,20 +890,7 @@ int32_t rows_plan(rt_ctx* ctx, const T* src, typename S::Out* out, uint64_t rows
         }
     }
     if (R <= kTileMaxR && R * sizeof(T) < 2048) {                // from 2 KiB per row a wave per row is faster (f32 rows of 1024: 0.194 / 0.157 ms)
-        TileArgs a;
-        a.rows = rows;
-        a.R = (uint32_t)R;
-        a.pitch = rt_tile_pitch(a.R, (uint32_t)sizeof(T));
-        a.rpb = (uint32_t)(kTileBytes / sizeof(T) - (a.pitch == a.R ? 16 / sizeof(T) : 0)) / a.pitch;
-        a.r_div = make_fastdiv(a.R);
-        uint32_t g = 1;                                           // lanes per row: fill the block, at most one wave, at most R
-        while (g < 64 && (uint64_t)g * 2 * a.rpb <= (uint64_t)kBlock && g * 2 <= a.R) g <<= 1;
-        a.G = g;
-        const uint64_t blocks = (rows + a.rpb - 1) / a.rpb;
-        if (blocks >= (1ull << 31)) return too_many();
-        hipLaunchKernelGGL((st_rows_tile_kernel<S, T>), dim3((unsigned)blocks), dim3(kBlock), 0, s, src, out, a, flags);
-        RT_HIP(hipGetLastError());
-        return RT_OK;
+        return tile_plan<S, T>(ctx, src, out, rows, R, 1, flags);
     }
     const uint64_t want = (uint64_t)ctx->num_cus * 8;
     if (R * sizeof(T) < 16384 && rows >= want / 2) {             // a block per row from 16 KiB on, as for the plain reductions
@@ -1036,11 +1056,14 @@ int32_t plan(rt_ctx* ctx, const void* src_v, void* out_v, uint64_t outer, uint64
     }
     if (inner == 1) return rows_plan<S, T>(ctx, src, out, outer, R, flags);
     constexpr int N = 16 / sizeof(T);
+    // small slabs with a few columns: through LDS (see TileArgs)
+    if (inner <= 64 && R >= 2 && R * inner * sizeof(T) <= 8192 && outer >= 1024) return tile_plan<S, T>(ctx, src, out, outer, R, inner, flags);
     // short reduced axis: a lane per output vector (the plain reductions' rule, but only up to 16 rows: variance over the middle axis of
-    // (32768, 32, 256) f32 0.77 of peak on the column kernel, 0.74 here)
-    if ((R <= 16 || (R <= 256 && R * inner * sizeof(T) <= 8192)) && inner <= 1024) {
-        const bool v = inner % N == 0;                                          // rows may start at any element
-        const uint64_t ivecs = v ? inner / N : inner;
+    // (32768, 32, 256) f32 0.77 of peak on the column kernel, 0.74 here; up to 32 rows for slabs within 24 KiB: (61440, 17, 257) 0.44 there);
+    // an axis of up to four elements with any inner
+    if ((R <= 16 || (R <= 32 && R * inner * sizeof(T) <= 24576) || (R <= 256 && R * inner * sizeof(T) <= 8192)) && (inner <= 1024 || R <= 4)) {
+        const bool v = inner >= (uint64_t)N;                                    // rows may start at any element and have any length
+        const uint64_t ivecs = v ? (inner + N - 1) / N : inner;
         if (ivecs < (1ull << 31) && outer * ivecs < (1ull << 31)) {
             const uint64_t nvec_out = outer * ivecs;
             const uint64_t blocks = (nvec_out + kBlock - 1) / kBlock;

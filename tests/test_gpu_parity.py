@@ -1528,6 +1528,10 @@ def test_reduction_shapes_short_rows_narrow_columns_short_axis(hip, dtype):
     for outer, R, inner in ((2, 300, 257), (1, 5003, 1001), (3, 100, 129), (1, 2000, 1030), (1, 70, 4099), (2, 40, 131)):
         for offset in (0, 1, 3):
             _check_reduce(hip, dtype, outer, R, inner, rng, offset=offset)
+    # many small slabs with a few columns (staged through LDS, a group of lanes per column); a short axis over ragged rows
+    for outer, R, inner in ((3000, 33, 2), (5000, 17, 5), (2000, 100, 3), (1500, 8, 32), (1100, 33, 60), (4000, 2, 2), (1024, 300, 2), (1030, 1000, 2), (1200, 5, 17),
+                            (500, 3, 257), (100, 1, 4097), (50, 2, 4097), (700, 17, 257), (40, 3, 30001)):
+        _check_reduce(hip, dtype, outer, R, inner, rng, offset=int(rng.integers(0, 5)))
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f64"])
@@ -1541,7 +1545,8 @@ def test_float_max_min_keep_the_first_zero_in_every_kernel_shape(hip, dtype):
     rng = np.random.default_rng(zlib.crc32(b"zero-sign" + dtype.encode()))
     shapes = [(4, 100000, 1), (3000, 5000, 1), (1, 1 << 21, 1), (5000, 600, 1), (3000, 2000, 1), (20000, 100, 1), (20000, 10, 1), (40000, 64, 1),
               (8192, 256, 1), (70, 33, 1), (1, 5000, 512), (8, 300, 1024), (1, 4096, 4096), (2, 3000, 1001), (1, 100000, 3), (4, 5000, 100),
-              (5000, 16, 64), (100, 8, 1000), (1, 70001, 17), (300, 200, 8), (1, 70000, 128), (1, 65536, 256), (1, 30000, 1000), (1, 70001, 128)]
+              (5000, 16, 64), (100, 8, 1000), (1, 70001, 17), (300, 200, 8), (1, 70000, 128), (1, 65536, 256), (1, 30000, 1000), (1, 70001, 128),
+              (3000, 33, 2), (5000, 17, 5), (2000, 100, 3), (1100, 33, 60), (1024, 300, 2), (500, 3, 257), (50, 2, 4097)]
     for outer, R, inner in shapes:
         n = outer * R * inner
         mag = np.abs(rng.normal(size=n)).astype(npd) + npd(0.5)
@@ -1629,6 +1634,9 @@ STAT_SHAPES = ([(rows, R, 1) for R in (1, 2, 3, 7, 8, 31, 32, 33, 64, 65, 100, 2
                + [(outer, R, inner) for inner in (2, 3, 5, 17, 63, 64, 100, 128) for R, outer in ((64, 3), (1000, 1), (5003, 2), (70001, 1))]
                + [(outer, R, inner) for R in (1, 2, 5, 16, 33) for inner, outer in ((2, 1000), (3, 1), (64, 50), (1028, 2))]
                + [(1, 65536, 256), (1, 30000, 1000), (1, 8192, 2048)]                  # rows regrouped before the column kernel reads them
+               # many small slabs with a few columns (staged through LDS); a short axis over ragged rows (vectors that overlap at a row's end)
+               + [(3000, 33, 2), (5000, 17, 5), (2000, 100, 3), (1500, 8, 32), (1100, 33, 60), (4000, 2, 2), (1024, 300, 2), (1030, 1000, 2), (1200, 5, 17)]
+               + [(500, 3, 257), (100, 1, 4097), (50, 2, 4097), (700, 17, 257), (40, 3, 30001)]
                + [(1, 300, 5000), (2, 4000, 260), (1, 70, 2052), (2, 300, 257), (1, 5003, 1001), (3, 100, 129), (1, 2000, 1030), (1, 70, 4099), (2, 40, 131)])
 
 
@@ -1692,7 +1700,8 @@ def test_logsumexp_special_values_in_every_kernel_shape(hip, dtype):
     npd = np.dtype(cpu.NP_DTYPE[code]).type
     rng = np.random.default_rng(zlib.crc32(b"lse-special" + dtype.encode()))
     shapes = [(4, 100000, 1), (3000, 5000, 1), (1, 1 << 20, 1), (5000, 600, 1), (20000, 100, 1), (20000, 10, 1), (40000, 64, 1), (8192, 256, 1),
-              (40000, 4, 1), (70, 33, 1), (1, 5000, 512), (8, 300, 1024), (1, 4096, 2048), (1, 100000, 3), (4, 5000, 100), (5000, 16, 64), (300, 200, 8)]
+              (40000, 4, 1), (70, 33, 1), (1, 5000, 512), (8, 300, 1024), (1, 4096, 2048), (1, 100000, 3), (4, 5000, 100), (5000, 16, 64), (300, 200, 8),
+              (3000, 33, 2), (5000, 17, 5), (2000, 100, 3), (1100, 33, 60), (1024, 300, 2), (500, 3, 257), (50, 2, 4097)]
     for outer, R, inner in shapes:
         x = (rng.normal(size=(outer, R, inner)) * 3).astype(npd)
         x[rng.random(size=x.shape) < 0.02] -= npd(800.0)
