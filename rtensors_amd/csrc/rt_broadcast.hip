@@ -597,7 +597,14 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
     };
     bool flat_good = count >= (uint64_t)N && row_major_run(2) && (reinterpret_cast<uintptr_t>(d + dsc.offset[2]) & 15) == 0;
     for (int o = 0; o < (OP == kOpCopy ? 1 : 2) && flat_good; ++o) flat_good = row_major_run(o) || repeated_row_or_element(o);
-    if (rank >= 1 && !prefer_flat && count < (1ull << 31) && dsc.stride[2][rank - 1] == 1 && dsc.shape[rank - 1] >= 2 * N &&
+    // Short rows under a short loop dim leave a block of the row kernel next to nothing (out (19737, 100, 2, 17) = (19737, 1, 2, 17) +
+    // (1, 100, 1, 17): two rows of 17 per block, 0.04 of peak): when dst is one aligned run, the flat kernel, one dst vector per lane
+    // with the inputs gathered by index, does far better whatever the inputs look like.  The same for rows of less than 128 bytes under
+    // any loop dim, of which a lane of the row kernel gets a ragged piece ((963, 4097, 1, 17) + (963, 1, 1, 17) f32: 0.25 -> 0.70 of peak;
+    // from 128 bytes on the row kernel wins: rows of 100 f32 0.64 against 0.27).
+    const bool tiny_blocks = rank >= 2 && row_major_run(2) && (reinterpret_cast<uintptr_t>(d + dsc.offset[2]) & 15) == 0 && count >= (uint64_t)N &&
+                             ((uint64_t)dsc.shape[rank - 1] * (uint64_t)dsc.shape[rank - 2] * sizeof(T) < 2048 || (uint64_t)dsc.shape[rank - 1] * sizeof(T) < 128);
+    if (rank >= 1 && !prefer_flat && !tiny_blocks && count < (1ull << 31) && dsc.stride[2][rank - 1] == 1 && dsc.shape[rank - 1] >= 2 * N &&
         (rows_aligned(2, d) || !flat_good)) {
         RowArgs a;
         memset(&a, 0, sizeof(a));

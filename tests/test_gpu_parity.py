@@ -1534,6 +1534,40 @@ def test_reduction_shapes_short_rows_narrow_columns_short_axis(hip, dtype):
         _check_reduce(hip, dtype, outer, R, inner, rng, offset=int(rng.integers(0, 5)))
 
 
+@pytest.mark.parametrize("dtype", ["f32", "i32", "u8", "f64"])
+def test_broadcast_short_rows_under_short_loop_dims(hip, dtype):
+    """Outputs whose rows are a few elements long, with operands that repeat along different dims: the shapes on which a block of
+    the row kernel would be left with a couple of short rows, and which the flat kernel takes instead (dst one aligned run, inputs
+    gathered by index).  Against numpy's broadcasting, bit for bit, for add, mul and sub in either operand order."""
+    from rtensors_amd import hip as H
+    code = cpu.DTYPE_BY_NAME[dtype]
+    npd = cpu.NP_DTYPE[code]
+    rng = np.random.default_rng(zlib.crc32(b"short-rows" + dtype.encode()))
+    pairs = [((50, 1, 2, 17), (1, 7, 1, 17)), ((300, 5, 3, 3), (300, 1, 3, 3)), ((40, 100, 1, 17), (40, 100, 3, 1)), ((200, 2, 1, 17), (200, 1, 1, 17)),
+             ((9, 257, 1, 17), (9, 1, 1, 17)), ((33, 17, 17, 2), (33, 1, 17, 2)), ((60, 3, 100, 1), (1, 1, 1, 17)), ((700, 1, 1, 17), (700, 1, 17, 1)),
+             ((1000, 3, 2, 5), (1000, 1, 2, 5)), ((5, 1, 257, 3), (1, 11, 1, 3)), ((123, 1, 5, 31), (1, 4, 1, 31)), ((64, 2, 2, 8), (64, 1, 2, 1))]
+    for sa, sb in pairs:
+        a = rand_values(dtype, int(np.prod(sa)), rng, -50, 50).reshape(sa)
+        b = rand_values(dtype, int(np.prod(sb)), rng, -50, 50).reshape(sb)
+        out_shape = [max(x, y) for x, y in zip(sa, sb)]
+        n = int(np.prod(out_shape))
+
+        def strides(shape):
+            st, acc = [], 1
+            for d, od in zip(reversed(shape), reversed(out_shape)):
+                st.append(0 if d == 1 and od != 1 else acc)
+                acc *= d
+            return list(reversed(st))
+        ga, gb, gd = hip.alloc_from_slice(code, a.reshape(-1)), hip.alloc_from_slice(code, b.reshape(-1)), hip.alloc(code, n)
+        dst_meta = (0, out_shape, strides(out_shape))
+        for op, fn in (("add", np.add), ("mul", np.multiply), ("sub", np.subtract)):
+            for (x, gx, sx), (y, gy, sy) in (((a, ga, sa), (b, gb, sb)), ((b, gb, sb), (a, ga, sa))):
+                hip.broadcast((gx, (0, out_shape, strides(sx))), (gy, (0, out_shape, strides(sy))), (gd, dst_meta), op)
+                with np.errstate(all="ignore"):
+                    want = fn(x, y).astype(npd)
+                assert hip.dump(gd).tobytes() == np.ascontiguousarray(want).tobytes(), (dtype, op, sx, sy)
+
+
 @pytest.mark.parametrize("dtype", ["f32", "f64"])
 def test_float_max_min_keep_the_first_zero_in_every_kernel_shape(hip, dtype):
     """max over values <= 0 and min over values >= 0 whose zeros come in both signs, in either order, or in one sign only: the
