@@ -783,7 +783,10 @@ int32_t launch_view(rt_ctx* ctx, T* base, const NdDesc& d, uint64_t count, F f) 
     constexpr int64_t N = 16 / sizeof(T);
     // rows form: unit-stride inner dim of at least two vectors; the rows may start at any element (`m[:, 1:]` of a 8192 x 32768
     // f32 matrix: relu in place 0.57 ms element by element, 0.36 ms with unaligned vectors)
-    const bool rows_ok = d.stride[0][d.rank - 1] == 1 && d.shape[d.rank - 1] >= 2 * N;
+    // (not when a block would be left with a couple of short rows -- rows of 17 under a loop dim of 3, relu on m[..., :17] of
+    // (310689, 3, 3, 18) f32: 0.16 of peak; the element kernel below takes those)
+    const bool rows_ok = d.stride[0][d.rank - 1] == 1 && d.shape[d.rank - 1] >= 2 * N &&
+                         (uint64_t)d.shape[d.rank - 1] * (uint64_t)d.shape[d.rank - 2] * sizeof(T) >= 2048;
     if (rows_ok) {
         RowsArgs r;
         memset(&r, 0, sizeof(r));
