@@ -182,6 +182,36 @@ class Workloads:
     def var_inner3(self): return self._stat_shape("var", 1, (1 << 28) // 3, 3)                # per-channel statistics of pixels
     def var_mid64(self): return self._stat_shape("var", 65536, 64, 64)
 
+    # ---- shapes off the configs that have work forms of their own ------------------------------------------------------------
+    def _shape(self, op, dtype_name, outer, R, inner):
+        """`op` over the middle axis of a (outer, R, inner) view of 1 GiB of normal(0, 1) data."""
+        H = self.H
+        code, es = (H.F64, 8) if dtype_name == "f64" else (H.F32, 4)
+        a = self._gen("gib" + dtype_name, code, (1 << 30) // es, "normal", 1, 0)
+        d = self._out("gibout" + dtype_name, code, (1 << 30) // es // 2)
+        shape, strides = [outer, R, inner], [R * inner, inner, 1]
+        return (lambda: self.hip.apply_reduce_contiguous_nd((a, (0, shape, strides)), d, 1, op)), (outer * R * inner + outer * inner) * es, outer * R * inner
+
+    def lse_f64_rows32768(self): return self._shape("logsumexp", "f64", 4096, 32768, 1)       # f64 logsumexp: the exponential written for it
+    def var_rows512(self): return self._shape("var", "f32", 1 << 19, 512, 1)                  # rows of 2 KiB: 16 lanes per row
+    def var_f64_rows256(self): return self._shape("var", "f64", 1 << 19, 256, 1)
+    def var_mid4(self): return self._shape("var", "f32", 1 << 20, 4, 64)                      # a short middle axis: a lane per output vector
+    def sum_slab33x2(self): return self._shape("sum", "f32", (1 << 28) // 66, 33, 2)          # many small slabs with two columns: through LDS
+    def lse_slab300x2(self): return self._shape("logsumexp", "f32", (1 << 28) // 600, 300, 2)
+    def max_cols128(self): return self._shape("max", "f32", 1, 1 << 21, 128)                  # float max over regrouped rows
+    def var_cols50176(self): return self._shape("var", "f32", 1, 5349, 50176)                 # 196 column tiles: the split by rounds of blocks
+
+    def bcast_rows17(self):
+        """out (19737, 100, 2, 17) = (19737, 1, 2, 17) + (1, 100, 1, 17): rows of 17 elements under a loop dim of 2 (the flat kernel)."""
+        H = self.H
+        o = [19737, 100, 2, 17]
+        n = o[0] * o[1] * o[2] * o[3]
+        a = self._gen("c2a", H.F32, 1 << 28, "normal", 1, 0)
+        b = self._gen("c2b", H.F32, 1 << 28, "normal", 1, 1)
+        d = self._out("c2cf32", H.F32, 1 << 28)
+        ls, rs, ds = [2 * 17, 0, 17, 1], [0, 17, 0, 1], [100 * 2 * 17, 2 * 17, 17, 1]
+        return (lambda: self.hip.broadcast((a, (0, o, ls)), (b, (0, o, rs)), (d, (0, o, ds)), "add")), (19737 * 34 + 1700 + n) * 4, n
+
     def c4_sum_all(self):
         t = self._c4("f32")
         out = self._out("c4oall", t.dtype, 1)

@@ -430,7 +430,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(const T* __restrict
 // 0.69 -> 0.76 of peak, variance 0.71 -> 0.77, sum 0.71 -> 0.76; rows of 100: 0.67 -> 0.73, 0.73 -> 0.79, 0.73 -> 0.81; 16, 20, 22 and
 // 26 KiB lie between, 48 KiB (three blocks) loses 10 %.
 constexpr uint32_t kRowsTileBytes = 24576;
-// The same kernel takes small slabs with a few columns ((outer, R, inner) with inner <= 64 and R * inner elements in at most 8 KiB):
+// The same kernel takes small slabs with a few columns ((outer, R, inner) with inner <= 128 and R * inner elements in at most 8 KiB):
 // a "row" of the tile is then the slab of one outer index, L = R * inner elements, and a group of lanes folds one of its columns,
 // elements c, c + inner, ...  (A lane per output read such slabs from memory with a stride of one slab between lanes: 1 GiB f32
 // summed over the middle axis of (2033601, 33, 2) ran at 0.11 of peak.)
@@ -1020,11 +1020,16 @@ int32_t reduce_typed(rt_ctx* ctx, const T* src, T* out, uint64_t outer, uint64_t
     // gave 0.3-2.3, lanes along a narrow inner 0.2-1.2.
     // short reduced axis: a lane per output vector.  Also for slabs of at most 8 KiB with up to 256 rows, which leave a block of the
     // narrow-column kernel too little to do ((262144, 64, 16) f32: 0.35 -> 0.61 of peak; from 16 KiB on the narrow kernel wins)
-    // small slabs with a few columns: through LDS (see RowsTileArgs)
-    // (up to 8 KiB: from there on a block per slab streams them faster, sum over (67108, 2000, 2) f32 0.82 of peak against 0.72 here)
-    if (inner <= 64 && R >= 2 && R * inner * sizeof(T) <= 8192 && outer >= 1024) return tile_launch<OP, T>(ctx, src, out, outer, R, inner, R);
-    // an axis of up to four elements is an elementwise pass over `inner` lanes wide: any inner
-    if ((R <= 32 || (R <= 256 && R * inner * sizeof(T) <= 8192)) && (inner <= 1024 || R <= 4)) {
+    // A short reduced axis goes to a lane per output vector, many small slabs with a few columns through LDS (see RowsTileArgs).  Where
+    // both apply, the lane-per-vector form when the rows of a slab are whole 128-byte lines, or at most four of them of 32 elements
+    // and more (f32 sum over (.., 4, 64): 0.85 of peak against 0.82; over (.., 8, 12): 0.41 against 0.79).  Slabs of more than 8 KiB are
+    // streamed by a block each (sum over (67108, 2000, 2) f32: 0.82 against 0.72 through LDS).
+    // An axis of up to four elements is an elementwise pass over `inner` lanes wide: any inner.
+    const bool short_ok = (R <= 32 || (R <= 256 && R * inner * sizeof(T) <= 8192)) && (inner <= 1024 || R <= 4);
+    const bool slab_ok = inner <= 128 && R >= 2 && R * inner * sizeof(T) <= 8192 && outer >= 1024;
+    const bool prefer_short = short_ok && ((inner * sizeof(T)) % 128 == 0 || (R <= 4 && inner >= 32));
+    if (slab_ok && !prefer_short) return tile_launch<OP, T>(ctx, src, out, outer, R, inner, R);
+    if (short_ok) {
         const bool v = inner >= (uint64_t)N;                                    // rows may start at any element and have any length
         const uint64_t ivecs = v ? (inner + N - 1) / N : inner;
         if (ivecs < (1ull << 31) && outer * ivecs < (1ull << 31)) {

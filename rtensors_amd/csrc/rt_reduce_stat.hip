@@ -1066,13 +1066,18 @@ int32_t plan(rt_ctx* ctx, const void* src_v, void* out_v, uint64_t outer, uint64
     if (R == 1 && outer > 1) { inner *= outer; outer = 1; }       // an axis of one element: one run of outer * inner independent outputs
     if (inner == 1) return rows_plan<S, T>(ctx, src, out, outer, R, flags);
     constexpr int N = 16 / sizeof(T);
-    // small slabs with a few columns: through LDS (see TileArgs); up to a whole tile per slab (variance over (89478, 1000, 3) f32: 0.28 of
-    // peak with a block streaming each slab, 0.64 here)
-    if (inner <= 128 && R >= 2 && R * inner * sizeof(T) <= kTileBytes - 64 && outer >= 1024) return tile_plan<S, T>(ctx, src, out, outer, R, inner, flags);
-    // short reduced axis: a lane per output vector (the plain reductions' rule, but only up to 16 rows: variance over the middle axis of
-    // (32768, 32, 256) f32 0.77 of peak on the column kernel, 0.74 here; up to 32 rows for slabs within 24 KiB: (61440, 17, 257) 0.44 there);
-    // an axis of up to four elements with any inner
-    if ((R <= 16 || (R <= 32 && R * inner * sizeof(T) <= 24576) || (R <= 256 && R * inner * sizeof(T) <= 8192)) && (inner <= 1024 || R <= 4)) {
+    // A short reduced axis goes to a lane per output vector, many small slabs with a few columns through LDS (see TileArgs) -- slabs of
+    // up to a whole tile (variance over (89478, 1000, 3) f32: 0.28 of peak with a block streaming each slab, 0.69 through LDS).  Where both
+    // apply, the lane-per-vector form when the rows of a slab are whole 128-byte lines, or at most four of them of 32 elements and more
+    // (f32 variance over (.., 4, 64): 0.85 against 0.68; over (.., 8, 12): 0.42 against 0.74).
+    // The lane-per-vector form: up to 16 rows (variance over the middle axis of (32768, 32, 256) f32 0.77 of peak on the column kernel,
+    // 0.74 here), up to 32 for slabs within 24 KiB ((61440, 17, 257): 0.44 on the column kernel), up to 256 within 8 KiB; an axis of up to
+    // four elements with any inner.
+    const bool short_ok = (R <= 16 || (R <= 32 && R * inner * sizeof(T) <= 24576) || (R <= 256 && R * inner * sizeof(T) <= 8192)) && (inner <= 1024 || R <= 4);
+    const bool slab_ok = inner <= 128 && R >= 2 && R * inner * sizeof(T) <= kTileBytes - 64 && outer >= 1024;
+    const bool prefer_short = short_ok && ((inner * sizeof(T)) % 128 == 0 || (R <= 4 && inner >= 32));
+    if (slab_ok && !prefer_short) return tile_plan<S, T>(ctx, src, out, outer, R, inner, flags);
+    if (short_ok) {
         const bool v = inner >= (uint64_t)N;                                    // rows may start at any element and have any length
         const uint64_t ivecs = v ? (inner + N - 1) / N : inner;
         if (ivecs < (1ull << 31) && outer * ivecs < (1ull << 31)) {
