@@ -439,6 +439,26 @@ class Workloads:
         c = self._out("c2cf32", H.F32, n * n)
         return (lambda: self.hip.gather(a, (0, [n, n], [1, n]), c)), 2 * n * n * 4, n * n
 
+    def gather_rows42(self):
+        """Row-major copy of a (64, 3, 2, 4096, 42) f32 view with strides (1, 262144, 786432, 64, 1572864): dst rows of 42 elements,
+        src unit-stride along the outermost dim (the N-d tile copy through LDS)."""
+        H = self.H
+        shape, strides = [64, 3, 2, 4096, 42], [1, 262144, 786432, 64, 1572864]
+        n = 64 * 3 * 2 * 4096 * 42
+        a = self._gen("c2a", H.F32, 1 << 28, "normal", 1, 0)
+        c = self._out("c2cf32", H.F32, 1 << 28)
+        return (lambda: self.hip.gather(a, (0, shape, strides), c)), 2 * n * 4, n
+
+    def gather_unit7(self):
+        """Row-major copy of a (7, 3300, 2905) f32 view with strides (1, 7, 23100): a (2905, 3300, 7) tensor with its axes reversed,
+        whose unit-stride dim has 7 elements."""
+        H = self.H
+        shape, strides = [7, 3300, 2905], [1, 7, 23100]
+        n = 7 * 3300 * 2905
+        a = self._gen("c2a", H.F32, 1 << 28, "normal", 1, 0)
+        c = self._out("c2cf32", H.F32, 1 << 28)
+        return (lambda: self.hip.gather(a, (0, shape, strides), c)), 2 * n * 4, n
+
     def c1_add(self):
         H = self.H
         a = self._gen("c1a", H.F32, 4096, "uniform", 0, 0); b = self._gen("c1b", H.F32, 4096, "uniform", 0, 1)

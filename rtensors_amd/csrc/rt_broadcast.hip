@@ -526,10 +526,12 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
         }
     }
 
-    // (2a) interleaved -> planar copy, and the tile kernel for one "transposed" input (rt_broadcast_tile.hip)
+    // (2a) copies only: interleaved -> planar, and views whose contiguous pieces are short on one side or both (rt_permute.hip);
+    // then the tile kernel for one "transposed" input (rt_broadcast_tile.hip)
     if constexpr (OP == kOpCopy && std::is_integral<T>::value && sizeof(T) <= 8) {
         int32_t status = RT_OK;
         if (planar_copy_try<T>(ctx, dsc, count, l, d, &status)) return status;
+        if (permute_try<T>(ctx, dsc, count, l, d, &status)) return status;
     }
     {
         int32_t status = RT_OK;

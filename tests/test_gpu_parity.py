@@ -1111,6 +1111,47 @@ def test_gather_transposed_views(hip, dtype):
                 assert gv.contiguous().dump().tobytes() == ov.to_numpy().tobytes(), (dtype, shape, perm, variant)
 
 
+@pytest.mark.parametrize("dtype", ["f32", "u8", "i16", "f64", "i64"])
+def test_gather_views_with_short_contiguous_pieces(hip, dtype):
+    """Row-major copy of views whose contiguous pieces are short in src, in dst or in both (the N-d tile copy through LDS): permuted
+    parents with dims of 2 .. 7 elements next to long ones, dst rows of a few elements, one dim reversed, stepped or cut so that the
+    edge tiles are ragged along several dims at once, vector and single-element loads and stores.  Against numpy's own copy of the
+    same view, bit for bit."""
+    rng = np.random.default_rng(41)
+    npd = cpu.NP_DTYPE[cpu.DTYPE_BY_NAME[dtype]]
+    dims = (2, 3, 7, 16, 33, 42, 64, 100, 129, 256)
+    fixed = [((42, 96, 2, 3, 64), (4, 2, 3, 1, 0)),          # dst rows of 42, src unit-stride along a dim of 64 elsewhere
+             ((130, 33, 100, 7), (3, 2, 1, 0)),              # unit-stride dim of 7
+             ((2995, 16, 7, 2), (3, 1, 2, 0)),               # the fastest 224 elements of src permuted among themselves
+             ((20971, 16, 2), (1, 0, 2)),                    # rows of 2 regrouped
+             ((64, 4096, 16), (0, 2, 1)), ((300, 300), (1, 0)), ((1000, 7), (1, 0)), ((7, 1000), (1, 0)), ((33, 5, 16, 9), (2, 0, 3, 1))]
+    cases = [(shape, perm, 0) for shape, perm in fixed]
+    for trial in range(40):
+        rank = int(rng.choice((3, 3, 4, 4, 5)))
+        while True:
+            shape = tuple(int(rng.choice(dims)) for _ in range(rank))
+            if 20000 <= int(np.prod(shape)) <= 400000:
+                break
+        perm = list(range(rank))
+        while perm == sorted(perm):
+            rng.shuffle(perm)
+        cases.append((shape, tuple(int(x) for x in perm), int(rng.integers(0, 4))))
+    for shape, perm, variant in cases:
+        vals = rand_values(dtype, int(np.prod(shape)), rng)
+        g = G(hip, dtype, vals, list(shape)).permute(list(perm))
+        want = vals.reshape(shape).transpose(perm)
+        ax = int(rng.integers(0, len(shape)))
+        if variant == 1:                                     # one dim reversed
+            g, want = g.slice(ax, Slice(None, None, -1)), np.flip(want, ax)
+        elif variant == 2:                                   # every second or third index of one dim
+            k = int(rng.choice((2, 3)))
+            g, want = g.slice(ax, Slice(None, None, k)), want[(slice(None),) * ax + (slice(None, None, k),)]
+        elif variant == 3 and want.shape[ax] > 3:            # a corner of the parent
+            g, want = g.slice(ax, Slice(1, want.shape[ax] - 2, 1)), want[(slice(None),) * ax + (slice(1, want.shape[ax] - 2),)]
+        got = g.contiguous().dump()
+        assert got.dtype == npd and got.tobytes() == np.ascontiguousarray(want).tobytes(), (dtype, shape, perm, variant, ax)
+
+
 @pytest.mark.parametrize("dtype", ["f32", "u8", "i16", "f64"])
 def test_gather_interleaved_to_planar(hip, dtype):
     """(.., M, C) -> (.., C, M) with a short C (pixels to planes): the LDS-staged planar copy, with odd plane lengths, a batch
