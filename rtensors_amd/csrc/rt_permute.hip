@@ -68,6 +68,7 @@ bool permute_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* src, T
     rt_permute_set_widths(&a, v, w);
     dim3 grid((unsigned)blocks), blk(kPBlock);
     const uint32_t lds = rt_permute_lds_bytes(a, (uint32_t)sizeof(T));
+    if (lds > 64u * 1024u) return false;                           // (the plan stays below 52 KiB: a 40 KiB tile and 12 KiB of tables)
     auto go = [&](auto wc) {
         constexpr int W = decltype(wc)::value;
         if (v == N) hipLaunchKernelGGL((permute_tile_kernel<T, W, (int)N>), grid, blk, lds, ctx->stream, sp, dp, a);
