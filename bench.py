@@ -449,6 +449,18 @@ class Workloads:
         c = self._out("c2cf32", H.F32, 1 << 28)
         return (lambda: self.hip.gather(a, (0, shape, strides), c)), 2 * n * 4, n
 
+    def add_perm_rows42(self):
+        """c = a + v with v the (64, 3, 2, 4096, 42) view of gather_rows42 and a, c row-major: the permuted operand goes through a row-major
+        temporary (the N-d tile copy, then the contiguous add).  Algorithmic bytes are the three tensors once."""
+        H = self.H
+        shape, strides = [64, 3, 2, 4096, 42], [1, 262144, 786432, 64, 1572864]
+        n = 64 * 3 * 2 * 4096 * 42
+        rm = [3 * 2 * 4096 * 42, 2 * 4096 * 42, 4096 * 42, 42, 1]
+        a = self._gen("c2a", H.F32, 1 << 28, "normal", 1, 0)
+        b = self._gen("c2b", H.F32, 1 << 28, "normal", 1, 1)
+        c = self._out("c2cf32", H.F32, 1 << 28)
+        return (lambda: self.hip.broadcast((a, (0, shape, rm)), (b, (0, shape, strides)), (c, (0, shape, rm)), "add")), 3 * n * 4, n
+
     def gather_unit7(self):
         """Row-major copy of a (7, 3300, 2905) f32 view with strides (1, 7, 23100): a (2905, 3300, 7) tensor with its axes reversed,
         whose unit-stride dim has 7 elements."""

@@ -526,6 +526,71 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
         }
     }
 
+    // (1b) an input that is a permuted view with short contiguous pieces -- it steps by 64 bytes or more along dst's inner dim, is
+    // unit-stride along some other dim, and the transposing kernels below do not fit it (dst rows or that unit-stride dim too
+    // short): read along dst's rows it costs a cache line per element (f32 `a + b.permute(..)` over 256 MiB operands: median 0.27
+    // of peak over 54 such views, the lowest tenth 0.08).  It is first copied into a row-major temporary by the N-d tile copy
+    // (rt_permute.hip), then the op runs on the temporary: two more passes over that operand, 0.37 - 0.48 of peak on the same views.
+    // The temporary comes from the context's block cache and goes back to it; all work is on the context's stream.
+    if constexpr (OP != kOpCopy && sizeof(T) <= 8) {
+        auto short_pieces = [&](int o) {
+            const int64_t is1 = dsc.stride[o][rank - 1], mag1 = is1 < 0 ? -is1 : is1;
+            if (mag1 <= 1 || (uint64_t)mag1 * sizeof(T) < 64) return false;
+            bool unit_dim = false, transposable = false;
+            uint64_t inside = 1;                                       // dst elements per index of the innermost unit-stride dim
+            for (int k = 0; k < rank; ++k) {
+                if (dsc.stride[o][k] == 0) return false;               // a repeated dim: the temporary would hold every repeat
+                const bool unit = dsc.stride[o][k] == 1 || dsc.stride[o][k] == -1;
+                unit_dim = unit_dim || unit;
+                transposable = transposable || (unit && k < rank - 1 && dsc.shape[k] >= 16);
+                inside = unit ? 1 : inside * (uint64_t)dsc.shape[k];
+            }
+            // With fewer than 32 dst elements inside the unit-stride dim (dst rows of 16 down a column of 4096), the rows that use one
+            // cache line of the input follow each other closely and the row kernel's gathers hit in cache: 0.65 - 0.86 of peak there
+            // against 0.48 - 0.50 in two passes; from 33 on the two passes win (0.38 against 0.46 and further apart).
+            if (!unit_dim || inside < 32) return false;
+            // (the transposing kernels take dst rows from a quarter of their tile's columns on)
+            const int64_t tile_rows_from = sizeof(T) == 1 ? 128 : 256 / (int64_t)sizeof(T);
+            return !(transposable && dsc.shape[rank - 1] >= tile_rows_from);
+        };
+        if (rank >= 2 && count < (1ull << 31) && count * sizeof(T) >= (256u << 10) && dsc.stride[2][rank - 1] == 1) {
+            const bool p0 = short_pieces(0), p1 = short_pieces(1);
+            if (p0 != p1) {
+                const int o = p0 ? 0 : 1;
+                typedef typename std::conditional<sizeof(T) == 1, uint8_t, typename std::conditional<sizeof(T) == 2, uint16_t,
+                        typename std::conditional<sizeof(T) == 4, uint32_t, uint64_t>::type>::type>::type Word;
+                void* tmp = nullptr;
+                if (rt_alloc_bytes(ctx, (size_t)count * sizeof(T), &tmp) == RT_OK) {
+                    NdDesc gd = dsc, d2 = dsc;
+                    int64_t acc = 1;
+                    bool others_are_runs = true;
+                    for (int k = rank - 1; k >= 0; --k) {
+                        gd.stride[0][k] = dsc.stride[o][k];
+                        gd.stride[1][k] = 0;
+                        gd.stride[2][k] = acc;
+                        d2.stride[o][k] = acc;
+                        others_are_runs = others_are_runs && dsc.stride[2][k] == acc && dsc.stride[1 - o][k] == acc;
+                        acc *= dsc.shape[k];
+                    }
+                    gd.offset[0] = dsc.offset[o];
+                    gd.offset[1] = dsc.offset[o];
+                    gd.offset[2] = 0;
+                    d2.offset[o] = 0;
+                    if (others_are_runs) {                              // three row-major runs: one dim
+                        d2.rank = 1;
+                        d2.shape[0] = (int64_t)count;
+                        for (int q = 0; q < 3; ++q) d2.stride[q][0] = 1;
+                    }
+                    int32_t status = RT_OK;
+                    const bool copied = permute_try<Word>(ctx, gd, count, (const Word*)(o == 0 ? lv : rv), (Word*)tmp, &status, /*force=*/true);
+                    if (copied && status == RT_OK) status = broadcast_typed<T, OP>(ctx, d2, count, o == 0 ? tmp : lv, o == 1 ? tmp : rv, dv);
+                    const int32_t freed = rt_free_locked(ctx, tmp);
+                    if (copied) return status != RT_OK ? status : freed;
+                }
+            }
+        }
+    }
+
     // (2a) copies only: interleaved -> planar, and views whose contiguous pieces are short on one side or both (rt_permute.hip);
     // then the tile kernel for one "transposed" input (rt_broadcast_tile.hip)
     if constexpr (OP == kOpCopy && std::is_integral<T>::value && sizeof(T) <= 8) {

@@ -244,8 +244,9 @@ template <class T>
 bool planar_copy_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* src, T* dst, int32_t* status);
 
 // Row-major copy of a view through N-d tiles in LDS (rt_permute.hip): for views whose contiguous pieces are short in src, in dst or
-// in both.  Returns false when the copy is not for it; instantiated for the four word sizes the gather uses.
+// in both.  Returns false when the copy is not for it (`force`: take every view the plan can handle, not only those it is the
+// fastest kernel for); instantiated for the four word sizes the gather uses.
 template <class T>
-bool permute_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* src, T* dst, int32_t* status);
+bool permute_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* src, T* dst, int32_t* status, bool force = false);
 
 }  // namespace rtb

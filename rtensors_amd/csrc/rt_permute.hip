@@ -25,7 +25,7 @@ __global__ __launch_bounds__(kPBlock) void permute_tile_kernel(const T* __restri
 namespace rtb {
 
 template <class T>
-bool permute_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* src, T* dst, int32_t* status) {
+bool permute_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* src, T* dst, int32_t* status, bool force) {
     constexpr uint32_t N = 16 / sizeof(T);
     if (dsc.rank < 2 || count >= (1ull << 31)) return false;
     PermArgs a;
@@ -56,7 +56,7 @@ bool permute_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* src, T
         wanted = (mag1 > 1 && unit_dim && (uint64_t)mag1 * sizeof(T) >= 64) || (mag1 == 1 && row_bytes < 256 && (is1 == 1 || row_bytes >= 64));
     else
         wanted = (mag1 > 1 && unit_dim && (uint64_t)mag1 * sizeof(T) >= 64 && !tile_kernel_fits) || (is1 == 1 && row_bytes < 64);
-    if (!wanted) return false;
+    if (!wanted && !force) return false;
     if (!rt_permute_plan(dsc.rank, dsc.shape, dsc.stride[0], dsc.stride[2], (uint32_t)sizeof(T), &a, &blocks)) return false;
     const T* sp = src + dsc.offset[0];
     T* dp = dst + dsc.offset[2];
@@ -82,9 +82,9 @@ bool permute_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* src, T
     return true;
 }
 
-template bool permute_try<uint8_t>(rt_ctx*, const NdDesc&, uint64_t, const uint8_t*, uint8_t*, int32_t*);
-template bool permute_try<uint16_t>(rt_ctx*, const NdDesc&, uint64_t, const uint16_t*, uint16_t*, int32_t*);
-template bool permute_try<uint32_t>(rt_ctx*, const NdDesc&, uint64_t, const uint32_t*, uint32_t*, int32_t*);
-template bool permute_try<uint64_t>(rt_ctx*, const NdDesc&, uint64_t, const uint64_t*, uint64_t*, int32_t*);
+template bool permute_try<uint8_t>(rt_ctx*, const NdDesc&, uint64_t, const uint8_t*, uint8_t*, int32_t*, bool);
+template bool permute_try<uint16_t>(rt_ctx*, const NdDesc&, uint64_t, const uint16_t*, uint16_t*, int32_t*, bool);
+template bool permute_try<uint32_t>(rt_ctx*, const NdDesc&, uint64_t, const uint32_t*, uint32_t*, int32_t*, bool);
+template bool permute_try<uint64_t>(rt_ctx*, const NdDesc&, uint64_t, const uint64_t*, uint64_t*, int32_t*, bool);
 
 }  // namespace rtb

@@ -2046,3 +2046,66 @@ def test_matmul_descriptor_checks(hip):
     hip.fill_contiguous(d, 7.0, 0, 16)
     hip.matmul((a, (0, [3, 0], [0, 1]), "row_major"), (b, (0, [0, 3], [3, 1]), "row_major"), d, 1, 3, 0, 3)
     assert hip.dump(d).tolist() == [0.0] * 9 + [7.0] * 7
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64", "i16", "u8", "i32"])
+def test_broadcast_with_a_permuted_operand_of_short_pieces(hip, dtype):
+    """`a op b.permute(..)` where the permuted operand's contiguous pieces are short (a unit-stride dim of a few elements, or dst rows of
+    a few elements) and large enough for the two-pass form: the operand is copied into a row-major temporary by the N-d tile copy and
+    the op runs on the temporary.  Either operand order, in place, with a reversed dim, into a dst that is itself a view; add, sub, mul
+    and (integers) a division with the fault for a zero divisor.  Against numpy on the same view, bit for bit."""
+    code = cpu.DTYPE_BY_NAME[dtype]
+    npd = cpu.NP_DTYPE[code]
+    rng = np.random.default_rng(zlib.crc32(b"permuted-operand" + dtype.encode()))
+    cases = [((42, 96, 2, 3, 64), (4, 2, 3, 1, 0)), ((130, 33, 100, 7), (3, 2, 1, 0)), ((2995, 16, 7, 2), (3, 1, 2, 0)), ((20971, 16, 2), (1, 0, 2)),
+             ((33, 50, 16, 9, 4), (2, 0, 4, 3, 1)), ((1000, 7, 100), (1, 2, 0))]
+    es = np.dtype(npd).itemsize
+    for shape, perm in cases:
+        n = int(np.prod(shape))
+        assert n * es >= 256 << 10
+        parent = rand_values(dtype, n, rng, 1, 60).reshape(shape)           # no zeros: the divisions below are defined
+        view = parent.transpose(perm)
+        out_shape = list(view.shape)
+        vst = [int(x) // es for x in view.strides]
+        other = rand_values(dtype, n, rng, 1, 60).reshape(out_shape)
+        row_major = [int(x) // es for x in other.strides]
+        gp, go, gd = hip.alloc_from_slice(code, parent.reshape(-1)), hip.alloc_from_slice(code, other.reshape(-1)), hip.alloc(code, n)
+        ops = [("add", np.add), ("sub", np.subtract), ("mul", np.multiply)]
+        if npd.kind in "iu":
+            ops.append(("div", lambda x, y: (np.trunc(x.astype(np.float64) / y.astype(np.float64))).astype(npd)))
+        for op, fn in ops:
+            for view_is_left in (True, False):
+                l = (gp, (0, out_shape, vst)) if view_is_left else (go, (0, out_shape, row_major))
+                r = (go, (0, out_shape, row_major)) if view_is_left else (gp, (0, out_shape, vst))
+                hip.broadcast(l, r, (gd, (0, out_shape, row_major)), op)
+                with np.errstate(all="ignore"):
+                    want = fn(view, other) if view_is_left else fn(other, view)
+                assert hip.dump(gd).tobytes() == np.ascontiguousarray(want.astype(npd)).tobytes(), (dtype, shape, perm, op, view_is_left)
+        # in place: other op= view, then with the view's last dim reversed
+        hip.broadcast((go, (0, out_shape, row_major)), (gp, (0, out_shape, vst)), (go, (0, out_shape, row_major)), "add")
+        with np.errstate(all="ignore"):
+            acc = np.add(other, view).astype(npd)
+        assert hip.dump(go).tobytes() == np.ascontiguousarray(acc).tobytes(), (dtype, shape, perm, "in place")
+        rst = list(vst); rst[-1] = -rst[-1]
+        hip.broadcast((go, (0, out_shape, row_major)), (gp, ((out_shape[-1] - 1) * vst[-1], out_shape, rst)), (go, (0, out_shape, row_major)), "sub")
+        with np.errstate(all="ignore"):
+            acc = np.subtract(acc, np.flip(view, -1)).astype(npd)
+        assert hip.dump(go).tobytes() == np.ascontiguousarray(acc).tobytes(), (dtype, shape, perm, "in place, reversed")
+    if npd.kind in "iu":
+        # a zero divisor inside the permuted operand: the fault the reference panics with, reported by the next call that waits
+        shape, perm = cases[0]
+        n = int(np.prod(shape))
+        parent = rand_values(dtype, n, rng, 1, 60).reshape(shape)
+        parent.reshape(-1)[n // 3] = 0
+        view = parent.transpose(perm)
+        out_shape = list(view.shape)
+        vst = [int(x) // es for x in view.strides]
+        other = rand_values(dtype, n, rng, 1, 60).reshape(out_shape)
+        row_major = [int(x) // es for x in other.strides]
+        gp, go, gd = hip.alloc_from_slice(code, parent.reshape(-1)), hip.alloc_from_slice(code, other.reshape(-1)), hip.alloc(code, n)
+        hip.broadcast((go, (0, out_shape, row_major)), (gp, (0, out_shape, vst)), (gd, (0, out_shape, row_major)), "div")
+        from rtensors_amd import hip as H
+        with pytest.raises(H.TensorError) as e:
+            hip.sync()
+        assert e.value.kind == "ArithmeticError"
+        hip.sync()                                                         # reported once, then clear
