@@ -535,6 +535,26 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
     if constexpr (OP != kOpCopy && sizeof(T) <= 8) {
         auto short_pieces = [&](int o) {
             const int64_t is1 = dsc.stride[o][rank - 1], mag1 = is1 < 0 ? -is1 : is1;
+            if (is1 == 1) {
+                // unit-stride rows of less than 256 bytes (64 for 1- and 2-byte elements): rows of 2 out of strides (2, 32, 1) ran at
+                // 0.16 of peak ...
+                const uint64_t row_bytes = (uint64_t)dsc.shape[rank - 1] * sizeof(T);
+                if (row_bytes >= (sizeof(T) >= 4 ? 256u : 64u)) return false;
+                // ... and whose rows lie scattered: the 4096 elements that dst's order visits next span more than four times their
+                // own size in the input.  Rows that are merely reversed or stepped stay compact, the row kernels find them in cache
+                // (rows of 7 under a reversed dim of 64: 0.79 there, 0.43 through a temporary).
+                uint64_t visited = 1, span = 1;
+                for (int k = rank - 1; k >= 0; --k) {
+                    if (dsc.stride[o][k] == 0) return false;
+                    if (visited >= 4096) continue;
+                    const uint64_t want = (4096 + visited - 1) / visited;
+                    const uint64_t take = (uint64_t)dsc.shape[k] < want ? (uint64_t)dsc.shape[k] : want;
+                    const int64_t st = dsc.stride[o][k];
+                    span += (take - 1) * (uint64_t)(st < 0 ? -st : st);
+                    visited *= take;
+                }
+                return span > 4 * visited;
+            }
             if (mag1 <= 1 || (uint64_t)mag1 * sizeof(T) < 64) return false;
             bool unit_dim = false, transposable = false;
             uint64_t inside = 1;                                       // dst elements per index of the innermost unit-stride dim
@@ -560,6 +580,31 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
                 typedef typename std::conditional<sizeof(T) == 1, uint8_t, typename std::conditional<sizeof(T) == 2, uint16_t,
                         typename std::conditional<sizeof(T) == 4, uint32_t, uint64_t>::type>::type>::type Word;
                 void* tmp = nullptr;
+                bool runs = true;                                       // dst and the other input are row-major runs over the dims
+                {
+                    int64_t acc = 1;
+                    for (int k = rank - 1; k >= 0; --k) {
+                        runs = runs && dsc.stride[2][k] == acc && dsc.stride[1 - o][k] == acc;
+                        acc *= dsc.shape[k];
+                    }
+                }
+                if constexpr (PermBinFused<T, OP>::value) {
+                    // float, double and the 32- / 64-bit carriers: the op rides on the tile copy's second stage, which loads the other
+                    // input's piece next to the tile's and stores the result -- one pass over each tensor
+                    if (runs) {
+                        NdDesc gd = dsc;
+                        int64_t acc = 1;
+                        for (int k = rank - 1; k >= 0; --k) {
+                            gd.stride[0][k] = dsc.stride[o][k];
+                            gd.stride[2][k] = acc;
+                            acc *= dsc.shape[k];
+                        }
+                        gd.offset[0] = dsc.offset[o];
+                        int32_t status = RT_OK;
+                        if (permute_bin_try<T, OP>(ctx, gd, count, o == 0 ? l : r, (o == 0 ? r : l) + dsc.offset[1 - o], d + dsc.offset[2], o == 0, &status))
+                            return status;
+                    }
+                }
                 if (rt_alloc_bytes(ctx, (size_t)count * sizeof(T), &tmp) == RT_OK) {
                     NdDesc gd = dsc, d2 = dsc;
                     int64_t acc = 1;

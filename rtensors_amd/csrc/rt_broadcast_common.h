@@ -249,4 +249,14 @@ bool planar_copy_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* sr
 template <class T>
 bool permute_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* src, T* dst, int32_t* status, bool force = false);
 
+// dst = xt (op) xo, or xo (op) xt, through the same N-d tiles: xt is the permuted input (dsc.stride[0], dsc.offset[0]); xo and dst
+// point at their first elements and are both laid out row-major over dsc.shape (dsc.stride[2]); dst may be xo.  Instantiated for
+// float and double with the four ops and for the 32- and 64-bit carriers with + - * (PermBinFused below).
+template <class T, int OP>
+bool permute_bin_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* xt, const T* xo, T* dst, bool tile_is_left, int32_t* status);
+template <class T, int OP> struct PermBinFused {
+    static constexpr bool value = std::is_same<T, float>::value || std::is_same<T, double>::value ||
+                                  ((std::is_same<T, uint32_t>::value || std::is_same<T, uint64_t>::value) && OP != RT_DIV && OP != kOpCopy);
+};
+
 }  // namespace rtb

@@ -251,9 +251,19 @@ __host__ __device__ __forceinline__ void pm_stage1(const T* src, const PermArgs&
     }
 }
 
+// What stage 2 does with a piece of the tile before it stores it.  The plain copy stores it as it is; a binary op whose other input
+// is laid out like dst loads that input's piece at the same byte offset -- before the LDS reads, so that the loads of all rows a lane
+// handles are in flight together: behind the stores they could not move up, because dst may be that very input (`c += v`) -- and
+// combines the two.
+struct PmCopy {
+    template <class VT> __host__ __device__ __forceinline__ VT fetch(uint32_t) const { return VT{}; }
+    template <class VT> __host__ __device__ __forceinline__ VT combine(const VT& tile_piece, const VT&) const { return tile_piece; }
+};
+
 // W: elements per store (rt_permute_store_width)
-template <class T, int W>
-__host__ __device__ __forceinline__ void pm_stage2(T* dst, const PermArgs& a, const PermBlock& b, uint32_t tid, const unsigned char* tile, const PermTables& tb) {
+template <class T, int W, class F>
+__host__ __device__ __forceinline__ void pm_stage2(T* dst, const PermArgs& a, const PermBlock& b, uint32_t tid, const unsigned char* tile, const PermTables& tb,
+                                                    const F& f) {
     constexpr int U = kPRows2;
     constexpr uint32_t ES = (uint32_t)sizeof(T);
     typedef typename PmVec<T, W>::type VT;
@@ -271,13 +281,16 @@ __host__ __device__ __forceinline__ void pm_stage2(T* dst, const PermArgs& a, co
             dof[u] = r < a.rows2 ? tb.row2_dst[r] : 0u;
         }
         for (uint32_t p = pos * W * ES; p < valid; p += lpr * W * ES) {
-            VT v[U];
+            VT v[U], o[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (lo[u] != kPNoRow) o[u] = f.template fetch<VT>(dof[u] + p);
 #pragma unroll
             for (int u = 0; u < U; ++u)
                 if (lo[u] != kPNoRow) v[u] = *reinterpret_cast<const VT*>(tile + pm_swizzle(lo[u] + p));
 #pragma unroll
             for (int u = 0; u < U; ++u)
-                if (lo[u] != kPNoRow) __builtin_nontemporal_store(v[u], reinterpret_cast<VT*>(dp + (dof[u] + p)));
+                if (lo[u] != kPNoRow) __builtin_nontemporal_store(f.template combine<VT>(v[u], o[u]), reinterpret_cast<VT*>(dp + (dof[u] + p)));
         }
     }
 }

@@ -23,7 +23,7 @@ static void run_blocks(PermArgs a, uint64_t blocks, const T* src, T* dst) {
         const PermBlock b = pm_block(a, (uint32_t)blk);
         for (uint32_t t = 0; t < (uint32_t)kPBlock; ++t) pm_stage0<T>(a, (uint32_t)blk, t, tb);
         for (uint32_t t = 0; t < (uint32_t)kPBlock; ++t) pm_stage1<T, V>(src, a, b, t, tile, tb);
-        for (uint32_t t = 0; t < (uint32_t)kPBlock; ++t) pm_stage2<T, W>(dst, a, b, t, tile, tb);
+        for (uint32_t t = 0; t < (uint32_t)kPBlock; ++t) pm_stage2<T, W>(dst, a, b, t, tile, tb, PmCopy{});
     }
 }
 
