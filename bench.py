@@ -450,8 +450,8 @@ class Workloads:
         return (lambda: self.hip.gather(a, (0, shape, strides), c)), 2 * n * 4, n
 
     def add_perm_rows42(self):
-        """c = a + v with v the (64, 3, 2, 4096, 42) view of gather_rows42 and a, c row-major: the permuted operand goes through a row-major
-        temporary (the N-d tile copy, then the contiguous add).  Algorithmic bytes are the three tensors once."""
+        """c = a + v with v the (64, 3, 2, 4096, 42) view of gather_rows42 and a, c row-major: the add rides on the second stage of the N-d
+        tile copy of v.  Algorithmic bytes are the three tensors once."""
         H = self.H
         shape, strides = [64, 3, 2, 4096, 42], [1, 262144, 786432, 64, 1572864]
         n = 64 * 3 * 2 * 4096 * 42

@@ -169,10 +169,11 @@ int32_t rt_scalar_nd(rt_ctx* ctx, int32_t dtype, int32_t op, void* buf, uint64_t
  * before the kernel has run; the kernel stores 0 / MIN for such elements and sets a fault word of the context, and the next
  * call that waits for the stream (rt_sync, rt_read, rt_dump, rt_equal) returns RT_E_ARITH once and clears it.  The same holds for
  * rt_scalar_* division of a signed tensor by -1.  A zero scalar divisor is refused at once.
- * Device memory: an input that is a permuted view with short contiguous pieces (256 KiB and more, stepping 64 bytes or more along
- * dst's inner dim) is first copied into a row-major temporary of its own size, taken from and returned to the context's block
- * cache like an rt_alloc_uninit / rt_free pair; if the block cannot be had the op runs without it, slower.  No other input layout
- * makes this call allocate. */
+ * Device memory: an input of 256 KiB and more that is a permuted view with short contiguous pieces (it steps 64 bytes or more along
+ * dst's inner dim, or its unit-stride rows are shorter than 256 bytes and lie scattered) may first be copied into a row-major
+ * temporary of its own size, taken from and returned to the context's block cache like an rt_alloc_uninit / rt_free pair -- not
+ * when dst and the other input are row-major runs of f32, f64 or 32- / 64-bit integers under + - * (floats also /), which one
+ * kernel handles.  If the block cannot be had the op runs without it, slower.  No other input layout makes this call allocate. */
 int32_t rt_broadcast(rt_ctx* ctx, int32_t dtype, int32_t op, int32_t rank, const uint64_t* shape,
                      const void* left, uint64_t left_len, uint64_t left_offset, const int64_t* left_strides,
                      const void* right, uint64_t right_len, uint64_t right_offset, const int64_t* right_strides,
