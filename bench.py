@@ -544,7 +544,7 @@ DETAIL = ["copy", "fill", "c1_add", "c1_sum1", "c2_mul", "c2_add", "c2_relu", "c
           "c2_fused", "c2_fused_f64", "c2_fused_i32",
           "c3a_add", "c3b_add", "c4_sum1", "c4_mean1", "c4_max1", "c4_sum0", "c4_sum_all", "c4_i32_sum1", "c4_i32_max1", "c4_i32_min0",
           "c4_var1", "c4_std0", "c4_lse1", "c4_argmax1", "c5_bias_add", "c5_colsum", "c5_fused_bias_relu", "c5_fused_l1_forward", "c5_fused_backward", "c5_fused2_forward", "c5_fused2_backward",
-          "view_relu", "tr_add", "tr_copy", "gather_rows42"]
+          "view_relu", "tr_add", "tr_copy", "gather_rows42", "add_perm_rows42"]
 KIND = {"copy": "elementwise", "fill": "elementwise"}
 
 

@@ -528,9 +528,11 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
 
     // (1b) an input that is a permuted view with short contiguous pieces -- it steps by 64 bytes or more along dst's inner dim, is
     // unit-stride along some other dim, and the transposing kernels below do not fit it (dst rows or that unit-stride dim too
-    // short): read along dst's rows it costs a cache line per element (f32 `a + b.permute(..)` over 256 MiB operands: median 0.27
-    // of peak over 54 such views, the lowest tenth 0.08).  It is first copied into a row-major temporary by the N-d tile copy
-    // (rt_permute.hip), then the op runs on the temporary: two more passes over that operand, 0.37 - 0.48 of peak on the same views.
+    // short); or its unit-stride rows are short and lie scattered.  Read along dst's rows it costs a cache line per element or per
+    // few elements (f32 `a + b.permute(..)` over 256 MiB operands: median 0.27 of peak over 54 such views, the lowest tenth 0.08).
+    // Where dst and the other input are row-major runs and the type allows, the op rides on the second stage of the N-d tile copy
+    // of that input (rt_permute.hip: one pass over each tensor, 0.45 - 0.75 of peak on those views); otherwise the input is copied
+    // into a row-major temporary by the tile copy and the op runs on the temporary (two more passes over that operand, 0.37 - 0.48).
     // The temporary comes from the context's block cache and goes back to it; all work is on the context's stream.
     if constexpr (OP != kOpCopy && sizeof(T) <= 8) {
         auto short_pieces = [&](int o) {
@@ -608,20 +610,18 @@ int32_t broadcast_typed(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const vo
                 if (rt_alloc_bytes(ctx, (size_t)count * sizeof(T), &tmp) == RT_OK) {
                     NdDesc gd = dsc, d2 = dsc;
                     int64_t acc = 1;
-                    bool others_are_runs = true;
                     for (int k = rank - 1; k >= 0; --k) {
                         gd.stride[0][k] = dsc.stride[o][k];
                         gd.stride[1][k] = 0;
                         gd.stride[2][k] = acc;
                         d2.stride[o][k] = acc;
-                        others_are_runs = others_are_runs && dsc.stride[2][k] == acc && dsc.stride[1 - o][k] == acc;
                         acc *= dsc.shape[k];
                     }
                     gd.offset[0] = dsc.offset[o];
                     gd.offset[1] = dsc.offset[o];
                     gd.offset[2] = 0;
                     d2.offset[o] = 0;
-                    if (others_are_runs) {                              // three row-major runs: one dim
+                    if (runs) {                                         // three row-major runs: one dim
                         d2.rank = 1;
                         d2.shape[0] = (int64_t)count;
                         for (int q = 0; q < 3; ++q) d2.stride[q][0] = 1;

@@ -28,7 +28,6 @@
 namespace rtp {
 
 constexpr int kPBlock = 256;
-constexpr int kPWaves = kPBlock / RT_WAVE;
 constexpr uint32_t kPTileBytes = 32768;      // payload of a tile
 constexpr uint32_t kPTabMax = 1024;          // positions of a src run
 constexpr uint32_t kPRowMax = 512;           // rows of a stage
