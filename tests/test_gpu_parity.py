@@ -2048,7 +2048,7 @@ def test_matmul_descriptor_checks(hip):
     assert hip.dump(d).tolist() == [0.0] * 9 + [7.0] * 7
 
 
-@pytest.mark.parametrize("dtype", ["f32", "f64", "i16", "u8", "i32"])
+@pytest.mark.parametrize("dtype", ["f32", "f64", "i16", "u8", "i32", "i64", "u32"])
 def test_broadcast_with_a_permuted_operand_of_short_pieces(hip, dtype):
     """`a op b.permute(..)` where the permuted operand's contiguous pieces are short (a unit-stride dim of a few elements, or dst rows of
     a few elements) and large enough for the two-pass form: the operand is copied into a row-major temporary by the N-d tile copy and
@@ -2073,6 +2073,8 @@ def test_broadcast_with_a_permuted_operand_of_short_pieces(hip, dtype):
         ops = [("add", np.add), ("sub", np.subtract), ("mul", np.multiply)]
         if npd.kind in "iu":
             ops.append(("div", lambda x, y: (np.trunc(x.astype(np.float64) / y.astype(np.float64))).astype(npd)))
+        else:
+            ops.append(("div", np.divide))
         for op, fn in ops:
             for view_is_left in (True, False):
                 l = (gp, (0, out_shape, vst)) if view_is_left else (go, (0, out_shape, row_major))
