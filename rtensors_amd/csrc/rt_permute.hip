@@ -12,8 +12,9 @@ template <class T, int W, int V>
 __global__ __launch_bounds__(kPBlock) void permute_tile_kernel(const T* __restrict__ src, T* __restrict__ dst, PermArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const PermTables tb = pm_tables(a, smem, (uint32_t)sizeof(T));
-    const PermBlock b = pm_block(a, blockIdx.x);
-    pm_stage0<T>(a, blockIdx.x, threadIdx.x, tb);
+    const uint32_t block = pm_remap(a, blockIdx.x);
+    const PermBlock b = pm_block(a, block);
+    pm_stage0<T>(a, block, threadIdx.x, tb);
     __syncthreads();
     pm_stage1<T, V>(src, a, b, threadIdx.x, smem, tb);
     __syncthreads();
@@ -43,8 +44,9 @@ template <class T, int OP, int W, int V>
 __global__ __launch_bounds__(kPBlock) void permute_bin_kernel(const T* __restrict__ xt, const T* xo, T* dst, PermArgs a, uint32_t tile_is_left) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const PermTables tb = pm_tables(a, smem, (uint32_t)sizeof(T));
-    const PermBlock b = pm_block(a, blockIdx.x);
-    pm_stage0<T>(a, blockIdx.x, threadIdx.x, tb);
+    const uint32_t block = pm_remap(a, blockIdx.x);
+    const PermBlock b = pm_block(a, block);
+    pm_stage0<T>(a, block, threadIdx.x, tb);
     __syncthreads();
     pm_stage1<T, V>(xt, a, b, threadIdx.x, smem, tb);
     __syncthreads();
@@ -89,9 +91,9 @@ bool permute_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* src, T
     else
         wanted = (mag1 > 1 && unit_dim && (uint64_t)mag1 * sizeof(T) >= 64 && !tile_kernel_fits) || (is1 == 1 && row_bytes < 64);
     if (!wanted && !force) return false;
-    if (!rt_permute_plan(dsc.rank, dsc.shape, dsc.stride[0], dsc.stride[2], (uint32_t)sizeof(T), &a, &blocks)) return false;
     const T* sp = src + dsc.offset[0];
     T* dp = dst + dsc.offset[2];
+    if (!rt_permute_plan(dsc.rank, dsc.shape, dsc.stride[0], dsc.stride[2], (uint32_t)sizeof(T), &a, &blocks, kPTileBytes, reinterpret_cast<uintptr_t>(sp) % 128 == 0)) return false;
     uint32_t w = rt_permute_store_width(a, N);
     while (w > 1 && (reinterpret_cast<uintptr_t>(dp) % (w * sizeof(T))) != 0) w >>= 1;
     constexpr uint32_t kWord = sizeof(T) < 4 ? 4 / sizeof(T) : 1;      // a 32-bit store of 1- and 2-byte elements
@@ -120,8 +122,8 @@ bool permute_bin_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* xt
     if (dsc.rank < 2 || count >= (1ull << 31)) return false;
     PermArgs a;
     uint64_t blocks = 0;
-    if (!rt_permute_plan(dsc.rank, dsc.shape, dsc.stride[0], dsc.stride[2], (uint32_t)sizeof(T), &a, &blocks)) return false;
     const T* sp = xt + dsc.offset[0];
+    if (!rt_permute_plan(dsc.rank, dsc.shape, dsc.stride[0], dsc.stride[2], (uint32_t)sizeof(T), &a, &blocks, kPTileBytes, reinterpret_cast<uintptr_t>(sp) % 128 == 0)) return false;
     uint32_t w = rt_permute_store_width(a, N);
     while (w > 1 && ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(xo)) % (w * sizeof(T))) != 0) w >>= 1;
     w = w == N ? N : 1u;

@@ -20,8 +20,9 @@ static void run_blocks(PermArgs a, uint64_t blocks, const T* src, T* dst) {
     unsigned char* tile = smem.data();
     const PermTables tb = pm_tables(a, smem.data(), (uint32_t)sizeof(T));
     for (uint64_t blk = 0; blk < blocks; ++blk) {
-        const PermBlock b = pm_block(a, (uint32_t)blk);
-        for (uint32_t t = 0; t < (uint32_t)kPBlock; ++t) pm_stage0<T>(a, (uint32_t)blk, t, tb);
+        const uint32_t which = pm_remap(a, (uint32_t)blk);
+        const PermBlock b = pm_block(a, which);
+        for (uint32_t t = 0; t < (uint32_t)kPBlock; ++t) pm_stage0<T>(a, which, t, tb);
         for (uint32_t t = 0; t < (uint32_t)kPBlock; ++t) pm_stage1<T, V>(src, a, b, t, tile, tb);
         for (uint32_t t = 0; t < (uint32_t)kPBlock; ++t) pm_stage2<T, W>(dst, a, b, t, tile, tb, PmCopy{});
     }
