@@ -67,7 +67,7 @@ bool permute_try(rt_ctx* ctx, const NdDesc& dsc, uint64_t count, const T* src, T
     // Where this kernel is the faster one, from timing permuted, reversed and stepped views of 256 MiB in every element size against
     // the row, flat and transposing kernels (fractions of the HBM peak, 2 x the view's bytes per copy):
     //   * src steps by 64 bytes or more along dst's inner dim and has a unit-stride dim somewhere else -- the permuted views proper.
-    //     4- and 8-byte elements: the median goes from 0.57 to 0.70, the lowest tenth from 0.22 to 0.47 (unit-stride dims of 2 .. 7
+    //     4- and 8-byte elements: the median goes from 0.57 to 0.71, the lowest tenth from 0.22 to 0.48 (unit-stride dims of 2 .. 7
     //     elements, dst rows of a few elements: 0.05 before).  1- and 2-byte elements only where the transposing tile kernel does
     //     not apply (it packs four or two of them per LDS word; this kernel moves them one by one);
     //   * src is unit-stride along dst's inner dim but the rows are shorter than 256 bytes (64 bytes for 1- and 2-byte elements):
